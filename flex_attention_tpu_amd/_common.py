@@ -1,0 +1,136 @@
+"""Host-side helpers shared by the three entry points: argument checks and C struct assembly."""
+from __future__ import annotations
+
+from typing import Callable, Dict, Optional, Tuple
+
+import numpy as np
+import torch
+
+from . import _lib
+from .block_mask import BlockMap, build_block_map, mask_spec_c, spec_of
+from .masks import DocIds, MaskSpec
+from .scores import ScoreSpec
+
+_slopes_cache: Dict[Tuple[Tuple[float, ...], str], torch.Tensor] = {}
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return _lib.BF16
+    if t.dtype == torch.float32:
+        return _lib.F32
+    raise NotImplementedError(f"dtype {t.dtype} is not supported (bfloat16 and float32 are)")
+
+
+def check_qkv(q, k, v, *others):
+    """Shape / layout checks in the spirit of the reference's rank asserts
+    (flex_attention_dq_bwd.py:161-164); returns (B, Hq, Hkv, Sq, Sk, D)."""
+    for name, t in (("q", q), ("k", k), ("v", v)) + tuple((f"arg{i}", o) for i, o in enumerate(others)):
+        if not isinstance(t, torch.Tensor):
+            raise TypeError(f"{name} must be a torch.Tensor")
+        if t.ndim != 4:
+            raise ValueError(f"{name} must have rank 4 [batch, heads, seq, head_dim], got {tuple(t.shape)}")
+        if not t.is_cuda:
+            raise ValueError(f"{name} must live on the GPU (got {t.device}); this package has no CPU path")
+        if not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous")
+        if t.dtype != q.dtype:
+            raise ValueError(f"{name} has dtype {t.dtype}, expected {q.dtype}")
+    B, Hq, Sq, D = q.shape
+    Bk, Hkv, Sk, Dk = k.shape
+    if v.shape != k.shape:
+        raise ValueError(f"k {tuple(k.shape)} and v {tuple(v.shape)} differ")
+    if Bk != B or Dk != D:
+        raise ValueError(f"q {tuple(q.shape)} and k {tuple(k.shape)} disagree on batch or head_dim")
+    if Hq % Hkv:
+        raise ValueError(f"query heads {Hq} not a multiple of kv heads {Hkv}")
+    for o in others:
+        if tuple(o.shape) != tuple(q.shape):
+            raise ValueError(f"expected shape {tuple(q.shape)}, got {tuple(o.shape)}")
+    return B, Hq, Hkv, Sq, Sk, D
+
+
+def check_rows(name, t, B, Hq, Sq, device):
+    if not isinstance(t, torch.Tensor) or tuple(t.shape) != (B, Hq, Sq):
+        raise ValueError(f"{name} must be a float32 tensor of shape {(B, Hq, Sq)}")
+    if t.dtype != torch.float32 or not t.is_contiguous() or t.device != device:
+        raise ValueError(f"{name} must be contiguous float32 on {device}")
+
+
+def check_blocks(Sq, Sk, block_q=None, block_k_major=None, block_k=None, block_q_major=None):
+    """Block sizes are tuning hints in the reference; here they are validated only
+    (the device tiles are the kernels' own)."""
+    def _div(name, blk, n):
+        if blk is None:
+            return
+        if not isinstance(blk, (int, np.integer)) or blk <= 0:
+            raise ValueError(f"{name}={blk!r} must be a positive int")
+        if n % blk:
+            raise ValueError(f"{name}={blk} does not divide sequence length {n}")
+    _div("block_q", block_q, Sq)
+    _div("block_q_major", block_q_major, Sq)
+    _div("block_k_major", block_k_major, Sk)
+    _div("block_k", block_k, Sk)
+    if block_k is not None and block_k_major is not None and block_k_major % block_k:
+        raise ValueError(f"block_k={block_k} does not divide block_k_major={block_k_major}")
+    if block_q is not None and block_q_major is not None and block_q_major % block_q:
+        raise ValueError(f"block_q={block_q} does not divide block_q_major={block_q_major}")
+
+
+def resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk) -> MaskSpec:
+    """Single MaskSpec for the closures, the ``causal`` flag and ``segment_ids`` (AND of all)."""
+    spec = spec_of(mask_fn, block_mask_fn)
+    if causal:
+        spec = spec.combine(MaskSpec(flags=_lib.MASK_CAUSAL))
+    if segment_ids is not None:
+        ids = segment_ids
+        if hasattr(ids, "q") and hasattr(ids, "kv"):
+            if not torch.equal(torch.as_tensor(ids.q), torch.as_tensor(ids.kv)):
+                raise NotImplementedError("distinct q / kv segment ids are not supported")
+            ids = ids.q
+        ids = torch.as_tensor(ids).detach().cpu()
+        if ids.ndim == 2:
+            if not bool((ids == ids[:1]).all()):
+                raise NotImplementedError("per-batch segment ids are not supported")
+            ids = ids[0]
+        arr = ids.numpy().astype(np.int64)
+        if arr.shape[0] != Sq or Sq != Sk:
+            raise ValueError("segment_ids must have one id per position of a self-attention sequence")
+        if np.any(np.diff(arr) < 0):
+            raise NotImplementedError("segment ids must be non-decreasing along the sequence")
+        spec = spec.combine(MaskSpec(flags=_lib.MASK_DOC, doc_ids=DocIds(arr)))
+    return spec
+
+
+def score_spec_c(score_fn: Optional[Callable], Hq: int, device, mod_q: int, mod_k: int) -> _lib.ScoreSpecC:
+    """C view of the score closure's spec.  ``mod_q``/``mod_k`` are the tile edges the reference
+    would call a tile-local score function with (block_q, block_k)."""
+    if score_fn is None:
+        return _lib.ScoreSpecC(_lib.SCORE_NONE, 0.0, 0.0, 1, 1, 0, None)
+    spec = getattr(score_fn, "spec", None)
+    if not isinstance(spec, ScoreSpec):
+        raise NotImplementedError(
+            "score_fn must come from flex_attention_tpu_amd.scores factories or util.make_jax_score_fn "
+            "(arbitrary Python callables cannot be compiled into the HIP kernels)")
+    slopes_ptr = None
+    if spec.kind == _lib.SCORE_ALIBI:
+        if len(spec.slopes) != Hq:
+            raise ValueError(f"ALiBi has {len(spec.slopes)} slopes for {Hq} heads")
+        key = (spec.slopes, str(device))
+        t = _slopes_cache.get(key)
+        if t is None:
+            t = torch.tensor(spec.slopes, dtype=torch.float32, device=device)
+            _slopes_cache[key] = t
+        slopes_ptr = t.data_ptr()
+    return _lib.ScoreSpecC(spec.kind, spec.cap, spec.slope, int(mod_q), int(mod_k), 0, slopes_ptr)
+
+
+def kernel_block_map(pass_id: int, spec: MaskSpec, q: torch.Tensor, Sq: int, Sk: int, D: int) -> BlockMap:
+    bq, bk = _lib.tile_shape(pass_id, dtype_code(q), D)
+    if Sq % bq or Sk % bk:
+        raise ValueError(f"sequence lengths ({Sq}, {Sk}) must be multiples of the kernel tile ({bq}, {bk})")
+    return build_block_map(spec, Sq, Sk, bq, bk, q.device)
+
+
+def stream_of(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream

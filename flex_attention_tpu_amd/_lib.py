@@ -1,0 +1,162 @@
+"""ctypes binding of libflexattn.so (the C ABI declared in include/flexattn.h).
+
+The library is the only compute path of this package: importing this module fails loudly when the
+shared object has not been built (``python -m flex_attention_tpu_amd.build``); there is no
+fallback implementation.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libflexattn.so")
+
+OK = 0
+EINVAL = -22
+ENOTSUP = -95
+ELAUNCH = -5
+
+BF16 = 0
+F32 = 1
+
+SCORE_NONE = 0
+SCORE_ALIBI = 1
+SCORE_SOFTCAP = 2
+SCORE_ALIBI_TILE = 3
+
+MASK_CAUSAL = 1
+MASK_WINDOW = 2
+MASK_DOC = 4
+MASK_S2 = 8
+
+PASS_FWD = 0
+PASS_DQ = 1
+PASS_DKV = 2
+
+
+class ScoreSpecC(C.Structure):
+    _fields_ = [
+        ("kind", C.c_int32),
+        ("cap", C.c_float),
+        ("slope", C.c_float),
+        ("mod_q", C.c_int32),
+        ("mod_k", C.c_int32),
+        ("reserved", C.c_int32),
+        ("slopes", C.c_void_p),
+    ]
+
+
+class MaskSpecC(C.Structure):
+    _fields_ = [
+        ("flags", C.c_int32),
+        ("window", C.c_int32),
+        ("stride", C.c_int32),
+        ("reserved", C.c_int32),
+        ("doc_q", C.c_void_p),
+        ("doc_k", C.c_void_p),
+    ]
+
+
+class BlockMapC(C.Structure):
+    _fields_ = [
+        ("state", C.c_void_p),
+        ("kv_cnt", C.c_void_p),
+        ("kv_idx", C.c_void_p),
+        ("q_cnt", C.c_void_p),
+        ("q_idx", C.c_void_p),
+        ("nq", C.c_int32),
+        ("nk", C.c_int32),
+        ("block_q", C.c_int32),
+        ("block_k", C.c_int32),
+    ]
+
+
+class FwdParamsC(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p),
+        ("o", C.c_void_p),
+        ("l", C.c_void_p), ("m", C.c_void_p),
+        ("B", C.c_int32), ("Hq", C.c_int32), ("Hkv", C.c_int32),
+        ("Sq", C.c_int32), ("Sk", C.c_int32), ("D", C.c_int32),
+        ("dtype", C.c_int32),
+        ("sm_scale", C.c_float),
+        ("score", ScoreSpecC),
+        ("mask", MaskSpecC),
+        ("map", BlockMapC),
+    ]
+
+
+class BwdParamsC(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("dout", C.c_void_p),
+        ("l", C.c_void_p), ("m", C.c_void_p), ("delta", C.c_void_p),
+        ("dq", C.c_void_p),
+        ("dk", C.c_void_p), ("dv", C.c_void_p),
+        ("B", C.c_int32), ("Hq", C.c_int32), ("Hkv", C.c_int32),
+        ("Sq", C.c_int32), ("Sk", C.c_int32), ("D", C.c_int32),
+        ("dtype", C.c_int32),
+        ("sm_scale", C.c_float),
+        ("score", ScoreSpecC),
+        ("mask", MaskSpecC),
+        ("map", BlockMapC),
+    ]
+
+
+EXPORTS = (
+    "flexattn_version",
+    "flexattn_last_error_string",
+    "flexattn_tile_shape",
+    "flexattn_build_block_mask",
+    "flexattn_fwd",
+    "flexattn_bwd_delta",
+    "flexattn_bwd_dq",
+    "flexattn_bwd_dkv",
+)
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Loads libflexattn.so once; raises ImportError if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m flex_attention_tpu_amd.build` "
+            "(hipcc, gfx950). This package has no other compute path.")
+    lib = C.CDLL(LIB_PATH)
+    lib.flexattn_version.restype = C.c_int
+    lib.flexattn_last_error_string.restype = C.c_char_p
+    lib.flexattn_tile_shape.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
+    lib.flexattn_build_block_mask.argtypes = [
+        C.POINTER(MaskSpecC), C.c_int32, C.c_int32, C.c_int32, C.c_int32,
+        C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.flexattn_fwd.argtypes = [C.POINTER(FwdParamsC), C.c_void_p]
+    lib.flexattn_bwd_delta.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
+    lib.flexattn_bwd_dq.argtypes = [C.POINTER(BwdParamsC), C.c_void_p]
+    lib.flexattn_bwd_dkv.argtypes = [C.POINTER(BwdParamsC), C.c_void_p]
+    for name in ("flexattn_tile_shape", "flexattn_build_block_mask", "flexattn_fwd", "flexattn_bwd_delta",
+                 "flexattn_bwd_dq", "flexattn_bwd_dkv"):
+        getattr(lib, name).restype = C.c_int
+    _lib = lib
+    return lib
+
+
+def check(rc: int) -> None:
+    """Maps a status code to the exception class the reference raises in the same situation."""
+    if rc == OK:
+        return
+    msg = load().flexattn_last_error_string().decode("utf-8", "replace")
+    if rc == EINVAL:
+        raise ValueError(msg)
+    if rc == ENOTSUP:
+        raise NotImplementedError(msg)
+    raise RuntimeError(f"flexattn error {rc}: {msg}")
+
+
+def tile_shape(pass_id: int, dtype: int, D: int):
+    bq, bk = C.c_int32(0), C.c_int32(0)
+    check(load().flexattn_tile_shape(pass_id, dtype, D, C.byref(bq), C.byref(bk)))
+    return bq.value, bk.value

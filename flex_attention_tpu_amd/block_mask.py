@@ -1,0 +1,127 @@
+"""Block-sparsity maps: the GPU builder (flexattn_build_block_mask) and its host-side handle.
+
+The reference evaluates ``block_mask_fn(q_block, kv_block)`` at every grid step and again inside
+the K/V index maps (flex_attention_kernel.py:97-106, 231-236).  Here the same predicate is
+evaluated once per (mask, shape, tile) by a small HIP kernel into a device-resident map that the
+attention kernels walk; maps are cached because they depend on nothing but the mask specification.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Callable, Dict, Optional, Tuple
+
+import torch
+
+from . import _lib
+from .masks import DocIds, MaskSpec
+
+
+class BlockMap:
+    """Device-resident block map at (block_q x block_k) granularity.
+
+    state[qb, kb]: 0 skip, 1 partial, 2 full.  kv_idx[qb, :kv_cnt[qb]] / q_idx[kb, :q_cnt[kb]] are
+    the ascending lists of blocks to visit per q-block row / kv-block column.
+    """
+
+    def __init__(self, spec: MaskSpec, Sq: int, Sk: int, block_q: int, block_k: int, device):
+        self.spec, self.Sq, self.Sk, self.block_q, self.block_k = spec, Sq, Sk, block_q, block_k
+        self.nq, self.nk = Sq // block_q, Sk // block_k
+        self.state = torch.empty(self.nq, self.nk, dtype=torch.uint8, device=device)
+        self.kv_cnt = torch.empty(self.nq, dtype=torch.int32, device=device)
+        self.kv_idx = torch.empty(self.nq, self.nk, dtype=torch.int32, device=device)
+        self.q_cnt = torch.empty(self.nk, dtype=torch.int32, device=device)
+        self.q_idx = torch.empty(self.nk, self.nq, dtype=torch.int32, device=device)
+
+    def as_c(self) -> _lib.BlockMapC:
+        return _lib.BlockMapC(self.state.data_ptr(), self.kv_cnt.data_ptr(), self.kv_idx.data_ptr(),
+                              self.q_cnt.data_ptr(), self.q_idx.data_ptr(), self.nq, self.nk,
+                              self.block_q, self.block_k)
+
+    def run_mask(self) -> torch.Tensor:
+        """bool [nq, nk]: tile must run (the quantity the reference's block closures return)."""
+        return self.state != 0
+
+
+_doc_cache: Dict[Tuple[DocIds, str], torch.Tensor] = {}
+_map_cache: Dict[tuple, BlockMap] = {}
+
+
+def doc_ids_on(doc: Optional[DocIds], device) -> Optional[torch.Tensor]:
+    """int32 device copy of the document ids (cached per device)."""
+    if doc is None:
+        return None
+    key = (doc, str(device))
+    t = _doc_cache.get(key)
+    if t is None:
+        t = torch.from_numpy(doc.array.copy()).to(device)
+        _doc_cache[key] = t
+    return t
+
+
+def mask_spec_c(spec: MaskSpec, Sq: int, Sk: int, device) -> _lib.MaskSpecC:
+    """C view of a MaskSpec; validates the document array length."""
+    doc_ptr = None
+    if spec.flags & _lib.MASK_DOC:
+        if spec.doc_ids is None:
+            raise ValueError("document mask without document ids")
+        if len(spec.doc_ids) < max(Sq, Sk):
+            raise ValueError(f"document ids cover {len(spec.doc_ids)} positions, need {max(Sq, Sk)}")
+        doc_ptr = doc_ids_on(spec.doc_ids, device).data_ptr()
+    return _lib.MaskSpecC(spec.flags, spec.window, spec.stride, 0, doc_ptr, doc_ptr)
+
+
+def build_block_map(spec: MaskSpec, Sq: int, Sk: int, block_q: int, block_k: int, device,
+                    cache: bool = True) -> BlockMap:
+    """Runs the GPU block-mask builder (or returns the cached map for this specification)."""
+    device = torch.device(device)
+    key = (spec, Sq, Sk, block_q, block_k, str(device))
+    if cache:
+        hit = _map_cache.get(key)
+        if hit is not None:
+            return hit
+    if Sq % block_q or Sk % block_k:
+        raise ValueError(f"Sq={Sq} / Sk={Sk} not divisible by blocks {block_q} / {block_k}")
+    lib = _lib.load()
+    bm = BlockMap(spec, Sq, Sk, block_q, block_k, device)
+    mc = mask_spec_c(spec, Sq, Sk, device)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    with torch.cuda.device(device):
+        _lib.check(lib.flexattn_build_block_mask(
+            C.byref(mc), Sq, Sk, block_q, block_k, bm.state.data_ptr(), bm.kv_cnt.data_ptr(),
+            bm.kv_idx.data_ptr(), bm.q_cnt.data_ptr(), bm.q_idx.data_ptr(), stream))
+    if cache:
+        _map_cache[key] = bm
+    return bm
+
+
+def create_block_mask(mask_fns, Sq: int, Sk: int, block_q: int, block_k: int, device="cuda") -> BlockMap:
+    """Block map of a ``(mask_fn, block_mask_fn)`` pair (or a MaskSpec) at the given granularity."""
+    spec = mask_fns if isinstance(mask_fns, MaskSpec) else spec_of(mask_fns[0], mask_fns[1])
+    return build_block_map(spec, Sq, Sk, block_q, block_k, device)
+
+
+def spec_of(mask_fn: Optional[Callable], block_mask_fn: Optional[Callable]) -> MaskSpec:
+    """MaskSpec carried by the closures.  Closures not produced by this package's factories cannot
+    be traced into a HIP kernel and are rejected."""
+    spec = None
+    for f in (mask_fn, block_mask_fn):
+        if f is None:
+            continue
+        s = getattr(f, "spec", None)
+        if s is None:
+            raise NotImplementedError(
+                "mask_fn/block_mask_fn must come from flex_attention_tpu_amd.masks factories "
+                "(arbitrary Python closures cannot be compiled into the HIP kernels)")
+        if spec is not None and s != spec:
+            raise ValueError("mask_fn and block_mask_fn describe different masks")
+        spec = s
+    return spec if spec is not None else MaskSpec()
+
+
+def host_block_map(block_mask_fn: Callable, nq: int, nk: int) -> torch.Tensor:
+    """bool [nq, nk] by calling the Python block closure on every tile (CPU; used by tests)."""
+    out = torch.empty(nq, nk, dtype=torch.bool)
+    for qb in range(nq):
+        for kb in range(nk):
+            out[qb, kb] = bool(block_mask_fn(qb, kb))
+    return out

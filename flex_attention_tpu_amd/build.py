@@ -1,0 +1,71 @@
+"""Builds libflexattn.so (gfx950) in-tree with hipcc.  Usage: python -m flex_attention_tpu_amd.build"""
+from __future__ import annotations
+
+import concurrent.futures
+import os
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG_DIR, "csrc")
+INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
+BUILD_DIR = os.path.join(CSRC, "_build")
+LIB_PATH = os.path.join(PKG_DIR, "libflexattn.so")
+
+SOURCES = [
+    "api.hip",
+    "block_mask.hip",
+    "delta.hip",
+    "attn_f32.hip",
+    "fwd_bf16.hip",
+    "bwd_dq_bf16.hip",
+    "bwd_dkv_bf16.hip",
+]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-ffast-math",
+    "-fno-finite-math-only",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+    f"-I{INCLUDE}",
+    f"-I{CSRC}",
+]
+
+
+def _compile(src: str, force: bool) -> str:
+    obj = os.path.join(BUILD_DIR, os.path.splitext(src)[0] + ".o")
+    src_path = os.path.join(CSRC, src)
+    if not force and os.path.exists(obj):
+        deps = [src_path] + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
+        deps.append(os.path.join(INCLUDE, "flexattn.h"))
+        if all(os.path.getmtime(d) <= os.path.getmtime(obj) for d in deps):
+            return obj
+    cmd = [HIPCC, *FLAGS, "-c", src_path, "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
+    warn = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and l.strip())
+    if warn:
+        sys.stderr.write(warn + "\n")
+    return obj
+
+
+def build_library(force: bool = True, jobs: int = 8) -> str:
+    """Compiles every HIP source for gfx950 and links libflexattn.so next to the package."""
+    os.makedirs(BUILD_DIR, exist_ok=True)
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(lambda s: _compile(s, force), SOURCES))
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_library(force="--incremental" not in sys.argv))

@@ -1,0 +1,232 @@
+// C ABI of libflexattn.so: argument validation and dispatch to the gfx950 kernels.
+#include <cstdarg>
+#include <cstdio>
+
+#include "fa_common.hpp"
+#include "launch.hpp"
+
+namespace fa {
+
+static thread_local char g_err[512] = "";
+
+int set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return FLEXATTN_OK;
+}
+
+static ScoreArgs to_args(const flexattn_score_spec& s) {
+  ScoreArgs r;
+  r.kind = s.kind;
+  r.cap = s.cap;
+  r.slope = s.slope;
+  r.mod_q = s.mod_q;
+  r.mod_k = s.mod_k;
+  r.slopes = s.slopes;
+  return r;
+}
+
+static MaskArgs to_args(const flexattn_mask_spec& m) {
+  MaskArgs r;
+  r.flags = m.flags;
+  r.window = m.window;
+  r.stride = m.stride;
+  r.doc_q = m.doc_q;
+  r.doc_k = m.doc_k;
+  return r;
+}
+
+static int check_score(const flexattn_score_spec& s) {
+  switch (s.kind) {
+    case FLEXATTN_SCORE_NONE: return FLEXATTN_OK;
+    case FLEXATTN_SCORE_ALIBI:
+      if (s.slopes == nullptr) return set_error(FLEXATTN_EINVAL, "score ALIBI needs a per-head slopes array");
+      return FLEXATTN_OK;
+    case FLEXATTN_SCORE_SOFTCAP:
+      if (!(s.cap > 0.f)) return set_error(FLEXATTN_EINVAL, "score SOFTCAP needs cap > 0 (got %g)", (double)s.cap);
+      return FLEXATTN_OK;
+    case FLEXATTN_SCORE_ALIBI_TILE:
+      if (s.mod_q <= 0 || s.mod_k <= 0)
+        return set_error(FLEXATTN_EINVAL, "score ALIBI_TILE needs mod_q, mod_k > 0 (got %d, %d)", s.mod_q, s.mod_k);
+      return FLEXATTN_OK;
+  }
+  return set_error(FLEXATTN_EINVAL, "unknown score kind %d", s.kind);
+}
+
+static int check_mask(const flexattn_mask_spec& m) {
+  const int known = FLEXATTN_MASK_CAUSAL | FLEXATTN_MASK_WINDOW | FLEXATTN_MASK_DOC | FLEXATTN_MASK_S2;
+  if (m.flags & ~known) return set_error(FLEXATTN_EINVAL, "unknown mask flags 0x%x", m.flags);
+  if ((m.flags & FLEXATTN_MASK_S2) && (m.flags & (FLEXATTN_MASK_CAUSAL | FLEXATTN_MASK_WINDOW)))
+    return set_error(FLEXATTN_EINVAL, "mask S2 already contains its window and causal terms; do not combine");
+  if ((m.flags & (FLEXATTN_MASK_WINDOW | FLEXATTN_MASK_S2)) && m.window <= 0)
+    return set_error(FLEXATTN_EINVAL, "mask window must be > 0 (got %d)", m.window);
+  if ((m.flags & FLEXATTN_MASK_S2) && m.stride <= 0)
+    return set_error(FLEXATTN_EINVAL, "mask S2 stride must be > 0 (got %d)", m.stride);
+  if ((m.flags & FLEXATTN_MASK_DOC) && (m.doc_q == nullptr || m.doc_k == nullptr))
+    return set_error(FLEXATTN_EINVAL, "mask DOC needs doc_q and doc_k arrays");
+  return FLEXATTN_OK;
+}
+
+static int tile_shape(int pass, int dtype, int D, int* bq, int* bk) {
+  if (dtype == FLEXATTN_F32) {
+    if (D != 64 && D != 128) return set_error(FLEXATTN_ENOTSUP, "fp32: head dim %d not in {64, 128}", D);
+    f32_tile(bq, bk);
+    return FLEXATTN_OK;
+  }
+  if (dtype == FLEXATTN_BF16) {
+    if (D != 128) return set_error(FLEXATTN_ENOTSUP, "bf16: head dim %d not supported (128 only)", D);
+    switch (pass) {
+      case FLEXATTN_PASS_FWD: fwd_bf16_d128_tile(bq, bk); return FLEXATTN_OK;
+      case FLEXATTN_PASS_DQ: bwd_dq_bf16_d128_tile(bq, bk); return FLEXATTN_OK;
+      case FLEXATTN_PASS_DKV: bwd_dkv_bf16_d128_tile(bq, bk); return FLEXATTN_OK;
+    }
+    return set_error(FLEXATTN_EINVAL, "unknown pass %d", pass);
+  }
+  return set_error(FLEXATTN_EINVAL, "unknown dtype %d", dtype);
+}
+
+static int check_shape(int pass, int B, int Hq, int Hkv, int Sq, int Sk, int D, int dtype,
+                       const flexattn_block_map& map) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || Sq <= 0 || Sk <= 0 || D <= 0)
+    return set_error(FLEXATTN_EINVAL, "non-positive dimension (B=%d Hq=%d Hkv=%d Sq=%d Sk=%d D=%d)", B, Hq, Hkv, Sq, Sk, D);
+  if (Hq % Hkv != 0) return set_error(FLEXATTN_EINVAL, "Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
+  int bq = 0, bk = 0;
+  int rc = tile_shape(pass, dtype, D, &bq, &bk);
+  if (rc != FLEXATTN_OK) return rc;
+  if (Sq % bq != 0) return set_error(FLEXATTN_EINVAL, "Sq=%d is not a multiple of the q tile %d", Sq, bq);
+  if (Sk % bk != 0) return set_error(FLEXATTN_EINVAL, "Sk=%d is not a multiple of the kv tile %d", Sk, bk);
+  if (map.state == nullptr) return set_error(FLEXATTN_EINVAL, "block map state is NULL");
+  if (map.block_q != bq || map.block_k != bk || map.nq != Sq / bq || map.nk != Sk / bk)
+    return set_error(FLEXATTN_EINVAL, "block map is %dx%d blocks of %dx%d, kernel needs %dx%d blocks of %dx%d",
+                     map.nq, map.nk, map.block_q, map.block_k, Sq / bq, Sk / bk, bq, bk);
+  if (pass == FLEXATTN_PASS_DKV) {
+    if (map.q_cnt == nullptr || map.q_idx == nullptr) return set_error(FLEXATTN_EINVAL, "block map lacks q_cnt/q_idx");
+  } else {
+    if (map.kv_cnt == nullptr || map.kv_idx == nullptr) return set_error(FLEXATTN_EINVAL, "block map lacks kv_cnt/kv_idx");
+  }
+  return FLEXATTN_OK;
+}
+
+static MapArgs row_view(const flexattn_block_map& m) {
+  MapArgs r;
+  r.state = m.state; r.cnt = m.kv_cnt; r.idx = m.kv_idx; r.nq = m.nq; r.nk = m.nk;
+  return r;
+}
+static MapArgs col_view(const flexattn_block_map& m) {
+  MapArgs r;
+  r.state = m.state; r.cnt = m.q_cnt; r.idx = m.q_idx; r.nq = m.nq; r.nk = m.nk;
+  return r;
+}
+
+static int to_bwd_args(const flexattn_bwd_params* p, int pass, BwdArgs* a) {
+  if (p == nullptr) return set_error(FLEXATTN_EINVAL, "params is NULL");
+  if (!p->q || !p->k || !p->v || !p->dout || !p->l || !p->m || !p->delta)
+    return set_error(FLEXATTN_EINVAL, "a required input pointer is NULL");
+  if (pass == FLEXATTN_PASS_DQ && !p->dq) return set_error(FLEXATTN_EINVAL, "dq is NULL");
+  if (pass == FLEXATTN_PASS_DKV && (!p->dk || !p->dv)) return set_error(FLEXATTN_EINVAL, "dk or dv is NULL");
+  int rc = check_shape(pass, p->B, p->Hq, p->Hkv, p->Sq, p->Sk, p->D, p->dtype, p->map);
+  if (rc != FLEXATTN_OK) return rc;
+  if ((rc = check_score(p->score)) != FLEXATTN_OK) return rc;
+  if ((rc = check_mask(p->mask)) != FLEXATTN_OK) return rc;
+  a->q = p->q; a->k = p->k; a->v = p->v; a->dout = p->dout;
+  a->l = p->l; a->m = p->m; a->delta = p->delta;
+  a->dq = p->dq; a->dk = p->dk; a->dv = p->dv;
+  a->B = p->B; a->Hq = p->Hq; a->Hkv = p->Hkv; a->Sq = p->Sq; a->Sk = p->Sk;
+  a->sm_scale = p->sm_scale;
+  a->score = to_args(p->score);
+  a->mask = to_args(p->mask);
+  a->map = (pass == FLEXATTN_PASS_DKV) ? col_view(p->map) : row_view(p->map);
+  return FLEXATTN_OK;
+}
+
+}  // namespace fa
+
+using namespace fa;
+
+extern "C" {
+
+int flexattn_version(void) { return FLEXATTN_VERSION; }
+
+const char* flexattn_last_error_string(void) { return g_err; }
+
+int flexattn_tile_shape(int32_t pass, int32_t dtype, int32_t D, int32_t* block_q, int32_t* block_k) {
+  if (block_q == nullptr || block_k == nullptr) return set_error(FLEXATTN_EINVAL, "block_q/block_k is NULL");
+  if (pass < FLEXATTN_PASS_FWD || pass > FLEXATTN_PASS_DKV) return set_error(FLEXATTN_EINVAL, "unknown pass %d", pass);
+  int bq = 0, bk = 0;
+  int rc = tile_shape(pass, dtype, D, &bq, &bk);
+  if (rc != FLEXATTN_OK) return rc;
+  *block_q = bq;
+  *block_k = bk;
+  return FLEXATTN_OK;
+}
+
+int flexattn_build_block_mask(const flexattn_mask_spec* mask, int32_t Sq, int32_t Sk, int32_t block_q,
+                              int32_t block_k, uint8_t* state, int32_t* kv_cnt, int32_t* kv_idx,
+                              int32_t* q_cnt, int32_t* q_idx, void* stream) {
+  if (mask == nullptr || state == nullptr) return set_error(FLEXATTN_EINVAL, "mask or state is NULL");
+  if (Sq <= 0 || Sk <= 0 || block_q <= 0 || block_k <= 0)
+    return set_error(FLEXATTN_EINVAL, "non-positive size (Sq=%d Sk=%d block_q=%d block_k=%d)", Sq, Sk, block_q, block_k);
+  if (Sq % block_q != 0 || Sk % block_k != 0)
+    return set_error(FLEXATTN_EINVAL, "Sq=%d / Sk=%d not divisible by blocks %d / %d", Sq, Sk, block_q, block_k);
+  if ((kv_cnt == nullptr) != (kv_idx == nullptr) || (q_cnt == nullptr) != (q_idx == nullptr))
+    return set_error(FLEXATTN_EINVAL, "count and index arrays must be given in pairs");
+  int rc = check_mask(*mask);
+  if (rc != FLEXATTN_OK) return rc;
+  return build_block_mask(to_args(*mask), Sq, Sk, block_q, block_k, state, kv_cnt, kv_idx, q_cnt, q_idx,
+                          static_cast<hipStream_t>(stream));
+}
+
+int flexattn_fwd(const flexattn_fwd_params* p, void* stream) {
+  if (p == nullptr) return set_error(FLEXATTN_EINVAL, "params is NULL");
+  if (!p->q || !p->k || !p->v || !p->o) return set_error(FLEXATTN_EINVAL, "q, k, v or o is NULL");
+  if ((p->l == nullptr) != (p->m == nullptr)) return set_error(FLEXATTN_EINVAL, "l and m must both be given or both NULL");
+  int rc = check_shape(FLEXATTN_PASS_FWD, p->B, p->Hq, p->Hkv, p->Sq, p->Sk, p->D, p->dtype, p->map);
+  if (rc != FLEXATTN_OK) return rc;
+  if ((rc = check_score(p->score)) != FLEXATTN_OK) return rc;
+  if ((rc = check_mask(p->mask)) != FLEXATTN_OK) return rc;
+  FwdArgs a;
+  a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.l = p->l; a.m = p->m;
+  a.B = p->B; a.Hq = p->Hq; a.Hkv = p->Hkv; a.Sq = p->Sq; a.Sk = p->Sk;
+  a.sm_scale = p->sm_scale;
+  a.score = to_args(p->score);
+  a.mask = to_args(p->mask);
+  a.map = row_view(p->map);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (p->dtype == FLEXATTN_BF16) return fwd_bf16_d128(a, s);
+  return fwd_f32(a, p->D, s);
+}
+
+int flexattn_bwd_delta(const void* o, const void* dout, float* delta, int64_t rows, int32_t D, int32_t dtype,
+                       void* stream) {
+  if (!o || !dout || !delta) return set_error(FLEXATTN_EINVAL, "o, dout or delta is NULL");
+  if (rows <= 0) return set_error(FLEXATTN_EINVAL, "rows=%lld must be positive", (long long)rows);
+  return bwd_delta(o, dout, delta, rows, D, dtype, static_cast<hipStream_t>(stream));
+}
+
+int flexattn_bwd_dq(const flexattn_bwd_params* p, void* stream) {
+  BwdArgs a;
+  int rc = to_bwd_args(p, FLEXATTN_PASS_DQ, &a);
+  if (rc != FLEXATTN_OK) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (p->dtype == FLEXATTN_BF16) return bwd_dq_bf16_d128(a, s);
+  return bwd_dq_f32(a, p->D, s);
+}
+
+int flexattn_bwd_dkv(const flexattn_bwd_params* p, void* stream) {
+  BwdArgs a;
+  int rc = to_bwd_args(p, FLEXATTN_PASS_DKV, &a);
+  if (rc != FLEXATTN_OK) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (p->dtype == FLEXATTN_BF16) return bwd_dkv_bf16_d128(a, s);
+  return bwd_dkv_f32(a, p->D, s);
+}
+
+}  // extern "C"

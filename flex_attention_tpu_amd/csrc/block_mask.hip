@@ -1,0 +1,78 @@
+// Block-mask builder: one launch turns a mask specification into the tile state map and the
+// compacted per-row / per-column visit lists that the attention kernels walk.
+#include "fa_common.hpp"
+#include "launch.hpp"
+
+namespace fa {
+
+// State of tile (qb, kb): 0 skip, 1 partial, 2 full.  `run` is the AND of the block predicates
+// of the flags set: causal k_start <= q_end; window q_start - k_end < window; document: the id
+// ranges read at the block ends overlap (ids are non-decreasing); S2: k_start <= q_end.
+__device__ __forceinline__ int tile_state(const MaskArgs& mk, int qb, int kb, int bq, int bk) {
+  const int q_start = qb * bq, q_end = q_start + bq - 1;
+  const int k_start = kb * bk, k_end = k_start + bk - 1;
+  bool run = true, full = true;
+  if (mk.flags & FLEXATTN_MASK_S2) {
+    run = k_start <= q_end;
+    full = (k_end <= q_start) && (q_end - k_start < mk.window);
+  } else {
+    if (mk.flags & FLEXATTN_MASK_CAUSAL) {
+      run = run && (k_start <= q_end);
+      full = full && (k_end <= q_start);
+    }
+    if (mk.flags & FLEXATTN_MASK_WINDOW) {
+      run = run && (q_start - k_end < mk.window);
+      full = full && (q_end - k_start < mk.window);
+    }
+  }
+  if (mk.flags & FLEXATTN_MASK_DOC) {
+    const int qmin = mk.doc_q[q_start], qmax = mk.doc_q[q_end];
+    const int kmin = mk.doc_k[k_start], kmax = mk.doc_k[k_end];
+    const int lo = qmin > kmin ? qmin : kmin;
+    const int hi = qmax < kmax ? qmax : kmax;
+    run = run && (lo <= hi);
+    full = full && (qmin == qmax) && (kmin == kmax) && (qmin == kmin);
+  }
+  return run ? (full ? 2 : 1) : 0;
+}
+
+// Work-groups [0, nq) own one q-block row each: write its states and its ascending kv list.
+// Work-groups [nq, nq + nk) own one kv-block column each: write its ascending q list.
+__global__ __launch_bounds__(64) void block_mask_kernel(MaskArgs mk, int nq, int nk, int bq, int bk,
+                                                        uint8_t* state, int* kv_cnt, int* kv_idx,
+                                                        int* q_cnt, int* q_idx) {
+  const int lane = threadIdx.x;
+  const bool is_row = (int)blockIdx.x < nq;
+  const int major = is_row ? blockIdx.x : blockIdx.x - nq;
+  const int n_minor = is_row ? nk : nq;
+  int* cnt = is_row ? kv_cnt : q_cnt;
+  int* idx = is_row ? kv_idx : q_idx;
+  int total = 0;
+  for (int base = 0; base < n_minor; base += 64) {
+    const int minor = base + lane;
+    int st = 0;
+    if (minor < n_minor) {
+      st = is_row ? tile_state(mk, major, minor, bq, bk) : tile_state(mk, minor, major, bq, bk);
+      if (is_row) state[(size_t)major * nk + minor] = (uint8_t)st;
+    }
+    const unsigned long long ballot = __ballot(st != 0);
+    if (idx != nullptr && st != 0) {
+      const int pos = total + __popcll(ballot & ((1ull << lane) - 1ull));
+      idx[(size_t)major * n_minor + pos] = minor;
+    }
+    total += __popcll(ballot);
+  }
+  if (cnt != nullptr && lane == 0) cnt[major] = total;
+}
+
+int build_block_mask(const MaskArgs& mask, int Sq, int Sk, int block_q, int block_k, uint8_t* state,
+                     int* kv_cnt, int* kv_idx, int* q_cnt, int* q_idx, hipStream_t stream) {
+  const int nq = Sq / block_q, nk = Sk / block_k;
+  const bool want_cols = q_cnt != nullptr;
+  const int grid = nq + (want_cols ? nk : 0);
+  hipLaunchKernelGGL(block_mask_kernel, dim3(grid), dim3(64), 0, stream, mask, nq, nk, block_q, block_k,
+                     state, kv_cnt, kv_idx, q_cnt, q_idx);
+  return check_launch("flexattn_build_block_mask");
+}
+
+}  // namespace fa

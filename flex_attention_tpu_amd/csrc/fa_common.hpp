@@ -1,0 +1,206 @@
+// Shared device-side definitions for the gfx950 flex-attention kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "flexattn.h"
+
+namespace fa {
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kNegInf = -__builtin_huge_valf();
+
+// Kernel-side views of the C ABI structs (pointers already typed).
+struct ScoreArgs {
+  int kind;
+  float cap;
+  float slope;
+  int mod_q, mod_k;
+  const float* slopes;
+};
+struct MaskArgs {
+  int flags;
+  int window;
+  int stride;
+  const int* doc_q;
+  const int* doc_k;
+};
+// One direction of the block map: for "major" block r, idx[r*n_minor + t], t < cnt[r], are the
+// minor blocks to visit; state is always indexed [q block][kv block].
+struct MapArgs {
+  const uint8_t* state;
+  const int* cnt;
+  const int* idx;
+  int nq, nk;
+};
+
+struct FwdArgs {
+  const void* q; const void* k; const void* v;
+  void* o; float* l; float* m;
+  int B, Hq, Hkv, Sq, Sk;
+  float sm_scale;
+  ScoreArgs score;
+  MaskArgs mask;
+  MapArgs map;
+};
+
+struct BwdArgs {
+  const void* q; const void* k; const void* v; const void* dout;
+  const float* l; const float* m; const float* delta;
+  void* dq; void* dk; void* dv;
+  int B, Hq, Hkv, Sq, Sk;
+  float sm_scale;
+  ScoreArgs score;
+  MaskArgs mask;
+  MapArgs map;
+};
+
+// ------------------------------------------------------------------------------------------
+// MFMA wrappers.  v_mfma_f32_32x32x16_bf16: A is 32(M) x 16(K), B is 16(K) x 32(N).
+// Lane L supplies A[L%32][8*(L/32) .. +8) and B[8*(L/32) .. +8)[L%32]; it receives
+// C[8*(i/4) + 4*(L/32) + i%4][L%32] in accumulator element i.
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// Row index inside a 32x32 accumulator tile held by (half = lane/32, element i).
+__device__ __forceinline__ constexpr int acc_row(int i, int half) { return 8 * (i >> 2) + 4 * half + (i & 3); }
+
+// Transposing LDS read: inside each group of 16 lanes, lane i receives elements j = 0..3 taken
+// from the 8-byte chunk addressed by lane 4*j + i/4, at position i%4.
+__device__ __forceinline__ s16x4 lds_read_tr16(const bf16_t* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (s16x4 __attribute__((address_space(3)))*)(__attribute__((address_space(3))) void*)(p));
+}
+
+__device__ __forceinline__ bf16x8 join_tr(s16x4 lo, s16x4 hi) {
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  s16x8 r = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8, r);
+}
+
+// Reductions across the two 32-lane halves of a wave (lane L with lane L^32).
+// v_permlane32_swap exchanges lanes 32-63 of its first register with lanes 0-31 of its second;
+// fed two copies of x, every lane ends up holding both halves' values, one in each register, and
+// max / sum are symmetric in them.  Written as inline asm: through the compiler builtin the two
+// results were folded into one value.  The s_nop cover the VALU-write -> permlane read hazard the
+// compiler would otherwise pad itself.
+__device__ __forceinline__ void half_pair(float x, float& r0, float& r1) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  r0 = a;
+  r1 = b;
+}
+__device__ __forceinline__ float half_max(float x) {
+  float r0, r1;
+  half_pair(x, r0, r1);
+  return fmaxf(r0, r1);
+}
+__device__ __forceinline__ float half_sum(float x) {
+  float r0, r1;
+  half_pair(x, r0, r1);
+  return r0 + r1;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+__device__ __forceinline__ bf16x2 pack_bf16(float a, float b) {
+  f32x2 v = {a, b};
+  return __builtin_convertvector(v, bf16x2);
+}
+
+// ------------------------------------------------------------------------------------------
+// Element mask, evaluated only on tiles the block map marks partial.
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ bool keep_elem(const MaskArgs& mk, int i, int j, int doc_i, int doc_j) {
+  bool keep = true;
+  if (mk.flags & FLEXATTN_MASK_S2) {
+    int d = i - j;
+    keep = (d >= 0) && ((d < mk.window) || (j % mk.stride == 0));
+  } else {
+    if (mk.flags & FLEXATTN_MASK_CAUSAL) keep = keep && (i >= j);
+    if (mk.flags & FLEXATTN_MASK_WINDOW) keep = keep && ((i - j) < mk.window);
+  }
+  if (mk.flags & FLEXATTN_MASK_DOC) keep = keep && (doc_i == doc_j);
+  return keep;
+}
+
+// ------------------------------------------------------------------------------------------
+// Score modification.  `raw` is <q_i, k_j>.  to_log2() returns the modified logit multiplied by
+// log2(e) so that probabilities are exp2(t - lse2).  dfactor() returns d(s')/d(raw) given the
+// already transformed logit t (log2 domain).
+// ------------------------------------------------------------------------------------------
+template <int KIND>
+struct ScoreMod {
+  float c2;      // sm_scale * log2e
+  float scale;   // sm_scale
+  float a0, a1;  // kind-specific
+  int mod_q, mod_k;
+
+  __device__ __forceinline__ void init(const ScoreArgs& s, float sm_scale, int head) {
+    scale = sm_scale;
+    c2 = sm_scale * kLog2e;
+    mod_q = s.mod_q;
+    mod_k = s.mod_k;
+    if (KIND == FLEXATTN_SCORE_ALIBI) {
+      a0 = s.slopes[head] * kLog2e;
+    } else if (KIND == FLEXATTN_SCORE_ALIBI_TILE) {
+      a0 = s.slope * kLog2e;
+    } else if (KIND == FLEXATTN_SCORE_SOFTCAP) {
+      a0 = 2.0f * kLog2e * sm_scale / s.cap;  // exponent scale for exp(2 s / cap)
+      a1 = s.cap * kLog2e;                    // cap in the log2 domain
+    }
+  }
+
+  __device__ __forceinline__ float to_log2(float raw, int i, int j) const {
+    if (KIND == FLEXATTN_SCORE_NONE) {
+      return raw * c2;
+    } else if (KIND == FLEXATTN_SCORE_ALIBI) {
+      return __builtin_fmaf(raw, c2, a0 * (float)(j - i));
+    } else if (KIND == FLEXATTN_SCORE_ALIBI_TILE) {
+      int d = (i % mod_q) - (j % mod_k);
+      d = d < 0 ? -d : d;
+      return __builtin_fmaf(raw, c2, -a0 * (float)d);
+    } else {
+      // cap*tanh(x) = cap*(1 - 2/(1 + exp(2x))), x = sm_scale*raw/cap
+      float e = fast_exp2(raw * a0);
+      float r = fast_rcp(1.0f + e);
+      return __builtin_fmaf(-2.0f * a1, r, a1);
+    }
+  }
+
+  // d(s')/d(raw) in natural units, from the log2-domain modified logit t.
+  __device__ __forceinline__ float dfactor(float t) const {
+    if (KIND == FLEXATTN_SCORE_SOFTCAP) {
+      float y = t * fast_rcp(a1);  // tanh
+      return scale * (1.0f - y * y);
+    }
+    return scale;
+  }
+};
+
+// XCD-aware work-group remap: consecutive hardware work-group ids go round-robin to the 8 XCDs,
+// each with a private L2.  Give every XCD a contiguous range of logical ids so that tiles sharing
+// one head's K/V run on the same XCD.
+__device__ __forceinline__ int xcd_remap(int wg, int n_wg) {
+  constexpr int kXcd = 8;
+  if (n_wg % kXcd != 0) return wg;
+  return (wg % kXcd) * (n_wg / kXcd) + wg / kXcd;
+}
+
+}  // namespace fa

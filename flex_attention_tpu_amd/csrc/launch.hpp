@@ -1,0 +1,34 @@
+// Host-side helpers shared by the launch code: error recording and kernel entry declarations.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "fa_common.hpp"
+
+namespace fa {
+
+// Records a printf-style message for flexattn_last_error_string() and returns `code`.
+int set_error(int code, const char* fmt, ...);
+
+// Returns FLEXATTN_OK, or records hipGetLastError() under `what`.
+int check_launch(const char* what);
+
+// bf16, head dim 128 (MFMA kernels)
+int fwd_bf16_d128(const FwdArgs& a, hipStream_t stream);
+void fwd_bf16_d128_tile(int* bq, int* bk);
+int bwd_dq_bf16_d128(const BwdArgs& a, hipStream_t stream);
+void bwd_dq_bf16_d128_tile(int* bq, int* bk);
+int bwd_dkv_bf16_d128(const BwdArgs& a, hipStream_t stream);
+void bwd_dkv_bf16_d128_tile(int* bq, int* bk);
+
+// fp32, head dim 64 or 128 (FMA kernels, exact-arithmetic path)
+int fwd_f32(const FwdArgs& a, int D, hipStream_t stream);
+int bwd_dq_f32(const BwdArgs& a, int D, hipStream_t stream);
+int bwd_dkv_f32(const BwdArgs& a, int D, hipStream_t stream);
+void f32_tile(int* bq, int* bk);
+
+int bwd_delta(const void* o, const void* dout, float* delta, int64_t rows, int D, int dtype, hipStream_t stream);
+
+int build_block_mask(const MaskArgs& mask, int Sq, int Sk, int block_q, int block_k, uint8_t* state,
+                     int* kv_cnt, int* kv_idx, int* q_cnt, int* q_idx, hipStream_t stream);
+
+}  // namespace fa

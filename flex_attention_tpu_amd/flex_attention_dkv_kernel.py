@@ -1,0 +1,37 @@
+"""dk/dv backward entry point, same name and argument list as the reference's
+``flash_attention_bwd_dkv`` (flex_attention_dkv_kernel.py:23-174), plus the ``mask_fn`` /
+``block_mask_fn`` keywords of its mask-aware twin (flash_attention_dkv_bwd.py:27-48)."""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._common import check_blocks, check_qkv, check_rows, kernel_block_map, resolve_mask, stream_of
+from .flex_attention_dq_bwd import bwd_params
+
+
+def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=None, block_q, block_q_major,
+                            block_k_major, block_k, sm_scale, causal, debug, score_fn=None, mask_fn=None,
+                            block_mask_fn=None):
+    """(dk, dv): dv = P^T do, dk = dS^T * d(score)/dk with P recomputed from (l, m) and
+    dS = P (dP - di) (flex_attention_dkv_kernel.py:237-272).  With grouped KV heads the gradients
+    of all query heads of a group are summed inside the kernel.  ``causal`` is honoured
+    (the reference's north-star file ignores it; its mask-aware twin gets the same effect from
+    ``mask_fn``)."""
+    if ab is not None:
+        raise NotImplementedError("additive bias `ab` is not supported")
+    B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v, do)
+    for name, t in (("l", l), ("m", m), ("di", di)):
+        check_rows(name, t, B, Hq, Sq, q.device)
+    check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k,
+                 block_q_major=block_q_major)
+    spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk)
+    bm = kernel_block_map(_lib.PASS_DKV, spec, q, Sq, Sk, D)
+    dk = torch.empty_like(k)
+    dv = torch.empty_like(v)
+    p = bwd_params(q, k, v, l, m, do, di, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dk=dk, dv=dv)
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.load().flexattn_bwd_dkv(C.byref(p), stream_of(q)))
+    return dk, dv

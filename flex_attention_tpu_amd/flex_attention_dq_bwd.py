@@ -1,0 +1,61 @@
+"""dq backward entry point, same name and argument list as the reference's
+``flex_attention_bwd_dq`` (flex_attention_dq_bwd.py:114-267), on torch tensors."""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._common import (check_blocks, check_qkv, check_rows, dtype_code, kernel_block_map, resolve_mask,
+                      score_spec_c, stream_of)
+from .block_mask import mask_spec_c
+
+
+def compute_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
+    """d = sum(o * do, axis=-1) in float32, [B, H, Sq] -- the reduction the reference leaves to the
+    caller (flex_attention_dq_bwd.py:932, flash_attention_dkv_bwd.py:925), as one HIP launch."""
+    if o.shape != do.shape or o.dtype != do.dtype or o.ndim != 4:
+        raise ValueError("o and do must be rank-4 tensors of the same shape and dtype")
+    if not (o.is_cuda and o.is_contiguous() and do.is_contiguous()):
+        raise ValueError("o and do must be contiguous GPU tensors")
+    B, H, S, D = o.shape
+    d = torch.empty(B, H, S, dtype=torch.float32, device=o.device)
+    with torch.cuda.device(o.device):
+        _lib.check(_lib.load().flexattn_bwd_delta(o.data_ptr(), do.data_ptr(), d.data_ptr(), B * H * S, D,
+                                                  dtype_code(o), stream_of(o)))
+    return d
+
+
+def bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, mod_q, mod_k, dq=None, dk=None, dv=None):
+    B, Hq, Sq, D = q.shape
+    _, Hkv, Sk, _ = k.shape
+    return _lib.BwdParamsC(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), l.data_ptr(), m.data_ptr(), d.data_ptr(),
+        dq.data_ptr() if dq is not None else None,
+        dk.data_ptr() if dk is not None else None, dv.data_ptr() if dv is not None else None,
+        B, Hq, Hkv, Sq, Sk, D, dtype_code(q), float(sm_scale),
+        score_spec_c(score_fn, Hq, q.device, mod_q, mod_k), mask_spec_c(spec, Sq, Sk, q.device), bm.as_c())
+
+
+def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, block_q, block_k_major,
+                          block_k, sm_scale, debug, score_fn=None, mask_fn=None, block_mask_fn=None,
+                          causal=False):
+    """dq = sum_j dS_ij * d(score)/dq, with P_ij = exp(S_ij - m_i) / l_i recomputed from the saved
+    statistics, dP = do v^T, dS = P (dP - d) (flex_attention_dq_bwd.py:340-378).  ``o`` is only
+    shape-checked, as in the reference (:163); ``d`` is the caller's delta (see compute_delta)."""
+    if ab is not None:
+        raise NotImplementedError("additive bias `ab` is not supported")
+    B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v, do)
+    if o is not None and tuple(o.shape) != tuple(q.shape):
+        raise ValueError(f"o has shape {tuple(o.shape)}, expected {tuple(q.shape)}")
+    for name, t in (("l", l), ("m", m), ("d", d)):
+        check_rows(name, t, B, Hq, Sq, q.device)
+    check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k)
+    spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk)
+    bm = kernel_block_map(_lib.PASS_DQ, spec, q, Sq, Sk, D)
+    dq = torch.empty_like(q)
+    p = bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dq=dq)
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.load().flexattn_bwd_dq(C.byref(p), stream_of(q)))
+    return dq

@@ -1,0 +1,51 @@
+"""Flex-attention forward entry point, same name and argument list as the reference's
+``_flex_attention_impl`` (flex_attention_kernel.py:66-193), on torch tensors.
+
+The reference builds a Pallas grid and traces ``score_fn`` / ``mask_fn`` / ``block_mask_fn`` into
+the kernel; here the closures' ``.spec`` selects a compiled HIP functor, the block map is built on
+the GPU once per mask, and one ``flexattn_fwd`` launch does the rest on the current stream.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._common import (check_blocks, check_qkv, dtype_code, kernel_block_map, resolve_mask, score_spec_c,
+                      stream_of)
+from .block_mask import mask_spec_c
+
+
+def _flex_attention_impl(q, k, v, ab, segment_ids, save_residuals, causal, sm_scale, block_b, block_q,
+                         block_k_major, block_k, debug, block_mask_fn, mask_fn, score_fn):
+    """Returns ``o`` (q.dtype) or ``(o, l, m)`` with float32 ``l, m`` of shape [B, H, Sq].
+
+    Semantics (flex_attention_kernel.py:248-319): S = score_mod(sm_scale * q k^T); masked
+    positions are excluded; m = rowmax S, l = sum exp(S - m), o = exp(S - m) v / l.
+    Unlike the reference's flex forward, ``causal=True`` is honoured (ANDed with ``mask_fn``), as
+    flash_attention_fwd_ref.py:78-86 and the dense reference do.
+    """
+    if ab is not None:
+        raise NotImplementedError("additive bias `ab` is not supported")
+    B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v)
+    check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k)
+    spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk)
+    bm = kernel_block_map(_lib.PASS_FWD, spec, q, Sq, Sk, D)
+    o = torch.empty_like(q)
+    l = m = None
+    if save_residuals:
+        l = torch.empty(B, Hq, Sq, dtype=torch.float32, device=q.device)
+        m = torch.empty(B, Hq, Sq, dtype=torch.float32, device=q.device)
+    p = _lib.FwdParamsC(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+        l.data_ptr() if l is not None else None, m.data_ptr() if m is not None else None,
+        B, Hq, Hkv, Sq, Sk, D, dtype_code(q), float(sm_scale),
+        score_spec_c(score_fn, Hq, q.device, block_q or 1, block_k or 1),
+        mask_spec_c(spec, Sq, Sk, q.device), bm.as_c())
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.load().flexattn_fwd(C.byref(p), stream_of(q)))
+    if debug:
+        print(f"[flexattn_fwd] B={B} Hq={Hq} Hkv={Hkv} Sq={Sq} Sk={Sk} D={D} dtype={q.dtype} "
+              f"mask_flags={spec.flags} tiles_run={int((bm.state != 0).sum())}/{bm.nq * bm.nk}")
+    return (o, l, m) if save_residuals else o

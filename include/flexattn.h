@@ -1,0 +1,155 @@
+/*
+ * flexattn.h -- C ABI of libflexattn.so: flex-attention forward, dq backward, dk/dv backward,
+ * delta pre-pass and block-mask builder for AMD MI355X (gfx950), hand-written HIP.
+ *
+ * The reference project has no FFI: its boundary is three Python functions that hand arrays to
+ * `pl.pallas_call`.  Each entry point below replaces one of those device hand-offs; the citation
+ * next to it names the reference call site (paths relative to the reference repository).
+ *
+ * Conventions
+ *  - All tensors are contiguous row-major [B, H, S, D] device memory owned by the caller.
+ *    q/o/do/dq have Hq heads, k/v/dk/dv have Hkv heads, Hq % Hkv == 0 (kv head = h / (Hq/Hkv)).
+ *  - l, m, delta are float32 [B, Hq, Sq].
+ *  - Every function returns FLEXATTN_OK or a negative error code, never throws or aborts, and
+ *    records a message readable with flexattn_last_error_string() (thread-local).
+ *  - Launches are asynchronous on `stream` (a hipStream_t passed as void*; NULL = default stream).
+ *  - Entry points are re-entrant and keep no mutable global state.
+ */
+#ifndef FLEXATTN_H_
+#define FLEXATTN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FLEXATTN_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* status codes */
+#define FLEXATTN_OK 0
+#define FLEXATTN_EINVAL (-22)   /* bad argument (null pointer, bad enum, non-divisible shape) */
+#define FLEXATTN_ENOTSUP (-95)  /* valid request this build has no kernel for */
+#define FLEXATTN_ELAUNCH (-5)   /* HIP reported a launch error */
+
+/* element types */
+#define FLEXATTN_BF16 0
+#define FLEXATTN_F32 1
+
+/* score modifications: s' = f(sm_scale * <q_i, k_j>, b, h, i, j) with global token indices.
+ * Reference: scores.py:3-18 (tile callables traced into the kernels at
+ * flex_attention_kernel.py:248-255). */
+#define FLEXATTN_SCORE_NONE 0
+#define FLEXATTN_SCORE_ALIBI 1      /* s + slopes[h] * (j - i)                     */
+#define FLEXATTN_SCORE_SOFTCAP 2    /* cap * tanh(s / cap)            scores.py:13-18 */
+#define FLEXATTN_SCORE_ALIBI_TILE 3 /* s - slope * |i % mod_q - j % mod_k|  scores.py:3-11 */
+
+typedef struct flexattn_score_spec {
+  int32_t kind;
+  float cap;           /* SOFTCAP */
+  float slope;         /* ALIBI_TILE */
+  int32_t mod_q;       /* ALIBI_TILE */
+  int32_t mod_k;       /* ALIBI_TILE */
+  int32_t reserved;
+  const float* slopes; /* ALIBI: device float32 [Hq] */
+} flexattn_score_spec;
+
+/* element masks (keep = attend), AND-composed.  Reference: masks.py:15-16 (causal),
+ * :45-59 (window: i - j < window, no causal bound of its own), :105-110 (document),
+ * :146-158 (S2: (0 <= i-j < window) | (j % stride == 0 & i >= j); excludes CAUSAL/WINDOW). */
+#define FLEXATTN_MASK_CAUSAL 1
+#define FLEXATTN_MASK_WINDOW 2
+#define FLEXATTN_MASK_DOC 4
+#define FLEXATTN_MASK_S2 8
+
+typedef struct flexattn_mask_spec {
+  int32_t flags;
+  int32_t window;
+  int32_t stride;
+  int32_t reserved;
+  const int32_t* doc_q; /* DOC: device int32 [Sq] */
+  const int32_t* doc_k; /* DOC: device int32 [Sk] (may equal doc_q) */
+} flexattn_mask_spec;
+
+/* Block-sparsity map at (block_q x block_k) granularity, as produced by
+ * flexattn_build_block_mask.  state: 0 = skip, 1 = partial (element mask applied),
+ * 2 = full (no element is masked).  kv_idx[qb*nk + t], t < kv_cnt[qb], lists ascending the kv
+ * blocks with state != 0 of q block qb; q_idx[kb*nq + t], t < q_cnt[kb], the q blocks of kv block kb. */
+typedef struct flexattn_block_map {
+  const uint8_t* state; /* [nq, nk] */
+  const int32_t* kv_cnt; /* [nq] */
+  const int32_t* kv_idx; /* [nq, nk] */
+  const int32_t* q_cnt;  /* [nk] */
+  const int32_t* q_idx;  /* [nk, nq] */
+  int32_t nq, nk, block_q, block_k;
+} flexattn_block_map;
+
+typedef struct flexattn_fwd_params {
+  const void* q; const void* k; const void* v; /* in  */
+  void* o;                                      /* out [B,Hq,Sq,D], dtype of q */
+  float* l; float* m;                           /* out [B,Hq,Sq] or both NULL   */
+  int32_t B, Hq, Hkv, Sq, Sk, D;
+  int32_t dtype;
+  float sm_scale;
+  flexattn_score_spec score;
+  flexattn_mask_spec mask;
+  flexattn_block_map map; /* granularity must equal flexattn_tile_shape(FLEXATTN_PASS_FWD, ...) */
+} flexattn_fwd_params;
+
+typedef struct flexattn_bwd_params {
+  const void* q; const void* k; const void* v; const void* dout;
+  const float* l; const float* m; const float* delta; /* [B,Hq,Sq] */
+  void* dq;            /* out of flexattn_bwd_dq  [B,Hq,Sq,D]  */
+  void* dk; void* dv;  /* out of flexattn_bwd_dkv [B,Hkv,Sk,D] */
+  int32_t B, Hq, Hkv, Sq, Sk, D;
+  int32_t dtype;
+  float sm_scale;
+  flexattn_score_spec score;
+  flexattn_mask_spec mask;
+  flexattn_block_map map; /* granularity of the pass being launched */
+} flexattn_bwd_params;
+
+#define FLEXATTN_PASS_FWD 0
+#define FLEXATTN_PASS_DQ 1
+#define FLEXATTN_PASS_DKV 2
+
+int flexattn_version(void);
+
+/* Message for the calling thread's most recent non-OK return ("" if none). */
+const char* flexattn_last_error_string(void);
+
+/* Tile granularity (block_q, block_k) the kernels of `pass` expect of the block map for this
+ * dtype and head dimension. */
+int flexattn_tile_shape(int32_t pass, int32_t dtype, int32_t D, int32_t* block_q, int32_t* block_k);
+
+/* Block-mask builder.  Replaces the per-grid-step evaluation of the `block_mask_fn` closures
+ * (masks.py:20-28, 63-81, 113-139, 161-177; consumed at flex_attention_kernel.py:97-106,231-236,
+ * flex_attention_dq_bwd.py:167-177,318-323, flash_attention_dkv_bwd.py:76-85,224-230).
+ * `state != 0` equals the AND of the reference closures of the flags set, bit for bit.
+ * All five output arrays are caller-allocated device memory of the sizes given at
+ * flexattn_block_map; any of kv_cnt/kv_idx/q_cnt/q_idx may be NULL in pairs. */
+int flexattn_build_block_mask(const flexattn_mask_spec* mask, int32_t Sq, int32_t Sk,
+                              int32_t block_q, int32_t block_k, uint8_t* state,
+                              int32_t* kv_cnt, int32_t* kv_idx, int32_t* q_cnt, int32_t* q_idx,
+                              void* stream);
+
+/* Forward.  Replaces the pallas_call in _flex_attention_impl (flex_attention_kernel.py:173-187). */
+int flexattn_fwd(const flexattn_fwd_params* p, void* stream);
+
+/* delta_i = sum_c o_ic * do_ic in float32.  Replaces the caller-side reduction at
+ * flex_attention_dq_bwd.py:932 and flash_attention_dkv_bwd.py:925.  rows = B*Hq*Sq. */
+int flexattn_bwd_delta(const void* o, const void* dout, float* delta, int64_t rows, int32_t D,
+                       int32_t dtype, void* stream);
+
+/* dq backward.  Replaces the pallas_call in flex_attention_bwd_dq (flex_attention_dq_bwd.py:251-265). */
+int flexattn_bwd_dq(const flexattn_bwd_params* p, void* stream);
+
+/* dk/dv backward.  Replaces the pallas_call in flash_attention_bwd_dkv
+ * (flex_attention_dkv_kernel.py:158-172; mask-aware twin flash_attention_dkv_bwd.py:164-178). */
+int flexattn_bwd_dkv(const flexattn_bwd_params* p, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLEXATTN_H_ */
