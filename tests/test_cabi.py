@@ -1,0 +1,80 @@
+"""The C-ABI shared library loads, exports every symbol include/flexattn.h declares, and rejects
+bad arguments with error codes (no GPU work is launched by these tests)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from flex_attention_tpu_amd import _lib
+
+HEADER = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "flexattn.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(flexattn_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(lib):
+    names = _declared_symbols()
+    assert len(names) >= 8
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in flexattn.h but not exported"
+    assert sorted(_lib.EXPORTS) == names
+
+
+def test_version_matches_header(lib):
+    ver = int(re.search(r"#define FLEXATTN_VERSION (\d+)", open(HEADER).read()).group(1))
+    assert lib.flexattn_version() == ver
+
+
+def test_struct_sizes_follow_c_layout():
+    # pointers 8-byte aligned, no surprises in the ctypes mirrors
+    assert C.sizeof(_lib.ScoreSpecC) == 32
+    assert C.sizeof(_lib.MaskSpecC) == 32
+    assert C.sizeof(_lib.BlockMapC) == 56
+    assert C.sizeof(_lib.FwdParamsC) == 6 * 8 + 8 * 4 + 32 + 32 + 56
+    assert C.sizeof(_lib.BwdParamsC) == 10 * 8 + 8 * 4 + 32 + 32 + 56
+
+
+def test_tile_shapes(lib):
+    assert _lib.tile_shape(_lib.PASS_FWD, _lib.BF16, 128)[0] % 64 == 0
+    for p in (_lib.PASS_FWD, _lib.PASS_DQ, _lib.PASS_DKV):
+        bq, bk = _lib.tile_shape(p, _lib.F32, 64)
+        assert bq > 0 and bk > 0
+    with pytest.raises(NotImplementedError):
+        _lib.tile_shape(_lib.PASS_FWD, _lib.BF16, 96)
+    with pytest.raises(ValueError):
+        _lib.tile_shape(7, _lib.BF16, 128)
+
+
+def test_error_codes_and_messages(lib):
+    assert lib.flexattn_fwd(None, None) == _lib.EINVAL
+    assert b"NULL" in lib.flexattn_last_error_string()
+    assert lib.flexattn_bwd_dq(None, None) == _lib.EINVAL
+    assert lib.flexattn_bwd_dkv(None, None) == _lib.EINVAL
+    assert lib.flexattn_bwd_delta(None, None, None, 1, 128, 0, None) == _lib.EINVAL
+    m = _lib.MaskSpecC(_lib.MASK_WINDOW, 0, 0, 0, None, None)
+    dummy = C.create_string_buffer(64)
+    rc = lib.flexattn_build_block_mask(C.byref(m), 256, 256, 128, 128, dummy, None, None, None, None, None)
+    assert rc == _lib.EINVAL and b"window" in lib.flexattn_last_error_string()
+    m = _lib.MaskSpecC(_lib.MASK_CAUSAL, 0, 0, 0, None, None)
+    rc = lib.flexattn_build_block_mask(C.byref(m), 250, 256, 128, 128, dummy, None, None, None, None, None)
+    assert rc == _lib.EINVAL and b"divisible" in lib.flexattn_last_error_string()
+    # shape errors are caught before any launch
+    p = _lib.FwdParamsC()
+    p.q = p.k = p.v = p.o = C.addressof(dummy)
+    p.B, p.Hq, p.Hkv, p.Sq, p.Sk, p.D, p.dtype = 1, 3, 2, 128, 128, 128, _lib.BF16
+    assert lib.flexattn_fwd(C.byref(p), None) == _lib.EINVAL
+    assert b"multiple" in lib.flexattn_last_error_string()
+    p.Hq = 2
+    p.Sq = 100
+    assert lib.flexattn_fwd(C.byref(p), None) == _lib.EINVAL
+    p.Sq, p.D = 128, 96
+    assert lib.flexattn_fwd(C.byref(p), None) == _lib.ENOTSUP
+    with pytest.raises(NotImplementedError):
+        _lib.check(_lib.ENOTSUP)
+    with pytest.raises(ValueError):
+        _lib.check(_lib.EINVAL)

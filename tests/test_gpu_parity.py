@@ -1,0 +1,291 @@
+"""GPU parity tests: the HIP kernels, called through the Python entry points (and therefore the
+C ABI of libflexattn.so), against the CPU oracle on identical seeded inputs.
+
+Tolerances (north star): block map bit-exact; bf16 max-abs <= 2e-2 and rel-L2 <= 1e-2 on
+o, dq, dk, dv; fp32 <= 1e-5 for both (see helpers.assert_close for the magnitude scaling of the
+absolute bound).  Full-size configurations are checked against the oracle on sampled q rows /
+whole heads and through size-independent invariants.
+"""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_close, oracle_kwargs
+from oracle import mha_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def F():
+    import flex_attention_tpu_amd as F
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return F
+
+
+def _fwd(F, q, k, v, sc, mf, bf, score_fn, causal=False, blk=128):
+    return F._flex_attention_impl(q, k, v, None, None, True, causal, sc, 1, blk, blk, blk, False, bf, mf, score_fn)
+
+
+def _dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, score_fn, causal=False, blk=128):
+    return F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=blk, block_k_major=blk,
+                                   block_k=blk, sm_scale=sc, debug=False, score_fn=score_fn, mask_fn=mf,
+                                   block_mask_fn=bf, causal=causal)
+
+
+def _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, score_fn, causal=False, blk=128):
+    return F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=blk, block_q_major=blk,
+                                     block_k_major=blk, block_k=blk, sm_scale=sc, causal=causal, debug=False,
+                                     score_fn=score_fn, mask_fn=mf, block_mask_fn=bf)
+
+
+# ------------------------------------------------------------------------------------------------
+# block-mask builder: bit-exact
+# ------------------------------------------------------------------------------------------------
+def _mask_cases(S, bq, bk):
+    from flex_attention_tpu_amd import masks
+    lens = O.make_segment_lengths(S, lo=max(8, S // 16), hi=max(16, S // 3), seed=4)
+    return [
+        ("none", masks.place_holder(bq, bk), {}),
+        ("causal", masks.make_causal_mask_fns(bq, bk), dict(causal=True)),
+        ("window", masks.make_sliding_window_mask_fns(bq, bk, S // 5 + 3), dict(window_size=S // 5 + 3)),
+        ("causal_window", masks.make_causal_sliding_window_mask_fns(bq, bk, S // 7 + 1),
+         dict(causal=True, window_size=S // 7 + 1)),
+        ("jagged", masks.make_jagged_mask_fns(bq, bk, lens), dict(causal=True, segment_ids=O.doc_ids_from_lengths(lens))),
+        ("s2", masks.make_s2_mask_fns(bq, bk, S // 9 + 2, 2 * bk), dict(window_size=S // 9 + 2, s2_stride=2 * bk)),
+    ]
+
+
+@pytest.mark.parametrize("S,bq,bk", [(1024, 128, 64), (1024, 64, 128), (2048, 128, 128), (768, 64, 64), (512, 32, 16)])
+def test_block_mask_builder_bit_exact(F, S, bq, bk):
+    from flex_attention_tpu_amd import block_mask
+    for name, (mf, bf), kw in _mask_cases(S, bq, bk):
+        bm = block_mask.create_block_mask((mf, bf), S, S, bq, bk, DEV)
+        nq, nk = S // bq, S // bk
+        state = bm.state.cpu()
+        run = state != 0
+        host = block_mask.host_block_map(bf, nq, nk)
+        assert torch.equal(run, host), f"{name}: run-map differs from the block closure"
+        keep = O.dense_mask(S, S, **kw) if kw else torch.ones(S, S, dtype=torch.bool)
+        brute = O.block_map_bruteforce(keep, bq, bk)
+        assert bool(((state == 2) <= (brute == 2)).all()), f"{name}: a tile marked full has masked elements"
+        assert bool(((state == 0) <= (brute == 0)).all()), f"{name}: a skipped tile has kept elements"
+        if name in ("none", "causal", "window", "jagged"):
+            assert torch.equal(state, brute), f"{name}: state map differs from brute force"
+        kv_cnt, kv_idx = bm.kv_cnt.cpu(), bm.kv_idx.cpu()
+        q_cnt, q_idx = bm.q_cnt.cpu(), bm.q_idx.cpu()
+        for qb in range(nq):
+            assert kv_idx[qb, : kv_cnt[qb]].tolist() == torch.nonzero(run[qb]).flatten().tolist()
+        for kb in range(nk):
+            assert q_idx[kb, : q_cnt[kb]].tolist() == torch.nonzero(run[:, kb]).flatten().tolist()
+
+
+def test_block_mask_builder_matches_config_fixtures(F):
+    from flex_attention_tpu_amd import block_mask, configs
+    g = np.load(os.path.join(GOLDEN, "block_maps.npz"))
+    for name in ("cfg2", "cfg4", "cfg5"):
+        cfg = configs.CONFIGS[name]
+        n = int(g[name + "_n"])
+        gold = torch.from_numpy(np.unpackbits(g[name], axis=1)[:, :n].astype(bool))
+        bm = block_mask.create_block_mask(configs.mask_fns(cfg), cfg.S, cfg.S, 128, 128, DEV)
+        run = bm.run_mask().cpu()
+        if name == "cfg4":
+            assert bool((run | ~gold).all()) and int(run.sum()) == 540
+        else:
+            assert torch.equal(run, gold), name
+
+
+# ------------------------------------------------------------------------------------------------
+# small-shape parity matrix (oracle runs whole tensors in float64)
+# ------------------------------------------------------------------------------------------------
+def _small_cases():
+    from flex_attention_tpu_amd import masks, scores
+    lens = [300, 212, 512]
+    sc = 1 / math.sqrt(128)
+    c = []
+    c.append(("plain", (1, 2, 2, 512, 512), None, None, {}, sc))
+    c.append(("causal", (2, 2, 2, 512, 512), masks.make_causal_mask_fns(128, 128), None, dict(causal=True), sc))
+    c.append(("window", (1, 2, 2, 1024, 1024), masks.make_sliding_window_mask_fns(128, 128, 200), None, dict(window_size=200), sc))
+    c.append(("causal_window", (1, 2, 2, 1024, 1024), masks.make_causal_sliding_window_mask_fns(128, 128, 257), None,
+              dict(causal=True, window_size=257), sc))
+    c.append(("jagged", (1, 2, 2, 1024, 1024), masks.make_jagged_mask_fns(128, 128, lens), None,
+              dict(causal=True, segment_ids=O.doc_ids_from_lengths(lens)), sc))
+    c.append(("s2", (1, 2, 2, 1024, 1024), masks.make_s2_mask_fns(128, 128, 128, 64), None,
+              dict(mask=O.dense_mask(1024, 1024, window_size=128, s2_stride=64)), sc))
+    c.append(("softcap", (1, 2, 2, 512, 512), masks.make_causal_mask_fns(128, 128), scores.make_softcap_score_fn(5.0),
+              dict(causal=True, score_mod=O.score_mod_softcap(5.0)), sc))
+    c.append(("alibi_global", (1, 4, 4, 512, 512), masks.make_causal_mask_fns(128, 128), scores.make_alibi_global_score_fn(4),
+              dict(causal=True, score_mod=O.score_mod_alibi_global(O.alibi_slopes(4))), sc))
+    c.append(("alibi_tile", (1, 2, 2, 512, 512), None, scores.make_alibi_score_fn(0.5),
+              dict(score_mod=O.score_mod_alibi_tile_local(0.5, 128, 128)), sc))
+    c.append(("gqa", (1, 8, 2, 512, 512), masks.make_causal_mask_fns(128, 128), None, dict(causal=True), sc))
+    c.append(("cross", (1, 2, 2, 256, 768), None, None, {}, sc))
+    return c
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+@pytest.mark.parametrize("case", _small_cases(), ids=lambda c: c[0])
+def test_small_shapes_all_passes(F, case, dtype):
+    name, (B, Hq, Hkv, Sq, Sk), mask_pair, score_fn, okw, sc = case
+    D = 128
+    q, k, v, do = O.make_inputs(B, Hq, Hkv, Sq, Sk, D, dtype=dtype, seed=17)
+    ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, **okw)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, sm_scale=sc, **okw)
+    q, k, v, do = [x.to(DEV) for x in (q, k, v, do)]
+    mf, bf = mask_pair if mask_pair else (None, None)
+    o, l, m = _fwd(F, q, k, v, sc, mf, bf, score_fn)
+    assert_close("o", o, ro, dtype)
+    assert_close("lse", m + l.log(), rm + rl.log(), dtype if dtype == torch.bfloat16 else torch.bfloat16)
+    d = F.compute_delta(o, do)
+    assert_close("delta", d, O.delta(o.cpu(), do.cpu()), torch.float32)
+    dq = _dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, score_fn)
+    dk, dv = _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, score_fn)
+    assert_close("dq", dq, rdq, dtype)
+    assert_close("dk", dk, rdk, dtype)
+    assert_close("dv", dv, rdv, dtype)
+
+
+def test_causal_flag_and_segment_ids_arguments(F):
+    """`causal=True` and `segment_ids=` are honoured by all three entry points."""
+    sc = 0.1
+    lens = [100, 156]
+    sid = O.doc_ids_from_lengths(lens)
+    q, k, v, do = O.make_inputs(1, 2, 2, 256, 256, 128, dtype=torch.bfloat16, seed=5)
+    ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, causal=True, segment_ids=sid)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, sm_scale=sc, causal=True, segment_ids=sid)
+    q, k, v, do = [x.to(DEV) for x in (q, k, v, do)]
+    o, l, m = F._flex_attention_impl(q, k, v, None, sid, True, True, sc, 1, 128, 128, 128, False, None, None, None)
+    assert_close("o", o, ro, torch.bfloat16)
+    d = F.compute_delta(o, do)
+    dq = F.flex_attention_bwd_dq(q, k, v, None, sid, l, m, o, do, d, block_b=1, block_q=128, block_k_major=128,
+                                 block_k=128, sm_scale=sc, debug=False, causal=True)
+    dk, dv = F.flash_attention_bwd_dkv(k, v, q, None, sid, l, m, d, do, block_b=1, block_q=128, block_q_major=128,
+                                       block_k_major=128, block_k=128, sm_scale=sc, causal=True, debug=False)
+    assert_close("dq", dq, rdq, torch.bfloat16)
+    assert_close("dk", dk, rdk, torch.bfloat16)
+    assert_close("dv", dv, rdv, torch.bfloat16)
+    # save_residuals=False returns the output only
+    o2 = F._flex_attention_impl(q, k, v, None, sid, False, True, sc, 1, 128, 128, 128, False, None, None, None)
+    assert torch.equal(o2, o)
+
+
+def test_entry_points_reject_bad_arguments_on_gpu(F):
+    q = torch.zeros(1, 2, 192, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError):  # 192 is not a multiple of the 128-row q tile
+        F._flex_attention_impl(q, q, q, None, None, False, False, 1.0, 1, 64, 64, 64, False, None, None, None)
+    q = torch.zeros(1, 2, 256, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(NotImplementedError):  # bf16 kernels exist for head dim 128 only
+        F._flex_attention_impl(q, q, q, None, None, False, False, 1.0, 1, 128, 128, 128, False, None, None, None)
+    q = torch.zeros(1, 2, 256, 128, dtype=torch.float16, device=DEV)
+    with pytest.raises(NotImplementedError):
+        F._flex_attention_impl(q, q, q, None, None, False, False, 1.0, 1, 128, 128, 128, False, None, None, None)
+
+
+# ------------------------------------------------------------------------------------------------
+# the five benchmark configurations at full size
+# ------------------------------------------------------------------------------------------------
+def test_cfg1_fp32_full(F):
+    from flex_attention_tpu_amd import configs
+    cfg = configs.CONFIGS["cfg1"]
+    q, k, v, do = configs.make_inputs(cfg)
+    sc = cfg.sm_scale
+    ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, sm_scale=sc)
+    q, k, v, do = [x.to(DEV) for x in (q, k, v, do)]
+    o, l, m = _fwd(F, q, k, v, sc, None, None, None)
+    d = F.compute_delta(o, do)
+    dq = _dq(F, q, k, v, l, m, o, do, d, sc, None, None, None)
+    dk, dv = _dkv(F, q, k, v, l, m, do, d, sc, None, None, None)
+    for name, t, r in (("o", o, ro), ("m", m, rm), ("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+        assert_close(name, t, r, torch.float32)
+    assert O.rel_l2(l, rl) <= 1e-5
+
+
+def _full_config_check(F, name, n_rows, heads_q):
+    """Runs forward, delta, dq and dk/dv of a full-size configuration and checks
+    (1) o, l, m and dq on `n_rows` sampled q rows of the heads `heads_q` against the oracle,
+    (2) dk, dv against the oracle with dO zeroed outside the sampled rows (the gradients are linear
+        in dO, so this exercises every kv position at full sequence length),
+    (3) invariants of the dense-dO run: sum_i q_i.dq_i == sum_j k_j.dk_j per kv head, and
+        row-stochastic P (v = 1 gives o = 1)."""
+    from flex_attention_tpu_amd import configs
+    cfg = configs.CONFIGS[name]
+    sc = cfg.sm_scale
+    okw = oracle_kwargs(cfg)
+    q, k, v, do = configs.make_inputs(cfg)
+    mf, bf = configs.mask_fns(cfg)
+    sfn = configs.score_fn(cfg)
+    g = torch.Generator().manual_seed(1)
+    rows = torch.sort(torch.randperm(cfg.S, generator=g)[:n_rows]).values
+    rows[0], rows[-1] = 0, cfg.S - 1
+    heads = [(b, h) for (b, h) in heads_q]
+    ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, q_rows=rows, heads=heads, **okw)
+    rdq, _, _ = O.mha_bwd_reference(q, k, v, ro, do[:, :, rows], rl, rm, sm_scale=sc, q_rows=rows, heads=heads, **okw)
+    do_sparse = torch.zeros_like(do)
+    do_sparse[:, :, rows] = do[:, :, rows]
+    _, rdk_s, rdv_s = O.mha_bwd_reference(q, k, v, ro, do[:, :, rows], rl, rm, sm_scale=sc, q_rows=rows, heads=heads, **okw)
+
+    qg, kg, vg, dog, dosg = [x.to(DEV) for x in (q, k, v, do, do_sparse)]
+    o, l, m = _fwd(F, qg, kg, vg, sc, mf, bf, sfn)
+    d = F.compute_delta(o, dog)
+    dq = _dq(F, qg, kg, vg, l, m, o, dog, d, sc, mf, bf, sfn)
+    dk, dv = _dkv(F, qg, kg, vg, l, m, dog, d, sc, mf, bf, sfn)
+    d_s = F.compute_delta(o, dosg)
+    dk_s, dv_s = _dkv(F, qg, kg, vg, l, m, dosg, d_s, sc, mf, bf, sfn)
+    torch.cuda.synchronize()
+
+    group = cfg.Hq // cfg.Hkv
+    for (b, h) in heads:
+        assert_close(f"o[{b},{h}]", o[b, h, rows.to(DEV)], ro[b, h], cfg.dtype)
+        assert_close(f"lse[{b},{h}]", (m + l.log())[b, h, rows.to(DEV)], (rm + rl.log())[b, h], cfg.dtype)
+        assert_close(f"dq[{b},{h}]", dq[b, h, rows.to(DEV)], rdq[b, h], cfg.dtype)
+    kv_heads = sorted({(b, h // group) for (b, h) in heads})
+    for (b, hk) in kv_heads:
+        assert all((b, hk * group + gq) in heads for gq in range(group)), "sample whole KV groups"
+        assert_close(f"dk[{b},{hk}]", dk_s[b, hk], rdk_s[b, hk], cfg.dtype)
+        assert_close(f"dv[{b},{hk}]", dv_s[b, hk], rdv_s[b, hk], cfg.dtype)
+
+    # invariants of the dense run (float64 sums of the bf16 results)
+    qd = (qg.double() * dq.double()).sum(dim=(2, 3)).reshape(cfg.B, cfg.Hkv, group).sum(-1)
+    kd = (kg.double() * dk.double()).sum(dim=(2, 3))
+    scale = (qg.double().abs() * dq.double().abs()).sum(dim=(2, 3)).reshape(cfg.B, cfg.Hkv, group).sum(-1)
+    assert float(((qd - kd).abs() / scale).max()) < 2e-3, "sum q.dq != sum k.dk"
+    o1 = _fwd(F, qg, kg, torch.ones_like(vg), sc, mf, bf, sfn)[0]
+    assert float((o1.float() - 1).abs().max()) < 1e-2, "P rows do not sum to 1"
+    return dict(o=o, l=l, m=m, dq=dq, dk=dk, dv=dv)
+
+
+def test_cfg2_cfg3_causal_bf16_full(F):
+    _full_config_check(F, "cfg2", n_rows=384, heads_q=[(0, 0), (3, 31)])
+
+
+def test_cfg4_alibi_window_bf16_full(F):
+    _full_config_check(F, "cfg4", n_rows=384, heads_q=[(0, 0), (1, 15)])
+
+
+def test_cfg5_gqa_softcap_document_bf16_full(F):
+    _full_config_check(F, "cfg5", n_rows=384, heads_q=[(0, 4), (0, 5), (0, 6), (0, 7)])
+
+
+def test_whole_head_oracle_at_s4096(F):
+    """Configuration 2/3 shape: two whole heads against the dense oracle (float32 CPU math)."""
+    from flex_attention_tpu_amd import configs, masks
+    cfg = configs.CONFIGS["cfg2"]
+    sc = cfg.sm_scale
+    q, k, v, do = O.make_inputs(1, 2, 2, cfg.S, cfg.S, cfg.D, dtype=cfg.dtype, seed=0)
+    ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, causal=True, compute_dtype=torch.float32)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, sm_scale=sc, causal=True, compute_dtype=torch.float32)
+    mf, bf = masks.make_causal_mask_fns(128, 128)
+    q, k, v, do = [x.to(DEV) for x in (q, k, v, do)]
+    o, l, m = _fwd(F, q, k, v, sc, mf, bf, None)
+    d = F.compute_delta(o, do)
+    dq = _dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, None)
+    dk, dv = _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, None)
+    for name, t, r in (("o", o, ro), ("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+        assert_close(name, t, r, torch.bfloat16)

@@ -1,0 +1,150 @@
+"""CPU tests of the host-side mirror of the reference's Python surface: mask / score factories,
+MaskSpec composition, argument validation."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from flex_attention_tpu_amd import _lib, block_mask, configs, masks, scores
+from oracle import mha_oracle as O
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _dense(mask_fn, S):
+    idx = torch.arange(S)
+    return mask_fn(idx, idx)
+
+
+def test_mask_closures_match_oracle_dense_masks():
+    S = 96
+    lens = [20, 41, 35]
+    cases = [
+        (masks.make_causal_mask_fns(16, 16), dict(causal=True)),
+        (masks.make_sliding_window_mask_fns(16, 16, 23), dict(window_size=23)),
+        (masks.make_causal_sliding_window_mask_fns(16, 16, 10), dict(causal=True, window_size=10)),
+        (masks.make_jagged_mask_fns(16, 16, lens), dict(causal=True, segment_ids=O.doc_ids_from_lengths(lens))),
+        (masks.make_s2_mask_fns(16, 16, 9, 8), dict(window_size=9, s2_stride=8)),
+    ]
+    for (mf, bf), kw in cases:
+        assert torch.equal(_dense(mf, S), O.dense_mask(S, S, **kw)), kw
+        # closures also accept numpy index arrays, as the reference's accept jnp arrays
+        idx = np.arange(S)
+        assert np.array_equal(np.asarray(mf(idx, idx)), O.dense_mask(S, S, **kw).numpy())
+
+
+def test_block_closures_match_closed_form_and_bruteforce():
+    S, bq, bk = 256, 32, 16
+    lens = [40, 100, 7, 109]
+    sid = O.doc_ids_from_lengths(lens)
+    cases = [
+        (masks.make_causal_mask_fns(bq, bk), dict(causal=True), True),
+        (masks.make_sliding_window_mask_fns(bq, bk, 50), dict(window_size=50), True),
+        (masks.make_jagged_mask_fns(bq, bk, lens), dict(causal=True, segment_ids=sid), True),
+        (masks.make_causal_sliding_window_mask_fns(bq, bk, 33), dict(causal=True, window_size=33), False),
+        (masks.make_s2_mask_fns(bq, bk, 40, 16), dict(window_size=40, s2_stride=16), False),
+    ]
+    for (mf, bf), kw, exact in cases:
+        host = block_mask.host_block_map(bf, S // bq, S // bk)
+        closed = O.block_map_closed_form(S // bq, S // bk, bq, bk, **kw)
+        assert torch.equal(host, closed), kw
+        brute = O.block_map_bruteforce(_dense(mf, S), bq, bk) != 0
+        if exact:
+            assert torch.equal(host, brute), kw
+        else:
+            assert bool((host | ~brute).all()), kw  # conservative: never skips a tile with kept elements
+
+
+def test_place_holder_and_spec_composition():
+    p, pb = masks.place_holder(128, 128)
+    assert p(3, 4) is True and p.spec.flags == 0
+    c = masks.make_causal_mask_fns(8, 8)[0].spec
+    w = masks.make_sliding_window_mask_fns(8, 8, 5)[0].spec
+    cw = c.combine(w)
+    assert cw.flags == (_lib.MASK_CAUSAL | _lib.MASK_WINDOW) and cw.window == 5
+    assert w.combine(masks.MaskSpec(flags=_lib.MASK_WINDOW, window=3)).window == 3
+    s2 = masks.make_s2_mask_fns(8, 8, 4, 2)[0].spec
+    assert s2.combine(c) == s2
+    with pytest.raises(NotImplementedError):
+        s2.combine(w)
+    j1 = masks.make_jagged_mask_fns(8, 8, [8, 8])[0].spec
+    j2 = masks.make_jagged_mask_fns(8, 8, [4, 12])[0].spec
+    assert j1.combine(c) == j1
+    with pytest.raises(NotImplementedError):
+        j1.combine(j2)
+
+
+def test_document_mask_from_segment_ids():
+    ids = torch.tensor([0, 0, 0, 1, 1, 2, 2, 2])
+    mf, bf = masks.make_document_mask_fns(4, 4, ids)
+    assert torch.equal(_dense(mf, 8), O.dense_mask(8, 8, causal=True, segment_ids=ids))
+    mf2, _ = masks.make_document_mask_fns(4, 4, ids, causal=False)
+    assert torch.equal(_dense(mf2, 8), O.dense_mask(8, 8, segment_ids=ids))
+    with pytest.raises(NotImplementedError):
+        masks.make_document_mask_fns(4, 4, torch.tensor([1, 0, 0, 1]))
+
+
+def test_score_closures_match_oracle_mods():
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(16, 8, generator=g, dtype=torch.float64)
+    k = torch.randn(16, 8, generator=g, dtype=torch.float64)
+    i = torch.arange(16)[:, None]
+    j = torch.arange(16)[None, :]
+    s = q @ k.T
+    assert torch.allclose(scores.make_softcap_score_fn(3.0)(q, k), O.score_mod_softcap(3.0)(s, 0, 0, i, j))
+    assert torch.allclose(scores.make_alibi_score_fn(0.5)(q, k), O.score_mod_alibi_tile_local(0.5, 16, 16)(s, 0, 0, i, j))
+    fn = scores.make_alibi_global_score_fn(4)
+    ref = O.score_mod_alibi_global(O.alibi_slopes(4))(s, 0, 2, i + 32, j + 16)
+    assert torch.allclose(fn(q, k, head=2, q_start=32, k_start=16), ref)
+    assert fn.spec.kind == _lib.SCORE_ALIBI and len(fn.spec.slopes) == 4
+    assert abs(fn.spec.slopes[0] - 2 ** (-8 / 4)) < 1e-15
+
+
+def test_config_helpers_match_oracle_and_fixtures():
+    with open(os.path.join(GOLDEN, "cfg5_doc_lengths.json")) as f:
+        gold = json.load(f)
+    for seed in range(4):
+        assert configs.segment_lengths(16384, seed=seed) == gold[str(seed)] == O.make_segment_lengths(16384, seed=seed)
+    c2, c4 = configs.CONFIGS["cfg2"], configs.CONFIGS["cfg4"]
+    assert configs.n_pairs_per_head(c2) == 4096 * 4096 / 2
+    assert configs.n_pairs_per_head(c4) == 7_872_000  # 524800 + 7168*1025
+    assert abs(configs.flops_fwd(c2) - 5.498e11) / 5.498e11 < 1e-3
+    a = configs.make_inputs(configs.CONFIGS["cfg1"])
+    b = O.make_inputs(1, 4, 4, 512, 512, 64, dtype=torch.float32, seed=0)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+
+
+def test_block_map_fixtures_match_closures():
+    """Committed brute-force run-maps of the benchmark configurations == the block closures."""
+    g = np.load(os.path.join(GOLDEN, "block_maps.npz"))
+    for name in ("cfg2", "cfg4", "cfg5"):
+        cfg = configs.CONFIGS[name]
+        n = int(g[name + "_n"])
+        gold = torch.from_numpy(np.unpackbits(g[name], axis=1)[:, :n].astype(bool))
+        _, bf = configs.mask_fns(cfg)
+        host = block_mask.host_block_map(bf, n, n)
+        if name == "cfg4":  # AND of two closures is conservative
+            assert bool((host | ~gold).all()) and int(host.sum()) == 540
+        else:
+            assert torch.equal(host, gold), name
+    assert int(torch.from_numpy(np.unpackbits(g["cfg2"], axis=1)[:, :32]).sum()) == 528
+
+
+def test_entry_points_validate_arguments_without_gpu():
+    import flex_attention_tpu_amd as F
+    q = torch.zeros(1, 2, 128, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="GPU"):
+        F._flex_attention_impl(q, q, q, None, None, False, False, 1.0, 1, 128, 128, 128, False, None, None, None)
+    with pytest.raises(NotImplementedError, match="ab"):
+        F._flex_attention_impl(q, q, q, q, None, False, False, 1.0, 1, 128, 128, 128, False, None, None, None)
+    with pytest.raises(NotImplementedError):
+        block_mask.spec_of(lambda a, b: a[:, None] >= b[None, :], None)
+    from flex_attention_tpu_amd._common import check_blocks, score_spec_c
+    with pytest.raises(ValueError):
+        check_blocks(512, 512, block_q=100)
+    with pytest.raises(ValueError):
+        check_blocks(512, 512, block_k_major=256, block_k=96)
+    with pytest.raises(NotImplementedError):
+        score_spec_c(lambda a, b: a @ b.T, 2, "cpu", 1, 1)
