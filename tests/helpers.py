@@ -10,21 +10,7 @@ F32_ABS, F32_REL = 1e-5, 1e-5
 
 def oracle_kwargs(cfg):
     """Oracle keywords equivalent to a flex_attention_tpu_amd.configs.AttnConfig."""
-    from flex_attention_tpu_amd import configs
-    kw = {}
-    if cfg.mask == "causal":
-        kw["causal"] = True
-    elif cfg.mask == "causal_window":
-        kw["causal"] = True
-        kw["window_size"] = cfg.window + 1
-    elif cfg.mask == "document":
-        kw["causal"] = True
-        kw["segment_ids"] = O.doc_ids_from_lengths(configs.segment_lengths(cfg.S, seed=cfg.seed))
-    if cfg.score == "alibi":
-        kw["score_mod"] = O.score_mod_alibi_global(O.alibi_slopes(cfg.Hq))
-    elif cfg.score == "softcap":
-        kw["score_mod"] = O.score_mod_softcap(cfg.cap)
-    return kw
+    return O.kwargs_for_config(cfg)
 
 
 def assert_close(name, test, ref, dtype):
