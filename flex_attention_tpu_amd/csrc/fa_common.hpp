@@ -128,15 +128,15 @@ __device__ __forceinline__ bf16x2 pack_bf16(float a, float b) {
 // Element mask, evaluated only on tiles the block map marks partial.
 // ------------------------------------------------------------------------------------------
 __device__ __forceinline__ bool keep_elem(const MaskArgs& mk, int i, int j, int doc_i, int doc_j) {
-  bool keep = true;
-  if (mk.flags & FLEXATTN_MASK_S2) {
-    int d = i - j;
-    keep = (d >= 0) && ((d < mk.window) || (j % mk.stride == 0));
-  } else {
-    if (mk.flags & FLEXATTN_MASK_CAUSAL) keep = keep && (i >= j);
-    if (mk.flags & FLEXATTN_MASK_WINDOW) keep = keep && ((i - j) < mk.window);
-  }
-  if (mk.flags & FLEXATTN_MASK_DOC) keep = keep && (doc_i == doc_j);
+  // Branch-free: every term is computed and selected by the (wave-uniform) flag bits.
+  const bool f_causal = (mk.flags & FLEXATTN_MASK_CAUSAL) != 0;
+  const bool f_window = (mk.flags & FLEXATTN_MASK_WINDOW) != 0;
+  const bool f_doc = (mk.flags & FLEXATTN_MASK_DOC) != 0;
+  const bool f_s2 = (mk.flags & FLEXATTN_MASK_S2) != 0;
+  const int d = i - j;
+  const bool in_window = d < mk.window;
+  bool keep = (!f_causal | (d >= 0)) & (!f_window | in_window) & (!f_doc | (doc_i == doc_j));
+  if (f_s2) keep = keep & (d >= 0) & (in_window | ((j % mk.stride) == 0));
   return keep;
 }
 

@@ -3,30 +3,28 @@
 // One work-group = 4 waves = one 128-row Q tile of one (batch, head); each wave owns 32 q rows.
 // The kernel works on S^T = K Q^T so that one lane holds one q row's scores: softmax statistics
 // stay lane-private apart from one exchange between the two 32-lane halves.  K/V tiles of 64 rows
-// are double-buffered in LDS; P goes straight from the QK accumulators to the B operand of the
-// PV MFMA (O^T = V^T P^T), V^T is fetched with transposing LDS reads.
+// are double-buffered in LDS by LDS-direct loads issued one tile ahead; P goes straight from the
+// QK accumulators to the B operand of the PV MFMA (O^T = V^T P^T); V^T is fetched with
+// transposing LDS reads.
 #include "fa_common.hpp"
 #include "launch.hpp"
+#include "tile_io.hpp"
 
 namespace fa {
 
 namespace fwd_cfg {
-constexpr int BM = 128;          // q rows per work-group
-constexpr int BN = 64;           // kv rows per step
+constexpr int BM = 128;  // q rows per work-group
+constexpr int BN = 64;   // kv rows per step
 constexpr int D = 128;
-constexpr int KSTR = D + 8;      // LDS row stride of K (elements): 16 B pad -> conflict-free b128 row reads
-constexpr int VSTR = D + 32;     // LDS row stride of V: 64 B pad -> 4 rows x 64 B of a transposing read hit distinct banks
-constexpr int K_TILE = BN * KSTR;
-constexpr int V_TILE = BN * VSTR;
-constexpr int LDS_BYTES = 2 * (K_TILE + V_TILE) * 2;
+constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2
 }  // namespace fwd_cfg
 
 template <int SCORE>
 __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
   using namespace fwd_cfg;
-  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   bf16_t* sK = reinterpret_cast<bf16_t*>(smem_raw);
-  bf16_t* sV = sK + 2 * K_TILE;
+  bf16_t* sV = sK + 2 * kTileElems;
 
   const int nQ = a.Sq / BM;
   const int nK = a.map.nk;
@@ -73,115 +71,152 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int e = 0; e < 16; ++e) o_acc[i][e] = 0.f;
-  float m_run = kNegInf;  // running max, log2 domain
+  float m_run = kNegInf;  // running max: raw dot-product units (plain score) or log2-domain logits
   float l_run = 0.f;      // this lane's half of the running sum
 
-  // global -> LDS copy: 64 rows x 16 chunks of 16 B; thread handles chunk tid%16 of rows tid/16 + 16*j.
-  const int cp_chunk = tid & 15;
-  const int cp_row = tid >> 4;
-  bf16x8 kst[4], vst[4];
-  auto g_load = [&](int kb) {
-    const bf16_t* kp = Kg + ((size_t)kb * BN + cp_row) * D + cp_chunk * 8;
-    const bf16_t* vp = Vg + ((size_t)kb * BN + cp_row) * D + cp_chunk * 8;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      kst[j] = *reinterpret_cast<const bf16x8*>(kp + (size_t)j * 16 * D);
-      vst[j] = *reinterpret_cast<const bf16x8*>(vp + (size_t)j * 16 * D);
-    }
-  };
-  auto s_store = [&](int buf) {
-    bf16_t* kd = sK + buf * K_TILE + cp_row * KSTR + cp_chunk * 8;
-    bf16_t* vd = sV + buf * V_TILE + cp_row * VSTR + cp_chunk * 8;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      *reinterpret_cast<bf16x8*>(kd + j * 16 * KSTR) = kst[j];
-      *reinterpret_cast<bf16x8*>(vd + j * 16 * VSTR) = vst[j];
-    }
-  };
-
+  // Tile indices and states are fetched ahead of use (index three tiles, state two tiles ahead) so
+  // that no iteration waits on a load it has just issued.
+  int kb_cur = 0, kb_nxt = 0, kb_n2 = 0, st_cur = 0, st_nxt = 0;
+  if (n_tiles > 0) kb_cur = tile_idx[0];
+  if (n_tiles > 1) kb_nxt = tile_idx[1];
+  if (n_tiles > 2) kb_n2 = tile_idx[2];
+  if (n_tiles > 0) st_cur = tile_state[kb_cur];
+  if (n_tiles > 1) st_nxt = tile_state[kb_nxt];
+  TileLoader loader;
+  loader.init(__builtin_amdgcn_readfirstlane(w), lane);
   if (n_tiles > 0) {
-    g_load(tile_idx[0]);
-    s_store(0);
+    const int kb0 = __builtin_amdgcn_readfirstlane(kb_cur);
+    loader.load(Kg + (size_t)kb0 * BN * D, sK);
+    loader.load(Vg + (size_t)kb0 * BN * D, sV);
   }
+  wait_vmem_all();
   __syncthreads();
+
+  // lane-constant pieces of the LDS addresses
+  const int k_sw = swz(l32);                               // row reads: rows l32 (+32c)
+  const int v_row = 4 * hh + ((lane & 15) >> 2);           // transposing reads: row inside a 16-row group
+  const int v_chunk = 2 * ((lane & 31) >> 4) + ((lane & 3) >> 1);
+  const int v_half = 4 * (lane & 1);
 
   for (int t = 0; t < n_tiles; ++t) {
     const int buf = t & 1;
-    const int kb = tile_idx[t];
-    const bool partial = tile_state[kb] == 1;
-    if (t + 1 < n_tiles) g_load(tile_idx[t + 1]);
+    const int kb = __builtin_amdgcn_readfirstlane(kb_cur);
+    const bool partial = __builtin_amdgcn_readfirstlane(st_cur) == 1;
+    const int kb_n3 = (t + 3 < n_tiles) ? tile_idx[t + 3] : 0;
+    const int st_n2 = (t + 2 < n_tiles) ? tile_state[kb_n2] : 0;
+    if (t + 1 < n_tiles) {
+      const int kbn = __builtin_amdgcn_readfirstlane(kb_nxt);
+      loader.load(Kg + (size_t)kbn * BN * D, sK + (buf ^ 1) * kTileElems);
+      loader.load(Vg + (size_t)kbn * BN * D, sV + (buf ^ 1) * kTileElems);
+    }
 
     // ---- S^T = K Q^T : two 32(kv) x 32(q) accumulator tiles ----
     f32x16 s_acc[2];
-    const bf16_t* kbase = sK + buf * K_TILE + l32 * KSTR + hh * 8;
+    const bf16_t* kt = sK + buf * kTileElems + l32 * kTileD;
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
+      bf16x8 kf[8];
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks)
+        kf[ks] = *reinterpret_cast<const bf16x8*>(kt + c * 32 * kTileD + (((2 * ks + hh) ^ k_sw) << 3));
 #pragma unroll
       for (int e = 0; e < 16; ++e) s_acc[c][e] = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        bf16x8 kf = *reinterpret_cast<const bf16x8*>(kbase + c * 32 * KSTR + ks * 16);
-        s_acc[c] = mfma32(kf, qreg[ks], s_acc[c]);
-      }
+      for (int ks = 0; ks < 8; ++ks) s_acc[c] = mfma32(kf[ks], qreg[ks], s_acc[c]);
     }
 
-    // ---- score mod, mask, online softmax (log2 domain) ----
+    // ---- score mod, mask, online softmax ----
+    // For the plain score the running maximum is kept on the raw dot products and the scale is
+    // folded into the exponent (one FMA per element); score mods go through the log2-domain logit.
     const int kv0 = kb * BN;
+    constexpr bool kPlain = (SCORE == FLEXATTN_SCORE_NONE);
     float m_tile = kNegInf;
+    if (!partial) {
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
+      for (int c = 0; c < 2; ++c) {
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int j = kv0 + 32 * c + acc_row(e, hh);
-        float tv = sm.to_log2(s_acc[c][e], q_idx, j);
-        if (partial) {
-          int doc_j = 0;
-          if (a.mask.flags & FLEXATTN_MASK_DOC) doc_j = a.mask.doc_k[j];
-          if (!keep_elem(a.mask, q_idx, j, doc_i, doc_j)) tv = kNegInf;
+        for (int e = 0; e < 16; ++e) {
+          if (!kPlain) s_acc[c][e] = sm.to_log2(s_acc[c][e], q_idx, kv0 + 32 * c + acc_row(e, hh));
+          m_tile = fmaxf(m_tile, s_acc[c][e]);
         }
-        s_acc[c][e] = tv;
-        m_tile = fmaxf(m_tile, tv);
+      }
+    } else {
+      // the lane's kv indices come in runs of 4: kv0 + 32c + 8g + 4hh + {0..3}
+      const bool has_doc = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int j0 = kv0 + 32 * c + 8 * g + 4 * hh;
+          int dj[4] = {0, 0, 0, 0};
+          if (has_doc) {
+            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_k + j0);
+            dj[0] = d4[0]; dj[1] = d4[1]; dj[2] = d4[2]; dj[3] = d4[3];
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int e = 4 * g + u;
+            float tv = kPlain ? s_acc[c][e] : sm.to_log2(s_acc[c][e], q_idx, j0 + u);
+            tv = keep_elem(a.mask, q_idx, j0 + u, doc_i, dj[u]) ? tv : kNegInf;
+            s_acc[c][e] = tv;
+            m_tile = fmaxf(m_tile, tv);
+          }
+        }
       }
     }
     m_tile = half_max(m_tile);
     const float m_new = fmaxf(m_run, m_tile);
     const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
-    const float alpha = fast_exp2(m_run - m_safe);
-    m_run = m_new;
+    const float e_scale = kPlain ? sm.c2 : 1.0f;  // exponent = e_scale * (s - m)
+    // Rescale the accumulators only when some row's maximum moved (wave-uniform test).
+    if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+      const float alpha = fast_exp2((m_run - m_safe) * e_scale);
+      l_run *= alpha;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o_acc[db][e] *= alpha;
+      m_run = m_new;
+    }
+    const float neg_m = -m_safe * e_scale;
     float l_tile = 0.f;
     bf16x8 p[4];
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
 #pragma unroll
       for (int e = 0; e < 16; e += 2) {
-        float p0 = fast_exp2(s_acc[c][e] - m_safe);
-        float p1 = fast_exp2(s_acc[c][e + 1] - m_safe);
+        float p0, p1;
+        if (kPlain) {
+          p0 = fast_exp2(__builtin_fmaf(s_acc[c][e], e_scale, neg_m));
+          p1 = fast_exp2(__builtin_fmaf(s_acc[c][e + 1], e_scale, neg_m));
+        } else {
+          p0 = fast_exp2(s_acc[c][e] + neg_m);
+          p1 = fast_exp2(s_acc[c][e + 1] + neg_m);
+        }
         l_tile += p0 + p1;
         bf16x2 pk = pack_bf16(p0, p1);
         p[2 * c + (e >> 3)][e & 7] = pk[0];
         p[2 * c + (e >> 3)][(e & 7) + 1] = pk[1];
       }
     }
-    l_run = l_run * alpha + l_tile;
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) o_acc[db][e] *= alpha;
+    l_run += l_tile;
 
     // ---- O^T += V^T P^T ----
-    const bf16_t* vbase = sV + buf * V_TILE + (4 * hh + ((lane & 15) >> 2)) * VSTR + 16 * ((lane & 31) >> 4) +
-                          4 * (lane & 3);
+    const bf16_t* vt = sV + buf * kTileElems + v_half;
 #pragma unroll
     for (int tt = 0; tt < 4; ++tt) {
 #pragma unroll
       for (int db = 0; db < 4; ++db) {
-        const bf16_t* vp = vbase + (16 * tt) * VSTR + 32 * db;
-        bf16x8 vf = join_tr(lds_read_tr16(vp), lds_read_tr16(vp + 8 * VSTR));
-        o_acc[db] = mfma32(vf, p[tt], o_acc[db]);
+        const int r_lo = 16 * tt + v_row;
+        s16x4 lo = lds_read_tr16(vt + tile_off(r_lo, 4 * db + v_chunk));
+        s16x4 hi = lds_read_tr16(vt + tile_off(r_lo + 8, 4 * db + v_chunk));
+        o_acc[db] = mfma32(join_tr(lo, hi), p[tt], o_acc[db]);
       }
     }
 
-    if (t + 1 < n_tiles) s_store(buf ^ 1);
+    kb_cur = kb_nxt; kb_nxt = kb_n2; kb_n2 = kb_n3;
+    st_cur = st_nxt; st_nxt = st_n2;
+    wait_vmem_all();
     __syncthreads();
   }
 
@@ -201,7 +236,7 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
   if (a.l != nullptr && hh == 0) {
     const size_t r = (size_t)bh * a.Sq + q_idx;
     a.l[r] = l_tot;
-    a.m[r] = m_run * kLn2;  // back to natural units
+    a.m[r] = (SCORE == FLEXATTN_SCORE_NONE) ? m_run * a.sm_scale : m_run * kLn2;  // natural units
   }
 }
 
