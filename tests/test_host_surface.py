@@ -148,3 +148,34 @@ def test_entry_points_validate_arguments_without_gpu():
         check_blocks(512, 512, block_k_major=256, block_k=96)
     with pytest.raises(NotImplementedError):
         score_spec_c(lambda a, b: a @ b.T, 2, "cpu", 1, 1)
+
+
+def test_make_jax_score_fn_recognises_functors():
+    from flex_attention_tpu_amd.util import make_jax_score_fn
+    cap = 30.0
+    slope = 0.25
+
+    def softcap(q_tile, k_tile):
+        logits = torch.matmul(q_tile, k_tile.T)
+        return cap * torch.tanh(logits / cap)
+
+    def alibi(q_tile, k_tile):
+        mm, nn = q_tile.shape[0], k_tile.shape[0]
+        dist = torch.abs(torch.arange(mm)[:, None] - torch.arange(nn)[None, :])
+        return q_tile @ k_tile.T - slope * dist
+
+    def plain(q_tile, k_tile):
+        return torch.einsum("qd,kd->qk", q_tile, k_tile)
+
+    def unsupported(q_tile, k_tile):
+        return (q_tile @ k_tile.T) ** 2
+
+    s = make_jax_score_fn(softcap).spec
+    assert s.kind == _lib.SCORE_SOFTCAP and abs(s.cap - cap) < 1e-6
+    s = make_jax_score_fn(alibi).spec
+    assert s.kind == _lib.SCORE_ALIBI_TILE and abs(s.slope - slope) < 1e-9
+    assert make_jax_score_fn(plain).spec.kind == _lib.SCORE_NONE
+    tagged = scores.make_softcap_score_fn(5.0)
+    assert make_jax_score_fn(tagged) is tagged
+    with pytest.raises(NotImplementedError):
+        make_jax_score_fn(unsupported)
