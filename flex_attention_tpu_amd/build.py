@@ -32,6 +32,7 @@ FLAGS = [
     "-fno-finite-math-only",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    "-Wno-inline-asm",
     f"-I{INCLUDE}",
     f"-I{CSRC}",
 ]

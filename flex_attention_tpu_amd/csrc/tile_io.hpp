@@ -24,31 +24,39 @@ __device__ __forceinline__ constexpr int tile_off(int row, int chunk) {
 // Asynchronous copy of a 64 x 128 bf16 tile (global row stride 128 elements) into LDS with
 // global_load_lds_dwordx4: the data never passes through registers.  Each instruction fills one
 // contiguous 1 KB block (4 tile rows); lane L's 16 bytes land at block + 16*L, so the swizzle is
-// applied on the global side.  The four waves of a work-group each copy four blocks.  The
+// applied on the global side.  The NWAVES waves of a work-group each copy 16/NWAVES blocks.  The
 // lane-dependent global offsets are loop invariant and are computed once (TileLoader::init); per
 // tile only the uniform base pointers change.  Completion = vmcnt(0) on every wave + barrier.
+template <int NWAVES>
 struct TileLoader {
-  unsigned goff[4];  // byte offset of this lane's 16 bytes inside the global tile, per block
+  static constexpr int kBlocks = 16 / NWAVES;  // 1 KB blocks copied per wave
+  unsigned goff[kBlocks];  // byte offset of this lane's 16 bytes inside the global tile, per block
   int wave;
 
   __device__ __forceinline__ void init(int wave_, int lane) {
     wave = wave_;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int row = (wave * 4 + i) * 4 + (lane >> 4);
+    for (int i = 0; i < kBlocks; ++i) {
+      const int row = (wave * kBlocks + i) * 4 + (lane >> 4);
       const int chunk = (lane & 15) ^ swz(row);
       goff[i] = (unsigned)(row * kTileD + chunk * 8) * 2u;
     }
   }
 
-  // g_tile and lds_tile must be wave-uniform.
+  // g_tile and lds_tile must be wave-uniform.  The load is written as inline asm (M0 = LDS
+  // destination of the wave's block, SGPR base + per-lane VGPR offset on the global side): issued
+  // through the compiler builtin, later LDS reads that the compiler cannot prove disjoint from the
+  // destination buffer get a vmcnt(0) wait in front of them, which serialises the prefetch.  The
+  // caller orders the copy itself with wait_vmem_all() + barrier before the tile is read.
   __device__ __forceinline__ void load(const bf16_t* g_tile, bf16_t* lds_tile) const {
-    const char* g = reinterpret_cast<const char*>(g_tile);
+    const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)(lds_tile);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(g + goff[i]),
-                                       (__attribute__((address_space(3))) void*)(lds_tile + (wave * 4 + i) * 512),
-                                       16, 0, 0);
+    for (int i = 0; i < kBlocks; ++i) {
+      const unsigned dst = lds_base + (unsigned)(wave * kBlocks + i) * 1024u;
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :
+                   : "v"(goff[i]), "s"(g_tile), "s"(dst)
+                   : "memory", "m0");
     }
   }
 };
