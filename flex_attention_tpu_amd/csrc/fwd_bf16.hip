@@ -1,39 +1,30 @@
 // Flex-attention forward, bf16, head dim 128, gfx950.
 //
-// One work-group = 8 waves = one 256-row Q tile of one (batch, head); each wave owns 32 q rows.
+// One work-group = 4 waves = one 128-row Q tile of one (batch, head); each wave owns 32 q rows.
 // The kernel works on S^T = K Q^T so that one lane holds one q row's scores: softmax statistics
-// stay lane-private apart from one exchange between the two 32-lane halves.  P goes straight from
-// the QK accumulators to the B operand of the PV MFMA (O^T = V^T P^T); V^T is fetched with
-// transposing LDS reads.  K/V tiles of 64 rows are double-buffered in LDS by LDS-direct loads.
-//
-// The two waves that share a SIMD (wave w and w+4) run half a step apart ("ping-pong"): while one
-// group of four waves is in its MFMA phase (QK^T of tile t and P V of tile t-1), the other group
-// is in its VALU phase (softmax of its tile), so the matrix pipe and the vector ALU of every SIMD
-// are busy at the same time.  All eight waves meet at one barrier per half step.
+// stay lane-private apart from one exchange between the two 32-lane halves.  K/V tiles of 64 rows
+// are double-buffered in LDS by LDS-direct loads issued one tile ahead; P goes straight from the
+// QK accumulators to the B operand of the PV MFMA (O^T = V^T P^T); V^T is fetched with
+// transposing LDS reads.
 #include "fa_common.hpp"
 #include "launch.hpp"
 #include "tile_io.hpp"
 
-#include <type_traits>
-
 namespace fa {
 
 namespace fwd_cfg {
-constexpr int BM = 256;        // q rows per work-group
-constexpr int BN = 64;         // kv rows per step
+constexpr int BM = 128;  // q rows per work-group
+constexpr int BN = 64;   // kv rows per step
 constexpr int D = 128;
-constexpr int THREADS = 512;
-constexpr int LIST_CAP = 4096;  // tile-list entries kept in LDS: Sk <= LIST_CAP * BN
-constexpr int LDS_BYTES = 4 * kTileElems * 2 + LIST_CAP * 4;  // K x2, V x2, tile list
+constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2
 }  // namespace fwd_cfg
 
 template <int SCORE>
-__global__ __launch_bounds__(512, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
+__global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
   using namespace fwd_cfg;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   bf16_t* sK = reinterpret_cast<bf16_t*>(smem_raw);
   bf16_t* sV = sK + 2 * kTileElems;
-  int* sList = reinterpret_cast<int*>(sV + 2 * kTileElems);
 
   const int nQ = a.Sq / BM;
   const int nK = a.map.nk;
@@ -46,8 +37,7 @@ __global__ __launch_bounds__(512, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
   const int hk = h / (a.Hq / a.Hkv);
 
   const int tid = threadIdx.x;
-  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int grp = w >> 2;  // 0: leads, 1: runs half a step behind
+  const int w = tid >> 6;
   const int lane = tid & 63;
   const int l32 = lane & 31;
   const int hh = lane >> 5;
@@ -69,16 +59,9 @@ __global__ __launch_bounds__(512, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
   for (int ks = 0; ks < 8; ++ks)
     qreg[ks] = *reinterpret_cast<const bf16x8*>(Qg + (size_t)q_local * D + ks * 16 + hh * 8);
 
-  // The q block's list of kv tiles to visit, packed (state << 24 | kv block), goes to LDS once.
-  const int T = a.map.cnt[qb];
-  {
-    const int* tile_idx = a.map.idx + (size_t)qb * nK;
-    const uint8_t* tile_state = a.map.state + (size_t)qb * nK;
-    for (int i = tid; i < T; i += THREADS) {
-      const int kb = tile_idx[i];
-      sList[i] = kb | ((int)tile_state[kb] << 24);
-    }
-  }
+  const int n_tiles = a.map.cnt[qb];
+  const int* tile_idx = a.map.idx + (size_t)qb * nK;
+  const uint8_t* tile_state = a.map.state + (size_t)qb * nK;
 
   int doc_i = 0;
   if (a.mask.flags & FLEXATTN_MASK_DOC) doc_i = a.mask.doc_q[q_idx];
@@ -91,40 +74,31 @@ __global__ __launch_bounds__(512, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
   float m_run = kNegInf;  // running max: raw dot-product units (plain score) or log2-domain logits
   float l_run = 0.f;      // this lane's half of the running sum
 
-  TileLoader<8> loader;
-  loader.init(w, lane);
-  __syncthreads();  // tile list visible
-
-  // Loads issued at even half steps: K(t+1) and V(t).  Both groups issue their share.
-  auto issue_loads = [&](int t) {
-    if (t + 1 < T) {
-      const int kb = __builtin_amdgcn_readfirstlane(sList[t + 1]) & 0xFFFFFF;
-      loader.load(Kg + (size_t)kb * BN * D, sK + ((t + 1) & 1) * kTileElems);
-    }
-    if (t < T) {
-      const int kb = __builtin_amdgcn_readfirstlane(sList[t]) & 0xFFFFFF;
-      loader.load(Vg + (size_t)kb * BN * D, sV + (t & 1) * kTileElems);
-    }
-  };
-
-  if (T > 0) {
-    const int kb0 = __builtin_amdgcn_readfirstlane(sList[0]) & 0xFFFFFF;
+  // Tile indices and states are fetched ahead of use (index three tiles, state two tiles ahead) so
+  // that no iteration waits on a load it has just issued.
+  int kb_cur = 0, kb_nxt = 0, kb_n2 = 0, st_cur = 0, st_nxt = 0;
+  if (n_tiles > 0) kb_cur = tile_idx[0];
+  if (n_tiles > 1) kb_nxt = tile_idx[1];
+  if (n_tiles > 2) kb_n2 = tile_idx[2];
+  if (n_tiles > 0) st_cur = tile_state[kb_cur];
+  if (n_tiles > 1) st_nxt = tile_state[kb_nxt];
+  TileLoader<4> loader;
+  loader.init(__builtin_amdgcn_readfirstlane(w), lane);
+  if (n_tiles > 0) {
+    const int kb0 = __builtin_amdgcn_readfirstlane(kb_cur);
     loader.load(Kg + (size_t)kb0 * BN * D, sK);
+    loader.load(Vg + (size_t)kb0 * BN * D, sV);
   }
   wait_vmem_all();
-  __builtin_amdgcn_s_barrier();
-  if (grp == 1) {
-    issue_loads(0);
-    __builtin_amdgcn_s_barrier();  // the trailing group starts half a step late
-  }
+  __syncthreads();
 
   // lane-constant pieces of the LDS addresses
   const int k_sw = swz(l32);                               // row reads: rows l32 (+32c)
   const int v_row = 4 * hh + ((lane & 15) >> 2);           // transposing reads: row inside a 16-row group
   const int v_chunk = 2 * ((lane & 31) >> 4) + ((lane & 3) >> 1);
   const int v_half = 4 * (lane & 1);
-  // Byte offsets inside a tile of this lane's operand reads; the tile row block (32c for K rows,
-  // 16tt for V^T groups) and the buffer are added as immediates / a per-step base.
+  // Byte offsets inside a tile of this lane's operand reads; the row block (32c for K rows, 16tt
+  // for V^T groups) is an immediate and the buffer a per-step base.
   unsigned k_off[8], v_off[4][2];
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) k_off[ks] = (unsigned)(l32 * kTileD + (((2 * ks + hh) ^ k_sw) << 3)) * 2u;
@@ -133,31 +107,37 @@ __global__ __launch_bounds__(512, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
     v_off[db][0] = (unsigned)(tile_off(v_row, 4 * db + v_chunk) + v_half) * 2u;
     v_off[db][1] = (unsigned)(tile_off(v_row + 8, 4 * db + v_chunk) + v_half) * 2u;
   }
+#define FA_INTERLEAVE(N_MFMA, READS)                                   \
+  _Pragma("unroll") for (int i_ = 0; i_ < (N_MFMA); ++i_) {            \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 \
+    __builtin_amdgcn_sched_group_barrier(0x100, (READS), 0);           \
+  }
 
-  f32x16 s_acc[2];
-  bf16x8 p[4];
+  for (int t = 0; t < n_tiles; ++t) {
+    const int buf = t & 1;
+    const int kb = __builtin_amdgcn_readfirstlane(kb_cur);
+    const bool partial = __builtin_amdgcn_readfirstlane(st_cur) == 1;
+    const int kb_n3 = (t + 3 < n_tiles) ? tile_idx[t + 3] : 0;
+    const int st_n2 = (t + 2 < n_tiles) ? tile_state[kb_n2] : 0;
+    if (t + 1 < n_tiles) {
+      const int kbn = __builtin_amdgcn_readfirstlane(kb_nxt);
+      loader.load(Kg + (size_t)kbn * BN * D, sK + (buf ^ 1) * kTileElems);
+      loader.load(Vg + (size_t)kbn * BN * D, sV + (buf ^ 1) * kTileElems);
+    }
 
-  // MFMA phase of step t: S^T = K(t) Q^T (if QK) and O^T += V(t-1)^T P(t-1)^T (if PV).  The LDS
-  // operand reads are issued ahead of the MFMAs that consume them and interleaved with the MFMAs
-  // of the other product, so the LDS pipe and the matrix pipe run concurrently.
-  auto mfma_phase = [&](int t, auto has_qk, auto has_pv) {
-    constexpr bool QK = decltype(has_qk)::value;
-    constexpr bool PV = decltype(has_pv)::value;
-    const char* kt = reinterpret_cast<const char*>(sK + (t & 1) * kTileElems);
-    const char* vt = reinterpret_cast<const char*>(sV + ((t - 1) & 1) * kTileElems);
-    // A dependent MFMA (same accumulator) can only issue once its predecessor has drained, so
-    // the products are interleaved: consecutive MFMAs go to S(c=0), O(db), S(c=1), O(db+1), ...
-    // giving six independent accumulator chains.  Operands are fetched one stage (4 S-MFMAs and
-    // 4 O-MFMAs) ahead, interleaved with the MFMAs of the current stage; sched_barrier fences
-    // the stages so at most two stages' operands are live.
-    bf16x8 kf[4][4];             // stage g: k-steps 2g, 2g+1 for c = 0, 1  -> [g][2*j + c]
-    s16x4 vlo[4][4], vhi[4][4];  // stage tt: [tt][db]
+    // ---- S^T = K Q^T : two 32(kv) x 32(q) accumulator tiles ----
+    // LDS operand reads run one stage (4 MFMAs) ahead of the MFMAs that consume them, so the LDS
+    // pipe and the matrix pipe overlap inside the wave; sched_barrier fences the stages.  The
+    // first half of V^T is fetched before the softmax, whose VALU work hides that latency.
+    f32x16 s_acc[2];
+    const char* kt = reinterpret_cast<const char*>(sK + buf * kTileElems);
+    const char* vt = reinterpret_cast<const char*>(sV + buf * kTileElems);
+    bf16x8 kf[4][4];             // [2c + ks/4][ks%4]
+    s16x4 vlo[4][4], vhi[4][4];  // [tt][db]
     auto read_k = [&](int g) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int c = 0; c < 2; ++c)
-          kf[g][2 * j + c] = *reinterpret_cast<const bf16x8*>(kt + k_off[2 * g + j] + c * 32 * kTileD * 2);
+      for (int i = 0; i < 4; ++i)
+        kf[g][i] = *reinterpret_cast<const bf16x8*>(kt + k_off[4 * (g & 1) + i] + (g >> 1) * 32 * kTileD * 2);
     };
     auto read_v = [&](int tt) {
 #pragma unroll
@@ -166,164 +146,123 @@ __global__ __launch_bounds__(512, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
         vhi[tt][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(vt + v_off[db][1] + tt * 16 * kTileD * 2));
       }
     };
-    auto mfma_stage = [&](int g) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (QK) {
-          const int c = i & 1, ks = 2 * g + (i >> 1);
-          s_acc[c] = mfma32(kf[g][i], qreg[ks], s_acc[c]);
-        }
-        if (PV) o_acc[i] = mfma32(join_tr(vlo[g][i], vhi[g][i]), p[g], o_acc[i]);
-      }
-    };
-#define FA_INTERLEAVE(N_MFMA, READS)                                   \
-  _Pragma("unroll") for (int i_ = 0; i_ < (N_MFMA); ++i_) {            \
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 \
-    __builtin_amdgcn_sched_group_barrier(0x100, (READS), 0);           \
-  }
-    if (QK) {
+    for (int c = 0; c < 2; ++c)
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) s_acc[c][e] = 0.f;
-      read_k(0);
-    }
-    if (PV) read_v(0);
+      for (int e = 0; e < 16; ++e) s_acc[c][e] = 0.f;
+    read_k(0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       if (g < 3) {
-        if (QK) read_k(g + 1);
-        if (PV) read_v(g + 1);
+        read_k(g + 1);
+      } else {
+        read_v(0);
       }
-      mfma_stage(g);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s_acc[g >> 1] = mfma32(kf[g][i], qreg[4 * (g & 1) + i], s_acc[g >> 1]);
       if (g < 3) {
-        if (QK && PV) {
-          FA_INTERLEAVE(8, 2)   // 4 + 8 reads behind 8 MFMAs (the last group takes what is left)
-        } else if (QK) {
-          FA_INTERLEAVE(4, 1)
-        } else {
-          FA_INTERLEAVE(4, 2)
-        }
+        FA_INTERLEAVE(4, 1)
+      } else {
+        FA_INTERLEAVE(4, 2)
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-  };
+    read_v(1);
 
-  // VALU phase of step t: score mod, mask, online softmax -> P(t).
-  auto valu_phase = [&](int t) {
-    {
-      // For the plain score the running maximum is kept on the raw dot products and the scale is
-      // folded into the exponent (one FMA per element); score mods go through the log2-domain logit.
-      const int entry = __builtin_amdgcn_readfirstlane(sList[t]);
-      const int kv0 = (entry & 0xFFFFFF) * BN;
-      const bool partial = (entry >> 24) == 1;
-      constexpr bool kPlain = (SCORE == FLEXATTN_SCORE_NONE);
-      float m_tile = kNegInf;
-      if (!partial) {
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            if (!kPlain) s_acc[c][e] = sm.to_log2(s_acc[c][e], q_idx, kv0 + 32 * c + acc_row(e, hh));
-            m_tile = fmaxf(m_tile, s_acc[c][e]);
-          }
-        }
-      } else {
-        // the lane's kv indices come in runs of 4: kv0 + 32c + 8g + 4hh + {0..3}
-        const bool has_doc = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const int j0 = kv0 + 32 * c + 8 * g + 4 * hh;
-            int dj[4] = {0, 0, 0, 0};
-            if (has_doc) {
-              const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_k + j0);
-              dj[0] = d4[0]; dj[1] = d4[1]; dj[2] = d4[2]; dj[3] = d4[3];
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-              const int e = 4 * g + u;
-              float tv = kPlain ? s_acc[c][e] : sm.to_log2(s_acc[c][e], q_idx, j0 + u);
-              tv = keep_elem(a.mask, q_idx, j0 + u, doc_i, dj[u]) ? tv : kNegInf;
-              s_acc[c][e] = tv;
-              m_tile = fmaxf(m_tile, tv);
-            }
-          }
-        }
-      }
-      m_tile = half_max(m_tile);
-      const float m_new = fmaxf(m_run, m_tile);
-      const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
-      const float e_scale = kPlain ? sm.c2 : 1.0f;  // exponent = e_scale * (s - m)
-      // Rescale the accumulators only when some row's maximum moved (wave-uniform test).
-      if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
-        const float alpha = fast_exp2((m_run - m_safe) * e_scale);
-        l_run *= alpha;
-#pragma unroll
-        for (int db = 0; db < 4; ++db)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) o_acc[db][e] *= alpha;
-        m_run = m_new;
-      }
-      const float neg_m = -m_safe * e_scale;
-      float l_tile = 0.f;
-      const bf16x2 ones2 = {(bf16_t)1.0f, (bf16_t)1.0f};
+    // ---- score mod, mask, online softmax ----
+    // For the plain score the running maximum is kept on the raw dot products and the scale is
+    // folded into the exponent (one FMA per element); score mods go through the log2-domain logit.
+    const int kv0 = kb * BN;
+    constexpr bool kPlain = (SCORE == FLEXATTN_SCORE_NONE);
+    float m_tile = kNegInf;
+    if (!partial) {
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
 #pragma unroll
-        for (int e = 0; e < 16; e += 2) {
-          float p0, p1;
-          if (kPlain) {
-            p0 = fast_exp2(__builtin_fmaf(s_acc[c][e], e_scale, neg_m));
-            p1 = fast_exp2(__builtin_fmaf(s_acc[c][e + 1], e_scale, neg_m));
-          } else {
-            p0 = fast_exp2(s_acc[c][e] + neg_m);
-            p1 = fast_exp2(s_acc[c][e + 1] + neg_m);
-          }
-          bf16x2 pk = pack_bf16(p0, p1);
-          l_tile = __builtin_amdgcn_fdot2_f32_bf16(pk, ones2, l_tile, false);  // sums what P V will use
-          p[2 * c + (e >> 3)][e & 7] = pk[0];
-          p[2 * c + (e >> 3)][(e & 7) + 1] = pk[1];
+        for (int e = 0; e < 16; ++e) {
+          if (!kPlain) s_acc[c][e] = sm.to_log2(s_acc[c][e], q_idx, kv0 + 32 * c + acc_row(e, hh));
+          m_tile = fmaxf(m_tile, s_acc[c][e]);
         }
       }
-      l_run += l_tile;
+    } else {
+      // the lane's kv indices come in runs of 4: kv0 + 32c + 8g + 4hh + {0..3}
+      const bool has_doc = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int j0 = kv0 + 32 * c + 8 * g + 4 * hh;
+          int dj[4] = {0, 0, 0, 0};
+          if (has_doc) {
+            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_k + j0);
+            dj[0] = d4[0]; dj[1] = d4[1]; dj[2] = d4[2]; dj[3] = d4[3];
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int e = 4 * g + u;
+            float tv = kPlain ? s_acc[c][e] : sm.to_log2(s_acc[c][e], q_idx, j0 + u);
+            tv = keep_elem(a.mask, q_idx, j0 + u, doc_i, dj[u]) ? tv : kNegInf;
+            s_acc[c][e] = tv;
+            m_tile = fmaxf(m_tile, tv);
+          }
+        }
+      }
     }
-  };
+    m_tile = half_max(m_tile);
+    const float m_new = fmaxf(m_run, m_tile);
+    const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
+    const float e_scale = kPlain ? sm.c2 : 1.0f;  // exponent = e_scale * (s - m)
+    // Rescale the accumulators only when some row's maximum moved (wave-uniform test).
+    if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+      const float alpha = fast_exp2((m_run - m_safe) * e_scale);
+      l_run *= alpha;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o_acc[db][e] *= alpha;
+      m_run = m_new;
+    }
+    const float neg_m = -m_safe * e_scale;
+    float l_tile = 0.f;
+    const bf16x2 ones2 = {(bf16_t)1.0f, (bf16_t)1.0f};
+    bf16x8 p[4];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+#pragma unroll
+      for (int e = 0; e < 16; e += 2) {
+        float p0, p1;
+        if (kPlain) {
+          p0 = fast_exp2(__builtin_fmaf(s_acc[c][e], e_scale, neg_m));
+          p1 = fast_exp2(__builtin_fmaf(s_acc[c][e + 1], e_scale, neg_m));
+        } else {
+          p0 = fast_exp2(s_acc[c][e] + neg_m);
+          p1 = fast_exp2(s_acc[c][e + 1] + neg_m);
+        }
+        bf16x2 pk = pack_bf16(p0, p1);
+        l_tile = __builtin_amdgcn_fdot2_f32_bf16(pk, ones2, l_tile, false);  // sums what P V will use
+        p[2 * c + (e >> 3)][e & 7] = pk[0];
+        p[2 * c + (e >> 3)][(e & 7) + 1] = pk[1];
+      }
+    }
+    l_run += l_tile;
 
-  // One step = MFMA phase, barrier, VALU phase, barrier.  Loads are issued at even half steps by
-  // both groups: the leading group at the start of its MFMA phase, the trailing group at the start
-  // of its VALU phase; each group waits for its loads right before the barrier that ends the
-  // following (odd) half step.
-  auto end_mfma = [&]() {
-    if (grp == 1) wait_vmem_all();
-    __builtin_amdgcn_s_barrier();
-  };
-  auto end_valu = [&]() {
-    if (grp == 0) wait_vmem_all();
-    __builtin_amdgcn_s_barrier();
-  };
-  if (T > 0) {
-    if (grp == 0) issue_loads(0);
-    mfma_phase(0, std::true_type{}, std::false_type{});
-    end_mfma();
-    if (grp == 1) issue_loads(1);
-    valu_phase(0);
-    end_valu();
-    for (int t = 1; t < T; ++t) {
-      if (grp == 0) issue_loads(t);
-      mfma_phase(t, std::true_type{}, std::true_type{});
-      end_mfma();
-      if (grp == 1) issue_loads(t + 1);
-      valu_phase(t);
-      end_valu();
+    // ---- O^T += V^T P^T ----
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+      if (tt < 2) read_v(tt + 2);
+#pragma unroll
+      for (int db = 0; db < 4; ++db) o_acc[db] = mfma32(join_tr(vlo[tt][db], vhi[tt][db]), p[tt], o_acc[db]);
+      if (tt < 2) { FA_INTERLEAVE(4, 2) }
+      __builtin_amdgcn_sched_barrier(0);
     }
-    mfma_phase(T, std::false_type{}, std::true_type{});
-    end_mfma();
-    end_valu();
+
+    kb_cur = kb_nxt; kb_nxt = kb_n2; kb_n2 = kb_n3;
+    st_cur = st_nxt; st_nxt = st_n2;
+    wait_vmem_all();
+    __syncthreads();
   }
-  if (grp == 0) __builtin_amdgcn_s_barrier();  // both groups execute the same number of barriers
 
   // ---- epilogue ----
   const float l_tot = half_sum(l_run);
@@ -348,14 +287,12 @@ __global__ __launch_bounds__(512, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
 template <int SCORE>
 static int launch_fwd(const FwdArgs& a, hipStream_t stream) {
   using namespace fwd_cfg;
-  if (a.map.nk > LIST_CAP)
-    return set_error(FLEXATTN_ENOTSUP, "bf16 forward: Sk=%d exceeds %d (tile list capacity)", a.Sk, LIST_CAP * BN);
   auto kern = fwd_bf16_d128_kernel<SCORE>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(fwd): %s", hipGetErrorString(attr));
   const int n_wg = a.B * a.Hq * (a.Sq / BM);
-  hipLaunchKernelGGL(kern, dim3(n_wg), dim3(THREADS), LDS_BYTES, stream, a);
+  hipLaunchKernelGGL(kern, dim3(n_wg), dim3(256), LDS_BYTES, stream, a);
   return check_launch("flexattn_fwd bf16");
 }
 
