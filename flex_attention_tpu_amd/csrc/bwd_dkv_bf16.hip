@@ -1,15 +1,19 @@
 // Flex-attention dk/dv backward, bf16, head dim 128, gfx950.
 //
 // One work-group = 4 waves = one 128-row KV tile of one (batch, kv head); each wave owns 32 kv
-// rows, whose K and V stay in registers as MFMA B operands.  Q / dO tiles of 64 rows (with their
-// lse and delta) stream through double-buffered LDS, for every query head of the KV group and
-// every q tile the transposed block map lists.  Per tile:
+// rows, whose K and V stay in registers as MFMA B operands.  Q / dO tiles of 64 rows stream
+// through double-buffered LDS (LDS-direct loads, swizzled unpadded tiles) together with their
+// lse and delta, for every query head of the KV group and every q tile the transposed block map
+// lists.  Per tile:
 //   S = Q K^T,  dP = dO V^T   (lane owns a kv column, accumulator rows are q),
 //   P = exp2(S' - lse_q),  dS = P (dP - delta_q) f'(S),
 //   dv^T += dO^T P,  dk^T += Q^T dS   (dO^T, Q^T via transposing LDS reads).
 // Each dk/dv tile has exactly one writer, so the result is deterministic and needs no atomics.
 #include "fa_common.hpp"
 #include "launch.hpp"
+#include "tile_io.hpp"
+
+#include <type_traits>
 
 namespace fa {
 
@@ -17,18 +21,16 @@ namespace dkv_cfg {
 constexpr int BNK = 128;  // kv rows per work-group
 constexpr int BQ = 64;    // q rows per step
 constexpr int D = 128;
-constexpr int QSTR = D + 24;  // 304 B rows: conflict-free for b128 row reads and transposing reads
-constexpr int Q_TILE = BQ * QSTR;
-constexpr int LDS_BYTES = 2 * (2 * Q_TILE * 2 + 2 * BQ * 4);
+constexpr int LDS_BYTES = 4 * kTileElems * 2 + 4 * BQ * 4;  // Q x2, dO x2, lse x2, delta x2
 }  // namespace dkv_cfg
 
 template <int SCORE>
 __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
   using namespace dkv_cfg;
-  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   bf16_t* sQ = reinterpret_cast<bf16_t*>(smem_raw);
-  bf16_t* sDO = sQ + 2 * Q_TILE;
-  float* sLse = reinterpret_cast<float*>(sDO + 2 * Q_TILE);
+  bf16_t* sDO = sQ + 2 * kTileElems;
+  float* sLse = reinterpret_cast<float*>(sDO + 2 * kTileElems);
   float* sDl = sLse + 2 * BQ;
 
   const int nKb = a.Sk / BNK;
@@ -42,7 +44,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
   const int group = a.Hq / a.Hkv;
 
   const int tid = threadIdx.x;
-  const int w = tid >> 6;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int l32 = lane & 31;
   const int hh = lane >> 5;
@@ -52,6 +54,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
   const size_t kv_off = ((size_t)bhk * a.Sk + (size_t)kb * BNK) * D;
   const bf16_t* Kg = static_cast<const bf16_t*>(a.k) + kv_off;
   const bf16_t* Vg = static_cast<const bf16_t*>(a.v) + kv_off;
+  const bf16_t* Qall = static_cast<const bf16_t*>(a.q);
+  const bf16_t* dOall = static_cast<const bf16_t*>(a.dout);
 
   bf16x8 kreg[8], vreg[8];
 #pragma unroll
@@ -75,62 +79,71 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
   const int* tile_idx = a.map.idx + (size_t)kb * nQ;
   const int n_iter = n_tiles * group;
 
-  const int cp_chunk = tid & 15;
-  const int cp_row = tid >> 4;
-  bf16x8 qst[4], dost[4];
+  // Iteration `it` covers q tile tile_idx[it % n_tiles] of query head hk*group + it / n_tiles.
+  // Its q block index is fetched two iterations ahead, its state one iteration ahead.
+  auto q_block_of = [&](int it) { return tile_idx[it % n_tiles]; };
+  int qb_cur = 0, qb_nxt = 0, st_cur = 0;
+  if (n_iter > 0) qb_cur = q_block_of(0);
+  if (n_iter > 1) qb_nxt = q_block_of(1);
+  if (n_iter > 0) st_cur = a.map.state[(size_t)qb_cur * a.map.nk + kb];
+
+  TileLoader<4> loader;
+  loader.init(w, lane);
   float lse_st = 0.f, dl_st = 0.f;
-  auto g_load = [&](int it) {
+  auto issue_tile = [&](int it, int qb, int buf) {
     const int g = it / n_tiles;
-    const int qb = tile_idx[it - g * n_tiles];
     const size_t rbase = ((size_t)(b * a.Hq + hk * group + g) * a.Sq + (size_t)qb * BQ);
-    const bf16_t* qp = static_cast<const bf16_t*>(a.q) + (rbase + cp_row) * D + cp_chunk * 8;
-    const bf16_t* dp = static_cast<const bf16_t*>(a.dout) + (rbase + cp_row) * D + cp_chunk * 8;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      qst[j] = *reinterpret_cast<const bf16x8*>(qp + (size_t)j * 16 * D);
-      dost[j] = *reinterpret_cast<const bf16x8*>(dp + (size_t)j * 16 * D);
-    }
+    loader.load(Qall + rbase * D, sQ + buf * kTileElems);
+    loader.load(dOall + rbase * D, sDO + buf * kTileElems);
     if (tid < BQ) {
       const float l_i = a.l[rbase + tid], m_i = a.m[rbase + tid];
       lse_st = (l_i > 0.f) ? __builtin_fmaf(m_i, kLog2e, log2f(l_i)) : __builtin_huge_valf();
       dl_st = a.delta[rbase + tid];
     }
   };
-  auto s_store = [&](int buf) {
-    bf16_t* qd = sQ + buf * Q_TILE + cp_row * QSTR + cp_chunk * 8;
-    bf16_t* dd = sDO + buf * Q_TILE + cp_row * QSTR + cp_chunk * 8;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      *reinterpret_cast<bf16x8*>(qd + j * 16 * QSTR) = qst[j];
-      *reinterpret_cast<bf16x8*>(dd + j * 16 * QSTR) = dost[j];
-    }
+  auto store_rows = [&](int buf) {
     if (tid < BQ) {
       sLse[buf * BQ + tid] = lse_st;
       sDl[buf * BQ + tid] = dl_st;
     }
   };
-
   if (n_iter > 0) {
-    g_load(0);
-    s_store(0);
+    issue_tile(0, __builtin_amdgcn_readfirstlane(qb_cur), 0);
+    store_rows(0);
   }
+  wait_vmem_all();
   __syncthreads();
+
+  // lane-constant byte offsets of the operand reads inside a tile (see tile_io.hpp)
+  const int r_sw = swz(l32);
+  const int t_row = 4 * hh + ((lane & 15) >> 2);
+  const int t_chunk = 2 * ((lane & 31) >> 4) + ((lane & 3) >> 1);
+  const int t_half = 4 * (lane & 1);
+  unsigned r_off[8], t_off[4][2];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) r_off[ks] = (unsigned)(l32 * kTileD + (((2 * ks + hh) ^ r_sw) << 3)) * 2u;
+#pragma unroll
+  for (int db = 0; db < 4; ++db) {
+    t_off[db][0] = (unsigned)(tile_off(t_row, 4 * db + t_chunk) + t_half) * 2u;
+    t_off[db][1] = (unsigned)(tile_off(t_row + 8, 4 * db + t_chunk) + t_half) * 2u;
+  }
 
   ScoreMod<SCORE> sm;
   for (int it = 0; it < n_iter; ++it) {
     const int buf = it & 1;
-    const int g = it / n_tiles;
-    const int qb = tile_idx[it - g * n_tiles];
-    const bool partial = a.map.state[(size_t)qb * a.map.nk + kb] == 1;
-    sm.init(a.score, a.sm_scale, hk * group + g);
-    if (it + 1 < n_iter) g_load(it + 1);
+    const int qb = __builtin_amdgcn_readfirstlane(qb_cur);
+    const bool partial = __builtin_amdgcn_readfirstlane(st_cur) == 1;
+    sm.init(a.score, a.sm_scale, hk * group + it / n_tiles);
+    const int qb_n2 = (it + 2 < n_iter) ? q_block_of(it + 2) : 0;
+    int st_nxt = 0;
+    if (it + 1 < n_iter) {
+      const int qbn = __builtin_amdgcn_readfirstlane(qb_nxt);
+      st_nxt = a.map.state[(size_t)qbn * a.map.nk + kb];
+      issue_tile(it + 1, qbn, buf ^ 1);
+    }
     const int q0 = qb * BQ;
-
-    const bf16_t* qbase = sQ + buf * Q_TILE + l32 * QSTR + hh * 8;
-    const bf16_t* dobase = sDO + buf * Q_TILE + l32 * QSTR + hh * 8;
-    const int tr_off = (4 * hh + ((lane & 15) >> 2)) * QSTR + 16 * ((lane & 31) >> 4) + 4 * (lane & 3);
-    const bf16_t* qtbase = sQ + buf * Q_TILE + tr_off;
-    const bf16_t* dotbase = sDO + buf * Q_TILE + tr_off;
+    const char* qt = reinterpret_cast<const char*>(sQ + buf * kTileElems);
+    const char* dot = reinterpret_cast<const char*>(sDO + buf * kTileElems);
 
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
@@ -140,63 +153,90 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
         s_acc[e] = 0.f;
         dp_acc[e] = 0.f;
       }
+      {
+        bf16x8 qf[8];
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        bf16x8 qf = *reinterpret_cast<const bf16x8*>(qbase + c * 32 * QSTR + ks * 16);
-        s_acc = mfma32(qf, kreg[ks], s_acc);
+        for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qt + r_off[ks] + c * 32 * kTileD * 2);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) s_acc = mfma32(qf[ks], kreg[ks], s_acc);
       }
+      {
+        bf16x8 df[8];
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        bf16x8 df = *reinterpret_cast<const bf16x8*>(dobase + c * 32 * QSTR + ks * 16);
-        dp_acc = mfma32(df, vreg[ks], dp_acc);
+        for (int ks = 0; ks < 8; ++ks) df[ks] = *reinterpret_cast<const bf16x8*>(dot + r_off[ks] + c * 32 * kTileD * 2);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) dp_acc = mfma32(df[ks], vreg[ks], dp_acc);
       }
-      bf16x8 pb[2], dsb[2];
+      // transposed fragments of this 32-row q block for the dv / dk products
+      s16x4 dolo[2][4], dohi[2][4], qlo[2][4], qhi[2][4];
 #pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4) {
-        const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sLse + buf * BQ + 32 * c + 8 * g4 + 4 * hh);
-        const f32x4 dl4 = *reinterpret_cast<const f32x4*>(sDl + buf * BQ + 32 * c + 8 * g4 + 4 * hh);
-        float pv[4], dsv[4];
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int e = 4 * g4 + u;
-          const int i = q0 + 32 * c + 8 * g4 + 4 * hh + u;
-          float tv = sm.to_log2(s_acc[e], i, k_idx);
-          bool keep = true;
-          if (partial) {
-            int doc_i = 0;
-            if (a.mask.flags & FLEXATTN_MASK_DOC) doc_i = a.mask.doc_q[i];
-            keep = keep_elem(a.mask, i, k_idx, doc_i, doc_j);
-          }
-          const float p = fast_exp2(tv - lse4[u]);
-          const float gd = p * (dp_acc[e] - dl4[u]) * sm.dfactor(tv);
-          pv[u] = keep ? p : 0.f;
-          dsv[u] = keep ? gd : 0.f;
+        for (int db = 0; db < 4; ++db) {
+          const int off = (32 * c + 16 * u) * kTileD * 2;
+          dolo[u][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(dot + t_off[db][0] + off));
+          dohi[u][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(dot + t_off[db][1] + off));
+          qlo[u][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(qt + t_off[db][0] + off));
+          qhi[u][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(qt + t_off[db][1] + off));
         }
-        bf16x2 p01 = pack_bf16(pv[0], pv[1]), p23 = pack_bf16(pv[2], pv[3]);
-        bf16x2 d01 = pack_bf16(dsv[0], dsv[1]), d23 = pack_bf16(dsv[2], dsv[3]);
-        const int o = 4 * (g4 & 1);
-        pb[g4 >> 1][o] = p01[0]; pb[g4 >> 1][o + 1] = p01[1]; pb[g4 >> 1][o + 2] = p23[0]; pb[g4 >> 1][o + 3] = p23[1];
-        dsb[g4 >> 1][o] = d01[0]; dsb[g4 >> 1][o + 1] = d01[1]; dsb[g4 >> 1][o + 2] = d23[0]; dsb[g4 >> 1][o + 3] = d23[1];
+
+      bf16x8 pb[2], dsb[2];
+      auto elementwise = [&](auto masked) {
+        constexpr bool MASKED = decltype(masked)::value;
+        const bool has_doc = MASKED && (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int r0 = 32 * c + 8 * g4 + 4 * hh;  // the lane's q rows come in runs of 4
+          const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sLse + buf * BQ + r0);
+          const f32x4 dl4 = *reinterpret_cast<const f32x4*>(sDl + buf * BQ + r0);
+          int di[4] = {0, 0, 0, 0};
+          if (MASKED && has_doc) {
+            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_q + q0 + r0);
+            di[0] = d4[0]; di[1] = d4[1]; di[2] = d4[2]; di[3] = d4[3];
+          }
+          float pv[4], dsv[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int e = 4 * g4 + u;
+            const int i = q0 + r0 + u;
+            const float tv = sm.to_log2(s_acc[e], i, k_idx);
+            float pe = fast_exp2(tv - lse4[u]);
+            float gd = pe * (dp_acc[e] - dl4[u]) * sm.dfactor(tv);
+            if (MASKED) {
+              const bool keep = keep_elem(a.mask, i, k_idx, di[u], doc_j);
+              pe = keep ? pe : 0.f;
+              gd = keep ? gd : 0.f;
+            }
+            pv[u] = pe;
+            dsv[u] = gd;
+          }
+          const bf16x2 p01 = pack_bf16(pv[0], pv[1]), p23 = pack_bf16(pv[2], pv[3]);
+          const bf16x2 d01 = pack_bf16(dsv[0], dsv[1]), d23 = pack_bf16(dsv[2], dsv[3]);
+          const int o = 4 * (g4 & 1);
+          pb[g4 >> 1][o] = p01[0]; pb[g4 >> 1][o + 1] = p01[1]; pb[g4 >> 1][o + 2] = p23[0]; pb[g4 >> 1][o + 3] = p23[1];
+          dsb[g4 >> 1][o] = d01[0]; dsb[g4 >> 1][o + 1] = d01[1]; dsb[g4 >> 1][o + 2] = d23[0]; dsb[g4 >> 1][o + 3] = d23[1];
+        }
+      };
+      if (partial) {
+        elementwise(std::true_type{});
+      } else {
+        elementwise(std::false_type{});
       }
+
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        const int tt = 2 * c + u;  // 16-row q group inside the 64-row tile
 #pragma unroll
         for (int db = 0; db < 4; ++db) {
-          const bf16_t* dp = dotbase + (16 * tt) * QSTR + 32 * db;
-          bf16x8 dof = join_tr(lds_read_tr16(dp), lds_read_tr16(dp + 8 * QSTR));
-          dv_acc[db] = mfma32(dof, pb[u], dv_acc[db]);
-        }
-#pragma unroll
-        for (int db = 0; db < 4; ++db) {
-          const bf16_t* qp = qtbase + (16 * tt) * QSTR + 32 * db;
-          bf16x8 qf = join_tr(lds_read_tr16(qp), lds_read_tr16(qp + 8 * QSTR));
-          dk_acc[db] = mfma32(qf, dsb[u], dk_acc[db]);
+          dv_acc[db] = mfma32(join_tr(dolo[u][db], dohi[u][db]), pb[u], dv_acc[db]);
+          dk_acc[db] = mfma32(join_tr(qlo[u][db], qhi[u][db]), dsb[u], dk_acc[db]);
         }
       }
     }
 
-    if (it + 1 < n_iter) s_store(buf ^ 1);
+    qb_cur = qb_nxt; qb_nxt = qb_n2;
+    st_cur = st_nxt;
+    if (it + 1 < n_iter) store_rows(buf ^ 1);
+    wait_vmem_all();
     __syncthreads();
   }
 

@@ -1,12 +1,16 @@
 // Flex-attention dq backward, bf16, head dim 128, gfx950.
 //
 // Same decomposition as the forward: one work-group = 4 waves = one 128-row Q tile, 32 q rows per
-// wave, kv tiles of 64 rows double-buffered in LDS, everything computed transposed so that a lane
-// owns one q row:   S^T = K Q^T,  dP^T = V dO^T,  P = exp2(S' - lse),  dS = P (dP - delta) f'(S),
-// dq^T += K^T dS^T.  K is read twice from LDS: row-wise for S^T and with transposing reads for
-// the K^T operand of the dq product.
+// wave, kv tiles of 64 rows double-buffered in LDS by LDS-direct loads (swizzled, unpadded tiles),
+// everything computed transposed so that a lane owns one q row:
+//   S^T = K Q^T,  dP^T = V dO^T,  P = exp2(S' - lse),  dS = P (dP - delta) f'(S),  dq^T += K^T dS^T.
+// K is read twice from LDS: row-wise for S^T and with transposing reads for the K^T operand of
+// the dq product.  Q and dO stay in registers as MFMA B operands.
 #include "fa_common.hpp"
 #include "launch.hpp"
+#include "tile_io.hpp"
+
+#include <type_traits>
 
 namespace fa {
 
@@ -14,19 +18,15 @@ namespace dq_cfg {
 constexpr int BM = 128;
 constexpr int BN = 64;
 constexpr int D = 128;
-constexpr int KSTR = D + 24;  // 304 B rows: conflict-free for both b128 row reads and transposing reads
-constexpr int VSTR = D + 8;   // 272 B rows: V is only read row-wise
-constexpr int K_TILE = BN * KSTR;
-constexpr int V_TILE = BN * VSTR;
-constexpr int LDS_BYTES = 2 * (K_TILE + V_TILE) * 2;
+constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2
 }  // namespace dq_cfg
 
 template <int SCORE>
 __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
   using namespace dq_cfg;
-  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   bf16_t* sK = reinterpret_cast<bf16_t*>(smem_raw);
-  bf16_t* sV = sK + 2 * K_TILE;
+  bf16_t* sV = sK + 2 * kTileElems;
 
   const int nQ = a.Sq / BM;
   const int nK = a.map.nk;
@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
   const int hk = h / (a.Hq / a.Hkv);
 
   const int tid = threadIdx.x;
-  const int w = tid >> 6;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int l32 = lane & 31;
   const int hh = lane >> 5;
@@ -80,99 +80,133 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) dq_acc[i][e] = 0.f;
 
-  const int cp_chunk = tid & 15;
-  const int cp_row = tid >> 4;
-  bf16x8 kst[4], vst[4];
-  auto g_load = [&](int kb) {
-    const bf16_t* kp = Kg + ((size_t)kb * BN + cp_row) * D + cp_chunk * 8;
-    const bf16_t* vp = Vg + ((size_t)kb * BN + cp_row) * D + cp_chunk * 8;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      kst[j] = *reinterpret_cast<const bf16x8*>(kp + (size_t)j * 16 * D);
-      vst[j] = *reinterpret_cast<const bf16x8*>(vp + (size_t)j * 16 * D);
-    }
-  };
-  auto s_store = [&](int buf) {
-    bf16_t* kd = sK + buf * K_TILE + cp_row * KSTR + cp_chunk * 8;
-    bf16_t* vd = sV + buf * V_TILE + cp_row * VSTR + cp_chunk * 8;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      *reinterpret_cast<bf16x8*>(kd + j * 16 * KSTR) = kst[j];
-      *reinterpret_cast<bf16x8*>(vd + j * 16 * VSTR) = vst[j];
-    }
-  };
-
+  // Tile indices and states are fetched ahead of use (index three tiles, state two tiles ahead) so
+  // that no iteration waits on a load it has just issued.
+  int kb_cur = 0, kb_nxt = 0, kb_n2 = 0, st_cur = 0, st_nxt = 0;
+  if (n_tiles > 0) kb_cur = tile_idx[0];
+  if (n_tiles > 1) kb_nxt = tile_idx[1];
+  if (n_tiles > 2) kb_n2 = tile_idx[2];
+  if (n_tiles > 0) st_cur = tile_state[kb_cur];
+  if (n_tiles > 1) st_nxt = tile_state[kb_nxt];
+  TileLoader<4> loader;
+  loader.init(w, lane);
   if (n_tiles > 0) {
-    g_load(tile_idx[0]);
-    s_store(0);
+    const int kb0 = __builtin_amdgcn_readfirstlane(kb_cur);
+    loader.load(Kg + (size_t)kb0 * BN * D, sK);
+    loader.load(Vg + (size_t)kb0 * BN * D, sV);
   }
+  wait_vmem_all();
   __syncthreads();
+
+  // lane-constant byte offsets of the operand reads inside a tile (see tile_io.hpp)
+  const int k_sw = swz(l32);
+  const int t_row = 4 * hh + ((lane & 15) >> 2);
+  const int t_chunk = 2 * ((lane & 31) >> 4) + ((lane & 3) >> 1);
+  const int t_half = 4 * (lane & 1);
+  unsigned r_off[8], t_off[4][2];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) r_off[ks] = (unsigned)(l32 * kTileD + (((2 * ks + hh) ^ k_sw) << 3)) * 2u;
+#pragma unroll
+  for (int db = 0; db < 4; ++db) {
+    t_off[db][0] = (unsigned)(tile_off(t_row, 4 * db + t_chunk) + t_half) * 2u;
+    t_off[db][1] = (unsigned)(tile_off(t_row + 8, 4 * db + t_chunk) + t_half) * 2u;
+  }
 
   for (int t = 0; t < n_tiles; ++t) {
     const int buf = t & 1;
-    const int kb = tile_idx[t];
-    const bool partial = tile_state[kb] == 1;
-    if (t + 1 < n_tiles) g_load(tile_idx[t + 1]);
+    const int kb = __builtin_amdgcn_readfirstlane(kb_cur);
+    const bool partial = __builtin_amdgcn_readfirstlane(st_cur) == 1;
+    const int kb_n3 = (t + 3 < n_tiles) ? tile_idx[t + 3] : 0;
+    const int st_n2 = (t + 2 < n_tiles) ? tile_state[kb_n2] : 0;
+    if (t + 1 < n_tiles) {
+      const int kbn = __builtin_amdgcn_readfirstlane(kb_nxt);
+      loader.load(Kg + (size_t)kbn * BN * D, sK + (buf ^ 1) * kTileElems);
+      loader.load(Vg + (size_t)kbn * BN * D, sV + (buf ^ 1) * kTileElems);
+    }
     const int kv0 = kb * BN;
+    const char* kt = reinterpret_cast<const char*>(sK + buf * kTileElems);
+    const char* vt = reinterpret_cast<const char*>(sV + buf * kTileElems);
 
-    const bf16_t* kbase = sK + buf * K_TILE + l32 * KSTR + hh * 8;
-    const bf16_t* vbase = sV + buf * V_TILE + l32 * VSTR + hh * 8;
-    const bf16_t* ktbase = sK + buf * K_TILE + (4 * hh + ((lane & 15) >> 2)) * KSTR + 16 * ((lane & 31) >> 4) +
-                           4 * (lane & 3);
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
+      // ---- S^T and dP^T for kv rows [32c, 32c+32) ----
       f32x16 s_acc, dp_acc;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         s_acc[e] = 0.f;
         dp_acc[e] = 0.f;
       }
+      {
+        bf16x8 kf[8];
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        bf16x8 kf = *reinterpret_cast<const bf16x8*>(kbase + c * 32 * KSTR + ks * 16);
-        s_acc = mfma32(kf, qreg[ks], s_acc);
+        for (int ks = 0; ks < 8; ++ks) kf[ks] = *reinterpret_cast<const bf16x8*>(kt + r_off[ks] + c * 32 * kTileD * 2);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) s_acc = mfma32(kf[ks], qreg[ks], s_acc);
       }
+      {
+        bf16x8 vf[8];
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        bf16x8 vf = *reinterpret_cast<const bf16x8*>(vbase + c * 32 * VSTR + ks * 16);
-        dp_acc = mfma32(vf, doreg[ks], dp_acc);
+        for (int ks = 0; ks < 8; ++ks) vf[ks] = *reinterpret_cast<const bf16x8*>(vt + r_off[ks] + c * 32 * kTileD * 2);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) dp_acc = mfma32(vf[ks], doreg[ks], dp_acc);
       }
-      bf16x8 ds[2];
-#pragma unroll
-      for (int e = 0; e < 16; e += 2) {
-        float dsv[2];
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          const int j = kv0 + 32 * c + acc_row(e + u, hh);
-          float tv = sm.to_log2(s_acc[e + u], q_idx, j);
-          bool keep = true;
-          if (partial) {
-            int doc_j = 0;
-            if (a.mask.flags & FLEXATTN_MASK_DOC) doc_j = a.mask.doc_k[j];
-            keep = keep_elem(a.mask, q_idx, j, doc_i, doc_j);
-          }
-          const float p = fast_exp2(tv - lse2);
-          const float g = p * (dp_acc[e + u] - delta) * sm.dfactor(tv);
-          dsv[u] = keep ? g : 0.f;
-        }
-        bf16x2 pk = pack_bf16(dsv[0], dsv[1]);
-        ds[e >> 3][e & 7] = pk[0];
-        ds[e >> 3][(e & 7) + 1] = pk[1];
-      }
-      // dq^T += K^T dS^T for the two 16-row kv groups of this 32-row block
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int tt = 2 * c + u;
+      // K^T fragments for the dq product
+      s16x4 klo[2][4], khi[2][4];
+      auto read_kt = [&](int u) {
 #pragma unroll
         for (int db = 0; db < 4; ++db) {
-          const bf16_t* kp = ktbase + (16 * tt) * KSTR + 32 * db;
-          bf16x8 kf = join_tr(lds_read_tr16(kp), lds_read_tr16(kp + 8 * KSTR));
-          dq_acc[db] = mfma32(kf, ds[u], dq_acc[db]);
+          const int off = (32 * c + 16 * u) * kTileD * 2;
+          klo[u][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(kt + t_off[db][0] + off));
+          khi[u][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(kt + t_off[db][1] + off));
         }
+      };
+
+      // ---- P, dS -> bf16 ----
+      bf16x8 ds[2];
+      auto elementwise = [&](auto masked) {
+        constexpr bool MASKED = decltype(masked)::value;
+        const bool has_doc = MASKED && (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int j0 = kv0 + 32 * c + 8 * g + 4 * hh;
+          int dj[4] = {0, 0, 0, 0};
+          if (MASKED && has_doc) {
+            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_k + j0);
+            dj[0] = d4[0]; dj[1] = d4[1]; dj[2] = d4[2]; dj[3] = d4[3];
+          }
+          float dsv[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int e = 4 * g + u;
+            const float tv = sm.to_log2(s_acc[e], q_idx, j0 + u);
+            const float pe = fast_exp2(tv - lse2);
+            float gd = pe * (dp_acc[e] - delta) * sm.dfactor(tv);
+            if (MASKED) gd = keep_elem(a.mask, q_idx, j0 + u, doc_i, dj[u]) ? gd : 0.f;
+            dsv[u] = gd;
+          }
+          const bf16x2 d01 = pack_bf16(dsv[0], dsv[1]), d23 = pack_bf16(dsv[2], dsv[3]);
+          const int o = 4 * (g & 1);
+          ds[g >> 1][o] = d01[0]; ds[g >> 1][o + 1] = d01[1]; ds[g >> 1][o + 2] = d23[0]; ds[g >> 1][o + 3] = d23[1];
+        }
+      };
+      if (partial) {
+        elementwise(std::true_type{});
+      } else {
+        elementwise(std::false_type{});
       }
+
+      // ---- dq^T += K^T dS^T for the two 16-row kv groups of this block ----
+      read_kt(0);
+      read_kt(1);
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int db = 0; db < 4; ++db) dq_acc[db] = mfma32(join_tr(klo[u][db], khi[u][db]), ds[u], dq_acc[db]);
     }
 
-    if (t + 1 < n_tiles) s_store(buf ^ 1);
+    kb_cur = kb_nxt; kb_nxt = kb_n2; kb_n2 = kb_n3;
+    st_cur = st_nxt; st_nxt = st_n2;
+    wait_vmem_all();
     __syncthreads();
   }
 
