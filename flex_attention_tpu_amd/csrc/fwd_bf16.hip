@@ -119,11 +119,11 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
     const bool partial = __builtin_amdgcn_readfirstlane(st_cur) == 1;
     const int kb_n3 = (t + 3 < n_tiles) ? tile_idx[t + 3] : 0;
     const int st_n2 = (t + 2 < n_tiles) ? tile_state[kb_n2] : 0;
-    if (t + 1 < n_tiles) {
-      const int kbn = __builtin_amdgcn_readfirstlane(kb_nxt);
-      loader.load(Kg + (size_t)kbn * BN * D, sK + (buf ^ 1) * kTileElems);
-      loader.load(Vg + (size_t)kbn * BN * D, sV + (buf ^ 1) * kTileElems);
-    }
+    // The next tile's LDS-direct loads are issued two at a time between the MFMA stages below.
+    const bool prefetch = t + 1 < n_tiles;
+    const int kbn = __builtin_amdgcn_readfirstlane(kb_nxt);
+    const bf16_t* k_next = Kg + (size_t)kbn * BN * D;
+    const bf16_t* v_next = Vg + (size_t)kbn * BN * D;
 
     // ---- S^T = K Q^T : two 32(kv) x 32(q) accumulator tiles ----
     // LDS operand reads run one stage (4 MFMAs) ahead of the MFMAs that consume them, so the LDS
@@ -167,6 +167,10 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
         FA_INTERLEAVE(4, 2)
       }
       __builtin_amdgcn_sched_barrier(0);
+      if (prefetch) {
+        loader.load_block(k_next, sK + (buf ^ 1) * kTileElems, g);
+        loader.load_block(v_next, sV + (buf ^ 1) * kTileElems, g);
+      }
     }
     read_v(1);
 

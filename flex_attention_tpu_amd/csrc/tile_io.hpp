@@ -49,15 +49,19 @@ struct TileLoader {
   // destination buffer get a vmcnt(0) wait in front of them, which serialises the prefetch.  The
   // caller orders the copy itself with wait_vmem_all() + barrier before the tile is read.
   __device__ __forceinline__ void load(const bf16_t* g_tile, bf16_t* lds_tile) const {
-    const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)(lds_tile);
 #pragma unroll
-    for (int i = 0; i < kBlocks; ++i) {
-      const unsigned dst = lds_base + (unsigned)(wave * kBlocks + i) * 1024u;
-      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                   :
-                   : "v"(goff[i]), "s"(g_tile), "s"(dst)
-                   : "memory", "m0");
-    }
+    for (int i = 0; i < kBlocks; ++i) load_block(g_tile, lds_tile, i);
+  }
+
+  // One of the wave's kBlocks 1 KB blocks; lets a caller spread the load issue between other work
+  // (back-to-back LDS-direct loads occupy the issuing wave for tens of cycles each).
+  __device__ __forceinline__ void load_block(const bf16_t* g_tile, bf16_t* lds_tile, int i) const {
+    const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)(lds_tile);
+    const unsigned dst = lds_base + (unsigned)(wave * kBlocks + i) * 1024u;
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(goff[i]), "s"(g_tile), "s"(dst)
+                 : "memory", "m0");
   }
 };
 
