@@ -79,39 +79,50 @@ def main():
     def fwd():
         return F._flex_attention_impl(q, k, v, None, None, True, False, sc, 1, blk, blk, blk, False, bf, mf, sfn)
 
-    def step(ev=None):
-        if ev is not None:
-            ev[0].record()
+    def step():
         o, l, m = fwd()
-        if ev is not None:
-            ev[1].record()
         d = F.compute_delta(o, do)
-        if ev is not None:
-            ev[2].record()
         dq = F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=blk, block_k_major=blk,
                                      block_k=blk, sm_scale=sc, debug=False, score_fn=sfn, mask_fn=mf, block_mask_fn=bf)
-        if ev is not None:
-            ev[3].record()
         dk, dv = F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=blk, block_q_major=blk,
                                            block_k_major=blk, block_k=blk, sm_scale=sc, causal=False, debug=False,
                                            score_fn=sfn, mask_fn=mf, block_mask_fn=bf)
-        if ev is not None:
-            ev[4].record()
         return o, dq, dk, dv
 
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(events[i])
+        step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
 
-    names = ["fwd", "delta", "dq", "dkv"]
-    ms = {n: sum(events[i][j].elapsed_time(events[i][j + 1]) for i in range(args.steps)) / args.steps
-          for j, n in enumerate(names)}
+    # Per-kernel launch durations: K back-to-back launches of one kernel between two HIP events on
+    # the launch stream (single launches bracketed by events carry several us of marker overhead).
+    o, l, m = fwd()
+    d = F.compute_delta(o, do)
+    launches = {
+        "fwd": fwd,
+        "delta": lambda: F.compute_delta(o, do),
+        "dq": lambda: F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=blk,
+                                              block_k_major=blk, block_k=blk, sm_scale=sc, debug=False, score_fn=sfn,
+                                              mask_fn=mf, block_mask_fn=bf),
+        "dkv": lambda: F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=blk,
+                                                 block_q_major=blk, block_k_major=blk, block_k=blk, sm_scale=sc,
+                                                 causal=False, debug=False, score_fn=sfn, mask_fn=mf, block_mask_fn=bf),
+    }
+    ms = {}
+    for name_k, fn in launches.items():
+        fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ms[name_k] = e0.elapsed_time(e1) / args.steps
+
     ms_step = wall * 1e3 / args.steps
     f_fwd = configs.flops_fwd(cfg)
     f_bwd = 2.5 * f_fwd

@@ -1,7 +1,7 @@
 // Flex-attention dk/dv backward, bf16, head dim 128, gfx950.
 //
 // One work-group = 4 waves = one 128-row KV tile of one (batch, kv head); each wave owns 32 kv
-// rows, whose K and V stay in registers as MFMA B operands.  Q / dO tiles of 64 rows stream
+// rows, whose K and V stay in registers as MFMA B operands.  Q / dO tiles of 128 rows stream
 // through double-buffered LDS (LDS-direct loads, swizzled unpadded tiles) together with their
 // lse and delta, for every query head of the KV group and every q tile the transposed block map
 // lists.  Per tile:
@@ -19,9 +19,9 @@ namespace fa {
 
 namespace dkv_cfg {
 constexpr int BNK = 128;  // kv rows per work-group
-constexpr int BQ = 64;    // q rows per step
+constexpr int BQ = 128;   // q rows per step (two 64-row LDS tiles)
 constexpr int D = 128;
-constexpr int LDS_BYTES = 4 * kTileElems * 2 + 4 * BQ * 4;  // Q x2, dO x2, lse x2, delta x2
+constexpr int LDS_BYTES = 8 * kTileElems * 2 + 4 * BQ * 4;  // (Q, dO) x 2 buffers x 2 tiles, lse x2, delta x2
 }  // namespace dkv_cfg
 
 template <int SCORE>
@@ -29,8 +29,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
   using namespace dkv_cfg;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   bf16_t* sQ = reinterpret_cast<bf16_t*>(smem_raw);
-  bf16_t* sDO = sQ + 2 * kTileElems;
-  float* sLse = reinterpret_cast<float*>(sDO + 2 * kTileElems);
+  bf16_t* sDO = sQ + 4 * kTileElems;
+  float* sLse = reinterpret_cast<float*>(sDO + 4 * kTileElems);
   float* sDl = sLse + 2 * BQ;
 
   const int nKb = a.Sk / BNK;
@@ -93,8 +93,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
   auto issue_tile = [&](int it, int qb, int buf) {
     const int g = it / n_tiles;
     const size_t rbase = ((size_t)(b * a.Hq + hk * group + g) * a.Sq + (size_t)qb * BQ);
-    loader.load(Qall + rbase * D, sQ + buf * kTileElems);
-    loader.load(dOall + rbase * D, sDO + buf * kTileElems);
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      loader.load(Qall + (rbase + half * kTileRows) * D, sQ + (2 * buf + half) * kTileElems);
+      loader.load(dOall + (rbase + half * kTileRows) * D, sDO + (2 * buf + half) * kTileElems);
+    }
     if (tid < BQ) {
       const float l_i = a.l[rbase + tid], m_i = a.m[rbase + tid];
       lse_st = (l_i > 0.f) ? __builtin_fmaf(m_i, kLog2e, log2f(l_i)) : __builtin_huge_valf();
@@ -142,11 +145,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
       issue_tile(it + 1, qbn, buf ^ 1);
     }
     const int q0 = qb * BQ;
-    const char* qt = reinterpret_cast<const char*>(sQ + buf * kTileElems);
-    const char* dot = reinterpret_cast<const char*>(sDO + buf * kTileElems);
-
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
+    for (int cc = 0; cc < 4; ++cc) {
+      const int c = cc & 1;  // 32-row block inside the 64-row LDS tile cc >> 1
+      const char* qt = reinterpret_cast<const char*>(sQ + (2 * buf + (cc >> 1)) * kTileElems);
+      const char* dot = reinterpret_cast<const char*>(sDO + (2 * buf + (cc >> 1)) * kTileElems);
       f32x16 s_acc, dp_acc;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
@@ -186,7 +189,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
         const bool has_doc = MASKED && (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
-          const int r0 = 32 * c + 8 * g4 + 4 * hh;  // the lane's q rows come in runs of 4
+          const int r0 = 32 * cc + 8 * g4 + 4 * hh;  // the lane's q rows come in runs of 4
           const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sLse + buf * BQ + r0);
           const f32x4 dl4 = *reinterpret_cast<const f32x4*>(sDl + buf * BQ + r0);
           int di[4] = {0, 0, 0, 0};
