@@ -20,6 +20,12 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA peak
 PEAK_HBM_GBS = 8000.0
 
 
+# HBM bytes per launch on the default workload (cfg2), from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this script, each counter scaled by its reading for the 256 MiB device copy that
+# main() ends with (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Counter-derived, not measured per run.
+HBM_TRAFFIC_BYTES = {"fwd": 560272240, "dq": 682352053, "dkv": 812530413}
+
+
 def cpu_baseline(cfg, budget_s=12.0):
     """Times the CPU oracle (float32 math on the dtype-rounded inputs) on a bounded sample of the
     same workload: whole (batch, head) pairs of the configuration, forward + backward."""
@@ -123,6 +129,14 @@ def main():
         torch.cuda.synchronize()
         ms[name_k] = e0.elapsed_time(e1) / args.steps
 
+    # A plain device copy of known size (256 MiB read + 256 MiB written per launch): the reference
+    # dispatch that FETCH_SIZE / WRITE_SIZE counter readings of the attention kernels are scaled by.
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+
     ms_step = wall * 1e3 / args.steps
     f_fwd = configs.flops_fwd(cfg)
     f_bwd = 2.5 * f_fwd
@@ -136,7 +150,8 @@ def main():
     dom = max(algo, key=lambda n: ms[n])
     roofline = {
         "kernel": dom, "bound": "mfma", "achieved": tf(algo[dom], ms[dom]), "peak": PEAK_BF16_TFLOPS,
-        "unit": "TFLOP/s", "frac": tf(algo[dom], ms[dom]) / PEAK_BF16_TFLOPS, "traffic": None,
+        "unit": "TFLOP/s", "frac": tf(algo[dom], ms[dom]) / PEAK_BF16_TFLOPS,
+        "traffic": HBM_TRAFFIC_BYTES.get(dom) if name == "cfg2" else None,
         "launch_ms": ms[dom],
     }
     out = {
