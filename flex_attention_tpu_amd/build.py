@@ -22,6 +22,9 @@ SOURCES = [
     "bwd_dkv_bf16.hip",
 ]
 
+# instruction streams generated before compiling: (generator script, output it writes next to itself)
+GENERATED = [("gen_dkv_tile.py", "bwd_dkv_tile.inc")]
+
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950",
@@ -42,7 +45,7 @@ def _compile(src: str, force: bool) -> str:
     obj = os.path.join(BUILD_DIR, os.path.splitext(src)[0] + ".o")
     src_path = os.path.join(CSRC, src)
     if not force and os.path.exists(obj):
-        deps = [src_path] + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
+        deps = [src_path] + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hpp", ".inc"))]
         deps.append(os.path.join(INCLUDE, "flexattn.h"))
         if all(os.path.getmtime(d) <= os.path.getmtime(obj) for d in deps):
             return obj
@@ -59,6 +62,10 @@ def _compile(src: str, force: bool) -> str:
 def build_library(force: bool = True, jobs: int = 8) -> str:
     """Compiles every HIP source for gfx950 and links libflexattn.so next to the package."""
     os.makedirs(BUILD_DIR, exist_ok=True)
+    for gen, out in GENERATED:
+        r = subprocess.run([sys.executable, os.path.join(CSRC, gen), os.path.join(CSRC, out)], capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"{gen} failed:\n{r.stdout}\n{r.stderr}")
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(lambda s: _compile(s, force), SOURCES))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH]

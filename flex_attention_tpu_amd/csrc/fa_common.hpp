@@ -192,6 +192,17 @@ struct ScoreMod {
     }
     return scale;
   }
+
+  // dfactor() split into an element-wise part and a constant that a kernel may apply once to
+  // its accumulated result: dfactor(t) == dfactor_unscaled(t) * dfactor_post_scale(sm_scale).
+  __device__ __forceinline__ float dfactor_unscaled(float t) const {
+    if (KIND == FLEXATTN_SCORE_SOFTCAP) return dfactor(t);
+    return 1.0f;
+  }
+  __device__ __forceinline__ float dfactor_post_scale(float sm_scale) const {
+    if (KIND == FLEXATTN_SCORE_SOFTCAP) return 1.0f;
+    return sm_scale;
+  }
 };
 
 // XCD-aware work-group remap: consecutive hardware work-group ids go round-robin to the 8 XCDs,

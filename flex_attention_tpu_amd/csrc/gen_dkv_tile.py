@@ -1,0 +1,278 @@
+#!/usr/bin/env python3
+"""Generator of the hand-scheduled gfx950 instruction stream for one full (unmasked, plain-score)
+128 x 128 tile of the bf16 dk/dv kernel.  Writes bwd_dkv_tile.inc: string-literal macros (the stream for
+full tiles and the one for partially masked tiles, selected by a scalar branch inside one statement,
+plus prologue / epilogue register moves) that bwd_dkv_bf16.hip places inside `asm volatile` statements.
+
+Why generated assembly: with 128 accumulator and 64 K/V operand registers the kernel runs one wave
+per SIMD, so MFMA, VALU and LDS work only overlap if they are interleaved inside the wave, and the
+register budget only closes with a fixed allocation.  The stream below is a software pipeline over
+the tile's four 32-row q blocks c = 0..3:
+
+    A(c): S = Q K^T, dP = dO V^T         16 MFMAs, operands: 16 ds_read_b128 (rows of Q, dO)
+    E(c): P = exp2(S c2 - lse), dS = P (dP - delta)   80 VALU ops, 8 ds_read_b128 (lse, delta)
+    B(c): dv^T += dO^T P, dk^T += Q^T dS 16 MFMAs, operands: 32 ds_read_b64_tr_b16
+
+    MFMA order:  A0 | A1 | A2 B0 | A3 B1 | B2 | B3      VALU:  - | E0 | E1 | E2 | E3 | -
+
+LDS reads are issued PREFETCH MFMA pairs ahead of their use into a rotating pool of staging
+registers; the next step's Q / dO tiles are copied global -> LDS by 16 loads spread over the stream.
+The emitter (gfx950_stream.py) inserts the s_nop / s_waitcnt that the hardware hazards require.
+
+Register contract with the C++ side (every asm statement names the accumulation registers with
+physical-register constraints; prologue / epilogue macros are generated here too):
+    a[0:63]    dv accumulators (4 x 16)      a[64:127]  dk accumulators (4 x 16)
+    a[128:159] K fragments (8 x 4)           a[160:191] V fragments (8 x 4)
+    v[68:255]  scratch of this stream (clobbered)
+    %[r0..r7]  byte address of the lane's row fragment ks in the step's Q half-tile 0
+    %[t0..t7]  byte address of the lane's transposed fragment (2 db + hi) in Q half-tile 0
+    %[la]      byte address of the lane's first lse value of the step;  %[c2] sm_scale * log2(e)
+    %[partial] scalar, non-zero selects the masked stream
+    %[g0..g3]  the lane's byte offsets inside a global half tile for the wave's four 1 KB blocks;
+    %[gq0], %[gq1], %[gd0], %[gd1]  global addresses (SGPR pairs) of the next step's Q / dO half tiles;
+    %[ldsn]    LDS byte address of the wave's first block in the next step's buffer
+    %[m0], %[m1]  (masked stream only) the lane's keep bits: bit 16 (c & 1) + e of m[c >> 1] is
+               element e of the S accumulator of q block c; dropped elements get P = 0
+LDS layout of one step buffer (bytes): Q half 0, Q half 1, dO half 0, dO half 1 (16 KiB each);
+lse [128] floats, delta 1 KiB after it.
+"""
+import argparse
+import os
+import sys
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+from gfx950_stream import Emitter, ar, aset, vr, vset  # noqa: E402
+
+NSLOT = 8        # staging slots of 8 VGPRs
+PREFETCH = 4     # MFMA pairs between the LDS reads of a pair and its MFMAs
+LOAD_FIRST = 2   # MFMA slot of the first LDS-direct load of the next step
+LOAD_EVERY = 6   # slots between two of them
+DROP = ()        # instruction classes left out (--drop, timing studies only)
+
+TILE = 16384
+V_S = [72, 104]
+V_DP = [88, 120]
+V_PB = 136
+V_DSB = 152
+V_LSE = 168   # 3 buffers x 4
+V_DL = 180    # 3 buffers x 4
+V_STG = 192
+V_TMP = 68    # 4 temporaries of the masked variant
+DL_OFFSET = 1024
+
+
+def build(masked):
+    em = Emitter()
+    em._raw("s_waitcnt lgkmcnt(0)")
+
+    # ---- MFMA pairs in issue order -------------------------------------------------------
+    pairs = []
+    def add_A(c):
+        for ks in range(8):
+            pairs.append(("A", c, ks))
+    def add_B(c):
+        for u in range(2):
+            for db in range(4):
+                pairs.append(("B", c, (u, db)))
+    add_A(0)
+    stage_first_slot = {}
+    stage_first_slot[0] = 2 * len(pairs); add_A(1)
+    stage_first_slot[1] = 2 * len(pairs); add_A(2); add_B(0)
+    stage_first_slot[2] = 2 * len(pairs); add_A(3); add_B(1)
+    stage_first_slot[3] = 2 * len(pairs); add_B(2)
+    stage_end = 2 * len(pairs); add_B(3)
+    n_slots = 2 * len(pairs)
+    stage_last_slot = {0: stage_first_slot[1], 1: stage_first_slot[2], 2: stage_first_slot[3], 3: stage_end}
+
+    def half_off(c):
+        return (c >> 1) * TILE + (c & 1) * (TILE // 2)
+
+    def pair_loads(k):
+        kind, c, x = pairs[k]
+        base = V_STG + 8 * (k % NSLOT)
+        loads = []
+        if kind == "A":
+            ks = x
+            loads.append((f"ds_read_b128 {vr(base, 4)}, %[r{ks}] offset:{half_off(c)}", vset(base, 4)))
+            loads.append((f"ds_read_b128 {vr(base + 4, 4)}, %[r{ks}] offset:{2 * TILE + half_off(c)}", vset(base + 4, 4)))
+        else:
+            u, db = x
+            off = half_off(c) + u * 4096
+            for which, reg0 in ((2 * TILE, base), (0, base + 4)):  # dO fragment, then Q fragment
+                for hi in range(2):
+                    loads.append((f"ds_read_b64_tr_b16 {vr(reg0 + 2 * hi, 2)}, %[t{2 * db + hi}] offset:{which + off}",
+                                  vset(reg0 + 2 * hi, 2)))
+        return loads
+
+    def pair_mfmas(k):
+        kind, c, x = pairs[k]
+        base = V_STG + 8 * (k % NSLOT)
+        if kind == "A":
+            ks = x
+            s, dp = V_S[c & 1], V_DP[c & 1]
+            cs = "0" if ks == 0 else vr(s, 16)
+            cd = "0" if ks == 0 else vr(dp, 16)
+            return [
+                (vr(s, 16), vr(base, 4), ar(128 + 4 * ks, 4), cs, vset(s, 16), vset(base, 4), aset(128 + 4 * ks, 4),
+                 set() if ks == 0 else vset(s, 16)),
+                (vr(dp, 16), vr(base + 4, 4), ar(160 + 4 * ks, 4), cd, vset(dp, 16), vset(base + 4, 4),
+                 aset(160 + 4 * ks, 4), set() if ks == 0 else vset(dp, 16)),
+            ]
+        u, db = x
+        pb = V_PB + 8 * (c & 1) + 4 * u
+        dsb = V_DSB + 8 * (c & 1) + 4 * u
+        return [
+            (ar(16 * db, 16), vr(base, 4), vr(pb, 4), ar(16 * db, 16), aset(16 * db, 16), vset(base, 4), vset(pb, 4),
+             aset(16 * db, 16)),
+            (ar(64 + 16 * db, 16), vr(base + 4, 4), vr(dsb, 4), ar(64 + 16 * db, 16), aset(64 + 16 * db, 16),
+             vset(base + 4, 4), vset(dsb, 4), aset(64 + 16 * db, 16)),
+        ]
+
+    # ---- VALU work of E(c), spread over the MFMA slots of stage c ---------------------------
+    slot_valu = {m: [] for m in range(n_slots)}
+    slot_lds = {m: [] for m in range(n_slots)}
+    pre_lds = []
+    for c in range(4):
+        s, dp = V_S[c & 1], V_DP[c & 1]
+        ops = []
+        group_first_op = []
+        for g in range(4):
+            kbuf = (4 * c + g) % 3
+            lse, dl = V_LSE + 4 * kbuf, V_DL + 4 * kbuf
+            group_first_op.append(len(ops))
+            for u in range(4):
+                e = 4 * g + u
+                ops.append((f"v_fma_f32 {vr(s + e)}, {vr(s + e)}, %[c2], -{vr(lse + u)}", vset(s + e), vset(s + e) | vset(lse + u), False))
+            for u in range(4):
+                e = 4 * g + u
+                ops.append((f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
+            if masked:
+                # keep bit of element e of block c: bit 16 (c & 1) + e of %[m0] (c < 2) or %[m1]
+                for u in range(4):
+                    e = 4 * g + u
+                    tmp = V_TMP + u
+                    ops.append((f"v_bfe_i32 {vr(tmp)}, %[m{c >> 1}], {16 * (c & 1) + e}, 1", vset(tmp), set(), False))
+                for u in range(4):
+                    e = 4 * g + u
+                    tmp = V_TMP + u
+                    ops.append((f"v_and_b32_e32 {vr(s + e)}, {vr(s + e)}, {vr(tmp)}", vset(s + e), vset(s + e) | vset(tmp), False))
+            for u in range(4):
+                e = 4 * g + u
+                ops.append((f"v_sub_f32_e32 {vr(dp + e)}, {vr(dp + e)}, {vr(dl + u)}", vset(dp + e), vset(dp + e) | vset(dl + u), False))
+            for u in range(4):
+                e = 4 * g + u
+                ops.append((f"v_mul_f32_e32 {vr(dp + e)}, {vr(s + e)}, {vr(dp + e)}", vset(dp + e), vset(dp + e) | vset(s + e), False))
+            # bf16x8 operand u2 = g >> 1, registers 2 (g & 1) + {0, 1} hold elements (0,1), (2,3) of the group
+            pb = V_PB + 8 * (c & 1) + 4 * (g >> 1) + 2 * (g & 1)
+            dsb = V_DSB + 8 * (c & 1) + 4 * (g >> 1) + 2 * (g & 1)
+            for h in range(2):
+                e = 4 * g + 2 * h
+                ops.append((f"v_cvt_pk_bf16_f32 {vr(pb + h)}, {vr(s + e)}, {vr(s + e + 1)}", vset(pb + h), vset(s + e, 2), False))
+                ops.append((f"v_cvt_pk_bf16_f32 {vr(dsb + h)}, {vr(dp + e)}, {vr(dp + e + 1)}", vset(dsb + h), vset(dp + e, 2), False))
+        first = stage_first_slot[c] + (6 if c == 0 else 0)  # E(0) directly follows A(0): give its results time
+        last = stage_last_slot[c]
+        span = last - first
+        op_slot = [first + (i * span) // len(ops) for i in range(len(ops))]
+        for i, op in enumerate(ops):
+            slot_valu[op_slot[i]].append(op)
+        for g in range(4):
+            kbuf = (4 * c + g) % 3
+            lse, dl = V_LSE + 4 * kbuf, V_DL + 4 * kbuf
+            off = (32 * c + 8 * g) * 4
+            rd = [(f"ds_read_b128 {vr(lse, 4)}, %[la] offset:{off}", vset(lse, 4)),
+                  (f"ds_read_b128 {vr(dl, 4)}, %[la] offset:{off + DL_OFFSET}", vset(dl, 4))]
+            # issue when the previous group starts (three buffers: the one reloaded here was last read two groups ago)
+            if g > 0:
+                at = op_slot[group_first_op[g - 1]]
+            else:
+                at = first - 4
+            if at < 0:
+                pre_lds.extend(rd)
+            else:
+                slot_lds[at].extend(rd)
+
+    # ---- LDS reads of the MFMA pairs, PREFETCH pairs ahead ---------------------------------
+    for k in range(len(pairs)):
+        at = 2 * (k - PREFETCH)
+        if at < 0:
+            pre_lds.extend(pair_loads(k))
+        else:
+            slot_lds[at] = pair_loads(k) + slot_lds[at]
+
+    # ---- next step's Q / dO tiles: 16 LDS-direct loads per wave spread over the stream ----------
+    # (issued back to back they hold the wave for about a thousand cycles: one CU moves 64 B / clk)
+    slot_vmem = {m: [] for m in range(n_slots)}
+    k = 0
+    for t, gbase in enumerate(("gq0", "gq1", "gd0", "gd1")):  # half tiles in LDS order
+        for i in range(4):
+            slot_vmem[LOAD_FIRST + LOAD_EVERY * k].append((t * TILE + i * 1024, f"g{i}", gbase))
+            k += 1
+
+    # ---- emission ------------------------------------------------------------------------------
+    for text, dst in pre_lds:
+        em.lds_read(text, dst)
+    for m in range(n_slots):
+        for ld in slot_vmem[m]:
+            if 'vmem' in DROP:
+                continue
+            em.lds_direct_load(*ld)
+        lds = slot_lds[m]
+        for text, dst in lds:
+            if 'lds' in DROP:
+                continue
+            em.lds_read(text, dst)
+        mf = pair_mfmas(m // 2)[m % 2]
+        if 'mfma' not in DROP:
+            em.mfma(*mf)
+        for text, dst, src, trans in slot_valu[m]:
+            if 'valu' in DROP:
+                continue
+            em.valu(text, dst, src, trans)
+    em.drain()
+    return em
+
+
+def main():
+    global DROP
+    here = os.path.dirname(os.path.abspath(__file__))
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("out", nargs="?", default=os.path.join(here, "bwd_dkv_tile.inc"))
+    ap.add_argument("--drop", default="", help="comma list of mfma,valu,lds,vmem: leave these instruction classes out "
+                    "(the stream then computes nothing useful; for timing what bounds it)")
+    args = ap.parse_args()
+    DROP = tuple(x for x in args.drop.split(",") if x)
+    path = args.out
+    with open(path, "w") as f:
+        f.write("// Generated by gen_dkv_tile.py; do not edit.\n")
+        # one statement for both kinds of tile: a second asm statement on another control-flow
+        # path makes the compiler shuffle the pinned registers around each of them
+        full, masked = build(False), build(True)
+        lines = (["s_cmp_eq_u32 %[partial], 0", "s_cbranch_scc1 .Lfa_dkv_full_%="] + masked.out
+                 + ["s_branch .Lfa_dkv_done_%=", ".Lfa_dkv_full_%=:"] + full.out + [".Lfa_dkv_done_%=:"])
+        f.write("#define FA_DKV_TILE \\\n")
+        f.write(" \\\n".join(f'  "{line}\\n"' for line in lines))
+        f.write("\n\n")
+        for name, em in (("full", full), ("masked", masked)):
+            print(f"{path}: {name}: {len(em.out)} instructions, {em.stats}", file=sys.stderr)
+
+        def macro(name, lines):
+            f.write(f"#define {name} \\\n")
+            f.write(" \\\n".join(f'  "{line}\\n"' for line in lines))
+            f.write("\n\n")
+
+        # accumulators to zero (prologue)
+        macro("FA_DKV_ZERO_ACC", [f"v_accvgpr_write_b32 a{i}, 0" for i in range(128)])
+        # K / V fragment ks from 8 dword operands (prologue)
+        for ks in range(8):
+            macro(f"FA_DKV_PUT_KV_{ks}",
+                  [f"v_accvgpr_write_b32 a{128 + 4 * ks + i}, %{2 + i}" for i in range(4)]
+                  + [f"v_accvgpr_write_b32 a{160 + 4 * ks + i}, %{6 + i}" for i in range(4)])
+        # accumulator tile t (0-3 dv, 4-7 dk) into 16 dword operands (epilogue); the leading s_nop
+        # covers the MFMA -> read hazard of the last tile stream
+        for t in range(8):
+            macro(f"FA_DKV_GET_ACC_{t}", ["s_nop 15"] + [f"v_accvgpr_read_b32 %{i}, a{16 * t + i}" for i in range(16)])
+        # (operand numbers: PUT_KV has two pinned outputs before its 8 inputs)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,127 @@
+"""Emitter for hand-scheduled gfx950 instruction streams placed in `asm volatile` statements.
+
+Streams are written by generator scripts (gen_*_tile.py) as a sequence of MFMA, VALU and LDS
+operations with explicit registers.  The emitter keeps the order it is given and inserts what the
+hardware leaves to software on gfx950:
+    MFMA (8 pass) result -> VALU / LDS / MFMA-A/B use     12 wait states
+    VALU result          -> MFMA operand                   2 wait states
+    transcendental result-> VALU use                        1 wait state
+    LDS read result      -> any use                         s_waitcnt lgkmcnt (reads return in order)
+Registers are ("v", n) / ("a", n) pairs; operands supplied by the compiler (%[name]) are never
+written by a stream and need no tracking.
+"""
+
+
+def vr(lo, n=1):
+    return f"v{lo}" if n == 1 else f"v[{lo}:{lo + n - 1}]"
+
+
+def ar(lo, n=1):
+    return f"a{lo}" if n == 1 else f"a[{lo}:{lo + n - 1}]"
+
+
+def vset(lo, n=1):
+    return {("v", lo + i) for i in range(n)}
+
+
+def aset(lo, n=1):
+    return {("a", lo + i) for i in range(n)}
+
+
+class Emitter:
+    def __init__(self):
+        self.out = []
+        self.t = 0                 # wait states issued so far
+        self.mfma_w = {}           # reg -> time of the MFMA that wrote it
+        self.valu_w = {}
+        self.trans_w = {}
+        self.lds_fifo = []         # outstanding LDS reads, oldest first: sets of dst regs
+        self.stats = {"nop": 0, "wait": 0, "mfma": 0, "valu": 0, "lds": 0}
+
+    def _raw(self, text, states=1):
+        self.out.append(text)
+        self.t += states
+
+    def _need_gap(self, t_def, gap):
+        between = self.t - t_def - 1
+        if between < gap:
+            n = gap - between
+            self.stats["nop"] += n
+            while n > 0:
+                k = min(n, 16)
+                self._raw(f"s_nop {k - 1}", k)
+                n -= k
+
+    def _wait_lds(self, regs):
+        need = None
+        for i, dst in enumerate(self.lds_fifo):
+            if dst & regs:
+                need = i
+        if need is None:
+            return
+        newer = len(self.lds_fifo) - 1 - need
+        self.stats["wait"] += 1
+        self._raw(f"s_waitcnt lgkmcnt({min(newer, 15)})")
+        # everything up to `need` has returned (and more, if the count was clamped)
+        done = max(need + 1, len(self.lds_fifo) - 15) if newer > 15 else need + 1
+        self.lds_fifo = self.lds_fifo[done:]
+
+    def mfma(self, dst, a, b, c, dst_regs, a_regs, b_regs, c_regs):
+        self._wait_lds(a_regs | b_regs | c_regs | dst_regs)
+        for r in a_regs | b_regs:
+            if r in self.mfma_w:
+                self._need_gap(self.mfma_w[r], 12)
+        for r in a_regs | b_regs | c_regs:
+            if r in self.valu_w:
+                self._need_gap(self.valu_w[r], 2)
+        for r in dst_regs - c_regs:  # overwriting without accumulating: order after VALU writers
+            if r in self.valu_w:
+                self._need_gap(self.valu_w[r], 2)
+        self._raw(f"v_mfma_f32_32x32x16_bf16 {dst}, {a}, {b}, {c}")
+        for r in dst_regs:
+            self.mfma_w[r] = self.t - 1
+            self.valu_w.pop(r, None)
+            self.trans_w.pop(r, None)
+        self.stats["mfma"] += 1
+
+    def valu(self, text, dst_regs, src_regs, trans=False):
+        self._wait_lds(dst_regs | src_regs)
+        for r in dst_regs | src_regs:
+            if r in self.mfma_w:
+                self._need_gap(self.mfma_w[r], 12)
+        for r in src_regs:
+            if r in self.trans_w:
+                self._need_gap(self.trans_w[r], 1)
+        self._raw(text)
+        for r in dst_regs:
+            self.mfma_w.pop(r, None)
+            self.valu_w[r] = self.t - 1
+            if trans:
+                self.trans_w[r] = self.t - 1
+            else:
+                self.trans_w.pop(r, None)
+        self.stats["valu"] += 1
+
+    def lds_read(self, text, dst_regs):
+        self._wait_lds(dst_regs)  # an older read into the same registers must have landed
+        for r in dst_regs:
+            if r in self.mfma_w:
+                self._need_gap(self.mfma_w[r], 12)
+            self.mfma_w.pop(r, None)
+            self.valu_w.pop(r, None)
+            self.trans_w.pop(r, None)
+        self._raw(text)
+        self.lds_fifo.append(set(dst_regs))
+        self.stats["lds"] += 1
+
+    def lds_direct_load(self, lds_imm, goff, gbase):
+        """Next step's global -> LDS copy of one 1 KB block (M0 = LDS destination)."""
+        self._raw(f"s_add_u32 m0, %[ldsn], {lds_imm}")
+        self._raw("s_nop 0")
+        self._raw(f"global_load_lds_dwordx4 %[{goff}], %[{gbase}]")
+        self.stats["vmem"] = self.stats.get("vmem", 0) + 1
+
+    def drain(self):
+        if self.lds_fifo:
+            self._raw("s_waitcnt lgkmcnt(0)")
+            self.lds_fifo = []

@@ -1,0 +1,179 @@
+"""Checks of the generated gfx950 instruction streams that need no GPU.
+
+The generators declare, next to every instruction's text, the registers it reads and writes; the
+emitter derives s_nop / s_waitcnt from those declarations.  Here the emitted TEXT is parsed again,
+registers and all, and the hazard distances are re-derived from the text alone, so a declaration
+that does not match its instruction (a wrong register number, a forgotten operand) fails.
+"""
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "flex_attention_tpu_amd", "csrc")
+sys.path.insert(0, CSRC)
+
+REG = re.compile(r"\b([va])(?:\[(\d+):(\d+)\]|(\d+))")
+
+
+def regs_of(token):
+    out = set()
+    for m in REG.finditer(token):
+        if m.group(4) is not None:
+            out.add((m.group(1), int(m.group(4))))
+        else:
+            out.update((m.group(1), i) for i in range(int(m.group(2)), int(m.group(3)) + 1))
+    return out
+
+
+def split_operands(line):
+    op, _, rest = line.partition(" ")
+    rest = re.sub(r"offset:\d+", "", rest)
+    return op, [t.strip() for t in rest.split(",")] if rest.strip() else []
+
+
+def check_stream(lines):
+    """Replays a stream; returns the number of instructions checked."""
+    t = 0
+    mfma_w, valu_w, trans_w = {}, {}, {}
+    fifo = []  # outstanding LDS reads: destination register sets, oldest first
+    n = 0
+
+    def gap(t_def):
+        return t - t_def - 1
+
+    def lds_pending(regs):
+        return any(dst & regs for dst in fifo)
+
+    for line in lines:
+        op, ops = split_operands(line)
+        if op == "s_nop":
+            t += int(ops[0]) + 1
+            continue
+        if op == "s_waitcnt":
+            k = int(re.search(r"lgkmcnt\((\d+)\)", line).group(1))
+            if len(fifo) > k:
+                del fifo[: len(fifo) - k]
+            t += 1
+            continue
+        if op.startswith("s_") or op.endswith(":") or op.startswith(".L"):
+            t += 1
+            continue
+        n += 1
+        if op.startswith("v_mfma"):
+            dst, a, b, c = (regs_of(x) for x in ops)
+            assert not lds_pending(dst | a | b | c), f"MFMA uses a register with an LDS read in flight: {line}"
+            for r in a | b:
+                assert r not in mfma_w or gap(mfma_w[r]) >= 12, f"MFMA result used as A/B too early: {line}"
+            for r in a | b | c | dst:
+                assert r not in valu_w or gap(valu_w[r]) >= 2, f"VALU result used by MFMA too early: {line}"
+            if c:
+                assert c == dst, f"accumulating MFMA must read its own destination: {line}"
+            for r in dst:
+                mfma_w[r] = t
+                valu_w.pop(r, None)
+                trans_w.pop(r, None)
+        elif op.startswith("ds_read"):
+            dst = regs_of(ops[0])
+            assert not lds_pending(dst), f"LDS read into registers of an older read in flight: {line}"
+            for r in dst:
+                assert r not in mfma_w or gap(mfma_w[r]) >= 12, f"LDS read overwrites a fresh MFMA result: {line}"
+                mfma_w.pop(r, None)
+                valu_w.pop(r, None)
+                trans_w.pop(r, None)
+            fifo.append(dst)
+        elif op.startswith("global_load_lds"):
+            pass  # operands come from the compiler; the destination is LDS through M0
+        elif op.startswith("v_"):
+            dst = regs_of(ops[0])
+            src = set().union(*[regs_of(x) for x in ops[1:]]) if len(ops) > 1 else set()
+            assert not lds_pending(dst | src), f"VALU uses a register with an LDS read in flight: {line}"
+            for r in dst | src:
+                assert r not in mfma_w or gap(mfma_w[r]) >= 12, f"VALU touches a fresh MFMA result: {line}"
+            for r in src:
+                assert r not in trans_w or gap(trans_w[r]) >= 1, f"VALU reads a fresh transcendental result: {line}"
+            for r in dst:
+                mfma_w.pop(r, None)
+                valu_w[r] = t
+                if op.startswith("v_exp") or op.startswith("v_rcp") or op.startswith("v_log"):
+                    trans_w[r] = t
+                else:
+                    trans_w.pop(r, None)
+        else:
+            raise AssertionError(f"unknown instruction in stream: {line}")
+        t += 1
+    assert not fifo, "stream ends with LDS reads in flight"
+    return n
+
+
+def scratch_ok(lines, lo, hi, agpr_hi):
+    """Every VGPR a stream names lies in its declared scratch range, every AGPR in the pinned range."""
+    for line in lines:
+        for kind, i in regs_of(line):
+            if kind == "v":
+                assert lo <= i <= hi, f"v{i} outside the stream's scratch range: {line}"
+            else:
+                assert 0 <= i <= agpr_hi, f"a{i} outside the pinned range: {line}"
+
+
+def test_dkv_tile_streams_respect_hazards():
+    import gen_dkv_tile as g
+
+    for masked in (False, True):
+        em = g.build(masked)
+        n = check_stream(em.out)
+        assert em.stats["mfma"] == 128  # 4 q blocks x (8 S + 8 dP + 8 dv + 8 dk)
+        assert n == em.stats["mfma"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
+        scratch_ok(em.out, 68, 255, 191)
+
+
+def test_hazard_checker_catches_a_bad_stream():
+    bad = ["v_mfma_f32_32x32x16_bf16 v[72:87], v[192:195], a[128:131], 0", "v_exp_f32_e32 v72, v72"]
+    with pytest.raises(AssertionError):
+        check_stream(bad)
+    bad = ["ds_read_b128 v[192:195], %[r0] offset:0", "v_mfma_f32_32x32x16_bf16 v[72:87], v[192:195], a[128:131], 0"]
+    with pytest.raises(AssertionError):
+        check_stream(bad)
+    bad = ["v_cvt_pk_bf16_f32 v136, v72, v73", "v_mfma_f32_32x32x16_bf16 a[0:15], v[192:195], v[136:139], a[0:15]"]
+    with pytest.raises(AssertionError):
+        check_stream(bad)
+
+
+def test_generated_include_matches_generator(tmp_path):
+    out = tmp_path / "tile.inc"
+    subprocess.run([sys.executable, os.path.join(CSRC, "gen_dkv_tile.py"), str(out)], check=True, capture_output=True)
+    text = out.read_text()
+    for macro in ("FA_DKV_TILE", "FA_DKV_ZERO_ACC", "FA_DKV_PUT_KV_7", "FA_DKV_GET_ACC_7"):
+        assert f"#define {macro} " in text
+
+
+@pytest.mark.skipif(not os.path.exists("/opt/rocm/bin/hipcc"), reason="needs hipcc")
+def test_compiler_keeps_out_of_the_pinned_registers(tmp_path):
+    """Outside the asm statements the plain-score dk/dv kernel must not touch a[0:191] (the streams'
+    accumulators and K/V fragments) and must not spill: both would mean the compiler moved the
+    pinned state around the statements."""
+    from flex_attention_tpu_amd import build as B
+
+    gen = tmp_path / "bwd_dkv_tile.inc"
+    subprocess.run([sys.executable, os.path.join(CSRC, "gen_dkv_tile.py"), str(gen)], check=True, capture_output=True)
+    asm = tmp_path / "dkv.s"
+    flags = [f for f in B.FLAGS if f != "-fPIC"]
+    r = subprocess.run([B.HIPCC, *flags, f"-I{tmp_path}", "-S", "--cuda-device-only", os.path.join(CSRC, "bwd_dkv_bf16.hip"),
+                        "-o", str(asm)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    text = asm.read_text().split("\n")
+    start = next(i for i, l in enumerate(text) if l.startswith("_ZN2fa24bwd_dkv_bf16_d128_kernelILi0E"))
+    end = next(i for i, l in enumerate(text) if i > start and l.startswith("_ZN2fa24bwd_dkv_bf16_d128_kernelILi1E"))
+    in_asm = False
+    for line in text[start:end]:
+        if "#ASMSTART" in line:
+            in_asm = True
+        elif "#ASMEND" in line:
+            in_asm = False
+        elif not in_asm and not line.strip().startswith((";", ".")):
+            assert "scratch_" not in line, f"spill in the plain-score dk/dv kernel: {line}"
+            for kind, i in regs_of(line.split(";")[0]):
+                assert not (kind == "a" and i <= 191), f"compiler touches a pinned register: {line}"
