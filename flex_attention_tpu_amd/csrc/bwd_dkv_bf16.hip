@@ -10,9 +10,9 @@
 //   dv^T += dO^T P,  dk^T += Q^T dS   (dO^T, Q^T via transposing LDS reads).
 // Each dk/dv tile has exactly one writer, so the result is deterministic and needs no atomics.
 //
-// Full (unmasked) tiles of the plain score run a generated, hand-scheduled instruction stream
-// (gen_dkv_tile.py -> bwd_dkv_tile.inc) that software-pipelines MFMA, VALU and LDS work inside the
-// wave with a fixed register allocation; partial tiles and score modifications run the C++ path.
+// The plain score runs generated, hand-scheduled instruction streams (gen_dkv_tile.py ->
+// bwd_dkv_tile.inc) that software-pipeline MFMA, VALU and LDS work inside the wave with a fixed
+// register allocation; score modifications run the compiled C++ kernel.
 #include "fa_common.hpp"
 #include "launch.hpp"
 #include "tile_io.hpp"
@@ -36,6 +36,9 @@
   "v238", "v239", "v240", "v241", "v242", "v243", "v244", "v245", "v246", "v247", "v248", "v249", "v250", \
   "v251", "v252", "v253", "v254", "v255"
 
+// scalar registers of the generated run loop
+#define FA_DKV_RUN_SGPRS "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", "s87", "s88", "s89", "s90", "s91", "s92", "s93", "s94", "s95", "s96", "s97", "s98", "s99", "s100"
+
 #include "bwd_dkv_tile.inc"
 
 namespace fa {
@@ -44,7 +47,9 @@ namespace dkv_cfg {
 constexpr int BNK = 128;  // kv rows per work-group
 constexpr int BQ = 128;   // q rows per step (two 64-row LDS tiles)
 constexpr int D = 128;
-constexpr int LDS_BYTES = 8 * kTileElems * 2 + 4 * BQ * 4;  // (Q, dO) x 2 buffers x 2 tiles, lse x2, delta x2
+constexpr int MAX_LIST = 1024;  // longest q tile list the plain-score kernel caches in LDS
+// (Q, dO) x 2 buffers x 2 tiles, lse x2, delta x2, run-loop tables, cached q tile list and its partial flags
+constexpr int LDS_BYTES = 8 * kTileElems * 2 + 4 * BQ * 4 + 4 * 16 * 4 + MAX_LIST * 5;
 }  // namespace dkv_cfg
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
@@ -64,15 +69,14 @@ struct PinnedState {
       "+{a[160:163]}"(st.v[0]), "+{a[164:167]}"(st.v[1]), "+{a[168:171]}"(st.v[2]), "+{a[172:175]}"(st.v[3]), \
       "+{a[176:179]}"(st.v[4]), "+{a[180:183]}"(st.v[5]), "+{a[184:187]}"(st.v[6]), "+{a[188:191]}"(st.v[7])
 
+// Score modifications: compiled C++ path, one 128 x 128 tile per loop iteration.
 template <int SCORE>
 __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
   using namespace dkv_cfg;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
-  // step buffer b: Q half 0, Q half 1, dO half 0, dO half 1 (64 KiB); then lse[2][BQ], delta[2][BQ]
-  bf16_t* sT = reinterpret_cast<bf16_t*>(smem_raw);
-  auto sQ = [&](int buf, int half) { return sT + (4 * buf + half) * kTileElems; };
-  auto sDO = [&](int buf, int half) { return sT + (4 * buf + 2 + half) * kTileElems; };
-  float* sLse = reinterpret_cast<float*>(sT + 8 * kTileElems);
+  bf16_t* sQ = reinterpret_cast<bf16_t*>(smem_raw);
+  bf16_t* sDO = sQ + 4 * kTileElems;
+  float* sLse = reinterpret_cast<float*>(sDO + 4 * kTileElems);
   float* sDl = sLse + 2 * BQ;
 
   const int nKb = a.Sk / BNK;
@@ -99,34 +103,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
   const bf16_t* Qall = static_cast<const bf16_t*>(a.q);
   const bf16_t* dOall = static_cast<const bf16_t*>(a.dout);
 
-  // Plain score: the dk / dv accumulators (a[0:127]) and the K, V fragments (a[128:191]) live in
-  // accumulation registers that only the asm statements of this kernel read or write.
-  constexpr bool kAsmTiles = SCORE == FLEXATTN_SCORE_NONE;
   bf16x8 kreg[8], vreg[8];
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) {
     kreg[ks] = *reinterpret_cast<const bf16x8*>(Kg + (size_t)kv_local * D + ks * 16 + hh * 8);
     vreg[ks] = *reinterpret_cast<const bf16x8*>(Vg + (size_t)kv_local * D + ks * 16 + hh * 8);
-  }
-  PinnedState st;
-  if constexpr (kAsmTiles) {
-    // the outputs are written by the statement: no ordinary initial value is needed
-    asm volatile(FA_DKV_ZERO_ACC
-                 : "={a[0:15]}"(st.dv[0]), "={a[16:31]}"(st.dv[1]), "={a[32:47]}"(st.dv[2]), "={a[48:63]}"(st.dv[3]),
-                   "={a[64:79]}"(st.dk[0]), "={a[80:95]}"(st.dk[1]), "={a[96:111]}"(st.dk[2]), "={a[112:127]}"(st.dk[3]));
-#define FA_PUT(KS, KR, VR)                                                                          \
-  {                                                                                                 \
-    const u32x4 kw = __builtin_bit_cast(u32x4, kreg[KS]);                                           \
-    const u32x4 vw = __builtin_bit_cast(u32x4, vreg[KS]);                                           \
-    asm volatile(FA_DKV_PUT_KV_##KS                                                                 \
-                 : "={" KR "}"(st.k[KS]), "={" VR "}"(st.v[KS])                                     \
-                 : "v"(kw[0]), "v"(kw[1]), "v"(kw[2]), "v"(kw[3]), "v"(vw[0]), "v"(vw[1]), "v"(vw[2]), "v"(vw[3])); \
-  }
-    FA_PUT(0, "a[128:131]", "a[160:163]") FA_PUT(1, "a[132:135]", "a[164:167]")
-    FA_PUT(2, "a[136:139]", "a[168:171]") FA_PUT(3, "a[140:143]", "a[172:175]")
-    FA_PUT(4, "a[144:147]", "a[176:179]") FA_PUT(5, "a[148:151]", "a[180:183]")
-    FA_PUT(6, "a[152:155]", "a[184:187]") FA_PUT(7, "a[156:159]", "a[188:191]")
-#undef FA_PUT
   }
   int doc_j = 0;
   if (a.mask.flags & FLEXATTN_MASK_DOC) doc_j = a.mask.doc_k[k_idx];
@@ -144,49 +125,39 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
   const int* tile_idx = a.map.idx + (size_t)kb * nQ;
   const int n_iter = n_tiles * group;
 
-  // Iteration `it` covers q tile tile_idx[it % n_tiles] of query head hk*group + it / n_tiles; the
-  // quotient and remainders of it, it + 1 and it + 2 are carried along instead of divided out.
+  // Iteration `it` covers q tile tile_idx[it % n_tiles] of query head hk*group + it / n_tiles.
   // Its q block index is fetched two iterations ahead, its state one iteration ahead.
-  int g_cur = 0, g_nxt = 0, t_nxt = 1, t_n2 = 2;  // it / n_tiles, (it + 1) / n_tiles, (it + 1) % n_tiles, (it + 2) % n_tiles
-  if (t_nxt >= n_tiles) { t_nxt -= n_tiles; g_nxt = 1; }
-  if (t_n2 >= n_tiles) t_n2 -= n_tiles;
-  if (t_n2 >= n_tiles) t_n2 -= n_tiles;
+  auto q_block_of = [&](int it) { return tile_idx[it % n_tiles]; };
   int qb_cur = 0, qb_nxt = 0, st_cur = 0;
-  if (n_iter > 0) qb_cur = tile_idx[0];
-  if (n_iter > 1) qb_nxt = tile_idx[t_nxt];
+  if (n_iter > 0) qb_cur = q_block_of(0);
+  if (n_iter > 1) qb_nxt = q_block_of(1);
   if (n_iter > 0) st_cur = a.map.state[(size_t)qb_cur * a.map.nk + kb];
 
   TileLoader<4> loader;
   loader.init(w, lane);
-  float l_st = 0.f, m_st = 0.f, dl_st = 0.f;
-  // With `tiles_too` false only the per-row values are fetched: the generated tile stream copies
-  // the next step's Q / dO tiles itself, spread between its MFMAs.
-  size_t next_rbase = 0;
-  auto issue_tile = [&](int g, int qb, int buf, bool tiles_too) {
+  float lse_st = 0.f, dl_st = 0.f;
+  auto issue_tile = [&](int it, int qb, int buf) {
+    const int g = it / n_tiles;
     const size_t rbase = ((size_t)(b * a.Hq + hk * group + g) * a.Sq + (size_t)qb * BQ);
-    next_rbase = rbase;
-    if (tiles_too) {
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        loader.load(Qall + (rbase + half * kTileRows) * D, sQ(buf, half));
-        loader.load(dOall + (rbase + half * kTileRows) * D, sDO(buf, half));
-      }
+    for (int half = 0; half < 2; ++half) {
+      loader.load(Qall + (rbase + half * kTileRows) * D, sQ + (2 * buf + half) * kTileElems);
+      loader.load(dOall + (rbase + half * kTileRows) * D, sDO + (2 * buf + half) * kTileElems);
     }
-    // raw values only: using them here would make the wave wait for every load issued above
     if (tid < BQ) {
-      l_st = a.l[rbase + tid];
-      m_st = a.m[rbase + tid];
+      const float l_i = a.l[rbase + tid], m_i = a.m[rbase + tid];
+      lse_st = (l_i > 0.f) ? __builtin_fmaf(m_i, kLog2e, log2f(l_i)) : __builtin_huge_valf();
       dl_st = a.delta[rbase + tid];
     }
   };
   auto store_rows = [&](int buf) {
     if (tid < BQ) {
-      sLse[buf * BQ + tid] = (l_st > 0.f) ? __builtin_fmaf(m_st, kLog2e, log2f(l_st)) : __builtin_huge_valf();
+      sLse[buf * BQ + tid] = lse_st;
       sDl[buf * BQ + tid] = dl_st;
     }
   };
   if (n_iter > 0) {
-    issue_tile(0, __builtin_amdgcn_readfirstlane(qb_cur), 0, true);
+    issue_tile(0, __builtin_amdgcn_readfirstlane(qb_cur), 0);
     store_rows(0);
   }
   wait_vmem_all();
@@ -211,45 +182,20 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
     const int buf = it & 1;
     const int qb = __builtin_amdgcn_readfirstlane(qb_cur);
     const bool partial = __builtin_amdgcn_readfirstlane(st_cur) == 1;
-    sm.init(a.score, a.sm_scale, hk * group + g_cur);
-    const int q0 = qb * BQ;
-    // The lane's keep bits of a partial tile: element e of q block c sits at bit 16 (c & 1) + e of
-    // km[c >> 1].  Computed before the next step's loads are issued: the document-id loads would
-    // otherwise wait for them.
-    unsigned km[2] = {0u, 0u};
-    if (kAsmTiles && partial) {
-      const bool has_doc = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
-#pragma unroll
-      for (int cc = 0; cc < 4; ++cc) {
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          const int r0 = 32 * cc + 8 * g4 + 4 * hh;
-          int di[4] = {0, 0, 0, 0};
-          if (has_doc) {
-            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_q + q0 + r0);
-            di[0] = d4[0]; di[1] = d4[1]; di[2] = d4[2]; di[3] = d4[3];
-          }
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const bool keep = keep_elem(a.mask, q0 + r0 + u, k_idx, di[u], doc_j);
-            km[cc >> 1] |= (keep ? 1u : 0u) << (16 * (cc & 1) + 4 * g4 + u);
-          }
-        }
-      }
-    }
-    const int qb_n2 = (it + 2 < n_iter) ? tile_idx[t_n2] : 0;
+    sm.init(a.score, a.sm_scale, hk * group + it / n_tiles);
+    const int qb_n2 = (it + 2 < n_iter) ? q_block_of(it + 2) : 0;
     int st_nxt = 0;
     if (it + 1 < n_iter) {
       const int qbn = __builtin_amdgcn_readfirstlane(qb_nxt);
       st_nxt = a.map.state[(size_t)qbn * a.map.nk + kb];
-      issue_tile(g_nxt, qbn, buf ^ 1, !kAsmTiles);
+      issue_tile(it + 1, qbn, buf ^ 1);
     }
-    auto tile_cpp = [&]() {
+    const int q0 = qb * BQ;
 #pragma unroll
     for (int cc = 0; cc < 4; ++cc) {
       const int c = cc & 1;  // 32-row block inside the 64-row LDS tile cc >> 1
-      const char* qt = reinterpret_cast<const char*>(sQ(buf, cc >> 1));
-      const char* dot = reinterpret_cast<const char*>(sDO(buf, cc >> 1));
+      const char* qt = reinterpret_cast<const char*>(sQ + (2 * buf + (cc >> 1)) * kTileElems);
+      const char* dot = reinterpret_cast<const char*>(sDO + (2 * buf + (cc >> 1)) * kTileElems);
       f32x16 s_acc, dp_acc;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
@@ -304,7 +250,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
             const int i = q0 + r0 + u;
             const float tv = sm.to_log2(s_acc[e], i, k_idx);
             float pe = fast_exp2(tv - lse4[u]);
-            float gd = pe * (dp_acc[e] - dl4[u]) * sm.dfactor_unscaled(tv);
+            float gd = pe * (dp_acc[e] - dl4[u]) * sm.dfactor(tv);
             if (MASKED) {
               const bool keep = keep_elem(a.mask, i, k_idx, di[u], doc_j);
               pe = keep ? pe : 0.f;
@@ -335,73 +281,13 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
         }
       }
     }
-    };
-    if constexpr (kAsmTiles) {
-      // byte addresses of the lane's fragments in this step buffer (LDS addresses fit 32 bits)
-      const unsigned bbase = (unsigned)(size_t)sQ(buf, 0);
-      unsigned ra[8], ta[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        ra[i] = bbase + r_off[i];
-        ta[i] = bbase + t_off[i >> 1][i & 1];
-      }
-      const unsigned la = (unsigned)(size_t)(sLse + buf * BQ + 4 * hh);
-      const float c2 = sm.c2;
-#define FA_DKV_TILE_ADDRS                                                                                          \
-  [r0] "v"(ra[0]), [r1] "v"(ra[1]), [r2] "v"(ra[2]), [r3] "v"(ra[3]), [r4] "v"(ra[4]), [r5] "v"(ra[5]),            \
-      [r6] "v"(ra[6]), [r7] "v"(ra[7]), [t0] "v"(ta[0]), [t1] "v"(ta[1]), [t2] "v"(ta[2]), [t3] "v"(ta[3]),        \
-      [t4] "v"(ta[4]), [t5] "v"(ta[5]), [t6] "v"(ta[6]), [t7] "v"(ta[7]), [la] "v"(la), [c2] "s"(c2)
-      const int partial_flag = __builtin_amdgcn_readfirstlane(partial ? 1 : 0);
-      // next step's tiles (after the last step: this step's again, into the idle buffer)
-      const bf16_t* gq0 = Qall + next_rbase * D;
-      const bf16_t* gq1 = gq0 + kTileRows * D;
-      const bf16_t* gd0 = dOall + next_rbase * D;
-      const bf16_t* gd1 = gd0 + kTileRows * D;
-      const unsigned ldsn = (unsigned)(size_t)sQ(buf ^ 1, 0) + (unsigned)w * 4096u;
-      asm volatile(FA_DKV_TILE
-                   : FA_DKV_PINNED(st)
-                   : FA_DKV_TILE_ADDRS, [m0] "v"(km[0]), [m1] "v"(km[1]), [partial] "s"(partial_flag),
-                     [g0] "v"(loader.goff[0]), [g1] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]), [g3] "v"(loader.goff[3]),
-                     [gq0] "s"(gq0), [gq1] "s"(gq1), [gd0] "s"(gd0), [gd1] "s"(gd1), [ldsn] "s"(ldsn)
-                   : "memory", "scc", "m0", FA_DKV_TILE_CLOBBERS);
-#undef FA_DKV_TILE_ADDRS
-    } else {
-      tile_cpp();
-    }
 
     qb_cur = qb_nxt; qb_nxt = qb_n2;
-    g_cur = g_nxt;
-    if (++t_nxt == n_tiles) { t_nxt = 0; ++g_nxt; }
-    if (++t_n2 == n_tiles) t_n2 = 0;
     st_cur = st_nxt;
     if (it + 1 < n_iter) store_rows(buf ^ 1);
     wait_vmem_all();
     __syncthreads();
   }
-
-  if constexpr (kAsmTiles) {
-#define FA_GET(T, SRC, REG, DST)                                                                                   \
-  {                                                                                                                \
-    float x[16];                                                                                                   \
-    asm volatile(FA_DKV_GET_ACC_##T                                                                                \
-                 : "=v"(x[0]), "=v"(x[1]), "=v"(x[2]), "=v"(x[3]), "=v"(x[4]), "=v"(x[5]), "=v"(x[6]), "=v"(x[7]), \
-                   "=v"(x[8]), "=v"(x[9]), "=v"(x[10]), "=v"(x[11]), "=v"(x[12]), "=v"(x[13]), "=v"(x[14]),        \
-                   "=v"(x[15])                                                                                     \
-                 : "{" REG "}"(SRC));                                                                              \
-    _Pragma("unroll") for (int e = 0; e < 16; ++e) DST[e] = x[e];                                                  \
-  }
-    FA_GET(0, st.dv[0], "a[0:15]", dv_acc[0]) FA_GET(1, st.dv[1], "a[16:31]", dv_acc[1])
-    FA_GET(2, st.dv[2], "a[32:47]", dv_acc[2]) FA_GET(3, st.dv[3], "a[48:63]", dv_acc[3])
-    FA_GET(4, st.dk[0], "a[64:79]", dk_acc[0]) FA_GET(5, st.dk[1], "a[80:95]", dk_acc[1])
-    FA_GET(6, st.dk[2], "a[96:111]", dk_acc[2]) FA_GET(7, st.dk[3], "a[112:127]", dk_acc[3])
-#undef FA_GET
-  }
-  // the constant part of d(s')/d(raw) was left out of dS: apply it to dk once
-  const float dk_scale = sm.dfactor_post_scale(a.sm_scale);
-#pragma unroll
-  for (int db = 0; db < 4; ++db)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) dk_acc[db][e] *= dk_scale;
 
   bf16_t* dKg = static_cast<bf16_t*>(a.dk) + kv_off;
   bf16_t* dVg = static_cast<bf16_t*>(a.dv) + kv_off;
@@ -421,6 +307,291 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
   }
 }
 
+// Static schedule of the plain-score kernel when it runs one work-group per CU (256 CUs = 8 XCDs x
+// 32, consecutive work-group ids go round-robin to the XCDs).  Every XCD takes a contiguous share
+// of the (batch, kv head) pairs; its 32 work-groups walk through the share's heads together, so
+// they stream the same Q / dO through the XCD's L2, each taking the kv tiles c, c + 32, ... of a
+// head.  On every other head the order of the kv tiles is reversed: under causal masks tile kb has
+// nKb - kb q tiles, so a work-group alternates long and short items and all finish together.
+__host__ __device__ inline bool dkv_persistent_ok(int n_wg, int nKb) {
+  if (n_wg % 256 != 0 || (n_wg / 8) % nKb != 0) return false;
+  const int heads = n_wg / 8 / nKb;
+  if (nKb % 32 == 0) return true;
+  return 32 % nKb == 0 && heads % (32 / nKb) == 0;
+}
+__device__ __forceinline__ int dkv_work_item(int j, int item, int grid, int n_wg, int nKb) {
+  if (grid == n_wg) return xcd_remap(j, n_wg);
+  const int share = j & 7, c = j >> 3;
+  const int heads = n_wg / 8 / nKb;
+  int head, kb;
+  if (nKb >= 32) {
+    const int m = nKb / 32;
+    head = item / m;
+    const int kx = c + 32 * (item % m);
+    kb = (head & 1) ? nKb - 1 - kx : kx;
+  } else {
+    const int r = 32 / nKb;
+    head = item * r + c / nKb;
+    kb = (item & 1) ? nKb - 1 - c % nKb : c % nKb;
+  }
+  return (share * heads + head) * nKb + kb;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Plain score: the whole main loop runs inside generated asm statements (gen_dkv_tile.py).  One
+// statement executes a run of consecutive full tiles, or one partial tile with the lane's keep bits;
+// C++ only finds the runs, and builds the keep bits of partial tiles.  The kernel has no static
+// shared memory, so the dynamic buffer starts at LDS address 0 (the run loop toggles buffers by
+// address bits).
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs a) {
+  using namespace dkv_cfg;
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  bf16_t* sT = reinterpret_cast<bf16_t*>(smem_raw);
+  float* sLse = reinterpret_cast<float*>(sT + 8 * kTileElems);
+  float* sDl = sLse + 2 * BQ;
+
+  const int nKb = a.Sk / BNK;
+  const int nQ = a.map.nq;
+  const int n_wg = a.B * a.Hkv * nKb;
+  const int group = a.Hq / a.Hkv;
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int l32 = lane & 31;
+  const int hh = lane >> 5;
+
+  // One work-group per CU when the launcher found a balanced static schedule (dkv_persistent_grid):
+  // it then runs n_wg / gridDim.x work items back to back, which saves the gap between the end of a
+  // work-group and the start of the next one on the CU (only one fits at a time).
+  const int n_items = n_wg / (int)gridDim.x;
+  for (int item = 0; item < n_items; ++item) {
+  const int wg = dkv_work_item((int)blockIdx.x, item, (int)gridDim.x, n_wg, nKb);
+  const int bhk = wg / nKb;
+  const int kb = wg % nKb;
+  const int b = bhk / a.Hkv;
+  const int hk = bhk % a.Hkv;
+  if (item > 0) __syncthreads();  // the previous item's LDS contents are dead from here
+
+  const int kv_local = w * 32 + l32;
+  const int k_idx = kb * BNK + kv_local;
+  const size_t kv_off = ((size_t)bhk * a.Sk + (size_t)kb * BNK) * D;
+  const bf16_t* Kg = static_cast<const bf16_t*>(a.k) + kv_off;
+  const bf16_t* Vg = static_cast<const bf16_t*>(a.v) + kv_off;
+  const size_t rows0 = (size_t)(b * a.Hq + hk * group) * a.Sq;  // first row of the group's first query head
+  const bf16_t* Qg = static_cast<const bf16_t*>(a.q) + rows0 * D;
+  const bf16_t* dOg = static_cast<const bf16_t*>(a.dout) + rows0 * D;
+  // waves 0, 1 turn (l, m) into lse for rows tid & 127; waves 2, 3 pass delta through
+  const bool lse_wave = w < 2;
+  const float* rowa = (lse_wave ? a.l : a.delta) + rows0;
+  const float* rowb = (lse_wave ? a.m : a.delta) + rows0;
+  const int row = tid & (BQ - 1);
+
+  PinnedState st;
+  asm volatile(FA_DKV_ZERO_ACC
+               : "={a[0:15]}"(st.dv[0]), "={a[16:31]}"(st.dv[1]), "={a[32:47]}"(st.dv[2]), "={a[48:63]}"(st.dv[3]),
+                 "={a[64:79]}"(st.dk[0]), "={a[80:95]}"(st.dk[1]), "={a[96:111]}"(st.dk[2]), "={a[112:127]}"(st.dk[3]));
+#define FA_PUT(KS, KR, VR)                                                                                          \
+  {                                                                                                                 \
+    const u32x4 kw = *reinterpret_cast<const u32x4*>(Kg + (size_t)kv_local * D + KS * 16 + hh * 8);                 \
+    const u32x4 vw = *reinterpret_cast<const u32x4*>(Vg + (size_t)kv_local * D + KS * 16 + hh * 8);                 \
+    asm volatile(FA_DKV_PUT_KV_##KS                                                                                 \
+                 : "={" KR "}"(st.k[KS]), "={" VR "}"(st.v[KS])                                                     \
+                 : "v"(kw[0]), "v"(kw[1]), "v"(kw[2]), "v"(kw[3]), "v"(vw[0]), "v"(vw[1]), "v"(vw[2]), "v"(vw[3])); \
+  }
+  FA_PUT(0, "a[128:131]", "a[160:163]") FA_PUT(1, "a[132:135]", "a[164:167]")
+  FA_PUT(2, "a[136:139]", "a[168:171]") FA_PUT(3, "a[140:143]", "a[172:175]")
+  FA_PUT(4, "a[144:147]", "a[176:179]") FA_PUT(5, "a[148:151]", "a[180:183]")
+  FA_PUT(6, "a[152:155]", "a[184:187]") FA_PUT(7, "a[156:159]", "a[188:191]")
+#undef FA_PUT
+  int doc_j = 0;
+  if (a.mask.flags & FLEXATTN_MASK_DOC) doc_j = a.mask.doc_k[k_idx];
+
+  const int* tile_idx = a.map.idx + (size_t)kb * nQ;
+  const int qb_first = tile_idx[0];  // (nQ >= 1: always readable; used only if the list is not empty)
+  const int n_tiles = __builtin_amdgcn_readfirstlane(a.map.cnt[kb]);
+  const int n_iter = n_tiles * group;
+
+  // The kv tile's q list and which of its tiles are partial, cached in LDS: finding runs of full
+  // tiles then costs no dependent global loads.
+  int* sIdx = reinterpret_cast<int*>(sDl + 2 * BQ) + 4 * 16;
+  unsigned char* sPart = reinterpret_cast<unsigned char*>(sIdx + MAX_LIST);
+  for (int t = tid; t < n_tiles; t += 256) {
+    const int q = tile_idx[t];
+    sIdx[t] = q;
+    sPart[t] = a.map.state[(size_t)q * a.map.nk + kb] == 1 ? 1 : 0;
+  }
+
+  TileLoader<4> loader;
+  loader.init(w, lane);
+  if (n_iter > 0) {
+    // first step: tiles and row values into buffer 0
+    const int qb0 = __builtin_amdgcn_readfirstlane(qb_first);
+    const size_t r0 = (size_t)qb0 * BQ;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      loader.load(Qg + (r0 + half * kTileRows) * D, sT + half * kTileElems);
+      loader.load(dOg + (r0 + half * kTileRows) * D, sT + (2 + half) * kTileElems);
+    }
+    const float x = rowa[r0 + row], y = rowb[r0 + row];
+    if (lse_wave) {
+      sLse[row] = (x > 0.f) ? __builtin_fmaf(y, kLog2e, log2f(x)) : __builtin_huge_valf();
+    } else {
+      sDl[row] = x;
+    }
+  }
+  wait_vmem_all();
+  __syncthreads();
+
+  // byte addresses of the lane's operand fragments in buffer 0 (see tile_io.hpp); the run loop
+  // flips them between the buffers together with `buf`
+  const int r_sw = swz(l32);
+  const int t_row = 4 * hh + ((lane & 15) >> 2);
+  const int t_chunk = 2 * ((lane & 31) >> 4) + ((lane & 3) >> 1);
+  const int t_half = 4 * (lane & 1);
+  const unsigned base0 = (unsigned)(size_t)sT;
+  unsigned ra[8], ta[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) ra[ks] = base0 + (unsigned)(l32 * kTileD + (((2 * ks + hh) ^ r_sw) << 3)) * 2u;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    ta[i] = base0 + (unsigned)(tile_off(t_row + 8 * (i & 1), 4 * (i >> 1) + t_chunk) + t_half) * 2u;
+  unsigned la = (unsigned)(size_t)(sLse + 4 * hh);
+  unsigned lw = (unsigned)(size_t)((lse_wave ? sLse : sDl) + BQ + row);  // this lane's row value of the NEXT buffer
+  const unsigned tid4 = (unsigned)row * 4u;
+  // Work-group constants of the run loop, one 16-dword table per wave behind the row values
+  // (order: TABLE in gen_dkv_tile.py).  Written and read by the same wave: no barrier needed.
+  unsigned* tbl = reinterpret_cast<unsigned*>(sDl + 2 * BQ) + w * 16;
+  if (lane == 0) {
+    tbl[0] = (unsigned)n_tiles;
+    tbl[1] = (unsigned)(group - 1);
+    tbl[2] = (unsigned)a.Sq;
+    tbl[3] = base0 + (unsigned)w * 4096u;  // LDS address of the wave's first 1 KB block in buffer 0
+    tbl[4] = __builtin_bit_cast(unsigned, a.sm_scale * kLog2e);
+    tbl[5] = lse_wave ? 1u : 0u;
+    tbl[6] = (unsigned)(size_t)tile_idx;
+    tbl[7] = (unsigned)((size_t)tile_idx >> 32);
+    tbl[8] = (unsigned)(size_t)Qg;
+    tbl[9] = (unsigned)((size_t)Qg >> 32);
+    tbl[10] = (unsigned)(size_t)dOg;
+    tbl[11] = (unsigned)((size_t)dOg >> 32);
+    tbl[12] = (unsigned)(size_t)rowa;
+    tbl[13] = (unsigned)((size_t)rowa >> 32);
+    tbl[14] = (unsigned)(size_t)rowb;
+    tbl[15] = (unsigned)((size_t)rowb >> 32);
+  }
+  const unsigned tbl_addr = (unsigned)(size_t)tbl;
+
+  // Step `it` is q tile tile_idx[it % n_tiles] of query head it / n_tiles of the group.  Carried:
+  // the list positions of steps it + 1 and it + 2, the head of step it + 1, its q block index.
+  int it = 0, buf = 0, g1 = 0, p1 = 1, p2 = 2;
+  if (p1 >= n_tiles) { p1 -= n_tiles; g1 = 1; }
+  if (p2 >= n_tiles) p2 -= n_tiles;
+  if (p2 >= n_tiles) p2 -= n_tiles;
+  int qb1 = (n_iter > 0) ? __builtin_amdgcn_readfirstlane(sIdx[p1]) : 0;
+
+  while (it < n_iter) {
+    // position of step `it` in the list, its q block and state
+    int p0 = p1 - 1;
+    if (p0 < 0) p0 += n_tiles;
+    const int qb = __builtin_amdgcn_readfirstlane(sIdx[p0]);
+    const bool partial = __builtin_amdgcn_readfirstlane((int)sPart[p0]) == 1;
+    int it_end = it + 1;
+    unsigned km[2] = {0u, 0u};
+    if (partial) {
+      // the lane's keep bits: element e of q block c sits at bit 16 (c & 1) + e of km[c >> 1]
+      const int q0 = qb * BQ;
+      const bool has_doc = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
+#pragma unroll
+      for (int cc = 0; cc < 4; ++cc) {
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int r0 = 32 * cc + 8 * g4 + 4 * hh;
+          int di[4] = {0, 0, 0, 0};
+          if (has_doc) {
+            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_q + q0 + r0);
+            di[0] = d4[0]; di[1] = d4[1]; di[2] = d4[2]; di[3] = d4[3];
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const bool keep = keep_elem(a.mask, q0 + r0 + u, k_idx, di[u], doc_j);
+            km[cc >> 1] |= (keep ? 1u : 0u) << (16 * (cc & 1) + 4 * g4 + u);
+          }
+        }
+      }
+    } else {
+      // the run of full tiles ends before the next partial one: lanes look 64 steps ahead at a time
+      bool found = false;
+      while (!found && it_end < n_iter) {
+        const int j = it_end + lane;
+        bool is_partial = false;
+        if (j < n_iter) {
+          const int pj = (p0 + (j - it)) % n_tiles;
+          is_partial = sPart[pj] == 1;
+        }
+        const unsigned long long hits = __ballot(is_partial);
+        if (hits != 0ull) {
+          it_end += __builtin_ctzll(hits);
+          found = true;
+        } else {
+          it_end = (it_end + 64 < n_iter) ? it_end + 64 : n_iter;
+        }
+      }
+    }
+    it_end = __builtin_amdgcn_readfirstlane(it_end);
+    const int partial_flag = partial ? 1 : 0;
+    // no scalar operands (see gen_dkv_tile.py): the loop state travels in VGPRs
+    asm volatile(FA_DKV_RUN
+                 : FA_DKV_PINNED(st), [it] "+v"(it), [p1] "+v"(p1), [g1] "+v"(g1), [p2] "+v"(p2), [qb1] "+v"(qb1),
+                   [buf] "+v"(buf), [r0] "+v"(ra[0]), [r1] "+v"(ra[1]), [r2] "+v"(ra[2]), [r3] "+v"(ra[3]),
+                   [r4] "+v"(ra[4]), [r5] "+v"(ra[5]), [r6] "+v"(ra[6]), [r7] "+v"(ra[7]), [t0] "+v"(ta[0]),
+                   [t1] "+v"(ta[1]), [t2] "+v"(ta[2]), [t3] "+v"(ta[3]), [t4] "+v"(ta[4]), [t5] "+v"(ta[5]),
+                   [t6] "+v"(ta[6]), [t7] "+v"(ta[7]), [la] "+v"(la), [lw] "+v"(lw)
+                 : [it_end] "v"(it_end), [partial] "v"(partial_flag), [tbl] "v"(tbl_addr), [g0] "v"(loader.goff[0]),
+                   [g1v] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]), [g3] "v"(loader.goff[3]), [m0] "v"(km[0]),
+                   [m1] "v"(km[1]), [tid4] "v"(tid4)
+                 : "memory", "scc", "vcc", "m0", FA_DKV_RUN_SGPRS, "v67", FA_DKV_TILE_CLOBBERS);
+    it = __builtin_amdgcn_readfirstlane(it);
+    p1 = __builtin_amdgcn_readfirstlane(p1);
+  }
+
+  f32x16 dk_acc[4], dv_acc[4];
+#define FA_GET(T, SRC, REG, DST)                                                                                   \
+  {                                                                                                                \
+    float x[16];                                                                                                   \
+    asm volatile(FA_DKV_GET_ACC_##T                                                                                \
+                 : "=v"(x[0]), "=v"(x[1]), "=v"(x[2]), "=v"(x[3]), "=v"(x[4]), "=v"(x[5]), "=v"(x[6]), "=v"(x[7]), \
+                   "=v"(x[8]), "=v"(x[9]), "=v"(x[10]), "=v"(x[11]), "=v"(x[12]), "=v"(x[13]), "=v"(x[14]),        \
+                   "=v"(x[15])                                                                                     \
+                 : "{" REG "}"(SRC));                                                                              \
+    _Pragma("unroll") for (int e = 0; e < 16; ++e) DST[e] = x[e];                                                  \
+  }
+  FA_GET(0, st.dv[0], "a[0:15]", dv_acc[0]) FA_GET(1, st.dv[1], "a[16:31]", dv_acc[1])
+  FA_GET(2, st.dv[2], "a[32:47]", dv_acc[2]) FA_GET(3, st.dv[3], "a[48:63]", dv_acc[3])
+  FA_GET(4, st.dk[0], "a[64:79]", dk_acc[0]) FA_GET(5, st.dk[1], "a[80:95]", dk_acc[1])
+  FA_GET(6, st.dk[2], "a[96:111]", dk_acc[2]) FA_GET(7, st.dk[3], "a[112:127]", dk_acc[3])
+#undef FA_GET
+
+  // the streams leave the constant sm_scale out of dS: apply it to dk once
+  bf16_t* dKg = static_cast<bf16_t*>(a.dk) + kv_off;
+  bf16_t* dVg = static_cast<bf16_t*>(a.dv) + kv_off;
+#pragma unroll
+  for (int db = 0; db < 4; ++db) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      bf16x2 lo = pack_bf16(dk_acc[db][4 * g] * a.sm_scale, dk_acc[db][4 * g + 1] * a.sm_scale);
+      bf16x2 hi = pack_bf16(dk_acc[db][4 * g + 2] * a.sm_scale, dk_acc[db][4 * g + 3] * a.sm_scale);
+      bf16x4 out = {lo[0], lo[1], hi[0], hi[1]};
+      *reinterpret_cast<bf16x4*>(dKg + (size_t)kv_local * D + 32 * db + 8 * g + 4 * hh) = out;
+      lo = pack_bf16(dv_acc[db][4 * g], dv_acc[db][4 * g + 1]);
+      hi = pack_bf16(dv_acc[db][4 * g + 2], dv_acc[db][4 * g + 3]);
+      bf16x4 out2 = {lo[0], lo[1], hi[0], hi[1]};
+      *reinterpret_cast<bf16x4*>(dVg + (size_t)kv_local * D + 32 * db + 8 * g + 4 * hh) = out2;
+    }
+  }
+  }  // work items
+}
+
 template <int SCORE>
 static int launch_dkv(const BwdArgs& a, hipStream_t stream) {
   using namespace dkv_cfg;
@@ -433,9 +604,23 @@ static int launch_dkv(const BwdArgs& a, hipStream_t stream) {
   return check_launch("flexattn_bwd_dkv bf16");
 }
 
+static int launch_dkv_plain(const BwdArgs& a, hipStream_t stream) {
+  using namespace dkv_cfg;
+  auto kern = bwd_dkv_bf16_d128_plain_kernel;
+  static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+  if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(dkv): %s", hipGetErrorString(attr));
+  const int n_wg = a.B * a.Hkv * (a.Sk / BNK);
+  const int grid = dkv_persistent_ok(n_wg, a.Sk / BNK) ? 256 : n_wg;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), LDS_BYTES, stream, a);
+  return check_launch("flexattn_bwd_dkv bf16");
+}
+
 int bwd_dkv_bf16_d128(const BwdArgs& a, hipStream_t stream) {
   switch (a.score.kind) {
-    case FLEXATTN_SCORE_NONE: return launch_dkv<FLEXATTN_SCORE_NONE>(a, stream);
+    case FLEXATTN_SCORE_NONE:
+      // (the generated-stream kernel caches the q tile list in LDS)
+      return a.map.nq <= dkv_cfg::MAX_LIST ? launch_dkv_plain(a, stream) : launch_dkv<FLEXATTN_SCORE_NONE>(a, stream);
     case FLEXATTN_SCORE_ALIBI: return launch_dkv<FLEXATTN_SCORE_ALIBI>(a, stream);
     case FLEXATTN_SCORE_SOFTCAP: return launch_dkv<FLEXATTN_SCORE_SOFTCAP>(a, stream);
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_dkv<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);

@@ -23,10 +23,10 @@ Register contract with the C++ side (every asm statement names the accumulation 
 physical-register constraints; prologue / epilogue macros are generated here too):
     a[0:63]    dv accumulators (4 x 16)      a[64:127]  dk accumulators (4 x 16)
     a[128:159] K fragments (8 x 4)           a[160:191] V fragments (8 x 4)
-    v[68:255]  scratch of this stream (clobbered)
+    v[67:255]  scratch of the run loop and its streams (clobbered), s[84:100], vcc, m0 likewise
     %[r0..r7]  byte address of the lane's row fragment ks in the step's Q half-tile 0
     %[t0..t7]  byte address of the lane's transposed fragment (2 db + hi) in Q half-tile 0
-    %[la]      byte address of the lane's first lse value of the step;  %[c2] sm_scale * log2(e)
+    %[la]      byte address of the lane's first lse value of the step;  s64 sm_scale * log2(e)
     %[partial] scalar, non-zero selects the masked stream
     %[g0..g3]  the lane's byte offsets inside a global half tile for the wave's four 1 KB blocks;
     %[gq0], %[gq1], %[gd0], %[gd1]  global addresses (SGPR pairs) of the next step's Q / dO half tiles;
@@ -50,6 +50,26 @@ LOAD_EVERY = 6   # slots between two of them
 DROP = ()        # instruction classes left out (--drop, timing studies only)
 
 TILE = 16384
+# Scalar registers owned by the run loop (all clobbered).  The compiler hands scalars to an asm
+# statement unreliably once many are live (it may keep a uniform value in a VGPR and print that
+# VGPR for an "s" operand), so the statement takes none: work-group constants come from a 16-dword
+# per-wave table in LDS, the loop state from VGPR operands, both through v_readfirstlane_b32.
+TABLE = ["n_tiles", "gmax", "sq", "w4k", "c2", "lsew", "idx_lo", "idx_hi", "qg_lo", "qg_hi", "dog_lo", "dog_hi",
+         "rowa_lo", "rowa_hi", "rowb_lo", "rowb_hi"]  # order of the table's dwords
+SREG = {"n_tiles": "s60", "gmax": "s61", "sq": "s62", "w4k": "s63", "c2": "s64", "lsew": "s65",
+        "idx_lo": "s66", "idx_hi": "s67", "qg_lo": "s68", "qg_hi": "s69", "dog_lo": "s70", "dog_hi": "s71",
+        "rowa_lo": "s72", "rowa_hi": "s73", "rowb_lo": "s74", "rowb_hi": "s75",
+        "it": "s76", "p1": "s77", "g1": "s78", "p2": "s79", "qb1": "s80", "buf": "s81", "it_end": "s82", "partial": "s83",
+        "idx": "s[66:67]"}
+STATE_IO = ["it", "p1", "g1", "p2", "qb1", "buf"]   # VGPR operands read at entry, written back at exit
+STATE_IN = ["it_end", "partial"]                    # VGPR operands read at entry
+V_TBL = 72      # 16 scratch VGPRs the table is read into at entry
+S_T = ["s84", "s85", "s86", "s87"]
+S_GQ0, S_GQ1, S_GD0, S_GD1, S_RA, S_RB = "s[88:89]", "s[90:91]", "s[92:93]", "s[94:95]", "s[96:97]", "s[98:99]"
+S_LDSN = "s100"
+V_QB2 = 67      # q block index of the step after the next one, across the stream
+ROW_SLOT = 28   # MFMA slot at which the next step's lse / delta values are turned around
+V_ROW = 144     # 4 temporaries for that, inside pb[1] (first written by E(1), after ROW_SLOT)
 V_S = [72, 104]
 V_DP = [88, 120]
 V_PB = 136
@@ -63,7 +83,6 @@ DL_OFFSET = 1024
 
 def build(masked):
     em = Emitter()
-    em._raw("s_waitcnt lgkmcnt(0)")
 
     # ---- MFMA pairs in issue order -------------------------------------------------------
     pairs = []
@@ -142,7 +161,7 @@ def build(masked):
             group_first_op.append(len(ops))
             for u in range(4):
                 e = 4 * g + u
-                ops.append((f"v_fma_f32 {vr(s + e)}, {vr(s + e)}, %[c2], -{vr(lse + u)}", vset(s + e), vset(s + e) | vset(lse + u), False))
+                ops.append((f"v_fma_f32 {vr(s + e)}, {vr(s + e)}, s64, -{vr(lse + u)}", vset(s + e), vset(s + e) | vset(lse + u), False))
             for u in range(4):
                 e = 4 * g + u
                 ops.append((f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
@@ -203,19 +222,39 @@ def build(masked):
     # (issued back to back they hold the wave for about a thousand cycles: one CU moves 64 B / clk)
     slot_vmem = {m: [] for m in range(n_slots)}
     k = 0
-    for t, gbase in enumerate(("gq0", "gq1", "gd0", "gd1")):  # half tiles in LDS order
+    for t, gbase in enumerate((S_GQ0, S_GQ1, S_GD0, S_GD1)):  # half tiles in LDS order
         for i in range(4):
-            slot_vmem[LOAD_FIRST + LOAD_EVERY * k].append((t * TILE + i * 1024, f"g{i}", gbase))
+            slot_vmem[LOAD_FIRST + LOAD_EVERY * k].append((t * TILE + i * 1024, "%[g1v]" if i == 1 else f"%[g{i}]", gbase, S_LDSN))
             k += 1
 
     # ---- emission ------------------------------------------------------------------------------
     for text, dst in pre_lds:
         em.lds_read(text, dst)
+    n_direct = 0
     for m in range(n_slots):
         for ld in slot_vmem[m]:
             if 'vmem' in DROP:
                 continue
             em.lds_direct_load(*ld)
+            n_direct += 1
+        if m == ROW_SLOT and 'vmem' not in DROP:
+            # The two per-row values this lane fetched at the top of the step (older than every
+            # LDS-direct load) have arrived once at most n_direct vector-memory operations are open.
+            # Waves 0, 1: (l, m) -> lse = m log2(e) + log2(l), +inf where l = 0; waves 2, 3: delta
+            # passes through (%[lsew] is non-zero resp. zero).  One LDS store into the next buffer.
+            ra_, rb_, rt_, inf_ = V_ROW, V_ROW + 1, V_ROW + 2, V_ROW + 3
+            em.raw(f"s_waitcnt vmcnt({n_direct})")
+            em.valu(f"v_log_f32_e32 {vr(rt_)}, {vr(ra_)}", vset(rt_), vset(ra_), True)
+            em.valu(f"v_mul_f32_e32 {vr(rb_)}, 0x3fb8aa3b, {vr(rb_)}", vset(rb_), vset(rb_))
+            em.valu(f"v_mov_b32_e32 {vr(inf_)}, 0x7f800000", vset(inf_), set())
+            em.valu(f"v_add_f32_e32 {vr(rt_)}, {vr(rt_)}, {vr(rb_)}", vset(rt_), vset(rt_) | vset(rb_))
+            em.valu(f"v_cmp_lt_f32_e32 vcc, 0, {vr(ra_)}", set(), vset(ra_))
+            em.valu(f"v_cndmask_b32_e32 {vr(rt_)}, {vr(inf_)}, {vr(rt_)}, vcc", vset(rt_), vset(rt_) | vset(inf_))
+            em.raw("s_cmp_lg_u32 s65, 0")
+            em.raw("s_cselect_b64 vcc, -1, 0")
+            em.raw("s_nop 3")
+            em.valu(f"v_cndmask_b32_e32 {vr(rt_)}, {vr(ra_)}, {vr(rt_)}, vcc", vset(rt_), vset(rt_) | vset(ra_))
+            em.lds_write(f"ds_write_b32 %[lw], {vr(rt_)}", vset(rt_))
         lds = slot_lds[m]
         for text, dst in lds:
             if 'lds' in DROP:
@@ -232,6 +271,73 @@ def build(masked):
     return em
 
 
+def run_loop(full, masked):
+    """One asm statement: a run of consecutive steps [it, it_end) of one work-group, all full or a
+    single partial one.  At entry the step's Q / dO tiles and row values are resident in LDS buffer
+    s81; each pass computes the next step's addresses, streams the tile (which copies the next
+    step's data into the other buffer), synchronises the work-group and advances."""
+    t0, t1, t2, t3 = S_T
+    lo = lambda pair: pair[2:].split(":")[0]  # "s[88:89]" -> "88"
+    entry = [f"ds_read_b128 {vr(V_TBL + 4 * i, 4)}, %[tbl] offset:{16 * i}" for i in range(4)]
+    entry += ["s_waitcnt lgkmcnt(0)"]  # (the streams count LDS operations from zero)
+    entry += [f"v_readfirstlane_b32 {SREG[n]}, {vr(V_TBL + i)}" for i, n in enumerate(TABLE)]
+    entry += [f"v_readfirstlane_b32 {SREG[n]}, %[{n}]" for n in STATE_IO + STATE_IN]
+    top = entry + [
+        ".Lfa_dkv_loop_%=:",
+        # row of the next step relative to the first head of the group: min(g1, gmax) Sq + 128 qb1
+        f"s_min_u32 {t0}, s78, s61",
+        f"s_mul_i32 {t0}, {t0}, s62",
+        f"s_lshl_b32 {t1}, s80, 7",
+        f"s_add_u32 {t0}, {t0}, {t1}",
+        f"s_lshl_b32 {t2}, {t0}, 8",
+        f"s_lshr_b32 {t3}, {t0}, 24",
+    ]
+    for pair, base in ((S_GQ0, "qg"), (S_GD0, "dog")):
+        n = int(lo(pair))
+        top += [f"s_add_u32 s{n}, {SREG[base + '_lo']}, {t2}", f"s_addc_u32 s{n + 1}, {SREG[base + '_hi']}, {t3}",
+                f"s_add_u32 s{n + 2}, s{n}, 0x4000", f"s_addc_u32 s{n + 3}, s{n + 1}, 0"]
+    top += [f"s_lshl_b32 {t2}, {t0}, 2", f"s_lshr_b32 {t3}, {t0}, 30"]
+    for pair, base in ((S_RA, "rowa"), (S_RB, "rowb")):
+        n = int(lo(pair))
+        top += [f"s_add_u32 s{n}, {SREG[base + '_lo']}, {t2}", f"s_addc_u32 s{n + 1}, {SREG[base + '_hi']}, {t3}"]
+    top += [
+        f"s_xor_b32 {t1}, s81, 1",
+        f"s_lshl_b32 {t1}, {t1}, 16",
+        f"s_add_u32 {S_LDSN}, {t1}, s63",
+        # q block of the step after the next one (the list position wraps inside the list: always valid)
+        # (a vector load: an open scalar load would disturb the streams' lgkmcnt bookkeeping)
+        f"s_lshl_b32 {t1}, s79, 2",
+        f"v_mov_b32_e32 {vr(V_QB2)}, {t1}",
+        f"global_load_dword {vr(V_QB2)}, {vr(V_QB2)}, s[66:67]",
+        f"global_load_dword {vr(V_ROW)}, %[tid4], {S_RA}",
+        f"global_load_dword {vr(V_ROW + 1)}, %[tid4], {S_RB}",
+        "s_cmp_eq_u32 s83, 0",
+        "s_cbranch_scc1 .Lfa_dkv_full_%=",
+    ]
+    tail = [
+        ".Lfa_dkv_tail_%=:",
+        "s_waitcnt vmcnt(0) lgkmcnt(0)",
+        "s_barrier",
+        "s_add_u32 s76, s76, 1",
+        f"v_readfirstlane_b32 s80, {vr(V_QB2)}",
+        "s_add_u32 s77, s77, 1",
+        "s_cmp_eq_u32 s77, s60",
+        "s_cselect_b32 s77, 0, s77",
+        f"s_cselect_b32 {t0}, 1, 0",
+        f"s_add_u32 s78, s78, {t0}",
+        "s_add_u32 s79, s79, 1",
+        "s_cmp_eq_u32 s79, s60",
+        "s_cselect_b32 s79, 0, s79",
+        "s_xor_b32 s81, s81, 1",
+    ]
+    tail += [f"v_xor_b32_e32 %[r{i}], 0x10000, %[r{i}]" for i in range(8)]
+    tail += [f"v_xor_b32_e32 %[t{i}], 0x10000, %[t{i}]" for i in range(8)]
+    tail += ["v_xor_b32_e32 %[la], 0x200, %[la]", "v_xor_b32_e32 %[lw], 0x200, %[lw]",
+             "s_cmp_lt_u32 s76, s82", "s_cbranch_scc1 .Lfa_dkv_loop_%="]
+    tail += [f"v_mov_b32_e32 %[{n}], {SREG[n]}" for n in STATE_IO]
+    return (top + masked.out + ["s_branch .Lfa_dkv_tail_%=", ".Lfa_dkv_full_%=:"] + full.out + tail)
+
+
 def main():
     global DROP
     here = os.path.dirname(os.path.abspath(__file__))
@@ -240,16 +346,16 @@ def main():
     ap.add_argument("--drop", default="", help="comma list of mfma,valu,lds,vmem: leave these instruction classes out "
                     "(the stream then computes nothing useful; for timing what bounds it)")
     args = ap.parse_args()
-    DROP = tuple(x for x in args.drop.split(",") if x)
+    if args.drop:
+        DROP = tuple(x for x in args.drop.split(",") if x)
     path = args.out
     with open(path, "w") as f:
         f.write("// Generated by gen_dkv_tile.py; do not edit.\n")
         # one statement for both kinds of tile: a second asm statement on another control-flow
         # path makes the compiler shuffle the pinned registers around each of them
         full, masked = build(False), build(True)
-        lines = (["s_cmp_eq_u32 %[partial], 0", "s_cbranch_scc1 .Lfa_dkv_full_%="] + masked.out
-                 + ["s_branch .Lfa_dkv_done_%=", ".Lfa_dkv_full_%=:"] + full.out + [".Lfa_dkv_done_%=:"])
-        f.write("#define FA_DKV_TILE \\\n")
+        lines = run_loop(full, masked)
+        f.write("#define FA_DKV_RUN \\\n")
         f.write(" \\\n".join(f'  "{line}\\n"' for line in lines))
         f.write("\n\n")
         for name, em in (("full", full), ("masked", masked)):

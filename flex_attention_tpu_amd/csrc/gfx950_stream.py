@@ -114,12 +114,26 @@ class Emitter:
         self.lds_fifo.append(set(dst_regs))
         self.stats["lds"] += 1
 
-    def lds_direct_load(self, lds_imm, goff, gbase):
+    def lds_direct_load(self, lds_imm, goff, gbase, ldsn="%[ldsn]"):
         """Next step's global -> LDS copy of one 1 KB block (M0 = LDS destination)."""
-        self._raw(f"s_add_u32 m0, %[ldsn], {lds_imm}")
+        self._raw(f"s_add_u32 m0, {ldsn}, {lds_imm}")
         self._raw("s_nop 0")
-        self._raw(f"global_load_lds_dwordx4 %[{goff}], %[{gbase}]")
+        self._raw(f"global_load_lds_dwordx4 {goff}, {gbase}")
         self.stats["vmem"] = self.stats.get("vmem", 0) + 1
+
+    def lds_write(self, text, src_regs):
+        """An LDS store: takes a place in the in-order LDS queue like a read."""
+        self._wait_lds(src_regs)
+        for r in src_regs:
+            if r in self.mfma_w:
+                self._need_gap(self.mfma_w[r], 12)
+        self._raw(text)
+        self.lds_fifo.append(set())
+        self.stats["lds"] += 1
+
+    def raw(self, text):
+        """Scalar or wait instruction with no tracked vector registers."""
+        self._raw(text)
 
     def drain(self):
         if self.lds_fifo:

@@ -54,9 +54,9 @@ def check_stream(lines):
             t += int(ops[0]) + 1
             continue
         if op == "s_waitcnt":
-            k = int(re.search(r"lgkmcnt\((\d+)\)", line).group(1))
-            if len(fifo) > k:
-                del fifo[: len(fifo) - k]
+            m = re.search(r"lgkmcnt\((\d+)\)", line)
+            if m and len(fifo) > int(m.group(1)):
+                del fifo[: len(fifo) - int(m.group(1))]
             t += 1
             continue
         if op.startswith("s_") or op.endswith(":") or op.startswith(".L"):
@@ -87,6 +87,10 @@ def check_stream(lines):
             fifo.append(dst)
         elif op.startswith("global_load_lds"):
             pass  # operands come from the compiler; the destination is LDS through M0
+        elif op.startswith("ds_write"):
+            src = regs_of(ops[1])
+            assert not lds_pending(src), f"LDS store of a register with an LDS read in flight: {line}"
+            fifo.append(set())
         elif op.startswith("v_"):
             dst = regs_of(ops[0])
             src = set().union(*[regs_of(x) for x in ops[1:]]) if len(ops) > 1 else set()
@@ -146,7 +150,7 @@ def test_generated_include_matches_generator(tmp_path):
     out = tmp_path / "tile.inc"
     subprocess.run([sys.executable, os.path.join(CSRC, "gen_dkv_tile.py"), str(out)], check=True, capture_output=True)
     text = out.read_text()
-    for macro in ("FA_DKV_TILE", "FA_DKV_ZERO_ACC", "FA_DKV_PUT_KV_7", "FA_DKV_GET_ACC_7"):
+    for macro in ("FA_DKV_RUN", "FA_DKV_ZERO_ACC", "FA_DKV_PUT_KV_7", "FA_DKV_GET_ACC_7"):
         assert f"#define {macro} " in text
 
 
@@ -165,8 +169,8 @@ def test_compiler_keeps_out_of_the_pinned_registers(tmp_path):
                         "-o", str(asm)], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr
     text = asm.read_text().split("\n")
-    start = next(i for i, l in enumerate(text) if l.startswith("_ZN2fa24bwd_dkv_bf16_d128_kernelILi0E"))
-    end = next(i for i, l in enumerate(text) if i > start and l.startswith("_ZN2fa24bwd_dkv_bf16_d128_kernelILi1E"))
+    start = next(i for i, l in enumerate(text) if l.startswith("_ZN2fa30bwd_dkv_bf16_d128_plain_kernel"))
+    end = next(i for i, l in enumerate(text) if i > start and l.strip() == "s_endpgm")
     in_asm = False
     for line in text[start:end]:
         if "#ASMSTART" in line:
