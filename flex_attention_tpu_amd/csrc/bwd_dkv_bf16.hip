@@ -307,36 +307,6 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
   }
 }
 
-// Static schedule of the plain-score kernel when it runs one work-group per CU (256 CUs = 8 XCDs x
-// 32, consecutive work-group ids go round-robin to the XCDs).  Every XCD takes a contiguous share
-// of the (batch, kv head) pairs; its 32 work-groups walk through the share's heads together, so
-// they stream the same Q / dO through the XCD's L2, each taking the kv tiles c, c + 32, ... of a
-// head.  On every other head the order of the kv tiles is reversed: under causal masks tile kb has
-// nKb - kb q tiles, so a work-group alternates long and short items and all finish together.
-__host__ __device__ inline bool dkv_persistent_ok(int n_wg, int nKb) {
-  if (n_wg % 256 != 0 || (n_wg / 8) % nKb != 0) return false;
-  const int heads = n_wg / 8 / nKb;
-  if (nKb % 32 == 0) return true;
-  return 32 % nKb == 0 && heads % (32 / nKb) == 0;
-}
-__device__ __forceinline__ int dkv_work_item(int j, int item, int grid, int n_wg, int nKb) {
-  if (grid == n_wg) return xcd_remap(j, n_wg);
-  const int share = j & 7, c = j >> 3;
-  const int heads = n_wg / 8 / nKb;
-  int head, kb;
-  if (nKb >= 32) {
-    const int m = nKb / 32;
-    head = item / m;
-    const int kx = c + 32 * (item % m);
-    kb = (head & 1) ? nKb - 1 - kx : kx;
-  } else {
-    const int r = 32 / nKb;
-    head = item * r + c / nKb;
-    kb = (item & 1) ? nKb - 1 - c % nKb : c % nKb;
-  }
-  return (share * heads + head) * nKb + kb;
-}
-
 // ------------------------------------------------------------------------------------------------
 // Plain score: the whole main loop runs inside generated asm statements (gen_dkv_tile.py).  One
 // statement executes a run of consecutive full tiles, or one partial tile with the lane's keep bits;
@@ -361,12 +331,12 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   const int l32 = lane & 31;
   const int hh = lane >> 5;
 
-  // One work-group per CU when the launcher found a balanced static schedule (dkv_persistent_grid):
+  // One work-group per CU when the launcher found a balanced static schedule (persistent_ok):
   // it then runs n_wg / gridDim.x work items back to back, which saves the gap between the end of a
   // work-group and the start of the next one on the CU (only one fits at a time).
   const int n_items = n_wg / (int)gridDim.x;
   for (int item = 0; item < n_items; ++item) {
-  const int wg = dkv_work_item((int)blockIdx.x, item, (int)gridDim.x, n_wg, nKb);
+  const int wg = persistent_item((int)blockIdx.x, item, (int)gridDim.x, n_wg, nKb);
   const int bhk = wg / nKb;
   const int kb = wg % nKb;
   const int b = bhk / a.Hkv;
@@ -512,11 +482,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
             const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_q + q0 + r0);
             di[0] = d4[0]; di[1] = d4[1]; di[2] = d4[2]; di[3] = d4[3];
           }
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const bool keep = keep_elem(a.mask, q0 + r0 + u, k_idx, di[u], doc_j);
-            km[cc >> 1] |= (keep ? 1u : 0u) << (16 * (cc & 1) + 4 * g4 + u);
-          }
+          km[cc >> 1] |= keep_bits4_queries(a.mask, q0 + r0, k_idx, di, doc_j) << (16 * (cc & 1) + 4 * g4);
         }
       }
     } else {
@@ -611,7 +577,7 @@ static int launch_dkv_plain(const BwdArgs& a, hipStream_t stream) {
                                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(dkv): %s", hipGetErrorString(attr));
   const int n_wg = a.B * a.Hkv * (a.Sk / BNK);
-  const int grid = dkv_persistent_ok(n_wg, a.Sk / BNK) ? 256 : n_wg;
+  const int grid = persistent_ok(n_wg, a.Sk / BNK) ? 256 : n_wg;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), LDS_BYTES, stream, a);
   return check_launch("flexattn_bwd_dkv bf16");
 }

@@ -12,6 +12,25 @@
 
 #include <type_traits>
 
+// registers of the generated run loop (gen_dq_tile.py): v[66:215], s[60:100]
+#define FA_DQ_RUN_VGPRS "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", \
+  "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", \
+  "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", \
+  "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", \
+  "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", \
+  "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", \
+  "v146", "v147", "v148", "v149", "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", \
+  "v159", "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167", "v168", "v169", "v170", "v171", \
+  "v172", "v173", "v174", "v175", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", \
+  "v185", "v186", "v187", "v188", "v189", "v190", "v191", "v192", "v193", "v194", "v195", "v196", "v197", \
+  "v198", "v199", "v200", "v201", "v202", "v203", "v204", "v205", "v206", "v207", "v208", "v209", "v210", \
+  "v211", "v212", "v213", "v214", "v215"
+#define FA_DQ_RUN_SGPRS "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", \
+  "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", \
+  "s87", "s88", "s89", "s90", "s91", "s92", "s93", "s94", "s95", "s96", "s97", "s98", "s99", "s100"
+
+#include "bwd_dq_tile.inc"
+
 namespace fa {
 
 namespace dq_cfg {
@@ -19,7 +38,25 @@ constexpr int BM = 128;
 constexpr int BN = 64;
 constexpr int D = 128;
 constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2
+// plain-score kernel: steps of two kv tiles, (K, K, V, V) x 2 buffers, per-wave tables, cached kv list + states
+constexpr int MAX_LIST = 2048;
+constexpr int PLAIN_LDS_BYTES = 8 * kTileElems * 2 + 4 * 16 * 4 + MAX_LIST * 5;
 }  // namespace dq_cfg
+
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+// Register-resident state of the generated streams: every asm statement names it with the same
+// physical-register constraints, so it stays put and the compiler keeps those registers free.
+struct DqPinned {
+  f32x16 dq[4];      // a[0:63]
+  bf16x8 q[8], d[8];  // a[64:95], a[96:127]
+};
+#define FA_DQ_PINNED(st)                                                                                      \
+  "+{a[0:15]}"(st.dq[0]), "+{a[16:31]}"(st.dq[1]), "+{a[32:47]}"(st.dq[2]), "+{a[48:63]}"(st.dq[3]),          \
+      "+{a[64:67]}"(st.q[0]), "+{a[68:71]}"(st.q[1]), "+{a[72:75]}"(st.q[2]), "+{a[76:79]}"(st.q[3]),         \
+      "+{a[80:83]}"(st.q[4]), "+{a[84:87]}"(st.q[5]), "+{a[88:91]}"(st.q[6]), "+{a[92:95]}"(st.q[7]),         \
+      "+{a[96:99]}"(st.d[0]), "+{a[100:103]}"(st.d[1]), "+{a[104:107]}"(st.d[2]), "+{a[108:111]}"(st.d[3]),   \
+      "+{a[112:115]}"(st.d[4]), "+{a[116:119]}"(st.d[5]), "+{a[120:123]}"(st.d[6]), "+{a[124:127]}"(st.d[7])
 
 template <int SCORE>
 __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
@@ -234,9 +271,313 @@ static int launch_dq(const BwdArgs& a, hipStream_t stream) {
   return check_launch("flexattn_bwd_dq bf16");
 }
 
+// ------------------------------------------------------------------------------------------------
+// Plain score: the main loop runs inside generated asm statements (gen_dq_tile.py).  A step is two
+// entries of the q tile's kv list (128 kv rows); one statement executes a run of consecutive full
+// steps, or one partial step with the lane's keep bits.  Work-groups are persistent (one per CU)
+// when persistent_ok() finds a balanced schedule.  The kernel has no static shared memory: the
+// dynamic buffer starts at LDS address 0 (the run loop toggles buffers by address bits).
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs a) {
+  using namespace dq_cfg;
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  bf16_t* sT = reinterpret_cast<bf16_t*>(smem_raw);  // buffer b: K tile 0, K tile 1, V tile 0, V tile 1
+  unsigned* sTbl = reinterpret_cast<unsigned*>(sT + 8 * kTileElems);
+  int* sIdx = reinterpret_cast<int*>(sTbl + 4 * 16);
+  unsigned char* sSt = reinterpret_cast<unsigned char*>(sIdx + MAX_LIST);
+
+  const int nQ = a.Sq / BM;
+  const int nK = a.map.nk;
+  const int n_wg = a.B * a.Hq * nQ;
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int l32 = lane & 31;
+  const int hh = lane >> 5;
+  const int q_local = w * 32 + l32;
+
+  TileLoader<4> loader;
+  loader.init(w, lane);
+  const int r_sw = swz(l32);
+  const int t_row = 4 * hh + ((lane & 15) >> 2);
+  const int t_chunk = 2 * ((lane & 31) >> 4) + ((lane & 3) >> 1);
+  const int t_half = 4 * (lane & 1);
+  const unsigned base0 = (unsigned)(size_t)sT;
+
+  // Everything an item needs from global memory before its first step.  It is fetched while the
+  // previous item runs (plain loads whose values are not touched until then), so that an item
+  // starts after one memory round trip (its first kv tiles) instead of a chain of dependent ones.
+  constexpr int kListRegs = MAX_LIST / 256;
+  struct ItemRegs {
+    u32x4 qw[8], dw[8];  // Q^T / dO^T fragments of the lane's q row
+    float l, m, delta;
+    int doc;
+    int n_tiles, kb0, kb1;         // list length and its first two entries
+    int idx[kListRegs];            // kv list entries tid + 256 j
+    unsigned char st[kListRegs];   // state of kv tile tid + 256 j in the q tile's state row
+  };
+  const int n_items = n_wg / (int)gridDim.x;
+  auto geometry = [&](int item, int& bh, int& qb) {
+    const int wg = persistent_item((int)blockIdx.x, item, (int)gridDim.x, n_wg, nQ);
+    bh = wg / nQ;
+    qb = (gridDim.x == (unsigned)n_wg) ? nQ - 1 - (wg % nQ) : wg % nQ;  // one item each: longest first
+  };
+  auto fetch = [&](int item, ItemRegs& r) {
+    int bh, qb;
+    geometry(item, bh, qb);
+    const size_t q_off = ((size_t)bh * a.Sq + (size_t)qb * BM + q_local) * D;
+    const bf16_t* Qg = static_cast<const bf16_t*>(a.q) + q_off;
+    const bf16_t* dOg = static_cast<const bf16_t*>(a.dout) + q_off;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      r.qw[ks] = *reinterpret_cast<const u32x4*>(Qg + ks * 16 + hh * 8);
+      r.dw[ks] = *reinterpret_cast<const u32x4*>(dOg + ks * 16 + hh * 8);
+    }
+    const size_t row = (size_t)bh * a.Sq + qb * BM + q_local;
+    r.l = a.l[row];
+    r.m = a.m[row];
+    r.delta = a.delta[row];
+    r.doc = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[qb * BM + q_local] : 0;
+    r.n_tiles = a.map.cnt[qb];
+    const int* tile_idx = a.map.idx + (size_t)qb * nK;
+    r.kb0 = tile_idx[0];                // (nK >= 1: always readable; meaningful only if the list is not empty)
+    r.kb1 = tile_idx[nK > 1 ? 1 : 0];
+    const uint8_t* tile_state = a.map.state + (size_t)qb * nK;
+#pragma unroll
+    for (int j = 0; j < kListRegs; ++j) {
+      const int t = tid + 256 * j;
+      r.idx[j] = (t < nK) ? tile_idx[t] : 0;  // (slots past the list length hold no valid entry and are never used)
+      r.st[j] = (t < nK) ? tile_state[t] : 0;
+    }
+  };
+
+  // Byte addresses of the lane's operand fragments in LDS step buffer 0; the run loop flips them
+  // between the two buffers together with `buf`, across items too.
+  unsigned ra[8], ta[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) ra[ks] = base0 + (unsigned)(l32 * kTileD + (((2 * ks + hh) ^ r_sw) << 3)) * 2u;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    ta[i] = base0 + (unsigned)(tile_off(t_row + 8 * (i & 1), 4 * (i >> 1) + t_chunk) + t_half) * 2u;
+  int buf = 0;
+  bool resident = false;  // the item's first step was already copied into buffer `buf` by the previous item's last step
+
+  ItemRegs pre;
+  fetch(0, pre);
+  for (int item = 0; item < n_items; ++item) {
+    int bh, qb;
+    geometry(item, bh, qb);
+    const int b = bh / a.Hq;
+    const int h = bh % a.Hq;
+    const int hk = h / (a.Hq / a.Hkv);
+    if (item > 0) __syncthreads();  // the previous item's LDS contents are dead from here
+
+    bf16_t* dQg = static_cast<bf16_t*>(a.dq) + ((size_t)bh * a.Sq + (size_t)qb * BM) * D;
+    const bf16_t* Kg = static_cast<const bf16_t*>(a.k) + ((size_t)(b * a.Hkv + hk) * a.Sk) * D;
+    const bf16_t* Vg = static_cast<const bf16_t*>(a.v) + ((size_t)(b * a.Hkv + hk) * a.Sk) * D;
+    const int q_idx = qb * BM + q_local;
+    const int* tile_idx = a.map.idx + (size_t)qb * nK;
+
+    // the q tile's kv list and its state row into LDS
+    const int n_tiles = __builtin_amdgcn_readfirstlane(pre.n_tiles);
+    const int n_steps = (n_tiles + 1) >> 1;
+#pragma unroll
+    for (int j = 0; j < kListRegs; ++j) {
+      const int t = tid + 256 * j;
+      if (t < nK) {
+        sIdx[t] = pre.idx[j];
+        sSt[t] = pre.st[j];
+      }
+    }
+
+    DqPinned st;
+    asm volatile(FA_DQ_ZERO_ACC
+                 : "={a[0:15]}"(st.dq[0]), "={a[16:31]}"(st.dq[1]), "={a[32:47]}"(st.dq[2]), "={a[48:63]}"(st.dq[3]));
+#define FA_PUT(KS, QR, DR)                                                                                    \
+  asm volatile(FA_DQ_PUT_##KS                                                                                 \
+               : "={" QR "}"(st.q[KS]), "={" DR "}"(st.d[KS])                                                 \
+               : "v"(pre.qw[KS][0]), "v"(pre.qw[KS][1]), "v"(pre.qw[KS][2]), "v"(pre.qw[KS][3]), "v"(pre.dw[KS][0]), \
+                 "v"(pre.dw[KS][1]), "v"(pre.dw[KS][2]), "v"(pre.dw[KS][3]));
+    FA_PUT(0, "a[64:67]", "a[96:99]") FA_PUT(1, "a[68:71]", "a[100:103]") FA_PUT(2, "a[72:75]", "a[104:107]")
+    FA_PUT(3, "a[76:79]", "a[108:111]") FA_PUT(4, "a[80:83]", "a[112:115]") FA_PUT(5, "a[84:87]", "a[116:119]")
+    FA_PUT(6, "a[88:91]", "a[120:123]") FA_PUT(7, "a[92:95]", "a[124:127]")
+#undef FA_PUT
+    const float lse2 = (pre.l > 0.f) ? __builtin_fmaf(pre.m, kLog2e, log2f(pre.l)) : __builtin_huge_valf();
+    const float delta = pre.delta;
+    const int doc_i = pre.doc;
+    const int kb_first = __builtin_amdgcn_readfirstlane(pre.kb0);
+    const int kb_second = (n_tiles > 1) ? __builtin_amdgcn_readfirstlane(pre.kb1) : kb_first;
+    if (n_tiles > 0 && !resident) {
+      // first step into the current buffer (a missing second entry repeats the first: finite data, masked out)
+      bf16_t* dst = sT + (size_t)buf * 4 * kTileElems;
+      loader.load(Kg + (size_t)kb_first * BN * D, dst);
+      loader.load(Kg + (size_t)kb_second * BN * D, dst + kTileElems);
+      loader.load(Vg + (size_t)kb_first * BN * D, dst + 2 * kTileElems);
+      loader.load(Vg + (size_t)kb_second * BN * D, dst + 3 * kTileElems);
+    }
+    unsigned* tbl = sTbl + w * 16;
+    const unsigned tbl_addr = (unsigned)(size_t)tbl;
+    wait_vmem_all();
+    __syncthreads();
+    // the next item's data lands while this item's first step runs
+    int bh_n = bh, qb_n = qb;
+    if (item + 1 < n_items) {
+      fetch(item + 1, pre);
+      geometry(item + 1, bh_n, qb_n);
+    }
+    const int b_n = bh_n / a.Hq, hk_n = (bh_n % a.Hq) / (a.Hq / a.Hkv);
+    const bf16_t* Kg_n = static_cast<const bf16_t*>(a.k) + ((size_t)(b_n * a.Hkv + hk_n) * a.Sk) * D;
+    const bf16_t* Vg_n = static_cast<const bf16_t*>(a.v) + ((size_t)(b_n * a.Hkv + hk_n) * a.Sk) * D;
+
+    // carried: the kv tile indices of step it + 1 (clamped into the list)
+    int it = 0;
+    auto entry = [&](int e) { return sIdx[e < n_tiles ? e : n_tiles - 1]; };
+    int kba1 = (n_tiles > 0) ? __builtin_amdgcn_readfirstlane(entry(2)) : 0;
+    int kbb1 = (n_tiles > 0) ? __builtin_amdgcn_readfirstlane(entry(3)) : 0;
+    // step s is full when both of its entries exist and are full
+    auto step_full = [&](int sidx) {
+      return sSt[sIdx[2 * sidx]] == 2 && 2 * sidx + 1 < n_tiles && sSt[sIdx[2 * sidx + 1]] == 2;
+    };
+
+    while (it < n_steps) {
+      const bool partial = __builtin_amdgcn_readfirstlane(step_full(it) ? 0 : 1) == 1;
+      int it_end = it + 1;
+      unsigned km[2] = {0u, 0u};
+      if (partial) {
+        // the lane's keep bits: element e of kv block c sits at bit 16 (c & 1) + e of km[c >> 1]
+        const bool has_doc = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
+#pragma unroll
+        for (int hx = 0; hx < 2; ++hx) {
+          const int e = 2 * it + hx;
+          if (e >= n_tiles) continue;  // missing half: all dropped
+          const int state = __builtin_amdgcn_readfirstlane((int)sSt[sIdx[e]]);
+          if (state == 2) {
+            km[hx] = 0xffffffffu;
+            continue;
+          }
+          const int kv0 = __builtin_amdgcn_readfirstlane(sIdx[e]) * BN;
+#pragma unroll
+          for (int c = 0; c < 2; ++c) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              const int j0 = kv0 + 32 * c + 8 * g + 4 * hh;
+              int dj[4] = {0, 0, 0, 0};
+              if (has_doc) {
+                const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_k + j0);
+                dj[0] = d4[0]; dj[1] = d4[1]; dj[2] = d4[2]; dj[3] = d4[3];
+              }
+              km[hx] |= keep_bits4_keys(a.mask, q_idx, j0, doc_i, dj) << (16 * c + 4 * g);
+            }
+          }
+        }
+      } else {
+        // the run of full steps ends before the next partial one: lanes look 64 steps ahead at a time
+        bool found = false;
+        while (!found && it_end < n_steps) {
+          const int j = it_end + lane;
+          const bool is_partial = j < n_steps && !step_full(j);
+          const unsigned long long hits = __ballot(is_partial);
+          if (hits != 0ull) {
+            it_end += __builtin_ctzll(hits);
+            found = true;
+          } else {
+            it_end = (it_end + 64 < n_steps) ? it_end + 64 : n_steps;
+          }
+        }
+      }
+      it_end = __builtin_amdgcn_readfirstlane(it_end);
+      const int partial_flag = partial ? 1 : 0;
+      // Work-group constants of the run loop, one table per wave (order: TABLE in gen_dq_tile.py),
+      // written and read by the same wave.  A run that ends the item also names the next item's
+      // first step (its values were fetched at the start of this item; only now are they touched).
+      {
+        int kb_na = kb_first, kb_nb = kb_second;
+        if (it_end == n_steps && item + 1 < n_items) {
+          const int nt = __builtin_amdgcn_readfirstlane(pre.n_tiles);
+          kb_na = nt > 0 ? __builtin_amdgcn_readfirstlane(pre.kb0) : 0;
+          kb_nb = nt > 1 ? __builtin_amdgcn_readfirstlane(pre.kb1) : kb_na;
+        }
+        if (lane == 0) {
+          tbl[0] = (unsigned)n_tiles;
+          tbl[1] = base0 + (unsigned)w * 4096u;  // LDS address of the wave's first 1 KB block in buffer 0
+          tbl[2] = __builtin_bit_cast(unsigned, a.sm_scale * kLog2e);
+          tbl[3] = (unsigned)n_steps;
+          tbl[4] = (unsigned)(size_t)tile_idx;
+          tbl[5] = (unsigned)((size_t)tile_idx >> 32);
+          tbl[6] = (unsigned)(size_t)Kg;
+          tbl[7] = (unsigned)((size_t)Kg >> 32);
+          tbl[8] = (unsigned)(size_t)Vg;
+          tbl[9] = (unsigned)((size_t)Vg >> 32);
+          tbl[10] = (unsigned)kb_na;
+          tbl[11] = (unsigned)kb_nb;
+          tbl[12] = (unsigned)(size_t)Kg_n;
+          tbl[13] = (unsigned)((size_t)Kg_n >> 32);
+          tbl[14] = (unsigned)(size_t)Vg_n;
+          tbl[15] = (unsigned)((size_t)Vg_n >> 32);
+        }
+      }
+      // no scalar operands (see gen_dq_tile.py): the loop state travels in VGPRs
+      asm volatile(FA_DQ_RUN
+                   : FA_DQ_PINNED(st), [it] "+v"(it), [kba1] "+v"(kba1), [kbb1] "+v"(kbb1), [buf] "+v"(buf),
+                     [r0] "+v"(ra[0]), [r1] "+v"(ra[1]), [r2] "+v"(ra[2]), [r3] "+v"(ra[3]), [r4] "+v"(ra[4]),
+                     [r5] "+v"(ra[5]), [r6] "+v"(ra[6]), [r7] "+v"(ra[7]), [t0] "+v"(ta[0]), [t1] "+v"(ta[1]),
+                     [t2] "+v"(ta[2]), [t3] "+v"(ta[3]), [t4] "+v"(ta[4]), [t5] "+v"(ta[5]), [t6] "+v"(ta[6]),
+                     [t7] "+v"(ta[7])
+                   : [it_end] "v"(it_end), [partial] "v"(partial_flag), [tbl] "v"(tbl_addr), [lse] "v"(lse2),
+                     [dl] "v"(delta), [g0] "v"(loader.goff[0]), [g1v] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]),
+                     [g3] "v"(loader.goff[3]), [m0] "v"(km[0]), [m1] "v"(km[1])
+                   : "memory", "scc", "vcc", "m0", FA_DQ_RUN_SGPRS, FA_DQ_RUN_VGPRS);
+      it = __builtin_amdgcn_readfirstlane(it);
+      buf = __builtin_amdgcn_readfirstlane(buf);
+    }
+    // the last step of a non-empty item copied the next item's first step into buffer `buf`
+    resident = n_steps > 0 && item + 1 < n_items && __builtin_amdgcn_readfirstlane(pre.n_tiles) > 0;
+
+    f32x16 dq_acc[4];
+#define FA_GET(T, SRC, REG, DST)                                                                                   \
+  {                                                                                                                \
+    float x[16];                                                                                                   \
+    asm volatile(FA_DQ_GET_ACC_##T                                                                                 \
+                 : "=v"(x[0]), "=v"(x[1]), "=v"(x[2]), "=v"(x[3]), "=v"(x[4]), "=v"(x[5]), "=v"(x[6]), "=v"(x[7]), \
+                   "=v"(x[8]), "=v"(x[9]), "=v"(x[10]), "=v"(x[11]), "=v"(x[12]), "=v"(x[13]), "=v"(x[14]),        \
+                   "=v"(x[15])                                                                                     \
+                 : "{" REG "}"(SRC));                                                                              \
+    _Pragma("unroll") for (int e = 0; e < 16; ++e) DST[e] = x[e];                                                  \
+  }
+    FA_GET(0, st.dq[0], "a[0:15]", dq_acc[0]) FA_GET(1, st.dq[1], "a[16:31]", dq_acc[1])
+    FA_GET(2, st.dq[2], "a[32:47]", dq_acc[2]) FA_GET(3, st.dq[3], "a[48:63]", dq_acc[3])
+#undef FA_GET
+    // the streams leave the constant sm_scale out of dS: apply it once
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        bf16x2 lo = pack_bf16(dq_acc[db][4 * g] * a.sm_scale, dq_acc[db][4 * g + 1] * a.sm_scale);
+        bf16x2 hi = pack_bf16(dq_acc[db][4 * g + 2] * a.sm_scale, dq_acc[db][4 * g + 3] * a.sm_scale);
+        bf16x4 out = {lo[0], lo[1], hi[0], hi[1]};
+        *reinterpret_cast<bf16x4*>(dQg + (size_t)q_local * D + 32 * db + 8 * g + 4 * hh) = out;
+      }
+    }
+  }  // work items
+}
+
+static int launch_dq_plain(const BwdArgs& a, hipStream_t stream) {
+  using namespace dq_cfg;
+  auto kern = bwd_dq_bf16_d128_plain_kernel;
+  static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, PLAIN_LDS_BYTES);
+  if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(dq): %s", hipGetErrorString(attr));
+  const int n_wg = a.B * a.Hq * (a.Sq / BM);
+  const int grid = persistent_ok(n_wg, a.Sq / BM) ? 256 : n_wg;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), PLAIN_LDS_BYTES, stream, a);
+  return check_launch("flexattn_bwd_dq bf16");
+}
+
 int bwd_dq_bf16_d128(const BwdArgs& a, hipStream_t stream) {
   switch (a.score.kind) {
-    case FLEXATTN_SCORE_NONE: return launch_dq<FLEXATTN_SCORE_NONE>(a, stream);
+    case FLEXATTN_SCORE_NONE:
+      // (the generated-stream kernel caches the kv list in LDS)
+      return a.map.nk <= dq_cfg::MAX_LIST ? launch_dq_plain(a, stream) : launch_dq<FLEXATTN_SCORE_NONE>(a, stream);
     case FLEXATTN_SCORE_ALIBI: return launch_dq<FLEXATTN_SCORE_ALIBI>(a, stream);
     case FLEXATTN_SCORE_SOFTCAP: return launch_dq<FLEXATTN_SCORE_SOFTCAP>(a, stream);
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_dq<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);

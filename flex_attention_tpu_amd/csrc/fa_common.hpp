@@ -140,6 +140,30 @@ __device__ __forceinline__ bool keep_elem(const MaskArgs& mk, int i, int j, int 
   return keep;
 }
 
+// Keep bits (bit u = element u) of four elements in a row of the score matrix: query i against
+// keys j0 .. j0 + 3 (keys_vary) or queries i0 .. i0 + 3 against key j.  The purely causal mask,
+// the common case, needs no per-element work.
+__device__ __forceinline__ unsigned keep_bits4_keys(const MaskArgs& mk, int i, int j0, int doc_i, const int (&dj)[4]) {
+  if (mk.flags == FLEXATTN_MASK_CAUSAL) {
+    const int n = min(max(i - j0 + 1, 0), 4);  // keys j0 .. j0 + n - 1 are not in the future
+    return (1u << n) - 1u;
+  }
+  unsigned bits = 0;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) bits |= (keep_elem(mk, i, j0 + u, doc_i, dj[u]) ? 1u : 0u) << u;
+  return bits;
+}
+__device__ __forceinline__ unsigned keep_bits4_queries(const MaskArgs& mk, int i0, int j, const int (&di)[4], int doc_j) {
+  if (mk.flags == FLEXATTN_MASK_CAUSAL) {
+    const int n = min(max(j - i0, 0), 4);  // queries i0 .. i0 + n - 1 come before the key
+    return (0xFu << n) & 0xFu;
+  }
+  unsigned bits = 0;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) bits |= (keep_elem(mk, i0 + u, j, di[u], doc_j) ? 1u : 0u) << u;
+  return bits;
+}
+
 // ------------------------------------------------------------------------------------------
 // Score modification.  `raw` is <q_i, k_j>.  to_log2() returns the modified logit multiplied by
 // log2(e) so that probabilities are exp2(t - lse2).  dfactor() returns d(s')/d(raw) given the
@@ -213,5 +237,37 @@ __device__ __forceinline__ int xcd_remap(int wg, int n_wg) {
   if (n_wg % kXcd != 0) return wg;
   return (wg % kXcd) * (n_wg / kXcd) + wg / kXcd;
 }
+
+// Static schedule of a generated-stream kernel when it runs one work-group per CU (256 CUs = 8 XCDs x
+// 32, consecutive work-group ids go round-robin to the XCDs).  Every XCD takes a contiguous share
+// of the (batch, kv head) pairs; its 32 work-groups walk through the share's heads together, so
+// they stream the same operand tiles through the XCD's L2, each taking the blocks c, c + 32, ... of a
+// head (kv tiles for dk/dv, q tiles for dq).  On every other head the block order is reversed: under
+// causal masks the work per block grows or shrinks linearly with its index, so a work-group
+// alternates long and short items and all finish together.
+__host__ __device__ inline bool persistent_ok(int n_wg, int nKb) {
+  if (n_wg % 256 != 0 || (n_wg / 8) % nKb != 0) return false;
+  const int heads = n_wg / 8 / nKb;
+  if (nKb % 32 == 0) return true;
+  return 32 % nKb == 0 && heads % (32 / nKb) == 0;
+}
+__device__ __forceinline__ int persistent_item(int j, int item, int grid, int n_wg, int nKb) {
+  if (grid == n_wg) return xcd_remap(j, n_wg);
+  const int share = j & 7, c = j >> 3;
+  const int heads = n_wg / 8 / nKb;
+  int head, kb;
+  if (nKb >= 32) {
+    const int m = nKb / 32;
+    head = item / m;
+    const int kx = c + 32 * (item % m);
+    kb = (head & 1) ? nKb - 1 - kx : kx;
+  } else {
+    const int r = 32 / nKb;
+    head = item * r + c / nKb;
+    kb = (item & 1) ? nKb - 1 - c % nKb : c % nKb;
+  }
+  return (share * heads + head) * nKb + kb;
+}
+
 
 }  // namespace fa

@@ -1,0 +1,306 @@
+#!/usr/bin/env python3
+"""Generator of the hand-scheduled gfx950 instruction streams of the bf16 dq kernel (plain score).
+Writes bwd_dq_tile.inc: string-literal macros that bwd_dq_bf16.hip places inside `asm volatile`
+statements: the run loop over steps of two 64-row kv tiles, and prologue / epilogue register moves.
+
+A wave owns 32 q rows (Q^T, dO^T fragments and the dq^T accumulators stay in accumulation
+registers); one step covers 128 kv rows = four 32-row kv blocks c = 0..3, software-pipelined:
+
+    A(c): S^T = K Q^T, dP^T = V dO^T       16 MFMAs, operands: 16 ds_read_b128 (rows of K, V)
+    E(c): dS^T = exp2(S^T c2 - lse) (dP^T - delta)   72 VALU ops
+    B(c): dq^T += K^T dS^T                  8 MFMAs, operands: 16 ds_read_b64_tr_b16 (K again)
+
+    MFMA order:  A0 | A1 | A2 B0 | A3 B1 | B2 | B3      VALU:  - | E0 | E1 | E2 | E3 | -
+
+LDS reads are issued PREFETCH MFMA pairs ahead of their use into a rotating pool of staging
+registers; the next step's K / V tiles are copied global -> LDS by 16 loads spread over the stream.
+The emitter (gfx950_stream.py) inserts the s_nop / s_waitcnt that the hardware hazards require.
+
+Register contract with the C++ side (every asm statement names the accumulation registers with
+physical-register constraints):
+    a[0:63]   dq^T accumulators (4 x 16)   a[64:95] Q^T fragments (8 x 4)   a[96:127] dO^T fragments
+    v[66:215], s[60:100], vcc, m0   scratch of the run loop (clobbered)
+    (the table also names the next work item's first step, copied into LDS during this item's last step)
+    %[r0..r7]  byte address of the lane's row fragment ks in K half-tile 0 of the current buffer
+    %[t0..t7]  byte address of the lane's transposed fragment (2 db + hi) in K half-tile 0
+    %[lse], %[dl]  the lane's q row: log2-domain logsumexp and delta
+    %[g0], %[g1v], %[g2], %[g3]  the lane's byte offsets inside a global half tile for the wave's 1 KB blocks
+    %[m0], %[m1]  (partial steps) the lane's keep bits: bit 16 (c & 1) + e of m[c >> 1] is element e
+               of the S^T accumulator of kv block c; dropped elements get dS = 0
+    %[tbl]     LDS byte address of the wave's table of work-group constants (TABLE below)
+    %[it], %[kba1], %[kbb1], %[buf]  loop state (in/out); %[it_end], %[partial]  (in)
+LDS layout of one step buffer (bytes): K tile 0, K tile 1, V tile 0, V tile 1 (16 KiB each); the two
+buffers are 64 KiB apart and the first starts at LDS address 0.
+"""
+import argparse
+import os
+import sys
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+from gfx950_stream import Emitter, ar, aset, vr, vset  # noqa: E402
+
+NSLOT = 8        # staging slots of 8 VGPRs
+PREFETCH = 4     # MFMA pairs between the LDS reads of a pair and its MFMAs
+LOAD_FIRST = 2   # MFMA slot of the first LDS-direct load of the next step
+LOAD_EVERY = 5   # slots between two of them
+DROP = ()        # instruction classes left out (--drop, timing studies only)
+
+TILE = 16384
+# No scalar operands: constants come from a per-wave table in LDS, loop state from VGPR operands
+# (the compiler may print a VGPR for an "s" operand once many uniform values are live).
+TABLE = ["n_tiles", "w4k", "c2", "n_steps", "idx_lo", "idx_hi", "kg_lo", "kg_hi", "vg_lo", "vg_hi", "kban", "kbbn",
+         "kgn_lo", "kgn_hi", "vgn_lo", "vgn_hi"]
+SREG = {"n_tiles": "s60", "w4k": "s61", "c2": "s62", "n_steps": "s63", "idx_lo": "s64", "idx_hi": "s65",
+        "kg_lo": "s66", "kg_hi": "s67", "vg_lo": "s68", "vg_hi": "s69", "kban": "s70", "kbbn": "s71",
+        "kgn_lo": "s78", "kgn_hi": "s79", "vgn_lo": "s80", "vgn_hi": "s81",
+        "it": "s72", "kba1": "s73", "kbb1": "s74", "buf": "s75", "it_end": "s76", "partial": "s77",
+        "idx": "s[64:65]"}
+S_SEL = ["s82", "s83", "s96", "s97", "s98", "s99"]  # this pass's tile indices and K / V bases (next step or next item)
+STATE_IO = ["it", "kba1", "kbb1", "buf"]
+STATE_IN = ["it_end", "partial"]
+S_T = ["s84", "s85", "s86", "s87"]
+S_GK0, S_GK1, S_GV0, S_GV1 = "s[88:89]", "s[90:91]", "s[92:93]", "s[94:95]"
+S_LDSN = "s100"
+V_KB2 = 66       # kv tile indices of the step after the next one (2 registers), across the stream
+V_TMP = 68       # 4 temporaries of the masked variant
+V_TBL = 72       # 12 scratch VGPRs the table is read into at entry
+V_S = [72, 104]
+V_DP = [88, 120]
+V_DS = 136       # dS^T as MFMA B operands: [c & 1][u] x 4 registers
+V_STG = 152
+V_END = 215
+A_DQ, A_Q, A_DO = 0, 64, 96
+
+
+def build(masked):
+    em = Emitter()
+    pairs = []
+
+    def add_A(c):
+        for ks in range(8):
+            pairs.append(("A", c, ks))
+
+    def add_B(c):
+        for u in range(2):
+            for j in range(2):
+                pairs.append(("B", c, (u, j)))
+
+    add_A(0)
+    first = {}
+    first[0] = 2 * len(pairs); add_A(1)
+    first[1] = 2 * len(pairs); add_A(2); add_B(0)
+    first[2] = 2 * len(pairs); add_A(3); add_B(1)
+    first[3] = 2 * len(pairs); add_B(2)
+    stage_end = 2 * len(pairs); add_B(3)
+    n_slots = 2 * len(pairs)
+    last = {0: first[1], 1: first[2], 2: first[3], 3: stage_end}
+
+    def half_off(c):
+        return (c >> 1) * TILE + (c & 1) * (TILE // 2)
+
+    def pair_loads(k):
+        kind, c, x = pairs[k]
+        base = V_STG + 8 * (k % NSLOT)
+        if kind == "A":
+            ks = x
+            return [(f"ds_read_b128 {vr(base, 4)}, %[r{ks}] offset:{half_off(c)}", vset(base, 4)),
+                    (f"ds_read_b128 {vr(base + 4, 4)}, %[r{ks}] offset:{2 * TILE + half_off(c)}", vset(base + 4, 4))]
+        u, j = x
+        off = half_off(c) + u * 4096
+        loads = []
+        for i, db in enumerate((2 * j, 2 * j + 1)):
+            for hi in range(2):
+                reg = base + 4 * i + 2 * hi
+                loads.append((f"ds_read_b64_tr_b16 {vr(reg, 2)}, %[t{2 * db + hi}] offset:{off}", vset(reg, 2)))
+        return loads
+
+    def pair_mfmas(k):
+        kind, c, x = pairs[k]
+        base = V_STG + 8 * (k % NSLOT)
+        if kind == "A":
+            ks = x
+            s, dp = V_S[c & 1], V_DP[c & 1]
+            cs = "0" if ks == 0 else vr(s, 16)
+            cd = "0" if ks == 0 else vr(dp, 16)
+            return [(vr(s, 16), vr(base, 4), ar(A_Q + 4 * ks, 4), cs, vset(s, 16), vset(base, 4), aset(A_Q + 4 * ks, 4),
+                     set() if ks == 0 else vset(s, 16)),
+                    (vr(dp, 16), vr(base + 4, 4), ar(A_DO + 4 * ks, 4), cd, vset(dp, 16), vset(base + 4, 4),
+                     aset(A_DO + 4 * ks, 4), set() if ks == 0 else vset(dp, 16))]
+        u, j = x
+        ds = V_DS + 8 * (c & 1) + 4 * u
+        out = []
+        for i, db in enumerate((2 * j, 2 * j + 1)):
+            acc = A_DQ + 16 * db
+            out.append((ar(acc, 16), vr(base + 4 * i, 4), vr(ds, 4), ar(acc, 16), aset(acc, 16), vset(base + 4 * i, 4),
+                        vset(ds, 4), aset(acc, 16)))
+        return out
+
+    # ---- VALU work of E(c), spread over the MFMA slots of stage c ---------------------------
+    slot_valu = {m: [] for m in range(n_slots)}
+    slot_lds = {m: [] for m in range(n_slots)}
+    pre_lds = []
+    c2 = SREG["c2"]
+    for c in range(4):
+        s, dp = V_S[c & 1], V_DP[c & 1]
+        ops = []
+        for g in range(4):
+            for u in range(4):
+                e = 4 * g + u
+                ops.append((f"v_fma_f32 {vr(s + e)}, {vr(s + e)}, {c2}, -%[lse]", vset(s + e), vset(s + e), False))
+            for u in range(4):
+                e = 4 * g + u
+                ops.append((f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
+            if masked:
+                for u in range(4):
+                    e = 4 * g + u
+                    ops.append((f"v_bfe_i32 {vr(V_TMP + u)}, %[m{c >> 1}], {16 * (c & 1) + e}, 1", vset(V_TMP + u), set(), False))
+                for u in range(4):
+                    e = 4 * g + u
+                    ops.append((f"v_and_b32_e32 {vr(s + e)}, {vr(s + e)}, {vr(V_TMP + u)}", vset(s + e),
+                                vset(s + e) | vset(V_TMP + u), False))
+            for u in range(4):
+                e = 4 * g + u
+                ops.append((f"v_sub_f32_e32 {vr(dp + e)}, {vr(dp + e)}, %[dl]", vset(dp + e), vset(dp + e), False))
+            for u in range(4):
+                e = 4 * g + u
+                ops.append((f"v_mul_f32_e32 {vr(dp + e)}, {vr(s + e)}, {vr(dp + e)}", vset(dp + e), vset(dp + e) | vset(s + e), False))
+            ds = V_DS + 8 * (c & 1) + 4 * (g >> 1) + 2 * (g & 1)
+            for h in range(2):
+                e = 4 * g + 2 * h
+                ops.append((f"v_cvt_pk_bf16_f32 {vr(ds + h)}, {vr(dp + e)}, {vr(dp + e + 1)}", vset(ds + h), vset(dp + e, 2), False))
+        lo = first[c] + (6 if c == 0 else 0)  # E(0) directly follows A(0): give its results time
+        span = last[c] - lo
+        for i, op in enumerate(ops):
+            slot_valu[lo + (i * span) // len(ops)].append(op)
+
+    for k in range(len(pairs)):
+        at = 2 * (k - PREFETCH)
+        if at < 0:
+            pre_lds.extend(pair_loads(k))
+        else:
+            slot_lds[at] = pair_loads(k) + slot_lds[at]
+
+    # next step's K / V tiles: 16 LDS-direct loads per wave spread over the stream
+    slot_vmem = {m: [] for m in range(n_slots)}
+    k = 0
+    for t, gbase in enumerate((S_GK0, S_GK1, S_GV0, S_GV1)):  # half tiles in LDS order
+        for i in range(4):
+            slot_vmem[LOAD_FIRST + LOAD_EVERY * k].append((t * TILE + i * 1024, "%[g1v]" if i == 1 else f"%[g{i}]", gbase, S_LDSN))
+            k += 1
+
+    for text, dst in pre_lds:
+        em.lds_read(text, dst)
+    for m in range(n_slots):
+        for ld in slot_vmem[m]:
+            if "vmem" not in DROP:
+                em.lds_direct_load(*ld)
+        for text, dst in slot_lds[m]:
+            if "lds" not in DROP:
+                em.lds_read(text, dst)
+        if "mfma" not in DROP:
+            em.mfma(*pair_mfmas(m // 2)[m % 2])
+        for text, dst, src, trans in slot_valu[m]:
+            if "valu" not in DROP:
+                em.valu(text, dst, src, trans)
+    em.drain()
+    return em
+
+
+def run_loop(full, masked):
+    """One asm statement: a run of consecutive steps [it, it_end) of one work item, all full or a
+    single partial one.  At entry the step's K / V tiles are resident in LDS buffer %[buf]; each pass
+    computes the next step's addresses, streams the step (which copies the next step's tiles into the
+    other buffer), synchronises the work-group and advances."""
+    t0, t1, t2, t3 = S_T
+    S = SREG
+    n_tbl = len(TABLE)
+    entry = [f"ds_read_b128 {vr(V_TBL + 4 * i, 4)}, %[tbl] offset:{16 * i}" for i in range(n_tbl // 4)]
+    entry += ["s_waitcnt lgkmcnt(0)"]  # (the streams count LDS operations from zero)
+    entry += [f"v_readfirstlane_b32 {S[n]}, {vr(V_TBL + i)}" for i, n in enumerate(TABLE)]
+    entry += [f"v_readfirstlane_b32 {S[n]}, %[{n}]" for n in STATE_IO + STATE_IN]
+    top = entry + [".Lfa_dq_loop_%=:"]
+    # On the item's last step the tiles copied "for the next step" are the first step of the next
+    # work item (its kv tiles and K / V bases come from the table; with no next item they repeat
+    # this one's): the next item then starts without waiting for memory.
+    ka, kb_, kglo, kghi, vglo, vghi = S_SEL
+    top += [f"s_add_u32 {t0}, {S['it']}, 1", f"s_cmp_eq_u32 {t0}, {S['n_steps']}",
+            f"s_cselect_b32 {ka}, {S['kban']}, {S['kba1']}", f"s_cselect_b32 {kb_}, {S['kbbn']}, {S['kbb1']}",
+            f"s_cselect_b32 {kglo}, {S['kgn_lo']}, {S['kg_lo']}", f"s_cselect_b32 {kghi}, {S['kgn_hi']}, {S['kg_hi']}",
+            f"s_cselect_b32 {vglo}, {S['vgn_lo']}, {S['vg_lo']}", f"s_cselect_b32 {vghi}, {S['vgn_hi']}, {S['vg_hi']}"]
+    for pair, (blo, bhi), kb in ((S_GK0, (kglo, kghi), ka), (S_GK1, (kglo, kghi), kb_), (S_GV0, (vglo, vghi), ka),
+                                 (S_GV1, (vglo, vghi), kb_)):
+        n = int(pair[2:].split(":")[0])
+        top += [f"s_lshl_b32 {t2}, {kb}, 14", f"s_lshr_b32 {t3}, {kb}, 18",  # 64 rows x 256 bytes per kv tile
+                f"s_add_u32 s{n}, {blo}, {t2}", f"s_addc_u32 s{n + 1}, {bhi}, {t3}"]
+    top += [
+        f"s_xor_b32 {t1}, {S['buf']}, 1",
+        f"s_lshl_b32 {t1}, {t1}, 16",
+        f"s_add_u32 {S_LDSN}, {t1}, {S['w4k']}",
+        # list entries of the step after the next one, clamped into the list: a second half past its
+        # end repeats the last tile (finite data; its keep bits are zero)
+        f"s_add_u32 {t0}, {S['it']}, 2",
+        f"s_lshl_b32 {t0}, {t0}, 1",
+        f"s_sub_u32 {t1}, {S['n_tiles']}, 1",
+        f"s_min_u32 {t2}, {t0}, {t1}",
+        f"s_add_u32 {t0}, {t0}, 1",
+        f"s_min_u32 {t3}, {t0}, {t1}",
+        f"s_lshl_b32 {t2}, {t2}, 2",
+        f"s_lshl_b32 {t3}, {t3}, 2",
+        f"v_mov_b32_e32 {vr(V_KB2)}, {t2}",
+        f"v_mov_b32_e32 {vr(V_KB2 + 1)}, {t3}",
+        f"global_load_dword {vr(V_KB2)}, {vr(V_KB2)}, {S['idx']}",
+        f"global_load_dword {vr(V_KB2 + 1)}, {vr(V_KB2 + 1)}, {S['idx']}",
+        f"s_cmp_eq_u32 {S['partial']}, 0",
+        "s_cbranch_scc1 .Lfa_dq_full_%=",
+    ]
+    tail = [
+        ".Lfa_dq_tail_%=:",
+        "s_waitcnt vmcnt(0) lgkmcnt(0)",
+        "s_barrier",
+        f"s_add_u32 {S['it']}, {S['it']}, 1",
+        f"v_readfirstlane_b32 {S['kba1']}, {vr(V_KB2)}",
+        f"v_readfirstlane_b32 {S['kbb1']}, {vr(V_KB2 + 1)}",
+        f"s_xor_b32 {S['buf']}, {S['buf']}, 1",
+    ]
+    tail += [f"v_xor_b32_e32 %[r{i}], 0x10000, %[r{i}]" for i in range(8)]
+    tail += [f"v_xor_b32_e32 %[t{i}], 0x10000, %[t{i}]" for i in range(8)]
+    tail += [f"s_cmp_lt_u32 {S['it']}, {S['it_end']}", "s_cbranch_scc1 .Lfa_dq_loop_%="]
+    tail += [f"v_mov_b32_e32 %[{n}], {S[n]}" for n in STATE_IO]
+    return top + masked.out + ["s_branch .Lfa_dq_tail_%=", ".Lfa_dq_full_%=:"] + full.out + tail
+
+
+def main():
+    global DROP
+    here = os.path.dirname(os.path.abspath(__file__))
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("out", nargs="?", default=os.path.join(here, "bwd_dq_tile.inc"))
+    ap.add_argument("--drop", default="", help="comma list of mfma,valu,lds,vmem: leave these instruction classes out "
+                    "(the stream then computes nothing useful; for timing what bounds it)")
+    args = ap.parse_args()
+    if args.drop:
+        DROP = tuple(x for x in args.drop.split(",") if x)
+    with open(args.out, "w") as f:
+        f.write("// Generated by gen_dq_tile.py; do not edit.\n")
+
+        def macro(name, lines):
+            f.write(f"#define {name} \\\n")
+            f.write(" \\\n".join(f'  "{line}\\n"' for line in lines))
+            f.write("\n\n")
+
+        full, masked = build(False), build(True)
+        macro("FA_DQ_RUN", run_loop(full, masked))
+        for name, em in (("full", full), ("masked", masked)):
+            print(f"{args.out}: {name}: {len(em.out)} instructions, {em.stats}", file=sys.stderr)
+        macro("FA_DQ_ZERO_ACC", [f"v_accvgpr_write_b32 a{A_DQ + i}, 0" for i in range(64)])
+        # Q^T / dO^T fragment ks from 8 dword operands (two pinned outputs come first)
+        for ks in range(8):
+            macro(f"FA_DQ_PUT_{ks}",
+                  [f"v_accvgpr_write_b32 a{A_Q + 4 * ks + i}, %{2 + i}" for i in range(4)]
+                  + [f"v_accvgpr_write_b32 a{A_DO + 4 * ks + i}, %{6 + i}" for i in range(4)])
+        # accumulator tile t into 16 dword operands; the s_nop covers the MFMA -> read hazard
+        for t in range(4):
+            macro(f"FA_DQ_GET_ACC_{t}", ["s_nop 15"] + [f"v_accvgpr_read_b32 %{i}, a{A_DQ + 16 * t + i}" for i in range(16)])
+
+
+if __name__ == "__main__":
+    main()

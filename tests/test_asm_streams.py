@@ -181,3 +181,14 @@ def test_compiler_keeps_out_of_the_pinned_registers(tmp_path):
             assert "scratch_" not in line, f"spill in the plain-score dk/dv kernel: {line}"
             for kind, i in regs_of(line.split(";")[0]):
                 assert not (kind == "a" and i <= 191), f"compiler touches a pinned register: {line}"
+
+
+def test_dq_tile_streams_respect_hazards():
+    import gen_dq_tile as g
+
+    for masked in (False, True):
+        em = g.build(masked)
+        n = check_stream(em.out)
+        assert em.stats["mfma"] == 96  # 4 kv blocks x (8 S + 8 dP + 8 dq)
+        assert n == em.stats["mfma"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
+        scratch_ok(em.out, 66, 215, 127)
