@@ -23,7 +23,8 @@ SOURCES = [
 ]
 
 # instruction streams generated before compiling: (generator script, output it writes next to itself)
-GENERATED = [("gen_dkv_tile.py", "bwd_dkv_tile.inc"), ("gen_dq_tile.py", "bwd_dq_tile.inc")]
+GENERATED = [("gen_dkv_tile.py", "bwd_dkv_tile.inc"), ("gen_dq_tile.py", "bwd_dq_tile.inc"),
+             ("gen_fwd_tile.py", "fwd_tile.inc")]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -19,22 +19,22 @@
 
 #include <type_traits>
 
-// registers v[68:255] belong to the generated tile streams
-#define FA_DKV_TILE_CLOBBERS "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", "v78", \
-  "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", \
-  "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", \
-  "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", \
-  "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", \
-  "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", \
-  "v147", "v148", "v149", "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", \
-  "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167", "v168", "v169", "v170", "v171", "v172", \
-  "v173", "v174", "v175", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", "v185", \
-  "v186", "v187", "v188", "v189", "v190", "v191", "v192", "v193", "v194", "v195", "v196", "v197", "v198", \
-  "v199", "v200", "v201", "v202", "v203", "v204", "v205", "v206", "v207", "v208", "v209", "v210", "v211", \
-  "v212", "v213", "v214", "v215", "v216", "v217", "v218", "v219", "v220", "v221", "v222", "v223", "v224", \
-  "v225", "v226", "v227", "v228", "v229", "v230", "v231", "v232", "v233", "v234", "v235", "v236", "v237", \
-  "v238", "v239", "v240", "v241", "v242", "v243", "v244", "v245", "v246", "v247", "v248", "v249", "v250", \
-  "v251", "v252", "v253", "v254", "v255"
+// v[68:191] and a[192:255] belong to the generated tile streams
+#define FA_DKV_TILE_CLOBBERS "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79", "v80", "v81", "v82", \
+  "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", \
+  "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", \
+  "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", \
+  "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", \
+  "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", \
+  "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", \
+  "v163", "v164", "v165", "v166", "v167", "v168", "v169", "v170", "v171", "v172", "v173", "v174", "v175", \
+  "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", "v185", "v186", "v187", "v188", \
+  "v189", "v190", "v191", "a192", "a193", "a194", "a195", "a196", "a197", "a198", "a199", "a200", "a201", \
+  "a202", "a203", "a204", "a205", "a206", "a207", "a208", "a209", "a210", "a211", "a212", "a213", "a214", \
+  "a215", "a216", "a217", "a218", "a219", "a220", "a221", "a222", "a223", "a224", "a225", "a226", "a227", \
+  "a228", "a229", "a230", "a231", "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239", "a240", \
+  "a241", "a242", "a243", "a244", "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", \
+  "a254", "a255"
 
 // scalar registers of the generated run loop
 #define FA_DKV_RUN_SGPRS "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", "s87", "s88", "s89", "s90", "s91", "s92", "s93", "s94", "s95", "s96", "s97", "s98", "s99", "s100"
@@ -49,7 +49,7 @@ constexpr int BQ = 128;   // q rows per step (two 64-row LDS tiles)
 constexpr int D = 128;
 constexpr int MAX_LIST = 1024;  // longest q tile list the plain-score kernel caches in LDS
 // (Q, dO) x 2 buffers x 2 tiles, lse x2, delta x2, run-loop tables, cached q tile list and its partial flags
-constexpr int LDS_BYTES = 8 * kTileElems * 2 + 4 * BQ * 4 + 4 * 16 * 4 + MAX_LIST * 5;
+constexpr int LDS_BYTES = 8 * kTileElems * 2 + 4 * BQ * 4 + 4 * 32 * 4 + MAX_LIST * 5;
 }  // namespace dkv_cfg
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
@@ -335,86 +335,99 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   // it then runs n_wg / gridDim.x work items back to back, which saves the gap between the end of a
   // work-group and the start of the next one on the CU (only one fits at a time).
   const int n_items = n_wg / (int)gridDim.x;
-  for (int item = 0; item < n_items; ++item) {
-  const int wg = persistent_item((int)blockIdx.x, item, (int)gridDim.x, n_wg, nKb);
-  const int bhk = wg / nKb;
-  const int kb = wg % nKb;
-  const int b = bhk / a.Hkv;
-  const int hk = bhk % a.Hkv;
-  if (item > 0) __syncthreads();  // the previous item's LDS contents are dead from here
-
   const int kv_local = w * 32 + l32;
-  const int k_idx = kb * BNK + kv_local;
-  const size_t kv_off = ((size_t)bhk * a.Sk + (size_t)kb * BNK) * D;
-  const bf16_t* Kg = static_cast<const bf16_t*>(a.k) + kv_off;
-  const bf16_t* Vg = static_cast<const bf16_t*>(a.v) + kv_off;
-  const size_t rows0 = (size_t)(b * a.Hq + hk * group) * a.Sq;  // first row of the group's first query head
-  const bf16_t* Qg = static_cast<const bf16_t*>(a.q) + rows0 * D;
-  const bf16_t* dOg = static_cast<const bf16_t*>(a.dout) + rows0 * D;
+  const int row = tid & (BQ - 1);
   // waves 0, 1 turn (l, m) into lse for rows tid & 127; waves 2, 3 pass delta through
   const bool lse_wave = w < 2;
-  const float* rowa = (lse_wave ? a.l : a.delta) + rows0;
-  const float* rowb = (lse_wave ? a.m : a.delta) + rows0;
-  const int row = tid & (BQ - 1);
-
-  PinnedState st;
-  asm volatile(FA_DKV_ZERO_ACC
-               : "={a[0:15]}"(st.dv[0]), "={a[16:31]}"(st.dv[1]), "={a[32:47]}"(st.dv[2]), "={a[48:63]}"(st.dv[3]),
-                 "={a[64:79]}"(st.dk[0]), "={a[80:95]}"(st.dk[1]), "={a[96:111]}"(st.dk[2]), "={a[112:127]}"(st.dk[3]));
-#define FA_PUT(KS, KR, VR)                                                                                          \
-  {                                                                                                                 \
-    const u32x4 kw = *reinterpret_cast<const u32x4*>(Kg + (size_t)kv_local * D + KS * 16 + hh * 8);                 \
-    const u32x4 vw = *reinterpret_cast<const u32x4*>(Vg + (size_t)kv_local * D + KS * 16 + hh * 8);                 \
-    asm volatile(FA_DKV_PUT_KV_##KS                                                                                 \
-                 : "={" KR "}"(st.k[KS]), "={" VR "}"(st.v[KS])                                                     \
-                 : "v"(kw[0]), "v"(kw[1]), "v"(kw[2]), "v"(kw[3]), "v"(vw[0]), "v"(vw[1]), "v"(vw[2]), "v"(vw[3])); \
-  }
-  FA_PUT(0, "a[128:131]", "a[160:163]") FA_PUT(1, "a[132:135]", "a[164:167]")
-  FA_PUT(2, "a[136:139]", "a[168:171]") FA_PUT(3, "a[140:143]", "a[172:175]")
-  FA_PUT(4, "a[144:147]", "a[176:179]") FA_PUT(5, "a[148:151]", "a[180:183]")
-  FA_PUT(6, "a[152:155]", "a[184:187]") FA_PUT(7, "a[156:159]", "a[188:191]")
-#undef FA_PUT
-  int doc_j = 0;
-  if (a.mask.flags & FLEXATTN_MASK_DOC) doc_j = a.mask.doc_k[k_idx];
-
-  const int* tile_idx = a.map.idx + (size_t)kb * nQ;
-  const int qb_first = tile_idx[0];  // (nQ >= 1: always readable; used only if the list is not empty)
-  const int n_tiles = __builtin_amdgcn_readfirstlane(a.map.cnt[kb]);
-  const int n_iter = n_tiles * group;
-
-  // The kv tile's q list and which of its tiles are partial, cached in LDS: finding runs of full
-  // tiles then costs no dependent global loads.
-  int* sIdx = reinterpret_cast<int*>(sDl + 2 * BQ) + 4 * 16;
-  unsigned char* sPart = reinterpret_cast<unsigned char*>(sIdx + MAX_LIST);
-  for (int t = tid; t < n_tiles; t += 256) {
-    const int q = tile_idx[t];
-    sIdx[t] = q;
-    sPart[t] = a.map.state[(size_t)q * a.map.nk + kb] == 1 ? 1 : 0;
-  }
-
+  int* sIdx = reinterpret_cast<int*>(sDl + 2 * BQ) + 4 * 32;
+  unsigned char* sPart = reinterpret_cast<unsigned char*>(sIdx + MAX_LIST);  // by q tile: 1 = partial with this kv tile
   TileLoader<4> loader;
   loader.init(w, lane);
-  if (n_iter > 0) {
-    // first step: tiles and row values into buffer 0
-    const int qb0 = __builtin_amdgcn_readfirstlane(qb_first);
-    const size_t r0 = (size_t)qb0 * BQ;
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      loader.load(Qg + (r0 + half * kTileRows) * D, sT + half * kTileElems);
-      loader.load(dOg + (r0 + half * kTileRows) * D, sT + (2 + half) * kTileElems);
-    }
-    const float x = rowa[r0 + row], y = rowb[r0 + row];
-    if (lse_wave) {
-      sLse[row] = (x > 0.f) ? __builtin_fmaf(y, kLog2e, log2f(x)) : __builtin_huge_valf();
-    } else {
-      sDl[row] = x;
-    }
-  }
-  wait_vmem_all();
-  __syncthreads();
 
-  // byte addresses of the lane's operand fragments in buffer 0 (see tile_io.hpp); the run loop
-  // flips them between the buffers together with `buf`
+  // An item is kv tile kb of (batch, kv head) pair bhk.  Its addresses are cheap to derive from the
+  // two numbers, so only those are carried from item to item.
+  struct Geometry {
+    int bhk, kb;
+  };
+  auto geometry = [&](int item) {
+    const int wg = persistent_item((int)blockIdx.x, item, (int)gridDim.x, n_wg, nKb);
+    Geometry g;
+    g.bhk = __builtin_amdgcn_readfirstlane(wg / nKb);
+    g.kb = __builtin_amdgcn_readfirstlane(wg % nKb);
+    return g;
+  };
+  auto kv_offset = [&](const Geometry& g) { return ((size_t)g.bhk * a.Sk + (size_t)g.kb * BNK) * D; };
+  // first row of the group's first query head: (b Hq + hk group) Sq with bhk = b Hkv + hk
+  auto first_row = [&](const Geometry& g) { return (size_t)g.bhk * group * a.Sq; };
+
+  // Everything an item needs from global memory before its first step is fetched while the previous
+  // item runs: plain loads whose values are not touched until that item's last step is done.  (They
+  // live in v[192:255] and the low registers, which the run loop leaves alone.)
+  constexpr int kListRegs = MAX_LIST / 256;
+  struct ItemRegs {
+    u32x4 kw[8], vw[8];            // K / V fragments of the lane's kv row
+    int doc, n_tiles, qb0;         // list length and its first entry
+    int idx[kListRegs];            // q list entries tid + 256 j
+    unsigned char part[kListRegs]; // state of q tile tid + 256 j against this kv tile
+  };
+  // (opaque(): addresses derived from its result are computed where they are used instead of once
+  // before the item loop, where they would have to be kept, spilled, through every run)
+  auto opaque = [](int x) {
+    asm volatile("" : "+v"(x));
+    return x;
+  };
+  auto fetch = [&](const Geometry& g, ItemRegs& r) {
+    const int tid_here = opaque(tid);
+    const bf16_t* Kg = static_cast<const bf16_t*>(a.k) + kv_offset(g);
+    const bf16_t* Vg = static_cast<const bf16_t*>(a.v) + kv_offset(g);
+    const int kv_here = (tid_here >> 6) * 32 + (tid_here & 31);
+    const int hh_here = (tid_here >> 5) & 1;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      r.kw[ks] = *reinterpret_cast<const u32x4*>(Kg + (size_t)kv_here * D + ks * 16 + hh_here * 8);
+      r.vw[ks] = *reinterpret_cast<const u32x4*>(Vg + (size_t)kv_here * D + ks * 16 + hh_here * 8);
+    }
+    r.doc = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_k[g.kb * BNK + kv_local] : 0;
+    const int* tile_idx = a.map.idx + (size_t)g.kb * nQ;
+    r.n_tiles = a.map.cnt[g.kb];
+    r.qb0 = tile_idx[0];  // (nQ >= 1: always readable; used only if the list is not empty)
+#pragma unroll
+    for (int j = 0; j < kListRegs; ++j) {
+      const int t = tid_here + 256 * j;
+      r.idx[j] = (t < nQ) ? tile_idx[t] : 0;  // (slots past the list length hold no valid entry and are never used)
+      r.part[j] = (t < nQ) ? a.map.state[(size_t)t * a.map.nk + g.kb] : 0;
+    }
+  };
+  // What is left of an item's fetched values once its K / V fragments sit in their registers.
+  struct ItemHead {
+    int doc, n_tiles, qb0;
+    int idx[kListRegs];
+    unsigned char part[kListRegs];
+  };
+  PinnedState st;
+  auto consume = [&](const ItemRegs& r, ItemHead& c) {
+#define FA_PUT(KS, KR, VR)                                                                                    \
+  asm volatile(FA_DKV_PUT_KV_##KS                                                                             \
+               : "={" KR "}"(st.k[KS]), "={" VR "}"(st.v[KS])                                                 \
+               : "v"(r.kw[KS][0]), "v"(r.kw[KS][1]), "v"(r.kw[KS][2]), "v"(r.kw[KS][3]), "v"(r.vw[KS][0]),    \
+                 "v"(r.vw[KS][1]), "v"(r.vw[KS][2]), "v"(r.vw[KS][3]));
+    FA_PUT(0, "a[128:131]", "a[160:163]") FA_PUT(1, "a[132:135]", "a[164:167]")
+    FA_PUT(2, "a[136:139]", "a[168:171]") FA_PUT(3, "a[140:143]", "a[172:175]")
+    FA_PUT(4, "a[144:147]", "a[176:179]") FA_PUT(5, "a[148:151]", "a[180:183]")
+    FA_PUT(6, "a[152:155]", "a[184:187]") FA_PUT(7, "a[156:159]", "a[188:191]")
+#undef FA_PUT
+    c.doc = r.doc;
+    c.n_tiles = __builtin_amdgcn_readfirstlane(r.n_tiles);
+    c.qb0 = __builtin_amdgcn_readfirstlane(r.qb0);
+#pragma unroll
+    for (int j = 0; j < kListRegs; ++j) {
+      c.idx[j] = r.idx[j];
+      c.part[j] = r.part[j];
+    }
+  };
+
+  // Byte addresses of the lane's operand fragments and row values in LDS step buffer 0 (see
+  // tile_io.hpp); the run loop flips them between the two buffers together with `buf`, across items too.
   const int r_sw = swz(l32);
   const int t_row = 4 * hh + ((lane & 15) >> 2);
   const int t_chunk = 2 * ((lane & 31) >> 4) + ((lane & 3) >> 1);
@@ -428,10 +441,76 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     ta[i] = base0 + (unsigned)(tile_off(t_row + 8 * (i & 1), 4 * (i >> 1) + t_chunk) + t_half) * 2u;
   unsigned la = (unsigned)(size_t)(sLse + 4 * hh);
   unsigned lw = (unsigned)(size_t)((lse_wave ? sLse : sDl) + BQ + row);  // this lane's row value of the NEXT buffer
+  int buf = 0;
+  bool resident = false;  // the item's first step was already copied into buffer `buf` by the previous item's last step
+
+  ItemRegs pre;
+  ItemHead cur;
+  Geometry geo = geometry(0);
+  fetch(geo, pre);
+  consume(pre, cur);
+
+  for (int item = 0; item < n_items; ++item) {
+  const int kb = geo.kb;
+  const int k_idx = kb * BNK + kv_local;
+  const size_t kv_off = kv_offset(geo);
+  const size_t rows0 = first_row(geo);
+  const bf16_t* Qg = static_cast<const bf16_t*>(a.q) + rows0 * D;
+  const bf16_t* dOg = static_cast<const bf16_t*>(a.dout) + rows0 * D;
+  const float* rowa = (lse_wave ? a.l : a.delta) + rows0;
+  const float* rowb = (lse_wave ? a.m : a.delta) + rows0;
+  const int doc_j = cur.doc;
+  const int* tile_idx = a.map.idx + (size_t)kb * nQ;
+  const int n_tiles = cur.n_tiles;
+  const int n_iter = n_tiles * group;
+  if (item > 0) __syncthreads();  // the previous item's list and row values are dead from here
+
+  asm volatile(FA_DKV_ZERO_ACC
+               : "={a[0:15]}"(st.dv[0]), "={a[16:31]}"(st.dv[1]), "={a[32:47]}"(st.dv[2]), "={a[48:63]}"(st.dv[3]),
+                 "={a[64:79]}"(st.dk[0]), "={a[80:95]}"(st.dk[1]), "={a[96:111]}"(st.dk[2]), "={a[112:127]}"(st.dk[3]));
+
+  // The kv tile's q list and which q tiles are partial against it, cached in LDS: finding runs of
+  // full tiles then costs no global loads.
+  const int tid_p = opaque(tid);  // (fresh per item: see opaque())
+#pragma unroll
+  for (int j = 0; j < kListRegs; ++j) {
+    const int t = tid_p + 256 * j;
+    if (t < nQ) {
+      sIdx[t] = cur.idx[j];
+      sPart[t] = cur.part[j] == 1 ? 1 : 0;
+    }
+  }
+  if (n_iter > 0 && !resident) {
+    // first step into the current buffer: tiles (LDS-direct) and the lane's row value
+    const size_t r0 = (size_t)cur.qb0 * BQ;
+    bf16_t* dst = sT + (size_t)buf * 4 * kTileElems;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      loader.load(Qg + (r0 + half * kTileRows) * D, dst + half * kTileElems);
+      loader.load(dOg + (r0 + half * kTileRows) * D, dst + (2 + half) * kTileElems);
+    }
+    const int row_p = tid_p & (BQ - 1);
+    const float x = rowa[r0 + row_p], y = rowb[r0 + row_p];
+    if (lse_wave) {
+      sLse[buf * BQ + row_p] = (x > 0.f) ? __builtin_fmaf(y, kLog2e, log2f(x)) : __builtin_huge_valf();
+    } else {
+      sDl[buf * BQ + row_p] = x;
+    }
+    wait_vmem_all();
+  }
+  resident = false;
+  __syncthreads();
+  // The next item's list lands while this item runs.  (The last item fetches itself again: every
+  // path then redefines the fetched registers, so none of them has to live through the run loop.)
+  const bool has_next = item + 1 < n_items;
+  const Geometry geo_n = has_next ? geometry(item + 1) : geo;
+  fetch(geo_n, pre);
+
   const unsigned tid4 = (unsigned)row * 4u;
-  // Work-group constants of the run loop, one 16-dword table per wave behind the row values
-  // (order: TABLE in gen_dkv_tile.py).  Written and read by the same wave: no barrier needed.
-  unsigned* tbl = reinterpret_cast<unsigned*>(sDl + 2 * BQ) + w * 16;
+  // Work-group constants of the run loop, one 32-dword table per wave behind the row values
+  // (order: TABLE in gen_dkv_tile.py; the second half names the next item's first step, see below).
+  // Written and read by the same wave: no barrier needed.
+  unsigned* tbl = reinterpret_cast<unsigned*>(sDl + 2 * BQ) + w * 32;
   if (lane == 0) {
     tbl[0] = (unsigned)n_tiles;
     tbl[1] = (unsigned)(group - 1);
@@ -454,7 +533,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
 
   // Step `it` is q tile tile_idx[it % n_tiles] of query head it / n_tiles of the group.  Carried:
   // the list positions of steps it + 1 and it + 2, the head of step it + 1, its q block index.
-  int it = 0, buf = 0, g1 = 0, p1 = 1, p2 = 2;
+  int it = 0, g1 = 0, p1 = 1, p2 = 2;
   if (p1 >= n_tiles) { p1 -= n_tiles; g1 = 1; }
   if (p2 >= n_tiles) p2 -= n_tiles;
   if (p2 >= n_tiles) p2 -= n_tiles;
@@ -465,7 +544,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     int p0 = p1 - 1;
     if (p0 < 0) p0 += n_tiles;
     const int qb = __builtin_amdgcn_readfirstlane(sIdx[p0]);
-    const bool partial = __builtin_amdgcn_readfirstlane((int)sPart[p0]) == 1;
+    const bool partial = __builtin_amdgcn_readfirstlane((int)sPart[qb]) == 1;
     int it_end = it + 1;
     unsigned km[2] = {0u, 0u};
     if (partial) {
@@ -493,7 +572,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
         bool is_partial = false;
         if (j < n_iter) {
           const int pj = (p0 + (j - it)) % n_tiles;
-          is_partial = sPart[pj] == 1;
+          is_partial = sPart[sIdx[pj]] == 1;
         }
         const unsigned long long hits = __ballot(is_partial);
         if (hits != 0ull) {
@@ -505,7 +584,34 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
       }
     }
     it_end = __builtin_amdgcn_readfirstlane(it_end);
-    const int partial_flag = partial ? 1 : 0;
+    // The run that ends the item copies the next item's first step during its last step (bit 1 of
+    // the flags; the table's second half says where it is).  The fetched values are first touched
+    // here, an item's length after their loads were issued.
+    int flags = partial ? 1 : 0;
+    if (it_end == n_iter && has_next) {
+      const int nt = __builtin_amdgcn_readfirstlane(pre.n_tiles);
+      if (nt > 0) {
+        flags |= 2;
+        const int qb0_n = __builtin_amdgcn_readfirstlane(pre.qb0);
+        const size_t rows_n = first_row(geo_n);
+        const bf16_t* Qg_n = static_cast<const bf16_t*>(a.q) + rows_n * D;
+        const bf16_t* dOg_n = static_cast<const bf16_t*>(a.dout) + rows_n * D;
+        const float* rowa_n = (lse_wave ? a.l : a.delta) + rows_n;
+        const float* rowb_n = (lse_wave ? a.m : a.delta) + rows_n;
+        if (lane == 0) {
+          tbl[16] = (unsigned)(size_t)Qg_n;
+          tbl[17] = (unsigned)((size_t)Qg_n >> 32);
+          tbl[18] = (unsigned)(size_t)dOg_n;
+          tbl[19] = (unsigned)((size_t)dOg_n >> 32);
+          tbl[20] = (unsigned)(size_t)rowa_n;
+          tbl[21] = (unsigned)((size_t)rowa_n >> 32);
+          tbl[22] = (unsigned)(size_t)rowb_n;
+          tbl[23] = (unsigned)((size_t)rowb_n >> 32);
+          tbl[24] = (unsigned)qb0_n;
+        }
+        resident = true;
+      }
+    }
     // no scalar operands (see gen_dkv_tile.py): the loop state travels in VGPRs
     asm volatile(FA_DKV_RUN
                  : FA_DKV_PINNED(st), [it] "+v"(it), [p1] "+v"(p1), [g1] "+v"(g1), [p2] "+v"(p2), [qb1] "+v"(qb1),
@@ -513,16 +619,29 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
                    [r4] "+v"(ra[4]), [r5] "+v"(ra[5]), [r6] "+v"(ra[6]), [r7] "+v"(ra[7]), [t0] "+v"(ta[0]),
                    [t1] "+v"(ta[1]), [t2] "+v"(ta[2]), [t3] "+v"(ta[3]), [t4] "+v"(ta[4]), [t5] "+v"(ta[5]),
                    [t6] "+v"(ta[6]), [t7] "+v"(ta[7]), [la] "+v"(la), [lw] "+v"(lw)
-                 : [it_end] "v"(it_end), [partial] "v"(partial_flag), [tbl] "v"(tbl_addr), [g0] "v"(loader.goff[0]),
+                 : [it_end] "v"(it_end), [partial] "v"(flags), [tbl] "v"(tbl_addr), [g0] "v"(loader.goff[0]),
                    [g1v] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]), [g3] "v"(loader.goff[3]), [m0] "v"(km[0]),
                    [m1] "v"(km[1]), [tid4] "v"(tid4)
                  : "memory", "scc", "vcc", "m0", FA_DKV_RUN_SGPRS, "v67", FA_DKV_TILE_CLOBBERS);
     it = __builtin_amdgcn_readfirstlane(it);
     p1 = __builtin_amdgcn_readfirstlane(p1);
+    buf = __builtin_amdgcn_readfirstlane(buf);
   }
 
-  f32x16 dk_acc[4], dv_acc[4];
-#define FA_GET(T, SRC, REG, DST)                                                                                   \
+  // ---- item epilogue ----
+  // The next item's K / V fragments go into their registers before this item's stores are issued
+  // (their loads are long done; behind the stores the wait would include the stores).
+  consume(pre, cur);
+
+  // dk / dv: bf16 rows staged through the wave's 16 KB of the free LDS step buffer (16-byte chunks XOR-swizzled
+  // by row), so that every store instruction writes four complete 256-byte rows.
+  {
+    // (buffer `buf` may hold the next item's first step: the other one is free)
+    char* stage = reinterpret_cast<char*>(sT + (size_t)(buf ^ 1) * 4 * kTileElems) + w * 16384;
+    const int lane_here = opaque(lane);
+    const int row_here = lane_here & 31;
+    const unsigned wr = (unsigned)row_here * 256u + 8u * (unsigned)(lane_here >> 5);
+#define FA_GET(T, SRC, REG, MAT, DB, SCALE)                                                                        \
   {                                                                                                                \
     float x[16];                                                                                                   \
     asm volatile(FA_DKV_GET_ACC_##T                                                                                \
@@ -530,31 +649,35 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
                    "=v"(x[8]), "=v"(x[9]), "=v"(x[10]), "=v"(x[11]), "=v"(x[12]), "=v"(x[13]), "=v"(x[14]),        \
                    "=v"(x[15])                                                                                     \
                  : "{" REG "}"(SRC));                                                                              \
-    _Pragma("unroll") for (int e = 0; e < 16; ++e) DST[e] = x[e];                                                  \
+    _Pragma("unroll") for (int g = 0; g < 4; ++g) {                                                                \
+      const bf16x2 lo = pack_bf16(x[4 * g] * SCALE, x[4 * g + 1] * SCALE);                                         \
+      const bf16x2 hi = pack_bf16(x[4 * g + 2] * SCALE, x[4 * g + 3] * SCALE);                                     \
+      const bf16x4 out = {lo[0], lo[1], hi[0], hi[1]};                                                             \
+      *reinterpret_cast<bf16x4*>(stage + MAT * 8192 + wr + (unsigned)(((4 * DB + g) ^ (row_here & 15)) << 4)) = out; \
+    }                                                                                                              \
   }
-  FA_GET(0, st.dv[0], "a[0:15]", dv_acc[0]) FA_GET(1, st.dv[1], "a[16:31]", dv_acc[1])
-  FA_GET(2, st.dv[2], "a[32:47]", dv_acc[2]) FA_GET(3, st.dv[3], "a[48:63]", dv_acc[3])
-  FA_GET(4, st.dk[0], "a[64:79]", dk_acc[0]) FA_GET(5, st.dk[1], "a[80:95]", dk_acc[1])
-  FA_GET(6, st.dk[2], "a[96:111]", dk_acc[2]) FA_GET(7, st.dk[3], "a[112:127]", dk_acc[3])
+    // the streams leave the constant sm_scale out of dS: dk takes it here
+    FA_GET(0, st.dv[0], "a[0:15]", 1, 0, 1.f) FA_GET(1, st.dv[1], "a[16:31]", 1, 1, 1.f)
+    FA_GET(2, st.dv[2], "a[32:47]", 1, 2, 1.f) FA_GET(3, st.dv[3], "a[48:63]", 1, 3, 1.f)
+    FA_GET(4, st.dk[0], "a[64:79]", 0, 0, a.sm_scale) FA_GET(5, st.dk[1], "a[80:95]", 0, 1, a.sm_scale)
+    FA_GET(6, st.dk[2], "a[96:111]", 0, 2, a.sm_scale) FA_GET(7, st.dk[3], "a[112:127]", 0, 3, a.sm_scale)
 #undef FA_GET
-
-  // the streams leave the constant sm_scale out of dS: apply it to dk once
-  bf16_t* dKg = static_cast<bf16_t*>(a.dk) + kv_off;
-  bf16_t* dVg = static_cast<bf16_t*>(a.dv) + kv_off;
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    bf16_t* dKg = static_cast<bf16_t*>(a.dk) + kv_off + (size_t)(w * 32) * D;
+    bf16_t* dVg = static_cast<bf16_t*>(a.dv) + kv_off + (size_t)(w * 32) * D;
+    const int chunk = lane_here & 15;
 #pragma unroll
-  for (int db = 0; db < 4; ++db) {
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      bf16x2 lo = pack_bf16(dk_acc[db][4 * g] * a.sm_scale, dk_acc[db][4 * g + 1] * a.sm_scale);
-      bf16x2 hi = pack_bf16(dk_acc[db][4 * g + 2] * a.sm_scale, dk_acc[db][4 * g + 3] * a.sm_scale);
-      bf16x4 out = {lo[0], lo[1], hi[0], hi[1]};
-      *reinterpret_cast<bf16x4*>(dKg + (size_t)kv_local * D + 32 * db + 8 * g + 4 * hh) = out;
-      lo = pack_bf16(dv_acc[db][4 * g], dv_acc[db][4 * g + 1]);
-      hi = pack_bf16(dv_acc[db][4 * g + 2], dv_acc[db][4 * g + 3]);
-      bf16x4 out2 = {lo[0], lo[1], hi[0], hi[1]};
-      *reinterpret_cast<bf16x4*>(dVg + (size_t)kv_local * D + 32 * db + 8 * g + 4 * hh) = out2;
+    for (int i = 0; i < 8; ++i) {
+      const int r = 4 * i + (lane_here >> 4);
+      const unsigned rd = (unsigned)r * 256u + (unsigned)((chunk ^ (r & 15)) << 4);
+      const u32x4 kx = *reinterpret_cast<const u32x4*>(stage + rd);
+      const u32x4 vx = *reinterpret_cast<const u32x4*>(stage + 8192 + rd);
+      *reinterpret_cast<u32x4*>(dKg + (size_t)r * D + chunk * 8) = kx;
+      *reinterpret_cast<u32x4*>(dVg + (size_t)r * D + chunk * 8) = vx;
     }
   }
+  geo = geo_n;
   }  // work items
 }
 

@@ -362,8 +362,45 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   int buf = 0;
   bool resident = false;  // the item's first step was already copied into buffer `buf` by the previous item's last step
 
+  // What is left of an item's fetched values once its Q^T / dO^T fragments sit in their registers.
+  struct ItemHead {
+    float l, m, delta;
+    int doc, n_tiles, kb0, kb1;
+    int idx[kListRegs];
+    unsigned char st[kListRegs];
+  };
+  DqPinned st;
+  auto consume = [&](const ItemRegs& r, ItemHead& c) {
+#define FA_PUT(KS, QR, DR)                                                                                    \
+  asm volatile(FA_DQ_PUT_##KS                                                                                 \
+               : "={" QR "}"(st.q[KS]), "={" DR "}"(st.d[KS])                                                 \
+               : "v"(r.qw[KS][0]), "v"(r.qw[KS][1]), "v"(r.qw[KS][2]), "v"(r.qw[KS][3]), "v"(r.dw[KS][0]),    \
+                 "v"(r.dw[KS][1]), "v"(r.dw[KS][2]), "v"(r.dw[KS][3]));
+    FA_PUT(0, "a[64:67]", "a[96:99]") FA_PUT(1, "a[68:71]", "a[100:103]") FA_PUT(2, "a[72:75]", "a[104:107]")
+    FA_PUT(3, "a[76:79]", "a[108:111]") FA_PUT(4, "a[80:83]", "a[112:115]") FA_PUT(5, "a[84:87]", "a[116:119]")
+    FA_PUT(6, "a[88:91]", "a[120:123]") FA_PUT(7, "a[92:95]", "a[124:127]")
+#undef FA_PUT
+    c.l = r.l; c.m = r.m; c.delta = r.delta; c.doc = r.doc;
+    c.n_tiles = __builtin_amdgcn_readfirstlane(r.n_tiles);
+    c.kb0 = __builtin_amdgcn_readfirstlane(r.kb0);
+    c.kb1 = __builtin_amdgcn_readfirstlane(r.kb1);
+#pragma unroll
+    for (int j = 0; j < kListRegs; ++j) {
+      c.idx[j] = r.idx[j];
+      c.st[j] = r.st[j];
+    }
+  };
+  // (opaque(): addresses derived from its result are computed where they are used instead of once
+  // before the item loop, where they would have to be kept through every run)
+  auto opaque = [](int x) {
+    asm volatile("" : "+v"(x));
+    return x;
+  };
+
   ItemRegs pre;
+  ItemHead cur;
   fetch(0, pre);
+  consume(pre, cur);
   for (int item = 0; item < n_items; ++item) {
     int bh, qb;
     geometry(item, bh, qb);
@@ -379,34 +416,25 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
     const int* tile_idx = a.map.idx + (size_t)qb * nK;
 
     // the q tile's kv list and its state row into LDS
-    const int n_tiles = __builtin_amdgcn_readfirstlane(pre.n_tiles);
+    const int n_tiles = cur.n_tiles;
     const int n_steps = (n_tiles + 1) >> 1;
+    const int tid_p = opaque(tid);  // (fresh per item: see opaque())
 #pragma unroll
     for (int j = 0; j < kListRegs; ++j) {
-      const int t = tid + 256 * j;
+      const int t = tid_p + 256 * j;
       if (t < nK) {
-        sIdx[t] = pre.idx[j];
-        sSt[t] = pre.st[j];
+        sIdx[t] = cur.idx[j];
+        sSt[t] = cur.st[j];
       }
     }
 
-    DqPinned st;
     asm volatile(FA_DQ_ZERO_ACC
                  : "={a[0:15]}"(st.dq[0]), "={a[16:31]}"(st.dq[1]), "={a[32:47]}"(st.dq[2]), "={a[48:63]}"(st.dq[3]));
-#define FA_PUT(KS, QR, DR)                                                                                    \
-  asm volatile(FA_DQ_PUT_##KS                                                                                 \
-               : "={" QR "}"(st.q[KS]), "={" DR "}"(st.d[KS])                                                 \
-               : "v"(pre.qw[KS][0]), "v"(pre.qw[KS][1]), "v"(pre.qw[KS][2]), "v"(pre.qw[KS][3]), "v"(pre.dw[KS][0]), \
-                 "v"(pre.dw[KS][1]), "v"(pre.dw[KS][2]), "v"(pre.dw[KS][3]));
-    FA_PUT(0, "a[64:67]", "a[96:99]") FA_PUT(1, "a[68:71]", "a[100:103]") FA_PUT(2, "a[72:75]", "a[104:107]")
-    FA_PUT(3, "a[76:79]", "a[108:111]") FA_PUT(4, "a[80:83]", "a[112:115]") FA_PUT(5, "a[84:87]", "a[116:119]")
-    FA_PUT(6, "a[88:91]", "a[120:123]") FA_PUT(7, "a[92:95]", "a[124:127]")
-#undef FA_PUT
-    const float lse2 = (pre.l > 0.f) ? __builtin_fmaf(pre.m, kLog2e, log2f(pre.l)) : __builtin_huge_valf();
-    const float delta = pre.delta;
-    const int doc_i = pre.doc;
-    const int kb_first = __builtin_amdgcn_readfirstlane(pre.kb0);
-    const int kb_second = (n_tiles > 1) ? __builtin_amdgcn_readfirstlane(pre.kb1) : kb_first;
+    const float lse2 = (cur.l > 0.f) ? __builtin_fmaf(cur.m, kLog2e, log2f(cur.l)) : __builtin_huge_valf();
+    const float delta = cur.delta;
+    const int doc_i = cur.doc;
+    const int kb_first = cur.kb0;
+    const int kb_second = (n_tiles > 1) ? cur.kb1 : kb_first;
     if (n_tiles > 0 && !resident) {
       // first step into the current buffer (a missing second entry repeats the first: finite data, masked out)
       bf16_t* dst = sT + (size_t)buf * 4 * kTileElems;
@@ -414,17 +442,17 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
       loader.load(Kg + (size_t)kb_second * BN * D, dst + kTileElems);
       loader.load(Vg + (size_t)kb_first * BN * D, dst + 2 * kTileElems);
       loader.load(Vg + (size_t)kb_second * BN * D, dst + 3 * kTileElems);
+      wait_vmem_all();
     }
     unsigned* tbl = sTbl + w * 16;
     const unsigned tbl_addr = (unsigned)(size_t)tbl;
-    wait_vmem_all();
     __syncthreads();
-    // the next item's data lands while this item's first step runs
+    // The next item's data lands while this item runs.  (The last item fetches itself again: every
+    // path then redefines the fetched registers, and the compiler need not merge old values in.)
+    const bool has_next = item + 1 < n_items;
     int bh_n = bh, qb_n = qb;
-    if (item + 1 < n_items) {
-      fetch(item + 1, pre);
-      geometry(item + 1, bh_n, qb_n);
-    }
+    if (has_next) geometry(item + 1, bh_n, qb_n);
+    fetch(has_next ? item + 1 : item, pre);
     const int b_n = bh_n / a.Hq, hk_n = (bh_n % a.Hq) / (a.Hq / a.Hkv);
     const bf16_t* Kg_n = static_cast<const bf16_t*>(a.k) + ((size_t)(b_n * a.Hkv + hk_n) * a.Sk) * D;
     const bf16_t* Vg_n = static_cast<const bf16_t*>(a.v) + ((size_t)(b_n * a.Hkv + hk_n) * a.Sk) * D;
@@ -492,7 +520,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
       // first step (its values were fetched at the start of this item; only now are they touched).
       {
         int kb_na = kb_first, kb_nb = kb_second;
-        if (it_end == n_steps && item + 1 < n_items) {
+        if (it_end == n_steps && has_next) {
           const int nt = __builtin_amdgcn_readfirstlane(pre.n_tiles);
           kb_na = nt > 0 ? __builtin_amdgcn_readfirstlane(pre.kb0) : 0;
           kb_nb = nt > 1 ? __builtin_amdgcn_readfirstlane(pre.kb1) : kb_na;
@@ -531,10 +559,22 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
       buf = __builtin_amdgcn_readfirstlane(buf);
     }
     // the last step of a non-empty item copied the next item's first step into buffer `buf`
-    resident = n_steps > 0 && item + 1 < n_items && __builtin_amdgcn_readfirstlane(pre.n_tiles) > 0;
+    resident = n_steps > 0 && has_next && __builtin_amdgcn_readfirstlane(pre.n_tiles) > 0;
 
-    f32x16 dq_acc[4];
-#define FA_GET(T, SRC, REG, DST)                                                                                   \
+    // ---- item epilogue ----
+    // The next item's Q^T / dO^T fragments go into their registers before this item's stores are
+    // issued (their loads are long done; behind the stores the wait would include the stores).
+    consume(pre, cur);
+
+    // dq: bf16 rows staged through the wave's 8 KB of the free LDS step buffer (16-byte chunks
+    // XOR-swizzled by row), so that every store instruction writes four complete 256-byte rows.
+    // (Buffer `buf` may hold the next item's first step: the other one is free.)
+    {
+      char* stage = reinterpret_cast<char*>(sT + (size_t)(buf ^ 1) * 4 * kTileElems) + w * 8192;
+      const int lane_here = opaque(lane);
+      const int row_here = lane_here & 31;
+      const unsigned wr = (unsigned)row_here * 256u + 8u * (unsigned)(lane_here >> 5);
+#define FA_GET(T, SRC, REG)                                                                                        \
   {                                                                                                                \
     float x[16];                                                                                                   \
     asm volatile(FA_DQ_GET_ACC_##T                                                                                 \
@@ -542,20 +582,26 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
                    "=v"(x[8]), "=v"(x[9]), "=v"(x[10]), "=v"(x[11]), "=v"(x[12]), "=v"(x[13]), "=v"(x[14]),        \
                    "=v"(x[15])                                                                                     \
                  : "{" REG "}"(SRC));                                                                              \
-    _Pragma("unroll") for (int e = 0; e < 16; ++e) DST[e] = x[e];                                                  \
+    _Pragma("unroll") for (int g = 0; g < 4; ++g) {                                                                \
+      /* the streams leave the constant sm_scale out of dS: apply it once */                                       \
+      const bf16x2 lo = pack_bf16(x[4 * g] * a.sm_scale, x[4 * g + 1] * a.sm_scale);                               \
+      const bf16x2 hi = pack_bf16(x[4 * g + 2] * a.sm_scale, x[4 * g + 3] * a.sm_scale);                           \
+      const bf16x4 out = {lo[0], lo[1], hi[0], hi[1]};                                                             \
+      *reinterpret_cast<bf16x4*>(stage + wr + (unsigned)(((4 * T + g) ^ (row_here & 15)) << 4)) = out;             \
+    }                                                                                                              \
   }
-    FA_GET(0, st.dq[0], "a[0:15]", dq_acc[0]) FA_GET(1, st.dq[1], "a[16:31]", dq_acc[1])
-    FA_GET(2, st.dq[2], "a[32:47]", dq_acc[2]) FA_GET(3, st.dq[3], "a[48:63]", dq_acc[3])
+      FA_GET(0, st.dq[0], "a[0:15]") FA_GET(1, st.dq[1], "a[16:31]")
+      FA_GET(2, st.dq[2], "a[32:47]") FA_GET(3, st.dq[3], "a[48:63]")
 #undef FA_GET
-    // the streams leave the constant sm_scale out of dS: apply it once
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      bf16_t* out_rows = dQg + (size_t)(w * 32) * D;
+      const int chunk = lane_here & 15;
 #pragma unroll
-    for (int db = 0; db < 4; ++db) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        bf16x2 lo = pack_bf16(dq_acc[db][4 * g] * a.sm_scale, dq_acc[db][4 * g + 1] * a.sm_scale);
-        bf16x2 hi = pack_bf16(dq_acc[db][4 * g + 2] * a.sm_scale, dq_acc[db][4 * g + 3] * a.sm_scale);
-        bf16x4 out = {lo[0], lo[1], hi[0], hi[1]};
-        *reinterpret_cast<bf16x4*>(dQg + (size_t)q_local * D + 32 * db + 8 * g + 4 * hh) = out;
+      for (int i = 0; i < 8; ++i) {
+        const int r = 4 * i + (lane_here >> 4);
+        const u32x4 x = *reinterpret_cast<const u32x4*>(stage + (unsigned)r * 256u + (unsigned)((chunk ^ (r & 15)) << 4));
+        *reinterpret_cast<u32x4*>(out_rows + (size_t)r * D + chunk * 8) = x;
       }
     }
   }  // work items

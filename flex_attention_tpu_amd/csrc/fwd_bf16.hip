@@ -6,9 +6,32 @@
 // are double-buffered in LDS by LDS-direct loads issued one tile ahead; P goes straight from the
 // QK accumulators to the B operand of the PV MFMA (O^T = V^T P^T); V^T is fetched with
 // transposing LDS reads.
+#include <cstdlib>
+
 #include "fa_common.hpp"
 #include "launch.hpp"
 #include "tile_io.hpp"
+
+// registers of the generated run loop (gen_fwd_tile.py): v[66:245], s[60:100]
+#define FA_FWD_RUN_VGPRS "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", \
+  "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", \
+  "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", \
+  "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", \
+  "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", \
+  "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", \
+  "v146", "v147", "v148", "v149", "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", \
+  "v159", "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167", "v168", "v169", "v170", "v171", \
+  "v172", "v173", "v174", "v175", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", \
+  "v185", "v186", "v187", "v188", "v189", "v190", "v191", "v192", "v193", "v194", "v195", "v196", "v197", \
+  "v198", "v199", "v200", "v201", "v202", "v203", "v204", "v205", "v206", "v207", "v208", "v209", "v210", \
+  "v211", "v212", "v213", "v214", "v215", "v216", "v217", "v218", "v219", "v220", "v221", "v222", "v223", \
+  "v224", "v225", "v226", "v227", "v228", "v229", "v230", "v231", "v232", "v233", "v234", "v235", "v236", \
+  "v237", "v238", "v239", "v240", "v241", "v242", "v243", "v244", "v245"
+#define FA_FWD_RUN_SGPRS "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", \
+  "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", \
+  "s87", "s88", "s89", "s90", "s91", "s92", "s93", "s94", "s95", "s96", "s97", "s98", "s99", "s100"
+
+#include "fwd_tile.inc"
 
 namespace fa {
 
@@ -17,7 +40,27 @@ constexpr int BM = 128;  // q rows per work-group
 constexpr int BN = 64;   // kv rows per step
 constexpr int D = 128;
 constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2
+// plain-score kernel: 256 q rows per work item, steps of two kv tiles: (K, K, V, V) x 2 buffers, per-wave
+// tables, wave counters, merged kv list, the two state rows
+constexpr int MAX_LIST = 1024;
+constexpr int PLAIN_LDS_BYTES = 8 * kTileElems * 2 + 4 * 16 * 4 + 16 + MAX_LIST * 4 + 2 * MAX_LIST;
 }  // namespace fwd_cfg
+
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+// Register-resident state of the generated streams: every asm statement names it with the same
+// physical-register constraints, so it stays put and the compiler keeps those registers free.
+struct FwdPinned {
+  f32x16 o[8];    // a[0:127]: O^T accumulators of q block 0 (4) and 1 (4)
+  bf16x8 q[16];   // a[128:191]: Q^T fragments of q block 0 (8) and 1 (8)
+};
+#define FA_FWD_PINNED(st)                                                                                       \
+  "+{a[0:15]}"(st.o[0]), "+{a[16:31]}"(st.o[1]), "+{a[32:47]}"(st.o[2]), "+{a[48:63]}"(st.o[3]),                \
+      "+{a[64:79]}"(st.o[4]), "+{a[80:95]}"(st.o[5]), "+{a[96:111]}"(st.o[6]), "+{a[112:127]}"(st.o[7]),        \
+      "+{a[128:131]}"(st.q[0]), "+{a[132:135]}"(st.q[1]), "+{a[136:139]}"(st.q[2]), "+{a[140:143]}"(st.q[3]),   \
+      "+{a[144:147]}"(st.q[4]), "+{a[148:151]}"(st.q[5]), "+{a[152:155]}"(st.q[6]), "+{a[156:159]}"(st.q[7]),   \
+      "+{a[160:163]}"(st.q[8]), "+{a[164:167]}"(st.q[9]), "+{a[168:171]}"(st.q[10]), "+{a[172:175]}"(st.q[11]), \
+      "+{a[176:179]}"(st.q[12]), "+{a[180:183]}"(st.q[13]), "+{a[184:187]}"(st.q[14]), "+{a[188:191]}"(st.q[15])
 
 template <int SCORE>
 __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
@@ -300,9 +343,341 @@ static int launch_fwd(const FwdArgs& a, hipStream_t stream) {
   return check_launch("flexattn_fwd bf16");
 }
 
+// ------------------------------------------------------------------------------------------------
+// Plain score: the main loop runs inside generated asm statements (gen_fwd_tile.py).  A work item is
+// a pair of 128-row q tiles of one head (q block x = tile 2 qb2 + x; wave w owns rows 32 w .. of
+// each); its kv tiles are the union of the two tiles' non-empty entries of the block map's state
+// rows, merged into one list in LDS.  A step is two list entries (128 kv rows); one statement
+// executes a run of consecutive full steps, or one partial step with the lane's keep bits.
+// Work-groups are persistent (one per CU) when persistent_ok() finds a balanced schedule.  The
+// kernel has no static shared memory: the dynamic buffer starts at LDS address 0.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) {
+  using namespace fwd_cfg;
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  bf16_t* sT = reinterpret_cast<bf16_t*>(smem_raw);  // buffer b: K tile 0, K tile 1, V tile 0, V tile 1
+  unsigned* sTbl = reinterpret_cast<unsigned*>(sT + 8 * kTileElems);
+  int* sCnt = reinterpret_cast<int*>(sTbl + 4 * 16);
+  int* sList = sCnt + 4;
+  unsigned char* sStA = reinterpret_cast<unsigned char*>(sList + MAX_LIST);
+  unsigned char* sStB = sStA + MAX_LIST;
+
+  const int nQ = a.Sq / BM;
+  const int nQ2 = (nQ + 1) >> 1;
+  const int nK = a.map.nk;
+  const int n_wg = a.B * a.Hq * nQ2;
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int l32 = lane & 31;
+  const int hh = lane >> 5;
+  const int q_local = w * 32 + l32;
+
+  TileLoader<4> loader;
+  loader.init(w, lane);
+  const int r_sw = swz(l32);
+  const int t_row = 4 * hh + ((lane & 15) >> 2);
+  const int t_chunk = 2 * ((lane & 31) >> 4) + ((lane & 3) >> 1);
+  const int t_half = 4 * (lane & 1);
+  const unsigned base0 = (unsigned)(size_t)sT;
+  // Byte addresses of the lane's operand fragments in LDS step buffer 0 (K half-tile 0); the run
+  // loop flips them between the two buffers together with `buf`, across items too.
+  unsigned ra[8], ta[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) ra[ks] = base0 + (unsigned)(l32 * kTileD + (((2 * ks + hh) ^ r_sw) << 3)) * 2u;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    ta[i] = base0 + (unsigned)(tile_off(t_row + 8 * (i & 1), 4 * (i >> 1) + t_chunk) + t_half) * 2u;
+  int buf = 0;
+
+  // Everything an item needs from global memory before its first step, fetched while the previous
+  // item runs (plain loads whose values are not touched until then).
+  constexpr int kListRegs = MAX_LIST / 256;
+  struct ItemRegs {
+    u32x4 qw[2][8];                 // Q^T fragments of the lane's two q rows
+    int doc[2];
+    unsigned char sa[kListRegs], sb[kListRegs];  // states of kv tile tid + 256 j in the two state rows
+  };
+  const int n_items = n_wg / (int)gridDim.x;
+  auto geometry = [&](int item, int& bh, int& qb2) {
+    const int wg = persistent_item((int)blockIdx.x, item, (int)gridDim.x, n_wg, nQ2);
+    bh = wg / nQ2;
+    qb2 = (gridDim.x == (unsigned)n_wg) ? nQ2 - 1 - (wg % nQ2) : wg % nQ2;  // one item each: longest first
+  };
+  auto fetch = [&](int item, ItemRegs& r) {
+    int bh, qb2;
+    geometry(item, bh, qb2);
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+      const int qb = min(2 * qb2 + x, nQ - 1);  // (a missing second tile repeats the first; nothing of it is stored)
+      const bf16_t* Qg = static_cast<const bf16_t*>(a.q) + ((size_t)bh * a.Sq + (size_t)qb * BM + q_local) * D;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) r.qw[x][ks] = *reinterpret_cast<const u32x4*>(Qg + ks * 16 + hh * 8);
+      r.doc[x] = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[qb * BM + q_local] : 0;
+      const uint8_t* row = a.map.state + (size_t)qb * nK;
+      const bool valid = 2 * qb2 + x < nQ;
+#pragma unroll
+      for (int j = 0; j < kListRegs; ++j) {
+        const int t = tid + 256 * j;
+        const unsigned char v = (valid && t < nK) ? row[t] : 0;
+        if (x == 0) r.sa[j] = v; else r.sb[j] = v;
+      }
+    }
+  };
+
+  ItemRegs pre;
+  fetch(0, pre);
+  for (int item = 0; item < n_items; ++item) {
+    int bh, qb2;
+    geometry(item, bh, qb2);
+    const int b = bh / a.Hq;
+    const int h = bh % a.Hq;
+    const int hk = h / (a.Hq / a.Hkv);
+    const bf16_t* Kg = static_cast<const bf16_t*>(a.k) + ((size_t)(b * a.Hkv + hk) * a.Sk) * D;
+    const bf16_t* Vg = static_cast<const bf16_t*>(a.v) + ((size_t)(b * a.Hkv + hk) * a.Sk) * D;
+    if (item > 0) __syncthreads();  // the previous item's LDS contents are dead from here
+
+    // the two state rows into LDS, then the merged list of kv tiles that are non-empty for either
+    // q tile, in ascending order (ballot compaction per wave, wave offsets through LDS)
+#pragma unroll
+    for (int j = 0; j < kListRegs; ++j) {
+      const int t = tid + 256 * j;
+      if (t < nK) {
+        sStA[t] = pre.sa[j];
+        sStB[t] = pre.sb[j];
+      }
+    }
+    int n_list = 0;
+#pragma unroll
+    for (int j = 0; j < kListRegs; ++j) {
+      if (256 * j < nK) {
+        const int t = tid + 256 * j;
+        const bool present = t < nK && (pre.sa[j] | pre.sb[j]) != 0;
+        const unsigned long long mask = __ballot(present);
+        if (lane == 0) sCnt[w] = __builtin_popcountll(mask);
+        __syncthreads();
+        int off = n_list;
+        for (int ww = 0; ww < 4; ++ww) {
+          const int cw = sCnt[ww];
+          if (ww < w) off += cw;
+          n_list += cw;
+        }
+        if (present) sList[off + __builtin_popcountll(mask & ((1ull << lane) - 1ull))] = t;
+        __syncthreads();
+      }
+    }
+    n_list = __builtin_amdgcn_readfirstlane(n_list);
+    const int n_steps = (n_list + 1) >> 1;
+
+    FwdPinned st;
+    asm volatile(FA_FWD_ZERO_ACC
+                 : "={a[0:15]}"(st.o[0]), "={a[16:31]}"(st.o[1]), "={a[32:47]}"(st.o[2]), "={a[48:63]}"(st.o[3]),
+                   "={a[64:79]}"(st.o[4]), "={a[80:95]}"(st.o[5]), "={a[96:111]}"(st.o[6]), "={a[112:127]}"(st.o[7]));
+#define FA_PUT(KS, Q0, Q1)                                                                                        \
+  asm volatile(FA_FWD_PUT_##KS                                                                                    \
+               : "={" Q0 "}"(st.q[KS]), "={" Q1 "}"(st.q[8 + KS])                                                 \
+               : "v"(pre.qw[0][KS][0]), "v"(pre.qw[0][KS][1]), "v"(pre.qw[0][KS][2]), "v"(pre.qw[0][KS][3]),      \
+                 "v"(pre.qw[1][KS][0]), "v"(pre.qw[1][KS][1]), "v"(pre.qw[1][KS][2]), "v"(pre.qw[1][KS][3]));
+    FA_PUT(0, "a[128:131]", "a[160:163]") FA_PUT(1, "a[132:135]", "a[164:167]") FA_PUT(2, "a[136:139]", "a[168:171]")
+    FA_PUT(3, "a[140:143]", "a[172:175]") FA_PUT(4, "a[144:147]", "a[176:179]") FA_PUT(5, "a[148:151]", "a[180:183]")
+    FA_PUT(6, "a[152:155]", "a[184:187]") FA_PUT(7, "a[156:159]", "a[188:191]")
+#undef FA_PUT
+    const int doc_i[2] = {pre.doc[0], pre.doc[1]};
+    const int q_idx[2] = {(2 * qb2) * BM + q_local, (2 * qb2 + 1) * BM + q_local};
+    // softmax state of the lane's two q rows (log2 domain): reference maximum (finite start value:
+    // -inf would turn 2^(score - M) of a masked score into NaN), true maximum, sum
+    float M[2] = {-1.0e30f, -1.0e30f}, Mt[2] = {kNegInf, kNegInf}, L[2] = {0.f, 0.f};
+
+    auto entry = [&](int e) { return sList[e < n_list ? e : n_list - 1]; };
+    if (n_list > 0) {
+      // first step into the current buffer (a missing second entry repeats the first: finite data, masked out)
+      const int ka = __builtin_amdgcn_readfirstlane(entry(0));
+      const int kbb = __builtin_amdgcn_readfirstlane(entry(1));
+      bf16_t* dst = sT + (size_t)buf * 4 * kTileElems;
+      loader.load(Kg + (size_t)ka * BN * D, dst);
+      loader.load(Kg + (size_t)kbb * BN * D, dst + kTileElems);
+      loader.load(Vg + (size_t)ka * BN * D, dst + 2 * kTileElems);
+      loader.load(Vg + (size_t)kbb * BN * D, dst + 3 * kTileElems);
+    }
+    unsigned* tbl = sTbl + w * 16;
+    const unsigned tbl_addr = (unsigned)(size_t)tbl;
+    const unsigned lst_addr = (unsigned)(size_t)sList;
+    wait_vmem_all();
+    __syncthreads();
+    if (item + 1 < n_items) fetch(item + 1, pre);  // lands while this item's first step runs
+
+    int it = 0;
+    int kba1 = (n_list > 0) ? __builtin_amdgcn_readfirstlane(entry(2)) : 0;
+    int kbb1 = (n_list > 0) ? __builtin_amdgcn_readfirstlane(entry(3)) : 0;
+    // a step is full when both of its entries exist and are full for both q tiles
+    auto entry_full = [&](int e) {
+      const int k = sList[e];
+      return sStA[k] == 2 && sStB[k] == 2;
+    };
+    auto step_full = [&](int sidx) { return 2 * sidx + 1 < n_list && entry_full(2 * sidx) && entry_full(2 * sidx + 1); };
+
+    while (it < n_steps) {
+      const bool partial = __builtin_amdgcn_readfirstlane(step_full(it) ? 0 : 1) == 1;
+      int it_end = it + 1;
+      unsigned km[4] = {0u, 0u, 0u, 0u};  // keep bits of q block x, kv tile hx of the step: km[2 x + hx]
+      if (partial) {
+        const bool has_doc = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
+#pragma unroll
+        for (int hx = 0; hx < 2; ++hx) {
+          const int e = 2 * it + hx;
+          if (e >= n_list) continue;  // missing half: all dropped
+          const int k = __builtin_amdgcn_readfirstlane(sList[e]);
+#pragma unroll
+          for (int x = 0; x < 2; ++x) {
+            const int state = __builtin_amdgcn_readfirstlane((int)(x == 0 ? sStA[k] : sStB[k]));
+            if (state == 0) continue;
+            if (state == 2) {
+              km[2 * x + hx] = 0xffffffffu;
+              continue;
+            }
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+#pragma unroll
+              for (int g = 0; g < 4; ++g) {
+                const int j0 = k * BN + 32 * c + 8 * g + 4 * hh;
+                int dj[4] = {0, 0, 0, 0};
+                if (has_doc) {
+                  const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_k + j0);
+                  dj[0] = d4[0]; dj[1] = d4[1]; dj[2] = d4[2]; dj[3] = d4[3];
+                }
+                km[2 * x + hx] |= keep_bits4_keys(a.mask, q_idx[x], j0, doc_i[x], dj) << (16 * c + 4 * g);
+              }
+            }
+          }
+        }
+      } else {
+        // the run of full steps ends before the next partial one: lanes look 64 steps ahead at a time
+        bool found = false;
+        while (!found && it_end < n_steps) {
+          const int j = it_end + lane;
+          const bool is_partial = j < n_steps && !step_full(j);
+          const unsigned long long hits = __ballot(is_partial);
+          if (hits != 0ull) {
+            it_end += __builtin_ctzll(hits);
+            found = true;
+          } else {
+            it_end = (it_end + 64 < n_steps) ? it_end + 64 : n_steps;
+          }
+        }
+      }
+      it_end = __builtin_amdgcn_readfirstlane(it_end);
+      const int partial_flag = partial ? 1 : 0;
+      // work-group constants of the run loop, one table per wave (order: TABLE in gen_fwd_tile.py),
+      // written and read by the same wave; "next item" entries repeat this item's (its first step is
+      // loaded by its own prologue)
+      if (lane == 0) {
+        const int ka = entry(0), kbb = entry(1);
+        tbl[0] = (unsigned)n_list;
+        tbl[1] = base0 + (unsigned)w * 4096u;  // LDS address of the wave's first 1 KB block in buffer 0
+        tbl[2] = __builtin_bit_cast(unsigned, a.sm_scale * kLog2e);
+        tbl[3] = (unsigned)n_steps;
+        tbl[4] = (unsigned)(size_t)Kg;
+        tbl[5] = (unsigned)((size_t)Kg >> 32);
+        tbl[6] = (unsigned)(size_t)Vg;
+        tbl[7] = (unsigned)((size_t)Vg >> 32);
+        tbl[8] = (unsigned)ka;
+        tbl[9] = (unsigned)kbb;
+        tbl[10] = (unsigned)(size_t)Kg;
+        tbl[11] = (unsigned)((size_t)Kg >> 32);
+        tbl[12] = (unsigned)(size_t)Vg;
+        tbl[13] = (unsigned)((size_t)Vg >> 32);
+        tbl[14] = 0u;
+        tbl[15] = 0u;
+      }
+      // no scalar operands (see gen_fwd_tile.py): the loop state travels in VGPRs
+      asm volatile(FA_FWD_RUN
+                   : FA_FWD_PINNED(st), [it] "+v"(it), [kba1] "+v"(kba1), [kbb1] "+v"(kbb1), [buf] "+v"(buf),
+                     [M0] "+v"(M[0]), [M1] "+v"(M[1]), [Mt0] "+v"(Mt[0]), [Mt1] "+v"(Mt[1]), [L0] "+v"(L[0]),
+                     [L1] "+v"(L[1]), [r0] "+v"(ra[0]), [r1] "+v"(ra[1]), [r2] "+v"(ra[2]), [r3] "+v"(ra[3]),
+                     [r4] "+v"(ra[4]), [r5] "+v"(ra[5]), [r6] "+v"(ra[6]), [r7] "+v"(ra[7]), [t0] "+v"(ta[0]),
+                     [t1] "+v"(ta[1]), [t2] "+v"(ta[2]), [t3] "+v"(ta[3]), [t4] "+v"(ta[4]), [t5] "+v"(ta[5]),
+                     [t6] "+v"(ta[6]), [t7] "+v"(ta[7])
+                   : [it_end] "v"(it_end), [partial] "v"(partial_flag), [tbl] "v"(tbl_addr), [lst] "v"(lst_addr),
+                     [g0] "v"(loader.goff[0]), [g1v] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]),
+                     [g3] "v"(loader.goff[3]), [m0] "v"(km[0]), [m1] "v"(km[1]), [m2] "v"(km[2]), [m3] "v"(km[3])
+                   : "memory", "scc", "vcc", "m0", FA_FWD_RUN_SGPRS, FA_FWD_RUN_VGPRS);
+      it = __builtin_amdgcn_readfirstlane(it);
+      buf = __builtin_amdgcn_readfirstlane(buf);
+    }
+
+    // ---- epilogue: O = O^T / l, exact (l, m) from the reference-maximum bookkeeping ----
+#define FA_GET(T, SRC, REG, DST)                                                                                   \
+  {                                                                                                                \
+    float xv[16];                                                                                                  \
+    asm volatile(FA_FWD_GET_ACC_##T                                                                                \
+                 : "=v"(xv[0]), "=v"(xv[1]), "=v"(xv[2]), "=v"(xv[3]), "=v"(xv[4]), "=v"(xv[5]), "=v"(xv[6]),      \
+                   "=v"(xv[7]), "=v"(xv[8]), "=v"(xv[9]), "=v"(xv[10]), "=v"(xv[11]), "=v"(xv[12]), "=v"(xv[13]),  \
+                   "=v"(xv[14]), "=v"(xv[15])                                                                      \
+                 : "{" REG "}"(SRC));                                                                              \
+    _Pragma("unroll") for (int e = 0; e < 16; ++e) DST[e] = xv[e];                                                 \
+  }
+    f32x16 o_acc[8];
+    FA_GET(0, st.o[0], "a[0:15]", o_acc[0]) FA_GET(1, st.o[1], "a[16:31]", o_acc[1])
+    FA_GET(2, st.o[2], "a[32:47]", o_acc[2]) FA_GET(3, st.o[3], "a[48:63]", o_acc[3])
+    FA_GET(4, st.o[4], "a[64:79]", o_acc[4]) FA_GET(5, st.o[5], "a[80:95]", o_acc[5])
+    FA_GET(6, st.o[6], "a[96:111]", o_acc[6]) FA_GET(7, st.o[7], "a[112:127]", o_acc[7])
+#undef FA_GET
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+      const float l_tot = half_sum(L[x]);
+      if (2 * qb2 + x < nQ) {
+        const float inv = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
+        bf16_t* Og = static_cast<bf16_t*>(a.o) + ((size_t)bh * a.Sq + (size_t)(2 * qb2 + x) * BM) * D;
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const f32x16& oa = o_acc[4 * x + db];
+            bf16x2 lo = pack_bf16(oa[4 * g] * inv, oa[4 * g + 1] * inv);
+            bf16x2 hi = pack_bf16(oa[4 * g + 2] * inv, oa[4 * g + 3] * inv);
+            bf16x4 out = {lo[0], lo[1], hi[0], hi[1]};
+            *reinterpret_cast<bf16x4*>(Og + (size_t)q_local * D + 32 * db + 8 * g + 4 * hh) = out;
+          }
+        }
+        if (a.l != nullptr && hh == 0) {
+          const size_t r = (size_t)bh * a.Sq + q_idx[x];
+          // sums were taken against the reference maximum M: move them to the true maximum Mt
+          a.l[r] = (l_tot > 0.f) ? l_tot * fast_exp2(M[x] - Mt[x]) : 0.f;
+          a.m[r] = Mt[x] * kLn2;  // natural units
+        }
+      }
+    }
+  }  // work items
+}
+
+static int launch_fwd_plain(const FwdArgs& a, hipStream_t stream) {
+  using namespace fwd_cfg;
+  auto kern = fwd_bf16_d128_plain_kernel;
+  static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, PLAIN_LDS_BYTES);
+  if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(fwd): %s", hipGetErrorString(attr));
+  const int nQ2 = (a.Sq / BM + 1) / 2;
+  const int n_wg = a.B * a.Hq * nQ2;
+  const int grid = persistent_ok(n_wg, nQ2) ? 256 : n_wg;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), PLAIN_LDS_BYTES, stream, a);
+  return check_launch("flexattn_fwd bf16");
+}
+
+static bool fwd_stream_requested() {
+  const char* v = std::getenv("FLEXATTN_FWD_STREAM");
+  return v != nullptr && v[0] == '1';
+}
+
 int fwd_bf16_d128(const FwdArgs& a, hipStream_t stream) {
   switch (a.score.kind) {
-    case FLEXATTN_SCORE_NONE: return launch_fwd<FLEXATTN_SCORE_NONE>(a, stream);
+    case FLEXATTN_SCORE_NONE:
+      // The generated-stream kernel (one wave per SIMD, 64 q rows per wave) is correct but its
+      // stream is bound by the VALU work of the online softmax and is slower than the compiled
+      // kernel (two waves per SIMD); it runs only on request, FLEXATTN_FWD_STREAM=1, for plain
+      // scores whose state rows and merged kv list fit in LDS, and needs sm_scale > 0.
+      return (fwd_stream_requested() && a.map.nk <= fwd_cfg::MAX_LIST && a.sm_scale > 0.f)
+                 ? launch_fwd_plain(a, stream)
+                 : launch_fwd<FLEXATTN_SCORE_NONE>(a, stream);
     case FLEXATTN_SCORE_ALIBI: return launch_fwd<FLEXATTN_SCORE_ALIBI>(a, stream);
     case FLEXATTN_SCORE_SOFTCAP: return launch_fwd<FLEXATTN_SCORE_SOFTCAP>(a, stream);
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_fwd<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);

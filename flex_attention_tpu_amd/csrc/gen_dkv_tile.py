@@ -23,11 +23,14 @@ Register contract with the C++ side (every asm statement names the accumulation 
 physical-register constraints; prologue / epilogue macros are generated here too):
     a[0:63]    dv accumulators (4 x 16)      a[64:127]  dk accumulators (4 x 16)
     a[128:159] K fragments (8 x 4)           a[160:191] V fragments (8 x 4)
-    v[67:255]  scratch of the run loop and its streams (clobbered), s[84:100], vcc, m0 likewise
+    v[67:191]  scratch of the run loop and its streams (clobbered), s[60:100], vcc, m0 likewise
+    a[192:255] staging slots of the LDS fragments (clobbered): MFMA operands only, so they can be
+               AGPRs, and v[192:255] stay with the compiler for what lives across the run loop
     %[r0..r7]  byte address of the lane's row fragment ks in the step's Q half-tile 0
     %[t0..t7]  byte address of the lane's transposed fragment (2 db + hi) in Q half-tile 0
     %[la]      byte address of the lane's first lse value of the step;  s64 sm_scale * log2(e)
-    %[partial] scalar, non-zero selects the masked stream
+    %[partial] flags: bit 0 selects the masked stream, bit 1 says that the run ends its work item and
+               that the table's second half (next item's Q, dO, row bases, first q block) is valid
     %[g0..g3]  the lane's byte offsets inside a global half tile for the wave's four 1 KB blocks;
     %[gq0], %[gq1], %[gd0], %[gd1]  global addresses (SGPR pairs) of the next step's Q / dO half tiles;
     %[ldsn]    LDS byte address of the wave's first block in the next step's buffer
@@ -43,7 +46,7 @@ import sys
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 from gfx950_stream import Emitter, ar, aset, vr, vset  # noqa: E402
 
-NSLOT = 8        # staging slots of 8 VGPRs
+NSLOT = 8        # staging slots of 8 registers
 PREFETCH = 4     # MFMA pairs between the LDS reads of a pair and its MFMAs
 LOAD_FIRST = 2   # MFMA slot of the first LDS-direct load of the next step
 LOAD_EVERY = 6   # slots between two of them
@@ -76,7 +79,7 @@ V_PB = 136
 V_DSB = 152
 V_LSE = 168   # 3 buffers x 4
 V_DL = 180    # 3 buffers x 4
-V_STG = 192
+A_STG = 192   # 8 staging slots x 8 registers for LDS fragments: AGPRs, which leaves v[192:255] to the compiler
 V_TMP = 68    # 4 temporaries of the masked variant
 DL_OFFSET = 1024
 
@@ -108,43 +111,43 @@ def build(masked):
 
     def pair_loads(k):
         kind, c, x = pairs[k]
-        base = V_STG + 8 * (k % NSLOT)
+        base = A_STG + 8 * (k % NSLOT)
         loads = []
         if kind == "A":
             ks = x
-            loads.append((f"ds_read_b128 {vr(base, 4)}, %[r{ks}] offset:{half_off(c)}", vset(base, 4)))
-            loads.append((f"ds_read_b128 {vr(base + 4, 4)}, %[r{ks}] offset:{2 * TILE + half_off(c)}", vset(base + 4, 4)))
+            loads.append((f"ds_read_b128 {ar(base, 4)}, %[r{ks}] offset:{half_off(c)}", aset(base, 4)))
+            loads.append((f"ds_read_b128 {ar(base + 4, 4)}, %[r{ks}] offset:{2 * TILE + half_off(c)}", aset(base + 4, 4)))
         else:
             u, db = x
             off = half_off(c) + u * 4096
             for which, reg0 in ((2 * TILE, base), (0, base + 4)):  # dO fragment, then Q fragment
                 for hi in range(2):
-                    loads.append((f"ds_read_b64_tr_b16 {vr(reg0 + 2 * hi, 2)}, %[t{2 * db + hi}] offset:{which + off}",
-                                  vset(reg0 + 2 * hi, 2)))
+                    loads.append((f"ds_read_b64_tr_b16 {ar(reg0 + 2 * hi, 2)}, %[t{2 * db + hi}] offset:{which + off}",
+                                  aset(reg0 + 2 * hi, 2)))
         return loads
 
     def pair_mfmas(k):
         kind, c, x = pairs[k]
-        base = V_STG + 8 * (k % NSLOT)
+        base = A_STG + 8 * (k % NSLOT)
         if kind == "A":
             ks = x
             s, dp = V_S[c & 1], V_DP[c & 1]
             cs = "0" if ks == 0 else vr(s, 16)
             cd = "0" if ks == 0 else vr(dp, 16)
             return [
-                (vr(s, 16), vr(base, 4), ar(128 + 4 * ks, 4), cs, vset(s, 16), vset(base, 4), aset(128 + 4 * ks, 4),
+                (vr(s, 16), ar(base, 4), ar(128 + 4 * ks, 4), cs, vset(s, 16), aset(base, 4), aset(128 + 4 * ks, 4),
                  set() if ks == 0 else vset(s, 16)),
-                (vr(dp, 16), vr(base + 4, 4), ar(160 + 4 * ks, 4), cd, vset(dp, 16), vset(base + 4, 4),
+                (vr(dp, 16), ar(base + 4, 4), ar(160 + 4 * ks, 4), cd, vset(dp, 16), aset(base + 4, 4),
                  aset(160 + 4 * ks, 4), set() if ks == 0 else vset(dp, 16)),
             ]
         u, db = x
         pb = V_PB + 8 * (c & 1) + 4 * u
         dsb = V_DSB + 8 * (c & 1) + 4 * u
         return [
-            (ar(16 * db, 16), vr(base, 4), vr(pb, 4), ar(16 * db, 16), aset(16 * db, 16), vset(base, 4), vset(pb, 4),
+            (ar(16 * db, 16), ar(base, 4), vr(pb, 4), ar(16 * db, 16), aset(16 * db, 16), aset(base, 4), vset(pb, 4),
              aset(16 * db, 16)),
-            (ar(64 + 16 * db, 16), vr(base + 4, 4), vr(dsb, 4), ar(64 + 16 * db, 16), aset(64 + 16 * db, 16),
-             vset(base + 4, 4), vset(dsb, 4), aset(64 + 16 * db, 16)),
+            (ar(64 + 16 * db, 16), ar(base + 4, 4), vr(dsb, 4), ar(64 + 16 * db, 16), aset(64 + 16 * db, 16),
+             aset(base + 4, 4), vset(dsb, 4), aset(64 + 16 * db, 16)),
         ]
 
     # ---- VALU work of E(c), spread over the MFMA slots of stage c ---------------------------
@@ -284,6 +287,21 @@ def run_loop(full, masked):
     entry += [f"v_readfirstlane_b32 {SREG[n]}, %[{n}]" for n in STATE_IO + STATE_IN]
     top = entry + [
         ".Lfa_dkv_loop_%=:",
+        # The last step of the run that ends an item (bit 1 of the flags) copies the next item's first
+        # step: that item's bases (second half of the table) and first q block replace this item's.
+        f"s_add_u32 {t0}, s76, 1",
+        f"s_cmp_lg_u32 {t0}, s82",
+        "s_cbranch_scc1 .Lfa_dkv_same_%=",
+        "s_bitcmp0_b32 s83, 1",
+        "s_cbranch_scc1 .Lfa_dkv_same_%=",
+        f"ds_read_b128 {vr(V_TBL, 4)}, %[tbl] offset:64",
+        f"ds_read_b128 {vr(V_TBL + 4, 4)}, %[tbl] offset:80",
+        f"ds_read_b32 {vr(V_TBL + 8)}, %[tbl] offset:96",
+        "s_waitcnt lgkmcnt(0)",
+    ] + [f"v_readfirstlane_b32 s{68 + i}, {vr(V_TBL + i)}" for i in range(8)] + [
+        f"v_readfirstlane_b32 s80, {vr(V_TBL + 8)}",
+        "s_mov_b32 s78, 0",
+        ".Lfa_dkv_same_%=:",
         # row of the next step relative to the first head of the group: min(g1, gmax) Sq + 128 qb1
         f"s_min_u32 {t0}, s78, s61",
         f"s_mul_i32 {t0}, {t0}, s62",
@@ -311,7 +329,7 @@ def run_loop(full, masked):
         f"global_load_dword {vr(V_QB2)}, {vr(V_QB2)}, s[66:67]",
         f"global_load_dword {vr(V_ROW)}, %[tid4], {S_RA}",
         f"global_load_dword {vr(V_ROW + 1)}, %[tid4], {S_RB}",
-        "s_cmp_eq_u32 s83, 0",
+        "s_bitcmp0_b32 s83, 0",
         "s_cbranch_scc1 .Lfa_dkv_full_%=",
     ]
     tail = [

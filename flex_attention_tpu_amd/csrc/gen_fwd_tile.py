@@ -1,0 +1,385 @@
+#!/usr/bin/env python3
+"""Generator of the hand-scheduled gfx950 instruction streams of the bf16 forward kernel (plain
+score).  Writes fwd_tile.inc: string-literal macros that fwd_bf16.hip places inside `asm volatile`
+statements: the run loop over steps of two 64-row kv tiles, and prologue / epilogue register moves.
+
+A wave owns 2 x 32 q rows (q blocks x = 0, 1): their Q^T fragments and O^T accumulators stay in
+accumulation registers, so every K / V fragment read from LDS feeds two MFMAs.  One step covers
+128 kv rows = four 32-row kv blocks c = 0..3, software-pipelined:
+
+    A(c): S^T = K Q^T for both q blocks      16 MFMAs, operands: 8 ds_read_b128 (rows of K)
+    E(c): online softmax of the 2 x 16 scores of the lane's two q rows (about 140 VALU ops)
+    B(c, x): O^T += V^T P^T of q block x      8 MFMAs, operands: 16 ds_read_b64_tr_b16 (V)
+
+    The two q blocks run half a stage apart: E(c, 0) under A(c+1)[k-steps 0-3] and B(c-1, 1),
+    E(c, 1) under A(c+1)[k-steps 4-7] and B(c, 0).
+
+Softmax bookkeeping per q row, all in the log2 domain (t = score * sm_scale * log2 e):
+    M   reference maximum the probabilities are taken against, p = 2^(t - M);
+    Mt  true running maximum;   L   running sum of p (of the bf16-rounded values the PV product uses).
+M is only raised when a block maximum exceeds it by more than TAU (p then stays below 2^TAU, well
+inside bf16 / fp32 range), which makes the rescaling of the O^T accumulators (alpha = 2^(M_old -
+M_new)) rare: it sits in a block at the start of the next stage that is skipped unless some lane
+of the wave raised M.  The C++ epilogue turns (M, Mt, L) into the exact (m, l) outputs.
+
+Register contract with the C++ side (every asm statement names the accumulation registers with
+physical-register constraints):
+    a[0:63], a[64:127]     O^T accumulators of q block 0, 1 (4 x 16 each)
+    a[128:159], a[160:191] Q^T fragments of q block 0, 1 (8 x 4 each)
+    v[66:245], s[60:100], vcc, m0   scratch of the run loop (clobbered)
+    %[r0..r7]  byte address of the lane's row fragment ks in K half-tile 0 of the current buffer
+    %[t0..t7]  byte address of the lane's transposed fragment (2 db + hi) in K half-tile 0 (the V
+               tiles lie 32 KiB behind the K tiles)
+    %[M0], %[M1], %[Mt0], %[Mt1], %[L0], %[L1]  softmax state of the lane's two q rows (in/out)
+    %[g0], %[g1v], %[g2], %[g3]  the lane's byte offsets inside a global half tile for the wave's 1 KB blocks
+    %[m0] .. %[m3]  (partial steps) keep bits of q block x, kv tile h in m[2 x + h]: bit 16 (c & 1) + e is
+               element e of kv block c (c >> 1 == h); dropped elements get score -inf
+    %[tbl]     LDS byte address of the wave's table of work-group constants (TABLE below)
+    %[lst]     LDS byte address of the item's merged kv tile list (int32 entries)
+    %[it], %[kba1], %[kbb1], %[buf]  loop state (in/out); %[it_end], %[partial]  (in)
+LDS layout of one step buffer (bytes): K tile 0, K tile 1, V tile 0, V tile 1 (16 KiB each); the two
+buffers are 64 KiB apart and the first starts at LDS address 0.
+"""
+import argparse
+import os
+import sys
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+from gfx950_stream import Emitter, ar, aset, vr, vset  # noqa: E402
+
+NSLOT = 8        # staging slots of 8 VGPRs
+PREFETCH = 4     # MFMA pairs between the LDS reads of a pair and its MFMAs
+LOAD_FIRST = 2   # MFMA slot of the first LDS-direct load of the next step
+LOAD_EVERY = 6   # slots between two of them
+TAU = "0x40c00000"  # 6.0: M is raised when a block maximum exceeds it by more than this
+DROP = ()        # instruction classes left out (--drop, timing studies only)
+
+TILE = 16384
+# No scalar operands: constants come from a per-wave table in LDS, loop state from VGPR operands.
+TABLE = ["n_list", "w4k", "c2", "n_steps", "kg_lo", "kg_hi", "vg_lo", "vg_hi", "kban", "kbbn", "kgn_lo", "kgn_hi",
+         "vgn_lo", "vgn_hi", "pad0", "pad1"]
+SREG = {"n_list": "s60", "w4k": "s61", "c2": "s62", "n_steps": "s63", "kg_lo": "s64", "kg_hi": "s65", "vg_lo": "s66",
+        "vg_hi": "s67", "kban": "s68", "kbbn": "s69", "kgn_lo": "s70", "kgn_hi": "s71", "vgn_lo": "s78", "vgn_hi": "s79",
+        "pad0": "s80", "pad1": "s81",
+        "it": "s72", "kba1": "s73", "kbb1": "s74", "buf": "s75", "it_end": "s76", "partial": "s77"}
+STATE_IO = ["it", "kba1", "kbb1", "buf"]
+STATE_IN = ["it_end", "partial"]
+S_T = ["s84", "s85", "s86", "s87"]
+S_GK0, S_GK1, S_GV0, S_GV1 = "s[88:89]", "s[90:91]", "s[92:93]", "s[94:95]"
+S_SEL = ["s82", "s83", "s96", "s97", "s98", "s99"]
+S_LDSN = "s100"
+S_FLAG = ["s80", "s81"]   # "some lane raised M" per q block, from E(c) to the rescale block (reuses the pad slots)
+V_KB2 = 66       # 2 temporaries of the loop tail
+V_MSK = 68       # 4 temporaries of the masked variant
+V_TBL = 72       # 16 scratch VGPRs the table is read into at entry
+V_S0 = 72        # S^T accumulators [c & 1][x] x 16
+V_P0 = 136       # P^T as MFMA B operands [c & 1][x][u] x 4
+V_STG = 168
+V_TMP = 232      # 10 temporaries of the softmax
+V_NEGINF = 242
+V_AL = 244       # alpha of q block 0, 1
+V_END = 245
+A_O, A_Q = 0, 128
+
+
+def v_s(c, x):
+    return V_S0 + 32 * (c & 1) + 16 * x
+
+
+def v_p(c, x, u):
+    return V_P0 + 16 * (c & 1) + 8 * x + 4 * u
+
+
+def build(masked):
+    em = Emitter()
+    # MFMA items (2 MFMAs + one staging slot each), in issue order.  The two q blocks of a kv block
+    # are processed half a stage apart: E(c, 0) runs under A(c+1)[ks 0-3] and B(c-1, 1), E(c, 1) under
+    # A(c+1)[ks 4-7] and B(c, 0), so every softmax has MFMAs of both kinds to hide under.
+    pairs = []
+    first, last = {}, {}   # MFMA slot range of half stage (c, q)
+
+    def add_A(c, lo, hi):
+        for ks in range(lo, hi):
+            pairs.append(("A", c, ks))
+
+    def add_B(c, q):
+        for u in range(2):
+            for j in range(2):
+                pairs.append(("B", c, (q, u, j)))
+
+    add_A(0, 0, 8)
+    for c in range(4):
+        for q in range(2):
+            first[(c, q)] = 2 * len(pairs)
+            if c < 3:
+                add_A(c + 1, 4 * q, 4 * q + 4)
+            if q == 1:
+                add_B(c, 0)
+            elif c > 0:
+                add_B(c - 1, 1)
+            last[(c, q)] = 2 * len(pairs)
+    stage_end = 2 * len(pairs)
+    add_B(3, 1)
+    n_slots = 2 * len(pairs)
+    # the rescale block of (c, q) sits in front of this MFMA slot: all B(c - 1, q) MFMAs are issued,
+    # no B(c, q) MFMA is
+    rescale_at = {}
+    for c in range(4):
+        rescale_at.setdefault(first[(c, 1)], []).append((c, 0))
+        rescale_at.setdefault(first[(c + 1, 0)] if c < 3 else stage_end, []).append((c, 1))
+
+    def half_off(c):
+        return (c >> 1) * TILE + (c & 1) * (TILE // 2)
+
+    def pair_loads(k):
+        kind, c, x = pairs[k]
+        base = V_STG + 8 * (k % NSLOT)
+        if kind == "A":
+            return [(f"ds_read_b128 {vr(base, 4)}, %[r{x}] offset:{half_off(c)}", vset(base, 4))]
+        q, u, j = x
+        off = 2 * TILE + half_off(c) + u * 4096
+        loads = []
+        for i, db in enumerate((2 * j, 2 * j + 1)):
+            for hi in range(2):
+                reg = base + 4 * i + 2 * hi
+                loads.append((f"ds_read_b64_tr_b16 {vr(reg, 2)}, %[t{2 * db + hi}] offset:{off}", vset(reg, 2)))
+        return loads
+
+    def pair_mfmas(k):
+        kind, c, x = pairs[k]
+        base = V_STG + 8 * (k % NSLOT)
+        out = []
+        if kind == "A":
+            ks = x
+            for q in range(2):
+                s = v_s(c, q)
+                cs = "0" if ks == 0 else vr(s, 16)
+                out.append((vr(s, 16), vr(base, 4), ar(A_Q + 32 * q + 4 * ks, 4), cs, vset(s, 16), vset(base, 4),
+                            aset(A_Q + 32 * q + 4 * ks, 4), set() if ks == 0 else vset(s, 16)))
+            return out
+        q, u, j = x
+        p = v_p(c, q, u)
+        for i, db in enumerate((2 * j, 2 * j + 1)):
+            acc = A_O + 64 * q + 16 * db
+            out.append((ar(acc, 16), vr(base + 4 * i, 4), vr(p, 4), ar(acc, 16), aset(acc, 16), vset(base + 4 * i, 4),
+                        vset(p, 4), aset(acc, 16)))
+        return out
+
+    # ---- VALU work of E(c): one list of (kind, ...) per stage ---------------------------------
+    c2 = SREG["c2"]
+    T = [V_TMP + i for i in range(10)]
+
+    def softmax_ops(c, q):
+        """Online softmax of the 16 scores of q block q in kv block c."""
+        s = v_s(c, q)
+        M, Mt, L, AL = f"%[M{q}]", f"%[Mt{q}]", f"%[L{q}]", V_AL + q
+        ops = []
+
+        def valu(text, dst, src, trans=False):
+            ops.append(("valu", text, dst, src, trans))
+
+        if masked:
+            for g in range(4):
+                for u in range(4):
+                    e = 4 * g + u
+                    valu(f"v_bfe_i32 {vr(V_MSK + u)}, %[m{2 * q + (c >> 1)}], {16 * (c & 1) + e}, 1", vset(V_MSK + u), set())
+                for u in range(4):
+                    e = 4 * g + u  # keep ? score : -inf
+                    valu(f"v_bfi_b32 {vr(s + e)}, {vr(V_MSK + u)}, {vr(s + e)}, {vr(V_NEGINF)}", vset(s + e),
+                         vset(s + e) | vset(V_MSK + u) | vset(V_NEGINF))
+        # block maximum of the lane's 16 scores, then across the two half-waves that share the q row
+        for i in range(5):
+            valu(f"v_max3_f32 {vr(T[i])}, {vr(s + 3 * i)}, {vr(s + 3 * i + 1)}, {vr(s + 3 * i + 2)}", vset(T[i]), vset(s + 3 * i, 3))
+        valu(f"v_max3_f32 {vr(T[0])}, {vr(T[0])}, {vr(T[1])}, {vr(T[2])}", vset(T[0]), vset(T[0]) | vset(T[1]) | vset(T[2]))
+        valu(f"v_max3_f32 {vr(T[3])}, {vr(T[3])}, {vr(T[4])}, {vr(s + 15)}", vset(T[3]), vset(T[3]) | vset(T[4]) | vset(s + 15))
+        valu(f"v_max_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[3])}", vset(T[0]), vset(T[0]) | vset(T[3]))
+        valu(f"v_mov_b32_e32 {vr(T[1])}, {vr(T[0])}", vset(T[1]), vset(T[0]))
+        ops.append(("raw", "s_nop 1"))
+        valu(f"v_permlane32_swap_b32 {vr(T[0])}, {vr(T[1])}", vset(T[0]) | vset(T[1]), vset(T[0]) | vset(T[1]))
+        ops.append(("raw", "s_nop 1"))
+        valu(f"v_max_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[1])}", vset(T[0]), vset(T[0]) | vset(T[1]))
+        valu(f"v_mul_f32_e32 {vr(T[0])}, {c2}, {vr(T[0])}", vset(T[0]), vset(T[0]))            # log2 domain (sm_scale > 0)
+        valu(f"v_max_f32_e32 {Mt}, {Mt}, {vr(T[0])}", set(), vset(T[0]))
+        valu(f"v_add_f32_e32 {vr(T[1])}, {TAU}, {M}", vset(T[1]), set())
+        valu(f"v_cmp_gt_f32_e32 vcc, {vr(T[0])}, {vr(T[1])}", set(), vset(T[0]) | vset(T[1]))
+        ops.append(("raw", "s_cmp_lg_u64 vcc, 0"))
+        ops.append(("raw", f"s_cselect_b32 {S_FLAG[q]}, 1, 0"))
+        valu(f"v_cndmask_b32_e32 {vr(T[2])}, {M}, {vr(T[0])}, vcc", vset(T[2]), vset(T[0]))   # M_new
+        valu(f"v_sub_f32_e32 {vr(T[3])}, {M}, {vr(T[2])}", vset(T[3]), vset(T[2]))
+        valu(f"v_exp_f32_e32 {vr(AL)}, {vr(T[3])}", vset(AL), vset(T[3]), True)                # alpha = 2^(M_old - M_new)
+        valu(f"v_mov_b32_e32 {M}, {vr(T[2])}", set(), vset(T[2]))
+        # p = 2^(score c2 - M), packed to bf16 B operands; the row sum adds the rounded values
+        for e in range(16):
+            valu(f"v_fma_f32 {vr(s + e)}, {vr(s + e)}, {c2}, -{M}", vset(s + e), vset(s + e))
+        for e in range(16):
+            valu(f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True)
+        valu(f"v_mov_b32_e32 {vr(T[4])}, 0", vset(T[4]), set())
+        for g in range(4):
+            for h in range(2):
+                e = 4 * g + 2 * h
+                p = v_p(c, q, g >> 1) + 2 * (g & 1) + h
+                valu(f"v_cvt_pk_bf16_f32 {vr(p)}, {vr(s + e)}, {vr(s + e + 1)}", vset(p), vset(s + e, 2))
+        for g in range(4):
+            for h in range(2):
+                p = v_p(c, q, g >> 1) + 2 * (g & 1) + h
+                valu(f"v_dot2c_f32_bf16_e32 {vr(T[4])}, 0x3f803f80, {vr(p)}", vset(T[4]), vset(T[4]) | vset(p))
+        valu(f"v_fma_f32 {L}, {L}, {vr(AL)}, {vr(T[4])}", set(), vset(AL) | vset(T[4]))
+        return ops
+
+    def rescale_ops(c, q):
+        """O^T of q block q times alpha, skipped unless a lane of the wave raised M in E(c)."""
+        ops = [("raw", f"s_cmp_eq_u32 {S_FLAG[q]}, 0"),
+               ("raw", f"s_cbranch_scc1 .Lfa_fwd_{'m' if masked else 'f'}_keep{c}{q}_%=")]
+        AL = V_AL + q
+        for i in range(64):
+            t = T[5 + (i % 4)]
+            a = A_O + 64 * q + i
+            ops.append(("valu", f"v_accvgpr_read_b32 {vr(t)}, {ar(a)}", vset(t), aset(a), False))
+            ops.append(("valu", f"v_mul_f32_e32 {vr(t)}, {vr(t)}, {vr(AL)}", vset(t), vset(t) | vset(AL), False))
+            ops.append(("valu", f"v_accvgpr_write_b32 {ar(a)}, {vr(t)}", aset(a), vset(t), False))
+        ops.append(("raw", f".Lfa_fwd_{'m' if masked else 'f'}_keep{c}{q}_%=:"))
+        return ops
+
+    slot_ops = {m: [] for m in range(n_slots + 1)}
+    slot_lds = {m: [] for m in range(n_slots)}
+    pre_lds = []
+    for c in range(4):
+        for q in range(2):
+            ops = softmax_ops(c, q)
+            lo = first[(c, q)] + (4 if (c, q) == (0, 0) else 0)  # E(0, 0) directly follows A(0): give its results time
+            span = last[(c, q)] - lo
+            for i, op in enumerate(ops):
+                slot_ops[lo + (i * span) // len(ops)].append(op)
+
+    for k in range(len(pairs)):
+        at = 2 * (k - PREFETCH)
+        if at < 0:
+            pre_lds.extend(pair_loads(k))
+        else:
+            slot_lds[at] = pair_loads(k) + slot_lds[at]
+
+    slot_vmem = {m: [] for m in range(n_slots)}
+    k = 0
+    for t, gbase in enumerate((S_GK0, S_GK1, S_GV0, S_GV1)):  # half tiles in LDS order
+        for i in range(4):
+            slot_vmem[LOAD_FIRST + LOAD_EVERY * k].append((t * TILE + i * 1024, "%[g1v]" if i == 1 else f"%[g{i}]", gbase, S_LDSN))
+            k += 1
+
+    def emit(op):
+        if op[0] == "raw":
+            em.raw(op[1])
+        elif "valu" not in DROP:
+            em.valu(*op[1:])
+
+    if masked:
+        em.valu(f"v_mov_b32_e32 {vr(V_NEGINF)}, 0xff800000", vset(V_NEGINF), set())
+    for text, dst in pre_lds:
+        em.lds_read(text, dst)
+    for m in range(n_slots):
+        if m in rescale_at and "valu" not in DROP:
+            for c, q in rescale_at[m]:
+                for op in rescale_ops(c, q):
+                    emit(op)
+        for ld in slot_vmem[m]:
+            if "vmem" not in DROP:
+                em.lds_direct_load(*ld)
+        for text, dst in slot_lds[m]:
+            if "lds" not in DROP:
+                em.lds_read(text, dst)
+        if "mfma" not in DROP:
+            em.mfma(*pair_mfmas(m // 2)[m % 2])
+        for op in slot_ops[m]:
+            emit(op)
+    em.drain()
+    return em
+
+
+def run_loop(full, masked):
+    """One asm statement: a run of consecutive steps [it, it_end) of one work item, all full or a
+    single partial one.  At entry the step's K / V tiles are resident in LDS buffer %[buf]."""
+    t0, t1, t2, t3 = S_T
+    S = SREG
+    entry = [f"ds_read_b128 {vr(V_TBL + 4 * i, 4)}, %[tbl] offset:{16 * i}" for i in range(len(TABLE) // 4)]
+    entry += ["s_waitcnt lgkmcnt(0)"]  # (the streams count LDS operations from zero)
+    entry += [f"v_readfirstlane_b32 {S[n]}, {vr(V_TBL + i)}" for i, n in enumerate(TABLE)]
+    entry += [f"v_readfirstlane_b32 {S[n]}, %[{n}]" for n in STATE_IO + STATE_IN]
+    top = entry + [".Lfa_fwd_loop_%=:"]
+    # on the item's last step the tiles copied "for the next step" are the first step of the next
+    # work item (from the table; with no next item they repeat this one's)
+    ka, kb_, kglo, kghi, vglo, vghi = S_SEL
+    top += [f"s_add_u32 {t0}, {S['it']}, 1", f"s_cmp_eq_u32 {t0}, {S['n_steps']}",
+            f"s_cselect_b32 {ka}, {S['kban']}, {S['kba1']}", f"s_cselect_b32 {kb_}, {S['kbbn']}, {S['kbb1']}",
+            f"s_cselect_b32 {kglo}, {S['kgn_lo']}, {S['kg_lo']}", f"s_cselect_b32 {kghi}, {S['kgn_hi']}, {S['kg_hi']}",
+            f"s_cselect_b32 {vglo}, {S['vgn_lo']}, {S['vg_lo']}", f"s_cselect_b32 {vghi}, {S['vgn_hi']}, {S['vg_hi']}"]
+    for pair, (blo, bhi), kb in ((S_GK0, (kglo, kghi), ka), (S_GK1, (kglo, kghi), kb_), (S_GV0, (vglo, vghi), ka),
+                                 (S_GV1, (vglo, vghi), kb_)):
+        n = int(pair[2:].split(":")[0])
+        top += [f"s_lshl_b32 {t2}, {kb}, 14", f"s_lshr_b32 {t3}, {kb}, 18",  # 64 rows x 256 bytes per kv tile
+                f"s_add_u32 s{n}, {blo}, {t2}", f"s_addc_u32 s{n + 1}, {bhi}, {t3}"]
+    top += [f"s_xor_b32 {t1}, {S['buf']}, 1", f"s_lshl_b32 {t1}, {t1}, 16", f"s_add_u32 {S_LDSN}, {t1}, {S['w4k']}",
+            f"s_cmp_eq_u32 {S['partial']}, 0", "s_cbranch_scc1 .Lfa_fwd_full_%="]
+    tail = [
+        ".Lfa_fwd_tail_%=:",
+        # list entries of the step after the next one, clamped into the list (a second half past its
+        # end repeats the last tile: finite data, its keep bits are zero)
+        f"s_add_u32 {t0}, {S['it']}, 2",
+        f"s_lshl_b32 {t0}, {t0}, 1",
+        f"s_sub_u32 {t1}, {S['n_list']}, 1",
+        f"s_min_u32 {t2}, {t0}, {t1}",
+        f"s_add_u32 {t0}, {t0}, 1",
+        f"s_min_u32 {t3}, {t0}, {t1}",
+        f"s_lshl_b32 {t2}, {t2}, 2",
+        f"s_lshl_b32 {t3}, {t3}, 2",
+        f"v_add_u32_e32 {vr(V_KB2)}, {t2}, %[lst]",
+        f"v_add_u32_e32 {vr(V_KB2 + 1)}, {t3}, %[lst]",
+        f"ds_read_b32 {vr(V_KB2)}, {vr(V_KB2)}",
+        f"ds_read_b32 {vr(V_KB2 + 1)}, {vr(V_KB2 + 1)}",
+        "s_waitcnt vmcnt(0) lgkmcnt(0)",
+        "s_barrier",
+        f"s_add_u32 {S['it']}, {S['it']}, 1",
+        f"v_readfirstlane_b32 {S['kba1']}, {vr(V_KB2)}",
+        f"v_readfirstlane_b32 {S['kbb1']}, {vr(V_KB2 + 1)}",
+        f"s_xor_b32 {S['buf']}, {S['buf']}, 1",
+    ]
+    tail += [f"v_xor_b32_e32 %[r{i}], 0x10000, %[r{i}]" for i in range(8)]
+    tail += [f"v_xor_b32_e32 %[t{i}], 0x10000, %[t{i}]" for i in range(8)]
+    tail += [f"s_cmp_lt_u32 {S['it']}, {S['it_end']}", "s_cbranch_scc1 .Lfa_fwd_loop_%="]
+    tail += [f"v_mov_b32_e32 %[{n}], {S[n]}" for n in STATE_IO]
+    return top + masked.out + ["s_branch .Lfa_fwd_tail_%=", ".Lfa_fwd_full_%=:"] + full.out + tail
+
+
+def main():
+    global DROP
+    here = os.path.dirname(os.path.abspath(__file__))
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("out", nargs="?", default=os.path.join(here, "fwd_tile.inc"))
+    ap.add_argument("--drop", default="", help="comma list of mfma,valu,lds,vmem: leave these instruction classes out "
+                    "(the stream then computes nothing useful; for timing what bounds it)")
+    args = ap.parse_args()
+    if args.drop:
+        DROP = tuple(x for x in args.drop.split(",") if x)
+    with open(args.out, "w") as f:
+        f.write("// Generated by gen_fwd_tile.py; do not edit.\n")
+
+        def macro(name, lines):
+            f.write(f"#define {name} \\\n")
+            f.write(" \\\n".join(f'  "{line}\\n"' for line in lines))
+            f.write("\n\n")
+
+        full, masked = build(False), build(True)
+        macro("FA_FWD_RUN", run_loop(full, masked))
+        for name, em in (("full", full), ("masked", masked)):
+            print(f"{args.out}: {name}: {len(em.out)} instructions, {em.stats}", file=sys.stderr)
+        macro("FA_FWD_ZERO_ACC", [f"v_accvgpr_write_b32 a{A_O + i}, 0" for i in range(128)])
+        # Q^T fragment ks of both q blocks from 8 dword operands (two pinned outputs come first)
+        for ks in range(8):
+            macro(f"FA_FWD_PUT_{ks}",
+                  [f"v_accvgpr_write_b32 a{A_Q + 4 * ks + i}, %{2 + i}" for i in range(4)]
+                  + [f"v_accvgpr_write_b32 a{A_Q + 32 + 4 * ks + i}, %{6 + i}" for i in range(4)])
+        # accumulator tile t (q block t / 4, d block t % 4) into 16 dword operands
+        for t in range(8):
+            macro(f"FA_FWD_GET_ACC_{t}", ["s_nop 15"] + [f"v_accvgpr_read_b32 %{i}, a{A_O + 16 * t + i}" for i in range(16)])
+
+
+if __name__ == "__main__":
+    main()

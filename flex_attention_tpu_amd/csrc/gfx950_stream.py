@@ -6,6 +6,7 @@ hardware leaves to software on gfx950:
     MFMA (8 pass) result -> VALU / LDS / MFMA-A/B use     12 wait states
     VALU result          -> MFMA operand                   2 wait states
     transcendental result-> VALU use                        1 wait state
+    dot (v_dot2c) result -> other VALU use / overwrite      4 wait states (accumulating dots chain freely)
     LDS read result      -> any use                         s_waitcnt lgkmcnt (reads return in order)
 Registers are ("v", n) / ("a", n) pairs; operands supplied by the compiler (%[name]) are never
 written by a stream and need no tracking.
@@ -35,6 +36,7 @@ class Emitter:
         self.mfma_w = {}           # reg -> time of the MFMA that wrote it
         self.valu_w = {}
         self.trans_w = {}
+        self.dot_w = {}
         self.lds_fifo = []         # outstanding LDS reads, oldest first: sets of dst regs
         self.stats = {"nop": 0, "wait": 0, "mfma": 0, "valu": 0, "lds": 0}
 
@@ -85,6 +87,7 @@ class Emitter:
         self.stats["mfma"] += 1
 
     def valu(self, text, dst_regs, src_regs, trans=False):
+        is_dot = text.startswith("v_dot2c")
         self._wait_lds(dst_regs | src_regs)
         for r in dst_regs | src_regs:
             if r in self.mfma_w:
@@ -92,6 +95,9 @@ class Emitter:
         for r in src_regs:
             if r in self.trans_w:
                 self._need_gap(self.trans_w[r], 1)
+        for r in dst_regs | src_regs:
+            if r in self.dot_w and not (is_dot and r in dst_regs):
+                self._need_gap(self.dot_w[r], 4)
         self._raw(text)
         for r in dst_regs:
             self.mfma_w.pop(r, None)
@@ -100,6 +106,10 @@ class Emitter:
                 self.trans_w[r] = self.t - 1
             else:
                 self.trans_w.pop(r, None)
+            if is_dot:
+                self.dot_w[r] = self.t - 1
+            else:
+                self.dot_w.pop(r, None)
         self.stats["valu"] += 1
 
     def lds_read(self, text, dst_regs):

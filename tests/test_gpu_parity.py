@@ -175,6 +175,22 @@ def test_causal_flag_and_segment_ids_arguments(F):
     assert torch.equal(o2, o)
 
 
+def test_forward_stream_kernel_on_request(F, monkeypatch):
+    """FLEXATTN_FWD_STREAM=1 routes plain-score bf16 forward calls to the generated-stream kernel:
+    same results as the oracle, including rows whose tiles are partly or entirely masked."""
+    monkeypatch.setenv("FLEXATTN_FWD_STREAM", "1")
+    for name, shape, mask_pair, score_fn, okw, sc in _small_cases():
+        if score_fn is not None:
+            continue
+        B, Hq, Hkv, Sq, Sk = shape
+        q, k, v, _ = O.make_inputs(B, Hq, Hkv, Sq, Sk, 128, dtype=torch.bfloat16, seed=23)
+        ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, **okw)
+        q, k, v = [x.to(DEV) for x in (q, k, v)]
+        mf, bf = mask_pair if mask_pair else (None, None)
+        o, l, m = _fwd(F, q, k, v, sc, mf, bf, None)
+        assert_close(name + " o", o, ro, torch.bfloat16)
+        assert_close(name + " lse", m + l.log(), rm + rl.log(), torch.bfloat16)
+
 def test_entry_points_reject_bad_arguments_on_gpu(F):
     q = torch.zeros(1, 2, 192, 128, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ValueError):  # 192 is not a multiple of the 128-row q tile
