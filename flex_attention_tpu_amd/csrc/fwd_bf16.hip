@@ -12,21 +12,22 @@
 #include "launch.hpp"
 #include "tile_io.hpp"
 
-// registers of the generated run loop (gen_fwd_tile.py): v[66:245], s[60:100]
-#define FA_FWD_RUN_VGPRS "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", \
-  "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", \
-  "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", \
-  "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", \
-  "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", \
-  "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", \
-  "v146", "v147", "v148", "v149", "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", \
-  "v159", "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167", "v168", "v169", "v170", "v171", \
-  "v172", "v173", "v174", "v175", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", \
-  "v185", "v186", "v187", "v188", "v189", "v190", "v191", "v192", "v193", "v194", "v195", "v196", "v197", \
-  "v198", "v199", "v200", "v201", "v202", "v203", "v204", "v205", "v206", "v207", "v208", "v209", "v210", \
-  "v211", "v212", "v213", "v214", "v215", "v216", "v217", "v218", "v219", "v220", "v221", "v222", "v223", \
-  "v224", "v225", "v226", "v227", "v228", "v229", "v230", "v231", "v232", "v233", "v234", "v235", "v236", \
-  "v237", "v238", "v239", "v240", "v241", "v242", "v243", "v244", "v245"
+// registers of the generated run loop (gen_fwd_tile.py): v[66:199], a[192:255], s[60:100]
+#define FA_FWD_RUN_VGPRS "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79", "v80", \
+  "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", \
+  "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", \
+  "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", \
+  "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", \
+  "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", \
+  "v149", "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", \
+  "v162", "v163", "v164", "v165", "v166", "v167", "v168", "v169", "v170", "v171", "v172", "v173", "v174", \
+  "v175", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", "v185", "v186", "v187", \
+  "v188", "v189", "v190", "v191", "v192", "v193", "v194", "v195", "v196", "v197", "v198", "v199", "a192", \
+  "a193", "a194", "a195", "a196", "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205", \
+  "a206", "a207", "a208", "a209", "a210", "a211", "a212", "a213", "a214", "a215", "a216", "a217", "a218", \
+  "a219", "a220", "a221", "a222", "a223", "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231", \
+  "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239", "a240", "a241", "a242", "a243", "a244", \
+  "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255"
 #define FA_FWD_RUN_SGPRS "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", \
   "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", \
   "s87", "s88", "s89", "s90", "s91", "s92", "s93", "s94", "s95", "s96", "s97", "s98", "s99", "s100"
@@ -390,13 +391,23 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
     ta[i] = base0 + (unsigned)(tile_off(t_row + 8 * (i & 1), 4 * (i >> 1) + t_chunk) + t_half) * 2u;
   int buf = 0;
 
+  bool resident = false;  // the item's first step was already copied into buffer `buf` by the previous item's last step
+
+  // (opaque(): addresses derived from its result are computed where they are used instead of once
+  // before the item loop, where they would have to be kept through every run)
+  auto opaque = [](int x) {
+    asm volatile("" : "+v"(x));
+    return x;
+  };
   // Everything an item needs from global memory before its first step, fetched while the previous
-  // item runs (plain loads whose values are not touched until then).
+  // item runs (plain loads whose values are not touched until that item's last run).
   constexpr int kListRegs = MAX_LIST / 256;
+  static_assert(kListRegs <= 4, "the packed state words hold four tiles per lane");
   struct ItemRegs {
-    u32x4 qw[2][8];                 // Q^T fragments of the lane's two q rows
+    u32x4 qw[2][8];     // Q^T fragments of the lane's two q rows
     int doc[2];
-    unsigned char sa[kListRegs], sb[kListRegs];  // states of kv tile tid + 256 j in the two state rows
+    unsigned sa, sb;    // byte j: state of kv tile tid + 256 j in the state row of q tile 0 / 1
+    unsigned head;      // states of kv tile `lane` in both rows: where the merged list starts
   };
   const int n_items = n_wg / (int)gridDim.x;
   auto geometry = [&](int item, int& bh, int& qb2) {
@@ -407,26 +418,65 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
   auto fetch = [&](int item, ItemRegs& r) {
     int bh, qb2;
     geometry(item, bh, qb2);
+    const int tid_here = opaque(tid);
+    const int lane_here = tid_here & 63;
+    const int row_here = (tid_here >> 6) * 32 + (lane_here & 31);
+    r.sa = r.sb = r.head = 0u;
 #pragma unroll
     for (int x = 0; x < 2; ++x) {
       const int qb = min(2 * qb2 + x, nQ - 1);  // (a missing second tile repeats the first; nothing of it is stored)
-      const bf16_t* Qg = static_cast<const bf16_t*>(a.q) + ((size_t)bh * a.Sq + (size_t)qb * BM + q_local) * D;
+      const bf16_t* Qg = static_cast<const bf16_t*>(a.q) + ((size_t)bh * a.Sq + (size_t)qb * BM + row_here) * D;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) r.qw[x][ks] = *reinterpret_cast<const u32x4*>(Qg + ks * 16 + hh * 8);
-      r.doc[x] = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[qb * BM + q_local] : 0;
+      for (int ks = 0; ks < 8; ++ks) r.qw[x][ks] = *reinterpret_cast<const u32x4*>(Qg + ks * 16 + (lane_here >> 5) * 8);
+      r.doc[x] = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[qb * BM + row_here] : 0;
       const uint8_t* row = a.map.state + (size_t)qb * nK;
       const bool valid = 2 * qb2 + x < nQ;
+      unsigned packed = 0u;
 #pragma unroll
       for (int j = 0; j < kListRegs; ++j) {
-        const int t = tid + 256 * j;
-        const unsigned char v = (valid && t < nK) ? row[t] : 0;
-        if (x == 0) r.sa[j] = v; else r.sb[j] = v;
+        const int t = tid_here + 256 * j;
+        const unsigned v = (valid && t < nK) ? row[t] : 0u;
+        packed |= v << (8 * j);
       }
+      if (x == 0) r.sa = packed; else r.sb = packed;
+      const unsigned hv = (valid && lane_here < nK) ? row[lane_here] : 0u;
+      r.head |= hv << (8 * x);
     }
+  };
+  // What is left of an item's fetched values once its Q^T fragments sit in their registers.
+  struct ItemHead {
+    int doc[2];
+    unsigned sa, sb;
+  };
+  FwdPinned st;
+  // Q goes in multiplied by sm_scale * log2(e): the streams' scores are then in the log2 domain
+  const float c2 = a.sm_scale * kLog2e;
+  auto scaled = [c2](unsigned two) {
+    const float lo = __builtin_bit_cast(float, two << 16) * c2;
+    const float hi = __builtin_bit_cast(float, two & 0xffff0000u) * c2;
+    return __builtin_bit_cast(unsigned, pack_bf16(lo, hi));
+  };
+  auto consume = [&](const ItemRegs& r, ItemHead& c) {
+#define FA_PUT(KS, Q0, Q1)                                                                                        \
+  asm volatile(FA_FWD_PUT_##KS                                                                                    \
+               : "={" Q0 "}"(st.q[KS]), "={" Q1 "}"(st.q[8 + KS])                                                 \
+               : "v"(scaled(r.qw[0][KS][0])), "v"(scaled(r.qw[0][KS][1])), "v"(scaled(r.qw[0][KS][2])),           \
+                 "v"(scaled(r.qw[0][KS][3])), "v"(scaled(r.qw[1][KS][0])), "v"(scaled(r.qw[1][KS][1])),           \
+                 "v"(scaled(r.qw[1][KS][2])), "v"(scaled(r.qw[1][KS][3])));
+    FA_PUT(0, "a[128:131]", "a[160:163]") FA_PUT(1, "a[132:135]", "a[164:167]") FA_PUT(2, "a[136:139]", "a[168:171]")
+    FA_PUT(3, "a[140:143]", "a[172:175]") FA_PUT(4, "a[144:147]", "a[176:179]") FA_PUT(5, "a[148:151]", "a[180:183]")
+    FA_PUT(6, "a[152:155]", "a[184:187]") FA_PUT(7, "a[156:159]", "a[188:191]")
+#undef FA_PUT
+    c.doc[0] = r.doc[0];
+    c.doc[1] = r.doc[1];
+    c.sa = r.sa;
+    c.sb = r.sb;
   };
 
   ItemRegs pre;
+  ItemHead cur;
   fetch(0, pre);
+  consume(pre, cur);
   for (int item = 0; item < n_items; ++item) {
     int bh, qb2;
     geometry(item, bh, qb2);
@@ -435,24 +485,25 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
     const int hk = h / (a.Hq / a.Hkv);
     const bf16_t* Kg = static_cast<const bf16_t*>(a.k) + ((size_t)(b * a.Hkv + hk) * a.Sk) * D;
     const bf16_t* Vg = static_cast<const bf16_t*>(a.v) + ((size_t)(b * a.Hkv + hk) * a.Sk) * D;
-    if (item > 0) __syncthreads();  // the previous item's LDS contents are dead from here
+    if (item > 0) __syncthreads();  // the previous item's list and state rows are dead from here
 
     // the two state rows into LDS, then the merged list of kv tiles that are non-empty for either
     // q tile, in ascending order (ballot compaction per wave, wave offsets through LDS)
+    const int tid_p = opaque(tid);  // (fresh per item: see opaque())
 #pragma unroll
     for (int j = 0; j < kListRegs; ++j) {
-      const int t = tid + 256 * j;
+      const int t = tid_p + 256 * j;
       if (t < nK) {
-        sStA[t] = pre.sa[j];
-        sStB[t] = pre.sb[j];
+        sStA[t] = (unsigned char)((cur.sa >> (8 * j)) & 0xffu);
+        sStB[t] = (unsigned char)((cur.sb >> (8 * j)) & 0xffu);
       }
     }
     int n_list = 0;
 #pragma unroll
     for (int j = 0; j < kListRegs; ++j) {
       if (256 * j < nK) {
-        const int t = tid + 256 * j;
-        const bool present = t < nK && (pre.sa[j] | pre.sb[j]) != 0;
+        const int t = tid_p + 256 * j;
+        const bool present = t < nK && (((cur.sa | cur.sb) >> (8 * j)) & 0xffu) != 0u;
         const unsigned long long mask = __ballot(present);
         if (lane == 0) sCnt[w] = __builtin_popcountll(mask);
         __syncthreads();
@@ -469,27 +520,17 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
     n_list = __builtin_amdgcn_readfirstlane(n_list);
     const int n_steps = (n_list + 1) >> 1;
 
-    FwdPinned st;
     asm volatile(FA_FWD_ZERO_ACC
                  : "={a[0:15]}"(st.o[0]), "={a[16:31]}"(st.o[1]), "={a[32:47]}"(st.o[2]), "={a[48:63]}"(st.o[3]),
                    "={a[64:79]}"(st.o[4]), "={a[80:95]}"(st.o[5]), "={a[96:111]}"(st.o[6]), "={a[112:127]}"(st.o[7]));
-#define FA_PUT(KS, Q0, Q1)                                                                                        \
-  asm volatile(FA_FWD_PUT_##KS                                                                                    \
-               : "={" Q0 "}"(st.q[KS]), "={" Q1 "}"(st.q[8 + KS])                                                 \
-               : "v"(pre.qw[0][KS][0]), "v"(pre.qw[0][KS][1]), "v"(pre.qw[0][KS][2]), "v"(pre.qw[0][KS][3]),      \
-                 "v"(pre.qw[1][KS][0]), "v"(pre.qw[1][KS][1]), "v"(pre.qw[1][KS][2]), "v"(pre.qw[1][KS][3]));
-    FA_PUT(0, "a[128:131]", "a[160:163]") FA_PUT(1, "a[132:135]", "a[164:167]") FA_PUT(2, "a[136:139]", "a[168:171]")
-    FA_PUT(3, "a[140:143]", "a[172:175]") FA_PUT(4, "a[144:147]", "a[176:179]") FA_PUT(5, "a[148:151]", "a[180:183]")
-    FA_PUT(6, "a[152:155]", "a[184:187]") FA_PUT(7, "a[156:159]", "a[188:191]")
-#undef FA_PUT
-    const int doc_i[2] = {pre.doc[0], pre.doc[1]};
+    const int doc_i[2] = {cur.doc[0], cur.doc[1]};
     const int q_idx[2] = {(2 * qb2) * BM + q_local, (2 * qb2 + 1) * BM + q_local};
-    // softmax state of the lane's two q rows (log2 domain): reference maximum (finite start value:
-    // -inf would turn 2^(score - M) of a masked score into NaN), true maximum, sum
-    float M[2] = {-1.0e30f, -1.0e30f}, Mt[2] = {kNegInf, kNegInf}, L[2] = {0.f, 0.f};
+    // softmax state of the lane's two q rows (log2 domain): reference maximum M, running maximum
+    // relative to it, sum of 2^(score - M)
+    float M[2] = {0.f, 0.f}, Mt[2] = {kNegInf, kNegInf}, L[2] = {0.f, 0.f};
 
     auto entry = [&](int e) { return sList[e < n_list ? e : n_list - 1]; };
-    if (n_list > 0) {
+    if (n_list > 0 && !resident) {
       // first step into the current buffer (a missing second entry repeats the first: finite data, masked out)
       const int ka = __builtin_amdgcn_readfirstlane(entry(0));
       const int kbb = __builtin_amdgcn_readfirstlane(entry(1));
@@ -498,17 +539,45 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
       loader.load(Kg + (size_t)kbb * BN * D, dst + kTileElems);
       loader.load(Vg + (size_t)ka * BN * D, dst + 2 * kTileElems);
       loader.load(Vg + (size_t)kbb * BN * D, dst + 3 * kTileElems);
+      wait_vmem_all();
     }
+    resident = false;
     unsigned* tbl = sTbl + w * 16;
     const unsigned tbl_addr = (unsigned)(size_t)tbl;
     const unsigned lst_addr = (unsigned)(size_t)sList;
-    wait_vmem_all();
     __syncthreads();
-    if (item + 1 < n_items) fetch(item + 1, pre);  // lands while this item's first step runs
+    // The next item's data lands while this item runs.  (The last item fetches itself again: every
+    // path then redefines the fetched registers, and the compiler need not merge old values in.)
+    const bool has_next = item + 1 < n_items;
+    int bh_n = bh, qb2_n = qb2;
+    if (has_next) geometry(item + 1, bh_n, qb2_n);
+    fetch(has_next ? item + 1 : item, pre);
 
     int it = 0;
     int kba1 = (n_list > 0) ? __builtin_amdgcn_readfirstlane(entry(2)) : 0;
     int kbb1 = (n_list > 0) ? __builtin_amdgcn_readfirstlane(entry(3)) : 0;
+    // Work-group constants of the run loop, one table per wave (order: TABLE in gen_fwd_tile.py),
+    // written and read by the same wave.  The "next item" entries start out as this item's own first
+    // step; the run that ends the item overwrites them when the next item's list head is known.
+    if (lane == 0 && n_list > 0) {
+      const int ka = entry(0), kbb = entry(1);
+      tbl[0] = (unsigned)n_list;
+      tbl[1] = base0 + (unsigned)w * 4096u;  // LDS address of the wave's first 1 KB block in buffer 0
+      tbl[2] = __builtin_bit_cast(unsigned, c2);
+      tbl[3] = (unsigned)n_steps;
+      tbl[4] = (unsigned)(size_t)Kg;
+      tbl[5] = (unsigned)((size_t)Kg >> 32);
+      tbl[6] = (unsigned)(size_t)Vg;
+      tbl[7] = (unsigned)((size_t)Vg >> 32);
+      tbl[8] = (unsigned)ka;
+      tbl[9] = (unsigned)kbb;
+      tbl[10] = (unsigned)(size_t)Kg;
+      tbl[11] = (unsigned)((size_t)Kg >> 32);
+      tbl[12] = (unsigned)(size_t)Vg;
+      tbl[13] = (unsigned)((size_t)Vg >> 32);
+      tbl[14] = 0u;
+      tbl[15] = 0u;
+    }
     // a step is full when both of its entries exist and are full for both q tiles
     auto entry_full = [&](int e) {
       const int k = sList[e];
@@ -567,27 +636,28 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
       }
       it_end = __builtin_amdgcn_readfirstlane(it_end);
       const int partial_flag = partial ? 1 : 0;
-      // work-group constants of the run loop, one table per wave (order: TABLE in gen_fwd_tile.py),
-      // written and read by the same wave; "next item" entries repeat this item's (its first step is
-      // loaded by its own prologue)
-      if (lane == 0) {
-        const int ka = entry(0), kbb = entry(1);
-        tbl[0] = (unsigned)n_list;
-        tbl[1] = base0 + (unsigned)w * 4096u;  // LDS address of the wave's first 1 KB block in buffer 0
-        tbl[2] = __builtin_bit_cast(unsigned, a.sm_scale * kLog2e);
-        tbl[3] = (unsigned)n_steps;
-        tbl[4] = (unsigned)(size_t)Kg;
-        tbl[5] = (unsigned)((size_t)Kg >> 32);
-        tbl[6] = (unsigned)(size_t)Vg;
-        tbl[7] = (unsigned)((size_t)Vg >> 32);
-        tbl[8] = (unsigned)ka;
-        tbl[9] = (unsigned)kbb;
-        tbl[10] = (unsigned)(size_t)Kg;
-        tbl[11] = (unsigned)((size_t)Kg >> 32);
-        tbl[12] = (unsigned)(size_t)Vg;
-        tbl[13] = (unsigned)((size_t)Vg >> 32);
-        tbl[14] = 0u;
-        tbl[15] = 0u;
+      if (it_end == n_steps && has_next) {
+        // The run ends the item: its last step copies the next item's first step, if that item's
+        // list starts within kv tiles 0..63 (every wave fetched those states).  The fetched values
+        // are first touched here, an item's length after their loads were issued.
+        const unsigned long long mask = __ballot(lane < nK && pre.head != 0u);
+        const int cnt = __builtin_popcountll(mask);
+        if (cnt >= 2 || (cnt == 1 && nK <= 64)) {
+          const int ka_n = __builtin_ctzll(mask);
+          const int kb_n = cnt >= 2 ? __builtin_ctzll(mask & (mask - 1ull)) : ka_n;
+          const int b_n = bh_n / a.Hq, hk_n = (bh_n % a.Hq) / (a.Hq / a.Hkv);
+          const bf16_t* Kg_n = static_cast<const bf16_t*>(a.k) + ((size_t)(b_n * a.Hkv + hk_n) * a.Sk) * D;
+          const bf16_t* Vg_n = static_cast<const bf16_t*>(a.v) + ((size_t)(b_n * a.Hkv + hk_n) * a.Sk) * D;
+          if (lane == 0) {
+            tbl[8] = (unsigned)ka_n;
+            tbl[9] = (unsigned)kb_n;
+            tbl[10] = (unsigned)(size_t)Kg_n;
+            tbl[11] = (unsigned)((size_t)Kg_n >> 32);
+            tbl[12] = (unsigned)(size_t)Vg_n;
+            tbl[13] = (unsigned)((size_t)Vg_n >> 32);
+          }
+          resident = true;
+        }
       }
       // no scalar operands (see gen_fwd_tile.py): the loop state travels in VGPRs
       asm volatile(FA_FWD_RUN
@@ -605,8 +675,33 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
       buf = __builtin_amdgcn_readfirstlane(buf);
     }
 
-    // ---- epilogue: O = O^T / l, exact (l, m) from the reference-maximum bookkeeping ----
-#define FA_GET(T, SRC, REG, DST)                                                                                   \
+    // ---- item epilogue ----
+    // The next item's Q^T fragments go into their registers before this item's stores are issued
+    // (their loads are long done; behind the stores the wait would include the stores).
+    consume(pre, cur);
+
+    // O = O^T / l as bf16 rows, staged through the wave's 16 KB of the free LDS step buffer (16-byte
+    // chunks XOR-swizzled by row) so that every store instruction writes four complete 256-byte rows;
+    // exact (l, m) from the reference-maximum bookkeeping.  (Buffer `buf` may hold the next item's
+    // first step: the other one is free.)
+    {
+      char* stage = reinterpret_cast<char*>(sT + (size_t)(buf ^ 1) * 4 * kTileElems) + w * 16384;
+      const int lane_here = opaque(lane);
+      const int row_here = lane_here & 31;
+      const unsigned wr = (unsigned)row_here * 256u + 8u * (unsigned)(lane_here >> 5);
+      float inv[2];
+#pragma unroll
+      for (int x = 0; x < 2; ++x) {
+        const float l_tot = half_sum(L[x]);
+        inv[x] = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
+        if (2 * qb2 + x < nQ && a.l != nullptr && lane_here < 32) {
+          const size_t r = (size_t)bh * a.Sq + q_idx[x];
+          // sums were taken against the reference maximum M: move them to the true maximum M + Mt
+          a.l[r] = (l_tot > 0.f) ? l_tot * fast_exp2(-Mt[x]) : 0.f;
+          a.m[r] = (l_tot > 0.f) ? (M[x] + Mt[x]) * kLn2 : kNegInf;  // natural units
+        }
+      }
+#define FA_GET(T, SRC, REG)                                                                                        \
   {                                                                                                                \
     float xv[16];                                                                                                  \
     asm volatile(FA_FWD_GET_ACC_##T                                                                                \
@@ -614,36 +709,33 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
                    "=v"(xv[7]), "=v"(xv[8]), "=v"(xv[9]), "=v"(xv[10]), "=v"(xv[11]), "=v"(xv[12]), "=v"(xv[13]),  \
                    "=v"(xv[14]), "=v"(xv[15])                                                                      \
                  : "{" REG "}"(SRC));                                                                              \
-    _Pragma("unroll") for (int e = 0; e < 16; ++e) DST[e] = xv[e];                                                 \
+    const float sc_ = inv[T / 4];                                                                                  \
+    _Pragma("unroll") for (int g = 0; g < 4; ++g) {                                                                \
+      const bf16x2 lo = pack_bf16(xv[4 * g] * sc_, xv[4 * g + 1] * sc_);                                           \
+      const bf16x2 hi = pack_bf16(xv[4 * g + 2] * sc_, xv[4 * g + 3] * sc_);                                       \
+      const bf16x4 out = {lo[0], lo[1], hi[0], hi[1]};                                                             \
+      *reinterpret_cast<bf16x4*>(stage + (T / 4) * 8192 + wr +                                                     \
+                                 (unsigned)(((4 * (T % 4) + g) ^ (row_here & 15)) << 4)) = out;                    \
+    }                                                                                                              \
   }
-    f32x16 o_acc[8];
-    FA_GET(0, st.o[0], "a[0:15]", o_acc[0]) FA_GET(1, st.o[1], "a[16:31]", o_acc[1])
-    FA_GET(2, st.o[2], "a[32:47]", o_acc[2]) FA_GET(3, st.o[3], "a[48:63]", o_acc[3])
-    FA_GET(4, st.o[4], "a[64:79]", o_acc[4]) FA_GET(5, st.o[5], "a[80:95]", o_acc[5])
-    FA_GET(6, st.o[6], "a[96:111]", o_acc[6]) FA_GET(7, st.o[7], "a[112:127]", o_acc[7])
+      FA_GET(0, st.o[0], "a[0:15]") FA_GET(1, st.o[1], "a[16:31]") FA_GET(2, st.o[2], "a[32:47]")
+      FA_GET(3, st.o[3], "a[48:63]") FA_GET(4, st.o[4], "a[64:79]") FA_GET(5, st.o[5], "a[80:95]")
+      FA_GET(6, st.o[6], "a[96:111]") FA_GET(7, st.o[7], "a[112:127]")
 #undef FA_GET
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      const int chunk = lane_here & 15;
 #pragma unroll
-    for (int x = 0; x < 2; ++x) {
-      const float l_tot = half_sum(L[x]);
-      if (2 * qb2 + x < nQ) {
-        const float inv = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
-        bf16_t* Og = static_cast<bf16_t*>(a.o) + ((size_t)bh * a.Sq + (size_t)(2 * qb2 + x) * BM) * D;
+      for (int x = 0; x < 2; ++x) {
+        if (2 * qb2 + x < nQ) {
+          bf16_t* Og = static_cast<bf16_t*>(a.o) + ((size_t)bh * a.Sq + (size_t)(2 * qb2 + x) * BM + w * 32) * D;
 #pragma unroll
-        for (int db = 0; db < 4; ++db) {
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const f32x16& oa = o_acc[4 * x + db];
-            bf16x2 lo = pack_bf16(oa[4 * g] * inv, oa[4 * g + 1] * inv);
-            bf16x2 hi = pack_bf16(oa[4 * g + 2] * inv, oa[4 * g + 3] * inv);
-            bf16x4 out = {lo[0], lo[1], hi[0], hi[1]};
-            *reinterpret_cast<bf16x4*>(Og + (size_t)q_local * D + 32 * db + 8 * g + 4 * hh) = out;
+          for (int i = 0; i < 8; ++i) {
+            const int r = 4 * i + (lane_here >> 4);
+            const u32x4 v = *reinterpret_cast<const u32x4*>(stage + x * 8192 + (unsigned)r * 256u +
+                                                            (unsigned)((chunk ^ (r & 15)) << 4));
+            *reinterpret_cast<u32x4*>(Og + (size_t)r * D + chunk * 8) = v;
           }
-        }
-        if (a.l != nullptr && hh == 0) {
-          const size_t r = (size_t)bh * a.Sq + q_idx[x];
-          // sums were taken against the reference maximum M: move them to the true maximum Mt
-          a.l[r] = (l_tot > 0.f) ? l_tot * fast_exp2(M[x] - Mt[x]) : 0.f;
-          a.m[r] = Mt[x] * kLn2;  // natural units
         }
       }
     }
@@ -663,19 +755,18 @@ static int launch_fwd_plain(const FwdArgs& a, hipStream_t stream) {
   return check_launch("flexattn_fwd bf16");
 }
 
-static bool fwd_stream_requested() {
+// FLEXATTN_FWD_STREAM=0 sends plain-score calls to the compiled kernel too (for comparisons).
+static bool fwd_stream_enabled() {
   const char* v = std::getenv("FLEXATTN_FWD_STREAM");
-  return v != nullptr && v[0] == '1';
+  return v == nullptr || v[0] != '0';
 }
 
 int fwd_bf16_d128(const FwdArgs& a, hipStream_t stream) {
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
-      // The generated-stream kernel (one wave per SIMD, 64 q rows per wave) is correct but its
-      // stream is bound by the VALU work of the online softmax and is slower than the compiled
-      // kernel (two waves per SIMD); it runs only on request, FLEXATTN_FWD_STREAM=1, for plain
-      // scores whose state rows and merged kv list fit in LDS, and needs sm_scale > 0.
-      return (fwd_stream_requested() && a.map.nk <= fwd_cfg::MAX_LIST && a.sm_scale > 0.f)
+      // The generated-stream kernel (one wave per SIMD, 64 q rows per wave) keeps the state rows and the
+      // merged kv list in LDS and folds sm_scale into Q, hence the two conditions.
+      return (fwd_stream_enabled() && a.map.nk <= fwd_cfg::MAX_LIST && a.sm_scale > 0.f)
                  ? launch_fwd_plain(a, stream)
                  : launch_fwd<FLEXATTN_SCORE_NONE>(a, stream);
     case FLEXATTN_SCORE_ALIBI: return launch_fwd<FLEXATTN_SCORE_ALIBI>(a, stream);

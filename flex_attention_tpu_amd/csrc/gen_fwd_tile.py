@@ -7,30 +7,38 @@ A wave owns 2 x 32 q rows (q blocks x = 0, 1): their Q^T fragments and O^T accum
 accumulation registers, so every K / V fragment read from LDS feeds two MFMAs.  One step covers
 128 kv rows = four 32-row kv blocks c = 0..3, software-pipelined:
 
-    A(c): S^T = K Q^T for both q blocks      16 MFMAs, operands: 8 ds_read_b128 (rows of K)
-    E(c): online softmax of the 2 x 16 scores of the lane's two q rows (about 140 VALU ops)
-    B(c, x): O^T += V^T P^T of q block x      8 MFMAs, operands: 16 ds_read_b64_tr_b16 (V)
+    A(c): S'^T = K Q^T - M for both q blocks   16 MFMAs, operands: 8 ds_read_b128 (rows of K)
+    E(c, x): online softmax of the lane's 16 scores of q block x (45 VALU ops)
+    B(c, x): O^T += V^T P^T of q block x       8 MFMAs, operands: 16 ds_read_b64_tr_b16 (V)
 
     The two q blocks run half a stage apart: E(c, 0) under A(c+1)[k-steps 0-3] and B(c-1, 1),
     E(c, 1) under A(c+1)[k-steps 4-7] and B(c, 0).
 
-Softmax bookkeeping per q row, all in the log2 domain (t = score * sm_scale * log2 e):
-    M   reference maximum the probabilities are taken against, p = 2^(t - M);
-    Mt  true running maximum;   L   running sum of p (of the bf16-rounded values the PV product uses).
-M is only raised when a block maximum exceeds it by more than TAU (p then stays below 2^TAU, well
-inside bf16 / fp32 range), which makes the rescaling of the O^T accumulators (alpha = 2^(M_old -
-M_new)) rare: it sits in a block at the start of the next stage that is skipped unless some lane
-of the wave raised M.  The C++ epilogue turns (M, Mt, L) into the exact (m, l) outputs.
+The softmax is arranged so that the common case costs no arithmetic beyond exp, pack and sum:
+  * Q arrives pre-multiplied by sm_scale * log2(e), so the MFMA result is already in the log2 domain;
+  * the reference maximum M the probabilities are taken against, p = 2^(t - M), enters through the
+    accumulator input of the first MFMA of each chain (16 registers per q block hold -M), so the
+    chain's result is t - M and p is a bare v_exp_f32;
+  * M only moves when the running maximum relative to it, Mt = max(t - M), leaves [-TAU, TAU] (p then
+    stays inside 2^+-TAU: safe for bf16 and fp32).  The move is a skipped-unless-needed block right
+    behind the test: O^T, L, the block's scores and the -M registers are corrected by the lane's
+    shift, and the chain of the next kv block, already in flight with the old -M, is corrected by a
+    second such block at the start of its own softmax;
+  * the row sum L adds the fp32 values of p.
+State per q row: M, Mt (true maximum = M + Mt), L.  The C++ epilogue turns them into the exact
+(m, l) outputs.
 
 Register contract with the C++ side (every asm statement names the accumulation registers with
 physical-register constraints):
     a[0:63], a[64:127]     O^T accumulators of q block 0, 1 (4 x 16 each)
-    a[128:159], a[160:191] Q^T fragments of q block 0, 1 (8 x 4 each)
-    v[66:245], s[60:100], vcc, m0   scratch of the run loop (clobbered)
+    a[128:159], a[160:191] Q^T fragments of q block 0, 1 (8 x 4 each), pre-scaled
+    a[192:255]             staging slots of the LDS fragments (clobbered)
+    v[66:199], s[60:100], vcc, m0   scratch of the run loop (clobbered)
     %[r0..r7]  byte address of the lane's row fragment ks in K half-tile 0 of the current buffer
     %[t0..t7]  byte address of the lane's transposed fragment (2 db + hi) in K half-tile 0 (the V
                tiles lie 32 KiB behind the K tiles)
-    %[M0], %[M1], %[Mt0], %[Mt1], %[L0], %[L1]  softmax state of the lane's two q rows (in/out)
+    %[M0], %[M1], %[Mt0], %[Mt1], %[L0], %[L1]  softmax state of the lane's two q rows (in/out);
+               start values 0, -inf, 0
     %[g0], %[g1v], %[g2], %[g3]  the lane's byte offsets inside a global half tile for the wave's 1 KB blocks
     %[m0] .. %[m3]  (partial steps) keep bits of q block x, kv tile h in m[2 x + h]: bit 16 (c & 1) + e is
                element e of kv block c (c >> 1 == h); dropped elements get score -inf
@@ -47,11 +55,11 @@ import sys
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 from gfx950_stream import Emitter, ar, aset, vr, vset  # noqa: E402
 
-NSLOT = 8        # staging slots of 8 VGPRs
+NSLOT = 8        # staging slots of 8 registers
 PREFETCH = 4     # MFMA pairs between the LDS reads of a pair and its MFMAs
-LOAD_FIRST = 2   # MFMA slot of the first LDS-direct load of the next step
-LOAD_EVERY = 6   # slots between two of them
-TAU = "0x40c00000"  # 6.0: M is raised when a block maximum exceeds it by more than this
+LOAD_FIRST = 0   # MFMA slot of the first LDS-direct load of the next step
+LOAD_EVERY = 3   # slots between two of them
+TAU = "0x40c00000"  # 6.0: M moves when the running maximum relative to it leaves [-6, 6]
 DROP = ()        # instruction classes left out (--drop, timing studies only)
 
 TILE = 16384
@@ -64,22 +72,24 @@ SREG = {"n_list": "s60", "w4k": "s61", "c2": "s62", "n_steps": "s63", "kg_lo": "
         "it": "s72", "kba1": "s73", "kbb1": "s74", "buf": "s75", "it_end": "s76", "partial": "s77"}
 STATE_IO = ["it", "kba1", "kbb1", "buf"]
 STATE_IN = ["it_end", "partial"]
-S_T = ["s84", "s85", "s86", "s87"]
+S_T = ["s84", "s85", "s86", "s87"]   # temporaries of the loop top / tail; s[86:87] also inside the masked stream
 S_GK0, S_GK1, S_GV0, S_GV1 = "s[88:89]", "s[90:91]", "s[92:93]", "s[94:95]"
 S_SEL = ["s82", "s83", "s96", "s97", "s98", "s99"]
 S_LDSN = "s100"
-S_FLAG = ["s80", "s81"]   # "some lane raised M" per q block, from E(c) to the rescale block (reuses the pad slots)
+S_PEND = ["s80", "s81"]   # per q block: the chain in flight still carries the old -M (reuses the pad slots)
 V_KB2 = 66       # 2 temporaries of the loop tail
 V_MSK = 68       # 4 temporaries of the masked variant
 V_TBL = 72       # 16 scratch VGPRs the table is read into at entry
 V_S0 = 72        # S^T accumulators [c & 1][x] x 16
-V_P0 = 136       # P^T as MFMA B operands [c & 1][x][u] x 4
-V_STG = 168
-V_TMP = 232      # 10 temporaries of the softmax
-V_NEGINF = 242
-V_AL = 244       # alpha of q block 0, 1
-V_END = 245
-A_O, A_Q = 0, 128
+V_P0 = 136       # P^T as MFMA B operands [x][u] x 4 (B(c, x) has issued before E(c + 1, x) writes again)
+V_NEGM = 152     # -M of q block 0, 1, 16 copies each: accumulator input of a chain's first MFMA
+V_TMP = 184      # 10 temporaries of the softmax
+V_NEGINF = 194
+V_TAU = 195
+V_D = 196        # shift of M of q block 0, 1 (0 in lanes that keep theirs)
+V_AL = 198       # 2^-shift of q block 0, 1
+V_END = 199
+A_O, A_Q, A_STG = 0, 128, 192
 
 
 def v_s(c, x):
@@ -87,7 +97,7 @@ def v_s(c, x):
 
 
 def v_p(c, x, u):
-    return V_P0 + 16 * (c & 1) + 8 * x + 4 * u
+    return V_P0 + 8 * x + 4 * u
 
 
 def build(masked):
@@ -121,63 +131,72 @@ def build(masked):
     stage_end = 2 * len(pairs)
     add_B(3, 1)
     n_slots = 2 * len(pairs)
-    # the rescale block of (c, q) sits in front of this MFMA slot: all B(c - 1, q) MFMAs are issued,
-    # no B(c, q) MFMA is
-    rescale_at = {}
-    for c in range(4):
-        rescale_at.setdefault(first[(c, 1)], []).append((c, 0))
-        rescale_at.setdefault(first[(c + 1, 0)] if c < 3 else stage_end, []).append((c, 1))
-
     def half_off(c):
         return (c >> 1) * TILE + (c & 1) * (TILE // 2)
 
     def pair_loads(k):
         kind, c, x = pairs[k]
-        base = V_STG + 8 * (k % NSLOT)
+        base = A_STG + 8 * (k % NSLOT)
         if kind == "A":
-            return [(f"ds_read_b128 {vr(base, 4)}, %[r{x}] offset:{half_off(c)}", vset(base, 4))]
+            return [(f"ds_read_b128 {ar(base, 4)}, %[r{x}] offset:{half_off(c)}", aset(base, 4))]
         q, u, j = x
         off = 2 * TILE + half_off(c) + u * 4096
         loads = []
         for i, db in enumerate((2 * j, 2 * j + 1)):
             for hi in range(2):
                 reg = base + 4 * i + 2 * hi
-                loads.append((f"ds_read_b64_tr_b16 {vr(reg, 2)}, %[t{2 * db + hi}] offset:{off}", vset(reg, 2)))
+                loads.append((f"ds_read_b64_tr_b16 {ar(reg, 2)}, %[t{2 * db + hi}] offset:{off}", aset(reg, 2)))
         return loads
 
     def pair_mfmas(k):
         kind, c, x = pairs[k]
-        base = V_STG + 8 * (k % NSLOT)
+        base = A_STG + 8 * (k % NSLOT)
         out = []
         if kind == "A":
             ks = x
             for q in range(2):
                 s = v_s(c, q)
-                cs = "0" if ks == 0 else vr(s, 16)
-                out.append((vr(s, 16), vr(base, 4), ar(A_Q + 32 * q + 4 * ks, 4), cs, vset(s, 16), vset(base, 4),
-                            aset(A_Q + 32 * q + 4 * ks, 4), set() if ks == 0 else vset(s, 16)))
+                # the chain starts from -M: its result is the score relative to the reference maximum
+                cin = V_NEGM + 16 * q if ks == 0 else s
+                out.append((vr(s, 16), ar(base, 4), ar(A_Q + 32 * q + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(base, 4),
+                            aset(A_Q + 32 * q + 4 * ks, 4), vset(cin, 16)))
             return out
         q, u, j = x
         p = v_p(c, q, u)
         for i, db in enumerate((2 * j, 2 * j + 1)):
             acc = A_O + 64 * q + 16 * db
-            out.append((ar(acc, 16), vr(base + 4 * i, 4), vr(p, 4), ar(acc, 16), aset(acc, 16), vset(base + 4 * i, 4),
+            out.append((ar(acc, 16), ar(base + 4 * i, 4), vr(p, 4), ar(acc, 16), aset(acc, 16), aset(base + 4 * i, 4),
                         vset(p, 4), aset(acc, 16)))
         return out
 
-    # ---- VALU work of E(c): one list of (kind, ...) per stage ---------------------------------
-    c2 = SREG["c2"]
+    # ---- VALU work of E(c, q): a list of (kind, ...) ------------------------------------------
     T = [V_TMP + i for i in range(10)]
+    tag = "m" if masked else "f"
 
     def softmax_ops(c, q):
-        """Online softmax of the 16 scores of q block q in kv block c."""
+        """Online softmax of the lane's 16 scores (relative to M) of q block q in kv block c."""
         s = v_s(c, q)
-        M, Mt, L, AL = f"%[M{q}]", f"%[Mt{q}]", f"%[L{q}]", V_AL + q
+        M, Mt, L = f"%[M{q}]", f"%[Mt{q}]", f"%[L{q}]"
+        kM, kMt, kL = {("op", f"M{q}")}, {("op", f"Mt{q}")}, {("op", f"L{q}")}
+        D, AL, negm = V_D + q, V_AL + q, V_NEGM + 16 * q
         ops = []
 
         def valu(text, dst, src, trans=False):
             ops.append(("valu", text, dst, src, trans))
 
+        def raw(text):
+            ops.append(("raw", text))
+
+        if c > 0:
+            # M moved while this block's chain was in flight with the old -M: apply the shift now
+            raw(f"s_cmp_eq_u32 {S_PEND[q]}, 0")
+            raw(f"s_cbranch_scc1 .Lfa_fwd_{tag}_late{c}{q}_%=")
+            ops.append(("skip_begin",))
+            for e in range(16):
+                valu(f"v_sub_f32_e32 {vr(s + e)}, {vr(s + e)}, {vr(D)}", vset(s + e), vset(s + e) | vset(D))
+            raw(f"s_mov_b32 {S_PEND[q]}, 0")
+            ops.append(("skip_end",))
+            ops.append(("label", f".Lfa_fwd_{tag}_late{c}{q}_%=:"))
         if masked:
             for g in range(4):
                 for u in range(4):
@@ -194,50 +213,70 @@ def build(masked):
         valu(f"v_max3_f32 {vr(T[3])}, {vr(T[3])}, {vr(T[4])}, {vr(s + 15)}", vset(T[3]), vset(T[3]) | vset(T[4]) | vset(s + 15))
         valu(f"v_max_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[3])}", vset(T[0]), vset(T[0]) | vset(T[3]))
         valu(f"v_mov_b32_e32 {vr(T[1])}, {vr(T[0])}", vset(T[1]), vset(T[0]))
-        ops.append(("raw", "s_nop 1"))
+        raw("s_nop 1")
         valu(f"v_permlane32_swap_b32 {vr(T[0])}, {vr(T[1])}", vset(T[0]) | vset(T[1]), vset(T[0]) | vset(T[1]))
-        ops.append(("raw", "s_nop 1"))
+        raw("s_nop 1")
         valu(f"v_max_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[1])}", vset(T[0]), vset(T[0]) | vset(T[1]))
-        valu(f"v_mul_f32_e32 {vr(T[0])}, {c2}, {vr(T[0])}", vset(T[0]), vset(T[0]))            # log2 domain (sm_scale > 0)
-        valu(f"v_max_f32_e32 {Mt}, {Mt}, {vr(T[0])}", set(), vset(T[0]))
-        valu(f"v_add_f32_e32 {vr(T[1])}, {TAU}, {M}", vset(T[1]), set())
-        valu(f"v_cmp_gt_f32_e32 vcc, {vr(T[0])}, {vr(T[1])}", set(), vset(T[0]) | vset(T[1]))
-        ops.append(("raw", "s_cmp_lg_u64 vcc, 0"))
-        ops.append(("raw", f"s_cselect_b32 {S_FLAG[q]}, 1, 0"))
-        valu(f"v_cndmask_b32_e32 {vr(T[2])}, {M}, {vr(T[0])}, vcc", vset(T[2]), vset(T[0]))   # M_new
-        valu(f"v_sub_f32_e32 {vr(T[3])}, {M}, {vr(T[2])}", vset(T[3]), vset(T[2]))
-        valu(f"v_exp_f32_e32 {vr(AL)}, {vr(T[3])}", vset(AL), vset(T[3]), True)                # alpha = 2^(M_old - M_new)
-        valu(f"v_mov_b32_e32 {M}, {vr(T[2])}", set(), vset(T[2]))
-        # p = 2^(score c2 - M), packed to bf16 B operands; the row sum adds the rounded values
-        for e in range(16):
-            valu(f"v_fma_f32 {vr(s + e)}, {vr(s + e)}, {c2}, -{M}", vset(s + e), vset(s + e))
-        for e in range(16):
-            valu(f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True)
-        valu(f"v_mov_b32_e32 {vr(T[4])}, 0", vset(T[4]), set())
-        for g in range(4):
-            for h in range(2):
-                e = 4 * g + 2 * h
-                p = v_p(c, q, g >> 1) + 2 * (g & 1) + h
-                valu(f"v_cvt_pk_bf16_f32 {vr(p)}, {vr(s + e)}, {vr(s + e + 1)}", vset(p), vset(s + e, 2))
-        for g in range(4):
-            for h in range(2):
-                p = v_p(c, q, g >> 1) + 2 * (g & 1) + h
-                valu(f"v_dot2c_f32_bf16_e32 {vr(T[4])}, 0x3f803f80, {vr(p)}", vset(T[4]), vset(T[4]) | vset(p))
-        valu(f"v_fma_f32 {L}, {L}, {vr(AL)}, {vr(T[4])}", set(), vset(AL) | vset(T[4]))
-        return ops
-
-    def rescale_ops(c, q):
-        """O^T of q block q times alpha, skipped unless a lane of the wave raised M in E(c)."""
-        ops = [("raw", f"s_cmp_eq_u32 {S_FLAG[q]}, 0"),
-               ("raw", f"s_cbranch_scc1 .Lfa_fwd_{'m' if masked else 'f'}_keep{c}{q}_%=")]
-        AL = V_AL + q
+        valu(f"v_max_f32_e32 {Mt}, {Mt}, {vr(T[0])}", kMt, kMt | vset(T[0]))
+        # does the running maximum leave [-TAU, TAU] (and is it finite: rows that kept nothing so far stay put)?
+        valu(f"v_cmp_gt_f32_e64 vcc, |{Mt}|, {vr(V_TAU)}", set(), kMt | vset(V_TAU))
+        if masked:
+            valu(f"v_cmp_neq_f32_e64 s[86:87], {Mt}, {vr(V_NEGINF)}", set(), kMt | vset(V_NEGINF))
+            raw("s_and_b64 vcc, vcc, s[86:87]")
+        raw(f"s_cbranch_vccz .Lfa_fwd_{tag}_keep{c}{q}_%=")
+        ops.append(("skip_begin",))
+        raw("s_nop 3")
+        valu(f"v_cndmask_b32_e32 {vr(D)}, 0, {Mt}, vcc", vset(D), kMt)                 # the lane's shift
+        valu(f"v_exp_f32_e64 {vr(AL)}, -{vr(D)}", vset(AL), vset(D), True)
+        valu(f"v_sub_f32_e32 {Mt}, {Mt}, {vr(D)}", kMt, kMt | vset(D))
+        valu(f"v_add_f32_e32 {M}, {M}, {vr(D)}", kM, kM | vset(D))
+        valu(f"v_mul_f32_e32 {L}, {L}, {vr(AL)}", kL, kL | vset(AL))
         for i in range(64):
             t = T[5 + (i % 4)]
-            a = A_O + 64 * q + i
-            ops.append(("valu", f"v_accvgpr_read_b32 {vr(t)}, {ar(a)}", vset(t), aset(a), False))
-            ops.append(("valu", f"v_mul_f32_e32 {vr(t)}, {vr(t)}, {vr(AL)}", vset(t), vset(t) | vset(AL), False))
-            ops.append(("valu", f"v_accvgpr_write_b32 {ar(a)}, {vr(t)}", aset(a), vset(t), False))
-        ops.append(("raw", f".Lfa_fwd_{'m' if masked else 'f'}_keep{c}{q}_%=:"))
+            acc = A_O + 64 * q + i
+            valu(f"v_accvgpr_read_b32 {vr(t)}, {ar(acc)}", vset(t), aset(acc))
+            valu(f"v_mul_f32_e32 {vr(t)}, {vr(t)}, {vr(AL)}", vset(t), vset(t) | vset(AL))
+            valu(f"v_accvgpr_write_b32 {ar(acc)}, {vr(t)}", aset(acc), vset(t))
+        for e in range(16):
+            valu(f"v_sub_f32_e32 {vr(s + e)}, {vr(s + e)}, {vr(D)}", vset(s + e), vset(s + e) | vset(D))
+        for e in range(16):
+            valu(f"v_sub_f32_e32 {vr(negm + e)}, {vr(negm + e)}, {vr(D)}", vset(negm + e), vset(negm + e) | vset(D))
+        if c < 3:
+            raw(f"s_mov_b32 {S_PEND[q]}, 1")  # (kv block c + 1 of this step is in flight; block 0 of the next step is not)
+        ops.append(("skip_end",))
+        ops.append(("label", f".Lfa_fwd_{tag}_keep{c}{q}_%=:"))
+        # p = 2^(score - M), packed to bf16 B operands.  The row sum adds the fp32 values in four
+        # interleaved partial sums (plain adds hide under the MFMAs; v_dot2c on the packed values
+        # measured 9 cycles apiece).
+        def exps(g):
+            for u in range(4):
+                e = 4 * g + u
+                valu(f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True)
+
+        def packs(g):
+            for h in range(2):
+                e = 4 * g + 2 * h
+                pr = v_p(c, q, g >> 1) + 2 * (g & 1) + h
+                valu(f"v_cvt_pk_bf16_f32 {vr(pr)}, {vr(s + e)}, {vr(s + e + 1)}", vset(pr), vset(s + e, 2))
+
+        def sums(g):
+            for u in range(4):
+                e = 4 * g + u
+                if g == 1:
+                    valu(f"v_add_f32_e32 {vr(T[u])}, {vr(s + u)}, {vr(s + e)}", vset(T[u]), vset(s + u) | vset(s + e))
+                elif g > 1:
+                    valu(f"v_add_f32_e32 {vr(T[u])}, {vr(T[u])}, {vr(s + e)}", vset(T[u]), vset(T[u]) | vset(s + e))
+
+        exps(0)
+        for g in range(4):
+            if g < 3:
+                exps(g + 1)
+            sums(g)
+            packs(g)
+        valu(f"v_add_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[1])}", vset(T[0]), vset(T[0]) | vset(T[1]))
+        valu(f"v_add_f32_e32 {vr(T[2])}, {vr(T[2])}, {vr(T[3])}", vset(T[2]), vset(T[2]) | vset(T[3]))
+        valu(f"v_add_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[2])}", vset(T[0]), vset(T[0]) | vset(T[2]))
+        valu(f"v_add_f32_e32 {L}, {L}, {vr(T[0])}", kL, kL | vset(T[0]))
         return ops
 
     slot_ops = {m: [] for m in range(n_slots + 1)}
@@ -246,10 +285,29 @@ def build(masked):
     for c in range(4):
         for q in range(2):
             ops = softmax_ops(c, q)
-            lo = first[(c, q)] + (4 if (c, q) == (0, 0) else 0)  # E(0, 0) directly follows A(0): give its results time
+            lo = first[(c, q)] + 4  # the block's last MFMAs were issued just before: give their results time
             span = last[(c, q)] - lo
+            # a branch, the block it may skip and its label stay in one slot (no MFMA or LDS read may
+            # end up inside the skipped range); the block counts for nothing when the work is spread
+            total = 0
+            inside = False
+            for op in ops:
+                if op[0] == "skip_begin":
+                    inside = True
+                if not inside and op[0] != "label":
+                    total += 1
+                if op[0] == "skip_end":
+                    inside = False
+            done = 0
+            pinned = None
             for i, op in enumerate(ops):
-                slot_ops[lo + (i * span) // len(ops)].append(op)
+                if pinned is None and i + 1 < len(ops) and ops[i + 1][0] == "skip_begin":
+                    pinned = lo + (done * span) // total  # (op is the branch)
+                slot_ops[pinned if pinned is not None else lo + (done * span) // total].append(op)
+                if pinned is None or i + 1 < len(ops) and ops[i + 1][0] == "skip_begin":
+                    done += 1
+                if op[0] == "label":
+                    pinned = None
 
     for k in range(len(pairs)):
         at = 2 * (k - PREFETCH)
@@ -268,6 +326,12 @@ def build(masked):
     def emit(op):
         if op[0] == "raw":
             em.raw(op[1])
+        elif op[0] == "label":
+            em.label(op[1])
+        elif op[0] == "skip_begin":
+            em.skip_begin()
+        elif op[0] == "skip_end":
+            em.skip_end()
         elif "valu" not in DROP:
             em.valu(*op[1:])
 
@@ -276,10 +340,6 @@ def build(masked):
     for text, dst in pre_lds:
         em.lds_read(text, dst)
     for m in range(n_slots):
-        if m in rescale_at and "valu" not in DROP:
-            for c, q in rescale_at[m]:
-                for op in rescale_ops(c, q):
-                    emit(op)
         for ld in slot_vmem[m]:
             if "vmem" not in DROP:
                 em.lds_direct_load(*ld)
@@ -303,6 +363,8 @@ def run_loop(full, masked):
     entry += ["s_waitcnt lgkmcnt(0)"]  # (the streams count LDS operations from zero)
     entry += [f"v_readfirstlane_b32 {S[n]}, {vr(V_TBL + i)}" for i, n in enumerate(TABLE)]
     entry += [f"v_readfirstlane_b32 {S[n]}, %[{n}]" for n in STATE_IO + STATE_IN]
+    entry += [f"v_mov_b32_e32 {vr(V_TAU)}, {TAU}", f"s_mov_b32 {S_PEND[0]}, 0", f"s_mov_b32 {S_PEND[1]}, 0"]
+    entry += [f"v_sub_f32_e32 {vr(V_NEGM + 16 * q + e)}, 0, %[M{q}]" for q in range(2) for e in range(16)]
     top = entry + [".Lfa_fwd_loop_%=:"]
     # on the item's last step the tiles copied "for the next step" are the first step of the next
     # work item (from the table; with no next item they repeat this one's)

@@ -7,9 +7,14 @@ hardware leaves to software on gfx950:
     VALU result          -> MFMA operand                   2 wait states
     transcendental result-> VALU use                        1 wait state
     dot (v_dot2c) result -> other VALU use / overwrite      4 wait states (accumulating dots chain freely)
+    MFMA reading C from registers other than its destination -> VALU write of them   12 wait states
     LDS read result      -> any use                         s_waitcnt lgkmcnt (reads return in order)
-Registers are ("v", n) / ("a", n) pairs; operands supplied by the compiler (%[name]) are never
-written by a stream and need no tracking.
+Registers are ("v", n) / ("a", n) pairs, or any other hashable key a generator chooses for a
+compiler-supplied operand it wants tracked (("op", name)).
+
+Blocks that a scalar branch may skip (skip_begin / skip_end around them) are scheduled as if executed,
+and the code behind them is scheduled for both cases: as if the block had taken no time, with the
+block's register writes as recent as possible and the writes before the block still remembered.
 """
 
 
@@ -37,6 +42,8 @@ class Emitter:
         self.valu_w = {}
         self.trans_w = {}
         self.dot_w = {}
+        self.c_read = {}           # reg -> time of the MFMA that read it as C without writing it
+        self._skip = None
         self.lds_fifo = []         # outstanding LDS reads, oldest first: sets of dst regs
         self.stats = {"nop": 0, "wait": 0, "mfma": 0, "valu": 0, "lds": 0}
 
@@ -80,6 +87,8 @@ class Emitter:
             if r in self.valu_w:
                 self._need_gap(self.valu_w[r], 2)
         self._raw(f"v_mfma_f32_32x32x16_bf16 {dst}, {a}, {b}, {c}")
+        for r in c_regs - dst_regs:
+            self.c_read[r] = self.t - 1
         for r in dst_regs:
             self.mfma_w[r] = self.t - 1
             self.valu_w.pop(r, None)
@@ -98,6 +107,9 @@ class Emitter:
         for r in dst_regs | src_regs:
             if r in self.dot_w and not (is_dot and r in dst_regs):
                 self._need_gap(self.dot_w[r], 4)
+        for r in dst_regs:
+            if r in self.c_read:
+                self._need_gap(self.c_read.pop(r), 12)
         self._raw(text)
         for r in dst_regs:
             self.mfma_w.pop(r, None)
@@ -144,6 +156,27 @@ class Emitter:
     def raw(self, text):
         """Scalar or wait instruction with no tracked vector registers."""
         self._raw(text)
+
+    def label(self, text):
+        self._raw(text, 0)
+
+    _TRACKED = ("mfma_w", "valu_w", "trans_w", "dot_w", "c_read")
+
+    def skip_begin(self):
+        """The instructions up to skip_end() may be jumped over by the branch emitted just before."""
+        assert self._skip is None
+        self._skip = (self.t, {n: dict(getattr(self, n)) for n in self._TRACKED}, len(self.lds_fifo))
+
+    def skip_end(self):
+        t0, saved, n_lds = self._skip
+        self._skip = None
+        assert len(self.lds_fifo) == n_lds, "no LDS operations inside a skippable block"
+        for n in self._TRACKED:
+            merged = dict(saved[n])
+            for r, t in getattr(self, n).items():
+                merged[r] = max(merged.get(r, -1 << 30), min(t, t0 - 1))
+            setattr(self, n, merged)
+        self.t = t0
 
     def drain(self):
         if self.lds_fifo:

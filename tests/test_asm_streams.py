@@ -38,8 +38,10 @@ def split_operands(line):
 def check_stream(lines):
     """Replays a stream; returns the number of instructions checked."""
     t = 0
-    mfma_w, valu_w, trans_w, dot_w = {}, {}, {}, {}
+    mfma_w, valu_w, trans_w, dot_w, c_read = {}, {}, {}, {}, {}
+    tracked = (mfma_w, valu_w, trans_w, dot_w, c_read)
     fifo = []  # outstanding LDS reads: destination register sets, oldest first
+    skips = {}  # label -> (time behind the forward branch, copies of the tracked maps, LDS queue length)
     n = 0
 
     def gap(t_def):
@@ -59,7 +61,27 @@ def check_stream(lines):
                 del fifo[: len(fifo) - int(m.group(1))]
             t += 1
             continue
-        if op.startswith("s_") or op.endswith(":") or op.startswith(".L"):
+        if op.endswith(":"):
+            # A label that a forward branch of the stream jumps to: what follows must hold both after
+            # the skipped block (executed) and without it (no time passed, older writes still there).
+            if op[:-1] in skips:
+                t0, saved, n_fifo = skips.pop(op[:-1])
+                assert len(fifo) == n_fifo, f"LDS traffic inside a skippable block: {line}"
+                for cur, old in zip(tracked, saved):
+                    merged = dict(old)
+                    for r, tw in cur.items():
+                        merged[r] = max(merged.get(r, -1 << 30), min(tw, t0 - 1))
+                    cur.clear()
+                    cur.update(merged)
+                t = t0
+            continue
+        if op.startswith("s_cbranch"):
+            t += 1
+            label = ops[0]
+            if any(l.strip() == label + ":" for l in lines[lines.index(line) + 1:]):
+                skips[label] = (t, [dict(d) for d in tracked], len(fifo))
+            continue
+        if op.startswith("s_"):
             t += 1
             continue
         n += 1
@@ -70,8 +92,9 @@ def check_stream(lines):
                 assert r not in mfma_w or gap(mfma_w[r]) >= 12, f"MFMA result used as A/B too early: {line}"
             for r in a | b | c | dst:
                 assert r not in valu_w or gap(valu_w[r]) >= 2, f"VALU result used by MFMA too early: {line}"
-            if c:
-                assert c == dst, f"accumulating MFMA must read its own destination: {line}"
+            for r in c - dst:
+                assert r not in mfma_w or gap(mfma_w[r]) >= 12, f"MFMA result used as C of another chain too early: {line}"
+                c_read[r] = t
             for r in dst:
                 mfma_w[r] = t
                 valu_w.pop(r, None)
@@ -104,6 +127,7 @@ def check_stream(lines):
                 if r in dot_w and not (is_dot and r in dst):
                     assert gap(dot_w[r]) >= 3, f"VALU uses a fresh dot-product result: {line}"
             for r in dst:
+                assert r not in c_read or gap(c_read.pop(r)) >= 12, f"VALU overwrites the C input of an MFMA in flight: {line}"
                 if is_dot:
                     dot_w[r] = t
                 else:
@@ -119,6 +143,7 @@ def check_stream(lines):
             raise AssertionError(f"unknown instruction in stream: {line}")
         t += 1
     assert not fifo, "stream ends with LDS reads in flight"
+    assert not skips, f"forward branch to a label that never came: {list(skips)}"
     return n
 
 
@@ -211,4 +236,15 @@ def test_fwd_tile_streams_respect_hazards():
         n = check_stream(em.out)
         assert em.stats["mfma"] == 128  # 4 kv blocks x 2 q blocks x (8 S + 8 PV)
         assert n == em.stats["mfma"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
-        scratch_ok(em.out, 66, 245, 191)
+        scratch_ok(em.out, 66, 199, 255)
+        # between a forward branch and its label there is only VALU / scalar work: a skipped MFMA,
+        # LDS read or wait would break the stream's bookkeeping
+        pending = None
+        for line in em.out:
+            if line.startswith("s_cbranch"):
+                pending = line.split()[1]
+            elif pending and line.strip() == pending + ":":
+                pending = None
+            elif pending:
+                assert not line.startswith(("v_mfma", "ds_", "global_load", "s_waitcnt")), (pending, line)
+        assert pending is None

@@ -175,10 +175,11 @@ def test_causal_flag_and_segment_ids_arguments(F):
     assert torch.equal(o2, o)
 
 
-def test_forward_stream_kernel_on_request(F, monkeypatch):
-    """FLEXATTN_FWD_STREAM=1 routes plain-score bf16 forward calls to the generated-stream kernel:
-    same results as the oracle, including rows whose tiles are partly or entirely masked."""
-    monkeypatch.setenv("FLEXATTN_FWD_STREAM", "1")
+def test_forward_compiled_kernel_on_request(F, monkeypatch):
+    """Plain-score bf16 forward calls run the generated-stream kernel (covered by every other test
+    here); FLEXATTN_FWD_STREAM=0 routes them to the compiled kernel, which must agree with the oracle
+    as well, including rows whose tiles are partly or entirely masked."""
+    monkeypatch.setenv("FLEXATTN_FWD_STREAM", "0")
     for name, shape, mask_pair, score_fn, okw, sc in _small_cases():
         if score_fn is not None:
             continue
@@ -190,6 +191,7 @@ def test_forward_stream_kernel_on_request(F, monkeypatch):
         o, l, m = _fwd(F, q, k, v, sc, mf, bf, None)
         assert_close(name + " o", o, ro, torch.bfloat16)
         assert_close(name + " lse", m + l.log(), rm + rl.log(), torch.bfloat16)
+
 
 def test_entry_points_reject_bad_arguments_on_gpu(F):
     q = torch.zeros(1, 2, 192, 128, dtype=torch.bfloat16, device=DEV)
