@@ -550,20 +550,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     if (partial) {
       // the lane's keep bits: element e of q block c sits at bit 16 (c & 1) + e of km[c >> 1]
       const int q0 = qb * BQ;
-      const bool has_doc = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
 #pragma unroll
-      for (int cc = 0; cc < 4; ++cc) {
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          const int r0 = 32 * cc + 8 * g4 + 4 * hh;
-          int di[4] = {0, 0, 0, 0};
-          if (has_doc) {
-            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_q + q0 + r0);
-            di[0] = d4[0]; di[1] = d4[1]; di[2] = d4[2]; di[3] = d4[3];
-          }
-          km[cc >> 1] |= keep_bits4_queries(a.mask, q0 + r0, k_idx, di, doc_j) << (16 * (cc & 1) + 4 * g4);
-        }
-      }
+      for (int half = 0; half < 2; ++half)
+        km[half] = keep_bits32<false>(a.mask, k_idx, q0 + 64 * half + 4 * hh, doc_j, a.mask.doc_q);
     } else {
       // the run of full tiles ends before the next partial one: lanes look 64 steps ahead at a time
       bool found = false;

@@ -473,30 +473,13 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
       unsigned km[2] = {0u, 0u};
       if (partial) {
         // the lane's keep bits: element e of kv block c sits at bit 16 (c & 1) + e of km[c >> 1]
-        const bool has_doc = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
 #pragma unroll
         for (int hx = 0; hx < 2; ++hx) {
           const int e = 2 * it + hx;
           if (e >= n_tiles) continue;  // missing half: all dropped
-          const int state = __builtin_amdgcn_readfirstlane((int)sSt[sIdx[e]]);
-          if (state == 2) {
-            km[hx] = 0xffffffffu;
-            continue;
-          }
-          const int kv0 = __builtin_amdgcn_readfirstlane(sIdx[e]) * BN;
-#pragma unroll
-          for (int c = 0; c < 2; ++c) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-              const int j0 = kv0 + 32 * c + 8 * g + 4 * hh;
-              int dj[4] = {0, 0, 0, 0};
-              if (has_doc) {
-                const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_k + j0);
-                dj[0] = d4[0]; dj[1] = d4[1]; dj[2] = d4[2]; dj[3] = d4[3];
-              }
-              km[hx] |= keep_bits4_keys(a.mask, q_idx, j0, doc_i, dj) << (16 * c + 4 * g);
-            }
-          }
+          const int kt = __builtin_amdgcn_readfirstlane(sIdx[e]);
+          const int state = __builtin_amdgcn_readfirstlane((int)sSt[kt]);
+          km[hx] = state == 2 ? 0xffffffffu : keep_bits32<true>(a.mask, q_idx, kt * BN + 4 * hh, doc_i, a.mask.doc_k);
         }
       } else {
         // the run of full steps ends before the next partial one: lanes look 64 steps ahead at a time

@@ -140,27 +140,47 @@ __device__ __forceinline__ bool keep_elem(const MaskArgs& mk, int i, int j, int 
   return keep;
 }
 
-// Keep bits (bit u = element u) of four elements in a row of the score matrix: query i against
-// keys j0 .. j0 + 3 (keys_vary) or queries i0 .. i0 + 3 against key j.  The purely causal mask,
-// the common case, needs no per-element work.
-__device__ __forceinline__ unsigned keep_bits4_keys(const MaskArgs& mk, int i, int j0, int doc_i, const int (&dj)[4]) {
-  if (mk.flags == FLEXATTN_MASK_CAUSAL) {
-    const int n = min(max(i - j0 + 1, 0), 4);  // keys j0 .. j0 + n - 1 are not in the future
-    return (1u << n) - 1u;
-  }
-  unsigned bits = 0;
-#pragma unroll
-  for (int u = 0; u < 4; ++u) bits |= (keep_elem(mk, i, j0 + u, doc_i, dj[u]) ? 1u : 0u) << u;
-  return bits;
+// Keep bits of a lane's 32 elements in a 64-wide strip of the score matrix, for the generated
+// streams: element (c, g, u), c < 2, g < 4, u < 4, lies at offset 32 c + 8 g + u from `base` along the
+// varying index (keys when KEYS, the query is then `fixed`; queries otherwise, the key is `fixed`)
+// and owns bit 16 c + 4 g + u.  The purely causal mask, the common case, has a closed form: a
+// 64-bit run of ones over the offsets, of which the even nibbles are the lane's elements.  Other
+// masks loop over the elements (rolled: the code stays small, these tiles are rare).
+__device__ __forceinline__ unsigned compress_even_nibbles(unsigned long long m) {
+  m &= 0x0F0F0F0F0F0F0F0Full;
+  m = (m | (m >> 4)) & 0x00FF00FF00FF00FFull;
+  m = (m | (m >> 8)) & 0x0000FFFF0000FFFFull;
+  m = (m | (m >> 16)) & 0x00000000FFFFFFFFull;
+  return (unsigned)m;
 }
-__device__ __forceinline__ unsigned keep_bits4_queries(const MaskArgs& mk, int i0, int j, const int (&di)[4], int doc_j) {
+template <bool KEYS>
+__device__ __forceinline__ unsigned keep_bits32(const MaskArgs& mk, int fixed, int base, int doc_fixed,
+                                                const int* doc_var) {
   if (mk.flags == FLEXATTN_MASK_CAUSAL) {
-    const int n = min(max(j - i0, 0), 4);  // queries i0 .. i0 + n - 1 come before the key
-    return (0xFu << n) & 0xFu;
+    if (KEYS) {
+      // key base + off is kept iff off <= fixed - base
+      const int d = fixed - base;
+      const unsigned long long run = d < 0 ? 0ull : (d >= 63 ? ~0ull : ((2ull << d) - 1ull));
+      return compress_even_nibbles(run);
+    }
+    // query base + off is kept iff off >= fixed - base
+    const int d = fixed - base;
+    const unsigned long long run = d <= 0 ? ~0ull : (d >= 64 ? 0ull : ~((1ull << d) - 1ull));
+    return compress_even_nibbles(run);
   }
+  const bool has_doc = (mk.flags & FLEXATTN_MASK_DOC) != 0;
   unsigned bits = 0;
+#pragma unroll 1
+  for (int cg = 0; cg < 8; ++cg) {
+    const int off = 32 * (cg >> 2) + 8 * (cg & 3);
 #pragma unroll
-  for (int u = 0; u < 4; ++u) bits |= (keep_elem(mk, i0 + u, j, di[u], doc_j) ? 1u : 0u) << u;
+    for (int u = 0; u < 4; ++u) {
+      const int idx = base + off + u;
+      const int doc = has_doc ? doc_var[idx] : 0;
+      const bool keep = KEYS ? keep_elem(mk, fixed, idx, doc_fixed, doc) : keep_elem(mk, idx, fixed, doc, doc_fixed);
+      bits |= (keep ? 1u : 0u) << (16 * (cg >> 2) + 4 * (cg & 3) + u);
+    }
+  }
   return bits;
 }
 

@@ -590,7 +590,6 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
       int it_end = it + 1;
       unsigned km[4] = {0u, 0u, 0u, 0u};  // keep bits of q block x, kv tile hx of the step: km[2 x + hx]
       if (partial) {
-        const bool has_doc = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
 #pragma unroll
         for (int hx = 0; hx < 2; ++hx) {
           const int e = 2 * it + hx;
@@ -599,23 +598,10 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
 #pragma unroll
           for (int x = 0; x < 2; ++x) {
             const int state = __builtin_amdgcn_readfirstlane((int)(x == 0 ? sStA[k] : sStB[k]));
-            if (state == 0) continue;
             if (state == 2) {
               km[2 * x + hx] = 0xffffffffu;
-              continue;
-            }
-#pragma unroll
-            for (int c = 0; c < 2; ++c) {
-#pragma unroll
-              for (int g = 0; g < 4; ++g) {
-                const int j0 = k * BN + 32 * c + 8 * g + 4 * hh;
-                int dj[4] = {0, 0, 0, 0};
-                if (has_doc) {
-                  const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_k + j0);
-                  dj[0] = d4[0]; dj[1] = d4[1]; dj[2] = d4[2]; dj[3] = d4[3];
-                }
-                km[2 * x + hx] |= keep_bits4_keys(a.mask, q_idx[x], j0, doc_i[x], dj) << (16 * c + 4 * g);
-              }
+            } else if (state == 1) {
+              km[2 * x + hx] = keep_bits32<true>(a.mask, q_idx[x], k * BN + 4 * hh, doc_i[x], a.mask.doc_k);
             }
           }
         }
