@@ -9,7 +9,8 @@ accumulation registers, so every K / V fragment read from LDS feeds two MFMAs.  
 
     A(c): S'^T = K Q^T - M for both q blocks   16 MFMAs, operands: 8 ds_read_b128 (rows of K)
     E(c, x): online softmax of the lane's 16 scores of q block x (45 VALU ops)
-    B(c, x): O^T += V^T P^T of q block x       8 MFMAs, operands: 16 ds_read_b64_tr_b16 (V)
+    B(c, x): O^T += V^T P^T of q block x       8 MFMAs, operands: 32 ds_read_b64_tr_b16 (V), read once
+             for both q blocks
 
     The two q blocks run half a stage apart: E(c, 0) under A(c+1)[k-steps 0-3] and B(c-1, 1),
     E(c, 1) under A(c+1)[k-steps 4-7] and B(c, 0).
@@ -55,7 +56,6 @@ import sys
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 from gfx950_stream import Emitter, ar, aset, vr, vset  # noqa: E402
 
-NSLOT = 8        # staging slots of 8 registers
 PREFETCH = 4     # MFMA pairs between the LDS reads of a pair and its MFMAs
 LOAD_FIRST = 0   # MFMA slot of the first LDS-direct load of the next step
 LOAD_EVERY = 3   # slots between two of them
@@ -134,26 +134,42 @@ def build(masked):
     def half_off(c):
         return (c >> 1) * TILE + (c & 1) * (TILE // 2)
 
+    # Staging registers.  K row fragments rotate through eight 4-register slots.  The V^T fragments of
+    # a kv block have fixed places: B(c, 0) loads them, B(c, 1) half a stage later uses them again,
+    # and the fragments of block c + 1 are read in once the MFMA of B(c, 1) that used the place has
+    # been issued (B(c + 1, 0) follows B(c, 1) at the same distance).
+    a_index = {}
+    for k, (kind, c, x) in enumerate(pairs):
+        if kind == "A":
+            a_index[k] = len(a_index)
+
+    def k_slot(k):
+        return A_STG + 32 + 4 * (a_index[k] % 8)
+
+    def v_place(u, db):
+        return A_STG + 4 * (4 * u + db)
+
     def pair_loads(k):
         kind, c, x = pairs[k]
-        base = A_STG + 8 * (k % NSLOT)
         if kind == "A":
-            return [(f"ds_read_b128 {ar(base, 4)}, %[r{x}] offset:{half_off(c)}", aset(base, 4))]
+            return [(f"ds_read_b128 {ar(k_slot(k), 4)}, %[r{x}] offset:{half_off(c)}", aset(k_slot(k), 4))]
         q, u, j = x
+        if q == 1:
+            return []
         off = 2 * TILE + half_off(c) + u * 4096
         loads = []
-        for i, db in enumerate((2 * j, 2 * j + 1)):
+        for db in (2 * j, 2 * j + 1):
             for hi in range(2):
-                reg = base + 4 * i + 2 * hi
+                reg = v_place(u, db) + 2 * hi
                 loads.append((f"ds_read_b64_tr_b16 {ar(reg, 2)}, %[t{2 * db + hi}] offset:{off}", aset(reg, 2)))
         return loads
 
     def pair_mfmas(k):
         kind, c, x = pairs[k]
-        base = A_STG + 8 * (k % NSLOT)
         out = []
         if kind == "A":
             ks = x
+            base = k_slot(k)
             for q in range(2):
                 s = v_s(c, q)
                 # the chain starts from -M: its result is the score relative to the reference maximum
@@ -163,10 +179,10 @@ def build(masked):
             return out
         q, u, j = x
         p = v_p(c, q, u)
-        for i, db in enumerate((2 * j, 2 * j + 1)):
+        for db in (2 * j, 2 * j + 1):
             acc = A_O + 64 * q + 16 * db
-            out.append((ar(acc, 16), ar(base + 4 * i, 4), vr(p, 4), ar(acc, 16), aset(acc, 16), aset(base + 4 * i, 4),
-                        vset(p, 4), aset(acc, 16)))
+            vt = v_place(u, db)
+            out.append((ar(acc, 16), ar(vt, 4), vr(p, 4), ar(acc, 16), aset(acc, 16), aset(vt, 4), vset(p, 4), aset(acc, 16)))
         return out
 
     # ---- VALU work of E(c, q): a list of (kind, ...) ------------------------------------------
@@ -310,7 +326,9 @@ def build(masked):
                     pinned = None
 
     for k in range(len(pairs)):
-        at = 2 * (k - PREFETCH)
+        # (V^T fragments one pair later than K rows: in the last stages, which have no A pairs, the
+        # place's previous user is only four pairs ahead and must have been issued)
+        at = 2 * (k - (PREFETCH if pairs[k][0] == "A" else PREFETCH - 1))
         if at < 0:
             pre_lds.extend(pair_loads(k))
         else:
@@ -339,6 +357,10 @@ def build(masked):
         em.valu(f"v_mov_b32_e32 {vr(V_NEGINF)}, 0xff800000", vset(V_NEGINF), set())
     for text, dst in pre_lds:
         em.lds_read(text, dst)
+    holds = {}  # V^T place -> kv block whose fragment was last read into it
+    for k, (kind, c, x) in enumerate(pairs):
+        if kind == "B" and x[0] == 0 and 2 * (k - (PREFETCH - 1)) < 0:
+            raise AssertionError("V^T fragments are never part of the preamble")
     for m in range(n_slots):
         for ld in slot_vmem[m]:
             if "vmem" not in DROP:
@@ -346,6 +368,14 @@ def build(masked):
         for text, dst in slot_lds[m]:
             if "lds" not in DROP:
                 em.lds_read(text, dst)
+        for k, (kind, c, x) in enumerate(pairs):  # bookkeeping of the V^T places (see v_place)
+            if kind == "B" and x[0] == 0 and 2 * (k - (PREFETCH - 1)) == m:
+                for db in (2 * x[2], 2 * x[2] + 1):
+                    holds[(x[1], db)] = c
+        kind, c, x = pairs[m // 2]
+        if kind == "B":
+            db = 2 * x[2] + (m % 2)
+            assert holds.get((x[1], db)) == c, f"B({c}, {x[0]}) would multiply with the V^T fragment of block {holds.get((x[1], db))}"
         if "mfma" not in DROP:
             em.mfma(*pair_mfmas(m // 2)[m % 2])
         for op in slot_ops[m]:
