@@ -12,19 +12,20 @@
 
 #include <type_traits>
 
-// registers of the generated run loop (gen_dq_tile.py): v[66:215], s[60:100]
-#define FA_DQ_RUN_VGPRS "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", \
-  "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", \
-  "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", \
-  "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", \
-  "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", \
-  "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", \
-  "v146", "v147", "v148", "v149", "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", \
-  "v159", "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167", "v168", "v169", "v170", "v171", \
-  "v172", "v173", "v174", "v175", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", \
-  "v185", "v186", "v187", "v188", "v189", "v190", "v191", "v192", "v193", "v194", "v195", "v196", "v197", \
-  "v198", "v199", "v200", "v201", "v202", "v203", "v204", "v205", "v206", "v207", "v208", "v209", "v210", \
-  "v211", "v212", "v213", "v214", "v215"
+// registers of the generated run loop (gen_dq_tile.py): v[66:167], a[128:191], s[60:100]
+#define FA_DQ_RUN_VGPRS "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79", "v80", \
+  "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", \
+  "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", \
+  "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", \
+  "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", \
+  "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", \
+  "v149", "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", \
+  "v162", "v163", "v164", "v165", "v166", "v167", "a128", "a129", "a130", "a131", "a132", "a133", "a134", \
+  "a135", "a136", "a137", "a138", "a139", "a140", "a141", "a142", "a143", "a144", "a145", "a146", "a147", \
+  "a148", "a149", "a150", "a151", "a152", "a153", "a154", "a155", "a156", "a157", "a158", "a159", "a160", \
+  "a161", "a162", "a163", "a164", "a165", "a166", "a167", "a168", "a169", "a170", "a171", "a172", "a173", \
+  "a174", "a175", "a176", "a177", "a178", "a179", "a180", "a181", "a182", "a183", "a184", "a185", "a186", \
+  "a187", "a188", "a189", "a190", "a191"
 #define FA_DQ_RUN_SGPRS "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", \
   "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", \
   "s87", "s88", "s89", "s90", "s91", "s92", "s93", "s94", "s95", "s96", "s97", "s98", "s99", "s100"
@@ -370,12 +371,19 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
     unsigned char st[kListRegs];
   };
   DqPinned st;
+  // Q goes in multiplied by sm_scale * log2(e): the streams' scores are then in the log2 domain
+  const float c2 = a.sm_scale * kLog2e;
+  auto scaled = [c2](unsigned two) {
+    const float lo = __builtin_bit_cast(float, two << 16) * c2;
+    const float hi = __builtin_bit_cast(float, two & 0xffff0000u) * c2;
+    return __builtin_bit_cast(unsigned, pack_bf16(lo, hi));
+  };
   auto consume = [&](const ItemRegs& r, ItemHead& c) {
 #define FA_PUT(KS, QR, DR)                                                                                    \
   asm volatile(FA_DQ_PUT_##KS                                                                                 \
                : "={" QR "}"(st.q[KS]), "={" DR "}"(st.d[KS])                                                 \
-               : "v"(r.qw[KS][0]), "v"(r.qw[KS][1]), "v"(r.qw[KS][2]), "v"(r.qw[KS][3]), "v"(r.dw[KS][0]),    \
-                 "v"(r.dw[KS][1]), "v"(r.dw[KS][2]), "v"(r.dw[KS][3]));
+               : "v"(scaled(r.qw[KS][0])), "v"(scaled(r.qw[KS][1])), "v"(scaled(r.qw[KS][2])),                \
+                 "v"(scaled(r.qw[KS][3])), "v"(r.dw[KS][0]), "v"(r.dw[KS][1]), "v"(r.dw[KS][2]), "v"(r.dw[KS][3]));
     FA_PUT(0, "a[64:67]", "a[96:99]") FA_PUT(1, "a[68:71]", "a[100:103]") FA_PUT(2, "a[72:75]", "a[104:107]")
     FA_PUT(3, "a[76:79]", "a[108:111]") FA_PUT(4, "a[80:83]", "a[112:115]") FA_PUT(5, "a[84:87]", "a[116:119]")
     FA_PUT(6, "a[88:91]", "a[120:123]") FA_PUT(7, "a[92:95]", "a[124:127]")

@@ -6,8 +6,10 @@ statements: the run loop over steps of two 64-row kv tiles, and prologue / epilo
 A wave owns 32 q rows (Q^T, dO^T fragments and the dq^T accumulators stay in accumulation
 registers); one step covers 128 kv rows = four 32-row kv blocks c = 0..3, software-pipelined:
 
-    A(c): S^T = K Q^T, dP^T = V dO^T       16 MFMAs, operands: 16 ds_read_b128 (rows of K, V)
-    E(c): dS^T = exp2(S^T c2 - lse) (dP^T - delta)   72 VALU ops
+    A(c): S'^T = K Q^T - lse, dP^T = V dO^T  16 MFMAs, operands: 16 ds_read_b128 (rows of K, V)
+          (Q arrives multiplied by sm_scale log2 e, and -lse enters through the accumulator input of
+          the chain's first MFMA, so the result is already the exponent)
+    E(c): dS^T = exp2(S'^T) (dP^T - delta)   56 VALU ops
     B(c): dq^T += K^T dS^T                  8 MFMAs, operands: 16 ds_read_b64_tr_b16 (K again)
 
     MFMA order:  A0 | A1 | A2 B0 | A3 B1 | B2 | B3      VALU:  - | E0 | E1 | E2 | E3 | -
@@ -18,8 +20,9 @@ The emitter (gfx950_stream.py) inserts the s_nop / s_waitcnt that the hardware h
 
 Register contract with the C++ side (every asm statement names the accumulation registers with
 physical-register constraints):
-    a[0:63]   dq^T accumulators (4 x 16)   a[64:95] Q^T fragments (8 x 4)   a[96:127] dO^T fragments
-    v[66:215], s[60:100], vcc, m0   scratch of the run loop (clobbered)
+    a[0:63]   dq^T accumulators (4 x 16)   a[64:95] Q^T fragments (8 x 4), pre-scaled   a[96:127] dO^T fragments
+    a[128:191] staging slots of the LDS fragments (clobbered)
+    v[66:167], s[60:100], vcc, m0   scratch of the run loop (clobbered)
     (the table also names the next work item's first step, copied into LDS during this item's last step)
     %[r0..r7]  byte address of the lane's row fragment ks in K half-tile 0 of the current buffer
     %[t0..t7]  byte address of the lane's transposed fragment (2 db + hi) in K half-tile 0
@@ -39,7 +42,7 @@ import sys
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 from gfx950_stream import Emitter, ar, aset, vr, vset  # noqa: E402
 
-NSLOT = 8        # staging slots of 8 VGPRs
+NSLOT = 8        # staging slots of 8 registers
 PREFETCH = 4     # MFMA pairs between the LDS reads of a pair and its MFMAs
 LOAD_FIRST = 2   # MFMA slot of the first LDS-direct load of the next step
 LOAD_EVERY = 5   # slots between two of them
@@ -67,9 +70,9 @@ V_TBL = 72       # 12 scratch VGPRs the table is read into at entry
 V_S = [72, 104]
 V_DP = [88, 120]
 V_DS = 136       # dS^T as MFMA B operands: [c & 1][u] x 4 registers
-V_STG = 152
-V_END = 215
-A_DQ, A_Q, A_DO = 0, 64, 96
+V_NL = 152       # -lse of the lane's q row, 16 copies: accumulator input of the first MFMA of an S chain
+V_END = 167
+A_DQ, A_Q, A_DO, A_STG = 0, 64, 96, 128
 
 
 def build(masked):
@@ -100,38 +103,38 @@ def build(masked):
 
     def pair_loads(k):
         kind, c, x = pairs[k]
-        base = V_STG + 8 * (k % NSLOT)
+        base = A_STG + 8 * (k % NSLOT)
         if kind == "A":
             ks = x
-            return [(f"ds_read_b128 {vr(base, 4)}, %[r{ks}] offset:{half_off(c)}", vset(base, 4)),
-                    (f"ds_read_b128 {vr(base + 4, 4)}, %[r{ks}] offset:{2 * TILE + half_off(c)}", vset(base + 4, 4))]
+            return [(f"ds_read_b128 {ar(base, 4)}, %[r{ks}] offset:{half_off(c)}", aset(base, 4)),
+                    (f"ds_read_b128 {ar(base + 4, 4)}, %[r{ks}] offset:{2 * TILE + half_off(c)}", aset(base + 4, 4))]
         u, j = x
         off = half_off(c) + u * 4096
         loads = []
         for i, db in enumerate((2 * j, 2 * j + 1)):
             for hi in range(2):
                 reg = base + 4 * i + 2 * hi
-                loads.append((f"ds_read_b64_tr_b16 {vr(reg, 2)}, %[t{2 * db + hi}] offset:{off}", vset(reg, 2)))
+                loads.append((f"ds_read_b64_tr_b16 {ar(reg, 2)}, %[t{2 * db + hi}] offset:{off}", aset(reg, 2)))
         return loads
 
     def pair_mfmas(k):
         kind, c, x = pairs[k]
-        base = V_STG + 8 * (k % NSLOT)
+        base = A_STG + 8 * (k % NSLOT)
         if kind == "A":
             ks = x
             s, dp = V_S[c & 1], V_DP[c & 1]
-            cs = "0" if ks == 0 else vr(s, 16)
+            cin = V_NL if ks == 0 else s
             cd = "0" if ks == 0 else vr(dp, 16)
-            return [(vr(s, 16), vr(base, 4), ar(A_Q + 4 * ks, 4), cs, vset(s, 16), vset(base, 4), aset(A_Q + 4 * ks, 4),
-                     set() if ks == 0 else vset(s, 16)),
-                    (vr(dp, 16), vr(base + 4, 4), ar(A_DO + 4 * ks, 4), cd, vset(dp, 16), vset(base + 4, 4),
+            return [(vr(s, 16), ar(base, 4), ar(A_Q + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(base, 4), aset(A_Q + 4 * ks, 4),
+                     vset(cin, 16)),
+                    (vr(dp, 16), ar(base + 4, 4), ar(A_DO + 4 * ks, 4), cd, vset(dp, 16), aset(base + 4, 4),
                      aset(A_DO + 4 * ks, 4), set() if ks == 0 else vset(dp, 16))]
         u, j = x
         ds = V_DS + 8 * (c & 1) + 4 * u
         out = []
         for i, db in enumerate((2 * j, 2 * j + 1)):
             acc = A_DQ + 16 * db
-            out.append((ar(acc, 16), vr(base + 4 * i, 4), vr(ds, 4), ar(acc, 16), aset(acc, 16), vset(base + 4 * i, 4),
+            out.append((ar(acc, 16), ar(base + 4 * i, 4), vr(ds, 4), ar(acc, 16), aset(acc, 16), aset(base + 4 * i, 4),
                         vset(ds, 4), aset(acc, 16)))
         return out
 
@@ -144,9 +147,6 @@ def build(masked):
         s, dp = V_S[c & 1], V_DP[c & 1]
         ops = []
         for g in range(4):
-            for u in range(4):
-                e = 4 * g + u
-                ops.append((f"v_fma_f32 {vr(s + e)}, {vr(s + e)}, {c2}, -%[lse]", vset(s + e), vset(s + e), False))
             for u in range(4):
                 e = 4 * g + u
                 ops.append((f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
@@ -218,6 +218,7 @@ def run_loop(full, masked):
     entry += ["s_waitcnt lgkmcnt(0)"]  # (the streams count LDS operations from zero)
     entry += [f"v_readfirstlane_b32 {S[n]}, {vr(V_TBL + i)}" for i, n in enumerate(TABLE)]
     entry += [f"v_readfirstlane_b32 {S[n]}, %[{n}]" for n in STATE_IO + STATE_IN]
+    entry += [f"v_sub_f32_e32 {vr(V_NL + e)}, 0, %[lse]" for e in range(16)]
     top = entry + [".Lfa_dq_loop_%=:"]
     # On the item's last step the tiles copied "for the next step" are the first step of the next
     # work item (its kv tiles and K / V bases come from the table; with no next item they repeat

@@ -57,7 +57,7 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 from gfx950_stream import Emitter, ar, aset, vr, vset  # noqa: E402
 
 PREFETCH = 4     # MFMA pairs between the LDS reads of a pair and its MFMAs
-LOAD_FIRST = 0   # MFMA slot of the first LDS-direct load of the next step
+LOAD_FIRST = 1   # MFMA slot of the first LDS-direct load of the next step
 LOAD_EVERY = 3   # slots between two of them
 TAU = "0x40c00000"  # 6.0: M moves when the running maximum relative to it leaves [-6, 6]
 DROP = ()        # instruction classes left out (--drop, timing studies only)
@@ -362,9 +362,9 @@ def build(masked):
         if kind == "B" and x[0] == 0 and 2 * (k - (PREFETCH - 1)) < 0:
             raise AssertionError("V^T fragments are never part of the preamble")
     for m in range(n_slots):
-        for ld in slot_vmem[m]:
+        for ld in slot_vmem[m]:  # (M0 was written in front of the previous MFMA)
             if "vmem" not in DROP:
-                em.lds_direct_load(*ld)
+                em.lds_direct_issue(ld[1], ld[2])
         for text, dst in slot_lds[m]:
             if "lds" not in DROP:
                 em.lds_read(text, dst)
@@ -376,6 +376,9 @@ def build(masked):
         if kind == "B":
             db = 2 * x[2] + (m % 2)
             assert holds.get((x[1], db)) == c, f"B({c}, {x[0]}) would multiply with the V^T fragment of block {holds.get((x[1], db))}"
+        for ld in slot_vmem.get(m + 1, []):  # (the MFMA below is the wait state between M0 and its load)
+            if "vmem" not in DROP:
+                em.lds_direct_dest(ld[0], ld[3])
         if "mfma" not in DROP:
             em.mfma(*pair_mfmas(m // 2)[m % 2])
         for op in slot_ops[m]:

@@ -138,8 +138,17 @@ class Emitter:
 
     def lds_direct_load(self, lds_imm, goff, gbase, ldsn="%[ldsn]"):
         """Next step's global -> LDS copy of one 1 KB block (M0 = LDS destination)."""
+        self.lds_direct_dest(lds_imm, ldsn)
+        self.lds_direct_issue(goff, gbase)
+
+    def lds_direct_dest(self, lds_imm, ldsn="%[ldsn]"):
+        """M0 for the next LDS-direct load.  The load needs one wait state after the write: callers
+        that put other instructions in between save the s_nop."""
         self._raw(f"s_add_u32 m0, {ldsn}, {lds_imm}")
-        self._raw("s_nop 0")
+        self._m0_t = self.t - 1
+
+    def lds_direct_issue(self, goff, gbase):
+        self._need_gap(self._m0_t, 1)
         self._raw(f"global_load_lds_dwordx4 {goff}, {gbase}")
         self.stats["vmem"] = self.stats.get("vmem", 0) + 1
 
