@@ -129,6 +129,8 @@ class Emitter:
         for r in dst_regs:
             if r in self.mfma_w:
                 self._need_gap(self.mfma_w[r], 12)
+            if r in self.c_read:
+                self._need_gap(self.c_read.pop(r), 12)
             self.mfma_w.pop(r, None)
             self.valu_w.pop(r, None)
             self.trans_w.pop(r, None)

@@ -165,7 +165,7 @@ def test_dkv_tile_streams_respect_hazards():
         n = check_stream(em.out)
         assert em.stats["mfma"] == 128  # 4 q blocks x (8 S + 8 dP + 8 dv + 8 dk)
         assert n == em.stats["mfma"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
-        scratch_ok(em.out, 68, 191, 255)
+        scratch_ok(em.out, 68, 195, 255)
 
 
 def test_hazard_checker_catches_a_bad_stream():
