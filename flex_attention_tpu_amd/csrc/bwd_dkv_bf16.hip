@@ -52,7 +52,6 @@ constexpr int MAX_LIST = 1024;  // longest q tile list the plain-score kernel ca
 constexpr int LDS_BYTES = 8 * kTileElems * 2 + 4 * BQ * 4 + 4 * 32 * 4 + MAX_LIST * 5;
 }  // namespace dkv_cfg
 
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 // The register-resident state of the generated tile streams.  Every asm statement that touches it
 // names it with the same physical-register constraints, so the values stay where the streams
@@ -365,7 +364,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   // live in v[192:255] and the low registers, which the run loop leaves alone.)
   constexpr int kListRegs = MAX_LIST / 256;
   struct ItemRegs {
-    u32x4 kw[8], vw[8];            // K / V fragments of the lane's kv row
+    RowBlock k, v;                 // the wave's 32 K / V rows (full-row layout, see rows_load)
     int doc, n_tiles, qb0;         // list length and its first entry
     int idx[kListRegs];            // q list entries tid + 256 j
     unsigned char part[kListRegs]; // state of q tile tid + 256 j against this kv tile
@@ -380,13 +379,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     const int tid_here = opaque(tid);
     const bf16_t* Kg = static_cast<const bf16_t*>(a.k) + kv_offset(g);
     const bf16_t* Vg = static_cast<const bf16_t*>(a.v) + kv_offset(g);
-    const int kv_here = (tid_here >> 6) * 32 + (tid_here & 31);
-    const int hh_here = (tid_here >> 5) & 1;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      r.kw[ks] = *reinterpret_cast<const u32x4*>(Kg + (size_t)kv_here * D + ks * 16 + hh_here * 8);
-      r.vw[ks] = *reinterpret_cast<const u32x4*>(Vg + (size_t)kv_here * D + ks * 16 + hh_here * 8);
-    }
+    rows_load(r.k, Kg + (size_t)(tid_here >> 6) * 32 * D, tid_here & 63);
+    rows_load(r.v, Vg + (size_t)(tid_here >> 6) * 32 * D, tid_here & 63);
     r.doc = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_k[g.kb * BNK + kv_local] : 0;
     const int* tile_idx = a.map.idx + (size_t)g.kb * nQ;
     r.n_tiles = a.map.cnt[g.kb];
@@ -412,12 +406,17 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     const float hi = __builtin_bit_cast(float, two & 0xffff0000u) * c2;
     return __builtin_bit_cast(unsigned, pack_bf16(lo, hi));
   };
-  auto consume = [&](const ItemRegs& r, ItemHead& c) {
+  // (`stage`: the wave's 16 KB of a free LDS step buffer)
+  auto consume = [&](const ItemRegs& r, ItemHead& c, char* stage) {
+    u32x4 kw[8], vw[8];
+    const int lane_here = opaque(lane);
+    rows_to_fragments(r.k, stage, lane_here, kw);
+    rows_to_fragments(r.v, stage + 8192, lane_here, vw);
 #define FA_PUT(KS, KR, VR)                                                                                    \
   asm volatile(FA_DKV_PUT_KV_##KS                                                                             \
                : "={" KR "}"(st.k[KS]), "={" VR "}"(st.v[KS])                                                 \
-               : "v"(scaled(r.kw[KS][0])), "v"(scaled(r.kw[KS][1])), "v"(scaled(r.kw[KS][2])),                \
-                 "v"(scaled(r.kw[KS][3])), "v"(r.vw[KS][0]), "v"(r.vw[KS][1]), "v"(r.vw[KS][2]), "v"(r.vw[KS][3]));
+               : "v"(scaled(kw[KS][0])), "v"(scaled(kw[KS][1])), "v"(scaled(kw[KS][2])), "v"(scaled(kw[KS][3])), \
+                 "v"(vw[KS][0]), "v"(vw[KS][1]), "v"(vw[KS][2]), "v"(vw[KS][3]));
     FA_PUT(0, "a[128:131]", "a[160:163]") FA_PUT(1, "a[132:135]", "a[164:167]")
     FA_PUT(2, "a[136:139]", "a[168:171]") FA_PUT(3, "a[140:143]", "a[172:175]")
     FA_PUT(4, "a[144:147]", "a[176:179]") FA_PUT(5, "a[148:151]", "a[180:183]")
@@ -455,7 +454,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   ItemHead cur;
   Geometry geo = geometry(0);
   fetch(geo, pre);
-  consume(pre, cur);
+  consume(pre, cur, reinterpret_cast<char*>(sT + 4 * kTileElems) + w * 16384);
 
   for (int item = 0; item < n_items; ++item) {
   const int kb = geo.kb;
@@ -627,13 +626,13 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   // ---- item epilogue ----
   // The next item's K / V fragments go into their registers before this item's stores are issued
   // (their loads are long done; behind the stores the wait would include the stores).
-  consume(pre, cur);
+  // (buffer `buf` may hold the next item's first step: the other one is free)
+  char* stage = reinterpret_cast<char*>(sT + (size_t)(buf ^ 1) * 4 * kTileElems) + w * 16384;
+  consume(pre, cur, stage);
 
   // dk / dv: bf16 rows staged through the wave's 16 KB of the free LDS step buffer (16-byte chunks XOR-swizzled
   // by row), so that every store instruction writes four complete 256-byte rows.
   {
-    // (buffer `buf` may hold the next item's first step: the other one is free)
-    char* stage = reinterpret_cast<char*>(sT + (size_t)(buf ^ 1) * 4 * kTileElems) + w * 16384;
     const int lane_here = opaque(lane);
     const int row_here = lane_here & 31;
     const unsigned wr = (unsigned)row_here * 256u + 8u * (unsigned)(lane_here >> 5);

@@ -44,7 +44,6 @@ constexpr int MAX_LIST = 2048;
 constexpr int PLAIN_LDS_BYTES = 8 * kTileElems * 2 + 4 * 16 * 4 + MAX_LIST * 5;
 }  // namespace dq_cfg
 
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 // Register-resident state of the generated streams: every asm statement names it with the same
 // physical-register constraints, so it stays put and the compiler keeps those registers free.
@@ -310,7 +309,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   // starts after one memory round trip (its first kv tiles) instead of a chain of dependent ones.
   constexpr int kListRegs = MAX_LIST / 256;
   struct ItemRegs {
-    u32x4 qw[8], dw[8];  // Q^T / dO^T fragments of the lane's q row
+    RowBlock q, d;       // the wave's 32 Q / dO rows (full-row layout, see rows_load)
     float l, m, delta;
     int doc;
     int n_tiles, kb0, kb1;         // list length and its first two entries
@@ -326,14 +325,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   auto fetch = [&](int item, ItemRegs& r) {
     int bh, qb;
     geometry(item, bh, qb);
-    const size_t q_off = ((size_t)bh * a.Sq + (size_t)qb * BM + q_local) * D;
-    const bf16_t* Qg = static_cast<const bf16_t*>(a.q) + q_off;
-    const bf16_t* dOg = static_cast<const bf16_t*>(a.dout) + q_off;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      r.qw[ks] = *reinterpret_cast<const u32x4*>(Qg + ks * 16 + hh * 8);
-      r.dw[ks] = *reinterpret_cast<const u32x4*>(dOg + ks * 16 + hh * 8);
-    }
+    const size_t q_off = ((size_t)bh * a.Sq + (size_t)qb * BM + w * 32) * D;
+    rows_load(r.q, static_cast<const bf16_t*>(a.q) + q_off, lane);
+    rows_load(r.d, static_cast<const bf16_t*>(a.dout) + q_off, lane);
     const size_t row = (size_t)bh * a.Sq + qb * BM + q_local;
     r.l = a.l[row];
     r.m = a.m[row];
@@ -378,12 +372,16 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
     const float hi = __builtin_bit_cast(float, two & 0xffff0000u) * c2;
     return __builtin_bit_cast(unsigned, pack_bf16(lo, hi));
   };
-  auto consume = [&](const ItemRegs& r, ItemHead& c) {
+  // (`stage`: the wave's 16 KB of a free LDS step buffer)
+  auto consume = [&](const ItemRegs& r, ItemHead& c, char* stage) {
+    u32x4 qw[8], dw[8];
+    rows_to_fragments(r.q, stage, lane, qw);
+    rows_to_fragments(r.d, stage + 8192, lane, dw);
 #define FA_PUT(KS, QR, DR)                                                                                    \
   asm volatile(FA_DQ_PUT_##KS                                                                                 \
                : "={" QR "}"(st.q[KS]), "={" DR "}"(st.d[KS])                                                 \
-               : "v"(scaled(r.qw[KS][0])), "v"(scaled(r.qw[KS][1])), "v"(scaled(r.qw[KS][2])),                \
-                 "v"(scaled(r.qw[KS][3])), "v"(r.dw[KS][0]), "v"(r.dw[KS][1]), "v"(r.dw[KS][2]), "v"(r.dw[KS][3]));
+               : "v"(scaled(qw[KS][0])), "v"(scaled(qw[KS][1])), "v"(scaled(qw[KS][2])), "v"(scaled(qw[KS][3])), \
+                 "v"(dw[KS][0]), "v"(dw[KS][1]), "v"(dw[KS][2]), "v"(dw[KS][3]));
     FA_PUT(0, "a[64:67]", "a[96:99]") FA_PUT(1, "a[68:71]", "a[100:103]") FA_PUT(2, "a[72:75]", "a[104:107]")
     FA_PUT(3, "a[76:79]", "a[108:111]") FA_PUT(4, "a[80:83]", "a[112:115]") FA_PUT(5, "a[84:87]", "a[116:119]")
     FA_PUT(6, "a[88:91]", "a[120:123]") FA_PUT(7, "a[92:95]", "a[124:127]")
@@ -408,7 +406,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   ItemRegs pre;
   ItemHead cur;
   fetch(0, pre);
-  consume(pre, cur);
+  consume(pre, cur, reinterpret_cast<char*>(sT + 4 * kTileElems) + w * 16384);
   for (int item = 0; item < n_items; ++item) {
     int bh, qb;
     geometry(item, bh, qb);
@@ -555,13 +553,13 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
     // ---- item epilogue ----
     // The next item's Q^T / dO^T fragments go into their registers before this item's stores are
     // issued (their loads are long done; behind the stores the wait would include the stores).
-    consume(pre, cur);
-
-    // dq: bf16 rows staged through the wave's 8 KB of the free LDS step buffer (16-byte chunks
-    // XOR-swizzled by row), so that every store instruction writes four complete 256-byte rows.
     // (Buffer `buf` may hold the next item's first step: the other one is free.)
+    char* stage = reinterpret_cast<char*>(sT + (size_t)(buf ^ 1) * 4 * kTileElems) + w * 16384;
+    consume(pre, cur, stage);
+
+    // dq: bf16 rows staged through the same wave-private LDS (16-byte chunks XOR-swizzled by row), so
+    // that every store instruction writes four complete 256-byte rows.
     {
-      char* stage = reinterpret_cast<char*>(sT + (size_t)(buf ^ 1) * 4 * kTileElems) + w * 8192;
       const int lane_here = opaque(lane);
       const int row_here = lane_here & 31;
       const unsigned wr = (unsigned)row_here * 256u + 8u * (unsigned)(lane_here >> 5);

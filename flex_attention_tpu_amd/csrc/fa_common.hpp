@@ -125,6 +125,38 @@ __device__ __forceinline__ bf16x2 pack_bf16(float a, float b) {
 }
 
 // ------------------------------------------------------------------------------------------
+// Row fragments of a wave's 32 x 128 bf16 block for the transposed MFMA formulations: lane
+// (l32 = lane & 31, hh = lane >> 5) needs the 16-byte chunks 2 ks + hh, ks = 0..7, of row l32.
+// Loading them directly makes every load instruction touch 32 cache lines; instead the block is
+// fetched with full-row loads (rows_load: four complete rows per instruction) and redistributed
+// through 8 KB of wave-private LDS when it is needed (rows_to_fragments; 16-byte chunks
+// XOR-swizzled by row: conflict-free both ways).
+// ------------------------------------------------------------------------------------------
+struct RowBlock {
+  u32x4 v[8];
+};
+__device__ __forceinline__ void rows_load(RowBlock& r, const bf16_t* block, int lane) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    r.v[i] = *reinterpret_cast<const u32x4*>(block + (size_t)(4 * i + (lane >> 4)) * 128 + (lane & 15) * 8);
+}
+__device__ __forceinline__ void rows_to_fragments(const RowBlock& r, char* stage, int lane, u32x4 (&frag)[8]) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = 4 * i + (lane >> 4);
+    *reinterpret_cast<u32x4*>(stage + row * 256 + (((lane & 15) ^ (row & 15)) << 4)) = r.v[i];
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  const int l32 = lane & 31, hh = lane >> 5;
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks)
+    frag[ks] = *reinterpret_cast<const u32x4*>(stage + l32 * 256 + (((2 * ks + hh) ^ (l32 & 15)) << 4));
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+// ------------------------------------------------------------------------------------------
 // Element mask, evaluated only on tiles the block map marks partial.
 // ------------------------------------------------------------------------------------------
 __device__ __forceinline__ bool keep_elem(const MaskArgs& mk, int i, int j, int doc_i, int doc_j) {

@@ -47,7 +47,6 @@ constexpr int MAX_LIST = 1024;
 constexpr int PLAIN_LDS_BYTES = 8 * kTileElems * 2 + 4 * 16 * 4 + 16 + MAX_LIST * 4 + 2 * MAX_LIST;
 }  // namespace fwd_cfg
 
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 // Register-resident state of the generated streams: every asm statement names it with the same
 // physical-register constraints, so it stays put and the compiler keeps those registers free.
@@ -404,7 +403,7 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
   constexpr int kListRegs = MAX_LIST / 256;
   static_assert(kListRegs <= 4, "the packed state words hold four tiles per lane");
   struct ItemRegs {
-    u32x4 qw[2][8];     // Q^T fragments of the lane's two q rows
+    RowBlock q[2];      // the wave's 32 Q rows of each q tile (full-row layout, see rows_load)
     int doc[2];
     unsigned sa, sb;    // byte j: state of kv tile tid + 256 j in the state row of q tile 0 / 1
     unsigned head;      // states of kv tile `lane` in both rows: where the merged list starts
@@ -421,13 +420,12 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
     const int tid_here = opaque(tid);
     const int lane_here = tid_here & 63;
     const int row_here = (tid_here >> 6) * 32 + (lane_here & 31);
+    const int w_here = tid_here >> 6;
     r.sa = r.sb = r.head = 0u;
 #pragma unroll
     for (int x = 0; x < 2; ++x) {
       const int qb = min(2 * qb2 + x, nQ - 1);  // (a missing second tile repeats the first; nothing of it is stored)
-      const bf16_t* Qg = static_cast<const bf16_t*>(a.q) + ((size_t)bh * a.Sq + (size_t)qb * BM + row_here) * D;
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) r.qw[x][ks] = *reinterpret_cast<const u32x4*>(Qg + ks * 16 + (lane_here >> 5) * 8);
+      rows_load(r.q[x], static_cast<const bf16_t*>(a.q) + ((size_t)bh * a.Sq + (size_t)qb * BM + w_here * 32) * D, lane_here);
       r.doc[x] = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[qb * BM + row_here] : 0;
       const uint8_t* row = a.map.state + (size_t)qb * nK;
       const bool valid = 2 * qb2 + x < nQ;
@@ -456,13 +454,17 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
     const float hi = __builtin_bit_cast(float, two & 0xffff0000u) * c2;
     return __builtin_bit_cast(unsigned, pack_bf16(lo, hi));
   };
-  auto consume = [&](const ItemRegs& r, ItemHead& c) {
+  // (`stage`: the wave's 16 KB of a free LDS step buffer)
+  auto consume = [&](const ItemRegs& r, ItemHead& c, char* stage) {
+    u32x4 q0[8], q1[8];
+    const int lane_here = opaque(lane);
+    rows_to_fragments(r.q[0], stage, lane_here, q0);
+    rows_to_fragments(r.q[1], stage + 8192, lane_here, q1);
 #define FA_PUT(KS, Q0, Q1)                                                                                        \
   asm volatile(FA_FWD_PUT_##KS                                                                                    \
                : "={" Q0 "}"(st.q[KS]), "={" Q1 "}"(st.q[8 + KS])                                                 \
-               : "v"(scaled(r.qw[0][KS][0])), "v"(scaled(r.qw[0][KS][1])), "v"(scaled(r.qw[0][KS][2])),           \
-                 "v"(scaled(r.qw[0][KS][3])), "v"(scaled(r.qw[1][KS][0])), "v"(scaled(r.qw[1][KS][1])),           \
-                 "v"(scaled(r.qw[1][KS][2])), "v"(scaled(r.qw[1][KS][3])));
+               : "v"(scaled(q0[KS][0])), "v"(scaled(q0[KS][1])), "v"(scaled(q0[KS][2])), "v"(scaled(q0[KS][3])),  \
+                 "v"(scaled(q1[KS][0])), "v"(scaled(q1[KS][1])), "v"(scaled(q1[KS][2])), "v"(scaled(q1[KS][3])));
     FA_PUT(0, "a[128:131]", "a[160:163]") FA_PUT(1, "a[132:135]", "a[164:167]") FA_PUT(2, "a[136:139]", "a[168:171]")
     FA_PUT(3, "a[140:143]", "a[172:175]") FA_PUT(4, "a[144:147]", "a[176:179]") FA_PUT(5, "a[148:151]", "a[180:183]")
     FA_PUT(6, "a[152:155]", "a[184:187]") FA_PUT(7, "a[156:159]", "a[188:191]")
@@ -476,7 +478,7 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
   ItemRegs pre;
   ItemHead cur;
   fetch(0, pre);
-  consume(pre, cur);
+  consume(pre, cur, reinterpret_cast<char*>(sT + 4 * kTileElems) + w * 16384);
   for (int item = 0; item < n_items; ++item) {
     int bh, qb2;
     geometry(item, bh, qb2);
@@ -664,14 +666,14 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
     // ---- item epilogue ----
     // The next item's Q^T fragments go into their registers before this item's stores are issued
     // (their loads are long done; behind the stores the wait would include the stores).
-    consume(pre, cur);
+    // (Buffer `buf` may hold the next item's first step: the other one is free.)
+    char* stage = reinterpret_cast<char*>(sT + (size_t)(buf ^ 1) * 4 * kTileElems) + w * 16384;
+    consume(pre, cur, stage);
 
-    // O = O^T / l as bf16 rows, staged through the wave's 16 KB of the free LDS step buffer (16-byte
-    // chunks XOR-swizzled by row) so that every store instruction writes four complete 256-byte rows;
-    // exact (l, m) from the reference-maximum bookkeeping.  (Buffer `buf` may hold the next item's
-    // first step: the other one is free.)
+    // O = O^T / l as bf16 rows, staged through the same wave-private LDS (16-byte chunks XOR-swizzled
+    // by row) so that every store instruction writes four complete 256-byte rows; exact (l, m) from
+    // the reference-maximum bookkeeping.
     {
-      char* stage = reinterpret_cast<char*>(sT + (size_t)(buf ^ 1) * 4 * kTileElems) + w * 16384;
       const int lane_here = opaque(lane);
       const int row_here = lane_here & 31;
       const unsigned wr = (unsigned)row_here * 256u + 8u * (unsigned)(lane_here >> 5);
