@@ -19,7 +19,7 @@
 
 #include <type_traits>
 
-// v[68:195] and a[192:255] belong to the generated tile streams
+// v[68:199] and a[192:255] belong to the generated tile streams
 #define FA_DKV_TILE_CLOBBERS "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79", "v80", "v81", "v82", \
   "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", \
   "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", \
@@ -29,12 +29,12 @@
   "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", \
   "v163", "v164", "v165", "v166", "v167", "v168", "v169", "v170", "v171", "v172", "v173", "v174", "v175", \
   "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", "v185", "v186", "v187", "v188", \
-  "v189", "v190", "v191", "v192", "v193", "v194", "v195", "a192", "a193", "a194", "a195", "a196", "a197", \
-  "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205", "a206", "a207", "a208", "a209", "a210", \
-  "a211", "a212", "a213", "a214", "a215", "a216", "a217", "a218", "a219", "a220", "a221", "a222", "a223", \
-  "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231", "a232", "a233", "a234", "a235", "a236", \
-  "a237", "a238", "a239", "a240", "a241", "a242", "a243", "a244", "a245", "a246", "a247", "a248", "a249", \
-  "a250", "a251", "a252", "a253", "a254", "a255"
+  "v189", "v190", "v191", "v192", "v193", "v194", "v195", "v196", "v197", "v198", "v199", "a192", "a193", \
+  "a194", "a195", "a196", "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205", "a206", \
+  "a207", "a208", "a209", "a210", "a211", "a212", "a213", "a214", "a215", "a216", "a217", "a218", "a219", \
+  "a220", "a221", "a222", "a223", "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231", "a232", \
+  "a233", "a234", "a235", "a236", "a237", "a238", "a239", "a240", "a241", "a242", "a243", "a244", "a245", \
+  "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255"
 
 // scalar registers of the generated run loop
 #define FA_DKV_RUN_SGPRS "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", "s87", "s88", "s89", "s90", "s91", "s92", "s93", "s94", "s95", "s96", "s97", "s98", "s99", "s100"
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   const int n_items = n_wg / (int)gridDim.x;
   const int kv_local = w * 32 + l32;
   const int row = tid & (BQ - 1);
-  // waves 0, 1 turn (l, m) into -lse for rows tid & 127; waves 2, 3 pass delta through
+  // waves 0, 1 turn (l, m) into -lse for rows tid & 127; waves 2, 3 store -delta
   const bool lse_wave = w < 2;
   int* sIdx = reinterpret_cast<int*>(sDl + 2 * BQ) + 4 * 32;
   unsigned char* sPart = reinterpret_cast<unsigned char*>(sIdx + MAX_LIST);  // by q tile: 1 = partial with this kv tile
@@ -499,8 +499,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     const float x = rowa[r0 + row_p], y = rowb[r0 + row_p];
     if (lse_wave) {  // (the streams want -lse: it is the accumulator input of the S chain)
       sLse[buf * BQ + row_p] = (x > 0.f) ? -__builtin_fmaf(y, kLog2e, log2f(x)) : -__builtin_huge_valf();
-    } else {
-      sDl[buf * BQ + row_p] = x;
+    } else {  // (and -delta, for the dP chain)
+      sDl[buf * BQ + row_p] = -x;
     }
     wait_vmem_all();
   }

@@ -9,10 +9,10 @@ per SIMD, so MFMA, VALU and LDS work only overlap if they are interleaved inside
 register budget only closes with a fixed allocation.  The stream below is a software pipeline over
 the tile's four 32-row q blocks c = 0..3:
 
-    A(c): S' = Q K^T - lse, dP = dO V^T  16 MFMAs, operands: 16 ds_read_b128 (rows of Q, dO)
-          (K arrives multiplied by sm_scale log2 e and LDS holds -lse, which enters through the
-          accumulator input of the chain's first MFMA: the result is already the exponent)
-    E(c): P = exp2(S'), dS = P (dP - delta)   64 VALU ops, 8 ds_read_b128 (-lse ahead of A(c), delta)
+    A(c): S' = Q K^T - lse, dP' = dO V^T - delta  16 MFMAs, operands: 16 ds_read_b128 (rows of Q, dO)
+          (K arrives multiplied by sm_scale log2 e and LDS holds -lse and -delta, which enter through
+          the accumulator input of each chain's first MFMA: S' is already the exponent)
+    E(c): P = exp2(S'), dS = P dP'       48 VALU ops; 8 ds_read_b128 (-lse, -delta) ahead of A(c)
     B(c): dv^T += dO^T P, dk^T += Q^T dS 16 MFMAs, operands: 32 ds_read_b64_tr_b16
 
     MFMA order:  A0 | A1 | A2 B0 | A3 B1 | B2 | B3      VALU:  - | E0 | E1 | E2 | E3 | -
@@ -25,7 +25,7 @@ Register contract with the C++ side (every asm statement names the accumulation 
 physical-register constraints; prologue / epilogue macros are generated here too):
     a[0:63]    dv accumulators (4 x 16)      a[64:127]  dk accumulators (4 x 16)
     a[128:159] K fragments (8 x 4), pre-scaled   a[160:191] V fragments (8 x 4)
-    v[67:195]  scratch of the run loop and its streams (clobbered), s[60:100], vcc, m0 likewise
+    v[67:199]  scratch of the run loop and its streams (clobbered), s[60:100], vcc, m0 likewise
     a[192:255] staging slots of the LDS fragments (clobbered): MFMA operands only, so they can be
                AGPRs, and v[192:255] stay with the compiler for what lives across the run loop
     %[r0..r7]  byte address of the lane's row fragment ks in the step's Q half-tile 0
@@ -39,7 +39,7 @@ physical-register constraints; prologue / epilogue macros are generated here too
     %[m0], %[m1]  (masked stream only) the lane's keep bits: bit 16 (c & 1) + e of m[c >> 1] is
                element e of the S accumulator of q block c; dropped elements get P = 0
 LDS layout of one step buffer (bytes): Q half 0, Q half 1, dO half 0, dO half 1 (16 KiB each);
--lse [128] floats, delta 1 KiB after it.
+-lse [128] floats, -delta 1 KiB after it.
 """
 import argparse
 import os
@@ -80,7 +80,7 @@ V_DP = [88, 120]
 V_PB = 136
 V_DSB = 152
 V_LSE = 168   # -lse of the 16 q rows of a block: accumulator input of the first MFMA of its S chain
-V_DL = 184    # 3 buffers x 4
+V_DL = 184    # -delta of the 16 q rows of a block, for the dP chain likewise
 A_STG = 192   # 8 staging slots x 8 registers for LDS fragments: AGPRs, which leaves v[192:255] to the compiler
 V_TMP = 68    # 4 temporaries of the masked variant
 DL_OFFSET = 1024
@@ -135,12 +135,12 @@ def build(masked):
             ks = x
             s, dp = V_S[c & 1], V_DP[c & 1]
             cin = V_LSE if ks == 0 else s
-            cd = "0" if ks == 0 else vr(dp, 16)
+            cdn = V_DL if ks == 0 else dp
             return [
                 (vr(s, 16), ar(base, 4), ar(128 + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(base, 4), aset(128 + 4 * ks, 4),
                  vset(cin, 16)),
-                (vr(dp, 16), ar(base + 4, 4), ar(160 + 4 * ks, 4), cd, vset(dp, 16), aset(base + 4, 4),
-                 aset(160 + 4 * ks, 4), set() if ks == 0 else vset(dp, 16)),
+                (vr(dp, 16), ar(base + 4, 4), ar(160 + 4 * ks, 4), vr(cdn, 16), vset(dp, 16), aset(base + 4, 4),
+                 aset(160 + 4 * ks, 4), vset(cdn, 16)),
             ]
         u, db = x
         pb = V_PB + 8 * (c & 1) + 4 * u
@@ -161,8 +161,6 @@ def build(masked):
         ops = []
         group_first_op = []
         for g in range(4):
-            kbuf = (4 * c + g) % 3
-            dl = V_DL + 4 * kbuf
             group_first_op.append(len(ops))
             for u in range(4):
                 e = 4 * g + u
@@ -179,9 +177,6 @@ def build(masked):
                     ops.append((f"v_and_b32_e32 {vr(s + e)}, {vr(s + e)}, {vr(tmp)}", vset(s + e), vset(s + e) | vset(tmp), False))
             for u in range(4):
                 e = 4 * g + u
-                ops.append((f"v_sub_f32_e32 {vr(dp + e)}, {vr(dp + e)}, {vr(dl + u)}", vset(dp + e), vset(dp + e) | vset(dl + u), False))
-            for u in range(4):
-                e = 4 * g + u
                 ops.append((f"v_mul_f32_e32 {vr(dp + e)}, {vr(s + e)}, {vr(dp + e)}", vset(dp + e), vset(dp + e) | vset(s + e), False))
             # bf16x8 operand u2 = g >> 1, registers 2 (g & 1) + {0, 1} hold elements (0,1), (2,3) of the group
             pb = V_PB + 8 * (c & 1) + 4 * (g >> 1) + 2 * (g & 1)
@@ -196,28 +191,16 @@ def build(masked):
         op_slot = [first + (i * span) // len(ops) for i in range(len(ops))]
         for i, op in enumerate(ops):
             slot_valu[op_slot[i]].append(op)
-        # -lse of block c: in place well before the first MFMA of A(c), one stage ahead of E(c) (the
-        # registers were last read by the first MFMA of A(c - 1), a whole stage earlier)
+        # -lse and -delta of block c: in place well before the first MFMAs of A(c), one stage ahead of
+        # E(c) (the registers were last read by the first MFMAs of A(c - 1), a whole stage earlier)
         rd = [(f"ds_read_b128 {vr(V_LSE + 4 * g, 4)}, %[la] offset:{(32 * c + 8 * g) * 4}", vset(V_LSE + 4 * g, 4)) for g in range(4)]
+        rd += [(f"ds_read_b128 {vr(V_DL + 4 * g, 4)}, %[la] offset:{(32 * c + 8 * g) * 4 + DL_OFFSET}", vset(V_DL + 4 * g, 4))
+               for g in range(4)]
         if c == 0:
             pre_lds.extend(rd)
         else:
             at = (stage_first_slot[c - 1] if c > 1 else 16) - 10
             slot_lds[at].extend(rd)
-        for g in range(4):
-            kbuf = (4 * c + g) % 3
-            dl = V_DL + 4 * kbuf
-            off = (32 * c + 8 * g) * 4
-            rd = [(f"ds_read_b128 {vr(dl, 4)}, %[la] offset:{off + DL_OFFSET}", vset(dl, 4))]
-            # issue when the previous group starts (three buffers: the one reloaded here was last read two groups ago)
-            if g > 0:
-                at = op_slot[group_first_op[g - 1]]
-            else:
-                at = first - 4
-            if at < 0:
-                pre_lds.extend(rd)
-            else:
-                slot_lds[at].extend(rd)
 
     # ---- LDS reads of the MFMA pairs, PREFETCH pairs ahead ---------------------------------
     for k in range(len(pairs)):
@@ -249,8 +232,8 @@ def build(masked):
         if m == ROW_SLOT and 'vmem' not in DROP:
             # The two per-row values this lane fetched at the top of the step (older than every
             # LDS-direct load) have arrived once at most n_direct vector-memory operations are open.
-            # Waves 0, 1: (l, m) -> -lse = -m log2(e) - log2(l), -inf where l = 0; waves 2, 3: delta
-            # passes through (%[lsew] is non-zero resp. zero).  One LDS store into the next buffer.
+            # Waves 0, 1: (l, m) -> -lse = -m log2(e) - log2(l), -inf where l = 0; waves 2, 3: -delta
+            # (%[lsew] is non-zero resp. zero).  One LDS store into the next buffer.
             ra_, rb_, rt_, inf_ = V_ROW, V_ROW + 1, V_ROW + 2, V_ROW + 3
             em.raw(f"s_waitcnt vmcnt({n_direct})")
             em.valu(f"v_log_f32_e32 {vr(rt_)}, {vr(ra_)}", vset(rt_), vset(ra_), True)
@@ -262,6 +245,7 @@ def build(masked):
             em.raw("s_cmp_lg_u32 s65, 0")
             em.raw("s_cselect_b64 vcc, -1, 0")
             em.raw("s_nop 3")
+            em.valu(f"v_xor_b32_e32 {vr(ra_)}, 0x80000000, {vr(ra_)}", vset(ra_), vset(ra_))
             em.valu(f"v_cndmask_b32_e32 {vr(rt_)}, {vr(ra_)}, {vr(rt_)}, vcc", vset(rt_), vset(rt_) | vset(ra_))
             em.lds_write(f"ds_write_b32 %[lw], {vr(rt_)}", vset(rt_))
         lds = slot_lds[m]

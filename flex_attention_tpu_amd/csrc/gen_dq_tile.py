@@ -6,10 +6,10 @@ statements: the run loop over steps of two 64-row kv tiles, and prologue / epilo
 A wave owns 32 q rows (Q^T, dO^T fragments and the dq^T accumulators stay in accumulation
 registers); one step covers 128 kv rows = four 32-row kv blocks c = 0..3, software-pipelined:
 
-    A(c): S'^T = K Q^T - lse, dP^T = V dO^T  16 MFMAs, operands: 16 ds_read_b128 (rows of K, V)
-          (Q arrives multiplied by sm_scale log2 e, and -lse enters through the accumulator input of
-          the chain's first MFMA, so the result is already the exponent)
-    E(c): dS^T = exp2(S'^T) (dP^T - delta)   56 VALU ops
+    A(c): S'^T = K Q^T - lse, dP'^T = V dO^T - delta  16 MFMAs, operands: 16 ds_read_b128 (rows of K, V)
+          (Q arrives multiplied by sm_scale log2 e; -lse and -delta enter through the accumulator
+          input of each chain's first MFMA, so S' is already the exponent)
+    E(c): dS^T = exp2(S'^T) dP'^T            40 VALU ops
     B(c): dq^T += K^T dS^T                  8 MFMAs, operands: 16 ds_read_b64_tr_b16 (K again)
 
     MFMA order:  A0 | A1 | A2 B0 | A3 B1 | B2 | B3      VALU:  - | E0 | E1 | E2 | E3 | -
@@ -22,7 +22,7 @@ Register contract with the C++ side (every asm statement names the accumulation 
 physical-register constraints):
     a[0:63]   dq^T accumulators (4 x 16)   a[64:95] Q^T fragments (8 x 4), pre-scaled   a[96:127] dO^T fragments
     a[128:191] staging slots of the LDS fragments (clobbered)
-    v[66:167], s[60:100], vcc, m0   scratch of the run loop (clobbered)
+    v[66:183], s[60:100], vcc, m0   scratch of the run loop (clobbered)
     (the table also names the next work item's first step, copied into LDS during this item's last step)
     %[r0..r7]  byte address of the lane's row fragment ks in K half-tile 0 of the current buffer
     %[t0..t7]  byte address of the lane's transposed fragment (2 db + hi) in K half-tile 0
@@ -71,7 +71,8 @@ V_S = [72, 104]
 V_DP = [88, 120]
 V_DS = 136       # dS^T as MFMA B operands: [c & 1][u] x 4 registers
 V_NL = 152       # -lse of the lane's q row, 16 copies: accumulator input of the first MFMA of an S chain
-V_END = 167
+V_ND = 168       # -delta of the lane's q row, 16 copies: accumulator input of the first MFMA of a dP chain
+V_END = 183
 A_DQ, A_Q, A_DO, A_STG = 0, 64, 96, 128
 
 
@@ -124,11 +125,11 @@ def build(masked):
             ks = x
             s, dp = V_S[c & 1], V_DP[c & 1]
             cin = V_NL if ks == 0 else s
-            cd = "0" if ks == 0 else vr(dp, 16)
+            cdn = V_ND if ks == 0 else dp
             return [(vr(s, 16), ar(base, 4), ar(A_Q + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(base, 4), aset(A_Q + 4 * ks, 4),
                      vset(cin, 16)),
-                    (vr(dp, 16), ar(base + 4, 4), ar(A_DO + 4 * ks, 4), cd, vset(dp, 16), aset(base + 4, 4),
-                     aset(A_DO + 4 * ks, 4), set() if ks == 0 else vset(dp, 16))]
+                    (vr(dp, 16), ar(base + 4, 4), ar(A_DO + 4 * ks, 4), vr(cdn, 16), vset(dp, 16), aset(base + 4, 4),
+                     aset(A_DO + 4 * ks, 4), vset(cdn, 16))]
         u, j = x
         ds = V_DS + 8 * (c & 1) + 4 * u
         out = []
@@ -158,9 +159,6 @@ def build(masked):
                     e = 4 * g + u
                     ops.append((f"v_and_b32_e32 {vr(s + e)}, {vr(s + e)}, {vr(V_TMP + u)}", vset(s + e),
                                 vset(s + e) | vset(V_TMP + u), False))
-            for u in range(4):
-                e = 4 * g + u
-                ops.append((f"v_sub_f32_e32 {vr(dp + e)}, {vr(dp + e)}, %[dl]", vset(dp + e), vset(dp + e), False))
             for u in range(4):
                 e = 4 * g + u
                 ops.append((f"v_mul_f32_e32 {vr(dp + e)}, {vr(s + e)}, {vr(dp + e)}", vset(dp + e), vset(dp + e) | vset(s + e), False))
@@ -219,6 +217,7 @@ def run_loop(full, masked):
     entry += [f"v_readfirstlane_b32 {S[n]}, {vr(V_TBL + i)}" for i, n in enumerate(TABLE)]
     entry += [f"v_readfirstlane_b32 {S[n]}, %[{n}]" for n in STATE_IO + STATE_IN]
     entry += [f"v_sub_f32_e32 {vr(V_NL + e)}, 0, %[lse]" for e in range(16)]
+    entry += [f"v_sub_f32_e32 {vr(V_ND + e)}, 0, %[dl]" for e in range(16)]
     top = entry + [".Lfa_dq_loop_%=:"]
     # On the item's last step the tiles copied "for the next step" are the first step of the next
     # work item (its kv tiles and K / V bases come from the table; with no next item they repeat

@@ -165,7 +165,7 @@ def test_dkv_tile_streams_respect_hazards():
         n = check_stream(em.out)
         assert em.stats["mfma"] == 128  # 4 q blocks x (8 S + 8 dP + 8 dv + 8 dk)
         assert n == em.stats["mfma"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
-        scratch_ok(em.out, 68, 195, 255)
+        scratch_ok(em.out, 68, 199, 255)
 
 
 def test_hazard_checker_catches_a_bad_stream():
@@ -225,7 +225,7 @@ def test_dq_tile_streams_respect_hazards():
         n = check_stream(em.out)
         assert em.stats["mfma"] == 96  # 4 kv blocks x (8 S + 8 dP + 8 dq)
         assert n == em.stats["mfma"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
-        scratch_ok(em.out, 66, 167, 191)
+        scratch_ok(em.out, 66, 183, 191)
 
 
 def test_fwd_tile_streams_respect_hazards():
