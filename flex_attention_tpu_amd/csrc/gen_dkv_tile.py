@@ -46,12 +46,13 @@ import os
 import sys
 
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
-from gfx950_stream import Emitter, ar, aset, vr, vset  # noqa: E402
+from gfx950_stream import Emitter, Op, ar, aset, schedule, vr, vset  # noqa: E402
 
 NSLOT = 8        # staging slots of 8 registers
-PREFETCH = 4     # MFMA pairs between the LDS reads of a pair and its MFMAs
-LOAD_FIRST = 2   # MFMA slot of the first LDS-direct load of the next step
-LOAD_EVERY = 6   # slots between two of them
+MIN_AHEAD = 2    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
+CAP = 4          # instructions the scheduler puts between two MFMAs unless deadlines force more
+LOAD_FIRST = 2   # MFMA gap from which the first LDS-direct load of the next step may go out
+LOAD_EVERY = 6   # gaps between two of them
 DROP = ()        # instruction classes left out (--drop, timing studies only)
 
 TILE = 16384
@@ -98,15 +99,15 @@ def build(masked):
         for u in range(2):
             for db in range(4):
                 pairs.append(("B", c, (u, db)))
-    add_A(0)
-    stage_first_slot = {}
-    stage_first_slot[0] = 2 * len(pairs); add_A(1)
-    stage_first_slot[1] = 2 * len(pairs); add_A(2); add_B(0)
-    stage_first_slot[2] = 2 * len(pairs); add_A(3); add_B(1)
-    stage_first_slot[3] = 2 * len(pairs); add_B(2)
-    stage_end = 2 * len(pairs); add_B(3)
-    n_slots = 2 * len(pairs)
-    stage_last_slot = {0: stage_first_slot[1], 1: stage_first_slot[2], 2: stage_first_slot[3], 3: stage_end}
+    add_A(0); add_A(1); add_A(2); add_B(0); add_A(3); add_B(1); add_B(2); add_B(3)
+    n_mfma = 2 * len(pairs)
+    idx = {}  # (kind, c, x) -> number of the pair's first MFMA
+    for k, key in enumerate(pairs):
+        idx[key] = 2 * k
+    first_A = {c: idx[("A", c, 0)] for c in range(4)}
+    last_A = {c: idx[("A", c, 7)] + 1 for c in range(4)}
+    first_B = {(c, u): idx[("B", c, (u, 0))] for c in range(4) for u in range(2)}
+    last_B = {(c, u): idx[("B", c, (u, 3))] + 1 for c in range(4) for u in range(2)}
 
     def half_off(c):
         return (c >> 1) * TILE + (c & 1) * (TILE // 2)
@@ -152,114 +153,122 @@ def build(masked):
              aset(base + 4, 4), vset(dsb, 4), aset(64 + 16 * db, 16)),
         ]
 
-    # ---- VALU work of E(c), spread over the MFMA slots of stage c ---------------------------
-    slot_valu = {m: [] for m in range(n_slots)}
-    slot_lds = {m: [] for m in range(n_slots)}
-    pre_lds = []
+    mfmas = [pair_mfmas(k)[j] for k in range(len(pairs)) for j in range(2)]
+    if "mfma" in DROP:
+        mfmas = []
+        n_gaps = n_mfma
+
+    def valu(text, dst, src, trans=False, **kw):
+        return Op((lambda e: e.valu(text, dst, src, trans)) if "valu" not in DROP else (lambda e: None), **kw)
+
+    def lds(text, dst, **kw):
+        return Op((lambda e: e.lds_read(text, dst)) if "lds" not in DROP else (lambda e: None), **kw)
+
+    chains = []
+    # ---- E(c): element-wise work between the block's S / dP chains and its B products -------
     for c in range(4):
         s, dp = V_S[c & 1], V_DP[c & 1]
         ops = []
-        group_first_op = []
         for g in range(4):
-            group_first_op.append(len(ops))
             for u in range(4):
                 e = 4 * g + u
-                ops.append((f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
+                ops.append(valu(f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
             if masked:
                 # keep bit of element e of block c: bit 16 (c & 1) + e of %[m0] (c < 2) or %[m1]
                 for u in range(4):
                     e = 4 * g + u
                     tmp = V_TMP + u
-                    ops.append((f"v_bfe_i32 {vr(tmp)}, %[m{c >> 1}], {16 * (c & 1) + e}, 1", vset(tmp), set(), False))
+                    ops.append(valu(f"v_bfe_i32 {vr(tmp)}, %[m{c >> 1}], {16 * (c & 1) + e}, 1", vset(tmp), set()))
                 for u in range(4):
                     e = 4 * g + u
                     tmp = V_TMP + u
-                    ops.append((f"v_and_b32_e32 {vr(s + e)}, {vr(s + e)}, {vr(tmp)}", vset(s + e), vset(s + e) | vset(tmp), False))
+                    ops.append(valu(f"v_and_b32_e32 {vr(s + e)}, {vr(s + e)}, {vr(tmp)}", vset(s + e), vset(s + e) | vset(tmp)))
             for u in range(4):
                 e = 4 * g + u
-                ops.append((f"v_mul_f32_e32 {vr(dp + e)}, {vr(s + e)}, {vr(dp + e)}", vset(dp + e), vset(dp + e) | vset(s + e), False))
-            # bf16x8 operand u2 = g >> 1, registers 2 (g & 1) + {0, 1} hold elements (0,1), (2,3) of the group
-            pb = V_PB + 8 * (c & 1) + 4 * (g >> 1) + 2 * (g & 1)
-            dsb = V_DSB + 8 * (c & 1) + 4 * (g >> 1) + 2 * (g & 1)
+                ops.append(valu(f"v_mul_f32_e32 {vr(dp + e)}, {vr(s + e)}, {vr(dp + e)}", vset(dp + e), vset(dp + e) | vset(s + e)))
+            # bf16x8 operand u2 = g >> 1, registers 2 (g & 1) + {0, 1} hold elements (0,1), (2,3) of the group.
+            # The registers are those of block c - 2: its B MFMAs that read them must have been issued;
+            # and this block's B MFMAs of half u2 wait for them.
+            u2 = g >> 1
+            pb = V_PB + 8 * (c & 1) + 4 * u2 + 2 * (g & 1)
+            dsb = V_DSB + 8 * (c & 1) + 4 * u2 + 2 * (g & 1)
+            war = last_B[(c - 2, u2)] + 1 if c >= 2 else 0
             for h in range(2):
                 e = 4 * g + 2 * h
-                ops.append((f"v_cvt_pk_bf16_f32 {vr(pb + h)}, {vr(s + e)}, {vr(s + e + 1)}", vset(pb + h), vset(s + e, 2), False))
-                ops.append((f"v_cvt_pk_bf16_f32 {vr(dsb + h)}, {vr(dp + e)}, {vr(dp + e + 1)}", vset(dsb + h), vset(dp + e, 2), False))
-        first = stage_first_slot[c] + (6 if c == 0 else 0)  # E(0) directly follows A(0): give its results time
-        last = stage_last_slot[c]
-        span = last - first
-        op_slot = [first + (i * span) // len(ops) for i in range(len(ops))]
-        for i, op in enumerate(ops):
-            slot_valu[op_slot[i]].append(op)
-        # -lse and -delta of block c: in place well before the first MFMAs of A(c), one stage ahead of
-        # E(c) (the registers were last read by the first MFMAs of A(c - 1), a whole stage earlier)
-        rd = [(f"ds_read_b128 {vr(V_LSE + 4 * g, 4)}, %[la] offset:{(32 * c + 8 * g) * 4}", vset(V_LSE + 4 * g, 4)) for g in range(4)]
-        rd += [(f"ds_read_b128 {vr(V_DL + 4 * g, 4)}, %[la] offset:{(32 * c + 8 * g) * 4 + DL_OFFSET}", vset(V_DL + 4 * g, 4))
-               for g in range(4)]
-        if c == 0:
-            pre_lds.extend(rd)
-        else:
-            at = (stage_first_slot[c - 1] if c > 1 else 16) - 10
-            slot_lds[at].extend(rd)
+                ops.append(valu(f"v_cvt_pk_bf16_f32 {vr(pb + h)}, {vr(s + e)}, {vr(s + e + 1)}", vset(pb + h), vset(s + e, 2),
+                                earliest=war, deadline=first_B[(c, u2)] - 1))
+                ops.append(valu(f"v_cvt_pk_bf16_f32 {vr(dsb + h)}, {vr(dp + e)}, {vr(dp + e + 1)}", vset(dsb + h), vset(dp + e, 2),
+                                earliest=war, deadline=first_B[(c, u2)] - 1))
+        ops[0].earliest = last_A[c] + 4            # the chains' last results need 12 wait states
+        if c + 2 < 4:
+            ops[-1].deadline = min(ops[-1].deadline, first_A[c + 2])  # A(c + 2) writes the same S / dP registers
+        chains.append(ops)
 
-    # ---- LDS reads of the MFMA pairs, PREFETCH pairs ahead ---------------------------------
+    # ---- LDS reads -----------------------------------------------------------------------------
+    # operand fragments of the MFMA pairs, in the order of their use: not before the pair that had
+    # the staging slot has been issued, at least MIN_AHEAD pairs before their own
+    reads = []
     for k in range(len(pairs)):
-        at = 2 * (k - PREFETCH)
-        if at < 0:
-            pre_lds.extend(pair_loads(k))
-        else:
-            slot_lds[at] = pair_loads(k) + slot_lds[at]
+        for text, dst in pair_loads(k):
+            reads.append(lds(text, dst, earliest=max(0, 2 * (k - NSLOT) + 2), deadline=max(0, 2 * (k - MIN_AHEAD))))
+    chains.append(reads)
+    # -lse and -delta of block c: behind the first MFMAs of A(c - 1), which read the registers, and
+    # well before the first MFMAs of A(c)
+    rows = []
+    for c in range(4):
+        for g in range(4):
+            for reg, off in ((V_LSE, 0), (V_DL, DL_OFFSET)):
+                rows.append(lds(f"ds_read_b128 {vr(reg + 4 * g, 4)}, %[la] offset:{(32 * c + 8 * g) * 4 + off}", vset(reg + 4 * g, 4),
+                                earliest=first_A[c - 1] + 6 if c else 0, deadline=max(0, first_A[c] - 6)))
+    chains.append(rows)
 
     # ---- next step's Q / dO tiles: 16 LDS-direct loads per wave spread over the stream ----------
     # (issued back to back they hold the wave for about a thousand cycles: one CU moves 64 B / clk)
-    slot_vmem = {m: [] for m in range(n_slots)}
+    state = {"direct": 0}
+
+    def direct(lds_imm, goff, gbase):
+        def emit(e):
+            if "vmem" in DROP:
+                return
+            e.lds_direct_load(lds_imm, goff, gbase, S_LDSN)
+            state["direct"] += 1
+        return emit
+
+    vm = []
     k = 0
     for t, gbase in enumerate((S_GQ0, S_GQ1, S_GD0, S_GD1)):  # half tiles in LDS order
         for i in range(4):
-            slot_vmem[LOAD_FIRST + LOAD_EVERY * k].append((t * TILE + i * 1024, "%[g1v]" if i == 1 else f"%[g{i}]", gbase, S_LDSN))
+            at = LOAD_FIRST + LOAD_EVERY * k
+            vm.append(Op(direct(t * TILE + i * 1024, "%[g1v]" if i == 1 else f"%[g{i}]", gbase), cost=3, earliest=at, deadline=at + 12))
             k += 1
+    chains.append(vm)
 
-    # ---- emission ------------------------------------------------------------------------------
-    for text, dst in pre_lds:
-        em.lds_read(text, dst)
-    n_direct = 0
-    for m in range(n_slots):
-        for ld in slot_vmem[m]:
-            if 'vmem' in DROP:
-                continue
-            em.lds_direct_load(*ld)
-            n_direct += 1
-        if m == ROW_SLOT and 'vmem' not in DROP:
-            # The two per-row values this lane fetched at the top of the step (older than every
-            # LDS-direct load) have arrived once at most n_direct vector-memory operations are open.
-            # Waves 0, 1: (l, m) -> -lse = -m log2(e) - log2(l), -inf where l = 0; waves 2, 3: -delta
-            # (%[lsew] is non-zero resp. zero).  One LDS store into the next buffer.
-            ra_, rb_, rt_, inf_ = V_ROW, V_ROW + 1, V_ROW + 2, V_ROW + 3
-            em.raw(f"s_waitcnt vmcnt({n_direct})")
-            em.valu(f"v_log_f32_e32 {vr(rt_)}, {vr(ra_)}", vset(rt_), vset(ra_), True)
-            em.valu(f"v_mul_f32_e32 {vr(rb_)}, 0xbfb8aa3b, {vr(rb_)}", vset(rb_), vset(rb_))
-            em.valu(f"v_mov_b32_e32 {vr(inf_)}, 0xff800000", vset(inf_), set())
-            em.valu(f"v_sub_f32_e32 {vr(rt_)}, {vr(rb_)}, {vr(rt_)}", vset(rt_), vset(rt_) | vset(rb_))
-            em.valu(f"v_cmp_lt_f32_e32 vcc, 0, {vr(ra_)}", set(), vset(ra_))
-            em.valu(f"v_cndmask_b32_e32 {vr(rt_)}, {vr(inf_)}, {vr(rt_)}, vcc", vset(rt_), vset(rt_) | vset(inf_))
-            em.raw("s_cmp_lg_u32 s65, 0")
-            em.raw("s_cselect_b64 vcc, -1, 0")
-            em.raw("s_nop 3")
-            em.valu(f"v_xor_b32_e32 {vr(ra_)}, 0x80000000, {vr(ra_)}", vset(ra_), vset(ra_))
-            em.valu(f"v_cndmask_b32_e32 {vr(rt_)}, {vr(ra_)}, {vr(rt_)}, vcc", vset(rt_), vset(rt_) | vset(ra_))
-            em.lds_write(f"ds_write_b32 %[lw], {vr(rt_)}", vset(rt_))
-        lds = slot_lds[m]
-        for text, dst in lds:
-            if 'lds' in DROP:
-                continue
-            em.lds_read(text, dst)
-        mf = pair_mfmas(m // 2)[m % 2]
-        if 'mfma' not in DROP:
-            em.mfma(*mf)
-        for text, dst, src, trans in slot_valu[m]:
-            if 'valu' in DROP:
-                continue
-            em.valu(text, dst, src, trans)
+    def row_turnaround(e):
+        if "vmem" in DROP:
+            return
+        # The two per-row values this lane fetched at the top of the step (older than every
+        # LDS-direct load) have arrived once at most as many vector-memory operations are open as
+        # LDS-direct loads were issued.  Waves 0, 1: (l, m) -> -lse = -m log2(e) - log2(l), -inf where
+        # l = 0; waves 2, 3: -delta (%[lsew] is non-zero resp. zero).  One LDS store into the next buffer.
+        ra_, rb_, rt_, inf_ = V_ROW, V_ROW + 1, V_ROW + 2, V_ROW + 3
+        e.raw(f"s_waitcnt vmcnt({state['direct']})")
+        e.valu(f"v_log_f32_e32 {vr(rt_)}, {vr(ra_)}", vset(rt_), vset(ra_), True)
+        e.valu(f"v_mul_f32_e32 {vr(rb_)}, 0xbfb8aa3b, {vr(rb_)}", vset(rb_), vset(rb_))
+        e.valu(f"v_mov_b32_e32 {vr(inf_)}, 0xff800000", vset(inf_), set())
+        e.valu(f"v_sub_f32_e32 {vr(rt_)}, {vr(rb_)}, {vr(rt_)}", vset(rt_), vset(rt_) | vset(rb_))
+        e.valu(f"v_cmp_lt_f32_e32 vcc, 0, {vr(ra_)}", set(), vset(ra_))
+        e.valu(f"v_cndmask_b32_e32 {vr(rt_)}, {vr(inf_)}, {vr(rt_)}, vcc", vset(rt_), vset(rt_) | vset(inf_))
+        e.raw("s_cmp_lg_u32 s65, 0")
+        e.raw("s_cselect_b64 vcc, -1, 0")
+        e.raw("s_nop 3")
+        e.valu(f"v_xor_b32_e32 {vr(ra_)}, 0x80000000, {vr(ra_)}", vset(ra_), vset(ra_))
+        e.valu(f"v_cndmask_b32_e32 {vr(rt_)}, {vr(ra_)}, {vr(rt_)}, vcc", vset(rt_), vset(rt_) | vset(ra_))
+        e.lds_write(f"ds_write_b32 %[lw], {vr(rt_)}", vset(rt_))
+
+    # V_ROW lies inside pb[1] (first written by E(1)): the turn-around runs before E(1) may start
+    chains.append([Op(row_turnaround, cost=8, earliest=ROW_SLOT, deadline=last_A[1] + 3)])
+
+    schedule(em, mfmas, chains, CAP)
     em.drain()
     return em
 

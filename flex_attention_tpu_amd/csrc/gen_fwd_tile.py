@@ -54,11 +54,12 @@ import os
 import sys
 
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
-from gfx950_stream import Emitter, ar, aset, vr, vset  # noqa: E402
+from gfx950_stream import Emitter, Op, ar, aset, schedule, vr, vset  # noqa: E402
 
-PREFETCH = 4     # MFMA pairs between the LDS reads of a pair and its MFMAs
-LOAD_FIRST = 1   # MFMA slot of the first LDS-direct load of the next step
-LOAD_EVERY = 3   # slots between two of them
+MIN_AHEAD = 2    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
+CAP = 5          # instructions the scheduler puts between two MFMAs unless deadlines force more
+LOAD_FIRST = 2   # MFMA gap from which the first LDS-direct load of the next step may go out
+LOAD_EVERY = 6   # gaps between two of them
 TAU = "0x40c00000"  # 6.0: M moves when the running maximum relative to it leaves [-6, 6]
 DROP = ()        # instruction classes left out (--drop, timing studies only)
 
@@ -102,11 +103,10 @@ def v_p(c, x, u):
 
 def build(masked):
     em = Emitter()
-    # MFMA items (2 MFMAs + one staging slot each), in issue order.  The two q blocks of a kv block
-    # are processed half a stage apart: E(c, 0) runs under A(c+1)[ks 0-3] and B(c-1, 1), E(c, 1) under
-    # A(c+1)[ks 4-7] and B(c, 0), so every softmax has MFMAs of both kinds to hide under.
+    # MFMA pairs (2 MFMAs each), in issue order.  The two q blocks of a kv block are processed half a
+    # stage apart: E(c, 0) runs under A(c+1)[ks 0-3] and B(c-1, 1), E(c, 1) under A(c+1)[ks 4-7] and
+    # B(c, 0), so every softmax has MFMAs of both kinds to hide under.
     pairs = []
-    first, last = {}, {}   # MFMA slot range of half stage (c, q)
 
     def add_A(c, lo, hi):
         for ks in range(lo, hi):
@@ -120,28 +120,37 @@ def build(masked):
     add_A(0, 0, 8)
     for c in range(4):
         for q in range(2):
-            first[(c, q)] = 2 * len(pairs)
             if c < 3:
                 add_A(c + 1, 4 * q, 4 * q + 4)
             if q == 1:
                 add_B(c, 0)
             elif c > 0:
                 add_B(c - 1, 1)
-            last[(c, q)] = 2 * len(pairs)
-    stage_end = 2 * len(pairs)
     add_B(3, 1)
-    n_slots = 2 * len(pairs)
+    idx = {key: 2 * k for k, key in enumerate(pairs)}  # number of the pair's first MFMA
+    n_mfma = 2 * len(pairs)
+
+    def a_mfma(c, ks, q):     # S chain of q block q: MFMA number of k-step ks
+        return idx[("A", c, ks)] + q
+
+    def b_first(c, q, u):
+        return idx[("B", c, (q, u, 0))]
+
+    def b_last(c, q, u):
+        return idx[("B", c, (q, u, 1))] + 1
+
     def half_off(c):
         return (c >> 1) * TILE + (c & 1) * (TILE // 2)
 
     # Staging registers.  K row fragments rotate through eight 4-register slots.  The V^T fragments of
     # a kv block have fixed places: B(c, 0) loads them, B(c, 1) half a stage later uses them again,
     # and the fragments of block c + 1 are read in once the MFMA of B(c, 1) that used the place has
-    # been issued (B(c + 1, 0) follows B(c, 1) at the same distance).
+    # been issued.
     a_index = {}
     for k, (kind, c, x) in enumerate(pairs):
         if kind == "A":
             a_index[k] = len(a_index)
+    a_pairs = [k for k in range(len(pairs)) if pairs[k][0] == "A"]
 
     def k_slot(k):
         return A_STG + 32 + 4 * (a_index[k] % 8)
@@ -149,47 +158,81 @@ def build(masked):
     def v_place(u, db):
         return A_STG + 4 * (4 * u + db)
 
-    def pair_loads(k):
-        kind, c, x = pairs[k]
-        if kind == "A":
-            return [(f"ds_read_b128 {ar(k_slot(k), 4)}, %[r{x}] offset:{half_off(c)}", aset(k_slot(k), 4))]
-        q, u, j = x
-        if q == 1:
-            return []
-        off = 2 * TILE + half_off(c) + u * 4096
-        loads = []
-        for db in (2 * j, 2 * j + 1):
-            for hi in range(2):
-                reg = v_place(u, db) + 2 * hi
-                loads.append((f"ds_read_b64_tr_b16 {ar(reg, 2)}, %[t{2 * db + hi}] offset:{off}", aset(reg, 2)))
-        return loads
+    holds = {}  # V^T place -> kv block whose fragment was last read into it
 
-    def pair_mfmas(k):
-        kind, c, x = pairs[k]
-        out = []
+    def valu(text, dst, src, trans=False, **kw):
+        return Op((lambda e: e.valu(text, dst, src, trans)) if "valu" not in DROP else (lambda e: None), **kw)
+
+    reads = []
+    for k, (kind, c, x) in enumerate(pairs):
         if kind == "A":
-            ks = x
-            base = k_slot(k)
-            for q in range(2):
-                s = v_s(c, q)
-                # the chain starts from -M: its result is the score relative to the reference maximum
-                cin = V_NEGM + 16 * q if ks == 0 else s
-                out.append((vr(s, 16), ar(base, 4), ar(A_Q + 32 * q + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(base, 4),
-                            aset(A_Q + 32 * q + 4 * ks, 4), vset(cin, 16)))
-            return out
-        q, u, j = x
+            ia = a_index[k]
+            text, dst = f"ds_read_b128 {ar(k_slot(k), 4)}, %[r{x}] offset:{half_off(c)}", aset(k_slot(k), 4)
+            earliest = 2 * a_pairs[ia - 8] + 2 if ia >= 8 else 0
+            reads.append((2 * k, Op((lambda e, t=text, d=dst: e.lds_read(t, d)) if "lds" not in DROP else (lambda e: None),
+                                    earliest=earliest, deadline=max(0, 2 * (k - MIN_AHEAD)))))
+        elif x[0] == 0:
+            q, u, j = x
+            off = 2 * TILE + half_off(c) + u * 4096
+            for db in (2 * j, 2 * j + 1):
+                for hi in range(2):
+                    reg = v_place(u, db) + 2 * hi
+                    text, dst = f"ds_read_b64_tr_b16 {ar(reg, 2)}, %[t{2 * db + hi}] offset:{off}", aset(reg, 2)
+
+                    def emit(e, t=text, d=dst, key=(u, db), blk=c):
+                        holds[key] = blk
+                        if "lds" not in DROP:
+                            e.lds_read(t, d)
+                    earliest = b_last(c - 1, 1, u) + 1 if c > 0 else 0
+                    reads.append((2 * k, Op(emit, earliest=earliest, deadline=2 * (k - MIN_AHEAD))))
+    reads.sort(key=lambda r: r[0])  # (stable: in the order of their use)
+
+    def mfma_of(k, j):
+        kind, c, x = pairs[k]
+        if kind == "A":
+            ks, q = x, j
+            s = v_s(c, q)
+            # the chain starts from -M: its result is the score relative to the reference maximum
+            cin = V_NEGM + 16 * q if ks == 0 else s
+            return (vr(s, 16), ar(k_slot(k), 4), ar(A_Q + 32 * q + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(k_slot(k), 4),
+                    aset(A_Q + 32 * q + 4 * ks, 4), vset(cin, 16))
+        q, u, jj = x
+        db = 2 * jj + j
         p = v_p(c, q, u)
-        for db in (2 * j, 2 * j + 1):
-            acc = A_O + 64 * q + 16 * db
-            vt = v_place(u, db)
-            out.append((ar(acc, 16), ar(vt, 4), vr(p, 4), ar(acc, 16), aset(acc, 16), aset(vt, 4), vset(p, 4), aset(acc, 16)))
-        return out
+        acc = A_O + 64 * q + 16 * db
+        vt = v_place(u, db)
+        args = (ar(acc, 16), ar(vt, 4), vr(p, 4), ar(acc, 16), aset(acc, 16), aset(vt, 4), vset(p, 4), aset(acc, 16))
 
-    # ---- VALU work of E(c, q): a list of (kind, ...) ------------------------------------------
+        def emit(e):
+            assert holds.get((u, db)) == c, f"B({c}, {q}) would multiply with the V^T fragment of block {holds.get((u, db))}"
+            e.mfma(*args)
+        return emit
+
+    mfmas = [mfma_of(k, j) for k in range(len(pairs)) for j in range(2)]
+    if "mfma" in DROP:
+        mfmas = [(lambda e: None)] * n_mfma
+
+    # ---- VALU work of E(c, q) -------------------------------------------------------------------
     T = [V_TMP + i for i in range(10)]
     tag = "m" if masked else "f"
 
-    def softmax_ops(c, q):
+    def block(ops, **kw):
+        """A branch, the block it may skip and its label, placed as one unit."""
+        def emit(e):
+            for op in ops:
+                if op[0] == "raw":
+                    e.raw(op[1])
+                elif op[0] == "label":
+                    e.label(op[1])
+                elif op[0] == "skip_begin":
+                    e.skip_begin()
+                elif op[0] == "skip_end":
+                    e.skip_end()
+                elif "valu" not in DROP:
+                    e.valu(*op[1:])
+        return Op(emit, cost=2, **kw)
+
+    def softmax_chain(c, q):
         """Online softmax of the lane's 16 scores (relative to M) of q block q in kv block c."""
         s = v_s(c, q)
         M, Mt, L = f"%[M{q}]", f"%[Mt{q}]", f"%[L{q}]"
@@ -197,91 +240,95 @@ def build(masked):
         D, AL, negm = V_D + q, V_AL + q, V_NEGM + 16 * q
         ops = []
 
-        def valu(text, dst, src, trans=False):
-            ops.append(("valu", text, dst, src, trans))
-
-        def raw(text):
-            ops.append(("raw", text))
-
         if c > 0:
             # M moved while this block's chain was in flight with the old -M: apply the shift now
-            raw(f"s_cmp_eq_u32 {S_PEND[q]}, 0")
-            raw(f"s_cbranch_scc1 .Lfa_fwd_{tag}_late{c}{q}_%=")
-            ops.append(("skip_begin",))
+            late = [("raw", f"s_cmp_eq_u32 {S_PEND[q]}, 0"), ("raw", f"s_cbranch_scc1 .Lfa_fwd_{tag}_late{c}{q}_%="), ("skip_begin",)]
             for e in range(16):
-                valu(f"v_sub_f32_e32 {vr(s + e)}, {vr(s + e)}, {vr(D)}", vset(s + e), vset(s + e) | vset(D))
-            raw(f"s_mov_b32 {S_PEND[q]}, 0")
-            ops.append(("skip_end",))
-            ops.append(("label", f".Lfa_fwd_{tag}_late{c}{q}_%=:"))
+                late.append(("valu", f"v_sub_f32_e32 {vr(s + e)}, {vr(s + e)}, {vr(D)}", vset(s + e), vset(s + e) | vset(D), False))
+            late += [("raw", f"s_mov_b32 {S_PEND[q]}, 0"), ("skip_end",), ("label", f".Lfa_fwd_{tag}_late{c}{q}_%=:")]
+            ops.append(block(late))
         if masked:
             for g in range(4):
                 for u in range(4):
                     e = 4 * g + u
-                    valu(f"v_bfe_i32 {vr(V_MSK + u)}, %[m{2 * q + (c >> 1)}], {16 * (c & 1) + e}, 1", vset(V_MSK + u), set())
+                    ops.append(valu(f"v_bfe_i32 {vr(V_MSK + u)}, %[m{2 * q + (c >> 1)}], {16 * (c & 1) + e}, 1", vset(V_MSK + u), set()))
                 for u in range(4):
                     e = 4 * g + u  # keep ? score : -inf
-                    valu(f"v_bfi_b32 {vr(s + e)}, {vr(V_MSK + u)}, {vr(s + e)}, {vr(V_NEGINF)}", vset(s + e),
-                         vset(s + e) | vset(V_MSK + u) | vset(V_NEGINF))
+                    ops.append(valu(f"v_bfi_b32 {vr(s + e)}, {vr(V_MSK + u)}, {vr(s + e)}, {vr(V_NEGINF)}", vset(s + e),
+                                    vset(s + e) | vset(V_MSK + u) | vset(V_NEGINF)))
         # block maximum of the lane's 16 scores, then across the two half-waves that share the q row
         for i in range(5):
-            valu(f"v_max3_f32 {vr(T[i])}, {vr(s + 3 * i)}, {vr(s + 3 * i + 1)}, {vr(s + 3 * i + 2)}", vset(T[i]), vset(s + 3 * i, 3))
-        valu(f"v_max3_f32 {vr(T[0])}, {vr(T[0])}, {vr(T[1])}, {vr(T[2])}", vset(T[0]), vset(T[0]) | vset(T[1]) | vset(T[2]))
-        valu(f"v_max3_f32 {vr(T[3])}, {vr(T[3])}, {vr(T[4])}, {vr(s + 15)}", vset(T[3]), vset(T[3]) | vset(T[4]) | vset(s + 15))
-        valu(f"v_max_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[3])}", vset(T[0]), vset(T[0]) | vset(T[3]))
-        valu(f"v_mov_b32_e32 {vr(T[1])}, {vr(T[0])}", vset(T[1]), vset(T[0]))
-        raw("s_nop 1")
-        valu(f"v_permlane32_swap_b32 {vr(T[0])}, {vr(T[1])}", vset(T[0]) | vset(T[1]), vset(T[0]) | vset(T[1]))
-        raw("s_nop 1")
-        valu(f"v_max_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[1])}", vset(T[0]), vset(T[0]) | vset(T[1]))
-        valu(f"v_max_f32_e32 {Mt}, {Mt}, {vr(T[0])}", kMt, kMt | vset(T[0]))
+            ops.append(valu(f"v_max3_f32 {vr(T[i])}, {vr(s + 3 * i)}, {vr(s + 3 * i + 1)}, {vr(s + 3 * i + 2)}", vset(T[i]), vset(s + 3 * i, 3)))
+        ops.append(valu(f"v_max3_f32 {vr(T[0])}, {vr(T[0])}, {vr(T[1])}, {vr(T[2])}", vset(T[0]), vset(T[0]) | vset(T[1]) | vset(T[2])))
+        ops.append(valu(f"v_max3_f32 {vr(T[3])}, {vr(T[3])}, {vr(T[4])}, {vr(s + 15)}", vset(T[3]), vset(T[3]) | vset(T[4]) | vset(s + 15)))
+        ops.append(valu(f"v_max_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[3])}", vset(T[0]), vset(T[0]) | vset(T[3])))
+        ops.append(valu(f"v_mov_b32_e32 {vr(T[1])}, {vr(T[0])}", vset(T[1]), vset(T[0])))
+
+        def swap(e):
+            e.raw("s_nop 1")
+            if "valu" not in DROP:
+                e.valu(f"v_permlane32_swap_b32 {vr(T[0])}, {vr(T[1])}", vset(T[0]) | vset(T[1]), vset(T[0]) | vset(T[1]))
+            e.raw("s_nop 1")
+        ops.append(Op(swap, cost=3))
+        ops.append(valu(f"v_max_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[1])}", vset(T[0]), vset(T[0]) | vset(T[1])))
+        ops.append(valu(f"v_max_f32_e32 {Mt}, {Mt}, {vr(T[0])}", kMt, kMt | vset(T[0])))
         # does the running maximum leave [-TAU, TAU] (and is it finite: rows that kept nothing so far stay put)?
-        valu(f"v_cmp_gt_f32_e64 vcc, |{Mt}|, {vr(V_TAU)}", set(), kMt | vset(V_TAU))
+        rare = [("valu", f"v_cmp_gt_f32_e64 vcc, |{Mt}|, {vr(V_TAU)}", set(), kMt | vset(V_TAU), False)]
         if masked:
-            valu(f"v_cmp_neq_f32_e64 s[86:87], {Mt}, {vr(V_NEGINF)}", set(), kMt | vset(V_NEGINF))
-            raw("s_and_b64 vcc, vcc, s[86:87]")
-        raw(f"s_cbranch_vccz .Lfa_fwd_{tag}_keep{c}{q}_%=")
-        ops.append(("skip_begin",))
-        raw("s_nop 3")
-        valu(f"v_cndmask_b32_e32 {vr(D)}, 0, {Mt}, vcc", vset(D), kMt)                 # the lane's shift
-        valu(f"v_exp_f32_e64 {vr(AL)}, -{vr(D)}", vset(AL), vset(D), True)
-        valu(f"v_sub_f32_e32 {Mt}, {Mt}, {vr(D)}", kMt, kMt | vset(D))
-        valu(f"v_add_f32_e32 {M}, {M}, {vr(D)}", kM, kM | vset(D))
-        valu(f"v_mul_f32_e32 {L}, {L}, {vr(AL)}", kL, kL | vset(AL))
+            rare.append(("valu", f"v_cmp_neq_f32_e64 s[86:87], {Mt}, {vr(V_NEGINF)}", set(), kMt | vset(V_NEGINF), False))
+            rare.append(("raw", "s_and_b64 vcc, vcc, s[86:87]"))
+        rare += [("raw", f"s_cbranch_vccz .Lfa_fwd_{tag}_keep{c}{q}_%="), ("skip_begin",), ("raw", "s_nop 3"),
+                 ("valu", f"v_cndmask_b32_e32 {vr(D)}, 0, {Mt}, vcc", vset(D), kMt, False),                 # the lane's shift
+                 ("valu", f"v_exp_f32_e64 {vr(AL)}, -{vr(D)}", vset(AL), vset(D), True),
+                 ("valu", f"v_sub_f32_e32 {Mt}, {Mt}, {vr(D)}", kMt, kMt | vset(D), False),
+                 ("valu", f"v_add_f32_e32 {M}, {M}, {vr(D)}", kM, kM | vset(D), False),
+                 ("valu", f"v_mul_f32_e32 {L}, {L}, {vr(AL)}", kL, kL | vset(AL), False)]
         for i in range(64):
             t = T[5 + (i % 4)]
             acc = A_O + 64 * q + i
-            valu(f"v_accvgpr_read_b32 {vr(t)}, {ar(acc)}", vset(t), aset(acc))
-            valu(f"v_mul_f32_e32 {vr(t)}, {vr(t)}, {vr(AL)}", vset(t), vset(t) | vset(AL))
-            valu(f"v_accvgpr_write_b32 {ar(acc)}, {vr(t)}", aset(acc), vset(t))
+            rare.append(("valu", f"v_accvgpr_read_b32 {vr(t)}, {ar(acc)}", vset(t), aset(acc), False))
+            rare.append(("valu", f"v_mul_f32_e32 {vr(t)}, {vr(t)}, {vr(AL)}", vset(t), vset(t) | vset(AL), False))
+            rare.append(("valu", f"v_accvgpr_write_b32 {ar(acc)}, {vr(t)}", aset(acc), vset(t), False))
         for e in range(16):
-            valu(f"v_sub_f32_e32 {vr(s + e)}, {vr(s + e)}, {vr(D)}", vset(s + e), vset(s + e) | vset(D))
+            rare.append(("valu", f"v_sub_f32_e32 {vr(s + e)}, {vr(s + e)}, {vr(D)}", vset(s + e), vset(s + e) | vset(D), False))
         for e in range(16):
-            valu(f"v_sub_f32_e32 {vr(negm + e)}, {vr(negm + e)}, {vr(D)}", vset(negm + e), vset(negm + e) | vset(D))
+            rare.append(("valu", f"v_sub_f32_e32 {vr(negm + e)}, {vr(negm + e)}, {vr(D)}", vset(negm + e), vset(negm + e) | vset(D), False))
         if c < 3:
-            raw(f"s_mov_b32 {S_PEND[q]}, 1")  # (kv block c + 1 of this step is in flight; block 0 of the next step is not)
-        ops.append(("skip_end",))
-        ops.append(("label", f".Lfa_fwd_{tag}_keep{c}{q}_%=:"))
+            rare.append(("raw", f"s_mov_b32 {S_PEND[q]}, 1"))  # (kv block c + 1 of this step is in flight; block 0 of the next step is not)
+        rare += [("skip_end",), ("label", f".Lfa_fwd_{tag}_keep{c}{q}_%=:")]
+        # The block rescales O^T: every B(c - 1, q) MFMA is out, no B(c, q) MFMA is; and the chain of
+        # kv block c + 1 has started (it carries the old -M and is corrected by its own "late" block).
+        rare_earliest = 0
+        if c > 0:
+            rare_earliest = b_last(c - 1, q, 1) + 1
+        if c < 3:
+            rare_earliest = max(rare_earliest, a_mfma(c + 1, 0, q) + 1)
+        ops.append(block(rare, earliest=rare_earliest))
+
         # p = 2^(score - M), packed to bf16 B operands.  The row sum adds the fp32 values in four
         # interleaved partial sums (plain adds hide under the MFMAs; v_dot2c on the packed values
         # measured 9 cycles apiece).
         def exps(g):
             for u in range(4):
                 e = 4 * g + u
-                valu(f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True)
+                ops.append(valu(f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
 
         def packs(g):
+            u2 = g >> 1
+            war = b_last(c - 1, q, u2) + 1 if c > 0 else 0   # the registers are those of block c - 1
             for h in range(2):
                 e = 4 * g + 2 * h
-                pr = v_p(c, q, g >> 1) + 2 * (g & 1) + h
-                valu(f"v_cvt_pk_bf16_f32 {vr(pr)}, {vr(s + e)}, {vr(s + e + 1)}", vset(pr), vset(s + e, 2))
+                pr = v_p(c, q, u2) + 2 * (g & 1) + h
+                ops.append(valu(f"v_cvt_pk_bf16_f32 {vr(pr)}, {vr(s + e)}, {vr(s + e + 1)}", vset(pr), vset(s + e, 2),
+                                earliest=war, deadline=b_first(c, q, u2) - 1))
 
         def sums(g):
             for u in range(4):
                 e = 4 * g + u
                 if g == 1:
-                    valu(f"v_add_f32_e32 {vr(T[u])}, {vr(s + u)}, {vr(s + e)}", vset(T[u]), vset(s + u) | vset(s + e))
+                    ops.append(valu(f"v_add_f32_e32 {vr(T[u])}, {vr(s + u)}, {vr(s + e)}", vset(T[u]), vset(s + u) | vset(s + e)))
                 elif g > 1:
-                    valu(f"v_add_f32_e32 {vr(T[u])}, {vr(T[u])}, {vr(s + e)}", vset(T[u]), vset(T[u]) | vset(s + e))
+                    ops.append(valu(f"v_add_f32_e32 {vr(T[u])}, {vr(T[u])}, {vr(s + e)}", vset(T[u]), vset(T[u]) | vset(s + e)))
 
         exps(0)
         for g in range(4):
@@ -289,100 +336,39 @@ def build(masked):
                 exps(g + 1)
             sums(g)
             packs(g)
-        valu(f"v_add_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[1])}", vset(T[0]), vset(T[0]) | vset(T[1]))
-        valu(f"v_add_f32_e32 {vr(T[2])}, {vr(T[2])}, {vr(T[3])}", vset(T[2]), vset(T[2]) | vset(T[3]))
-        valu(f"v_add_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[2])}", vset(T[0]), vset(T[0]) | vset(T[2]))
-        valu(f"v_add_f32_e32 {L}, {L}, {vr(T[0])}", kL, kL | vset(T[0]))
+        ops.append(valu(f"v_add_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[1])}", vset(T[0]), vset(T[0]) | vset(T[1])))
+        ops.append(valu(f"v_add_f32_e32 {vr(T[2])}, {vr(T[2])}, {vr(T[3])}", vset(T[2]), vset(T[2]) | vset(T[3])))
+        ops.append(valu(f"v_add_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[2])}", vset(T[0]), vset(T[0]) | vset(T[2])))
+        ops.append(valu(f"v_add_f32_e32 {L}, {L}, {vr(T[0])}", kL, kL | vset(T[0])))
+        ops[0].earliest = max(ops[0].earliest, a_mfma(c, 7, q) + 4)   # the chain's last result needs 12 wait states
+        if c + 2 < 4:
+            ops[-1].deadline = min(ops[-1].deadline or (1 << 30), a_mfma(c + 2, 0, q))  # A(c + 2) writes the same S registers
         return ops
 
-    slot_ops = {m: [] for m in range(n_slots + 1)}
-    slot_lds = {m: [] for m in range(n_slots)}
-    pre_lds = []
+    # The softmax chains share their temporaries: one after the other, in the order of the half stages.
+    soft = []
     for c in range(4):
         for q in range(2):
-            ops = softmax_ops(c, q)
-            lo = first[(c, q)] + 4  # the block's last MFMAs were issued just before: give their results time
-            span = last[(c, q)] - lo
-            # a branch, the block it may skip and its label stay in one slot (no MFMA or LDS read may
-            # end up inside the skipped range); the block counts for nothing when the work is spread
-            total = 0
-            inside = False
-            for op in ops:
-                if op[0] == "skip_begin":
-                    inside = True
-                if not inside and op[0] != "label":
-                    total += 1
-                if op[0] == "skip_end":
-                    inside = False
-            done = 0
-            pinned = None
-            for i, op in enumerate(ops):
-                if pinned is None and i + 1 < len(ops) and ops[i + 1][0] == "skip_begin":
-                    pinned = lo + (done * span) // total  # (op is the branch)
-                slot_ops[pinned if pinned is not None else lo + (done * span) // total].append(op)
-                if pinned is None or i + 1 < len(ops) and ops[i + 1][0] == "skip_begin":
-                    done += 1
-                if op[0] == "label":
-                    pinned = None
+            soft.extend(softmax_chain(c, q))
+    chains = [soft, [op for _, op in reads]]
 
-    for k in range(len(pairs)):
-        # (V^T fragments one pair later than K rows: in the last stages, which have no A pairs, the
-        # place's previous user is only four pairs ahead and must have been issued)
-        at = 2 * (k - (PREFETCH if pairs[k][0] == "A" else PREFETCH - 1))
-        if at < 0:
-            pre_lds.extend(pair_loads(k))
-        else:
-            slot_lds[at] = pair_loads(k) + slot_lds[at]
-
-    slot_vmem = {m: [] for m in range(n_slots)}
+    # ---- next step's K / V tiles: 16 LDS-direct loads per wave spread over the stream ------------
+    vm = []
     k = 0
     for t, gbase in enumerate((S_GK0, S_GK1, S_GV0, S_GV1)):  # half tiles in LDS order
         for i in range(4):
-            slot_vmem[LOAD_FIRST + LOAD_EVERY * k].append((t * TILE + i * 1024, "%[g1v]" if i == 1 else f"%[g{i}]", gbase, S_LDSN))
-            k += 1
+            at = LOAD_FIRST + LOAD_EVERY * k
 
-    def emit(op):
-        if op[0] == "raw":
-            em.raw(op[1])
-        elif op[0] == "label":
-            em.label(op[1])
-        elif op[0] == "skip_begin":
-            em.skip_begin()
-        elif op[0] == "skip_end":
-            em.skip_end()
-        elif "valu" not in DROP:
-            em.valu(*op[1:])
+            def emit(e, imm=t * TILE + i * 1024, goff="%[g1v]" if i == 1 else f"%[g{i}]", gb=gbase):
+                if "vmem" not in DROP:
+                    e.lds_direct_load(imm, goff, gb, S_LDSN)
+            vm.append(Op(emit, cost=3, earliest=at, deadline=at + 12))
+            k += 1
+    chains.append(vm)
 
     if masked:
         em.valu(f"v_mov_b32_e32 {vr(V_NEGINF)}, 0xff800000", vset(V_NEGINF), set())
-    for text, dst in pre_lds:
-        em.lds_read(text, dst)
-    holds = {}  # V^T place -> kv block whose fragment was last read into it
-    for k, (kind, c, x) in enumerate(pairs):
-        if kind == "B" and x[0] == 0 and 2 * (k - (PREFETCH - 1)) < 0:
-            raise AssertionError("V^T fragments are never part of the preamble")
-    for m in range(n_slots):
-        for ld in slot_vmem[m]:  # (M0 was written in front of the previous MFMA)
-            if "vmem" not in DROP:
-                em.lds_direct_issue(ld[1], ld[2])
-        for text, dst in slot_lds[m]:
-            if "lds" not in DROP:
-                em.lds_read(text, dst)
-        for k, (kind, c, x) in enumerate(pairs):  # bookkeeping of the V^T places (see v_place)
-            if kind == "B" and x[0] == 0 and 2 * (k - (PREFETCH - 1)) == m:
-                for db in (2 * x[2], 2 * x[2] + 1):
-                    holds[(x[1], db)] = c
-        kind, c, x = pairs[m // 2]
-        if kind == "B":
-            db = 2 * x[2] + (m % 2)
-            assert holds.get((x[1], db)) == c, f"B({c}, {x[0]}) would multiply with the V^T fragment of block {holds.get((x[1], db))}"
-        for ld in slot_vmem.get(m + 1, []):  # (the MFMA below is the wait state between M0 and its load)
-            if "vmem" not in DROP:
-                em.lds_direct_dest(ld[0], ld[3])
-        if "mfma" not in DROP:
-            em.mfma(*pair_mfmas(m // 2)[m % 2])
-        for op in slot_ops[m]:
-            emit(op)
+    schedule(em, mfmas, chains, CAP)
     em.drain()
     return em
 

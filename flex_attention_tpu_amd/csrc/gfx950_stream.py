@@ -193,3 +193,58 @@ class Emitter:
         if self.lds_fifo:
             self._raw("s_waitcnt lgkmcnt(0)")
             self.lds_fifo = []
+
+
+class Op:
+    """A unit the scheduler places as a whole: `emit(em)` writes it; `cost` is its share of an MFMA
+    gap; it goes into gap `earliest` at the soonest and must be out before MFMA number `deadline`."""
+
+    def __init__(self, emit, cost=1, earliest=0, deadline=None):
+        self.emit, self.cost, self.earliest, self.deadline = emit, cost, earliest, deadline
+
+
+def schedule(em, mfmas, chains, cap):
+    """Writes the MFMAs in order with the chains' operations in the gaps between them (gap g lies in
+    front of MFMA g; gap len(mfmas) behind the last one).  A single wave only keeps the matrix pipe
+    busy while the instructions between two MFMAs issue within the 32 cycles the first one runs, about
+    four of them: so every gap takes at most `cap` units of cost unless deadlines force more, picked
+    earliest-deadline-first among the chains' heads (order inside a chain is kept)."""
+    n = len(mfmas)
+    big = 1 << 30
+    for ch in chains:  # an operation inherits the needs of its neighbours in the chain
+        e = 0
+        for op in ch:
+            e = op.earliest = max(op.earliest, e)
+        d = big
+        for op in reversed(ch):
+            d = op.deadline = min(big if op.deadline is None else op.deadline, d)
+            assert op.earliest <= op.deadline, "an operation's window is empty"
+    heads = [0] * len(chains)
+    over = 0
+    for g in range(n + 1):
+        used = 0
+        while True:
+            best = None
+            for i, ch in enumerate(chains):
+                if heads[i] < len(ch):
+                    op = ch[heads[i]]
+                    if op.earliest <= g and (best is None or op.deadline < chains[best][heads[best]].deadline):
+                        best = i
+            if best is None:
+                break
+            op = chains[best][heads[best]]
+            forced = op.deadline <= g or g == n
+            if not forced and used + op.cost > cap:
+                break
+            op.emit(em)
+            used += op.cost
+            heads[best] += 1
+        over += max(0, used - cap)
+        if g < n:
+            if callable(mfmas[g]):
+                mfmas[g](em)
+            else:
+                em.mfma(*mfmas[g])
+    assert all(heads[i] == len(ch) for i, ch in enumerate(chains)), "operations left over"
+    em.stats["over_cap"] = over
+
