@@ -40,12 +40,13 @@ import os
 import sys
 
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
-from gfx950_stream import Emitter, ar, aset, vr, vset  # noqa: E402
+from gfx950_stream import Emitter, Op, ar, aset, schedule, vr, vset  # noqa: E402
 
 NSLOT = 8        # staging slots of 8 registers
-PREFETCH = 4     # MFMA pairs between the LDS reads of a pair and its MFMAs
-LOAD_FIRST = 2   # MFMA slot of the first LDS-direct load of the next step
-LOAD_EVERY = 5   # slots between two of them
+MIN_AHEAD = 2    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
+CAP = 4          # instructions the scheduler puts between two MFMAs unless deadlines force more
+LOAD_FIRST = 2   # MFMA gap from which the first LDS-direct load of the next step may go out
+LOAD_EVERY = 5   # gaps between two of them
 DROP = ()        # instruction classes left out (--drop, timing studies only)
 
 TILE = 16384
@@ -89,15 +90,12 @@ def build(masked):
             for j in range(2):
                 pairs.append(("B", c, (u, j)))
 
-    add_A(0)
-    first = {}
-    first[0] = 2 * len(pairs); add_A(1)
-    first[1] = 2 * len(pairs); add_A(2); add_B(0)
-    first[2] = 2 * len(pairs); add_A(3); add_B(1)
-    first[3] = 2 * len(pairs); add_B(2)
-    stage_end = 2 * len(pairs); add_B(3)
-    n_slots = 2 * len(pairs)
-    last = {0: first[1], 1: first[2], 2: first[3], 3: stage_end}
+    add_A(0); add_A(1); add_A(2); add_B(0); add_A(3); add_B(1); add_B(2); add_B(3)
+    idx = {key: 2 * k for k, key in enumerate(pairs)}  # number of the pair's first MFMA
+    first_A = {c: idx[("A", c, 0)] for c in range(4)}
+    last_A = {c: idx[("A", c, 7)] + 1 for c in range(4)}
+    first_B = {(c, u): idx[("B", c, (u, 0))] for c in range(4) for u in range(2)}
+    last_B = {(c, u): idx[("B", c, (u, 1))] + 1 for c in range(4) for u in range(2)}
 
     def half_off(c):
         return (c >> 1) * TILE + (c & 1) * (TILE // 2)
@@ -139,67 +137,70 @@ def build(masked):
                         vset(ds, 4), aset(acc, 16)))
         return out
 
-    # ---- VALU work of E(c), spread over the MFMA slots of stage c ---------------------------
-    slot_valu = {m: [] for m in range(n_slots)}
-    slot_lds = {m: [] for m in range(n_slots)}
-    pre_lds = []
-    c2 = SREG["c2"]
+    mfmas = [pair_mfmas(k)[j] for k in range(len(pairs)) for j in range(2)]
+    if "mfma" in DROP:
+        mfmas = [(lambda e: None)] * len(mfmas)
+
+    def valu(text, dst, src, trans=False, **kw):
+        return Op((lambda e: e.valu(text, dst, src, trans)) if "valu" not in DROP else (lambda e: None), **kw)
+
+    chains = []
+    # ---- E(c): element-wise work between the block's S / dP chains and its B product ----------
     for c in range(4):
         s, dp = V_S[c & 1], V_DP[c & 1]
         ops = []
         for g in range(4):
             for u in range(4):
                 e = 4 * g + u
-                ops.append((f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
+                ops.append(valu(f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
             if masked:
                 for u in range(4):
                     e = 4 * g + u
-                    ops.append((f"v_bfe_i32 {vr(V_TMP + u)}, %[m{c >> 1}], {16 * (c & 1) + e}, 1", vset(V_TMP + u), set(), False))
+                    ops.append(valu(f"v_bfe_i32 {vr(V_TMP + u)}, %[m{c >> 1}], {16 * (c & 1) + e}, 1", vset(V_TMP + u), set()))
                 for u in range(4):
                     e = 4 * g + u
-                    ops.append((f"v_and_b32_e32 {vr(s + e)}, {vr(s + e)}, {vr(V_TMP + u)}", vset(s + e),
-                                vset(s + e) | vset(V_TMP + u), False))
+                    ops.append(valu(f"v_and_b32_e32 {vr(s + e)}, {vr(s + e)}, {vr(V_TMP + u)}", vset(s + e), vset(s + e) | vset(V_TMP + u)))
             for u in range(4):
                 e = 4 * g + u
-                ops.append((f"v_mul_f32_e32 {vr(dp + e)}, {vr(s + e)}, {vr(dp + e)}", vset(dp + e), vset(dp + e) | vset(s + e), False))
-            ds = V_DS + 8 * (c & 1) + 4 * (g >> 1) + 2 * (g & 1)
+                ops.append(valu(f"v_mul_f32_e32 {vr(dp + e)}, {vr(s + e)}, {vr(dp + e)}", vset(dp + e), vset(dp + e) | vset(s + e)))
+            # dS^T operand u2 = g >> 1: the registers are those of block c - 2, whose B MFMAs that read
+            # them must have been issued; this block's B MFMAs of half u2 wait for them
+            u2 = g >> 1
+            ds = V_DS + 8 * (c & 1) + 4 * u2 + 2 * (g & 1)
+            war = last_B[(c - 2, u2)] + 1 if c >= 2 else 0
             for h in range(2):
                 e = 4 * g + 2 * h
-                ops.append((f"v_cvt_pk_bf16_f32 {vr(ds + h)}, {vr(dp + e)}, {vr(dp + e + 1)}", vset(ds + h), vset(dp + e, 2), False))
-        lo = first[c] + (6 if c == 0 else 0)  # E(0) directly follows A(0): give its results time
-        span = last[c] - lo
-        for i, op in enumerate(ops):
-            slot_valu[lo + (i * span) // len(ops)].append(op)
+                ops.append(valu(f"v_cvt_pk_bf16_f32 {vr(ds + h)}, {vr(dp + e)}, {vr(dp + e + 1)}", vset(ds + h), vset(dp + e, 2),
+                                earliest=war, deadline=first_B[(c, u2)] - 1))
+        ops[0].earliest = last_A[c] + 4            # the chains' last results need 12 wait states
+        if c + 2 < 4:
+            ops[-1].deadline = min(ops[-1].deadline, first_A[c + 2])  # A(c + 2) writes the same S / dP registers
+        chains.append(ops)
 
+    # ---- LDS reads of the MFMA pairs, in the order of their use: not before the pair that had the
+    # staging slot has been issued, at least MIN_AHEAD pairs before their own
+    reads = []
     for k in range(len(pairs)):
-        at = 2 * (k - PREFETCH)
-        if at < 0:
-            pre_lds.extend(pair_loads(k))
-        else:
-            slot_lds[at] = pair_loads(k) + slot_lds[at]
+        for text, dst in pair_loads(k):
+            reads.append(Op((lambda e, t=text, d=dst: e.lds_read(t, d)) if "lds" not in DROP else (lambda e: None),
+                            earliest=max(0, 2 * (k - NSLOT) + 2), deadline=max(0, 2 * (k - MIN_AHEAD))))
+    chains.append(reads)
 
-    # next step's K / V tiles: 16 LDS-direct loads per wave spread over the stream
-    slot_vmem = {m: [] for m in range(n_slots)}
+    # ---- next step's K / V tiles: 16 LDS-direct loads per wave spread over the stream ------------
+    vm = []
     k = 0
     for t, gbase in enumerate((S_GK0, S_GK1, S_GV0, S_GV1)):  # half tiles in LDS order
         for i in range(4):
-            slot_vmem[LOAD_FIRST + LOAD_EVERY * k].append((t * TILE + i * 1024, "%[g1v]" if i == 1 else f"%[g{i}]", gbase, S_LDSN))
-            k += 1
+            at = LOAD_FIRST + LOAD_EVERY * k
 
-    for text, dst in pre_lds:
-        em.lds_read(text, dst)
-    for m in range(n_slots):
-        for ld in slot_vmem[m]:
-            if "vmem" not in DROP:
-                em.lds_direct_load(*ld)
-        for text, dst in slot_lds[m]:
-            if "lds" not in DROP:
-                em.lds_read(text, dst)
-        if "mfma" not in DROP:
-            em.mfma(*pair_mfmas(m // 2)[m % 2])
-        for text, dst, src, trans in slot_valu[m]:
-            if "valu" not in DROP:
-                em.valu(text, dst, src, trans)
+            def emit(e, imm=t * TILE + i * 1024, goff="%[g1v]" if i == 1 else f"%[g{i}]", gb=gbase):
+                if "vmem" not in DROP:
+                    e.lds_direct_load(imm, goff, gb, S_LDSN)
+            vm.append(Op(emit, cost=3, earliest=at, deadline=at + 12))
+            k += 1
+    chains.append(vm)
+
+    schedule(em, mfmas, chains, CAP)
     em.drain()
     return em
 
