@@ -46,7 +46,7 @@ NSLOT = 8        # staging slots of 8 registers
 MIN_AHEAD = 2    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
 CAP = 4          # instructions the scheduler puts between two MFMAs unless deadlines force more
 LOAD_FIRST = 2   # MFMA gap from which the first LDS-direct load of the next step may go out
-LOAD_EVERY = 5   # gaps between two of them
+LOAD_EVERY = 2   # gaps between two of them
 DROP = ()        # instruction classes left out (--drop, timing studies only)
 
 TILE = 16384

@@ -59,7 +59,7 @@ from gfx950_stream import Emitter, Op, ar, aset, schedule, vr, vset  # noqa: E40
 MIN_AHEAD = 2    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
 CAP = 5          # instructions the scheduler puts between two MFMAs unless deadlines force more
 LOAD_FIRST = 2   # MFMA gap from which the first LDS-direct load of the next step may go out
-LOAD_EVERY = 6   # gaps between two of them
+LOAD_EVERY = 2   # gaps between two of them
 TAU = "0x40c00000"  # 6.0: M moves when the running maximum relative to it leaves [-6, 6]
 DROP = ()        # instruction classes left out (--drop, timing studies only)
 
