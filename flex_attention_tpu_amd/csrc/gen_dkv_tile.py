@@ -50,6 +50,7 @@ from gfx950_stream import Emitter, Op, ar, aset, schedule, vr, vset  # noqa: E40
 
 NSLOT = 8        # staging slots of 8 registers
 MIN_AHEAD = 2    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
+WAIT_OLD = 20    # a wait for LDS data also covers younger reads issued at least this many instructions ago
 CAP = 4          # instructions the scheduler puts between two MFMAs unless deadlines force more
 LOAD_FIRST = 2   # MFMA gap from which the first LDS-direct load of the next step may go out
 LOAD_EVERY = 2   # gaps between two of them
@@ -89,6 +90,7 @@ DL_OFFSET = 1024
 
 def build(masked):
     em = Emitter()
+    em.wait_old = WAIT_OLD
 
     # ---- MFMA pairs in issue order -------------------------------------------------------
     pairs = []

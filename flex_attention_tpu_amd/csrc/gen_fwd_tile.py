@@ -57,6 +57,7 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 from gfx950_stream import Emitter, Op, ar, aset, schedule, vr, vset  # noqa: E402
 
 MIN_AHEAD = 2    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
+WAIT_OLD = 20    # a wait for LDS data also covers younger reads issued at least this many instructions ago
 CAP = 5          # instructions the scheduler puts between two MFMAs unless deadlines force more
 LOAD_FIRST = 2   # MFMA gap from which the first LDS-direct load of the next step may go out
 LOAD_EVERY = 2   # gaps between two of them
@@ -103,6 +104,7 @@ def v_p(c, x, u):
 
 def build(masked):
     em = Emitter()
+    em.wait_old = WAIT_OLD
     # MFMA pairs (2 MFMAs each), in issue order.  The two q blocks of a kv block are processed half a
     # stage apart: E(c, 0) runs under A(c+1)[ks 0-3] and B(c-1, 1), E(c, 1) under A(c+1)[ks 4-7] and
     # B(c, 0), so every softmax has MFMAs of both kinds to hide under.

@@ -45,6 +45,8 @@ class Emitter:
         self.c_read = {}           # reg -> time of the MFMA that read it as C without writing it
         self._skip = None
         self.lds_fifo = []         # outstanding LDS reads, oldest first: sets of dst regs
+        self.lds_time = []         # ... and when each was issued
+        self.wait_old = None       # a wait also covers younger reads issued at least this long ago
         self.stats = {"nop": 0, "wait": 0, "mfma": 0, "valu": 0, "lds": 0}
 
     def _raw(self, text, states=1):
@@ -68,12 +70,18 @@ class Emitter:
                 need = i
         if need is None:
             return
+        if self.wait_old is not None:
+            # younger reads that have very likely landed as well: waiting for them too costs nothing
+            # now and saves the separate wait of their first use
+            while need + 1 < len(self.lds_fifo) and self.lds_time[need + 1] <= self.t - self.wait_old:
+                need += 1
         newer = len(self.lds_fifo) - 1 - need
         self.stats["wait"] += 1
         self._raw(f"s_waitcnt lgkmcnt({min(newer, 15)})")
         # everything up to `need` has returned (and more, if the count was clamped)
         done = max(need + 1, len(self.lds_fifo) - 15) if newer > 15 else need + 1
         self.lds_fifo = self.lds_fifo[done:]
+        self.lds_time = self.lds_time[done:]
 
     def mfma(self, dst, a, b, c, dst_regs, a_regs, b_regs, c_regs):
         self._wait_lds(a_regs | b_regs | c_regs | dst_regs)
@@ -136,6 +144,7 @@ class Emitter:
             self.trans_w.pop(r, None)
         self._raw(text)
         self.lds_fifo.append(set(dst_regs))
+        self.lds_time.append(self.t - 1)
         self.stats["lds"] += 1
 
     def lds_direct_load(self, lds_imm, goff, gbase, ldsn="%[ldsn]"):
@@ -162,6 +171,7 @@ class Emitter:
                 self._need_gap(self.mfma_w[r], 12)
         self._raw(text)
         self.lds_fifo.append(set())
+        self.lds_time.append(self.t - 1)
         self.stats["lds"] += 1
 
     def raw(self, text):
@@ -193,6 +203,7 @@ class Emitter:
         if self.lds_fifo:
             self._raw("s_waitcnt lgkmcnt(0)")
             self.lds_fifo = []
+            self.lds_time = []
 
 
 class Op:
