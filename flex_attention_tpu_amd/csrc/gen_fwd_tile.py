@@ -25,7 +25,7 @@ The softmax is arranged so that the common case costs no arithmetic beyond exp, 
     behind the test: O^T, L, the block's scores and the -M registers are corrected by the lane's
     shift, and the chain of the next kv block, already in flight with the old -M, is corrected by a
     second such block at the start of its own softmax;
-  * the row sum L adds the fp32 values of p.
+  * the row sum L accumulates the bf16-rounded p (what the PV product uses) with v_dot2c.
 State per q row: M, Mt (true maximum = M + Mt), L.  The C++ epilogue turns them into the exact
 (m, l) outputs.
 
@@ -307,9 +307,9 @@ def build(masked):
             rare_earliest = max(rare_earliest, a_mfma(c + 1, 0, q) + 1)
         ops.append(block(rare, earliest=rare_earliest))
 
-        # p = 2^(score - M), packed to bf16 B operands.  The row sum adds the fp32 values in four
-        # interleaved partial sums (plain adds hide under the MFMAs; v_dot2c on the packed values
-        # measured 9 cycles apiece).
+        # p = 2^(score - M), packed to bf16 B operands.  The row sum adds the ROUNDED values (v_dot2c on
+        # the packed pairs): o = sum(p v) / sum(p) is then consistent, which matters where a row keeps
+        # few keys (o of a single-key row is exactly v, and delta = o . dO matches dP in the backward).
         def exps(g):
             for u in range(4):
                 e = 4 * g + u
@@ -324,24 +324,18 @@ def build(masked):
                 ops.append(valu(f"v_cvt_pk_bf16_f32 {vr(pr)}, {vr(s + e)}, {vr(s + e + 1)}", vset(pr), vset(s + e, 2),
                                 earliest=war, deadline=b_first(c, q, u2) - 1))
 
-        def sums(g):
-            for u in range(4):
-                e = 4 * g + u
-                if g == 1:
-                    ops.append(valu(f"v_add_f32_e32 {vr(T[u])}, {vr(s + u)}, {vr(s + e)}", vset(T[u]), vset(s + u) | vset(s + e)))
-                elif g > 1:
-                    ops.append(valu(f"v_add_f32_e32 {vr(T[u])}, {vr(T[u])}, {vr(s + e)}", vset(T[u]), vset(T[u]) | vset(s + e)))
+        # (one accumulator: splitting the chain over two registers measured slower)
+        def dots(g):
+            for h in range(2):
+                pr = v_p(c, q, g >> 1) + 2 * (g & 1) + h
+                ops.append(valu(f"v_dot2c_f32_bf16_e32 {L}, 0x3f803f80, {vr(pr)}", kL, kL | vset(pr)))
 
         exps(0)
         for g in range(4):
+            packs(g)
             if g < 3:
                 exps(g + 1)
-            sums(g)
-            packs(g)
-        ops.append(valu(f"v_add_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[1])}", vset(T[0]), vset(T[0]) | vset(T[1])))
-        ops.append(valu(f"v_add_f32_e32 {vr(T[2])}, {vr(T[2])}, {vr(T[3])}", vset(T[2]), vset(T[2]) | vset(T[3])))
-        ops.append(valu(f"v_add_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[2])}", vset(T[0]), vset(T[0]) | vset(T[2])))
-        ops.append(valu(f"v_add_f32_e32 {L}, {L}, {vr(T[0])}", kL, kL | vset(T[0])))
+            dots(g)
         ops[0].earliest = max(ops[0].earliest, a_mfma(c, 7, q) + 4)   # the chain's last result needs 12 wait states
         if c + 2 < 4:
             ops[-1].deadline = min(ops[-1].deadline or (1 << 30), a_mfma(c + 2, 0, q))  # A(c + 2) writes the same S registers
