@@ -193,6 +193,22 @@ def test_forward_compiled_kernel_on_request(F, monkeypatch):
         assert_close(name + " lse", m + l.log(), rm + rl.log(), torch.bfloat16)
 
 
+def test_single_key_rows_are_exact(F):
+    """Under a causal mask query 0 keeps one key: o[0] must be v[0] bit for bit (the row sum has to add
+    the same rounded probabilities the PV product uses) and its dq, P (dP - delta) with dP = delta,
+    must vanish; both also at the first row of every later q tile of a document."""
+    from flex_attention_tpu_amd import masks
+    sc = 1 / math.sqrt(128)
+    q, k, v, do = O.make_inputs(2, 4, 4, 512, 512, 128, dtype=torch.bfloat16, seed=29)
+    q, k, v, do = [x.to(DEV) for x in (q, k, v, do)]
+    mf, bf = masks.make_causal_mask_fns(128, 128)
+    o, l, m = _fwd(F, q, k, v, sc, mf, bf, None)
+    assert torch.equal(o[:, :, 0, :], v[:, :, 0, :])
+    d = F.compute_delta(o, do)
+    dq = _dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, None)
+    assert float(dq[:, :, 0, :].float().abs().max()) <= 2e-3
+
+
 def test_entry_points_reject_bad_arguments_on_gpu(F):
     q = torch.zeros(1, 2, 192, 128, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ValueError):  # 192 is not a multiple of the 128-row q tile
