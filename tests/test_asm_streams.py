@@ -248,3 +248,86 @@ def test_fwd_tile_streams_respect_hazards():
             elif pending:
                 assert not line.startswith(("v_mfma", "ds_", "global_load", "s_waitcnt")), (pending, line)
         assert pending is None
+
+
+def check_dataflow(lines, reads_per_fragment, reads_per_packed):
+    """What the hazard rules cannot see: that the scheduler kept every value alive until its users
+    were issued.  Re-derived from the text alone:
+      * a staging register filled by an LDS read is read by exactly `reads_per_fragment` MFMAs (as A
+        operand) before the next LDS read overwrites it;
+      * a register written by v_cvt_pk_bf16_f32 (P, dS) is read by exactly `reads_per_packed` MFMAs
+        (as B operand) before it is packed again;
+      * an accumulation chain (first MFMA: C input is not its destination) consists of 8 MFMAs, and
+        no other instruction touches its destination before the eighth has been issued."""
+    frag_reads, packed_reads, chain = {}, {}, {}
+    skip = None
+    for line in lines:
+        op, ops = split_operands(line)
+        if op.startswith("s_cbranch"):
+            skip = ops[0]  # the correction blocks only run when needed: not part of the steady flow
+            continue
+        if skip is not None:
+            if line.strip() == skip + ":":
+                skip = None
+            continue
+        if op.startswith("v_mfma"):
+            dst, a, b, c = (regs_of(x) for x in ops)
+            for r in a:
+                if r in frag_reads:
+                    frag_reads[r] += 1
+            for r in b:
+                if r in packed_reads:
+                    packed_reads[r] += 1
+            if dst and next(iter(dst))[0] == "v":  # S / dP chains live in VGPRs
+                key = min(dst)
+                if c != dst:
+                    assert chain.get(key, 8) == 8, f"a chain restarts after {chain[key]} MFMAs: {line}"
+                    chain[key] = 1
+                else:
+                    chain[key] += 1
+                    assert chain[key] <= 8, f"more than 8 MFMAs in a chain: {line}"
+        elif op.startswith("ds_read"):
+            for r in regs_of(ops[0]):
+                if r[0] == "a":
+                    assert frag_reads.get(r, reads_per_fragment) == reads_per_fragment, \
+                        f"fragment in {r} overwritten after {frag_reads[r]} of {reads_per_fragment} uses: {line}"
+                    frag_reads[r] = 0
+        elif op.startswith("v_"):
+            touched = set().union(*[regs_of(x) for x in ops]) if ops else set()
+            for key, n in chain.items():
+                tup = {(key[0], key[1] + i) for i in range(16)}
+                assert not (touched & tup) or n == 8, f"chain at {key} used after {n} of 8 MFMAs: {line}"
+            if op.startswith("v_cvt_pk_bf16"):
+                for r in regs_of(ops[0]):
+                    assert packed_reads.get(r, reads_per_packed) == reads_per_packed, \
+                        f"packed operand {r} rewritten after {packed_reads[r]} of {reads_per_packed} uses: {line}"
+                    packed_reads[r] = 0
+    # the stream repeats: what is still open at its end is consumed... nothing may be open
+    for r, n in frag_reads.items():
+        assert n == reads_per_fragment, f"fragment in {r} used {n} times at the end of the stream"
+    for r, n in packed_reads.items():
+        assert n == reads_per_packed, f"packed operand {r} used {n} times at the end of the stream"
+    assert all(n == 8 for n in chain.values())
+
+
+def test_streams_keep_values_alive_for_their_users():
+    import gen_dkv_tile, gen_dq_tile, gen_fwd_tile
+
+    for masked in (False, True):
+        # dk/dv, dq: every fragment feeds one MFMA, every packed P / dS register four (d blocks)
+        check_dataflow(gen_dkv_tile.build(masked).out, 1, 4)
+        check_dataflow(gen_dq_tile.build(masked).out, 1, 4)
+        # forward: a K row fragment feeds both q blocks, a V^T fragment likewise
+        check_dataflow(gen_fwd_tile.build(masked).out, 2, 4)
+
+
+def test_dataflow_check_catches_an_early_overwrite():
+    import gen_dq_tile
+
+    out = list(gen_dq_tile.build(False).out)
+    i = next(k for k, l in enumerate(out) if l.startswith("ds_read_b128 a[136:139]"))
+    j = next(k for k in range(i + 1, len(out)) if out[k].startswith("v_mfma") and "a[136:139]" in out[k])
+    moved = out[:i] + out[i + 1:j + 1] + [out[i]] + out[j + 1:]  # the read now follows its user
+    with pytest.raises(AssertionError):
+        check_dataflow(moved, 1, 4)
+
