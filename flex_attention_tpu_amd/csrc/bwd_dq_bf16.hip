@@ -474,37 +474,49 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
       return sSt[sIdx[2 * sidx]] == 2 && 2 * sidx + 1 < n_tiles && sSt[sIdx[2 * sidx + 1]] == 2;
     };
 
+    // first partial step at or behind `from` (n_steps if none): lanes look 64 steps ahead at a time
+    auto next_partial = [&](int from) {
+      int pos = from;
+      bool found = false;
+      while (!found && pos < n_steps) {
+        const int j = pos + lane;
+        const bool is_partial = j < n_steps && !step_full(j);
+        const unsigned long long hits = __ballot(is_partial);
+        if (hits != 0ull) {
+          pos += __builtin_ctzll(hits);
+          found = true;
+        } else {
+          pos = (pos + 64 < n_steps) ? pos + 64 : n_steps;
+        }
+      }
+      return __builtin_amdgcn_readfirstlane(pos);
+    };
     while (it < n_steps) {
-      const bool partial = __builtin_amdgcn_readfirstlane(step_full(it) ? 0 : 1) == 1;
-      int it_end = it + 1;
+      // A run: at most one partial step and the full steps next to it.  Either it starts with the
+      // partial step and goes on to the step before the next partial one, or it starts with full
+      // steps and ends with the first partial step behind them.
+      int it_part = next_partial(it);
+      int it_end;
+      if (it_part == it) {
+        it_end = next_partial(it + 1);
+      } else {
+        it_end = (it_part < n_steps) ? it_part + 1 : n_steps;
+      }
       unsigned km[2] = {0u, 0u};
-      if (partial) {
+      if (it_part < n_steps) {
         // the lane's keep bits: element e of kv block c sits at bit 16 (c & 1) + e of km[c >> 1]
 #pragma unroll
         for (int hx = 0; hx < 2; ++hx) {
-          const int e = 2 * it + hx;
+          const int e = 2 * it_part + hx;
           if (e >= n_tiles) continue;  // missing half: all dropped
           const int kt = __builtin_amdgcn_readfirstlane(sIdx[e]);
           const int state = __builtin_amdgcn_readfirstlane((int)sSt[kt]);
           km[hx] = state == 2 ? 0xffffffffu : keep_bits32<true>(a.mask, q_idx, kt * BN + 4 * hh, doc_i, a.mask.doc_k);
         }
       } else {
-        // the run of full steps ends before the next partial one: lanes look 64 steps ahead at a time
-        bool found = false;
-        while (!found && it_end < n_steps) {
-          const int j = it_end + lane;
-          const bool is_partial = j < n_steps && !step_full(j);
-          const unsigned long long hits = __ballot(is_partial);
-          if (hits != 0ull) {
-            it_end += __builtin_ctzll(hits);
-            found = true;
-          } else {
-            it_end = (it_end + 64 < n_steps) ? it_end + 64 : n_steps;
-          }
-        }
+        it_part = -1;
       }
-      it_end = __builtin_amdgcn_readfirstlane(it_end);
-      const int partial_flag = partial ? 1 : 0;
+      const int partial_flag = it_part;  // the step of the run that takes the masked stream (-1: none)
       // Work-group constants of the run loop, one table per wave (order: TABLE in gen_dq_tile.py),
       // written and read by the same wave.  A run that ends the item also names the next item's
       // first step (its values were fetched at the start of this item; only now are they touched).

@@ -31,7 +31,8 @@ physical-register constraints):
     %[m0], %[m1]  (partial steps) the lane's keep bits: bit 16 (c & 1) + e of m[c >> 1] is element e
                of the S^T accumulator of kv block c; dropped elements get dS = 0
     %[tbl]     LDS byte address of the wave's table of work-group constants (TABLE below)
-    %[it], %[kba1], %[kbb1], %[buf]  loop state (in/out); %[it_end], %[partial]  (in)
+    %[it], %[kba1], %[kbb1], %[buf]  loop state (in/out); %[it_end] (in); %[partial] (in): the step of the
+               run that is partial and takes the masked stream with the keep bits (-1: none)
 LDS layout of one step buffer (bytes): K tile 0, K tile 1, V tile 0, V tile 1 (16 KiB each); the two
 buffers are 64 KiB apart and the first starts at LDS address 0.
 """
@@ -208,8 +209,8 @@ def build(masked):
 
 
 def run_loop(full, masked):
-    """One asm statement: a run of consecutive steps [it, it_end) of one work item, all full or a
-    single partial one.  At entry the step's K / V tiles are resident in LDS buffer %[buf]; each pass
+    """One asm statement: a run of consecutive steps [it, it_end) of one work item, at most one of
+    them partial.  At entry the step's K / V tiles are resident in LDS buffer %[buf]; each pass
     computes the next step's addresses, streams the step (which copies the next step's tiles into the
     other buffer), synchronises the work-group and advances."""
     t0, t1, t2, t3 = S_T
@@ -253,7 +254,7 @@ def run_loop(full, masked):
         f"v_mov_b32_e32 {vr(V_KB2 + 1)}, {t3}",
         f"global_load_dword {vr(V_KB2)}, {vr(V_KB2)}, {S['idx']}",
         f"global_load_dword {vr(V_KB2 + 1)}, {vr(V_KB2 + 1)}, {S['idx']}",
-        f"s_cmp_eq_u32 {S['partial']}, 0",
+        f"s_cmp_lg_u32 {S['it']}, {S['partial']}",
         "s_cbranch_scc1 .Lfa_dq_full_%=",
     ]
     tail = [
