@@ -392,10 +392,10 @@ def main():
             macro(f"FA_DKV_PUT_KV_{ks}",
                   [f"v_accvgpr_write_b32 a{128 + 4 * ks + i}, %{2 + i}" for i in range(4)]
                   + [f"v_accvgpr_write_b32 a{160 + 4 * ks + i}, %{6 + i}" for i in range(4)])
-        # accumulator tile t (0-3 dv, 4-7 dk) into 16 dword operands (epilogue); the leading s_nop
-        # covers the MFMA -> read hazard of the last tile stream
+        # accumulator tile t (0-3 dv, 4-7 dk) into 16 dword operands (epilogue); the s_nop of the
+        # first one covers the MFMA -> read hazard of the last tile stream
         for t in range(8):
-            macro(f"FA_DKV_GET_ACC_{t}", ["s_nop 15"] + [f"v_accvgpr_read_b32 %{i}, a{16 * t + i}" for i in range(16)])
+            macro(f"FA_DKV_GET_ACC_{t}", (["s_nop 15"] if t == 0 else []) + [f"v_accvgpr_read_b32 %{i}, a{16 * t + i}" for i in range(16)])
         # (operand numbers: PUT_KV has two pinned outputs before its 8 inputs)
 
 

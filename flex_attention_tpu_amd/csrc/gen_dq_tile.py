@@ -44,7 +44,7 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 from gfx950_stream import Emitter, Op, ar, aset, schedule, vr, vset  # noqa: E402
 
 NSLOT = 8        # staging slots of 8 registers
-MIN_AHEAD = 2    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
+MIN_AHEAD = 3    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
 WAIT_OLD = 20    # a wait for LDS data also covers younger reads issued at least this many instructions ago
 CAP = 4          # instructions the scheduler puts between two MFMAs unless deadlines force more
 LOAD_FIRST = 2   # MFMA gap from which the first LDS-direct load of the next step may go out
@@ -301,9 +301,9 @@ def main():
             macro(f"FA_DQ_PUT_{ks}",
                   [f"v_accvgpr_write_b32 a{A_Q + 4 * ks + i}, %{2 + i}" for i in range(4)]
                   + [f"v_accvgpr_write_b32 a{A_DO + 4 * ks + i}, %{6 + i}" for i in range(4)])
-        # accumulator tile t into 16 dword operands; the s_nop covers the MFMA -> read hazard
+        # accumulator tile t into 16 dword operands; the s_nop of the first one covers the MFMA -> read hazard
         for t in range(4):
-            macro(f"FA_DQ_GET_ACC_{t}", ["s_nop 15"] + [f"v_accvgpr_read_b32 %{i}, a{A_DQ + 16 * t + i}" for i in range(16)])
+            macro(f"FA_DQ_GET_ACC_{t}", (["s_nop 15"] if t == 0 else []) + [f"v_accvgpr_read_b32 %{i}, a{A_DQ + 16 * t + i}" for i in range(16)])
 
 
 if __name__ == "__main__":

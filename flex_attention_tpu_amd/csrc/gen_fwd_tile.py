@@ -453,9 +453,10 @@ def main():
             macro(f"FA_FWD_PUT_{ks}",
                   [f"v_accvgpr_write_b32 a{A_Q + 4 * ks + i}, %{2 + i}" for i in range(4)]
                   + [f"v_accvgpr_write_b32 a{A_Q + 32 + 4 * ks + i}, %{6 + i}" for i in range(4)])
-        # accumulator tile t (q block t / 4, d block t % 4) into 16 dword operands
+        # accumulator tile t (q block t / 4, d block t % 4) into 16 dword operands (they are read in order:
+        # the s_nop of the first one covers the MFMA -> read hazard)
         for t in range(8):
-            macro(f"FA_FWD_GET_ACC_{t}", ["s_nop 15"] + [f"v_accvgpr_read_b32 %{i}, a{A_O + 16 * t + i}" for i in range(16)])
+            macro(f"FA_FWD_GET_ACC_{t}", (["s_nop 15"] if t == 0 else []) + [f"v_accvgpr_read_b32 %{i}, a{A_O + 16 * t + i}" for i in range(16)])
 
 
 if __name__ == "__main__":
