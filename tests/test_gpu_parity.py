@@ -209,6 +209,40 @@ def test_single_key_rows_are_exact(F):
     assert float(dq[:, :, 0, :].float().abs().max()) <= 2e-3
 
 
+@pytest.mark.parametrize("shape", [(1, 1, 1, 128, 128), (1, 2, 1, 384, 384), (2, 3, 3, 640, 640), (1, 4, 2, 1152, 1152),
+                                   (2, 16, 16, 2048, 2048), (3, 16, 4, 2048, 2048), (8, 32, 32, 1024, 1024),
+                                   (1, 2, 2, 256, 1280), (1, 2, 2, 1280, 256)], ids=lambda s: "x".join(map(str, s)))
+def test_odd_shapes_against_the_fp32_kernels(F, shape):
+    """Shapes around the edges of the work schedules (one tile, odd tile counts, a missing second q tile
+    of a forward pair, grids below, at and above one work-group per CU, GQA, Sq != Sk): the bf16
+    generated-stream kernels against the fp32 kernels (exact arithmetic, independent code) on the
+    same bf16-rounded inputs, plain and with masks that leave partial and empty tiles."""
+    from flex_attention_tpu_amd import masks
+    B, Hq, Hkv, Sq, Sk = shape
+    sc = 1 / math.sqrt(128)
+    g = torch.Generator().manual_seed(Sq + 7 * Sk + Hq)
+    q, do = (torch.randn(B, Hq, Sq, 128, generator=g).to(torch.bfloat16).to(DEV) for _ in range(2))
+    k, v = (torch.randn(B, Hkv, Sk, 128, generator=g).to(torch.bfloat16).to(DEV) for _ in range(2))
+    pairs = [(None, None)]
+    if Sq == Sk:
+        lens, left = [], Sq
+        while left > 0:
+            lens.append(min(left, 128 + (len(lens) * 97) % 300))
+            left -= lens[-1]
+        pairs += [masks.make_causal_mask_fns(128, 128), masks.make_causal_sliding_window_mask_fns(128, 128, 300),
+                  masks.make_jagged_mask_fns(128, 128, lens)]
+    for mf, bf in pairs:
+        def all_passes(q_, k_, v_, do_):
+            o, l, m = _fwd(F, q_, k_, v_, sc, mf, bf, None)
+            d = F.compute_delta(o, do_)
+            return (o, m + l.log(), _dq(F, q_, k_, v_, l, m, o, do_, d, sc, mf, bf, None)) + tuple(
+                _dkv(F, q_, k_, v_, l, m, do_, d, sc, mf, bf, None))
+        got = all_passes(q, k, v, do)
+        ref = all_passes(q.float(), k.float(), v.float(), do.float())
+        for name, a, b in zip(("o", "lse", "dq", "dk", "dv"), got, ref):
+            assert O.rel_l2(a.float().cpu(), b.cpu()) <= 1e-2, (name, shape)
+
+
 def test_entry_points_reject_bad_arguments_on_gpu(F):
     q = torch.zeros(1, 2, 192, 128, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ValueError):  # 192 is not a multiple of the 128-row q tile
