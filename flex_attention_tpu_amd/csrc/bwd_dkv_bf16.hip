@@ -348,11 +348,12 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   struct Geometry {
     int bhk, kb;
   };
+  const PersistentPlan plan = persistent_plan((int)blockIdx.x, n_wg, nKb);
   auto geometry = [&](int item) {
-    const int wg = persistent_item((int)blockIdx.x, item, (int)gridDim.x, n_wg, nKb);
     Geometry g;
-    g.bhk = __builtin_amdgcn_readfirstlane(wg / nKb);
-    g.kb = __builtin_amdgcn_readfirstlane(wg % nKb);
+    persistent_item(plan, (int)blockIdx.x, item, (int)gridDim.x, n_wg, nKb, g.bhk, g.kb);
+    g.bhk = __builtin_amdgcn_readfirstlane(g.bhk);
+    g.kb = __builtin_amdgcn_readfirstlane(g.kb);
     return g;
   };
   auto kv_offset = [&](const Geometry& g) { return ((size_t)g.bhk * a.Sk + (size_t)g.kb * BNK) * D; };

@@ -318,11 +318,15 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
     unsigned char st[kListRegs];   // state of kv tile tid + 256 j in the q tile's state row
   };
   const int n_items = n_wg / (int)gridDim.x;
+  const PersistentPlan plan = persistent_plan((int)blockIdx.x, n_wg, nQ);
+  const int group = a.Hq / a.Hkv;
+  const float inv_group = 1.0f / (float)group;
   auto geometry = [&](int item, int& bh, int& qb) {
-    const int wg = persistent_item((int)blockIdx.x, item, (int)gridDim.x, n_wg, nQ);
-    bh = wg / nQ;
-    qb = (gridDim.x == (unsigned)n_wg) ? nQ - 1 - (wg % nQ) : wg % nQ;  // one item each: longest first
+    persistent_item(plan, (int)blockIdx.x, item, (int)gridDim.x, n_wg, nQ, bh, qb);
+    if (gridDim.x == (unsigned)n_wg) qb = nQ - 1 - qb;  // one item each: longest first
   };
+  // (batch, kv head) pair of a (batch, q head) pair: bh / group, exact for the small numbers involved
+  auto kv_pair = [&](int bh) { return group == 1 ? bh : (int)(((float)bh + 0.5f) * inv_group); };
   auto fetch = [&](int item, ItemRegs& r) {
     int bh, qb;
     geometry(item, bh, qb);
@@ -411,14 +415,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   for (int item = 0; item < n_items; ++item) {
     int bh, qb;
     geometry(item, bh, qb);
-    const int b = bh / a.Hq;
-    const int h = bh % a.Hq;
-    const int hk = h / (a.Hq / a.Hkv);
     if (item > 0) __syncthreads();  // the previous item's LDS contents are dead from here
 
     bf16_t* dQg = static_cast<bf16_t*>(a.dq) + ((size_t)bh * a.Sq + (size_t)qb * BM) * D;
-    const bf16_t* Kg = static_cast<const bf16_t*>(a.k) + ((size_t)(b * a.Hkv + hk) * a.Sk) * D;
-    const bf16_t* Vg = static_cast<const bf16_t*>(a.v) + ((size_t)(b * a.Hkv + hk) * a.Sk) * D;
+    const bf16_t* Kg = static_cast<const bf16_t*>(a.k) + ((size_t)kv_pair(bh) * a.Sk) * D;
+    const bf16_t* Vg = static_cast<const bf16_t*>(a.v) + ((size_t)kv_pair(bh) * a.Sk) * D;
     const int q_idx = qb * BM + q_local;
     const int* tile_idx = a.map.idx + (size_t)qb * nK;
 
@@ -460,9 +461,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
     int bh_n = bh, qb_n = qb;
     if (has_next) geometry(item + 1, bh_n, qb_n);
     fetch(has_next ? item + 1 : item, pre);
-    const int b_n = bh_n / a.Hq, hk_n = (bh_n % a.Hq) / (a.Hq / a.Hkv);
-    const bf16_t* Kg_n = static_cast<const bf16_t*>(a.k) + ((size_t)(b_n * a.Hkv + hk_n) * a.Sk) * D;
-    const bf16_t* Vg_n = static_cast<const bf16_t*>(a.v) + ((size_t)(b_n * a.Hkv + hk_n) * a.Sk) * D;
+    const bf16_t* Kg_n = static_cast<const bf16_t*>(a.k) + ((size_t)kv_pair(bh_n) * a.Sk) * D;
+    const bf16_t* Vg_n = static_cast<const bf16_t*>(a.v) + ((size_t)kv_pair(bh_n) * a.Sk) * D;
 
     // carried: the kv tile indices of step it + 1 (clamped into the list)
     int it = 0;

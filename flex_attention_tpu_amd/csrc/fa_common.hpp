@@ -303,22 +303,44 @@ __host__ __device__ inline bool persistent_ok(int n_wg, int nKb) {
   if (nKb % 32 == 0) return true;
   return 32 % nKb == 0 && heads % (32 / nKb) == 0;
 }
-__device__ __forceinline__ int persistent_item(int j, int item, int grid, int n_wg, int nKb) {
-  if (grid == n_wg) return xcd_remap(j, n_wg);
-  const int share = j & 7, c = j >> 3;
-  const int heads = n_wg / 8 / nKb;
-  int head, kb;
+// The work-group's walk through its items with the divisions done once (the kernels locate an item
+// three times per item): `base` = first (batch, head) pair of the XCD's share, x, y = (c, blocks per
+// head / 32) when a head has at least 32 blocks, else (c / nKb, c % nKb), c = position in the XCD.
+struct PersistentPlan {
+  int base, x, y;
+};
+__device__ __forceinline__ PersistentPlan persistent_plan(int j, int n_wg, int nKb) {
+  PersistentPlan p;
+  const int c = j >> 3;
+  p.base = (j & 7) * (n_wg / 8 / nKb);
   if (nKb >= 32) {
-    const int m = nKb / 32;
-    head = item / m;
-    const int kx = c + 32 * (item % m);
-    kb = (head & 1) ? nKb - 1 - kx : kx;
+    p.x = c;
+    p.y = nKb / 32;
   } else {
-    const int r = 32 / nKb;
-    head = item * r + c / nKb;
-    kb = (item & 1) ? nKb - 1 - c % nKb : c % nKb;
+    p.x = c / nKb;
+    p.y = c % nKb;
   }
-  return (share * heads + head) * nKb + kb;
+  return p;
+}
+// (batch, head) pair and block of item number `item` of work-group j
+__device__ __forceinline__ void persistent_item(const PersistentPlan& p, int j, int item, int grid, int n_wg, int nKb,
+                                                int& head, int& kb) {
+  if (grid == n_wg) {  // one item per work-group, no static schedule
+    const int wg = xcd_remap(j, n_wg);
+    head = wg / nKb;
+    kb = wg % nKb;
+    return;
+  }
+  int hd;
+  if (nKb >= 32) {
+    hd = p.y == 1 ? item : item / p.y;
+    const int kx = p.x + 32 * (item - hd * p.y);
+    kb = (hd & 1) ? nKb - 1 - kx : kx;
+  } else {
+    hd = item * (32 / nKb) + p.x;
+    kb = (item & 1) ? nKb - 1 - p.y : p.y;
+  }
+  head = p.base + hd;
 }
 
 

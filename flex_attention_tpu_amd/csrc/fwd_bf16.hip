@@ -409,11 +409,15 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
     unsigned head;      // states of kv tile `lane` in both rows: where the merged list starts
   };
   const int n_items = n_wg / (int)gridDim.x;
+  const PersistentPlan plan = persistent_plan((int)blockIdx.x, n_wg, nQ2);
+  const int group = a.Hq / a.Hkv;
+  const float inv_group = 1.0f / (float)group;
   auto geometry = [&](int item, int& bh, int& qb2) {
-    const int wg = persistent_item((int)blockIdx.x, item, (int)gridDim.x, n_wg, nQ2);
-    bh = wg / nQ2;
-    qb2 = (gridDim.x == (unsigned)n_wg) ? nQ2 - 1 - (wg % nQ2) : wg % nQ2;  // one item each: longest first
+    persistent_item(plan, (int)blockIdx.x, item, (int)gridDim.x, n_wg, nQ2, bh, qb2);
+    if (gridDim.x == (unsigned)n_wg) qb2 = nQ2 - 1 - qb2;  // one item each: longest first
   };
+  // (batch, kv head) pair of a (batch, q head) pair: bh / group, exact for the small numbers involved
+  auto kv_pair = [&](int bh) { return group == 1 ? bh : (int)(((float)bh + 0.5f) * inv_group); };
   auto fetch = [&](int item, ItemRegs& r) {
     int bh, qb2;
     geometry(item, bh, qb2);
@@ -482,11 +486,8 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
   for (int item = 0; item < n_items; ++item) {
     int bh, qb2;
     geometry(item, bh, qb2);
-    const int b = bh / a.Hq;
-    const int h = bh % a.Hq;
-    const int hk = h / (a.Hq / a.Hkv);
-    const bf16_t* Kg = static_cast<const bf16_t*>(a.k) + ((size_t)(b * a.Hkv + hk) * a.Sk) * D;
-    const bf16_t* Vg = static_cast<const bf16_t*>(a.v) + ((size_t)(b * a.Hkv + hk) * a.Sk) * D;
+    const bf16_t* Kg = static_cast<const bf16_t*>(a.k) + ((size_t)kv_pair(bh) * a.Sk) * D;
+    const bf16_t* Vg = static_cast<const bf16_t*>(a.v) + ((size_t)kv_pair(bh) * a.Sk) * D;
     if (item > 0) __syncthreads();  // the previous item's list and state rows are dead from here
 
     // the two state rows into LDS, then the merged list of kv tiles that are non-empty for either
@@ -633,9 +634,8 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
         if (cnt >= 2 || (cnt == 1 && nK <= 64)) {
           const int ka_n = __builtin_ctzll(mask);
           const int kb_n = cnt >= 2 ? __builtin_ctzll(mask & (mask - 1ull)) : ka_n;
-          const int b_n = bh_n / a.Hq, hk_n = (bh_n % a.Hq) / (a.Hq / a.Hkv);
-          const bf16_t* Kg_n = static_cast<const bf16_t*>(a.k) + ((size_t)(b_n * a.Hkv + hk_n) * a.Sk) * D;
-          const bf16_t* Vg_n = static_cast<const bf16_t*>(a.v) + ((size_t)(b_n * a.Hkv + hk_n) * a.Sk) * D;
+          const bf16_t* Kg_n = static_cast<const bf16_t*>(a.k) + ((size_t)kv_pair(bh_n) * a.Sk) * D;
+          const bf16_t* Vg_n = static_cast<const bf16_t*>(a.v) + ((size_t)kv_pair(bh_n) * a.Sk) * D;
           if (lane == 0) {
             tbl[8] = (unsigned)ka_n;
             tbl[9] = (unsigned)kb_n;
