@@ -313,6 +313,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
 // shared memory, so the dynamic buffer starts at LDS address 0 (the run loop toggles buffers by
 // address bits).
 // ------------------------------------------------------------------------------------------------
+// ALIBI: the score gets slopes[h] (j - i) added (one query head per kv head only).  With j0 the middle of
+// the item's kv tile, exp2(t + a (j - i)) = exp2(t - a (i - j0)) 2^(a (j - j0)): the query's share joins
+// -lse in the S chain's accumulator input, the key's share is a factor of whole dk / dv rows that the
+// item epilogue applies, so the tile streams are those of the plain score.
+template <bool ALIBI>
 __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs a) {
   using namespace dkv_cfg;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
@@ -367,6 +372,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   struct ItemRegs {
     RowBlock k, v;                 // the wave's 32 K / V rows (full-row layout, see rows_load)
     int doc, n_tiles, qb0;         // list length and its first entry
+    float na2;                     // -slopes[head] log2(e) (ALIBI)
     int idx[kListRegs];            // q list entries tid + 256 j
     unsigned char part[kListRegs]; // state of q tile tid + 256 j against this kv tile
   };
@@ -386,6 +392,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     const int* tile_idx = a.map.idx + (size_t)g.kb * nQ;
     r.n_tiles = a.map.cnt[g.kb];
     r.qb0 = tile_idx[0];  // (nQ >= 1: always readable; used only if the list is not empty)
+    r.na2 = ALIBI ? -a.score.slopes[g.bhk % a.Hkv] * kLog2e : 0.f;
 #pragma unroll
     for (int j = 0; j < kListRegs; ++j) {
       const int t = tid_here + 256 * j;
@@ -396,6 +403,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   // What is left of an item's fetched values once its K / V fragments sit in their registers.
   struct ItemHead {
     int doc, n_tiles, qb0;
+    float na2;
     int idx[kListRegs];
     unsigned char part[kListRegs];
   };
@@ -426,6 +434,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     c.doc = r.doc;
     c.n_tiles = __builtin_amdgcn_readfirstlane(r.n_tiles);
     c.qb0 = __builtin_amdgcn_readfirstlane(r.qb0);
+    c.na2 = ALIBI ? __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, r.na2))) : 0.f;
 #pragma unroll
     for (int j = 0; j < kListRegs; ++j) {
       c.idx[j] = r.idx[j];
@@ -470,6 +479,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   const int* tile_idx = a.map.idx + (size_t)kb * nQ;
   const int n_tiles = cur.n_tiles;
   const int n_iter = n_tiles * group;
+  const float na2 = cur.na2;
+  const int kc = kb * BNK + BNK / 2;  // j0
   if (item > 0) __syncthreads();  // the previous item's list and row values are dead from here
 
   asm volatile(FA_DKV_ZERO_ACC
@@ -499,7 +510,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     const int row_p = tid_p & (BQ - 1);
     const float x = rowa[r0 + row_p], y = rowb[r0 + row_p];
     if (lse_wave) {  // (the streams want -lse: it is the accumulator input of the S chain)
-      sLse[buf * BQ + row_p] = (x > 0.f) ? -__builtin_fmaf(y, kLog2e, log2f(x)) : -__builtin_huge_valf();
+      float neg_lse = (x > 0.f) ? -__builtin_fmaf(y, kLog2e, log2f(x)) : -__builtin_huge_valf();
+      if (ALIBI) neg_lse = __builtin_fmaf((float)((int)r0 + row_p - kc), na2, neg_lse);
+      sLse[buf * BQ + row_p] = neg_lse;
     } else {  // (and -delta, for the dP chain)
       sDl[buf * BQ + row_p] = -x;
     }
@@ -523,7 +536,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     tbl[1] = (unsigned)(group - 1);
     tbl[2] = (unsigned)a.Sq;
     tbl[3] = base0 + (unsigned)w * 4096u;  // LDS address of the wave's first 1 KB block in buffer 0
-    tbl[4] = __builtin_bit_cast(unsigned, a.sm_scale * kLog2e);
+    tbl[4] = __builtin_bit_cast(unsigned, na2);
     tbl[5] = lse_wave ? 1u : 0u;
     tbl[6] = (unsigned)(size_t)tile_idx;
     tbl[7] = (unsigned)((size_t)tile_idx >> 32);
@@ -604,21 +617,32 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
           tbl[22] = (unsigned)(size_t)rowb_n;
           tbl[23] = (unsigned)((size_t)rowb_n >> 32);
           tbl[24] = (unsigned)qb0_n;
+          if (ALIBI) {
+            tbl[26] = __builtin_bit_cast(unsigned, pre.na2);
+            tbl[27] = (unsigned)(geo_n.kb * BNK + BNK / 2);
+          }
         }
         resident = true;
       }
     }
     // no scalar operands (see gen_dkv_tile.py): the loop state travels in VGPRs
-    asm volatile(FA_DKV_RUN
-                 : FA_DKV_PINNED(st), [it] "+v"(it), [p1] "+v"(p1), [g1] "+v"(g1), [p2] "+v"(p2), [qb1] "+v"(qb1),
-                   [buf] "+v"(buf), [r0] "+v"(ra[0]), [r1] "+v"(ra[1]), [r2] "+v"(ra[2]), [r3] "+v"(ra[3]),
-                   [r4] "+v"(ra[4]), [r5] "+v"(ra[5]), [r6] "+v"(ra[6]), [r7] "+v"(ra[7]), [t0] "+v"(ta[0]),
-                   [t1] "+v"(ta[1]), [t2] "+v"(ta[2]), [t3] "+v"(ta[3]), [t4] "+v"(ta[4]), [t5] "+v"(ta[5]),
-                   [t6] "+v"(ta[6]), [t7] "+v"(ta[7]), [la] "+v"(la), [lw] "+v"(lw)
-                 : [it_end] "v"(it_end), [partial] "v"(flags), [tbl] "v"(tbl_addr), [g0] "v"(loader.goff[0]),
-                   [g1v] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]), [g3] "v"(loader.goff[3]), [m0] "v"(km[0]),
-                   [m1] "v"(km[1]), [tid4] "v"(tid4)
-                 : "memory", "scc", "vcc", "m0", FA_DKV_RUN_SGPRS, "v67", FA_DKV_TILE_CLOBBERS);
+#define FA_DKV_CALL(RUN, ...)                                                                                    \
+  asm volatile(RUN                                                                                               \
+               : FA_DKV_PINNED(st), [it] "+v"(it), [p1] "+v"(p1), [g1] "+v"(g1), [p2] "+v"(p2), [qb1] "+v"(qb1), \
+                 [buf] "+v"(buf), [r0] "+v"(ra[0]), [r1] "+v"(ra[1]), [r2] "+v"(ra[2]), [r3] "+v"(ra[3]),       \
+                 [r4] "+v"(ra[4]), [r5] "+v"(ra[5]), [r6] "+v"(ra[6]), [r7] "+v"(ra[7]), [t0] "+v"(ta[0]),       \
+                 [t1] "+v"(ta[1]), [t2] "+v"(ta[2]), [t3] "+v"(ta[3]), [t4] "+v"(ta[4]), [t5] "+v"(ta[5]),       \
+                 [t6] "+v"(ta[6]), [t7] "+v"(ta[7]), [la] "+v"(la), [lw] "+v"(lw)                                \
+               : [it_end] "v"(it_end), [partial] "v"(flags), [tbl] "v"(tbl_addr), [g0] "v"(loader.goff[0]),      \
+                 [g1v] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]), [g3] "v"(loader.goff[3]), [m0] "v"(km[0]), \
+                 [m1] "v"(km[1]), [tid4] "v"(tid4), ##__VA_ARGS__                                                \
+               : "memory", "scc", "vcc", "m0", FA_DKV_RUN_SGPRS, "s101", "v67", FA_DKV_TILE_CLOBBERS)
+    if constexpr (ALIBI) {
+      FA_DKV_CALL(FA_DKV_RUN_ALIBI, [kc] "v"(kc));
+    } else {
+      FA_DKV_CALL(FA_DKV_RUN);
+    }
+#undef FA_DKV_CALL
     it = __builtin_amdgcn_readfirstlane(it);
     p1 = __builtin_amdgcn_readfirstlane(p1);
     buf = __builtin_amdgcn_readfirstlane(buf);
@@ -652,11 +676,14 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
       *reinterpret_cast<bf16x4*>(stage + MAT * 8192 + wr + (unsigned)(((4 * DB + g) ^ (row_here & 15)) << 4)) = out; \
     }                                                                                                              \
   }
-    // the streams leave the constant sm_scale out of dS: dk takes it here
-    FA_GET(0, st.dv[0], "a[0:15]", 1, 0, 1.f) FA_GET(1, st.dv[1], "a[16:31]", 1, 1, 1.f)
-    FA_GET(2, st.dv[2], "a[32:47]", 1, 2, 1.f) FA_GET(3, st.dv[3], "a[48:63]", 1, 3, 1.f)
-    FA_GET(4, st.dk[0], "a[64:79]", 0, 0, a.sm_scale) FA_GET(5, st.dk[1], "a[80:95]", 0, 1, a.sm_scale)
-    FA_GET(6, st.dk[2], "a[96:111]", 0, 2, a.sm_scale) FA_GET(7, st.dk[3], "a[112:127]", 0, 3, a.sm_scale)
+    // the streams leave the constant sm_scale out of dS: dk takes it here; and both take the key's
+    // share of a position bias
+    const float ej = ALIBI ? exp2f(-na2 * (float)((lane_here & 31) + 32 * w - BNK / 2)) : 1.f;
+    const float ek = a.sm_scale * ej;
+    FA_GET(0, st.dv[0], "a[0:15]", 1, 0, ej) FA_GET(1, st.dv[1], "a[16:31]", 1, 1, ej)
+    FA_GET(2, st.dv[2], "a[32:47]", 1, 2, ej) FA_GET(3, st.dv[3], "a[48:63]", 1, 3, ej)
+    FA_GET(4, st.dk[0], "a[64:79]", 0, 0, ek) FA_GET(5, st.dk[1], "a[80:95]", 0, 1, ek)
+    FA_GET(6, st.dk[2], "a[96:111]", 0, 2, ek) FA_GET(7, st.dk[3], "a[112:127]", 0, 3, ek)
 #undef FA_GET
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -689,9 +716,10 @@ static int launch_dkv(const BwdArgs& a, hipStream_t stream) {
   return check_launch("flexattn_bwd_dkv bf16");
 }
 
+template <bool ALIBI>
 static int launch_dkv_plain(const BwdArgs& a, hipStream_t stream) {
   using namespace dkv_cfg;
-  auto kern = bwd_dkv_bf16_d128_plain_kernel;
+  auto kern = bwd_dkv_bf16_d128_plain_kernel<ALIBI>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(dkv): %s", hipGetErrorString(attr));
@@ -705,8 +733,10 @@ int bwd_dkv_bf16_d128(const BwdArgs& a, hipStream_t stream) {
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
       // (the generated-stream kernel caches the q tile list in LDS)
-      return a.map.nq <= dkv_cfg::MAX_LIST ? launch_dkv_plain(a, stream) : launch_dkv<FLEXATTN_SCORE_NONE>(a, stream);
-    case FLEXATTN_SCORE_ALIBI: return launch_dkv<FLEXATTN_SCORE_ALIBI>(a, stream);
+      return a.map.nq <= dkv_cfg::MAX_LIST ? launch_dkv_plain<false>(a, stream) : launch_dkv<FLEXATTN_SCORE_NONE>(a, stream);
+    case FLEXATTN_SCORE_ALIBI:
+      return (a.map.nq <= dkv_cfg::MAX_LIST && a.Hq == a.Hkv) ? launch_dkv_plain<true>(a, stream)
+                                                              : launch_dkv<FLEXATTN_SCORE_ALIBI>(a, stream);
     case FLEXATTN_SCORE_SOFTCAP: return launch_dkv<FLEXATTN_SCORE_SOFTCAP>(a, stream);
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_dkv<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);
   }

@@ -175,7 +175,7 @@ __device__ __forceinline__ bool keep_elem(const MaskArgs& mk, int i, int j, int 
 // Keep bits of a lane's 32 elements in a 64-wide strip of the score matrix, for the generated
 // streams: element (c, g, u), c < 2, g < 4, u < 4, lies at offset 32 c + 8 g + u from `base` along the
 // varying index (keys when KEYS, the query is then `fixed`; queries otherwise, the key is `fixed`)
-// and owns bit 16 c + 4 g + u.  The purely causal mask, the common case, has a closed form: a
+// and owns bit 16 c + 4 g + u.  Causal and window masks, the common cases, have a closed form: a
 // 64-bit run of ones over the offsets, of which the even nibbles are the lane's elements.  Other
 // masks loop over the elements (rolled: the code stays small, these tiles are rare).
 __device__ __forceinline__ unsigned compress_even_nibbles(unsigned long long m) {
@@ -188,17 +188,26 @@ __device__ __forceinline__ unsigned compress_even_nibbles(unsigned long long m) 
 template <bool KEYS>
 __device__ __forceinline__ unsigned keep_bits32(const MaskArgs& mk, int fixed, int base, int doc_fixed,
                                                 const int* doc_var) {
-  if (mk.flags == FLEXATTN_MASK_CAUSAL) {
-    if (KEYS) {
-      // key base + off is kept iff off <= fixed - base
-      const int d = fixed - base;
-      const unsigned long long run = d < 0 ? 0ull : (d >= 63 ? ~0ull : ((2ull << d) - 1ull));
-      return compress_even_nibbles(run);
-    }
-    // query base + off is kept iff off >= fixed - base
+  if (mk.flags != 0 && (mk.flags & ~(FLEXATTN_MASK_CAUSAL | FLEXATTN_MASK_WINDOW)) == 0) {
+    // kept offsets form one interval [lo, hi]: with d = fixed - base, keys keep d - window < off <= d,
+    // queries keep d <= off < d + window (the causal bound resp. the window bound, where present)
     const int d = fixed - base;
-    const unsigned long long run = d <= 0 ? ~0ull : (d >= 64 ? 0ull : ~((1ull << d) - 1ull));
-    return compress_even_nibbles(run);
+    const bool causal = (mk.flags & FLEXATTN_MASK_CAUSAL) != 0;
+    const bool window = (mk.flags & FLEXATTN_MASK_WINDOW) != 0;
+    const int width = mk.window < (1 << 28) ? mk.window : (1 << 28);  // (indices stay far below: no overflow)
+    int lo, hi;
+    if (KEYS) {
+      lo = window ? d - width + 1 : 0;
+      hi = causal ? d : 63;
+    } else {
+      lo = causal ? d : 0;
+      hi = window ? width + d - 1 : 63;
+    }
+    if (lo < 0) lo = 0;
+    if (hi > 63) hi = 63;
+    if (lo > hi) return 0u;
+    const unsigned long long upto = hi == 63 ? ~0ull : ((2ull << hi) - 1ull);
+    return compress_even_nibbles(upto & ~((1ull << lo) - 1ull));
   }
   const bool has_doc = (mk.flags & FLEXATTN_MASK_DOC) != 0;
   unsigned bits = 0;

@@ -61,9 +61,9 @@ TILE = 16384
 # statement unreliably once many are live (it may keep a uniform value in a VGPR and print that
 # VGPR for an "s" operand), so the statement takes none: work-group constants come from a 16-dword
 # per-wave table in LDS, the loop state from VGPR operands, both through v_readfirstlane_b32.
-TABLE = ["n_tiles", "gmax", "sq", "w4k", "c2", "lsew", "idx_lo", "idx_hi", "qg_lo", "qg_hi", "dog_lo", "dog_hi",
+TABLE = ["n_tiles", "gmax", "sq", "w4k", "na2", "lsew", "idx_lo", "idx_hi", "qg_lo", "qg_hi", "dog_lo", "dog_hi",
          "rowa_lo", "rowa_hi", "rowb_lo", "rowb_hi"]  # order of the table's dwords
-SREG = {"n_tiles": "s60", "gmax": "s61", "sq": "s62", "w4k": "s63", "c2": "s64", "lsew": "s65",
+SREG = {"n_tiles": "s60", "gmax": "s61", "sq": "s62", "w4k": "s63", "na2": "s64", "lsew": "s65",
         "idx_lo": "s66", "idx_hi": "s67", "qg_lo": "s68", "qg_hi": "s69", "dog_lo": "s70", "dog_hi": "s71",
         "rowa_lo": "s72", "rowa_hi": "s73", "rowb_lo": "s74", "rowb_hi": "s75",
         "it": "s76", "p1": "s77", "g1": "s78", "p2": "s79", "qb1": "s80", "buf": "s81", "it_end": "s82", "partial": "s83",
@@ -74,6 +74,7 @@ V_TBL = 72      # 16 scratch VGPRs the table is read into at entry
 S_T = ["s84", "s85", "s86", "s87"]
 S_GQ0, S_GQ1, S_GD0, S_GD1, S_RA, S_RB = "s[88:89]", "s[90:91]", "s[92:93]", "s[94:95]", "s[96:97]", "s[98:99]"
 S_LDSN = "s100"
+S_KC = "s101"     # (position-bias variant) 128 kb + 64: the middle of the item's kv tile
 V_QB2 = 67      # q block index of the step after the next one, across the stream
 ROW_SLOT = 28   # MFMA slot at which the next step's lse / delta values are turned around
 V_ROW = 144     # 4 temporaries for that, inside pb[1] (first written by E(1), after ROW_SLOT)
@@ -88,7 +89,7 @@ V_TMP = 68    # 4 temporaries of the masked variant
 DL_OFFSET = 1024
 
 
-def build(masked):
+def build(masked, alibi=False):
     em = Emitter()
     em.wait_old = WAIT_OLD
 
@@ -260,6 +261,16 @@ def build(masked):
         e.valu(f"v_sub_f32_e32 {vr(rt_)}, {vr(rb_)}, {vr(rt_)}", vset(rt_), vset(rt_) | vset(rb_))
         e.valu(f"v_cmp_lt_f32_e32 vcc, 0, {vr(ra_)}", set(), vset(ra_))
         e.valu(f"v_cndmask_b32_e32 {vr(rt_)}, {vr(inf_)}, {vr(rt_)}, vcc", vset(rt_), vset(rt_) | vset(inf_))
+        if alibi:
+            # + slope log2(e) (j0 - i) for query row i = 128 qb1 + row of the next step, relative to the
+            # middle j0 of the kv tile (s64 holds -slope log2 e): the key's share 2^(slope log2(e) (j - j0))
+            # is a factor of whole dk / dv rows, which the epilogue applies
+            e.raw(f"s_lshl_b32 {S_T[0]}, s80, 7")
+            e.raw(f"s_sub_i32 {S_T[0]}, {S_T[0]}, {S_KC}")
+            e.valu(f"v_lshrrev_b32_e32 {vr(inf_)}, 2, %[tid4]", vset(inf_), set())
+            e.valu(f"v_add_u32_e32 {vr(inf_)}, {S_T[0]}, {vr(inf_)}", vset(inf_), vset(inf_))
+            e.valu(f"v_cvt_f32_i32_e32 {vr(inf_)}, {vr(inf_)}", vset(inf_), vset(inf_))
+            e.valu(f"v_fma_f32 {vr(rt_)}, {vr(inf_)}, s64, {vr(rt_)}", vset(rt_), vset(rt_) | vset(inf_))
         e.raw("s_cmp_lg_u32 s65, 0")
         e.raw("s_cselect_b64 vcc, -1, 0")
         e.raw("s_nop 3")
@@ -275,7 +286,7 @@ def build(masked):
     return em
 
 
-def run_loop(full, masked):
+def run_loop(full, masked, alibi=False):
     """One asm statement: a run of consecutive steps [it, it_end) of one work-group, all full or a
     single partial one.  At entry the step's Q / dO tiles and row values are resident in LDS buffer
     s81; each pass computes the next step's addresses, streams the tile (which copies the next
@@ -286,6 +297,10 @@ def run_loop(full, masked):
     entry += ["s_waitcnt lgkmcnt(0)"]  # (the streams count LDS operations from zero)
     entry += [f"v_readfirstlane_b32 {SREG[n]}, {vr(V_TBL + i)}" for i, n in enumerate(TABLE)]
     entry += [f"v_readfirstlane_b32 {SREG[n]}, %[{n}]" for n in STATE_IO + STATE_IN]
+    if alibi:
+        entry += [f"v_readfirstlane_b32 {S_KC}, %[kc]"]
+    switch = ([f"ds_read_b64 {vr(V_TBL + 10, 2)}, %[tbl] offset:104"] if alibi else [])
+    switch_sgprs = ([f"v_readfirstlane_b32 s64, {vr(V_TBL + 10)}", f"v_readfirstlane_b32 {S_KC}, {vr(V_TBL + 11)}"] if alibi else [])
     top = entry + [
         ".Lfa_dkv_loop_%=:",
         # The last step of the run that ends an item (bit 1 of the flags) copies the next item's first
@@ -298,8 +313,9 @@ def run_loop(full, masked):
         f"ds_read_b128 {vr(V_TBL, 4)}, %[tbl] offset:64",
         f"ds_read_b128 {vr(V_TBL + 4, 4)}, %[tbl] offset:80",
         f"ds_read_b32 {vr(V_TBL + 8)}, %[tbl] offset:96",
+    ] + switch + [
         "s_waitcnt lgkmcnt(0)",
-    ] + [f"v_readfirstlane_b32 s{68 + i}, {vr(V_TBL + i)}" for i in range(8)] + [
+    ] + [f"v_readfirstlane_b32 s{68 + i}, {vr(V_TBL + i)}" for i in range(8)] + switch_sgprs + [
         f"v_readfirstlane_b32 s80, {vr(V_TBL + 8)}",
         "s_mov_b32 s78, 0",
         ".Lfa_dkv_same_%=:",
@@ -373,10 +389,11 @@ def main():
         # one statement for both kinds of tile: a second asm statement on another control-flow
         # path makes the compiler shuffle the pinned registers around each of them
         full, masked = build(False), build(True)
-        lines = run_loop(full, masked)
-        f.write("#define FA_DKV_RUN \\\n")
-        f.write(" \\\n".join(f'  "{line}\\n"' for line in lines))
-        f.write("\n\n")
+        for name, alibi in (("FA_DKV_RUN", False), ("FA_DKV_RUN_ALIBI", True)):
+            lines = run_loop(build(False, alibi), build(True, alibi), alibi)
+            f.write(f"#define {name} \\\n")
+            f.write(" \\\n".join(f'  "{line}\\n"' for line in lines))
+            f.write("\n\n")
         for name, em in (("full", full), ("masked", masked)):
             print(f"{path}: {name}: {len(em.out)} instructions, {em.stats}", file=sys.stderr)
 

@@ -243,6 +243,34 @@ def test_odd_shapes_against_the_fp32_kernels(F, shape):
             assert O.rel_l2(a.float().cpu(), b.cpu()) <= 1e-2, (name, shape)
 
 
+@pytest.mark.parametrize("shape", [(1, 2, 128, 128), (2, 3, 640, 640), (2, 16, 2048, 2048), (8, 32, 1024, 1024), (1, 2, 256, 1280),
+                                   (1, 2, 1280, 256)], ids=lambda s: "x".join(map(str, s)))
+def test_position_bias_against_the_fp32_kernels(F, shape):
+    """slopes[h] (j - i) added to the scores (one query head per kv head: the generated-stream kernels
+    take it in) against the fp32 kernels, without a mask (the bias grows towards later keys), under
+    the causal mask and under a causal window, on grids below and above one work-group per CU."""
+    from flex_attention_tpu_amd import masks, scores
+    B, H, Sq, Sk = shape
+    sc = 1 / math.sqrt(128)
+    g = torch.Generator().manual_seed(Sq + 7 * Sk + H)
+    q, do = (torch.randn(B, H, Sq, 128, generator=g).to(torch.bfloat16).to(DEV) for _ in range(2))
+    k, v = (torch.randn(B, H, Sk, 128, generator=g).to(torch.bfloat16).to(DEV) for _ in range(2))
+    sfn = scores.make_alibi_global_score_fn(H)
+    pairs = [(None, None)]
+    if Sq == Sk:
+        pairs += [masks.make_causal_mask_fns(128, 128), masks.make_causal_sliding_window_mask_fns(128, 128, 300)]
+    for mf, bf in pairs:
+        def all_passes(q_, k_, v_, do_):
+            o, l, m = _fwd(F, q_, k_, v_, sc, mf, bf, sfn)
+            d = F.compute_delta(o, do_)
+            return (o, m + l.log(), _dq(F, q_, k_, v_, l, m, o, do_, d, sc, mf, bf, sfn)) + tuple(
+                _dkv(F, q_, k_, v_, l, m, do_, d, sc, mf, bf, sfn))
+        got = all_passes(q, k, v, do)
+        ref = all_passes(q.float(), k.float(), v.float(), do.float())
+        for name, a, b in zip(("o", "lse", "dq", "dk", "dv"), got, ref):
+            assert O.rel_l2(a.float().cpu(), b.cpu()) <= 1e-2, (name, shape, mf is None)
+
+
 def test_entry_points_reject_bad_arguments_on_gpu(F):
     q = torch.zeros(1, 2, 192, 128, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ValueError):  # 192 is not a multiple of the 128-row q tile
