@@ -279,6 +279,9 @@ static int launch_dq(const BwdArgs& a, hipStream_t stream) {
 // when persistent_ok() finds a balanced schedule.  The kernel has no static shared memory: the
 // dynamic buffer starts at LDS address 0 (the run loop toggles buffers by address bits).
 // ------------------------------------------------------------------------------------------------
+// ALIBI: the score gets slopes[h] (j - i) added; the streams then build the accumulator input of every
+// S chain, slope' (j - i) - lse, with one fp32 MFMA per 32-key block (see gen_dq_tile.py).
+template <bool ALIBI>
 __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs a) {
   using namespace dq_cfg;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
@@ -440,6 +443,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
                  : "={a[0:15]}"(st.dq[0]), "={a[16:31]}"(st.dq[1]), "={a[32:47]}"(st.dq[2]), "={a[48:63]}"(st.dq[3]));
     const float lse2 = (cur.l > 0.f) ? __builtin_fmaf(cur.m, kLog2e, log2f(cur.l)) : __builtin_huge_valf();
     const float delta = cur.delta;
+    // operands of the fp32 MFMA that makes the S chains' accumulator input under a position bias
+    const float a2 = ALIBI ? a.score.slopes[bh % a.Hq] * kLog2e : 0.f;
+    const float aone = hh ? (float)l32 : 1.f;
+    const float mulv = hh ? 0.f : a2;
+    const float addv = hh ? a2 : -lse2;
     const int doc_i = cur.doc;
     const int kb_first = cur.kb0;
     const int kb_second = (n_tiles > 1) ? cur.kb1 : kb_first;
@@ -547,16 +555,26 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
         }
       }
       // no scalar operands (see gen_dq_tile.py): the loop state travels in VGPRs
-      asm volatile(FA_DQ_RUN
-                   : FA_DQ_PINNED(st), [it] "+v"(it), [kba1] "+v"(kba1), [kbb1] "+v"(kbb1), [buf] "+v"(buf),
-                     [r0] "+v"(ra[0]), [r1] "+v"(ra[1]), [r2] "+v"(ra[2]), [r3] "+v"(ra[3]), [r4] "+v"(ra[4]),
-                     [r5] "+v"(ra[5]), [r6] "+v"(ra[6]), [r7] "+v"(ra[7]), [t0] "+v"(ta[0]), [t1] "+v"(ta[1]),
-                     [t2] "+v"(ta[2]), [t3] "+v"(ta[3]), [t4] "+v"(ta[4]), [t5] "+v"(ta[5]), [t6] "+v"(ta[6]),
-                     [t7] "+v"(ta[7])
-                   : [it_end] "v"(it_end), [partial] "v"(partial_flag), [tbl] "v"(tbl_addr), [lse] "v"(lse2),
-                     [dl] "v"(delta), [g0] "v"(loader.goff[0]), [g1v] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]),
-                     [g3] "v"(loader.goff[3]), [m0] "v"(km[0]), [m1] "v"(km[1])
-                   : "memory", "scc", "vcc", "m0", FA_DQ_RUN_SGPRS, FA_DQ_RUN_VGPRS);
+#define FA_DQ_CALL(RUN, ...)                                                                                     \
+  asm volatile(RUN                                                                                               \
+               : FA_DQ_PINNED(st), [it] "+v"(it), [kba1] "+v"(kba1), [kbb1] "+v"(kbb1), [buf] "+v"(buf),          \
+                 [r0] "+v"(ra[0]), [r1] "+v"(ra[1]), [r2] "+v"(ra[2]), [r3] "+v"(ra[3]), [r4] "+v"(ra[4]),        \
+                 [r5] "+v"(ra[5]), [r6] "+v"(ra[6]), [r7] "+v"(ra[7]), [t0] "+v"(ta[0]), [t1] "+v"(ta[1]),        \
+                 [t2] "+v"(ta[2]), [t3] "+v"(ta[3]), [t4] "+v"(ta[4]), [t5] "+v"(ta[5]), [t6] "+v"(ta[6]),        \
+                 [t7] "+v"(ta[7])                                                                                \
+               : [it_end] "v"(it_end), [partial] "v"(partial_flag), [tbl] "v"(tbl_addr), [dl] "v"(delta),         \
+                 [g0] "v"(loader.goff[0]), [g1v] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]),                  \
+                 [g3] "v"(loader.goff[3]), [m0] "v"(km[0]), [m1] "v"(km[1]), __VA_ARGS__                          \
+               : "memory", "scc", "vcc", "m0", FA_DQ_RUN_SGPRS, "s101", FA_DQ_RUN_VGPRS, "v184", "v185", "v186")
+      if constexpr (ALIBI) {
+        const int ka0 = __builtin_amdgcn_readfirstlane(entry(2 * it));
+        const int kb0 = __builtin_amdgcn_readfirstlane(entry(2 * it + 1));
+        FA_DQ_CALL(FA_DQ_RUN_ALIBI, [aone] "v"(aone), [mulv] "v"(mulv), [addv] "v"(addv), [iq] "v"(q_idx), [ka0] "v"(ka0),
+                   [kb0] "v"(kb0));
+      } else {
+        FA_DQ_CALL(FA_DQ_RUN, [lse] "v"(lse2));
+      }
+#undef FA_DQ_CALL
       it = __builtin_amdgcn_readfirstlane(it);
       buf = __builtin_amdgcn_readfirstlane(buf);
     }
@@ -609,9 +627,10 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   }  // work items
 }
 
+template <bool ALIBI>
 static int launch_dq_plain(const BwdArgs& a, hipStream_t stream) {
   using namespace dq_cfg;
-  auto kern = bwd_dq_bf16_d128_plain_kernel;
+  auto kern = bwd_dq_bf16_d128_plain_kernel<ALIBI>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, PLAIN_LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(dq): %s", hipGetErrorString(attr));
@@ -625,8 +644,9 @@ int bwd_dq_bf16_d128(const BwdArgs& a, hipStream_t stream) {
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
       // (the generated-stream kernel caches the kv list in LDS)
-      return a.map.nk <= dq_cfg::MAX_LIST ? launch_dq_plain(a, stream) : launch_dq<FLEXATTN_SCORE_NONE>(a, stream);
-    case FLEXATTN_SCORE_ALIBI: return launch_dq<FLEXATTN_SCORE_ALIBI>(a, stream);
+      return a.map.nk <= dq_cfg::MAX_LIST ? launch_dq_plain<false>(a, stream) : launch_dq<FLEXATTN_SCORE_NONE>(a, stream);
+    case FLEXATTN_SCORE_ALIBI:
+      return a.map.nk <= dq_cfg::MAX_LIST ? launch_dq_plain<true>(a, stream) : launch_dq<FLEXATTN_SCORE_ALIBI>(a, stream);
     case FLEXATTN_SCORE_SOFTCAP: return launch_dq<FLEXATTN_SCORE_SOFTCAP>(a, stream);
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_dq<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);
   }

@@ -54,7 +54,8 @@ DROP = ()        # instruction classes left out (--drop, timing studies only)
 TILE = 16384
 # No scalar operands: constants come from a per-wave table in LDS, loop state from VGPR operands
 # (the compiler may print a VGPR for an "s" operand once many uniform values are live).
-TABLE = ["n_tiles", "w4k", "c2", "n_steps", "idx_lo", "idx_hi", "kg_lo", "kg_hi", "vg_lo", "vg_hi", "kban", "kbbn",
+TABLE = ["n_tiles", "w4k", "c2", "n_steps",  # (c2: unused; its register holds a tile index in the position-bias variant)
+         "idx_lo", "idx_hi", "kg_lo", "kg_hi", "vg_lo", "vg_hi", "kban", "kbbn",
          "kgn_lo", "kgn_hi", "vgn_lo", "vgn_hi"]
 SREG = {"n_tiles": "s60", "w4k": "s61", "c2": "s62", "n_steps": "s63", "idx_lo": "s64", "idx_hi": "s65",
         "kg_lo": "s66", "kg_hi": "s67", "vg_lo": "s68", "vg_hi": "s69", "kban": "s70", "kbbn": "s71",
@@ -76,10 +77,35 @@ V_DS = 136       # dS^T as MFMA B operands: [c & 1][u] x 4 registers
 V_NL = 152       # -lse of the lane's q row, 16 copies: accumulator input of the first MFMA of an S chain
 V_ND = 168       # -delta of the lane's q row, 16 copies: accumulator input of the first MFMA of a dP chain
 V_END = 183
+# Position-bias variant (score + slope (j - i)): the accumulator input of a block's S chain,
+# slope' (j - i) - lse with slope' = slope log2(e), is itself a matrix product, [1, r] x [b; slope'] with r the
+# key's row in the block and b = slope' (j0 - i) - lse for the block's first key j0: one fp32 MFMA per
+# block writes it into the registers that hold -lse in the plain variant.
+#   %[aone]  A operand: 1.0 in lanes 0-31, float(lane - 32) in lanes 32-63
+#   %[mulv]  slope' in lanes 0-31, 0 in lanes 32-63;  %[addv]  -lse of the lane's q row resp. slope'
+#   %[iq]    the lane's q index;  %[ka0], %[kb0]  kv tiles of the run's first step
+V_B = [184, 185]  # B operands (alternating), 186: a temporary
+V_T = 186
+V_END_ALIBI = 186
+S_CUR = ["s62", "s101"]  # kv tiles of the current step
 A_DQ, A_Q, A_DO, A_STG = 0, 64, 96, 128
 
 
-def build(masked):
+def bias_ops(e, block, tile, odd):
+    """The accumulator input of S chain `block` (its parity picks the B register) for the 32 keys from
+    64 `tile` + 32 `odd` on."""
+    t0 = S_T[0]
+    b = V_B[block & 1]
+    e.raw(f"s_lshl_b32 {t0}, {tile}, 6")
+    if odd:
+        e.raw(f"s_add_u32 {t0}, {t0}, 32")
+    e.valu(f"v_sub_u32_e32 {vr(V_T)}, {t0}, %[iq]", vset(V_T), set())
+    e.valu(f"v_cvt_f32_i32_e32 {vr(V_T)}, {vr(V_T)}", vset(V_T), vset(V_T))
+    e.valu(f"v_fma_f32 {vr(b)}, %[mulv], {vr(V_T)}, %[addv]", vset(b), vset(V_T))
+    e.mfma_f32x2(vr(V_NL, 16), "%[aone]", vr(b), vset(V_NL, 16), set(), vset(b))
+
+
+def build(masked, alibi=False):
     em = Emitter()
     em.wait_old = WAIT_OLD
     pairs = []
@@ -203,12 +229,22 @@ def build(masked):
             k += 1
     chains.append(vm)
 
+    if alibi:
+        # block c's input: behind the first MFMA of A(c - 1), which reads the registers, and 20 wait
+        # states before the first one of A(c); block 0 of the next step at the end (its tiles: S_SEL)
+        bias = []
+        for c in (1, 2, 3, 4):
+            tile = S_SEL[0] if c == 4 else S_CUR[c >> 1]
+            bias.append(Op(lambda e, c=c, tile=tile: bias_ops(e, c, tile, c & 1), cost=6, earliest=first_A[c - 1] + 1,
+                           deadline=first_A[c] - 6 if c < 4 else None))
+        chains.append(bias)
+
     schedule(em, mfmas, chains, CAP)
     em.drain()
     return em
 
 
-def run_loop(full, masked):
+def run_loop(full, masked, alibi=False):
     """One asm statement: a run of consecutive steps [it, it_end) of one work item, at most one of
     them partial.  At entry the step's K / V tiles are resident in LDS buffer %[buf]; each pass
     computes the next step's addresses, streams the step (which copies the next step's tiles into the
@@ -220,7 +256,13 @@ def run_loop(full, masked):
     entry += ["s_waitcnt lgkmcnt(0)"]  # (the streams count LDS operations from zero)
     entry += [f"v_readfirstlane_b32 {S[n]}, {vr(V_TBL + i)}" for i, n in enumerate(TABLE)]
     entry += [f"v_readfirstlane_b32 {S[n]}, %[{n}]" for n in STATE_IO + STATE_IN]
-    entry += [f"v_sub_f32_e32 {vr(V_NL + e)}, 0, %[lse]" for e in range(16)]
+    if alibi:
+        pre = Emitter()
+        entry += [f"v_readfirstlane_b32 {S_CUR[0]}, %[ka0]", f"v_readfirstlane_b32 {S_CUR[1]}, %[kb0]"]
+        bias_ops(pre, 0, S_CUR[0], 0)   # (used by the first MFMA of the loop, more than 20 instructions on)
+        entry += pre.out
+    else:
+        entry += [f"v_sub_f32_e32 {vr(V_NL + e)}, 0, %[lse]" for e in range(16)]
     entry += [f"v_sub_f32_e32 {vr(V_ND + e)}, 0, %[dl]" for e in range(16)]
     top = entry + [".Lfa_dq_loop_%=:"]
     # On the item's last step the tiles copied "for the next step" are the first step of the next
@@ -266,6 +308,8 @@ def run_loop(full, masked):
         f"v_readfirstlane_b32 {S['kbb1']}, {vr(V_KB2 + 1)}",
         f"s_xor_b32 {S['buf']}, {S['buf']}, 1",
     ]
+    if alibi:
+        tail += [f"s_mov_b32 {S_CUR[0]}, {ka}", f"s_mov_b32 {S_CUR[1]}, {kb_}"]
     tail += [f"v_xor_b32_e32 %[r{i}], 0x10000, %[r{i}]" for i in range(8)]
     tail += [f"v_xor_b32_e32 %[t{i}], 0x10000, %[t{i}]" for i in range(8)]
     tail += [f"s_cmp_lt_u32 {S['it']}, {S['it_end']}", "s_cbranch_scc1 .Lfa_dq_loop_%="]
@@ -293,6 +337,7 @@ def main():
 
         full, masked = build(False), build(True)
         macro("FA_DQ_RUN", run_loop(full, masked))
+        macro("FA_DQ_RUN_ALIBI", run_loop(build(False, True), build(True, True), True))
         for name, em in (("full", full), ("masked", masked)):
             print(f"{args.out}: {name}: {len(em.out)} instructions, {em.stats}", file=sys.stderr)
         macro("FA_DQ_ZERO_ACC", [f"v_accvgpr_write_b32 a{A_DQ + i}, 0" for i in range(64)])

@@ -8,6 +8,7 @@ hardware leaves to software on gfx950:
     transcendental result-> VALU use                        1 wait state
     dot (v_dot2c) result -> other VALU use / overwrite      4 wait states (accumulating dots chain freely)
     MFMA reading C from registers other than its destination -> VALU write of them   12 wait states
+    fp32 MFMA (32x32x2, 16 pass) result -> any use                20 wait states
     LDS read result      -> any use                         s_waitcnt lgkmcnt (reads return in order)
 Registers are ("v", n) / ("a", n) pairs, or any other hashable key a generator chooses for a
 compiler-supplied operand it wants tracked (("op", name)).
@@ -39,6 +40,7 @@ class Emitter:
         self.out = []
         self.t = 0                 # wait states issued so far
         self.mfma_w = {}           # reg -> time of the MFMA that wrote it
+        self.mfma_lat = {}         # reg -> wait states its MFMA result needs (12 where not listed)
         self.valu_w = {}
         self.trans_w = {}
         self.dot_w = {}
@@ -87,7 +89,10 @@ class Emitter:
         self._wait_lds(a_regs | b_regs | c_regs | dst_regs)
         for r in a_regs | b_regs:
             if r in self.mfma_w:
-                self._need_gap(self.mfma_w[r], 12)
+                self._need_gap(self.mfma_w[r], self.mfma_lat.get(r, 12))
+        for r in c_regs - dst_regs:  # the result of another chain as accumulator input
+            if r in self.mfma_w:
+                self._need_gap(self.mfma_w[r], self.mfma_lat.get(r, 12))
         for r in a_regs | b_regs | c_regs:
             if r in self.valu_w:
                 self._need_gap(self.valu_w[r], 2)
@@ -99,16 +104,35 @@ class Emitter:
             self.c_read[r] = self.t - 1
         for r in dst_regs:
             self.mfma_w[r] = self.t - 1
+            self.mfma_lat.pop(r, None)
             self.valu_w.pop(r, None)
             self.trans_w.pop(r, None)
         self.stats["mfma"] += 1
+
+    def mfma_f32x2(self, dst, a, b, dst_regs, a_regs, b_regs):
+        """D[32 x 32] = A[32 x 2] B[2 x 32] in fp32 (16 passes, no accumulator input): one register of A
+        (lane: row lane % 32, k = lane / 32) and one of B (k = lane / 32, column lane % 32)."""
+        self._wait_lds(a_regs | b_regs | dst_regs)
+        for r in a_regs | b_regs:
+            if r in self.mfma_w:
+                self._need_gap(self.mfma_w[r], self.mfma_lat.get(r, 12))
+        for r in a_regs | b_regs | dst_regs:
+            if r in self.valu_w:
+                self._need_gap(self.valu_w[r], 2)
+        self._raw(f"v_mfma_f32_32x32x2_f32 {dst}, {a}, {b}, 0")
+        for r in dst_regs:
+            self.mfma_w[r] = self.t - 1
+            self.mfma_lat[r] = 20
+            self.valu_w.pop(r, None)
+            self.trans_w.pop(r, None)
+        self.stats["mfma32"] = self.stats.get("mfma32", 0) + 1
 
     def valu(self, text, dst_regs, src_regs, trans=False):
         is_dot = text.startswith("v_dot2c")
         self._wait_lds(dst_regs | src_regs)
         for r in dst_regs | src_regs:
             if r in self.mfma_w:
-                self._need_gap(self.mfma_w[r], 12)
+                self._need_gap(self.mfma_w[r], self.mfma_lat.get(r, 12))
         for r in src_regs:
             if r in self.trans_w:
                 self._need_gap(self.trans_w[r], 1)
@@ -136,7 +160,7 @@ class Emitter:
         self._wait_lds(dst_regs)  # an older read into the same registers must have landed
         for r in dst_regs:
             if r in self.mfma_w:
-                self._need_gap(self.mfma_w[r], 12)
+                self._need_gap(self.mfma_w[r], self.mfma_lat.get(r, 12))
             if r in self.c_read:
                 self._need_gap(self.c_read.pop(r), 12)
             self.mfma_w.pop(r, None)
@@ -168,7 +192,7 @@ class Emitter:
         self._wait_lds(src_regs)
         for r in src_regs:
             if r in self.mfma_w:
-                self._need_gap(self.mfma_w[r], 12)
+                self._need_gap(self.mfma_w[r], self.mfma_lat.get(r, 12))
         self._raw(text)
         self.lds_fifo.append(set())
         self.lds_time.append(self.t - 1)
@@ -181,7 +205,7 @@ class Emitter:
     def label(self, text):
         self._raw(text, 0)
 
-    _TRACKED = ("mfma_w", "valu_w", "trans_w", "dot_w", "c_read")
+    _TRACKED = ("mfma_w", "valu_w", "trans_w", "dot_w", "c_read")  # (mfma_lat only grows entries for live mfma_w ones)
 
     def skip_begin(self):
         """The instructions up to skip_end() may be jumped over by the branch emitted just before."""

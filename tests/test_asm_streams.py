@@ -39,6 +39,7 @@ def check_stream(lines):
     """Replays a stream; returns the number of instructions checked."""
     t = 0
     mfma_w, valu_w, trans_w, dot_w, c_read = {}, {}, {}, {}, {}
+    slow = set()  # registers whose MFMA result came from a 16-pass fp32 MFMA: 20 wait states instead of 12
     tracked = (mfma_w, valu_w, trans_w, dot_w, c_read)
     fifo = []  # outstanding LDS reads: destination register sets, oldest first
     skips = {}  # label -> (time behind the forward branch, copies of the tracked maps, LDS queue length)
@@ -46,6 +47,9 @@ def check_stream(lines):
 
     def gap(t_def):
         return t - t_def - 1
+
+    def mfma_done(r):
+        return r not in mfma_w or gap(mfma_w[r]) >= (20 if r in slow else 12)
 
     def lds_pending(regs):
         return any(dst & regs for dst in fifo)
@@ -86,24 +90,26 @@ def check_stream(lines):
             continue
         n += 1
         if op.startswith("v_mfma"):
+            assert op in ("v_mfma_f32_32x32x16_bf16", "v_mfma_f32_32x32x2_f32"), line
             dst, a, b, c = (regs_of(x) for x in ops)
             assert not lds_pending(dst | a | b | c), f"MFMA uses a register with an LDS read in flight: {line}"
             for r in a | b:
-                assert r not in mfma_w or gap(mfma_w[r]) >= 12, f"MFMA result used as A/B too early: {line}"
+                assert mfma_done(r), f"MFMA result used as A/B too early: {line}"
             for r in a | b | c | dst:
                 assert r not in valu_w or gap(valu_w[r]) >= 2, f"VALU result used by MFMA too early: {line}"
             for r in c - dst:
-                assert r not in mfma_w or gap(mfma_w[r]) >= 12, f"MFMA result used as C of another chain too early: {line}"
+                assert mfma_done(r), f"MFMA result used as C of another chain too early: {line}"
                 c_read[r] = t
             for r in dst:
                 mfma_w[r] = t
+                (slow.add if op.endswith("_f32") else slow.discard)(r)
                 valu_w.pop(r, None)
                 trans_w.pop(r, None)
         elif op.startswith("ds_read"):
             dst = regs_of(ops[0])
             assert not lds_pending(dst), f"LDS read into registers of an older read in flight: {line}"
             for r in dst:
-                assert r not in mfma_w or gap(mfma_w[r]) >= 12, f"LDS read overwrites a fresh MFMA result: {line}"
+                assert mfma_done(r), f"LDS read overwrites a fresh MFMA result: {line}"
                 mfma_w.pop(r, None)
                 valu_w.pop(r, None)
                 trans_w.pop(r, None)
@@ -119,7 +125,7 @@ def check_stream(lines):
             src = set().union(*[regs_of(x) for x in ops[1:]]) if len(ops) > 1 else set()
             assert not lds_pending(dst | src), f"VALU uses a register with an LDS read in flight: {line}"
             for r in dst | src:
-                assert r not in mfma_w or gap(mfma_w[r]) >= 12, f"VALU touches a fresh MFMA result: {line}"
+                assert mfma_done(r), f"VALU touches a fresh MFMA result: {line}"
             for r in src:
                 assert r not in trans_w or gap(trans_w[r]) >= 1, f"VALU reads a fresh transcendental result: {line}"
             is_dot = op.startswith("v_dot2c")  # accumulates into its destination
@@ -178,6 +184,12 @@ def test_hazard_checker_catches_a_bad_stream():
     bad = ["v_cvt_pk_bf16_f32 v136, v72, v73", "v_mfma_f32_32x32x16_bf16 a[0:15], v[192:195], v[136:139], a[0:15]"]
     with pytest.raises(AssertionError):
         check_stream(bad)
+    # the result of the 16-pass fp32 MFMA as accumulator input of another chain: 20 wait states
+    slow = ["v_mfma_f32_32x32x2_f32 v[152:167], v0, v184, 0", "s_nop 15",
+            "v_mfma_f32_32x32x16_bf16 v[72:87], a[128:131], a[64:67], v[152:167]"]
+    with pytest.raises(AssertionError):
+        check_stream(slow)
+    check_stream(slow[:2] + ["s_nop 3"] + slow[2:])
 
 
 def test_generated_include_matches_generator(tmp_path):
@@ -226,6 +238,12 @@ def test_dq_tile_streams_respect_hazards():
         assert em.stats["mfma"] == 96  # 4 kv blocks x (8 S + 8 dP + 8 dq)
         assert n == em.stats["mfma"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
         scratch_ok(em.out, 66, 183, 191)
+        # position-bias variant: one fp32 MFMA per block more, writing the S chains' accumulator input
+        em = g.build(masked, True)
+        n = check_stream(em.out)
+        assert em.stats["mfma"] == 96 and em.stats["mfma32"] == 4
+        assert n == em.stats["mfma"] + em.stats["mfma32"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
+        scratch_ok(em.out, 66, 186, 191)
 
 
 def test_fwd_tile_streams_respect_hazards():
