@@ -626,7 +626,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
       }
     }
     // no scalar operands (see gen_dkv_tile.py): the loop state travels in VGPRs
-#define FA_DKV_CALL(RUN, ...)                                                                                    \
+#define FA_DKV_CALL(RUN, CLOB_MORE, ...)                                                                                 \
   asm volatile(RUN                                                                                               \
                : FA_DKV_PINNED(st), [it] "+v"(it), [p1] "+v"(p1), [g1] "+v"(g1), [p2] "+v"(p2), [qb1] "+v"(qb1), \
                  [buf] "+v"(buf), [r0] "+v"(ra[0]), [r1] "+v"(ra[1]), [r2] "+v"(ra[2]), [r3] "+v"(ra[3]),       \
@@ -636,13 +636,15 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
                : [it_end] "v"(it_end), [partial] "v"(flags), [tbl] "v"(tbl_addr), [g0] "v"(loader.goff[0]),      \
                  [g1v] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]), [g3] "v"(loader.goff[3]), [m0] "v"(km[0]), \
                  [m1] "v"(km[1]), [tid4] "v"(tid4), ##__VA_ARGS__                                                \
-               : "memory", "scc", "vcc", "m0", FA_DKV_RUN_SGPRS, "s101", "v67", FA_DKV_TILE_CLOBBERS)
+               : "memory", "scc", "vcc", "m0", FA_DKV_RUN_SGPRS, "v67", FA_DKV_TILE_CLOBBERS CLOB_MORE)
     if constexpr (ALIBI) {
-      FA_DKV_CALL(FA_DKV_RUN_ALIBI, [kc] "v"(kc));
+#define FA_DKV_ALIBI_CLOBBERS , "s101"
+      FA_DKV_CALL(FA_DKV_RUN_ALIBI, FA_DKV_ALIBI_CLOBBERS, [kc] "v"(kc));
     } else {
-      FA_DKV_CALL(FA_DKV_RUN);
+      FA_DKV_CALL(FA_DKV_RUN, );
     }
 #undef FA_DKV_CALL
+#undef FA_DKV_ALIBI_CLOBBERS
     it = __builtin_amdgcn_readfirstlane(it);
     p1 = __builtin_amdgcn_readfirstlane(p1);
     buf = __builtin_amdgcn_readfirstlane(buf);

@@ -555,7 +555,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
         }
       }
       // no scalar operands (see gen_dq_tile.py): the loop state travels in VGPRs
-#define FA_DQ_CALL(RUN, ...)                                                                                     \
+#define FA_DQ_CALL(RUN, CLOB_MORE, ...)                                                                                   \
   asm volatile(RUN                                                                                               \
                : FA_DQ_PINNED(st), [it] "+v"(it), [kba1] "+v"(kba1), [kbb1] "+v"(kbb1), [buf] "+v"(buf),          \
                  [r0] "+v"(ra[0]), [r1] "+v"(ra[1]), [r2] "+v"(ra[2]), [r3] "+v"(ra[3]), [r4] "+v"(ra[4]),        \
@@ -565,16 +565,18 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
                : [it_end] "v"(it_end), [partial] "v"(partial_flag), [tbl] "v"(tbl_addr), [dl] "v"(delta),         \
                  [g0] "v"(loader.goff[0]), [g1v] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]),                  \
                  [g3] "v"(loader.goff[3]), [m0] "v"(km[0]), [m1] "v"(km[1]), __VA_ARGS__                          \
-               : "memory", "scc", "vcc", "m0", FA_DQ_RUN_SGPRS, "s101", FA_DQ_RUN_VGPRS, "v184", "v185", "v186")
+               : "memory", "scc", "vcc", "m0", FA_DQ_RUN_SGPRS, FA_DQ_RUN_VGPRS CLOB_MORE)
       if constexpr (ALIBI) {
         const int ka0 = __builtin_amdgcn_readfirstlane(entry(2 * it));
         const int kb0 = __builtin_amdgcn_readfirstlane(entry(2 * it + 1));
-        FA_DQ_CALL(FA_DQ_RUN_ALIBI, [aone] "v"(aone), [mulv] "v"(mulv), [addv] "v"(addv), [iq] "v"(q_idx), [ka0] "v"(ka0),
+#define FA_DQ_ALIBI_CLOBBERS , "s101", "v184", "v185", "v186"
+        FA_DQ_CALL(FA_DQ_RUN_ALIBI, FA_DQ_ALIBI_CLOBBERS, [aone] "v"(aone), [mulv] "v"(mulv), [addv] "v"(addv), [iq] "v"(q_idx), [ka0] "v"(ka0),
                    [kb0] "v"(kb0));
       } else {
-        FA_DQ_CALL(FA_DQ_RUN, [lse] "v"(lse2));
+        FA_DQ_CALL(FA_DQ_RUN, , [lse] "v"(lse2));
       }
 #undef FA_DQ_CALL
+#undef FA_DQ_ALIBI_CLOBBERS
       it = __builtin_amdgcn_readfirstlane(it);
       buf = __builtin_amdgcn_readfirstlane(buf);
     }

@@ -352,6 +352,9 @@ static int launch_fwd(const FwdArgs& a, hipStream_t stream) {
 // Work-groups are persistent (one per CU) when persistent_ok() finds a balanced schedule.  The
 // kernel has no static shared memory: the dynamic buffer starts at LDS address 0.
 // ------------------------------------------------------------------------------------------------
+// ALIBI: the score gets slopes[h] (j - i) added; the streams then build the accumulator input of every
+// S chain, slope' (j - i) - M, with one fp32 MFMA per chain (see gen_fwd_tile.py).
+template <bool ALIBI>
 __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) {
   using namespace fwd_cfg;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
@@ -531,8 +534,17 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
     // softmax state of the lane's two q rows (log2 domain): reference maximum M, running maximum
     // relative to it, sum of 2^(score - M)
     float M[2] = {0.f, 0.f}, Mt[2] = {kNegInf, kNegInf}, L[2] = {0.f, 0.f};
+    // operands of the fp32 MFMA that makes the S chains' accumulator input under a position bias
+    // (addv: -M of the lane's q row in lanes 0-31, which the streams keep up to date; the slope in the others)
+    const float a2 = ALIBI ? a.score.slopes[bh % a.Hq] * kLog2e : 0.f;
+    const float aone = hh ? (float)l32 : 1.f;
+    const float mulv = hh ? 0.f : a2;
+    float addv[2] = {hh ? a2 : 0.f, hh ? a2 : 0.f};
 
-    auto entry = [&](int e) { return sList[e < n_list ? e : n_list - 1]; };
+    // entry e of the list in the order the steps take it: ascending kv tiles; descending under a position
+    // bias, which (slopes are positive) is largest at the last key, so that the running maximum settles early
+    auto list_at = [&](int e) { return sList[ALIBI ? n_list - 1 - e : e]; };
+    auto entry = [&](int e) { return list_at(e < n_list ? e : n_list - 1); };
     if (n_list > 0 && !resident) {
       // first step into the current buffer (a missing second entry repeats the first: finite data, masked out)
       const int ka = __builtin_amdgcn_readfirstlane(entry(0));
@@ -583,7 +595,7 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
     }
     // a step is full when both of its entries exist and are full for both q tiles
     auto entry_full = [&](int e) {
-      const int k = sList[e];
+      const int k = list_at(e);
       return sStA[k] == 2 && sStB[k] == 2;
     };
     auto step_full = [&](int sidx) { return 2 * sidx + 1 < n_list && entry_full(2 * sidx) && entry_full(2 * sidx + 1); };
@@ -597,7 +609,7 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
         for (int hx = 0; hx < 2; ++hx) {
           const int e = 2 * it + hx;
           if (e >= n_list) continue;  // missing half: all dropped
-          const int k = __builtin_amdgcn_readfirstlane(sList[e]);
+          const int k = __builtin_amdgcn_readfirstlane(list_at(e));
 #pragma unroll
           for (int x = 0; x < 2; ++x) {
             const int state = __builtin_amdgcn_readfirstlane((int)(x == 0 ? sStA[k] : sStB[k]));
@@ -629,11 +641,40 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
         // The run ends the item: its last step copies the next item's first step, if that item's
         // list starts within kv tiles 0..63 (every wave fetched those states).  The fetched values
         // are first touched here, an item's length after their loads were issued.
-        const unsigned long long mask = __ballot(lane < nK && pre.head != 0u);
-        const int cnt = __builtin_popcountll(mask);
-        if (cnt >= 2 || (cnt == 1 && nK <= 64)) {
-          const int ka_n = __builtin_ctzll(mask);
-          const int kb_n = cnt >= 2 ? __builtin_ctzll(mask & (mask - 1ull)) : ka_n;
+        int ka_n = -1, kb_n = -1;
+        if constexpr (ALIBI) {
+          // the next item's list is walked from its end: its last two tiles, from the packed state words
+          // (lane tid of the work-group holds tiles tid + 256 j), wave maxima exchanged through LDS
+          int top1 = -1, top2 = -1;
+#pragma unroll
+          for (int j = 0; j < kListRegs; ++j) {
+            unsigned long long m = __ballot((((pre.sa | pre.sb) >> (8 * j)) & 0xffu) != 0u && tid + 256 * j < nK);
+            while (m != 0ull && top2 < w * 64 + 256 * j) {  // (tiles of a later j are larger: they replace both)
+              const int t = w * 64 + 256 * j + 63 - __builtin_clzll(m);
+              m &= ~(1ull << (63 - __builtin_clzll(m)));
+              if (t > top1) { top2 = top1; top1 = t; } else if (t > top2) { top2 = t; }
+            }
+          }
+          if (lane == 0) sCnt[w] = (top1 & 0xffff) | (top2 << 16);
+          __syncthreads();
+#pragma unroll
+          for (int ww = 0; ww < 4; ++ww) {
+            const int v = sCnt[ww];
+            const int c1 = (int)(short)(v & 0xffff), c2x = v >> 16;
+            if (c1 > ka_n) { kb_n = ka_n > c2x ? ka_n : c2x; ka_n = c1; } else if (c1 > kb_n) { kb_n = c1; }
+          }
+          __syncthreads();
+          if (kb_n < 0) kb_n = ka_n;
+        } else {
+          // ... if that item's list starts within kv tiles 0..63 (every wave fetched those states)
+          const unsigned long long mask = __ballot(lane < nK && pre.head != 0u);
+          const int cnt = __builtin_popcountll(mask);
+          if (cnt >= 2 || (cnt == 1 && nK <= 64)) {
+            ka_n = __builtin_ctzll(mask);
+            kb_n = cnt >= 2 ? __builtin_ctzll(mask & (mask - 1ull)) : ka_n;
+          }
+        }
+        if (ka_n >= 0) {
           const bf16_t* Kg_n = static_cast<const bf16_t*>(a.k) + ((size_t)kv_pair(bh_n) * a.Sk) * D;
           const bf16_t* Vg_n = static_cast<const bf16_t*>(a.v) + ((size_t)kv_pair(bh_n) * a.Sk) * D;
           if (lane == 0) {
@@ -648,17 +689,32 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
         }
       }
       // no scalar operands (see gen_fwd_tile.py): the loop state travels in VGPRs
-      asm volatile(FA_FWD_RUN
-                   : FA_FWD_PINNED(st), [it] "+v"(it), [kba1] "+v"(kba1), [kbb1] "+v"(kbb1), [buf] "+v"(buf),
-                     [M0] "+v"(M[0]), [M1] "+v"(M[1]), [Mt0] "+v"(Mt[0]), [Mt1] "+v"(Mt[1]), [L0] "+v"(L[0]),
-                     [L1] "+v"(L[1]), [r0] "+v"(ra[0]), [r1] "+v"(ra[1]), [r2] "+v"(ra[2]), [r3] "+v"(ra[3]),
-                     [r4] "+v"(ra[4]), [r5] "+v"(ra[5]), [r6] "+v"(ra[6]), [r7] "+v"(ra[7]), [t0] "+v"(ta[0]),
-                     [t1] "+v"(ta[1]), [t2] "+v"(ta[2]), [t3] "+v"(ta[3]), [t4] "+v"(ta[4]), [t5] "+v"(ta[5]),
-                     [t6] "+v"(ta[6]), [t7] "+v"(ta[7])
-                   : [it_end] "v"(it_end), [partial] "v"(partial_flag), [tbl] "v"(tbl_addr), [lst] "v"(lst_addr),
-                     [g0] "v"(loader.goff[0]), [g1v] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]),
-                     [g3] "v"(loader.goff[3]), [m0] "v"(km[0]), [m1] "v"(km[1]), [m2] "v"(km[2]), [m3] "v"(km[3])
-                   : "memory", "scc", "vcc", "m0", FA_FWD_RUN_SGPRS, FA_FWD_RUN_VGPRS);
+#define FA_FWD_CALL(RUN, OUT_MORE, CLOB_MORE, ...)                                                                         \
+  asm volatile(RUN                                                                                               \
+               : FA_FWD_PINNED(st), [it] "+v"(it), [kba1] "+v"(kba1), [kbb1] "+v"(kbb1), [buf] "+v"(buf),         \
+                 [M0] "+v"(M[0]), [M1] "+v"(M[1]), [Mt0] "+v"(Mt[0]), [Mt1] "+v"(Mt[1]), [L0] "+v"(L[0]),         \
+                 [L1] "+v"(L[1]), [r0] "+v"(ra[0]), [r1] "+v"(ra[1]), [r2] "+v"(ra[2]), [r3] "+v"(ra[3]),         \
+                 [r4] "+v"(ra[4]), [r5] "+v"(ra[5]), [r6] "+v"(ra[6]), [r7] "+v"(ra[7]), [t0] "+v"(ta[0]),        \
+                 [t1] "+v"(ta[1]), [t2] "+v"(ta[2]), [t3] "+v"(ta[3]), [t4] "+v"(ta[4]), [t5] "+v"(ta[5]),        \
+                 [t6] "+v"(ta[6]), [t7] "+v"(ta[7]) OUT_MORE                                                     \
+               : [it_end] "v"(it_end), [partial] "v"(partial_flag), [tbl] "v"(tbl_addr), [lst] "v"(lst_addr),     \
+                 [g0] "v"(loader.goff[0]), [g1v] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]),                  \
+                 [g3] "v"(loader.goff[3]), [m0] "v"(km[0]), [m1] "v"(km[1]), [m2] "v"(km[2]), [m3] "v"(km[3]),    \
+                 ##__VA_ARGS__                                                                                   \
+               : "memory", "scc", "vcc", "m0", FA_FWD_RUN_SGPRS, FA_FWD_RUN_VGPRS CLOB_MORE)
+#define FA_FWD_ADDV , [addv0] "+v"(addv[0]), [addv1] "+v"(addv[1])
+#define FA_FWD_ALIBI_CLOBBERS , "s101", "v200", "v201"
+      if constexpr (ALIBI) {
+        const int ka0 = __builtin_amdgcn_readfirstlane(entry(2 * it));
+        const int kb0 = __builtin_amdgcn_readfirstlane(entry(2 * it + 1));
+        FA_FWD_CALL(FA_FWD_RUN_ALIBI, FA_FWD_ADDV, FA_FWD_ALIBI_CLOBBERS, [aone] "v"(aone), [mulv] "v"(mulv), [iq] "v"(q_idx[0]), [ka0] "v"(ka0),
+                    [kb0] "v"(kb0));
+      } else {
+        FA_FWD_CALL(FA_FWD_RUN, , );
+      }
+#undef FA_FWD_ADDV
+#undef FA_FWD_ALIBI_CLOBBERS
+#undef FA_FWD_CALL
       it = __builtin_amdgcn_readfirstlane(it);
       buf = __builtin_amdgcn_readfirstlane(buf);
     }
@@ -730,9 +786,10 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
   }  // work items
 }
 
+template <bool ALIBI>
 static int launch_fwd_plain(const FwdArgs& a, hipStream_t stream) {
   using namespace fwd_cfg;
-  auto kern = fwd_bf16_d128_plain_kernel;
+  auto kern = fwd_bf16_d128_plain_kernel<ALIBI>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, PLAIN_LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(fwd): %s", hipGetErrorString(attr));
@@ -755,9 +812,12 @@ int fwd_bf16_d128(const FwdArgs& a, hipStream_t stream) {
       // The generated-stream kernel (one wave per SIMD, 64 q rows per wave) keeps the state rows and the
       // merged kv list in LDS and folds sm_scale into Q, hence the two conditions.
       return (fwd_stream_enabled() && a.map.nk <= fwd_cfg::MAX_LIST && a.sm_scale > 0.f)
-                 ? launch_fwd_plain(a, stream)
+                 ? launch_fwd_plain<false>(a, stream)
                  : launch_fwd<FLEXATTN_SCORE_NONE>(a, stream);
-    case FLEXATTN_SCORE_ALIBI: return launch_fwd<FLEXATTN_SCORE_ALIBI>(a, stream);
+    case FLEXATTN_SCORE_ALIBI:
+      return (fwd_stream_enabled() && a.map.nk <= fwd_cfg::MAX_LIST && a.sm_scale > 0.f)
+                 ? launch_fwd_plain<true>(a, stream)
+                 : launch_fwd<FLEXATTN_SCORE_ALIBI>(a, stream);
     case FLEXATTN_SCORE_SOFTCAP: return launch_fwd<FLEXATTN_SCORE_SOFTCAP>(a, stream);
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_fwd<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);
   }

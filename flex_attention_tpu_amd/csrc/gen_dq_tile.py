@@ -235,7 +235,7 @@ def build(masked, alibi=False):
         bias = []
         for c in (1, 2, 3, 4):
             tile = S_SEL[0] if c == 4 else S_CUR[c >> 1]
-            bias.append(Op(lambda e, c=c, tile=tile: bias_ops(e, c, tile, c & 1), cost=6, earliest=first_A[c - 1] + 1,
+            bias.append(Op(lambda e, c=c, tile=tile: bias_ops(e, c, tile, c & 1), cost=CAP, earliest=first_A[c - 1] + 1,
                            deadline=first_A[c] - 6 if c < 4 else None))
         chains.append(bias)
 

@@ -92,6 +92,36 @@ V_D = 196        # shift of M of q block 0, 1 (0 in lanes that keep theirs)
 V_AL = 198       # 2^-shift of q block 0, 1
 V_END = 199
 A_O, A_Q, A_STG = 0, 128, 192
+# Position-bias variant (score + slope (j - i)): the accumulator input of the S chain of kv block c, q block
+# x, slope' (j - i) - M with slope' = slope log2(e), is itself a matrix product, [1, r] x [b; slope'] with r the
+# key's row in the block and b = slope' (j0 - i) - M for the block's first key j0: one fp32 MFMA per
+# chain writes it into the registers that hold -M in the plain variant.
+#   %[aone]  A operand: 1.0 in lanes 0-31, float(lane - 32) in lanes 32-63
+#   %[mulv]  slope' in lanes 0-31, 0 in lanes 32-63
+#   %[addv0], %[addv1]  -M of the lane's q row resp. slope' (in/out: they follow M)
+#   %[iq]    the lane's q index in q block 0 (q block 1: 128 more);  %[ka0], %[kb0]  kv tiles of the run's first step
+# The kv list is walked from its end: with a positive slope the bias grows with the key index, so the
+# running maximum settles in the first steps instead of moving the reference M at every block.
+V_B = [200, 201]   # B operands (alternating)
+V_T = V_TMP + 9
+V_END_ALIBI = 201
+S_CUR = ["s62", "s101"]  # kv tiles of the current step
+
+
+def bias_ops(e, c, q, tile):
+    """The accumulator input of the S chain (c, q): keys from 64 `tile` + 32 (c & 1) on, q rows 128 q on."""
+    t0 = S_T[0]
+    b = V_B[q]
+    off = 32 * (c & 1) - 128 * q
+    e.raw(f"s_lshl_b32 {t0}, {tile}, 6")
+    if off > 0:
+        e.raw(f"s_add_u32 {t0}, {t0}, {off}")
+    elif off < 0:
+        e.raw(f"s_sub_u32 {t0}, {t0}, {-off}")
+    e.valu(f"v_sub_u32_e32 {vr(V_T)}, {t0}, %[iq]", vset(V_T), set())
+    e.valu(f"v_cvt_f32_i32_e32 {vr(V_T)}, {vr(V_T)}", vset(V_T), vset(V_T))
+    e.valu(f"v_fma_f32 {vr(b)}, %[mulv], {vr(V_T)}, %[addv{q}]", vset(b), vset(V_T) | {("op", f"addv{q}")})
+    e.mfma_f32x2(vr(V_NEGM + 16 * q, 16), "%[aone]", vr(b), vset(V_NEGM + 16 * q, 16), set(), vset(b))
 
 
 def v_s(c, x):
@@ -102,7 +132,7 @@ def v_p(c, x, u):
     return V_P0 + 8 * x + 4 * u
 
 
-def build(masked):
+def build(masked, alibi=False):
     em = Emitter()
     em.wait_old = WAIT_OLD
     # MFMA pairs (2 MFMAs each), in issue order.  The two q blocks of a kv block are processed half a
@@ -281,7 +311,10 @@ def build(masked):
             rare.append(("raw", "s_and_b64 vcc, vcc, s[86:87]"))
         rare += [("raw", f"s_cbranch_vccz .Lfa_fwd_{tag}_keep{c}{q}_%="), ("skip_begin",), ("raw", "s_nop 3"),
                  ("valu", f"v_cndmask_b32_e32 {vr(D)}, 0, {Mt}, vcc", vset(D), kMt, False),                 # the lane's shift
-                 ("valu", f"v_exp_f32_e64 {vr(AL)}, -{vr(D)}", vset(AL), vset(D), True),
+                 # (2^-shift, the shift held above -126: what was summed against a reference more than 2^126 too
+                 # high has been flushed to zero and must stay zero, not become 0 x inf)
+                 ("valu", f"v_max_f32_e32 {vr(AL)}, 0xc2fc0000, {vr(D)}", vset(AL), vset(D), False),
+                 ("valu", f"v_exp_f32_e64 {vr(AL)}, -{vr(AL)}", vset(AL), vset(AL), True),
                  ("valu", f"v_sub_f32_e32 {Mt}, {Mt}, {vr(D)}", kMt, kMt | vset(D), False),
                  ("valu", f"v_add_f32_e32 {M}, {M}, {vr(D)}", kM, kM | vset(D), False),
                  ("valu", f"v_mul_f32_e32 {L}, {L}, {vr(AL)}", kL, kL | vset(AL), False)]
@@ -295,6 +328,12 @@ def build(masked):
             rare.append(("valu", f"v_sub_f32_e32 {vr(s + e)}, {vr(s + e)}, {vr(D)}", vset(s + e), vset(s + e) | vset(D), False))
         for e in range(16):
             rare.append(("valu", f"v_sub_f32_e32 {vr(negm + e)}, {vr(negm + e)}, {vr(D)}", vset(negm + e), vset(negm + e) | vset(D), False))
+        if alibi:
+            # -M in lanes 0-31 of the B operand's source follows M (lanes 32-63 hold the slope)
+            kA = {("op", f"addv{q}")}
+            rare += [("raw", "s_mov_b32 s86, -1"), ("raw", "s_mov_b32 s87, 0"),
+                     ("valu", f"v_cndmask_b32_e64 {vr(T[5])}, 0, {vr(D)}, s[86:87]", vset(T[5]), vset(D), False),
+                     ("valu", f"v_sub_f32_e32 %[addv{q}], %[addv{q}], {vr(T[5])}", kA, kA | vset(T[5]), False)]
         if c < 3:
             rare.append(("raw", f"s_mov_b32 {S_PEND[q]}, 1"))  # (kv block c + 1 of this step is in flight; block 0 of the next step is not)
         rare += [("skip_end",), ("label", f".Lfa_fwd_{tag}_keep{c}{q}_%=:")]
@@ -305,6 +344,14 @@ def build(masked):
             rare_earliest = b_last(c - 1, q, 1) + 1
         if c < 3:
             rare_earliest = max(rare_earliest, a_mfma(c + 1, 0, q) + 1)
+        if alibi and c < 3:
+            # The accumulator input of chain (c + 2, q) (block 0 of the next step for c = 2) right in front
+            # of the block that moves M, which corrects it like the plain -M: chain (c + 1, q), which read
+            # the registers, is out by then; 20 wait states before the chain's first MFMA.
+            cn = c + 2
+            tile = S_CUR[1] if cn < 4 else S_SEL[0]
+            ops.append(Op(lambda e: bias_ops(e, cn & 3, q, tile), cost=CAP, earliest=rare_earliest,
+                          deadline=a_mfma(cn, 0, q) - 6 if cn < 4 else None))
         ops.append(block(rare, earliest=rare_earliest))
 
         # p = 2^(score - M), packed to bf16 B operands.  The row sum adds the ROUNDED values (v_dot2c on
@@ -347,6 +394,10 @@ def build(masked):
         for q in range(2):
             soft.extend(softmax_chain(c, q))
     chains = [soft, [op for _, op in reads]]
+    if alibi:
+        # chain (1, q): behind the first MFMA of chain (0, q) and before this step's first softmax
+        chains.append([Op(lambda e, q=q: bias_ops(e, 1, q, S_CUR[0]), cost=CAP, earliest=2 + q, deadline=a_mfma(1, 0, q) - 6)
+                       for q in range(2)])
 
     # ---- next step's K / V tiles: 16 LDS-direct loads per wave spread over the stream ------------
     vm = []
@@ -369,7 +420,7 @@ def build(masked):
     return em
 
 
-def run_loop(full, masked):
+def run_loop(full, masked, alibi=False):
     """One asm statement: a run of consecutive steps [it, it_end) of one work item, all full or a
     single partial one.  At entry the step's K / V tiles are resident in LDS buffer %[buf]."""
     t0, t1, t2, t3 = S_T
@@ -379,7 +430,14 @@ def run_loop(full, masked):
     entry += [f"v_readfirstlane_b32 {S[n]}, {vr(V_TBL + i)}" for i, n in enumerate(TABLE)]
     entry += [f"v_readfirstlane_b32 {S[n]}, %[{n}]" for n in STATE_IO + STATE_IN]
     entry += [f"v_mov_b32_e32 {vr(V_TAU)}, {TAU}", f"s_mov_b32 {S_PEND[0]}, 0", f"s_mov_b32 {S_PEND[1]}, 0"]
-    entry += [f"v_sub_f32_e32 {vr(V_NEGM + 16 * q + e)}, 0, %[M{q}]" for q in range(2) for e in range(16)]
+    if alibi:
+        pre = Emitter()
+        entry += [f"v_readfirstlane_b32 {S_CUR[0]}, %[ka0]", f"v_readfirstlane_b32 {S_CUR[1]}, %[kb0]"]
+        for q in range(2):
+            bias_ops(pre, 0, q, S_CUR[0])   # (used by the first MFMAs of the loop, more than 20 instructions on)
+        entry += pre.out
+    else:
+        entry += [f"v_sub_f32_e32 {vr(V_NEGM + 16 * q + e)}, 0, %[M{q}]" for q in range(2) for e in range(16)]
     top = entry + [".Lfa_fwd_loop_%=:"]
     # on the item's last step the tiles copied "for the next step" are the first step of the next
     # work item (from the table; with no next item they repeat this one's)
@@ -405,6 +463,7 @@ def run_loop(full, masked):
         f"s_min_u32 {t2}, {t0}, {t1}",
         f"s_add_u32 {t0}, {t0}, 1",
         f"s_min_u32 {t3}, {t0}, {t1}",
+    ] + ([f"s_sub_u32 {t2}, {t1}, {t2}", f"s_sub_u32 {t3}, {t1}, {t3}"] if alibi else []) + [  # (the list is walked from its end)
         f"s_lshl_b32 {t2}, {t2}, 2",
         f"s_lshl_b32 {t3}, {t3}, 2",
         f"v_add_u32_e32 {vr(V_KB2)}, {t2}, %[lst]",
@@ -418,6 +477,8 @@ def run_loop(full, masked):
         f"v_readfirstlane_b32 {S['kbb1']}, {vr(V_KB2 + 1)}",
         f"s_xor_b32 {S['buf']}, {S['buf']}, 1",
     ]
+    if alibi:
+        tail += [f"s_mov_b32 {S_CUR[0]}, {ka}", f"s_mov_b32 {S_CUR[1]}, {kb_}"]
     tail += [f"v_xor_b32_e32 %[r{i}], 0x10000, %[r{i}]" for i in range(8)]
     tail += [f"v_xor_b32_e32 %[t{i}], 0x10000, %[t{i}]" for i in range(8)]
     tail += [f"s_cmp_lt_u32 {S['it']}, {S['it_end']}", "s_cbranch_scc1 .Lfa_fwd_loop_%="]
@@ -445,6 +506,7 @@ def main():
 
         full, masked = build(False), build(True)
         macro("FA_FWD_RUN", run_loop(full, masked))
+        macro("FA_FWD_RUN_ALIBI", run_loop(build(False, True), build(True, True), True))
         for name, em in (("full", full), ("masked", masked)):
             print(f"{args.out}: {name}: {len(em.out)} instructions, {em.stats}", file=sys.stderr)
         macro("FA_FWD_ZERO_ACC", [f"v_accvgpr_write_b32 a{A_O + i}, 0" for i in range(128)])

@@ -255,10 +255,16 @@ def test_fwd_tile_streams_respect_hazards():
         assert em.stats["mfma"] == 128  # 4 kv blocks x 2 q blocks x (8 S + 8 PV)
         assert n == em.stats["mfma"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
         scratch_ok(em.out, 66, 199, 255)
+        # position-bias variant: one fp32 MFMA per S chain more, writing the chain's accumulator input
+        ab = g.build(masked, True)
+        nb = check_stream(ab.out)
+        assert ab.stats["mfma"] == 128 and ab.stats["mfma32"] == 8
+        assert nb == ab.stats["mfma"] + ab.stats["mfma32"] + ab.stats["valu"] + ab.stats["lds"] + ab.stats["vmem"]
+        scratch_ok(ab.out, 66, 201, 255)
         # between a forward branch and its label there is only VALU / scalar work: a skipped MFMA,
         # LDS read or wait would break the stream's bookkeeping
         pending = None
-        for line in em.out:
+        for line in em.out + ab.out:
             if line.startswith("s_cbranch"):
                 pending = line.split()[1]
             elif pending and line.strip() == pending + ":":
