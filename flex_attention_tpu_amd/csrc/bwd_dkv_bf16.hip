@@ -13,6 +13,7 @@
 // The plain score runs generated, hand-scheduled instruction streams (gen_dkv_tile.py ->
 // bwd_dkv_tile.inc) that software-pipeline MFMA, VALU and LDS work inside the wave with a fixed
 // register allocation; score modifications run the compiled C++ kernel.
+#include <cstdlib>
 #include "fa_common.hpp"
 #include "launch.hpp"
 #include "tile_io.hpp"
@@ -49,7 +50,7 @@ constexpr int BQ = 128;   // q rows per step (two 64-row LDS tiles)
 constexpr int D = 128;
 constexpr int MAX_LIST = 1024;  // longest q tile list the plain-score kernel caches in LDS
 // (Q, dO) x 2 buffers x 2 tiles, lse x2, delta x2, run-loop tables, cached q tile list and its partial flags
-constexpr int LDS_BYTES = 8 * kTileElems * 2 + 4 * BQ * 4 + 4 * 32 * 4 + MAX_LIST * 5;
+constexpr int LDS_BYTES = 8 * kTileElems * 2 + 4 * BQ * 4 + 4 * 32 * 4 + MAX_LIST * 5 + kDocStageBytes;
 }  // namespace dkv_cfg
 
 
@@ -317,9 +318,18 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
 // the item's kv tile, exp2(t + a (j - i)) = exp2(t - a (i - j0)) 2^(a (j - j0)): the query's share joins
 // -lse in the S chain's accumulator input, the key's share is a factor of whole dk / dv rows that the
 // item epilogue applies, so the tile streams are those of the plain score.
-template <bool ALIBI>
+// SOFTCAP: s' = cap tanh(s / cap).  K goes in multiplied by 2 log2(e) sm_scale / cap, the streams turn the
+// chain's result u into r = 1 / (2^u + 1) (tanh = 1 - 2 r), the exponent (cap' - lse) - 2 cap' r with
+// cap' = cap log2(e) (LDS holds cap' - lse) and dS = P dP' r (1 - r); the factor 4 of 1 - tanh^2 = 4 r (1 - r)
+// goes into dk with sm_scale.
+// DOCS: the mask compares document ids; those of a partial q tile are staged through LDS (stage_doc_ids).
+// (A template parameter: the staging code in the kernel costs the other masks registers.)
+template <int SCORE, bool DOCS>
 __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs a) {
   using namespace dkv_cfg;
+  constexpr bool ALIBI = SCORE == FLEXATTN_SCORE_ALIBI;
+  constexpr bool SOFTCAP = SCORE == FLEXATTN_SCORE_SOFTCAP;
+  const float cap2 = SOFTCAP ? a.score.cap * kLog2e : 0.f;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   bf16_t* sT = reinterpret_cast<bf16_t*>(smem_raw);
   float* sLse = reinterpret_cast<float*>(sT + 8 * kTileElems);
@@ -409,7 +419,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   };
   PinnedState st;
   // K goes in multiplied by sm_scale * log2(e): the streams' scores are then in the log2 domain
-  const float c2 = a.sm_scale * kLog2e;
+  const float c2 = SOFTCAP ? 2.f * kLog2e * a.sm_scale / a.score.cap : a.sm_scale * kLog2e;
   auto scaled = [c2](unsigned two) {
     const float lo = __builtin_bit_cast(float, two << 16) * c2;
     const float hi = __builtin_bit_cast(float, two & 0xffff0000u) * c2;
@@ -512,6 +522,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     if (lse_wave) {  // (the streams want -lse: it is the accumulator input of the S chain)
       float neg_lse = (x > 0.f) ? -__builtin_fmaf(y, kLog2e, log2f(x)) : -__builtin_huge_valf();
       if (ALIBI) neg_lse = __builtin_fmaf((float)((int)r0 + row_p - kc), na2, neg_lse);
+      if (SOFTCAP) neg_lse += cap2;
       sLse[buf * BQ + row_p] = neg_lse;
     } else {  // (and -delta, for the dP chain)
       sDl[buf * BQ + row_p] = -x;
@@ -536,7 +547,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     tbl[1] = (unsigned)(group - 1);
     tbl[2] = (unsigned)a.Sq;
     tbl[3] = base0 + (unsigned)w * 4096u;  // LDS address of the wave's first 1 KB block in buffer 0
-    tbl[4] = __builtin_bit_cast(unsigned, na2);
+    tbl[4] = __builtin_bit_cast(unsigned, SOFTCAP ? cap2 : na2);
     tbl[5] = lse_wave ? 1u : 0u;
     tbl[6] = (unsigned)(size_t)tile_idx;
     tbl[7] = (unsigned)((size_t)tile_idx >> 32);
@@ -570,9 +581,17 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     if (partial) {
       // the lane's keep bits: element e of q block c sits at bit 16 (c & 1) + e of km[c >> 1]
       const int q0 = qb * BQ;
+      if constexpr (DOCS) {
+        int* sDoc = reinterpret_cast<int*>(sPart + MAX_LIST) + w * 128;  // the wave's stage for document ids
+        stage_doc_ids(a.mask.doc_q, q0, q0 + 64, lane, sDoc);
 #pragma unroll
-      for (int half = 0; half < 2; ++half)
-        km[half] = keep_bits32<false>(a.mask, k_idx, q0 + 64 * half + 4 * hh, doc_j, a.mask.doc_q);
+        for (int half = 0; half < 2; ++half)
+          km[half] = keep_bits32<false>(a.mask, k_idx, q0 + 64 * half + 4 * hh, doc_j, sDoc + 64 * half - (q0 + 64 * half));
+      } else {
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+          km[half] = keep_bits32<false>(a.mask, k_idx, q0 + 64 * half + 4 * hh, doc_j, a.mask.doc_q);
+      }
     } else {
       // the run of full tiles ends before the next partial one: lanes look 64 steps ahead at a time
       bool found = false;
@@ -637,9 +656,12 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
                  [g1v] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]), [g3] "v"(loader.goff[3]), [m0] "v"(km[0]), \
                  [m1] "v"(km[1]), [tid4] "v"(tid4), ##__VA_ARGS__                                                \
                : "memory", "scc", "vcc", "m0", FA_DKV_RUN_SGPRS, "v67", FA_DKV_TILE_CLOBBERS CLOB_MORE)
-    if constexpr (ALIBI) {
 #define FA_DKV_ALIBI_CLOBBERS , "s101"
+    if constexpr (ALIBI) {
       FA_DKV_CALL(FA_DKV_RUN_ALIBI, FA_DKV_ALIBI_CLOBBERS, [kc] "v"(kc));
+    } else if constexpr (SOFTCAP) {
+      const float k2 = -2.f * cap2;
+      FA_DKV_CALL(FA_DKV_RUN_SOFTCAP, FA_DKV_ALIBI_CLOBBERS, [k2] "v"(k2));
     } else {
       FA_DKV_CALL(FA_DKV_RUN, );
     }
@@ -681,7 +703,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     // the streams leave the constant sm_scale out of dS: dk takes it here; and both take the key's
     // share of a position bias
     const float ej = ALIBI ? exp2f(-na2 * (float)((lane_here & 31) + 32 * w - BNK / 2)) : 1.f;
-    const float ek = a.sm_scale * ej;
+    const float ek = (SOFTCAP ? 4.f : 1.f) * a.sm_scale * ej;
     FA_GET(0, st.dv[0], "a[0:15]", 1, 0, ej) FA_GET(1, st.dv[1], "a[16:31]", 1, 1, ej)
     FA_GET(2, st.dv[2], "a[32:47]", 1, 2, ej) FA_GET(3, st.dv[3], "a[48:63]", 1, 3, ej)
     FA_GET(4, st.dk[0], "a[64:79]", 0, 0, ek) FA_GET(5, st.dk[1], "a[80:95]", 0, 1, ek)
@@ -718,28 +740,39 @@ static int launch_dkv(const BwdArgs& a, hipStream_t stream) {
   return check_launch("flexattn_bwd_dkv bf16");
 }
 
-template <bool ALIBI>
-static int launch_dkv_plain(const BwdArgs& a, hipStream_t stream) {
+template <int SCORE, bool DOCS>
+static int launch_dkv_plain_on(const BwdArgs& a, hipStream_t stream) {
   using namespace dkv_cfg;
-  auto kern = bwd_dkv_bf16_d128_plain_kernel<ALIBI>;
+  auto kern = bwd_dkv_bf16_d128_plain_kernel<SCORE, DOCS>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(dkv): %s", hipGetErrorString(attr));
   const int n_wg = a.B * a.Hkv * (a.Sk / BNK);
-  const int grid = persistent_ok(n_wg, a.Sk / BNK) ? 256 : n_wg;
+  // (the static schedule balances masks whose work per tile is linear in the tile index; under
+  // document masks it does not: one item per work-group then, handed out by the hardware as CUs free up)
+  const bool irregular = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
+  const int grid = (persistent_ok(n_wg, a.Sk / BNK) && !irregular) ? 256 : n_wg;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), LDS_BYTES, stream, a);
   return check_launch("flexattn_bwd_dkv bf16");
+}
+
+template <int SCORE>
+static int launch_dkv_plain(const BwdArgs& a, hipStream_t stream) {
+  return (a.mask.flags & FLEXATTN_MASK_DOC) ? launch_dkv_plain_on<SCORE, true>(a, stream)
+                                            : launch_dkv_plain_on<SCORE, false>(a, stream);
 }
 
 int bwd_dkv_bf16_d128(const BwdArgs& a, hipStream_t stream) {
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
       // (the generated-stream kernel caches the q tile list in LDS)
-      return a.map.nq <= dkv_cfg::MAX_LIST ? launch_dkv_plain<false>(a, stream) : launch_dkv<FLEXATTN_SCORE_NONE>(a, stream);
+      return a.map.nq <= dkv_cfg::MAX_LIST ? launch_dkv_plain<FLEXATTN_SCORE_NONE>(a, stream) : launch_dkv<FLEXATTN_SCORE_NONE>(a, stream);
     case FLEXATTN_SCORE_ALIBI:
-      return (a.map.nq <= dkv_cfg::MAX_LIST && a.Hq == a.Hkv) ? launch_dkv_plain<true>(a, stream)
+      return (a.map.nq <= dkv_cfg::MAX_LIST && a.Hq == a.Hkv) ? launch_dkv_plain<FLEXATTN_SCORE_ALIBI>(a, stream)
                                                               : launch_dkv<FLEXATTN_SCORE_ALIBI>(a, stream);
-    case FLEXATTN_SCORE_SOFTCAP: return launch_dkv<FLEXATTN_SCORE_SOFTCAP>(a, stream);
+    case FLEXATTN_SCORE_SOFTCAP:
+      return (a.map.nq <= dkv_cfg::MAX_LIST && a.score.cap > 0.f) ? launch_dkv_plain<FLEXATTN_SCORE_SOFTCAP>(a, stream)
+                                                                   : launch_dkv<FLEXATTN_SCORE_SOFTCAP>(a, stream);
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_dkv<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);
   }
   return set_error(FLEXATTN_EINVAL, "unknown score kind %d", a.score.kind);

@@ -42,7 +42,7 @@ constexpr int D = 128;
 constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2
 // plain-score kernel: steps of two kv tiles, (K, K, V, V) x 2 buffers, per-wave tables, cached kv list + states
 constexpr int MAX_LIST = 2048;
-constexpr int PLAIN_LDS_BYTES = 8 * kTileElems * 2 + 4 * 16 * 4 + MAX_LIST * 5;
+constexpr int PLAIN_LDS_BYTES = 8 * kTileElems * 2 + 4 * 16 * 4 + MAX_LIST * 5 + kDocStageBytes;
 }  // namespace dq_cfg
 
 
@@ -513,13 +513,20 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
       unsigned km[2] = {0u, 0u};
       if (it_part < n_steps) {
         // the lane's keep bits: element e of kv block c sits at bit 16 (c & 1) + e of km[c >> 1]
+        int* sDoc = reinterpret_cast<int*>(sSt + MAX_LIST) + w * 128;  // the wave's stage for document ids
+        if (a.mask.flags & FLEXATTN_MASK_DOC) {
+          const int e1 = 2 * it_part + 1 < n_tiles ? 2 * it_part + 1 : 2 * it_part;
+          stage_doc_ids(a.mask.doc_k, __builtin_amdgcn_readfirstlane(sIdx[2 * it_part]) * BN,
+                        __builtin_amdgcn_readfirstlane(sIdx[e1]) * BN, lane, sDoc);
+        }
 #pragma unroll
         for (int hx = 0; hx < 2; ++hx) {
           const int e = 2 * it_part + hx;
           if (e >= n_tiles) continue;  // missing half: all dropped
           const int kt = __builtin_amdgcn_readfirstlane(sIdx[e]);
           const int state = __builtin_amdgcn_readfirstlane((int)sSt[kt]);
-          km[hx] = state == 2 ? 0xffffffffu : keep_bits32<true>(a.mask, q_idx, kt * BN + 4 * hh, doc_i, a.mask.doc_k);
+          km[hx] = state == 2 ? 0xffffffffu
+                              : keep_bits32<true>(a.mask, q_idx, kt * BN + 4 * hh, doc_i, sDoc + 64 * hx - kt * BN);
         }
       } else {
         it_part = -1;

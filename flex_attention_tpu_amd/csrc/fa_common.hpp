@@ -185,6 +185,20 @@ __device__ __forceinline__ unsigned compress_even_nibbles(unsigned long long m) 
   m = (m | (m >> 16)) & 0x00000000FFFFFFFFull;
   return (unsigned)m;
 }
+// Document ids of two 64-index strips, from `first_a` and `first_b` on (multiples of 4), into a
+// wave-private LDS stage of 128 ints: lanes 0-31 load and store 16 bytes each.  keep_bits32 then reads
+// a strip's ids from LDS (pass `stage [+ 64] - first` as its doc_var) instead of one dependent global
+// load per group of four elements.
+constexpr int kDocStageBytes = 4 * 128 * 4;  // four waves
+__device__ __forceinline__ void stage_doc_ids(const int* doc, int first_a, int first_b, int lane, int* stage) {
+  if (lane < 32) {
+    const int first = lane < 16 ? first_a : first_b;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(doc + first + 4 * (lane & 15));
+    *reinterpret_cast<u32x4*>(stage + 4 * lane) = v;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
 template <bool KEYS>
 __device__ __forceinline__ unsigned keep_bits32(const MaskArgs& mk, int fixed, int base, int doc_fixed,
                                                 const int* doc_var) {

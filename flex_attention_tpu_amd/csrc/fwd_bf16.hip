@@ -44,7 +44,7 @@ constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2
 // plain-score kernel: 256 q rows per work item, steps of two kv tiles: (K, K, V, V) x 2 buffers, per-wave
 // tables, wave counters, merged kv list, the two state rows
 constexpr int MAX_LIST = 1024;
-constexpr int PLAIN_LDS_BYTES = 8 * kTileElems * 2 + 4 * 16 * 4 + 16 + MAX_LIST * 4 + 2 * MAX_LIST;
+constexpr int PLAIN_LDS_BYTES = 8 * kTileElems * 2 + 4 * 16 * 4 + 16 + MAX_LIST * 4 + 2 * MAX_LIST + kDocStageBytes;
 }  // namespace fwd_cfg
 
 
@@ -354,7 +354,9 @@ static int launch_fwd(const FwdArgs& a, hipStream_t stream) {
 // ------------------------------------------------------------------------------------------------
 // ALIBI: the score gets slopes[h] (j - i) added; the streams then build the accumulator input of every
 // S chain, slope' (j - i) - M, with one fp32 MFMA per chain (see gen_fwd_tile.py).
-template <bool ALIBI>
+// DOCS: the mask compares document ids; those of a partial step's kv tiles are staged through LDS
+// (stage_doc_ids).  (A template parameter: the staging code costs the other masks registers.)
+template <bool ALIBI, bool DOCS>
 __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) {
   using namespace fwd_cfg;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
@@ -605,6 +607,10 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
       int it_end = it + 1;
       unsigned km[4] = {0u, 0u, 0u, 0u};  // keep bits of q block x, kv tile hx of the step: km[2 x + hx]
       if (partial) {
+        int* sDoc = reinterpret_cast<int*>(sStB + MAX_LIST) + w * 128;  // the wave's stage for document ids
+        if constexpr (DOCS)
+          stage_doc_ids(a.mask.doc_k, __builtin_amdgcn_readfirstlane(entry(2 * it)) * BN,
+                        __builtin_amdgcn_readfirstlane(entry(2 * it + 1)) * BN, lane, sDoc);
 #pragma unroll
         for (int hx = 0; hx < 2; ++hx) {
           const int e = 2 * it + hx;
@@ -616,7 +622,8 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
             if (state == 2) {
               km[2 * x + hx] = 0xffffffffu;
             } else if (state == 1) {
-              km[2 * x + hx] = keep_bits32<true>(a.mask, q_idx[x], k * BN + 4 * hh, doc_i[x], a.mask.doc_k);
+              km[2 * x + hx] = keep_bits32<true>(a.mask, q_idx[x], k * BN + 4 * hh, doc_i[x],
+                                                 DOCS ? sDoc + 64 * hx - k * BN : a.mask.doc_k);
             }
           }
         }
@@ -786,18 +793,26 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
   }  // work items
 }
 
-template <bool ALIBI>
-static int launch_fwd_plain(const FwdArgs& a, hipStream_t stream) {
+template <bool ALIBI, bool DOCS>
+static int launch_fwd_plain_on(const FwdArgs& a, hipStream_t stream) {
   using namespace fwd_cfg;
-  auto kern = fwd_bf16_d128_plain_kernel<ALIBI>;
+  auto kern = fwd_bf16_d128_plain_kernel<ALIBI, DOCS>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, PLAIN_LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(fwd): %s", hipGetErrorString(attr));
   const int nQ2 = (a.Sq / BM + 1) / 2;
   const int n_wg = a.B * a.Hq * nQ2;
-  const int grid = persistent_ok(n_wg, nQ2) ? 256 : n_wg;
+  // (under document masks the static schedule does not balance: one item per work-group then)
+  const bool irregular = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
+  const int grid = (persistent_ok(n_wg, nQ2) && !irregular) ? 256 : n_wg;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), PLAIN_LDS_BYTES, stream, a);
   return check_launch("flexattn_fwd bf16");
+}
+
+template <bool ALIBI>
+static int launch_fwd_plain(const FwdArgs& a, hipStream_t stream) {
+  return (a.mask.flags & FLEXATTN_MASK_DOC) ? launch_fwd_plain_on<ALIBI, true>(a, stream)
+                                            : launch_fwd_plain_on<ALIBI, false>(a, stream);
 }
 
 // FLEXATTN_FWD_STREAM=0 sends plain-score calls to the compiled kernel too (for comparisons).

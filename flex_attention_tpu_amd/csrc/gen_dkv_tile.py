@@ -75,6 +75,12 @@ S_T = ["s84", "s85", "s86", "s87"]
 S_GQ0, S_GQ1, S_GD0, S_GD1, S_RA, S_RB = "s[88:89]", "s[90:91]", "s[92:93]", "s[94:95]", "s[96:97]", "s[98:99]"
 S_LDSN = "s100"
 S_KC = "s101"     # (position-bias variant) 128 kb + 64: the middle of the item's kv tile
+# Softcap variant, s' = cap tanh(s / cap): K arrives multiplied by 2 log2(e) sm_scale / cap, so a chain started
+# from zero yields u with e^(2 s / cap) = 2^u; r = 1 / (2^u + 1) gives tanh = 1 - 2 r and the exponent
+# cap' - lse - 2 cap' r with cap' = cap log2(e) (LDS holds cap' - lse; s64 = cap', s101 = -2 cap'), and
+# ds'/ds = 1 - tanh^2 = 4 r (1 - r), whose factor 4 the epilogue applies to dk.
+S_CAP, S_K2 = "s64", "s101"
+CAP_SOFTCAP = 7   # instructions per MFMA gap in the softcap variant (8 VALU ops per element instead of 2)
 V_QB2 = 67      # q block index of the step after the next one, across the stream
 ROW_SLOT = 28   # MFMA slot at which the next step's lse / delta values are turned around
 V_ROW = 144     # 4 temporaries for that, inside pb[1] (first written by E(1), after ROW_SLOT)
@@ -89,7 +95,7 @@ V_TMP = 68    # 4 temporaries of the masked variant
 DL_OFFSET = 1024
 
 
-def build(masked, alibi=False):
+def build(masked, alibi=False, softcap=False):
     em = Emitter()
     em.wait_old = WAIT_OLD
 
@@ -140,9 +146,12 @@ def build(masked, alibi=False):
             s, dp = V_S[c & 1], V_DP[c & 1]
             cin = V_LSE if ks == 0 else s
             cdn = V_DL if ks == 0 else dp
+            first = ((vr(s, 16), ar(base, 4), ar(128 + 4 * ks, 4), "0", vset(s, 16), aset(base, 4), aset(128 + 4 * ks, 4), set())
+                     if softcap and ks == 0 else
+                     (vr(s, 16), ar(base, 4), ar(128 + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(base, 4), aset(128 + 4 * ks, 4),
+                      vset(cin, 16)))
             return [
-                (vr(s, 16), ar(base, 4), ar(128 + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(base, 4), aset(128 + 4 * ks, 4),
-                 vset(cin, 16)),
+                first,
                 (vr(dp, 16), ar(base + 4, 4), ar(160 + 4 * ks, 4), vr(cdn, 16), vset(dp, 16), aset(base + 4, 4),
                  aset(160 + 4 * ks, 4), vset(cdn, 16)),
             ]
@@ -168,6 +177,11 @@ def build(masked, alibi=False):
         return Op((lambda e: e.lds_read(text, dst)) if "lds" not in DROP else (lambda e: None), **kw)
 
     chains = []
+    e_chains = []
+
+    def lse_read(c, g):
+        return lds(f"ds_read_b128 {vr(V_LSE + 4 * g, 4)}, %[la] offset:{(32 * c + 8 * g) * 4}", vset(V_LSE + 4 * g, 4))
+
     # ---- E(c): element-wise work between the block's S / dP chains and its B products -------
     for c in range(4):
         s, dp = V_S[c & 1], V_DP[c & 1]
@@ -176,6 +190,26 @@ def build(masked, alibi=False):
             for u in range(4):
                 e = 4 * g + u
                 ops.append(valu(f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
+            if softcap:
+                # 2^u -> r = 1 / (2^u + 1); dP' r (1 - r); exponent (cap' - lse) - 2 cap' r -> P
+                for text, trans in (("v_add_f32_e32 {s}, 1.0, {s}", False), ("v_rcp_f32_e32 {s}, {s}", True)):
+                    for u in range(4):
+                        e = 4 * g + u
+                        ops.append(valu(text.format(s=vr(s + e)), vset(s + e), vset(s + e), trans))
+                for u in range(4):
+                    e = 4 * g + u
+                    ops.append(valu(f"v_mul_f32_e32 {vr(dp + e)}, {vr(dp + e)}, {vr(s + e)}", vset(dp + e), vset(dp + e) | vset(s + e)))
+                for u in range(4):
+                    e = 4 * g + u
+                    ops.append(valu(f"v_fma_f32 {vr(dp + e)}, -{vr(dp + e)}, {vr(s + e)}, {vr(dp + e)}", vset(dp + e), vset(dp + e) | vset(s + e)))
+                for u in range(4):
+                    e = 4 * g + u
+                    ops.append(valu(f"v_fma_f32 {vr(s + e)}, {vr(s + e)}, {S_K2}, {vr(V_LSE + e)}", vset(s + e), vset(s + e) | vset(V_LSE + e)))
+                if c < 3:
+                    ops.append(lse_read(c + 1, g))   # (the next block's row values take the registers just used)
+                for u in range(4):
+                    e = 4 * g + u
+                    ops.append(valu(f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
             if masked:
                 # keep bit of element e of block c: bit 16 (c & 1) + e of %[m0] (c < 2) or %[m1]
                 for u in range(4):
@@ -205,7 +239,12 @@ def build(masked, alibi=False):
         ops[0].earliest = last_A[c] + 4            # the chains' last results need 12 wait states
         if c + 2 < 4:
             ops[-1].deadline = min(ops[-1].deadline, first_A[c + 2])  # A(c + 2) writes the same S / dP registers
-        chains.append(ops)
+        e_chains.append(ops)
+    if softcap:
+        # one chain: block c + 1 must not read its row values before block c has put them there
+        chains.append([op for ops in e_chains for op in ops])
+    else:
+        chains.extend(e_chains)
 
     # ---- LDS reads -----------------------------------------------------------------------------
     # operand fragments of the MFMA pairs, in the order of their use: not before the pair that had
@@ -221,9 +260,15 @@ def build(masked, alibi=False):
     for c in range(4):
         for g in range(4):
             for reg, off in ((V_LSE, 0), (V_DL, DL_OFFSET)):
+                if softcap and reg == V_LSE:
+                    continue   # (used by E(c), not by the chain: read there, block 0 below)
                 rows.append(lds(f"ds_read_b128 {vr(reg + 4 * g, 4)}, %[la] offset:{(32 * c + 8 * g) * 4 + off}", vset(reg + 4 * g, 4),
                                 earliest=first_A[c - 1] + 6 if c else 0, deadline=max(0, first_A[c] - 6)))
     chains.append(rows)
+    if softcap:
+        first_rows = [lse_read(0, g) for g in range(4)]
+        first_rows[-1].deadline = last_A[0]
+        chains.append(first_rows)
 
     # ---- next step's Q / dO tiles: 16 LDS-direct loads per wave spread over the stream ----------
     # (issued back to back they hold the wave for about a thousand cycles: one CU moves 64 B / clk)
@@ -261,6 +306,8 @@ def build(masked, alibi=False):
         e.valu(f"v_sub_f32_e32 {vr(rt_)}, {vr(rb_)}, {vr(rt_)}", vset(rt_), vset(rt_) | vset(rb_))
         e.valu(f"v_cmp_lt_f32_e32 vcc, 0, {vr(ra_)}", set(), vset(ra_))
         e.valu(f"v_cndmask_b32_e32 {vr(rt_)}, {vr(inf_)}, {vr(rt_)}, vcc", vset(rt_), vset(rt_) | vset(inf_))
+        if softcap:
+            e.valu(f"v_add_f32_e32 {vr(rt_)}, {S_CAP}, {vr(rt_)}", vset(rt_), vset(rt_))   # cap' - lse
         if alibi:
             # + slope log2(e) (j0 - i) for query row i = 128 qb1 + row of the next step, relative to the
             # middle j0 of the kv tile (s64 holds -slope log2 e): the key's share 2^(slope log2(e) (j - j0))
@@ -281,12 +328,12 @@ def build(masked, alibi=False):
     # V_ROW lies inside pb[1] (first written by E(1)): the turn-around runs before E(1) may start
     chains.append([Op(row_turnaround, cost=8, earliest=ROW_SLOT, deadline=last_A[1] + 3)])
 
-    schedule(em, mfmas, chains, CAP)
+    schedule(em, mfmas, chains, CAP_SOFTCAP if softcap else CAP)
     em.drain()
     return em
 
 
-def run_loop(full, masked, alibi=False):
+def run_loop(full, masked, alibi=False, softcap=False):
     """One asm statement: a run of consecutive steps [it, it_end) of one work-group, all full or a
     single partial one.  At entry the step's Q / dO tiles and row values are resident in LDS buffer
     s81; each pass computes the next step's addresses, streams the tile (which copies the next
@@ -299,6 +346,8 @@ def run_loop(full, masked, alibi=False):
     entry += [f"v_readfirstlane_b32 {SREG[n]}, %[{n}]" for n in STATE_IO + STATE_IN]
     if alibi:
         entry += [f"v_readfirstlane_b32 {S_KC}, %[kc]"]
+    if softcap:
+        entry += [f"v_readfirstlane_b32 {S_K2}, %[k2]"]
     switch = ([f"ds_read_b64 {vr(V_TBL + 10, 2)}, %[tbl] offset:104"] if alibi else [])
     switch_sgprs = ([f"v_readfirstlane_b32 s64, {vr(V_TBL + 10)}", f"v_readfirstlane_b32 {S_KC}, {vr(V_TBL + 11)}"] if alibi else [])
     top = entry + [
@@ -389,8 +438,9 @@ def main():
         # one statement for both kinds of tile: a second asm statement on another control-flow
         # path makes the compiler shuffle the pinned registers around each of them
         full, masked = build(False), build(True)
-        for name, alibi in (("FA_DKV_RUN", False), ("FA_DKV_RUN_ALIBI", True)):
-            lines = run_loop(build(False, alibi), build(True, alibi), alibi)
+        for name, alibi, softcap in (("FA_DKV_RUN", False, False), ("FA_DKV_RUN_ALIBI", True, False),
+                                     ("FA_DKV_RUN_SOFTCAP", False, True)):
+            lines = run_loop(build(False, alibi, softcap), build(True, alibi, softcap), alibi, softcap)
             f.write(f"#define {name} \\\n")
             f.write(" \\\n".join(f'  "{line}\\n"' for line in lines))
             f.write("\n\n")

@@ -172,6 +172,13 @@ def test_dkv_tile_streams_respect_hazards():
         assert em.stats["mfma"] == 128  # 4 q blocks x (8 S + 8 dP + 8 dv + 8 dk)
         assert n == em.stats["mfma"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
         scratch_ok(em.out, 68, 199, 255)
+        # position-bias and softcap variants (the latter: 8 element-wise operations per score instead of 2)
+        for alibi, softcap in ((True, False), (False, True)):
+            v = g.build(masked, alibi, softcap)
+            nv = check_stream(v.out)
+            assert v.stats["mfma"] == 128
+            assert nv == v.stats["mfma"] + v.stats["valu"] + v.stats["lds"] + v.stats["vmem"]
+            scratch_ok(v.out, 68, 199, 255)
 
 
 def test_hazard_checker_catches_a_bad_stream():
@@ -215,7 +222,7 @@ def test_compiler_keeps_out_of_the_pinned_registers(tmp_path):
                         "-o", str(asm)], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr
     text = asm.read_text().split("\n")
-    start = next(i for i, l in enumerate(text) if l.startswith("_ZN2fa30bwd_dkv_bf16_d128_plain_kernel"))
+    start = next(i for i, l in enumerate(text) if l.startswith("_ZN2fa30bwd_dkv_bf16_d128_plain_kernelILi0ELb0E"))  # (the plain-score instantiation)
     end = next(i for i, l in enumerate(text) if i > start and l.strip() == "s_endpgm")
     in_asm = False
     for line in text[start:end]:

@@ -271,6 +271,40 @@ def test_position_bias_against_the_fp32_kernels(F, shape):
             assert O.rel_l2(a.float().cpu(), b.cpu()) <= 1e-2, (name, shape, mf is None)
 
 
+@pytest.mark.parametrize("shape", [(1, 2, 2, 128, 128), (2, 4, 2, 640, 640), (1, 16, 4, 2048, 2048), (4, 32, 32, 1024, 1024),
+                                   (1, 2, 2, 256, 1280)], ids=lambda s: "x".join(map(str, s)))
+def test_softcap_against_the_fp32_kernels(F, shape):
+    """cap tanh(s / cap) (the generated-stream kernels take it in where they can) against the fp32 kernels:
+    a small and the benchmark's cap, no mask, causal and document masks, GQA, grids below and above one
+    work-group per CU."""
+    from flex_attention_tpu_amd import masks, scores
+    B, Hq, Hkv, Sq, Sk = shape
+    sc = 1 / math.sqrt(128)
+    g = torch.Generator().manual_seed(Sq + 7 * Sk + Hq)
+    q, do = (torch.randn(B, Hq, Sq, 128, generator=g).to(torch.bfloat16).to(DEV) for _ in range(2))
+    k, v = (torch.randn(B, Hkv, Sk, 128, generator=g).to(torch.bfloat16).to(DEV) for _ in range(2))
+    q = q * 3  # (scores of several caps: the tanh saturates)
+    pairs = [(None, None)]
+    if Sq == Sk:
+        lens, left = [], Sq
+        while left > 0:
+            lens.append(min(left, 128 + (len(lens) * 97) % 300))
+            left -= lens[-1]
+        pairs += [masks.make_causal_mask_fns(128, 128), masks.make_jagged_mask_fns(128, 128, lens)]
+    for cap in (2.0, 30.0):
+        sfn = scores.make_softcap_score_fn(cap)
+        for mf, bf in pairs:
+            def all_passes(q_, k_, v_, do_):
+                o, l, m = _fwd(F, q_, k_, v_, sc, mf, bf, sfn)
+                d = F.compute_delta(o, do_)
+                return (o, m + l.log(), _dq(F, q_, k_, v_, l, m, o, do_, d, sc, mf, bf, sfn)) + tuple(
+                    _dkv(F, q_, k_, v_, l, m, do_, d, sc, mf, bf, sfn))
+            got = all_passes(q, k, v, do)
+            ref = all_passes(q.float(), k.float(), v.float(), do.float())
+            for name, a, b in zip(("o", "lse", "dq", "dk", "dv"), got, ref):
+                assert O.rel_l2(a.float().cpu(), b.cpu()) <= 1e-2, (name, shape, cap, mf is None)
+
+
 def test_entry_points_reject_bad_arguments_on_gpu(F):
     q = torch.zeros(1, 2, 192, 128, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ValueError):  # 192 is not a multiple of the 128-row q tile
