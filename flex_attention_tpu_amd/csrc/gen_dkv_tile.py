@@ -80,7 +80,7 @@ S_KC = "s101"     # (position-bias variant) 128 kb + 64: the middle of the item'
 # cap' - lse - 2 cap' r with cap' = cap log2(e) (LDS holds cap' - lse; s64 = cap', s101 = -2 cap'), and
 # ds'/ds = 1 - tanh^2 = 4 r (1 - r), whose factor 4 the epilogue applies to dk.
 S_CAP, S_K2 = "s64", "s101"
-CAP_SOFTCAP = 7   # instructions per MFMA gap in the softcap variant (8 VALU ops per element instead of 2)
+CAP_SOFTCAP = 8   # instructions per MFMA gap in the softcap variant (8 VALU ops per element instead of 2)
 V_QB2 = 67      # q block index of the step after the next one, across the stream
 ROW_SLOT = 28   # MFMA slot at which the next step's lse / delta values are turned around
 V_ROW = 144     # 4 temporaries for that, inside pb[1] (first written by E(1), after ROW_SLOT)
