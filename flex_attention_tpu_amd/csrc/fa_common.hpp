@@ -157,9 +157,10 @@ __device__ __forceinline__ void rows_to_fragments(const RowBlock& r, char* stage
 }
 
 // ------------------------------------------------------------------------------------------
-// Element mask, evaluated only on tiles the block map marks partial.
+// Element mask, evaluated only on tiles the block map marks partial.  (Integer code, also callable on the
+// host: a CPU test compares the closed forms below with the element-wise predicate.)
 // ------------------------------------------------------------------------------------------
-__device__ __forceinline__ bool keep_elem(const MaskArgs& mk, int i, int j, int doc_i, int doc_j) {
+__host__ __device__ __forceinline__ bool keep_elem(const MaskArgs& mk, int i, int j, int doc_i, int doc_j) {
   // Branch-free: every term is computed and selected by the (wave-uniform) flag bits.
   const bool f_causal = (mk.flags & FLEXATTN_MASK_CAUSAL) != 0;
   const bool f_window = (mk.flags & FLEXATTN_MASK_WINDOW) != 0;
@@ -178,7 +179,7 @@ __device__ __forceinline__ bool keep_elem(const MaskArgs& mk, int i, int j, int 
 // and owns bit 16 c + 4 g + u.  Causal and window masks, the common cases, have a closed form: a
 // 64-bit run of ones over the offsets, of which the even nibbles are the lane's elements.  Other
 // masks loop over the elements (rolled: the code stays small, these tiles are rare).
-__device__ __forceinline__ unsigned compress_even_nibbles(unsigned long long m) {
+__host__ __device__ __forceinline__ unsigned compress_even_nibbles(unsigned long long m) {
   m &= 0x0F0F0F0F0F0F0F0Full;
   m = (m | (m >> 4)) & 0x00FF00FF00FF00FFull;
   m = (m | (m >> 8)) & 0x0000FFFF0000FFFFull;
@@ -200,7 +201,7 @@ __device__ __forceinline__ void stage_doc_ids(const int* doc, int first_a, int f
   __builtin_amdgcn_wave_barrier();
 }
 template <bool KEYS>
-__device__ __forceinline__ unsigned keep_bits32(const MaskArgs& mk, int fixed, int base, int doc_fixed,
+__host__ __device__ __forceinline__ unsigned keep_bits32(const MaskArgs& mk, int fixed, int base, int doc_fixed,
                                                 const int* doc_var) {
   if (mk.flags != 0 && (mk.flags & ~(FLEXATTN_MASK_CAUSAL | FLEXATTN_MASK_WINDOW)) == 0) {
     // kept offsets form one interval [lo, hi]: with d = fixed - base, keys keep d - window < off <= d,
