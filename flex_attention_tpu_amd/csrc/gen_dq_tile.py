@@ -46,9 +46,10 @@ from gfx950_stream import Emitter, Op, ar, aset, schedule, vr, vset  # noqa: E40
 NSLOT = 8        # staging slots of 8 registers
 MIN_AHEAD = 3    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
 WAIT_OLD = 20    # a wait for LDS data also covers younger reads issued at least this many instructions ago
-CAP = 4          # instructions the scheduler puts between two MFMAs unless deadlines force more
+CAP = 6          # instructions the scheduler puts between two MFMAs unless deadlines force more
 LOAD_FIRST = 2   # MFMA gap from which the first LDS-direct load of the next step may go out
 LOAD_EVERY = 2   # gaps between two of them
+TRANS_COST = 2   # share of an MFMA gap a transcendental takes (it holds the wave's issue for two slots)
 DROP = ()        # instruction classes left out (--drop, timing studies only)
 
 TILE = 16384
@@ -171,7 +172,8 @@ def build(masked, alibi=False):
         mfmas = [(lambda e: None)] * len(mfmas)
 
     def valu(text, dst, src, trans=False, **kw):
-        return Op((lambda e: e.valu(text, dst, src, trans)) if "valu" not in DROP else (lambda e: None), **kw)
+        return Op((lambda e: e.valu(text, dst, src, trans)) if "valu" not in DROP else (lambda e: None),
+                  cost=TRANS_COST if trans else 1, **kw)
 
     chains = []
     # ---- E(c): element-wise work between the block's S / dP chains and its B product ----------

@@ -58,10 +58,11 @@ from gfx950_stream import Emitter, Op, ar, aset, schedule, vr, vset  # noqa: E40
 
 MIN_AHEAD = 2    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
 WAIT_OLD = 20    # a wait for LDS data also covers younger reads issued at least this many instructions ago
-CAP = 5          # instructions the scheduler puts between two MFMAs unless deadlines force more
+CAP = 6          # instructions the scheduler puts between two MFMAs unless deadlines force more
 LOAD_FIRST = 2   # MFMA gap from which the first LDS-direct load of the next step may go out
 LOAD_EVERY = 2   # gaps between two of them
 TAU = "0x40c00000"  # 6.0: M moves when the running maximum relative to it leaves [-6, 6]
+TRANS_COST = 2   # share of an MFMA gap a transcendental takes (it holds the wave's issue for two slots)
 DROP = ()        # instruction classes left out (--drop, timing studies only)
 
 TILE = 16384
@@ -193,7 +194,8 @@ def build(masked, alibi=False):
     holds = {}  # V^T place -> kv block whose fragment was last read into it
 
     def valu(text, dst, src, trans=False, **kw):
-        return Op((lambda e: e.valu(text, dst, src, trans)) if "valu" not in DROP else (lambda e: None), **kw)
+        return Op((lambda e: e.valu(text, dst, src, trans)) if "valu" not in DROP else (lambda e: None),
+                  cost=TRANS_COST if trans else 1, **kw)
 
     reads = []
     for k, (kind, c, x) in enumerate(pairs):
