@@ -586,7 +586,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
         stage_doc_ids(a.mask.doc_q, q0, q0 + 64, lane, sDoc);
 #pragma unroll
         for (int half = 0; half < 2; ++half)
-          km[half] = keep_bits32<false>(a.mask, k_idx, q0 + 64 * half + 4 * hh, doc_j, sDoc + 64 * half - (q0 + 64 * half));
+          km[half] = keep_bits32_staged<false>(a.mask, k_idx, q0 + 64 * half + 4 * hh, doc_j, sDoc + 64 * half + 4 * hh);
       } else {
 #pragma unroll
         for (int half = 0; half < 2; ++half)

@@ -525,8 +525,13 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
           if (e >= n_tiles) continue;  // missing half: all dropped
           const int kt = __builtin_amdgcn_readfirstlane(sIdx[e]);
           const int state = __builtin_amdgcn_readfirstlane((int)sSt[kt]);
-          km[hx] = state == 2 ? 0xffffffffu
-                              : keep_bits32<true>(a.mask, q_idx, kt * BN + 4 * hh, doc_i, sDoc + 64 * hx - kt * BN);
+          if (state == 2) {
+            km[hx] = 0xffffffffu;
+          } else if (a.mask.flags & FLEXATTN_MASK_DOC) {
+            km[hx] = keep_bits32_staged<true>(a.mask, q_idx, kt * BN + 4 * hh, doc_i, sDoc + 64 * hx + 4 * hh);
+          } else {
+            km[hx] = keep_bits32<true>(a.mask, q_idx, kt * BN + 4 * hh, doc_i, nullptr);
+          }
         }
       } else {
         it_part = -1;

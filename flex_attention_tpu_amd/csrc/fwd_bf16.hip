@@ -622,8 +622,10 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
             if (state == 2) {
               km[2 * x + hx] = 0xffffffffu;
             } else if (state == 1) {
-              km[2 * x + hx] = keep_bits32<true>(a.mask, q_idx[x], k * BN + 4 * hh, doc_i[x],
-                                                 DOCS ? sDoc + 64 * hx - k * BN : a.mask.doc_k);
+              if constexpr (DOCS)
+                km[2 * x + hx] = keep_bits32_staged<true>(a.mask, q_idx[x], k * BN + 4 * hh, doc_i[x], sDoc + 64 * hx + 4 * hh);
+              else
+                km[2 * x + hx] = keep_bits32<true>(a.mask, q_idx[x], k * BN + 4 * hh, doc_i[x], a.mask.doc_k);
             }
           }
         }
