@@ -50,7 +50,7 @@ constexpr int BQ = 128;   // q rows per step (two 64-row LDS tiles)
 constexpr int D = 128;
 constexpr int MAX_LIST = 1024;  // longest q tile list the plain-score kernel caches in LDS
 // (Q, dO) x 2 buffers x 2 tiles, lse x2, delta x2, run-loop tables, cached q tile list and its partial flags
-constexpr int LDS_BYTES = 8 * kTileElems * 2 + 4 * BQ * 4 + 4 * 32 * 4 + MAX_LIST * 5 + kDocStageBytes;
+constexpr int LDS_BYTES = 8 * kTileElems * 2 + 4 * BQ * 4 + 4 * 32 * 4 + MAX_LIST * 5 + kDocStageBytes + kMaxSortedItems * 4;
 }  // namespace dkv_cfg
 
 
@@ -364,9 +364,21 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     int bhk, kb;
   };
   const PersistentPlan plan = persistent_plan((int)blockIdx.x, n_wg, nKb);
+  // under document masks a persistent work-group takes its items from the longest-first schedule (sorted_items)
+  const bool sorted = DOCS && gridDim.x != (unsigned)n_wg;
+  int* sItems = reinterpret_cast<int*>(sPart + MAX_LIST) + 4 * 128;
+  if (DOCS && sorted)
+    sorted_items([&](int t) { return a.map.cnt[t]; }, nKb, n_wg / nKb, (int)blockIdx.x, n_items, tid,
+                 reinterpret_cast<int*>(smem_raw), sItems);
   auto geometry = [&](int item) {
     Geometry g;
-    persistent_item(plan, (int)blockIdx.x, item, (int)gridDim.x, n_wg, nKb, g.bhk, g.kb);
+    if (DOCS && sorted) {
+      const int v = sItems[item];
+      g.bhk = v >> 16;
+      g.kb = v & 0xffff;
+    } else {
+      persistent_item(plan, (int)blockIdx.x, item, (int)gridDim.x, n_wg, nKb, g.bhk, g.kb);
+    }
     g.bhk = __builtin_amdgcn_readfirstlane(g.bhk);
     g.kb = __builtin_amdgcn_readfirstlane(g.kb);
     return g;
@@ -748,10 +760,10 @@ static int launch_dkv_plain_on(const BwdArgs& a, hipStream_t stream) {
                                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(dkv): %s", hipGetErrorString(attr));
   const int n_wg = a.B * a.Hkv * (a.Sk / BNK);
-  // (the static schedule balances masks whose work per tile is linear in the tile index; under
-  // document masks it does not: one item per work-group then, handed out by the hardware as CUs free up)
-  const bool irregular = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
-  const int grid = (persistent_ok(n_wg, a.Sk / BNK) && !irregular) ? 256 : n_wg;
+  // (persistent_ok's schedule balances masks whose work per tile is linear in the tile index; document
+  // masks take the longest-first schedule of sorted_items; what fits neither runs one item per work-group)
+  const bool persistent = DOCS ? sorted_schedule_ok(n_wg, a.Sk / BNK) : persistent_ok(n_wg, a.Sk / BNK);
+  const int grid = (persistent && n_wg > 256) ? 256 : n_wg;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), LDS_BYTES, stream, a);
   return check_launch("flexattn_bwd_dkv bf16");
 }

@@ -42,7 +42,7 @@ constexpr int D = 128;
 constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2
 // plain-score kernel: steps of two kv tiles, (K, K, V, V) x 2 buffers, per-wave tables, cached kv list + states
 constexpr int MAX_LIST = 2048;
-constexpr int PLAIN_LDS_BYTES = 8 * kTileElems * 2 + 4 * 16 * 4 + MAX_LIST * 5 + kDocStageBytes;
+constexpr int PLAIN_LDS_BYTES = 8 * kTileElems * 2 + 4 * 16 * 4 + MAX_LIST * 5 + kDocStageBytes + kMaxSortedItems * 4;
 }  // namespace dq_cfg
 
 
@@ -281,7 +281,9 @@ static int launch_dq(const BwdArgs& a, hipStream_t stream) {
 // ------------------------------------------------------------------------------------------------
 // ALIBI: the score gets slopes[h] (j - i) added; the streams then build the accumulator input of every
 // S chain, slope' (j - i) - lse, with one fp32 MFMA per 32-key block (see gen_dq_tile.py).
-template <bool ALIBI>
+// DOCS: the mask compares document ids; a persistent work-group then takes its items from the longest-first
+// schedule (sorted_items).  (A template parameter: the code costs the other masks registers.)
+template <bool ALIBI, bool DOCS>
 __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs a) {
   using namespace dq_cfg;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
@@ -324,7 +326,18 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   const PersistentPlan plan = persistent_plan((int)blockIdx.x, n_wg, nQ);
   const int group = a.Hq / a.Hkv;
   const float inv_group = 1.0f / (float)group;
+  const bool sorted = DOCS && gridDim.x != (unsigned)n_wg;
+  int* sItems = reinterpret_cast<int*>(sSt + MAX_LIST) + 4 * 128;
+  if (DOCS && sorted)
+    sorted_items([&](int t) { return a.map.cnt[t]; }, nQ, n_wg / nQ, (int)blockIdx.x, n_items, tid,
+                 reinterpret_cast<int*>(smem_raw), sItems);
   auto geometry = [&](int item, int& bh, int& qb) {
+    if (DOCS && sorted) {
+      const int v = sItems[item];
+      bh = v >> 16;
+      qb = v & 0xffff;
+      return;
+    }
     persistent_item(plan, (int)blockIdx.x, item, (int)gridDim.x, n_wg, nQ, bh, qb);
     if (gridDim.x == (unsigned)n_wg) qb = nQ - 1 - qb;  // one item each: longest first
   };
@@ -641,17 +654,24 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   }  // work items
 }
 
-template <bool ALIBI>
-static int launch_dq_plain(const BwdArgs& a, hipStream_t stream) {
+template <bool ALIBI, bool DOCS>
+static int launch_dq_plain_on(const BwdArgs& a, hipStream_t stream) {
   using namespace dq_cfg;
-  auto kern = bwd_dq_bf16_d128_plain_kernel<ALIBI>;
+  auto kern = bwd_dq_bf16_d128_plain_kernel<ALIBI, DOCS>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, PLAIN_LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(dq): %s", hipGetErrorString(attr));
   const int n_wg = a.B * a.Hq * (a.Sq / BM);
-  const int grid = persistent_ok(n_wg, a.Sq / BM) ? 256 : n_wg;
+  const bool persistent = DOCS ? sorted_schedule_ok(n_wg, a.Sq / BM) : persistent_ok(n_wg, a.Sq / BM);
+  const int grid = (persistent && n_wg > 256) ? 256 : n_wg;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), PLAIN_LDS_BYTES, stream, a);
   return check_launch("flexattn_bwd_dq bf16");
+}
+
+template <bool ALIBI>
+static int launch_dq_plain(const BwdArgs& a, hipStream_t stream) {
+  return (a.mask.flags & FLEXATTN_MASK_DOC) ? launch_dq_plain_on<ALIBI, true>(a, stream)
+                                            : launch_dq_plain_on<ALIBI, false>(a, stream);
 }
 
 int bwd_dq_bf16_d128(const BwdArgs& a, hipStream_t stream) {

@@ -44,7 +44,7 @@ constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2
 // plain-score kernel: 256 q rows per work item, steps of two kv tiles: (K, K, V, V) x 2 buffers, per-wave
 // tables, wave counters, merged kv list, the two state rows
 constexpr int MAX_LIST = 1024;
-constexpr int PLAIN_LDS_BYTES = 8 * kTileElems * 2 + 4 * 16 * 4 + 16 + MAX_LIST * 4 + 2 * MAX_LIST + kDocStageBytes;
+constexpr int PLAIN_LDS_BYTES = 8 * kTileElems * 2 + 4 * 16 * 4 + 16 + MAX_LIST * 4 + 2 * MAX_LIST + kDocStageBytes + kMaxSortedItems * 4;
 }  // namespace fwd_cfg
 
 
@@ -417,7 +417,19 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
   const PersistentPlan plan = persistent_plan((int)blockIdx.x, n_wg, nQ2);
   const int group = a.Hq / a.Hkv;
   const float inv_group = 1.0f / (float)group;
+  // under document masks a persistent work-group takes its items from the longest-first schedule (sorted_items)
+  const bool sorted = DOCS && gridDim.x != (unsigned)n_wg;
+  int* sItems = reinterpret_cast<int*>(sStB + MAX_LIST) + 4 * 128;
+  if (DOCS && sorted)
+    sorted_items([&](int t) { return a.map.cnt[2 * t] + (2 * t + 1 < nQ ? a.map.cnt[2 * t + 1] : 0); }, nQ2, n_wg / nQ2,
+                 (int)blockIdx.x, n_items, tid, reinterpret_cast<int*>(smem_raw), sItems);
   auto geometry = [&](int item, int& bh, int& qb2) {
+    if (DOCS && sorted) {
+      const int v = sItems[item];
+      bh = v >> 16;
+      qb2 = v & 0xffff;
+      return;
+    }
     persistent_item(plan, (int)blockIdx.x, item, (int)gridDim.x, n_wg, nQ2, bh, qb2);
     if (gridDim.x == (unsigned)n_wg) qb2 = nQ2 - 1 - qb2;  // one item each: longest first
   };
@@ -804,9 +816,9 @@ static int launch_fwd_plain_on(const FwdArgs& a, hipStream_t stream) {
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(fwd): %s", hipGetErrorString(attr));
   const int nQ2 = (a.Sq / BM + 1) / 2;
   const int n_wg = a.B * a.Hq * nQ2;
-  // (under document masks the static schedule does not balance: one item per work-group then)
-  const bool irregular = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
-  const int grid = (persistent_ok(n_wg, nQ2) && !irregular) ? 256 : n_wg;
+  // (document masks take the longest-first schedule of sorted_items)
+  const bool persistent = DOCS ? sorted_schedule_ok(n_wg, nQ2) : persistent_ok(n_wg, nQ2);
+  const int grid = (persistent && n_wg > 256) ? 256 : n_wg;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), PLAIN_LDS_BYTES, stream, a);
   return check_launch("flexattn_fwd bf16");
 }

@@ -305,6 +305,29 @@ def test_softcap_against_the_fp32_kernels(F, shape):
                 assert O.rel_l2(a.float().cpu(), b.cpu()) <= 1e-2, (name, shape, cap, mf is None)
 
 
+def test_document_masks_longest_first_schedule(F):
+    """Enough (batch, head, tile) items that the persistent work-groups of all three generated-stream kernels
+    take the longest-first schedule that document masks get (eight items each), with documents of very
+    different lengths: against the fp32 kernels."""
+    from flex_attention_tpu_amd import masks
+    B, H, S = 16, 32, 1024
+    sc = 1 / math.sqrt(128)
+    g = torch.Generator().manual_seed(91)
+    q, do = (torch.randn(B, H, S, 128, generator=g).to(torch.bfloat16).to(DEV) for _ in range(2))
+    k, v = (torch.randn(B, H, S, 128, generator=g).to(torch.bfloat16).to(DEV) for _ in range(2))
+    mf, bf = masks.make_jagged_mask_fns(128, 128, [100, 412, 212, 300])
+
+    def all_passes(q_, k_, v_, do_):
+        o, l, m = _fwd(F, q_, k_, v_, sc, mf, bf, None)
+        d = F.compute_delta(o, do_)
+        return (o, m + l.log(), _dq(F, q_, k_, v_, l, m, o, do_, d, sc, mf, bf, None)) + tuple(
+            _dkv(F, q_, k_, v_, l, m, do_, d, sc, mf, bf, None))
+    got = all_passes(q, k, v, do)
+    ref = all_passes(q.float(), k.float(), v.float(), do.float())
+    for name, a, b in zip(("o", "lse", "dq", "dk", "dv"), got, ref):
+        assert O.rel_l2(a.float().cpu(), b.cpu()) <= 1e-2, name
+
+
 def test_entry_points_reject_bad_arguments_on_gpu(F):
     q = torch.zeros(1, 2, 192, 128, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ValueError):  # 192 is not a multiple of the 128-row q tile
