@@ -23,7 +23,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch on the default workload (cfg2), from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this script, each counter scaled by its reading for the 256 MiB device copy that
 # main() ends with (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Counter-derived, not measured per run.
-HBM_TRAFFIC_BYTES = {"fwd": 650650705, "dq": 688203812, "dkv": 947404680}
+HBM_TRAFFIC_BYTES = {"fwd": 668476257, "dq": 689215371, "dkv": 944777858}
 
 
 def cpu_baseline(cfg, budget_s=12.0):
