@@ -54,6 +54,7 @@ WAIT_OLD = 20    # a wait for LDS data also covers younger reads issued at least
 CAP = 6          # instructions the scheduler puts between two MFMAs unless deadlines force more
 LOAD_FIRST = 2   # MFMA gap from which the first LDS-direct load of the next step may go out
 LOAD_EVERY = 2   # gaps between two of them
+LOAD_COST = 3    # share of an MFMA gap one of them takes
 LDS_COST = 1     # share of an MFMA gap an LDS read takes
 TRANS_COST = 2   # share of an MFMA gap a transcendental takes (it holds the wave's issue for two slots)
 DROP = ()        # instruction classes left out (--drop, timing studies only)
@@ -290,7 +291,7 @@ def build(masked, alibi=False, softcap=False):
     for t, gbase in enumerate((S_GQ0, S_GQ1, S_GD0, S_GD1)):  # half tiles in LDS order
         for i in range(4):
             at = LOAD_FIRST + LOAD_EVERY * k
-            vm.append(Op(direct(t * TILE + i * 1024, "%[g1v]" if i == 1 else f"%[g{i}]", gbase), cost=3, earliest=at, deadline=at + 12))
+            vm.append(Op(direct(t * TILE + i * 1024, "%[g1v]" if i == 1 else f"%[g{i}]", gbase), cost=LOAD_COST, earliest=at, deadline=at + 12))
             k += 1
     chains.append(vm)
 

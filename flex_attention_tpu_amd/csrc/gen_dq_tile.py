@@ -49,6 +49,7 @@ WAIT_OLD = 20    # a wait for LDS data also covers younger reads issued at least
 CAP = 6          # instructions the scheduler puts between two MFMAs unless deadlines force more
 LOAD_FIRST = 2   # MFMA gap from which the first LDS-direct load of the next step may go out
 LOAD_EVERY = 2   # gaps between two of them
+LOAD_COST = 3    # share of an MFMA gap one of them takes
 TRANS_COST = 2   # share of an MFMA gap a transcendental takes (it holds the wave's issue for two slots)
 DROP = ()        # instruction classes left out (--drop, timing studies only)
 
@@ -227,7 +228,7 @@ def build(masked, alibi=False):
             def emit(e, imm=t * TILE + i * 1024, goff="%[g1v]" if i == 1 else f"%[g{i}]", gb=gbase):
                 if "vmem" not in DROP:
                     e.lds_direct_load(imm, goff, gb, S_LDSN)
-            vm.append(Op(emit, cost=3, earliest=at, deadline=at + 12))
+            vm.append(Op(emit, cost=LOAD_COST, earliest=at, deadline=at + 12))
             k += 1
     chains.append(vm)
 
