@@ -1,14 +1,18 @@
 """Benchmark of the flex-attention hot path on one MI355X.
 
 One step = one pass of the hot path over one batch of synthetic input resident in HBM:
-forward (saving l, m), delta pre-pass, dq backward, dk/dv backward, at B=4, H=32, S=4096, D=128,
-bf16, causal (benchmark configurations 2 and 3; pass --config cfg4 / cfg5 for the others).
+forward (saving l, m), delta pre-pass, dq backward, dk/dv backward.  The headline workload is
+benchmark configurations 2 + 3 (B=4, H=32, S=4096, D=128, bf16, causal); the other configurations
+(cfg1 fp32 small, cfg4 ALiBi + causal window, cfg5 GQA + soft-cap + documents) are measured in the
+same run and reported as sub-objects (`--config NAME` makes one of them the headline instead).
 Prints ONE JSON line: whole-step algorithmic TFLOP/s, per-pass TFLOP/s and fraction of the bf16
-MFMA peak, a roofline object for the dominant kernel and the CPU oracle timed on the host cores.
+MFMA peak, launch-time quantiles, a roofline object for the dominant kernel and the CPU oracle
+timed on the host cores.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -18,12 +22,21 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA peak
 PEAK_HBM_GBS = 8000.0
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_cfg2_hbm_traffic.txt")
 
 
-# HBM bytes per launch on the default workload (cfg2), from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of this script, each counter scaled by its reading for the 256 MiB device copy that
-# main() ends with (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Counter-derived, not measured per run.
-HBM_TRAFFIC_BYTES = {"fwd": 668476257, "dq": 689215371, "dkv": 944777858}
+def counter_traffic(kernel):
+    """HBM bytes per launch of `kernel` on cfg2 from the committed rocprofv3 counter summary (FETCH_SIZE
+    and WRITE_SIZE runs of this script, scaled by the 256 MiB device copy main() ends with), or None.
+    Counter-derived in a separate profiler run, not measured in this run."""
+    try:
+        for line in open(TRAFFIC_PROFILE):
+            f = line.split()
+            if len(f) >= 6 and f[0] == kernel and re.fullmatch(r"[0-9.]+", f[5]):
+                return int(float(f[5]) * 1e6)
+    except OSError:
+        pass
+    return None
 
 
 def cpu_baseline(cfg, budget_s=12.0):
@@ -58,76 +71,148 @@ def cpu_baseline(cfg, budget_s=12.0):
     }
 
 
+def quantiles(xs):
+    xs = sorted(xs)
+    pick = lambda f: xs[min(len(xs) - 1, int(round(f * (len(xs) - 1))))]
+    return {"median": pick(0.5), "p10": pick(0.1), "p90": pick(0.9)}
+
+
+def measure(cfg, steps, warmup):
+    """Wall time of `steps` whole steps and per-kernel launch durations of one configuration."""
+    import torch
+    import flex_attention_tpu_amd as F
+    from flex_attention_tpu_amd import configs
+    import warnings
+
+    dev = torch.device("cuda:0")
+    q, k, v, do = configs.make_inputs(cfg, dev)
+    mf, bf = configs.mask_fns(cfg)
+    sfn = configs.score_fn(cfg)
+    sc, blk = cfg.sm_scale, cfg.block
+    warnings.filterwarnings("ignore", message="score_fn with sm_scale")  # (the configurations use 1/sqrt(D) on purpose)
+
+    def fwd():
+        return F._flex_attention_impl(q, k, v, None, None, True, False, sc, 1, blk, blk, blk, False, bf, mf, sfn)
+
+    def dq_of(o, l, m, d):
+        return F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=blk, block_k_major=blk,
+                                       block_k=blk, sm_scale=sc, debug=False, score_fn=sfn, mask_fn=mf, block_mask_fn=bf)
+
+    def dkv_of(l, m, d):
+        return F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=blk, block_q_major=blk,
+                                         block_k_major=blk, block_k=blk, sm_scale=sc, causal=False, debug=False,
+                                         score_fn=sfn, mask_fn=mf, block_mask_fn=bf)
+
+    def step():
+        o, l, m = fwd()
+        d = F.compute_delta(o, do)
+        return o, dq_of(o, l, m, d), dkv_of(l, m, d)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    # Per-kernel launch durations: K back-to-back launches of one kernel between two HIP events on the launch
+    # stream give the mean (events around single launches carry several us of marker overhead); an event
+    # behind every launch of a second batch gives the launch-to-launch intervals for the quantiles.
+    o, l, m = fwd()
+    d = F.compute_delta(o, do)
+    launches = {"fwd": fwd, "delta": lambda: F.compute_delta(o, do), "dq": lambda: dq_of(o, l, m, d),
+                "dkv": lambda: dkv_of(l, m, d)}
+    ms, quant = {}, {}
+    for name, fn in launches.items():
+        fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ms[name] = e0.elapsed_time(e1) / steps
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+        fn()
+        ev[0].record()
+        for i in range(steps):
+            fn()
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        quant[name] = quantiles([ev[i].elapsed_time(ev[i + 1]) for i in range(steps)])
+    return {"ms_step": wall * 1e3 / steps, "ms": ms, "quantiles_ms": quant, "elem_bytes": q.element_size(),
+            "numel_q": q.numel(), "numel_k": k.numel()}
+
+
+def tf(fl, t_ms):
+    return fl / (t_ms * 1e-3) / 1e12
+
+
+def summary(cfg, r):
+    """Per-pass figures of one configuration: ms, TFLOP/s and fraction of the MFMA peak for the bf16
+    configurations; microseconds and GB/s of algorithmic traffic for the small fp32 one."""
+    from flex_attention_tpu_amd import configs
+    ms = r["ms"]
+    f_fwd = configs.flops_fwd(cfg)
+    ms_bwd = ms["delta"] + ms["dq"] + ms["dkv"]
+    eb, nq, nk = r["elem_bytes"], r["numel_q"], r["numel_k"]
+    rows = 4 * cfg.B * cfg.Hq * cfg.S
+    bytes_delta = 2 * nq * eb + rows
+    out = {
+        "workload": f"{cfg.name}: B={cfg.B} Hq={cfg.Hq} Hkv={cfg.Hkv} S={cfg.S} D={cfg.D} "
+                    f"{'bf16' if eb == 2 else 'fp32'}, mask={cfg.mask}, score={cfg.score}",
+        "ms_per_step": r["ms_step"], "step_tflops": tf(3.5 * f_fwd, r["ms_step"]),
+        "fwd": {"ms": ms["fwd"], "tflops": tf(f_fwd, ms["fwd"]), **r["quantiles_ms"]["fwd"]},
+        "bwd": {"ms": ms_bwd, "tflops": tf(2.5 * f_fwd, ms_bwd), "delta_ms": ms["delta"], "dq_ms": ms["dq"],
+                "dkv_ms": ms["dkv"], "delta_gbs": bytes_delta / (ms["delta"] * 1e-3) / 1e9,
+                "dq_quantiles_ms": r["quantiles_ms"]["dq"], "dkv_quantiles_ms": r["quantiles_ms"]["dkv"],
+                "delta_quantiles_ms": r["quantiles_ms"]["delta"]},
+    }
+    if eb == 2:
+        out["fwd"]["frac_of_peak"] = out["fwd"]["tflops"] / PEAK_BF16_TFLOPS
+        out["bwd"]["frac_of_peak"] = out["bwd"]["tflops"] / PEAK_BF16_TFLOPS
+    else:
+        # launch/latency-bound fp32 case: time per pass and algorithmic GB/s (warm caches: 2 MB of operands)
+        b_fwd = (nq + 2 * nk + nq) * eb + 2 * rows                  # q, k, v in; o, l, m out
+        b_dq = (2 * nq + 2 * nk) * eb + 3 * rows + nq * eb           # q, do, k, v, l, m, delta in; dq out
+        b_dkv = (2 * nq + 2 * nk) * eb + 3 * rows + 2 * nk * eb      # ... in; dk, dv out
+        out["fwd"].update(us=ms["fwd"] * 1e3, gbs=b_fwd / (ms["fwd"] * 1e-3) / 1e9)
+        out["bwd"].update(us=ms_bwd * 1e3, gbs=(bytes_delta + b_dq + b_dkv) / (ms_bwd * 1e-3) / 1e9,
+                          dq_gbs=b_dq / (ms["dq"] * 1e-3) / 1e9, dkv_gbs=b_dkv / (ms["dkv"] * 1e-3) / 1e9)
+        out["note"] = "warm-cache latency: operands (2 MB) stay in L2 between launches"
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--config", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--only", action="store_true", help="measure the headline configuration only")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (sharding is design-only, B x Hkv across GPUs)")
 
     import torch
-    import flex_attention_tpu_amd as F
     from flex_attention_tpu_amd import configs
 
     name = "cfg2" if args.config == "cfg3" else args.config
     cfg = configs.CONFIGS[name]
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    q, k, v, do = configs.make_inputs(cfg, dev)
-    mf, bf = configs.mask_fns(cfg)
-    sfn = configs.score_fn(cfg)
-    sc, blk = cfg.sm_scale, cfg.block
-
-    def fwd():
-        return F._flex_attention_impl(q, k, v, None, None, True, False, sc, 1, blk, blk, blk, False, bf, mf, sfn)
-
-    def step():
-        o, l, m = fwd()
-        d = F.compute_delta(o, do)
-        dq = F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=blk, block_k_major=blk,
-                                     block_k=blk, sm_scale=sc, debug=False, score_fn=sfn, mask_fn=mf, block_mask_fn=bf)
-        dk, dv = F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=blk, block_q_major=blk,
-                                           block_k_major=blk, block_k=blk, sm_scale=sc, causal=False, debug=False,
-                                           score_fn=sfn, mask_fn=mf, block_mask_fn=bf)
-        return o, dq, dk, dv
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-
-    # Per-kernel launch durations: K back-to-back launches of one kernel between two HIP events on
-    # the launch stream (single launches bracketed by events carry several us of marker overhead).
-    o, l, m = fwd()
-    d = F.compute_delta(o, do)
-    launches = {
-        "fwd": fwd,
-        "delta": lambda: F.compute_delta(o, do),
-        "dq": lambda: F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=blk,
-                                              block_k_major=blk, block_k=blk, sm_scale=sc, debug=False, score_fn=sfn,
-                                              mask_fn=mf, block_mask_fn=bf),
-        "dkv": lambda: F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=blk,
-                                                 block_q_major=blk, block_k_major=blk, block_k=blk, sm_scale=sc,
-                                                 causal=False, debug=False, score_fn=sfn, mask_fn=mf, block_mask_fn=bf),
-    }
-    ms = {}
-    for name_k, fn in launches.items():
-        fn()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(args.steps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        ms[name_k] = e0.elapsed_time(e1) / args.steps
+    r = measure(cfg, args.steps, args.warmup)
+    head = summary(cfg, r)
+    others = {}
+    if not args.only:
+        for other in ("cfg1", "cfg2", "cfg4", "cfg5"):
+            if other != name:
+                c = configs.CONFIGS[other]
+                others[other] = summary(c, measure(c, args.steps, args.warmup))
+                torch.cuda.empty_cache()
 
     # A plain device copy of known size (256 MiB read + 256 MiB written per launch): the reference
     # dispatch that FETCH_SIZE / WRITE_SIZE counter readings of the attention kernels are scaled by.
@@ -137,38 +222,39 @@ def main():
         dst.copy_(src)
     torch.cuda.synchronize()
 
-    ms_step = wall * 1e3 / args.steps
+    ms = r["ms"]
     f_fwd = configs.flops_fwd(cfg)
-    f_bwd = 2.5 * f_fwd
-    ms_bwd = ms["delta"] + ms["dq"] + ms["dkv"]
-    tf = lambda fl, t_ms: fl / (t_ms * 1e-3) / 1e12
-    bytes_delta = 2 * q.numel() * q.element_size() + 4 * cfg.B * cfg.Hq * cfg.S
-
+    bf16 = r["elem_bytes"] == 2
     # roofline of the dominant kernel; algorithmic FLOPs of one launch:
     #   fwd 2 matmuls = F_fwd, dq 3 matmuls = 1.5 F_fwd, dk/dv 4 matmuls = 2 F_fwd
     algo = {"fwd": f_fwd, "dq": 1.5 * f_fwd, "dkv": 2.0 * f_fwd}
     dom = max(algo, key=lambda n: ms[n])
+    traffic = counter_traffic(dom) if name == "cfg2" else None
     roofline = {
         "kernel": dom, "bound": "mfma", "achieved": tf(algo[dom], ms[dom]), "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s", "frac": tf(algo[dom], ms[dom]) / PEAK_BF16_TFLOPS,
-        "traffic": HBM_TRAFFIC_BYTES.get(dom) if name == "cfg2" else None,
-        "launch_ms": ms[dom],
+        "traffic": traffic,
+        "traffic_source": "profiles/bench_cfg2_hbm_traffic.txt (rocprofv3 --pmc runs of this script, not this run)"
+                          if traffic is not None else None,
+        "launch_ms": ms[dom], "launch_quantiles_ms": r["quantiles_ms"][dom],
     }
+    if not bf16:
+        b = head["bwd"]
+        roofline.update(bound="hbm", achieved=b["dkv_gbs"], peak=PEAK_HBM_GBS, unit="GB/s", frac=b["dkv_gbs"] / PEAK_HBM_GBS)
     out = {
         "metric": "fwd & bwd attention TFLOP/s (S=4096,D=128,bf16 causal); % of MFMA peak",
-        "value": tf(f_fwd + f_bwd, ms_step),
+        "value": head["step_tflops"],
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_step,
+        "ms_per_step": r["ms_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"{cfg.name}+cfg3: fwd + delta + dq + dk/dv, B={cfg.B} Hq={cfg.Hq} Hkv={cfg.Hkv} "
-                               f"S={cfg.S} D={cfg.D} bf16, mask={cfg.mask}, score={cfg.score}, sm_scale=1/sqrt(D)"},
-        "fwd": {"ms": ms["fwd"], "tflops": tf(f_fwd, ms["fwd"]), "frac_of_peak": tf(f_fwd, ms["fwd"]) / PEAK_BF16_TFLOPS},
-        "bwd": {"ms": ms_bwd, "tflops": tf(f_bwd, ms_bwd), "frac_of_peak": tf(f_bwd, ms_bwd) / PEAK_BF16_TFLOPS,
-                "delta_ms": ms["delta"], "dq_ms": ms["dq"], "dkv_ms": ms["dkv"],
-                "delta_gbs": bytes_delta / (ms["delta"] * 1e-3) / 1e9},
+        "dtype": "bf16" if bf16 else "f32", "data": "synthetic",
+        "config": {"workload": f"{cfg.name}{'+cfg3' if name == 'cfg2' else ''}: fwd + delta + dq + dk/dv, B={cfg.B} "
+                               f"Hq={cfg.Hq} Hkv={cfg.Hkv} S={cfg.S} D={cfg.D} {'bf16' if bf16 else 'fp32'}, "
+                               f"mask={cfg.mask}, score={cfg.score}, sm_scale=1/sqrt(D)"},
+        "fwd": head["fwd"], "bwd": head["bwd"],
         "roofline": roofline,
+        "other_configs": others,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg)

@@ -1,17 +1,20 @@
 """Host-side helpers shared by the three entry points: argument checks and C struct assembly."""
 from __future__ import annotations
 
-from typing import Callable, Dict, Optional, Tuple
+import warnings
+import weakref
+from typing import Callable, Optional
 
 import numpy as np
 import torch
 
 from . import _lib
-from .block_mask import BlockMap, build_block_map, mask_spec_c, spec_of
+from .block_mask import LRU, BlockMap, build_block_map, mask_spec_c, spec_of
 from .masks import DocIds, MaskSpec
 from .scores import ScoreSpec
 
-_slopes_cache: Dict[Tuple[Tuple[float, ...], str], torch.Tensor] = {}
+_slopes_cache = LRU(16)   # (slopes, device) -> float32 device array
+_segment_cache = LRU(16)  # id(tensor) -> (weak reference, tensor version, DocIds)
 
 
 def dtype_code(t: torch.Tensor) -> int:
@@ -77,36 +80,68 @@ def check_blocks(Sq, Sk, block_q=None, block_k_major=None, block_k=None, block_q
         raise ValueError(f"block_q={block_q} does not divide block_q_major={block_q_major}")
 
 
+def segment_doc_ids(segment_ids) -> DocIds:
+    """DocIds (host copy + hash) of a ``segment_ids`` argument: a 1-D id array, a [B, S] array whose rows
+    agree, or an object with equal ``.q`` / ``.kv`` arrays (the reference's SegmentIds,
+    jax_exp.py:37-51).  A DocIds passes through, and a tensor seen before (same object, unchanged) is
+    answered from a small cache, so that a training step does not copy the ids to the host and
+    hash them once per pass."""
+    if isinstance(segment_ids, DocIds):
+        return segment_ids
+    ids = segment_ids
+    if hasattr(ids, "q") and hasattr(ids, "kv"):
+        if ids.q is not ids.kv and not torch.equal(torch.as_tensor(ids.q), torch.as_tensor(ids.kv)):
+            raise NotImplementedError("distinct q / kv segment ids are not supported")
+        ids = ids.q
+    if isinstance(ids, DocIds):
+        return ids
+    key = id(ids)
+    if isinstance(ids, torch.Tensor):
+        hit = _segment_cache.get(key)
+        if hit is not None and hit[0]() is ids and hit[1] == ids._version:
+            return hit[2]
+    t = torch.as_tensor(ids).detach().cpu()
+    if t.ndim == 2:
+        if not bool((t == t[:1]).all()):
+            raise NotImplementedError("per-batch segment ids are not supported")
+        t = t[0]
+    if t.ndim != 1:
+        raise ValueError("segment_ids must be a 1-D (or [B, S]) array of ids")
+    arr = t.numpy().astype(np.int64)
+    if np.any(np.diff(arr) < 0):
+        raise NotImplementedError("segment ids must be non-decreasing along the sequence")
+    doc = DocIds(arr)
+    if isinstance(ids, torch.Tensor):
+        _segment_cache.put(key, (weakref.ref(ids), ids._version, doc))
+    return doc
+
+
 def resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk) -> MaskSpec:
     """Single MaskSpec for the closures, the ``causal`` flag and ``segment_ids`` (AND of all)."""
     spec = spec_of(mask_fn, block_mask_fn)
     if causal:
         spec = spec.combine(MaskSpec(flags=_lib.MASK_CAUSAL))
     if segment_ids is not None:
-        ids = segment_ids
-        if hasattr(ids, "q") and hasattr(ids, "kv"):
-            if not torch.equal(torch.as_tensor(ids.q), torch.as_tensor(ids.kv)):
-                raise NotImplementedError("distinct q / kv segment ids are not supported")
-            ids = ids.q
-        ids = torch.as_tensor(ids).detach().cpu()
-        if ids.ndim == 2:
-            if not bool((ids == ids[:1]).all()):
-                raise NotImplementedError("per-batch segment ids are not supported")
-            ids = ids[0]
-        arr = ids.numpy().astype(np.int64)
-        if arr.shape[0] != Sq or Sq != Sk:
+        doc = segment_doc_ids(segment_ids)
+        if len(doc) != Sq or Sq != Sk:
             raise ValueError("segment_ids must have one id per position of a self-attention sequence")
-        if np.any(np.diff(arr) < 0):
-            raise NotImplementedError("segment ids must be non-decreasing along the sequence")
-        spec = spec.combine(MaskSpec(flags=_lib.MASK_DOC, doc_ids=DocIds(arr)))
+        spec = spec.combine(MaskSpec(flags=_lib.MASK_DOC, doc_ids=doc))
     return spec
 
 
-def score_spec_c(score_fn: Optional[Callable], Hq: int, device, mod_q: int, mod_k: int) -> _lib.ScoreSpecC:
+def score_spec_c(score_fn: Optional[Callable], Hq: int, device, mod_q: int, mod_k: int, sm_scale=None) -> _lib.ScoreSpecC:
     """C view of the score closure's spec.  ``mod_q``/``mod_k`` are the tile edges the reference
     would call a tile-local score function with (block_q, block_k)."""
     if score_fn is None:
         return _lib.ScoreSpecC(_lib.SCORE_NONE, 0.0, 0.0, 1, 1, 0, None)
+    if sm_scale is not None and float(sm_scale) != 1.0 and getattr(score_fn, "spec", None) is not None \
+            and score_fn.spec.kind != _lib.SCORE_NONE:
+        # the reference's three kernels and its dense reference disagree about sm_scale next to a score_fn
+        # (flex_attention_kernel.py:249-255 ignores it, flex_attention_dq_bwd.py:340-345 multiplies the
+        # function's result); they coincide with this build's score_mod(sm_scale * <q, k>) only at 1
+        warnings.warn("score_fn with sm_scale != 1: this build computes score_mod(sm_scale * <q, k>); the reference's "
+                      "forward ignores sm_scale here and its backward kernels scale the function's result",
+                      UserWarning, stacklevel=3)
     spec = getattr(score_fn, "spec", None)
     if not isinstance(spec, ScoreSpec):
         raise NotImplementedError(
@@ -120,7 +155,7 @@ def score_spec_c(score_fn: Optional[Callable], Hq: int, device, mod_q: int, mod_
         t = _slopes_cache.get(key)
         if t is None:
             t = torch.tensor(spec.slopes, dtype=torch.float32, device=device)
-            _slopes_cache[key] = t
+            _slopes_cache.put(key, t)
         slopes_ptr = t.data_ptr()
     return _lib.ScoreSpecC(spec.kind, spec.cap, spec.slope, int(mod_q), int(mod_k), 0, slopes_ptr)
 

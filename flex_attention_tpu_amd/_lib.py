@@ -30,6 +30,8 @@ MASK_WINDOW = 2
 MASK_DOC = 4
 MASK_S2 = 8
 
+FLAG_COMPILED_LOOP = 1
+
 PASS_FWD = 0
 PASS_DQ = 1
 PASS_DKV = 2
@@ -81,6 +83,8 @@ class FwdParamsC(C.Structure):
         ("Sq", C.c_int32), ("Sk", C.c_int32), ("D", C.c_int32),
         ("dtype", C.c_int32),
         ("sm_scale", C.c_float),
+        ("flags", C.c_int32),
+        ("reserved", C.c_int32),
         ("score", ScoreSpecC),
         ("mask", MaskSpecC),
         ("map", BlockMapC),
@@ -97,6 +101,8 @@ class BwdParamsC(C.Structure):
         ("Sq", C.c_int32), ("Sk", C.c_int32), ("D", C.c_int32),
         ("dtype", C.c_int32),
         ("sm_scale", C.c_float),
+        ("flags", C.c_int32),
+        ("reserved", C.c_int32),
         ("score", ScoreSpecC),
         ("mask", MaskSpecC),
         ("map", BlockMapC),

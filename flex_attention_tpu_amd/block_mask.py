@@ -3,17 +3,46 @@
 The reference evaluates ``block_mask_fn(q_block, kv_block)`` at every grid step and again inside
 the K/V index maps (flex_attention_kernel.py:97-106, 231-236).  Here the same predicate is
 evaluated once per (mask, shape, tile) by a small HIP kernel into a device-resident map that the
-attention kernels walk; maps are cached because they depend on nothing but the mask specification.
+attention kernels walk; maps are cached (bounded, least recently used) because they depend on
+nothing but the mask specification.
 """
 from __future__ import annotations
 
+import collections
 import ctypes as C
-from typing import Callable, Dict, Optional, Tuple
+from typing import Callable, Optional
 
 import torch
 
 from . import _lib
 from .masks import DocIds, MaskSpec
+
+
+class LRU:
+    """Small least-recently-used cache: holds at most ``maxsize`` entries (each may pin device
+    tensors), so a training loop with a new document layout every batch does not grow it."""
+
+    def __init__(self, maxsize: int):
+        self.maxsize = maxsize
+        self._d = collections.OrderedDict()
+
+    def get(self, key):
+        v = self._d.get(key)
+        if v is not None:
+            self._d.move_to_end(key)
+        return v
+
+    def put(self, key, value):
+        self._d[key] = value
+        self._d.move_to_end(key)
+        while len(self._d) > self.maxsize:
+            self._d.popitem(last=False)
+
+    def clear(self):
+        self._d.clear()
+
+    def __len__(self):
+        return len(self._d)
 
 
 class BlockMap:
@@ -31,6 +60,14 @@ class BlockMap:
         self.kv_idx = torch.empty(self.nq, self.nk, dtype=torch.int32, device=device)
         self.q_cnt = torch.empty(self.nk, dtype=torch.int32, device=device)
         self.q_idx = torch.empty(self.nk, self.nq, dtype=torch.int32, device=device)
+        self.built_on = None   # stream the builder kernel was launched on
+        self.ready = None      # event recorded behind it
+
+    def wait_ready(self, device) -> None:
+        """Makes the current stream wait for the builder kernel if that ran on another stream."""
+        cur = torch.cuda.current_stream(device)
+        if self.ready is not None and cur.cuda_stream != self.built_on:
+            cur.wait_event(self.ready)
 
     def as_c(self) -> _lib.BlockMapC:
         return _lib.BlockMapC(self.state.data_ptr(), self.kv_cnt.data_ptr(), self.kv_idx.data_ptr(),
@@ -42,8 +79,11 @@ class BlockMap:
         return self.state != 0
 
 
-_doc_cache: Dict[Tuple[DocIds, str], torch.Tensor] = {}
-_map_cache: Dict[tuple, BlockMap] = {}
+# Bounded caches (least recently used entries are dropped; a dropped map is simply rebuilt):
+MAP_CACHE_SIZE = 64
+DOC_CACHE_SIZE = 64
+_doc_cache = LRU(DOC_CACHE_SIZE)   # (DocIds, device) -> int32 device array
+_map_cache = LRU(MAP_CACHE_SIZE)   # (spec, Sq, Sk, block_q, block_k, device) -> BlockMap
 
 
 def doc_ids_on(doc: Optional[DocIds], device) -> Optional[torch.Tensor]:
@@ -53,8 +93,8 @@ def doc_ids_on(doc: Optional[DocIds], device) -> Optional[torch.Tensor]:
     key = (doc, str(device))
     t = _doc_cache.get(key)
     if t is None:
-        t = torch.from_numpy(doc.array.copy()).to(device)
-        _doc_cache[key] = t
+        t = torch.from_numpy(doc.array.copy()).to(device)  # (pageable host memory: the copy is synchronous)
+        _doc_cache.put(key, t)
     return t
 
 
@@ -78,6 +118,7 @@ def build_block_map(spec: MaskSpec, Sq: int, Sk: int, block_q: int, block_k: int
     if cache:
         hit = _map_cache.get(key)
         if hit is not None:
+            hit.wait_ready(device)
             return hit
     if Sq % block_q or Sk % block_k:
         raise ValueError(f"Sq={Sq} / Sk={Sk} not divisible by blocks {block_q} / {block_k}")
@@ -89,8 +130,11 @@ def build_block_map(spec: MaskSpec, Sq: int, Sk: int, block_q: int, block_k: int
         _lib.check(lib.flexattn_build_block_mask(
             C.byref(mc), Sq, Sk, block_q, block_k, bm.state.data_ptr(), bm.kv_cnt.data_ptr(),
             bm.kv_idx.data_ptr(), bm.q_cnt.data_ptr(), bm.q_idx.data_ptr(), stream))
+        bm.built_on = stream
+        bm.ready = torch.cuda.Event()
+        bm.ready.record(torch.cuda.current_stream(device))
     if cache:
-        _map_cache[key] = bm
+        _map_cache.put(key, bm)
     return bm
 
 

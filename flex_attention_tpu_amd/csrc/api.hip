@@ -93,6 +93,15 @@ static int tile_shape(int pass, int dtype, int D, int* bq, int* bk) {
   return set_error(FLEXATTN_EINVAL, "unknown dtype %d", dtype);
 }
 
+// sm_scale must be positive (the kernels track maxima of unscaled products and fold the scale into an
+// operand); flags must be known.
+static int check_scale_flags(float sm_scale, int flags) {
+  if (!(sm_scale > 0.f) || !(sm_scale < __builtin_huge_valf()))
+    return set_error(FLEXATTN_EINVAL, "sm_scale must be positive and finite (got %g)", (double)sm_scale);
+  if (flags & ~FLEXATTN_FLAG_COMPILED_LOOP) return set_error(FLEXATTN_EINVAL, "unknown flags 0x%x", flags);
+  return FLEXATTN_OK;
+}
+
 static int check_shape(int pass, int B, int Hq, int Hkv, int Sq, int Sk, int D, int dtype,
                        const flexattn_block_map& map) {
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || Sq <= 0 || Sk <= 0 || D <= 0)
@@ -134,6 +143,7 @@ static int to_bwd_args(const flexattn_bwd_params* p, int pass, BwdArgs* a) {
   if (pass == FLEXATTN_PASS_DKV && (!p->dk || !p->dv)) return set_error(FLEXATTN_EINVAL, "dk or dv is NULL");
   int rc = check_shape(pass, p->B, p->Hq, p->Hkv, p->Sq, p->Sk, p->D, p->dtype, p->map);
   if (rc != FLEXATTN_OK) return rc;
+  if ((rc = check_scale_flags(p->sm_scale, p->flags)) != FLEXATTN_OK) return rc;
   if ((rc = check_score(p->score)) != FLEXATTN_OK) return rc;
   if ((rc = check_mask(p->mask)) != FLEXATTN_OK) return rc;
   a->q = p->q; a->k = p->k; a->v = p->v; a->dout = p->dout;
@@ -141,6 +151,7 @@ static int to_bwd_args(const flexattn_bwd_params* p, int pass, BwdArgs* a) {
   a->dq = p->dq; a->dk = p->dk; a->dv = p->dv;
   a->B = p->B; a->Hq = p->Hq; a->Hkv = p->Hkv; a->Sq = p->Sq; a->Sk = p->Sk;
   a->sm_scale = p->sm_scale;
+  a->flags = p->flags;
   a->score = to_args(p->score);
   a->mask = to_args(p->mask);
   a->map = (pass == FLEXATTN_PASS_DKV) ? col_view(p->map) : row_view(p->map);
@@ -190,12 +201,14 @@ int flexattn_fwd(const flexattn_fwd_params* p, void* stream) {
   if ((p->l == nullptr) != (p->m == nullptr)) return set_error(FLEXATTN_EINVAL, "l and m must both be given or both NULL");
   int rc = check_shape(FLEXATTN_PASS_FWD, p->B, p->Hq, p->Hkv, p->Sq, p->Sk, p->D, p->dtype, p->map);
   if (rc != FLEXATTN_OK) return rc;
+  if ((rc = check_scale_flags(p->sm_scale, p->flags)) != FLEXATTN_OK) return rc;
   if ((rc = check_score(p->score)) != FLEXATTN_OK) return rc;
   if ((rc = check_mask(p->mask)) != FLEXATTN_OK) return rc;
   FwdArgs a;
   a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.l = p->l; a.m = p->m;
   a.B = p->B; a.Hq = p->Hq; a.Hkv = p->Hkv; a.Sq = p->Sq; a.Sk = p->Sk;
   a.sm_scale = p->sm_scale;
+  a.flags = p->flags;
   a.score = to_args(p->score);
   a.mask = to_args(p->mask);
   a.map = row_view(p->map);

@@ -274,6 +274,15 @@ __global__ __launch_bounds__(256) void bwd_dkv_f32_kernel(BwdArgs a) {
         sDl[tid] = a.delta[rr];
       }
       __syncthreads();
+      // The tile's 64 terms are summed on their own and then added to the running totals: the
+      // rounding error of a long sum (thousands of q rows times the group's heads) then grows with
+      // the number of tiles, not of rows.
+      f32x4 dk_t[NV], dv_t[NV];
+#pragma unroll
+      for (int c = 0; c < NV; ++c) {
+        dk_t[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dv_t[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
       for (int ii = 0; ii < BQ; ++ii) {
         const int i = qb * BQ + ii;
         const float s = quad_sum(dot_slice<NV>(kv, sQ + ii * D, sub));
@@ -285,8 +294,13 @@ __global__ __launch_bounds__(256) void bwd_dkv_f32_kernel(BwdArgs a) {
         }
         const float p = exp2f(x - sLse[ii]);
         const float ds = (x == kNegInf) ? 0.f : p * (dp - sDl[ii]) * sm.dfactor(x);
-        axpy_slice<NV>(dv_acc, p, sDO + ii * D, sub);
-        axpy_slice<NV>(dk_acc, ds, sQ + ii * D, sub);
+        axpy_slice<NV>(dv_t, p, sDO + ii * D, sub);
+        axpy_slice<NV>(dk_t, ds, sQ + ii * D, sub);
+      }
+#pragma unroll
+      for (int c = 0; c < NV; ++c) {
+        dk_acc[c] += dk_t[c];
+        dv_acc[c] += dv_t[c];
       }
     }
   }

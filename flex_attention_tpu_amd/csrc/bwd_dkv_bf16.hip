@@ -430,13 +430,10 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     unsigned char part[kListRegs];
   };
   PinnedState st;
-  // K goes in multiplied by sm_scale * log2(e): the streams' scores are then in the log2 domain
+  // The streams multiply the fp32 products Q K^T by c2 (sm_scale * log2(e); softcap: 2 log2(e) sm_scale / cap)
+  // on their way into the exponent; K itself goes in as it is.
   const float c2 = SOFTCAP ? 2.f * kLog2e * a.sm_scale / a.score.cap : a.sm_scale * kLog2e;
-  auto scaled = [c2](unsigned two) {
-    const float lo = __builtin_bit_cast(float, two << 16) * c2;
-    const float hi = __builtin_bit_cast(float, two & 0xffff0000u) * c2;
-    return __builtin_bit_cast(unsigned, pack_bf16(lo, hi));
-  };
+  auto scaled = [](unsigned two) { return two; };
   // (`stage`: the wave's 16 KB of a free LDS step buffer)
   auto consume = [&](const ItemRegs& r, ItemHead& c, char* stage) {
     u32x4 kw[8], vw[8];
@@ -666,7 +663,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
                  [t6] "+v"(ta[6]), [t7] "+v"(ta[7]), [la] "+v"(la), [lw] "+v"(lw)                                \
                : [it_end] "v"(it_end), [partial] "v"(flags), [tbl] "v"(tbl_addr), [g0] "v"(loader.goff[0]),      \
                  [g1v] "v"(loader.goff[1]), [g2] "v"(loader.goff[2]), [g3] "v"(loader.goff[3]), [m0] "v"(km[0]), \
-                 [m1] "v"(km[1]), [tid4] "v"(tid4), ##__VA_ARGS__                                                \
+                 [m1] "v"(km[1]), [tid4] "v"(tid4), [c2v] "v"(c2), ##__VA_ARGS__                                                \
                : "memory", "scc", "vcc", "m0", FA_DKV_RUN_SGPRS, "v67", FA_DKV_TILE_CLOBBERS CLOB_MORE)
 #define FA_DKV_ALIBI_CLOBBERS , "s101"
     if constexpr (ALIBI) {
@@ -775,16 +772,16 @@ static int launch_dkv_plain(const BwdArgs& a, hipStream_t stream) {
 }
 
 int bwd_dkv_bf16_d128(const BwdArgs& a, hipStream_t stream) {
+  // (the generated-stream kernel caches the q tile list in LDS)
+  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nq <= dkv_cfg::MAX_LIST;
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
-      // (the generated-stream kernel caches the q tile list in LDS)
-      return a.map.nq <= dkv_cfg::MAX_LIST ? launch_dkv_plain<FLEXATTN_SCORE_NONE>(a, stream) : launch_dkv<FLEXATTN_SCORE_NONE>(a, stream);
+      return stream_ok ? launch_dkv_plain<FLEXATTN_SCORE_NONE>(a, stream) : launch_dkv<FLEXATTN_SCORE_NONE>(a, stream);
     case FLEXATTN_SCORE_ALIBI:
-      return (a.map.nq <= dkv_cfg::MAX_LIST && a.Hq == a.Hkv) ? launch_dkv_plain<FLEXATTN_SCORE_ALIBI>(a, stream)
-                                                              : launch_dkv<FLEXATTN_SCORE_ALIBI>(a, stream);
+      return (stream_ok && a.Hq == a.Hkv) ? launch_dkv_plain<FLEXATTN_SCORE_ALIBI>(a, stream)
+                                          : launch_dkv<FLEXATTN_SCORE_ALIBI>(a, stream);
     case FLEXATTN_SCORE_SOFTCAP:
-      return (a.map.nq <= dkv_cfg::MAX_LIST && a.score.cap > 0.f) ? launch_dkv_plain<FLEXATTN_SCORE_SOFTCAP>(a, stream)
-                                                                   : launch_dkv<FLEXATTN_SCORE_SOFTCAP>(a, stream);
+      return stream_ok ? launch_dkv_plain<FLEXATTN_SCORE_SOFTCAP>(a, stream) : launch_dkv<FLEXATTN_SCORE_SOFTCAP>(a, stream);
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_dkv<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);
   }
   return set_error(FLEXATTN_EINVAL, "unknown score kind %d", a.score.kind);

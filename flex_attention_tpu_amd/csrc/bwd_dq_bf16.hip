@@ -675,12 +675,13 @@ static int launch_dq_plain(const BwdArgs& a, hipStream_t stream) {
 }
 
 int bwd_dq_bf16_d128(const BwdArgs& a, hipStream_t stream) {
+  // (the generated-stream kernel caches the kv list in LDS)
+  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= dq_cfg::MAX_LIST;
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
-      // (the generated-stream kernel caches the kv list in LDS)
-      return a.map.nk <= dq_cfg::MAX_LIST ? launch_dq_plain<false>(a, stream) : launch_dq<FLEXATTN_SCORE_NONE>(a, stream);
+      return stream_ok ? launch_dq_plain<false>(a, stream) : launch_dq<FLEXATTN_SCORE_NONE>(a, stream);
     case FLEXATTN_SCORE_ALIBI:
-      return a.map.nk <= dq_cfg::MAX_LIST ? launch_dq_plain<true>(a, stream) : launch_dq<FLEXATTN_SCORE_ALIBI>(a, stream);
+      return stream_ok ? launch_dq_plain<true>(a, stream) : launch_dq<FLEXATTN_SCORE_ALIBI>(a, stream);
     case FLEXATTN_SCORE_SOFTCAP: return launch_dq<FLEXATTN_SCORE_SOFTCAP>(a, stream);
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_dq<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);
   }

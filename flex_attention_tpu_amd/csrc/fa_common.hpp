@@ -51,6 +51,7 @@ struct FwdArgs {
   void* o; float* l; float* m;
   int B, Hq, Hkv, Sq, Sk;
   float sm_scale;
+  int flags;  // FLEXATTN_FLAG_*
   ScoreArgs score;
   MaskArgs mask;
   MapArgs map;
@@ -62,6 +63,7 @@ struct BwdArgs {
   void* dq; void* dk; void* dv;
   int B, Hq, Hkv, Sq, Sk;
   float sm_scale;
+  int flags;  // FLEXATTN_FLAG_*
   ScoreArgs score;
   MaskArgs mask;
   MapArgs map;

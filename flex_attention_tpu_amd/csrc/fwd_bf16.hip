@@ -272,7 +272,6 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
     }
     const float neg_m = -m_safe * e_scale;
     float l_tile = 0.f;
-    const bf16x2 ones2 = {(bf16_t)1.0f, (bf16_t)1.0f};
     bf16x8 p[4];
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
@@ -287,7 +286,7 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
           p1 = fast_exp2(s_acc[c][e + 1] + neg_m);
         }
         bf16x2 pk = pack_bf16(p0, p1);
-        l_tile = __builtin_amdgcn_fdot2_f32_bf16(pk, ones2, l_tile, false);  // sums what P V will use
+        l_tile += p0 + p1;  // (the fp32 values: l is the softmax denominator the backward divides by)
         p[2 * c + (e >> 3)][e & 7] = pk[0];
         p[2 * c + (e >> 3)][(e & 7) + 1] = pk[1];
       }
@@ -829,24 +828,15 @@ static int launch_fwd_plain(const FwdArgs& a, hipStream_t stream) {
                                             : launch_fwd_plain_on<ALIBI, false>(a, stream);
 }
 
-// FLEXATTN_FWD_STREAM=0 sends plain-score calls to the compiled kernel too (for comparisons).
-static bool fwd_stream_enabled() {
-  const char* v = std::getenv("FLEXATTN_FWD_STREAM");
-  return v == nullptr || v[0] != '0';
-}
-
 int fwd_bf16_d128(const FwdArgs& a, hipStream_t stream) {
+  // The generated-stream kernel (one wave per SIMD, 64 q rows per wave) keeps the state rows and the
+  // merged kv list in LDS, hence the bound on the list length.
+  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= fwd_cfg::MAX_LIST;
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
-      // The generated-stream kernel (one wave per SIMD, 64 q rows per wave) keeps the state rows and the
-      // merged kv list in LDS and folds sm_scale into Q, hence the two conditions.
-      return (fwd_stream_enabled() && a.map.nk <= fwd_cfg::MAX_LIST && a.sm_scale > 0.f)
-                 ? launch_fwd_plain<false>(a, stream)
-                 : launch_fwd<FLEXATTN_SCORE_NONE>(a, stream);
+      return stream_ok ? launch_fwd_plain<false>(a, stream) : launch_fwd<FLEXATTN_SCORE_NONE>(a, stream);
     case FLEXATTN_SCORE_ALIBI:
-      return (fwd_stream_enabled() && a.map.nk <= fwd_cfg::MAX_LIST && a.sm_scale > 0.f)
-                 ? launch_fwd_plain<true>(a, stream)
-                 : launch_fwd<FLEXATTN_SCORE_ALIBI>(a, stream);
+      return stream_ok ? launch_fwd_plain<true>(a, stream) : launch_fwd<FLEXATTN_SCORE_ALIBI>(a, stream);
     case FLEXATTN_SCORE_SOFTCAP: return launch_fwd<FLEXATTN_SCORE_SOFTCAP>(a, stream);
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_fwd<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);
   }

@@ -9,10 +9,14 @@ per SIMD, so MFMA, VALU and LDS work only overlap if they are interleaved inside
 register budget only closes with a fixed allocation.  The stream below is a software pipeline over
 the tile's four 32-row q blocks c = 0..3:
 
-    A(c): S' = Q K^T - lse, dP' = dO V^T - delta  16 MFMAs, operands: 16 ds_read_b128 (rows of Q, dO)
-          (K arrives multiplied by sm_scale log2 e and LDS holds -lse and -delta, which enter through
-          the accumulator input of each chain's first MFMA: S' is already the exponent)
-    E(c): P = exp2(S'), dS = P dP'       48 VALU ops; 8 ds_read_b128 (-lse, -delta) ahead of A(c)
+    A(c): S = Q K^T, dP' = dO V^T - delta  16 MFMAs, operands: 16 ds_read_b128 (rows of Q, dO)
+          (LDS holds -lse and -delta; -delta enters through the accumulator input of the dP chain's
+          first MFMA)
+    E(c): P = exp2(c2 S - lse), dS = P dP'   64 VALU ops; 8 ds_read_b128 (-lse, -delta)
+          (c2 = sm_scale log2 e is applied to the fp32 products by the fma that subtracts lse.  Folding it
+          into the bf16 K operand instead saves those 16 fmas per block, but rounds every scaled K element
+          to bf16 again: the logits then carry an error of about 2e-3 rms with Gaussian tails, which was
+          the largest share of the maximum error of dk and dv)
     B(c): dv^T += dO^T P, dk^T += Q^T dS 16 MFMAs, operands: 32 ds_read_b64_tr_b16
 
     MFMA order:  A0 | A1 | A2 B0 | A3 B1 | B2 | B3      VALU:  - | E0 | E1 | E2 | E3 | -
@@ -24,7 +28,8 @@ The emitter (gfx950_stream.py) inserts the s_nop / s_waitcnt that the hardware h
 Register contract with the C++ side (every asm statement names the accumulation registers with
 physical-register constraints; prologue / epilogue macros are generated here too):
     a[0:63]    dv accumulators (4 x 16)      a[64:127]  dk accumulators (4 x 16)
-    a[128:159] K fragments (8 x 4), pre-scaled   a[160:191] V fragments (8 x 4)
+    a[128:159] K fragments (8 x 4)               a[160:191] V fragments (8 x 4)
+    %[c2v]     sm_scale log2(e) in every lane (softcap: 2 log2(e) sm_scale / cap)
     v[67:199]  scratch of the run loop and its streams (clobbered), s[60:100], vcc, m0 likewise
     a[192:255] staging slots of the LDS fragments (clobbered): MFMA operands only, so they can be
                AGPRs, and v[192:255] stay with the compiler for what lives across the run loop
@@ -78,8 +83,8 @@ S_T = ["s84", "s85", "s86", "s87"]
 S_GQ0, S_GQ1, S_GD0, S_GD1, S_RA, S_RB = "s[88:89]", "s[90:91]", "s[92:93]", "s[94:95]", "s[96:97]", "s[98:99]"
 S_LDSN = "s100"
 S_KC = "s101"     # (position-bias variant) 128 kb + 64: the middle of the item's kv tile
-# Softcap variant, s' = cap tanh(s / cap): K arrives multiplied by 2 log2(e) sm_scale / cap, so a chain started
-# from zero yields u with e^(2 s / cap) = 2^u; r = 1 / (2^u + 1) gives tanh = 1 - 2 r and the exponent
+# Softcap variant, s' = cap tanh(s / cap): the chain's result times 2 log2(e) sm_scale / cap (%[c2v]) is u with
+# e^(2 s / cap) = 2^u; r = 1 / (2^u + 1) gives tanh = 1 - 2 r and the exponent
 # cap' - lse - 2 cap' r with cap' = cap log2(e) (LDS holds cap' - lse; s64 = cap', s101 = -2 cap'), and
 # ds'/ds = 1 - tanh^2 = 4 r (1 - r), whose factor 4 the epilogue applies to dk.
 S_CAP, S_K2 = "s64", "s101"
@@ -147,10 +152,10 @@ def build(masked, alibi=False, softcap=False):
         if kind == "A":
             ks = x
             s, dp = V_S[c & 1], V_DP[c & 1]
-            cin = V_LSE if ks == 0 else s
+            cin = s
             cdn = V_DL if ks == 0 else dp
             first = ((vr(s, 16), ar(base, 4), ar(128 + 4 * ks, 4), "0", vset(s, 16), aset(base, 4), aset(128 + 4 * ks, 4), set())
-                     if softcap and ks == 0 else
+                     if ks == 0 else
                      (vr(s, 16), ar(base, 4), ar(128 + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(base, 4), aset(128 + 4 * ks, 4),
                       vset(cin, 16)))
             return [
@@ -191,6 +196,16 @@ def build(masked, alibi=False, softcap=False):
         s, dp = V_S[c & 1], V_DP[c & 1]
         ops = []
         for g in range(4):
+            c2v = {("op", "c2v")}
+            for u in range(4):
+                e = 4 * g + u
+                if softcap:
+                    ops.append(valu(f"v_mul_f32_e32 {vr(s + e)}, %[c2v], {vr(s + e)}", vset(s + e), vset(s + e) | c2v))
+                else:
+                    ops.append(valu(f"v_fma_f32 {vr(s + e)}, {vr(s + e)}, %[c2v], {vr(V_LSE + e)}", vset(s + e),
+                                    vset(s + e) | vset(V_LSE + e) | c2v))
+            if not softcap and c < 3:
+                ops.append(lse_read(c + 1, g))   # (the next block's row values take the registers just used)
             for u in range(4):
                 e = 4 * g + u
                 ops.append(valu(f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
@@ -244,11 +259,8 @@ def build(masked, alibi=False, softcap=False):
         if c + 2 < 4:
             ops[-1].deadline = min(ops[-1].deadline, first_A[c + 2])  # A(c + 2) writes the same S / dP registers
         e_chains.append(ops)
-    if softcap:
-        # one chain: block c + 1 must not read its row values before block c has put them there
-        chains.append([op for ops in e_chains for op in ops])
-    else:
-        chains.extend(e_chains)
+    # one chain: block c + 1 must not read its row values before block c has put them there
+    chains.append([op for ops in e_chains for op in ops])
 
     # ---- LDS reads -----------------------------------------------------------------------------
     # operand fragments of the MFMA pairs, in the order of their use: not before the pair that had
@@ -264,15 +276,14 @@ def build(masked, alibi=False, softcap=False):
     for c in range(4):
         for g in range(4):
             for reg, off in ((V_LSE, 0), (V_DL, DL_OFFSET)):
-                if softcap and reg == V_LSE:
+                if reg == V_LSE:
                     continue   # (used by E(c), not by the chain: read there, block 0 below)
                 rows.append(lds(f"ds_read_b128 {vr(reg + 4 * g, 4)}, %[la] offset:{(32 * c + 8 * g) * 4 + off}", vset(reg + 4 * g, 4),
                                 earliest=first_A[c - 1] + 6 if c else 0, deadline=max(0, first_A[c] - 6)))
     chains.append(rows)
-    if softcap:
-        first_rows = [lse_read(0, g) for g in range(4)]
-        first_rows[-1].deadline = last_A[0]
-        chains.append(first_rows)
+    first_rows = [lse_read(0, g) for g in range(4)]
+    first_rows[-1].deadline = last_A[0]
+    chains.append(first_rows)
 
     # ---- next step's Q / dO tiles: 16 LDS-direct loads per wave spread over the stream ----------
     # (issued back to back they hold the wave for about a thousand cycles: one CU moves 64 B / clk)

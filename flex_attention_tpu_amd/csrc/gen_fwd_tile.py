@@ -25,7 +25,7 @@ The softmax is arranged so that the common case costs no arithmetic beyond exp, 
     behind the test: O^T, L, the block's scores and the -M registers are corrected by the lane's
     shift, and the chain of the next kv block, already in flight with the old -M, is corrected by a
     second such block at the start of its own softmax;
-  * the row sum L accumulates the bf16-rounded p (what the PV product uses) with v_dot2c.
+  * the row sum L accumulates the fp32 p.
 State per q row: M, Mt (true maximum = M + Mt), L.  The C++ epilogue turns them into the exact
 (m, l) outputs.
 
@@ -64,6 +64,7 @@ LOAD_EVERY = 2   # gaps between two of them
 LOAD_COST = 3    # share of an MFMA gap one of them takes
 TAU = "0x40c00000"  # 6.0: M moves when the running maximum relative to it leaves [-6, 6]
 TRANS_COST = 2   # share of an MFMA gap a transcendental takes (it holds the wave's issue for two slots)
+ROUNDED_SUM = False  # row sums add the bf16-rounded probabilities (v_dot2c on the packed pairs) instead of the fp32 ones
 DROP = ()        # instruction classes left out (--drop, timing studies only)
 
 TILE = 16384
@@ -357,9 +358,12 @@ def build(masked, alibi=False):
                           deadline=a_mfma(cn, 0, q) - 6 if cn < 4 else None))
         ops.append(block(rare, earliest=rare_earliest))
 
-        # p = 2^(score - M), packed to bf16 B operands.  The row sum adds the ROUNDED values (v_dot2c on
-        # the packed pairs): o = sum(p v) / sum(p) is then consistent, which matters where a row keeps
-        # few keys (o of a single-key row is exactly v, and delta = o . dO matches dP in the backward).
+        # p = 2^(score - M), packed to bf16 B operands.  The row sum adds the fp32 values: l is then the
+        # softmax denominator of the logits themselves, which is what the backward kernels divide their
+        # recomputed probabilities by.  (Summing the rounded values, v_dot2c on the packed pairs, makes
+        # o = sum(p v) / sum(p) a convex combination whatever the rounding, but moves l, and with it every
+        # probability of the row in the backward, by up to 2^-8 relative where a row has few dominant keys:
+        # measured, that was the largest single share of the error of dk and dv.)
         def exps(g):
             for u in range(4):
                 e = 4 * g + u
@@ -376,9 +380,14 @@ def build(masked, alibi=False):
 
         # (one accumulator: splitting the chain over two registers measured slower)
         def dots(g):
-            for h in range(2):
-                pr = v_p(c, q, g >> 1) + 2 * (g & 1) + h
-                ops.append(valu(f"v_dot2c_f32_bf16_e32 {L}, 0x3f803f80, {vr(pr)}", kL, kL | vset(pr)))
+            if ROUNDED_SUM:
+                for h in range(2):
+                    pr = v_p(c, q, g >> 1) + 2 * (g & 1) + h
+                    ops.append(valu(f"v_dot2c_f32_bf16_e32 {L}, 0x3f803f80, {vr(pr)}", kL, kL | vset(pr)))
+            else:
+                for u in range(4):
+                    e = 4 * g + u
+                    ops.append(valu(f"v_add_f32_e32 {L}, {L}, {vr(s + e)}", kL, kL | vset(s + e)))
 
         exps(0)
         for g in range(4):

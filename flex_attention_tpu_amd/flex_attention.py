@@ -1,0 +1,71 @@
+"""End-to-end differentiable flex attention: forward + delta + dq + dk/dv behind one
+``torch.autograd.Function``.
+
+The reference wires its three kernels together with ``jax.custom_vjp`` (upstream copy in
+jax_exp.py:207-321: ``_flash_attention`` / ``_flash_attention_fwd`` saves ``(q, k, v, ab,
+segment_ids, o, l, m)``; ``_flash_attention_bwd`` computes ``di = sum(o * do, -1)`` in float32 and
+calls the dk/dv and the dq kernels).  This is the same wiring on the HIP entry points of this
+package, with the flex arguments (``score_fn``, ``mask_fn`` / ``block_mask_fn``) of
+flex_attention_kernel.py:66-83 carried through.
+"""
+from __future__ import annotations
+
+import math
+from typing import Callable, Optional, Tuple
+
+import torch
+
+from .flex_attention_dkv_kernel import flash_attention_bwd_dkv
+from .flex_attention_dq_bwd import compute_delta, flex_attention_bwd_dq
+from .flex_attention_kernel import _flex_attention_impl
+
+
+class _FlexAttention(torch.autograd.Function):
+    """o = softmax(mask(score_mod(sm_scale q k^T))) v with the saved statistics (l, m) for the backward."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, opts):
+        score_fn, mask_fn, block_mask_fn, segment_ids, causal, sm_scale, block_q, block_k = opts
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        o, l, m = _flex_attention_impl(q, k, v, None, segment_ids, True, causal, sm_scale, 1, block_q, block_k, block_k,
+                                       False, block_mask_fn, mask_fn, score_fn)
+        ctx.save_for_backward(q, k, v, o, l, m)
+        ctx.opts = opts
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, o, l, m = ctx.saved_tensors
+        score_fn, mask_fn, block_mask_fn, segment_ids, causal, sm_scale, block_q, block_k = ctx.opts
+        do = do.contiguous()
+        di = compute_delta(o, do)  # float32 [B, H, Sq]  (jax_exp.py:276-278)
+        dq = dk = dv = None
+        if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
+            dk, dv = flash_attention_bwd_dkv(k, v, q, None, segment_ids, l, m, di, do, block_b=1, block_q=block_q,
+                                             block_q_major=block_q, block_k_major=block_k, block_k=block_k,
+                                             sm_scale=sm_scale, causal=causal, debug=False, score_fn=score_fn,
+                                             mask_fn=mask_fn, block_mask_fn=block_mask_fn)
+        if ctx.needs_input_grad[0]:
+            dq = flex_attention_bwd_dq(q, k, v, None, segment_ids, l, m, o, do, di, block_b=1, block_q=block_q,
+                                       block_k_major=block_k, block_k=block_k, sm_scale=sm_scale, debug=False,
+                                       score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn, causal=causal)
+        return dq, dk, dv, None
+
+
+def flex_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, score_fn: Optional[Callable] = None,
+                   mask_fns: Optional[Tuple[Callable, Callable]] = None, *, segment_ids=None, causal: bool = False,
+                   sm_scale: Optional[float] = None, block_q: int = 128, block_k: int = 128) -> torch.Tensor:
+    """Differentiable flex attention on ``[B, H, S, D]`` GPU tensors (k, v may have fewer heads: GQA).
+
+    ``score_fn``   closure from ``scores`` (or ``util.make_jax_score_fn``), or None
+    ``mask_fns``   ``(mask_fn, block_mask_fn)`` pair from ``masks``, or None
+    ``segment_ids`` / ``causal``   as in the three entry points (ANDed with ``mask_fns``)
+    ``sm_scale``   default 1 / sqrt(D)
+    Gradients flow to q, k and v (``torch.autograd.grad`` / ``.backward()``); higher-order
+    differentiation is not supported, as in the reference (jax_exp.py:243-244).
+    """
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(q.shape[-1])
+    mask_fn, block_mask_fn = mask_fns if mask_fns is not None else (None, None)
+    opts = (score_fn, mask_fn, block_mask_fn, segment_ids, bool(causal), float(sm_scale), int(block_q), int(block_k))
+    return _FlexAttention.apply(q, k, v, opts)

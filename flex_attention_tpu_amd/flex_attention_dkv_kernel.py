@@ -14,7 +14,7 @@ from .flex_attention_dq_bwd import bwd_params
 
 def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=None, block_q, block_q_major,
                             block_k_major, block_k, sm_scale, causal, debug, score_fn=None, mask_fn=None,
-                            block_mask_fn=None):
+                            block_mask_fn=None, compiled_loop=False):
     """(dk, dv): dv = P^T do, dk = dS^T * d(score)/dk with P recomputed from (l, m) and
     dS = P (dP - di) (flex_attention_dkv_kernel.py:237-272).  With grouped KV heads the gradients
     of all query heads of a group are summed inside the kernel.  ``causal`` is honoured
@@ -31,7 +31,8 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     bm = kernel_block_map(_lib.PASS_DKV, spec, q, Sq, Sk, D)
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)
-    p = bwd_params(q, k, v, l, m, do, di, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dk=dk, dv=dv)
+    p = bwd_params(q, k, v, l, m, do, di, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dk=dk, dv=dv,
+                   compiled_loop=compiled_loop)
     with torch.cuda.device(q.device):
         _lib.check(_lib.load().flexattn_bwd_dkv(C.byref(p), stream_of(q)))
     return dk, dv

@@ -27,20 +27,21 @@ def compute_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
     return d
 
 
-def bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, mod_q, mod_k, dq=None, dk=None, dv=None):
+def bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, mod_q, mod_k, dq=None, dk=None, dv=None,
+               compiled_loop=False):
     B, Hq, Sq, D = q.shape
     _, Hkv, Sk, _ = k.shape
     return _lib.BwdParamsC(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), l.data_ptr(), m.data_ptr(), d.data_ptr(),
         dq.data_ptr() if dq is not None else None,
         dk.data_ptr() if dk is not None else None, dv.data_ptr() if dv is not None else None,
-        B, Hq, Hkv, Sq, Sk, D, dtype_code(q), float(sm_scale),
-        score_spec_c(score_fn, Hq, q.device, mod_q, mod_k), mask_spec_c(spec, Sq, Sk, q.device), bm.as_c())
+        B, Hq, Hkv, Sq, Sk, D, dtype_code(q), float(sm_scale), _lib.FLAG_COMPILED_LOOP if compiled_loop else 0, 0,
+        score_spec_c(score_fn, Hq, q.device, mod_q, mod_k, sm_scale), mask_spec_c(spec, Sq, Sk, q.device), bm.as_c())
 
 
 def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, block_q, block_k_major,
                           block_k, sm_scale, debug, score_fn=None, mask_fn=None, block_mask_fn=None,
-                          causal=False):
+                          causal=False, compiled_loop=False):
     """dq = sum_j dS_ij * d(score)/dq, with P_ij = exp(S_ij - m_i) / l_i recomputed from the saved
     statistics, dP = do v^T, dS = P (dP - d) (flex_attention_dq_bwd.py:340-378).  ``o`` is only
     shape-checked, as in the reference (:163); ``d`` is the caller's delta (see compute_delta)."""
@@ -55,7 +56,8 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk)
     bm = kernel_block_map(_lib.PASS_DQ, spec, q, Sq, Sk, D)
     dq = torch.empty_like(q)
-    p = bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dq=dq)
+    p = bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dq=dq,
+                   compiled_loop=compiled_loop)
     with torch.cuda.device(q.device):
         _lib.check(_lib.load().flexattn_bwd_dq(C.byref(p), stream_of(q)))
     return dq

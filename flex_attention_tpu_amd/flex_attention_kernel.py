@@ -18,13 +18,15 @@ from .block_mask import mask_spec_c
 
 
 def _flex_attention_impl(q, k, v, ab, segment_ids, save_residuals, causal, sm_scale, block_b, block_q,
-                         block_k_major, block_k, debug, block_mask_fn, mask_fn, score_fn):
+                         block_k_major, block_k, debug, block_mask_fn, mask_fn, score_fn, *, compiled_loop=False):
     """Returns ``o`` (q.dtype) or ``(o, l, m)`` with float32 ``l, m`` of shape [B, H, Sq].
 
     Semantics (flex_attention_kernel.py:248-319): S = score_mod(sm_scale * q k^T); masked
     positions are excluded; m = rowmax S, l = sum exp(S - m), o = exp(S - m) v / l.
     Unlike the reference's flex forward, ``causal=True`` is honoured (ANDed with ``mask_fn``), as
-    flash_attention_fwd_ref.py:78-86 and the dense reference do.
+    flash_attention_fwd_ref.py:78-86 and the dense reference do.  ``compiled_loop=True`` (not in the
+    reference) selects the bf16 kernel with a compiled main loop instead of the generated instruction
+    stream, for comparisons.
     """
     if ab is not None:
         raise NotImplementedError("additive bias `ab` is not supported")
@@ -40,8 +42,8 @@ def _flex_attention_impl(q, k, v, ab, segment_ids, save_residuals, causal, sm_sc
     p = _lib.FwdParamsC(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
         l.data_ptr() if l is not None else None, m.data_ptr() if m is not None else None,
-        B, Hq, Hkv, Sq, Sk, D, dtype_code(q), float(sm_scale),
-        score_spec_c(score_fn, Hq, q.device, block_q or 1, block_k or 1),
+        B, Hq, Hkv, Sq, Sk, D, dtype_code(q), float(sm_scale), _lib.FLAG_COMPILED_LOOP if compiled_loop else 0, 0,
+        score_spec_c(score_fn, Hq, q.device, block_q or 1, block_k or 1, sm_scale),
         mask_spec_c(spec, Sq, Sk, q.device), bm.as_c())
     with torch.cuda.device(q.device):
         _lib.check(_lib.load().flexattn_fwd(C.byref(p), stream_of(q)))

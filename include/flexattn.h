@@ -85,13 +85,21 @@ typedef struct flexattn_block_map {
   int32_t nq, nk, block_q, block_k;
 } flexattn_block_map;
 
+/* Call flags.  The bf16 kernels exist twice: with a generated, hand-scheduled instruction stream as
+ * main loop (the default wherever one exists for the request) and with a compiled loop (every
+ * score kind and list length).  Both meet the stated tolerances; the flag selects the compiled one
+ * for a call, for comparisons and tests. */
+#define FLEXATTN_FLAG_COMPILED_LOOP 1
+
 typedef struct flexattn_fwd_params {
   const void* q; const void* k; const void* v; /* in  */
   void* o;                                      /* out [B,Hq,Sq,D], dtype of q */
   float* l; float* m;                           /* out [B,Hq,Sq] or both NULL   */
   int32_t B, Hq, Hkv, Sq, Sk, D;
   int32_t dtype;
-  float sm_scale;
+  float sm_scale; /* > 0 */
+  int32_t flags;  /* FLEXATTN_FLAG_* */
+  int32_t reserved;
   flexattn_score_spec score;
   flexattn_mask_spec mask;
   flexattn_block_map map; /* granularity must equal flexattn_tile_shape(FLEXATTN_PASS_FWD, ...) */
@@ -104,7 +112,9 @@ typedef struct flexattn_bwd_params {
   void* dk; void* dv;  /* out of flexattn_bwd_dkv [B,Hkv,Sk,D] */
   int32_t B, Hq, Hkv, Sq, Sk, D;
   int32_t dtype;
-  float sm_scale;
+  float sm_scale; /* > 0 */
+  int32_t flags;  /* FLEXATTN_FLAG_* */
+  int32_t reserved;
   flexattn_score_spec score;
   flexattn_mask_spec mask;
   flexattn_block_map map; /* granularity of the pass being launched */

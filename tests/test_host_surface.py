@@ -179,3 +179,52 @@ def test_make_jax_score_fn_recognises_functors():
     assert make_jax_score_fn(tagged) is tagged
     with pytest.raises(NotImplementedError):
         make_jax_score_fn(unsupported)
+
+
+def test_tile_callable_convention_equals_score_mod_at_unit_scale():
+    """The reference hands `score_fn(q_tile, k_tile)` the raw tiles and applies no sm_scale in its
+    forward (flex_attention_kernel.py:249-255) nor in its dense reference (mha_reference.py:44-48);
+    the kernels here compute score_mod(sm_scale * <q, k>).  At sm_scale = 1 the two coincide: the
+    oracle's tile-callable path on this package's closures equals its score_mod path, forward and
+    backward, for the soft-cap and the tile-local ALiBi."""
+    q, k, v, do = O.make_inputs(1, 2, 2, 32, 32, 8, dtype=torch.float64, seed=5)
+    for fn, mod in ((scores.make_softcap_score_fn(3.0), O.score_mod_softcap(3.0)),
+                    (scores.make_alibi_score_fn(0.5), O.score_mod_alibi_tile_local(0.5, 32, 32))):
+        o1, l1, m1 = O.mha_reference(q, k, v, save_residuals=True, score_fn=fn, sm_scale=0.3)  # (sm_scale is ignored here)
+        o2, l2, m2 = O.mha_reference(q, k, v, save_residuals=True, score_mod=mod, sm_scale=1.0)
+        assert (o1 - o2).abs().max() < 1e-12 and (l1 - l2).abs().max() < 1e-12 and (m1 - m2).abs().max() < 1e-12
+        g1 = O.mha_bwd_reference(q, k, v, o1, do, l1, m1, score_fn=fn, sm_scale=1.0)
+        g2 = O.mha_bwd_reference(q, k, v, o2, do, l2, m2, score_mod=mod, sm_scale=1.0)
+        for a, b in zip(g1, g2):
+            assert (a - b).abs().max() < 1e-11
+
+
+def test_score_fn_with_non_unit_scale_warns():
+    from flex_attention_tpu_amd import _common
+    with pytest.warns(UserWarning, match="sm_scale"):
+        _common.score_spec_c(scores.make_softcap_score_fn(3.0), 2, "cpu", 128, 128, 0.5)
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        _common.score_spec_c(scores.make_softcap_score_fn(3.0), 2, "cpu", 128, 128, 1.0)
+        _common.score_spec_c(None, 2, "cpu", 128, 128, 0.5)
+
+
+def test_host_caches_are_bounded():
+    from flex_attention_tpu_amd import _common, block_mask
+    lru = block_mask.LRU(3)
+    for i in range(10):
+        lru.put(i, str(i))
+    assert len(lru) == 3 and lru.get(9) == "9" and lru.get(0) is None
+    lru.get(7)          # 7 becomes the most recent
+    lru.put(10, "10")   # drops 8
+    assert lru.get(8) is None and lru.get(7) == "7"
+    assert block_mask._map_cache.maxsize == block_mask.MAP_CACHE_SIZE
+    # a segment-id tensor is turned into host ids once per tensor object and version
+    ids = torch.tensor([0, 0, 1, 1, 2, 2, 2, 2], dtype=torch.int32)
+    d1 = _common.segment_doc_ids(ids)
+    assert _common.segment_doc_ids(ids) is d1
+    ids[4] = 1
+    d2 = _common.segment_doc_ids(ids)
+    assert d2 is not d1 and d2.array.tolist() == [0, 0, 1, 1, 1, 2, 2, 2]
+    assert _common.segment_doc_ids(d2) is d2
