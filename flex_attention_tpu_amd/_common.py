@@ -145,8 +145,8 @@ def score_spec_c(score_fn: Optional[Callable], Hq: int, device, mod_q: int, mod_
     spec = getattr(score_fn, "spec", None)
     if not isinstance(spec, ScoreSpec):
         raise NotImplementedError(
-            "score_fn must come from flex_attention_tpu_amd.scores factories or util.make_jax_score_fn "
-            "(arbitrary Python callables cannot be compiled into the HIP kernels)")
+            "score_fn must come from flex_attention_tpu_amd.scores factories, util.make_jax_score_fn or "
+            "compiler.compile_score_mod / compile_score_fn (which compile a Python function into the kernels)")
     slopes_ptr = None
     if spec.kind == _lib.SCORE_ALIBI:
         if len(spec.slopes) != Hq:
@@ -160,11 +160,23 @@ def score_spec_c(score_fn: Optional[Callable], Hq: int, device, mod_q: int, mod_
     return _lib.ScoreSpecC(spec.kind, spec.cap, spec.slope, int(mod_q), int(mod_k), 0, slopes_ptr)
 
 
-def kernel_block_map(pass_id: int, spec: MaskSpec, q: torch.Tensor, Sq: int, Sk: int, D: int) -> BlockMap:
+def kernel_block_map(pass_id: int, spec: MaskSpec, q: torch.Tensor, Sq: int, Sk: int, D: int, score_fn=None) -> BlockMap:
     bq, bk = _lib.tile_shape(pass_id, dtype_code(q), D)
     if Sq % bq or Sk % bk:
         raise ValueError(f"sequence lengths ({Sq}, {Sk}) must be multiples of the kernel tile ({bq}, {bk})")
-    return build_block_map(spec, Sq, Sk, bq, bk, q.device)
+    return build_block_map(spec, Sq, Sk, bq, bk, q.device, score_code=score_code_of(score_fn))
+
+
+def score_code_of(score_fn):
+    """compiler.CustomCode of a compiled score closure, else None."""
+    spec = getattr(score_fn, "spec", None)
+    return getattr(spec, "custom", None)
+
+
+def library_for(score_fn, spec: MaskSpec):
+    """The library that holds the kernels of this call: libflexattn.so, or the functor library of the call's
+    compiled closures (built at first use)."""
+    return _lib.load_for(score_code_of(score_fn), spec.custom)
 
 
 def stream_of(t: torch.Tensor) -> int:

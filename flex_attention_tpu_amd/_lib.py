@@ -24,11 +24,13 @@ SCORE_NONE = 0
 SCORE_ALIBI = 1
 SCORE_SOFTCAP = 2
 SCORE_ALIBI_TILE = 3
+SCORE_CUSTOM = 4
 
 MASK_CAUSAL = 1
 MASK_WINDOW = 2
 MASK_DOC = 4
 MASK_S2 = 8
+MASK_CUSTOM = 16
 
 FLAG_COMPILED_LOOP = 1
 
@@ -118,23 +120,17 @@ EXPORTS = (
     "flexattn_bwd_delta",
     "flexattn_bwd_dq",
     "flexattn_bwd_dkv",
+    "flexattn_custom_tag",
 )
 
 _lib = None
+_custom_libs = {}
 
 
-def load() -> C.CDLL:
-    """Loads libflexattn.so once; raises ImportError if it has not been built."""
-    global _lib
-    if _lib is not None:
-        return _lib
-    if not os.path.exists(LIB_PATH):
-        raise ImportError(
-            f"{LIB_PATH} is missing: build it with `python -m flex_attention_tpu_amd.build` "
-            "(hipcc, gfx950). This package has no other compute path.")
-    lib = C.CDLL(LIB_PATH)
+def _bind(lib: C.CDLL) -> C.CDLL:
     lib.flexattn_version.restype = C.c_int
     lib.flexattn_last_error_string.restype = C.c_char_p
+    lib.flexattn_custom_tag.restype = C.c_char_p
     lib.flexattn_tile_shape.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
     lib.flexattn_build_block_mask.argtypes = [
         C.POINTER(MaskSpecC), C.c_int32, C.c_int32, C.c_int32, C.c_int32,
@@ -146,15 +142,46 @@ def load() -> C.CDLL:
     for name in ("flexattn_tile_shape", "flexattn_build_block_mask", "flexattn_fwd", "flexattn_bwd_delta",
                  "flexattn_bwd_dq", "flexattn_bwd_dkv"):
         getattr(lib, name).restype = C.c_int
-    _lib = lib
     return lib
 
 
-def check(rc: int) -> None:
+def load() -> C.CDLL:
+    """Loads libflexattn.so once; raises ImportError if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m flex_attention_tpu_amd.build` "
+            "(hipcc, gfx950). This package has no other compute path.")
+    _lib = _bind(C.CDLL(LIB_PATH))
+    return _lib
+
+
+def load_for(score_code=None, mask_code=None) -> C.CDLL:
+    """The library whose kernels contain the given compiled closures (compiler.CustomCode objects, or None):
+    libflexattn.so when there is none, else the functor library of the pair, compiled with hipcc at first
+    use and cached on disk (compiler.build_functor_library)."""
+    if score_code is None and mask_code is None:
+        return load()
+    from . import compiler
+    key = compiler.functor_key(score_code, mask_code)
+    lib = _custom_libs.get(key)
+    if lib is None:
+        path = compiler.build_functor_library(score_code, mask_code)
+        lib = _bind(C.CDLL(path))
+        tag = lib.flexattn_custom_tag().decode()
+        if tag != key:
+            raise ImportError(f"{path} was built for functor {tag!r}, expected {key!r}: delete it and call again")
+        _custom_libs[key] = lib
+    return lib
+
+
+def check(rc: int, lib=None) -> None:
     """Maps a status code to the exception class the reference raises in the same situation."""
     if rc == OK:
         return
-    msg = load().flexattn_last_error_string().decode("utf-8", "replace")
+    msg = (lib or load()).flexattn_last_error_string().decode("utf-8", "replace")
     if rc == EINVAL:
         raise ValueError(msg)
     if rc == ENOTSUP:

@@ -111,8 +111,10 @@ def mask_spec_c(spec: MaskSpec, Sq: int, Sk: int, device) -> _lib.MaskSpecC:
 
 
 def build_block_map(spec: MaskSpec, Sq: int, Sk: int, block_q: int, block_k: int, device,
-                    cache: bool = True) -> BlockMap:
-    """Runs the GPU block-mask builder (or returns the cached map for this specification)."""
+                    cache: bool = True, score_code=None) -> BlockMap:
+    """Runs the GPU block-mask builder (or returns the cached map for this specification).  A compiled
+    mask closure is built by the functor library that holds it (`score_code`: the compiled score closure of
+    the same call, if any, so that one library serves both)."""
     device = torch.device(device)
     key = (spec, Sq, Sk, block_q, block_k, str(device))
     if cache:
@@ -122,14 +124,14 @@ def build_block_map(spec: MaskSpec, Sq: int, Sk: int, block_q: int, block_k: int
             return hit
     if Sq % block_q or Sk % block_k:
         raise ValueError(f"Sq={Sq} / Sk={Sk} not divisible by blocks {block_q} / {block_k}")
-    lib = _lib.load()
+    lib = _lib.load_for(score_code if spec.custom is not None else None, spec.custom)
     bm = BlockMap(spec, Sq, Sk, block_q, block_k, device)
     mc = mask_spec_c(spec, Sq, Sk, device)
     stream = torch.cuda.current_stream(device).cuda_stream
     with torch.cuda.device(device):
         _lib.check(lib.flexattn_build_block_mask(
             C.byref(mc), Sq, Sk, block_q, block_k, bm.state.data_ptr(), bm.kv_cnt.data_ptr(),
-            bm.kv_idx.data_ptr(), bm.q_cnt.data_ptr(), bm.q_idx.data_ptr(), stream))
+            bm.kv_idx.data_ptr(), bm.q_cnt.data_ptr(), bm.q_idx.data_ptr(), stream), lib)
         bm.built_on = stream
         bm.ready = torch.cuda.Event()
         bm.ready.record(torch.cuda.current_stream(device))
@@ -145,8 +147,8 @@ def create_block_mask(mask_fns, Sq: int, Sk: int, block_q: int, block_k: int, de
 
 
 def spec_of(mask_fn: Optional[Callable], block_mask_fn: Optional[Callable]) -> MaskSpec:
-    """MaskSpec carried by the closures.  Closures not produced by this package's factories cannot
-    be traced into a HIP kernel and are rejected."""
+    """MaskSpec carried by the closures: those of this package's factories, or of compiler.compile_mask_fn
+    for arbitrary element predicates.  Untagged closures are rejected."""
     spec = None
     for f in (mask_fn, block_mask_fn):
         if f is None:
@@ -154,8 +156,8 @@ def spec_of(mask_fn: Optional[Callable], block_mask_fn: Optional[Callable]) -> M
         s = getattr(f, "spec", None)
         if s is None:
             raise NotImplementedError(
-                "mask_fn/block_mask_fn must come from flex_attention_tpu_amd.masks factories "
-                "(arbitrary Python closures cannot be compiled into the HIP kernels)")
+                "mask_fn/block_mask_fn must come from flex_attention_tpu_amd.masks factories or from "
+                "flex_attention_tpu_amd.compiler.compile_mask_fn (which compiles a Python predicate into the kernels)")
         if spec is not None and s != spec:
             raise ValueError("mask_fn and block_mask_fn describe different masks")
         spec = s

@@ -42,15 +42,15 @@ FLAGS = [
 ]
 
 
-def _compile(src: str, force: bool) -> str:
-    obj = os.path.join(BUILD_DIR, os.path.splitext(src)[0] + ".o")
+def _compile(src: str, force: bool, build_dir: str = BUILD_DIR, extra_flags=()) -> str:
+    obj = os.path.join(build_dir, os.path.splitext(src)[0] + ".o")
     src_path = os.path.join(CSRC, src)
     if not force and os.path.exists(obj):
         deps = [src_path] + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hpp", ".inc"))]
         deps.append(os.path.join(INCLUDE, "flexattn.h"))
         if all(os.path.getmtime(d) <= os.path.getmtime(obj) for d in deps):
             return obj
-    cmd = [HIPCC, *FLAGS, "-c", src_path, "-o", obj]
+    cmd = [HIPCC, *FLAGS, *extra_flags, "-c", src_path, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
@@ -60,20 +60,22 @@ def _compile(src: str, force: bool) -> str:
     return obj
 
 
-def build_library(force: bool = True, jobs: int = 8) -> str:
-    """Compiles every HIP source for gfx950 and links libflexattn.so next to the package."""
-    os.makedirs(BUILD_DIR, exist_ok=True)
+def build_library(force: bool = True, jobs: int = 8, out_path: str = LIB_PATH, build_dir: str = BUILD_DIR,
+                  extra_flags=()) -> str:
+    """Compiles every HIP source for gfx950 and links libflexattn.so next to the package (or, with
+    `out_path` / `build_dir` / `extra_flags`, a functor library of compiler.py against its generated header)."""
+    os.makedirs(build_dir, exist_ok=True)
     for gen, out in GENERATED:
         r = subprocess.run([sys.executable, os.path.join(CSRC, gen), os.path.join(CSRC, out)], capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"{gen} failed:\n{r.stdout}\n{r.stderr}")
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(lambda s: _compile(s, force), SOURCES))
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH]
+        objs = list(ex.map(lambda s: _compile(s, force, build_dir, tuple(extra_flags)), SOURCES))
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out_path]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
-    return LIB_PATH
+    return out_path
 
 
 if __name__ == "__main__":

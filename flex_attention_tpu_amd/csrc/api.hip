@@ -57,13 +57,21 @@ static int check_score(const flexattn_score_spec& s) {
       if (s.mod_q <= 0 || s.mod_k <= 0)
         return set_error(FLEXATTN_EINVAL, "score ALIBI_TILE needs mod_q, mod_k > 0 (got %d, %d)", s.mod_q, s.mod_k);
       return FLEXATTN_OK;
+    case FLEXATTN_SCORE_CUSTOM:
+      if (!FLEXATTN_CUSTOM_HAS_SCORE)
+        return set_error(FLEXATTN_ENOTSUP, "score CUSTOM: this library was built without a compiled score function");
+      if (s.mod_q <= 0 || s.mod_k <= 0)
+        return set_error(FLEXATTN_EINVAL, "score CUSTOM needs mod_q, mod_k > 0 (got %d, %d)", s.mod_q, s.mod_k);
+      return FLEXATTN_OK;
   }
   return set_error(FLEXATTN_EINVAL, "unknown score kind %d", s.kind);
 }
 
 static int check_mask(const flexattn_mask_spec& m) {
-  const int known = FLEXATTN_MASK_CAUSAL | FLEXATTN_MASK_WINDOW | FLEXATTN_MASK_DOC | FLEXATTN_MASK_S2;
+  const int known = FLEXATTN_MASK_CAUSAL | FLEXATTN_MASK_WINDOW | FLEXATTN_MASK_DOC | FLEXATTN_MASK_S2 | FLEXATTN_MASK_CUSTOM;
   if (m.flags & ~known) return set_error(FLEXATTN_EINVAL, "unknown mask flags 0x%x", m.flags);
+  if ((m.flags & FLEXATTN_MASK_CUSTOM) && !FLEXATTN_CUSTOM_HAS_MASK)
+    return set_error(FLEXATTN_ENOTSUP, "mask CUSTOM: this library was built without a compiled mask function");
   if ((m.flags & FLEXATTN_MASK_S2) && (m.flags & (FLEXATTN_MASK_CAUSAL | FLEXATTN_MASK_WINDOW)))
     return set_error(FLEXATTN_EINVAL, "mask S2 already contains its window and causal terms; do not combine");
   if ((m.flags & (FLEXATTN_MASK_WINDOW | FLEXATTN_MASK_S2)) && m.window <= 0)
@@ -167,6 +175,8 @@ extern "C" {
 int flexattn_version(void) { return FLEXATTN_VERSION; }
 
 const char* flexattn_last_error_string(void) { return g_err; }
+
+const char* flexattn_custom_tag(void) { return FLEXATTN_CUSTOM_TAG; }
 
 int flexattn_tile_shape(int32_t pass, int32_t dtype, int32_t D, int32_t* block_q, int32_t* block_k) {
   if (block_q == nullptr || block_k == nullptr) return set_error(FLEXATTN_EINVAL, "block_q/block_k is NULL");

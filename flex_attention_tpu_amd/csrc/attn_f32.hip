@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void fwd_f32_kernel(FwdArgs a) {
   const float* Vg = static_cast<const float*>(a.v) + (size_t)(b * a.Hkv + hk) * a.Sk * D;
 
   ScoreMod<SCORE> sm;
-  sm.init(a.score, a.sm_scale, h);
+  sm.init(a.score, a.sm_scale, h, b);
   const int doc_i = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[q_idx] : 0;
 
   f32x4 qv[NV], acc[NV];
@@ -183,7 +183,7 @@ __global__ __launch_bounds__(256) void bwd_dq_f32_kernel(BwdArgs a) {
   const float* Vg = static_cast<const float*>(a.v) + (size_t)(b * a.Hkv + hk) * a.Sk * D;
 
   ScoreMod<SCORE> sm;
-  sm.init(a.score, a.sm_scale, h);
+  sm.init(a.score, a.sm_scale, h, b);
   const int doc_i = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[q_idx] : 0;
 
   f32x4 qv[NV], dov[NV], acc[NV];
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(256) void bwd_dq_f32_kernel(BwdArgs a) {
         if (!keep_elem(a.mask, q_idx, j, doc_i, doc_j)) x = kNegInf;
       }
       const float p = exp2f(x - lse2);
-      const float ds = (x == kNegInf) ? 0.f : p * (dp - dl) * sm.dfactor(x);
+      const float ds = (x == kNegInf) ? 0.f : p * (dp - dl) * sm.dfactor(x, s, q_idx, j);
       axpy_slice<NV>(acc, ds, sK + jj * D, sub);
     }
   }
@@ -261,7 +261,7 @@ __global__ __launch_bounds__(256) void bwd_dkv_f32_kernel(BwdArgs a) {
     const int h = hk * group + g;
     const size_t qbase = (size_t)(b * a.Hq + h) * a.Sq;
     ScoreMod<SCORE> sm;
-    sm.init(a.score, a.sm_scale, h);
+    sm.init(a.score, a.sm_scale, h, b);
     for (int t = 0; t < n_tiles; ++t) {
       const int qb = tile_idx[t];
       const bool partial = a.map.state[(size_t)qb * a.map.nk + kb] == 1;
@@ -293,7 +293,7 @@ __global__ __launch_bounds__(256) void bwd_dkv_f32_kernel(BwdArgs a) {
           if (!keep_elem(a.mask, i, k_idx, doc_i, doc_j)) x = kNegInf;
         }
         const float p = exp2f(x - sLse[ii]);
-        const float ds = (x == kNegInf) ? 0.f : p * (dp - sDl[ii]) * sm.dfactor(x);
+        const float ds = (x == kNegInf) ? 0.f : p * (dp - sDl[ii]) * sm.dfactor(x, s, i, k_idx);
         axpy_slice<NV>(dv_t, p, sDO + ii * D, sub);
         axpy_slice<NV>(dk_t, ds, sQ + ii * D, sub);
       }
@@ -330,6 +330,8 @@ static int launch_with_lds(Kern kern, int grid, int lds, const Args& a, hipStrea
       return launch_with_lds(KERNEL<DD, FLEXATTN_SCORE_SOFTCAP>, GRID, LDS, ARGS, stream, WHAT);      \
     case FLEXATTN_SCORE_ALIBI_TILE:                                                                   \
       return launch_with_lds(KERNEL<DD, FLEXATTN_SCORE_ALIBI_TILE>, GRID, LDS, ARGS, stream, WHAT);   \
+    case FLEXATTN_SCORE_CUSTOM:                                                                       \
+      return launch_with_lds(KERNEL<DD, FLEXATTN_SCORE_CUSTOM>, GRID, LDS, ARGS, stream, WHAT);       \
   }                                                                                                   \
   return set_error(FLEXATTN_EINVAL, "unknown score kind %d", (ARGS).score.kind);
 

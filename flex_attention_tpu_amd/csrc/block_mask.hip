@@ -8,9 +8,27 @@ namespace fa {
 // State of tile (qb, kb): 0 skip, 1 partial, 2 full.  `run` is the AND of the block predicates
 // of the flags set: causal k_start <= q_end; window q_start - k_end < window; document: the id
 // ranges read at the block ends overlap (ids are non-decreasing); S2: k_start <= q_end.
+// With a compiled mask predicate (FLEXATTN_MASK_CUSTOM) there is no closed form: the element predicate is
+// evaluated on every element of the tile, run = any kept, full = all kept, which is what the Python block
+// closure of a compiled mask returns (any(mask_fn over the tile)).
 __device__ __forceinline__ int tile_state(const MaskArgs& mk, int qb, int kb, int bq, int bk) {
   const int q_start = qb * bq, q_end = q_start + bq - 1;
   const int k_start = kb * bk, k_end = k_start + bk - 1;
+#if FLEXATTN_CUSTOM_HAS_MASK
+  if (mk.flags & FLEXATTN_MASK_CUSTOM) {
+    const bool has_doc = (mk.flags & FLEXATTN_MASK_DOC) != 0;
+    bool any = false, all = true;
+    for (int i = q_start; i <= q_end; ++i) {
+      const int doc_i = has_doc ? mk.doc_q[i] : 0;
+      for (int j = k_start; j <= k_end; ++j) {
+        const bool keep = keep_elem(mk, i, j, doc_i, has_doc ? mk.doc_k[j] : 0);
+        any = any | keep;
+        all = all & keep;
+      }
+    }
+    return any ? (all ? 2 : 1) : 0;
+  }
+#endif
   bool run = true, full = true;
   if (mk.flags & FLEXATTN_MASK_S2) {
     run = k_start <= q_end;

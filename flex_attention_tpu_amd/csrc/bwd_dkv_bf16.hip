@@ -182,7 +182,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
     const int buf = it & 1;
     const int qb = __builtin_amdgcn_readfirstlane(qb_cur);
     const bool partial = __builtin_amdgcn_readfirstlane(st_cur) == 1;
-    sm.init(a.score, a.sm_scale, hk * group + it / n_tiles);
+    sm.init(a.score, a.sm_scale, hk * group + it / n_tiles, b);
     const int qb_n2 = (it + 2 < n_iter) ? q_block_of(it + 2) : 0;
     int st_nxt = 0;
     if (it + 1 < n_iter) {
@@ -250,7 +250,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
             const int i = q0 + r0 + u;
             const float tv = sm.to_log2(s_acc[e], i, k_idx);
             float pe = fast_exp2(tv - lse4[u]);
-            float gd = pe * (dp_acc[e] - dl4[u]) * sm.dfactor(tv);
+            float gd = pe * (dp_acc[e] - dl4[u]) * sm.dfactor(tv, s_acc[e], i, k_idx);
             if (MASKED) {
               const bool keep = keep_elem(a.mask, i, k_idx, di[u], doc_j);
               pe = keep ? pe : 0.f;
@@ -307,6 +307,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
   }
 }
 
+#ifndef FLEXATTN_CUSTOM_ONLY
 // ------------------------------------------------------------------------------------------------
 // Plain score: the whole main loop runs inside generated asm statements (gen_dkv_tile.py).  One
 // statement executes a run of consecutive full tiles, or one partial tile with the lane's keep bits;
@@ -318,8 +319,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
 // the item's kv tile, exp2(t + a (j - i)) = exp2(t - a (i - j0)) 2^(a (j - j0)): the query's share joins
 // -lse in the S chain's accumulator input, the key's share is a factor of whole dk / dv rows that the
 // item epilogue applies, so the tile streams are those of the plain score.
-// SOFTCAP: s' = cap tanh(s / cap).  K goes in multiplied by 2 log2(e) sm_scale / cap, the streams turn the
-// chain's result u into r = 1 / (2^u + 1) (tanh = 1 - 2 r), the exponent (cap' - lse) - 2 cap' r with
+// SOFTCAP: s' = cap tanh(s / cap).  The streams turn the chain's result times 2 log2(e) sm_scale / cap, u, into r = 1 / (2^u + 1) (tanh = 1 - 2 r), the exponent (cap' - lse) - 2 cap' r with
 // cap' = cap log2(e) (LDS holds cap' - lse) and dS = P dP' r (1 - r); the factor 4 of 1 - tanh^2 = 4 r (1 - r)
 // goes into dk with sm_scale.
 // DOCS: the mask compares document ids; those of a partial q tile are staged through LDS (stage_doc_ids).
@@ -737,6 +737,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   }  // work items
 }
 
+#endif  // FLEXATTN_CUSTOM_ONLY
+
 template <int SCORE>
 static int launch_dkv(const BwdArgs& a, hipStream_t stream) {
   using namespace dkv_cfg;
@@ -749,6 +751,7 @@ static int launch_dkv(const BwdArgs& a, hipStream_t stream) {
   return check_launch("flexattn_bwd_dkv bf16");
 }
 
+#ifndef FLEXATTN_CUSTOM_ONLY
 template <int SCORE, bool DOCS>
 static int launch_dkv_plain_on(const BwdArgs& a, hipStream_t stream) {
   using namespace dkv_cfg;
@@ -771,7 +774,16 @@ static int launch_dkv_plain(const BwdArgs& a, hipStream_t stream) {
                                             : launch_dkv_plain_on<SCORE, false>(a, stream);
 }
 
+#endif  // FLEXATTN_CUSTOM_ONLY
+
 int bwd_dkv_bf16_d128(const BwdArgs& a, hipStream_t stream) {
+#ifdef FLEXATTN_CUSTOM_ONLY
+  switch (a.score.kind) {
+    case FLEXATTN_SCORE_NONE: return launch_dkv<FLEXATTN_SCORE_NONE>(a, stream);
+    case FLEXATTN_SCORE_CUSTOM: return launch_dkv<FLEXATTN_SCORE_CUSTOM>(a, stream);
+  }
+  return set_error(FLEXATTN_ENOTSUP, "this functor library holds the plain and the compiled score function only (kind %d asked)", a.score.kind);
+#else
   // (the generated-stream kernel caches the q tile list in LDS)
   const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nq <= dkv_cfg::MAX_LIST;
   switch (a.score.kind) {
@@ -785,6 +797,7 @@ int bwd_dkv_bf16_d128(const BwdArgs& a, hipStream_t stream) {
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_dkv<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);
   }
   return set_error(FLEXATTN_EINVAL, "unknown score kind %d", a.score.kind);
+#endif
 }
 
 void bwd_dkv_bf16_d128_tile(int* bq, int* bk) {

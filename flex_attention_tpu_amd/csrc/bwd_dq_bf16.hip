@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
   const size_t row = (size_t)bh * a.Sq + q_idx;
 
   ScoreMod<SCORE> sm;
-  sm.init(a.score, a.sm_scale, h);
+  sm.init(a.score, a.sm_scale, h, b);
 
   bf16x8 qreg[8], doreg[8];
 #pragma unroll
@@ -218,7 +218,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
             const int e = 4 * g + u;
             const float tv = sm.to_log2(s_acc[e], q_idx, j0 + u);
             const float pe = fast_exp2(tv - lse2);
-            float gd = pe * (dp_acc[e] - delta) * sm.dfactor(tv);
+            float gd = pe * (dp_acc[e] - delta) * sm.dfactor(tv, s_acc[e], q_idx, j0 + u);
             if (MASKED) gd = keep_elem(a.mask, q_idx, j0 + u, doc_i, dj[u]) ? gd : 0.f;
             dsv[u] = gd;
           }
@@ -272,6 +272,7 @@ static int launch_dq(const BwdArgs& a, hipStream_t stream) {
   return check_launch("flexattn_bwd_dq bf16");
 }
 
+#ifndef FLEXATTN_CUSTOM_ONLY
 // ------------------------------------------------------------------------------------------------
 // Plain score: the main loop runs inside generated asm statements (gen_dq_tile.py).  A step is two
 // entries of the q tile's kv list (128 kv rows); one statement executes a run of consecutive full
@@ -674,7 +675,16 @@ static int launch_dq_plain(const BwdArgs& a, hipStream_t stream) {
                                             : launch_dq_plain_on<ALIBI, false>(a, stream);
 }
 
+#endif  // FLEXATTN_CUSTOM_ONLY
+
 int bwd_dq_bf16_d128(const BwdArgs& a, hipStream_t stream) {
+#ifdef FLEXATTN_CUSTOM_ONLY
+  switch (a.score.kind) {
+    case FLEXATTN_SCORE_NONE: return launch_dq<FLEXATTN_SCORE_NONE>(a, stream);
+    case FLEXATTN_SCORE_CUSTOM: return launch_dq<FLEXATTN_SCORE_CUSTOM>(a, stream);
+  }
+  return set_error(FLEXATTN_ENOTSUP, "this functor library holds the plain and the compiled score function only (kind %d asked)", a.score.kind);
+#else
   // (the generated-stream kernel caches the kv list in LDS)
   const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= dq_cfg::MAX_LIST;
   switch (a.score.kind) {
@@ -686,6 +696,7 @@ int bwd_dq_bf16_d128(const BwdArgs& a, hipStream_t stream) {
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_dq<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);
   }
   return set_error(FLEXATTN_EINVAL, "unknown score kind %d", a.score.kind);
+#endif
 }
 
 void bwd_dq_bf16_d128_tile(int* bq, int* bk) {

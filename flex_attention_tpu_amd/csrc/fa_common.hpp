@@ -5,6 +5,21 @@
 
 #include "flexattn.h"
 
+// Functor libraries are compiled with FLEXATTN_CUSTOM_HEADER naming a generated header that defines
+// fa::custom_score, fa::custom_dscore and fa::custom_keep; the plain library gets the identities.
+#ifdef FLEXATTN_CUSTOM_HEADER
+#include FLEXATTN_CUSTOM_HEADER
+#else
+#define FLEXATTN_CUSTOM_TAG ""
+#define FLEXATTN_CUSTOM_HAS_SCORE 0
+#define FLEXATTN_CUSTOM_HAS_MASK 0
+namespace fa {
+__host__ __device__ inline float custom_score(float s, int, int, int, int, int, int) { return s; }
+__host__ __device__ inline float custom_dscore(float, int, int, int, int, int, int) { return 1.0f; }
+__host__ __device__ inline bool custom_keep(int, int) { return true; }
+}  // namespace fa
+#endif
+
 namespace fa {
 
 typedef __bf16 bf16_t;
@@ -172,6 +187,9 @@ __host__ __device__ __forceinline__ bool keep_elem(const MaskArgs& mk, int i, in
   const bool in_window = d < mk.window;
   bool keep = (!f_causal | (d >= 0)) & (!f_window | in_window) & (!f_doc | (doc_i == doc_j));
   if (f_s2) keep = keep & (d >= 0) & (in_window | ((j % mk.stride) == 0));
+#if FLEXATTN_CUSTOM_HAS_MASK
+  if (mk.flags & FLEXATTN_MASK_CUSTOM) keep = keep & custom_keep(i, j);
+#endif
   return keep;
 }
 
@@ -275,8 +293,11 @@ struct ScoreMod {
   float scale;   // sm_scale
   float a0, a1;  // kind-specific
   int mod_q, mod_k;
+  int bb, hh_;   // batch and head (custom functors)
 
-  __device__ __forceinline__ void init(const ScoreArgs& s, float sm_scale, int head) {
+  __device__ __forceinline__ void init(const ScoreArgs& s, float sm_scale, int head, int batch = 0) {
+    bb = batch;
+    hh_ = head;
     scale = sm_scale;
     c2 = sm_scale * kLog2e;
     mod_q = s.mod_q;
@@ -300,6 +321,8 @@ struct ScoreMod {
       int d = (i % mod_q) - (j % mod_k);
       d = d < 0 ? -d : d;
       return __builtin_fmaf(raw, c2, -a0 * (float)d);
+    } else if (KIND == FLEXATTN_SCORE_CUSTOM) {
+      return custom_score(raw * scale, bb, hh_, i, j, mod_q, mod_k) * kLog2e;
     } else {
       // cap*tanh(x) = cap*(1 - 2/(1 + exp(2x))), x = sm_scale*raw/cap
       float e = fast_exp2(raw * a0);
@@ -317,14 +340,24 @@ struct ScoreMod {
     return scale;
   }
 
+  // The same for kinds whose derivative depends on more than the transformed logit (compiled closures).
+  __device__ __forceinline__ float dfactor(float t, float raw, int i, int j) const {
+    if (KIND == FLEXATTN_SCORE_CUSTOM) return scale * custom_dscore(raw * scale, bb, hh_, i, j, mod_q, mod_k);
+    return dfactor(t);
+  }
+
   // dfactor() split into an element-wise part and a constant that a kernel may apply once to
   // its accumulated result: dfactor(t) == dfactor_unscaled(t) * dfactor_post_scale(sm_scale).
   __device__ __forceinline__ float dfactor_unscaled(float t) const {
     if (KIND == FLEXATTN_SCORE_SOFTCAP) return dfactor(t);
     return 1.0f;
   }
+  __device__ __forceinline__ float dfactor_unscaled(float t, float raw, int i, int j) const {
+    if (KIND == FLEXATTN_SCORE_CUSTOM) return dfactor(t, raw, i, j);
+    return dfactor_unscaled(t);
+  }
   __device__ __forceinline__ float dfactor_post_scale(float sm_scale) const {
-    if (KIND == FLEXATTN_SCORE_SOFTCAP) return 1.0f;
+    if (KIND == FLEXATTN_SCORE_SOFTCAP || KIND == FLEXATTN_SCORE_CUSTOM) return 1.0f;
     return sm_scale;
   }
 };

@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
   const int q_idx = qb * BM + q_local;
 
   ScoreMod<SCORE> sm;
-  sm.init(a.score, a.sm_scale, h);
+  sm.init(a.score, a.sm_scale, h, b);
 
   // Q^T as B operand: lane holds q row l32, 8 consecutive d per k-step.
   bf16x8 qreg[8];
@@ -342,6 +342,7 @@ static int launch_fwd(const FwdArgs& a, hipStream_t stream) {
   return check_launch("flexattn_fwd bf16");
 }
 
+#ifndef FLEXATTN_CUSTOM_ONLY
 // ------------------------------------------------------------------------------------------------
 // Plain score: the main loop runs inside generated asm statements (gen_fwd_tile.py).  A work item is
 // a pair of 128-row q tiles of one head (q block x = tile 2 qb2 + x; wave w owns rows 32 w .. of
@@ -828,7 +829,17 @@ static int launch_fwd_plain(const FwdArgs& a, hipStream_t stream) {
                                             : launch_fwd_plain_on<ALIBI, false>(a, stream);
 }
 
+#endif  // FLEXATTN_CUSTOM_ONLY
+
 int fwd_bf16_d128(const FwdArgs& a, hipStream_t stream) {
+#ifdef FLEXATTN_CUSTOM_ONLY
+  // functor library of a compiled score function: the kernels with a compiled main loop only
+  switch (a.score.kind) {
+    case FLEXATTN_SCORE_NONE: return launch_fwd<FLEXATTN_SCORE_NONE>(a, stream);
+    case FLEXATTN_SCORE_CUSTOM: return launch_fwd<FLEXATTN_SCORE_CUSTOM>(a, stream);
+  }
+  return set_error(FLEXATTN_ENOTSUP, "this functor library holds the plain and the compiled score function only (kind %d asked)", a.score.kind);
+#else
   // The generated-stream kernel (one wave per SIMD, 64 q rows per wave) keeps the state rows and the
   // merged kv list in LDS, hence the bound on the list length.
   const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= fwd_cfg::MAX_LIST;
@@ -841,6 +852,7 @@ int fwd_bf16_d128(const FwdArgs& a, hipStream_t stream) {
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_fwd<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);
   }
   return set_error(FLEXATTN_EINVAL, "unknown score kind %d", a.score.kind);
+#endif
 }
 
 void fwd_bf16_d128_tile(int* bq, int* bk) {

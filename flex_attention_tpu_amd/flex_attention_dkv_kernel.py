@@ -8,7 +8,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import check_blocks, check_qkv, check_rows, kernel_block_map, resolve_mask, stream_of
+from ._common import check_blocks, check_qkv, check_rows, kernel_block_map, library_for, resolve_mask, stream_of
 from .flex_attention_dq_bwd import bwd_params
 
 
@@ -28,11 +28,12 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k,
                  block_q_major=block_q_major)
     spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk)
-    bm = kernel_block_map(_lib.PASS_DKV, spec, q, Sq, Sk, D)
+    bm = kernel_block_map(_lib.PASS_DKV, spec, q, Sq, Sk, D, score_fn)
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)
     p = bwd_params(q, k, v, l, m, do, di, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dk=dk, dv=dv,
                    compiled_loop=compiled_loop)
     with torch.cuda.device(q.device):
-        _lib.check(_lib.load().flexattn_bwd_dkv(C.byref(p), stream_of(q)))
+        lib = library_for(score_fn, spec)
+        _lib.check(lib.flexattn_bwd_dkv(C.byref(p), stream_of(q)), lib)
     return dk, dv

@@ -12,8 +12,8 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (check_blocks, check_qkv, dtype_code, kernel_block_map, resolve_mask, score_spec_c,
-                      stream_of)
+from ._common import (check_blocks, check_qkv, dtype_code, kernel_block_map, library_for, resolve_mask,
+                      score_spec_c, stream_of)
 from .block_mask import mask_spec_c
 
 
@@ -33,7 +33,7 @@ def _flex_attention_impl(q, k, v, ab, segment_ids, save_residuals, causal, sm_sc
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v)
     check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k)
     spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk)
-    bm = kernel_block_map(_lib.PASS_FWD, spec, q, Sq, Sk, D)
+    bm = kernel_block_map(_lib.PASS_FWD, spec, q, Sq, Sk, D, score_fn)
     o = torch.empty_like(q)
     l = m = None
     if save_residuals:
@@ -46,7 +46,8 @@ def _flex_attention_impl(q, k, v, ab, segment_ids, save_residuals, causal, sm_sc
         score_spec_c(score_fn, Hq, q.device, block_q or 1, block_k or 1, sm_scale),
         mask_spec_c(spec, Sq, Sk, q.device), bm.as_c())
     with torch.cuda.device(q.device):
-        _lib.check(_lib.load().flexattn_fwd(C.byref(p), stream_of(q)))
+        lib = library_for(score_fn, spec)
+        _lib.check(lib.flexattn_fwd(C.byref(p), stream_of(q)), lib)
     if debug:
         print(f"[flexattn_fwd] B={B} Hq={Hq} Hkv={Hkv} Sq={Sq} Sk={Sk} D={D} dtype={q.dtype} "
               f"mask_flags={spec.flags} tiles_run={int((bm.state != 0).sum())}/{bm.nq * bm.nk}")

@@ -49,9 +49,17 @@ class MaskSpec:
     window: int = 0
     stride: int = 0
     doc_ids: Optional[DocIds] = None
+    custom: Optional[object] = None   # compiler.CustomCode of a compiled mask closure (flag MASK_CUSTOM)
 
     def combine(self, other: "MaskSpec") -> "MaskSpec":
         """Spec of the AND of two masks."""
+        if self.custom is not None and other.custom is not None and self.custom != other.custom:
+            raise NotImplementedError("two different compiled mask functions cannot be combined; AND them in one function")
+        custom = self.custom if self.custom is not None else other.custom
+        out = self._combine_builtin(other)
+        return MaskSpec(out.flags, out.window, out.stride, out.doc_ids, custom)
+
+    def _combine_builtin(self, other: "MaskSpec") -> "MaskSpec":
         if self.doc_ids is not None and other.doc_ids is not None and self.doc_ids != other.doc_ids:
             raise NotImplementedError("two different document masks cannot be combined")
         doc = self.doc_ids if self.doc_ids is not None else other.doc_ids

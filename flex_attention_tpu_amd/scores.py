@@ -22,6 +22,7 @@ class ScoreSpec:
     cap: float = 0.0
     slope: float = 0.0
     slopes: Optional[Tuple[float, ...]] = None  # per-head slopes (global ALiBi)
+    custom: Optional[object] = None             # compiler.CustomCode of a compiled closure (kind SCORE_CUSTOM)
 
 
 def _tag(fn, spec):

@@ -44,6 +44,8 @@ extern "C" {
 #define FLEXATTN_SCORE_ALIBI 1      /* s + slopes[h] * (j - i)                     */
 #define FLEXATTN_SCORE_SOFTCAP 2    /* cap * tanh(s / cap)            scores.py:13-18 */
 #define FLEXATTN_SCORE_ALIBI_TILE 3 /* s - slope * |i % mod_q - j % mod_k|  scores.py:3-11 */
+#define FLEXATTN_SCORE_CUSTOM 4     /* the score function compiled into this library (functor libraries only,
+                                       see flexattn_custom_tag); mod_q, mod_k: tile edges for tile-local indices */
 
 typedef struct flexattn_score_spec {
   int32_t kind;
@@ -62,6 +64,7 @@ typedef struct flexattn_score_spec {
 #define FLEXATTN_MASK_WINDOW 2
 #define FLEXATTN_MASK_DOC 4
 #define FLEXATTN_MASK_S2 8
+#define FLEXATTN_MASK_CUSTOM 16 /* AND the mask function compiled into this library (functor libraries only) */
 
 typedef struct flexattn_mask_spec {
   int32_t flags;
@@ -128,6 +131,13 @@ int flexattn_version(void);
 
 /* Message for the calling thread's most recent non-OK return ("" if none). */
 const char* flexattn_last_error_string(void);
+
+/* A functor library is this same library compiled against a generated header that defines a score
+ * function s' = f(s, b, h, i, j) with its derivative and / or a mask predicate keep(i, j): the successor of
+ * the reference's tracing of arbitrary closures into its kernels (flex_attention_kernel.py:248-255,
+ * 278-288; util.py:22-189, 196-259).  Returns the hash that names the functor pair, "" for the plain
+ * library, which rejects FLEXATTN_SCORE_CUSTOM and FLEXATTN_MASK_CUSTOM with FLEXATTN_ENOTSUP. */
+const char* flexattn_custom_tag(void);
 
 /* Tile granularity (block_q, block_k) the kernels of `pass` expect of the block map for this
  * dtype and head dimension. */

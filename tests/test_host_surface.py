@@ -168,7 +168,7 @@ def test_make_jax_score_fn_recognises_functors():
         return torch.einsum("qd,kd->qk", q_tile, k_tile)
 
     def unsupported(q_tile, k_tile):
-        return (q_tile @ k_tile.T) ** 2
+        return torch.softmax(q_tile @ k_tile.T, -1)
 
     s = make_jax_score_fn(softcap).spec
     assert s.kind == _lib.SCORE_SOFTCAP and abs(s.cap - cap) < 1e-6
