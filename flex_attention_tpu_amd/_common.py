@@ -68,6 +68,8 @@ def check_blocks(Sq, Sk, block_q=None, block_k_major=None, block_k=None, block_q
             return
         if not isinstance(blk, (int, np.integer)) or blk <= 0:
             raise ValueError(f"{name}={blk!r} must be a positive int")
+        if n % SEQ_ALIGN:
+            return  # ragged length: the tensors are padded to the tile; the reference floors silently here (flex_attention_kernel.py:91)
         if n % blk:
             raise ValueError(f"{name}={blk} does not divide sequence length {n}")
     _div("block_q", block_q, Sq)
@@ -80,19 +82,10 @@ def check_blocks(Sq, Sk, block_q=None, block_k_major=None, block_k=None, block_q
         raise ValueError(f"block_q={block_q} does not divide block_q_major={block_q_major}")
 
 
-def segment_doc_ids(segment_ids) -> DocIds:
-    """DocIds (host copy + hash) of a ``segment_ids`` argument: a 1-D id array, a [B, S] array whose rows
-    agree, or an object with equal ``.q`` / ``.kv`` arrays (the reference's SegmentIds,
-    jax_exp.py:37-51).  A DocIds passes through, and a tensor seen before (same object, unchanged) is
-    answered from a small cache, so that a training step does not copy the ids to the host and
-    hash them once per pass."""
-    if isinstance(segment_ids, DocIds):
-        return segment_ids
-    ids = segment_ids
-    if hasattr(ids, "q") and hasattr(ids, "kv"):
-        if ids.q is not ids.kv and not torch.equal(torch.as_tensor(ids.q), torch.as_tensor(ids.kv)):
-            raise NotImplementedError("distinct q / kv segment ids are not supported")
-        ids = ids.q
+def _doc_ids_of(ids) -> DocIds:
+    """DocIds (host copy + hash) of one id array.  A DocIds passes through, and a tensor seen before (same
+    object, unchanged) is answered from a small cache, so that a training step does not copy the ids to the
+    host and hash them once per pass."""
     if isinstance(ids, DocIds):
         return ids
     key = id(ids)
@@ -103,30 +96,75 @@ def segment_doc_ids(segment_ids) -> DocIds:
     t = torch.as_tensor(ids).detach().cpu()
     if t.ndim == 2:
         if not bool((t == t[:1]).all()):
-            raise NotImplementedError("per-batch segment ids are not supported")
+            raise NotImplementedError("per-batch segment ids are not supported (every batch entry must carry the same ids)")
         t = t[0]
     if t.ndim != 1:
         raise ValueError("segment_ids must be a 1-D (or [B, S]) array of ids")
-    arr = t.numpy().astype(np.int64)
-    if np.any(np.diff(arr) < 0):
-        raise NotImplementedError("segment ids must be non-decreasing along the sequence")
-    doc = DocIds(arr)
+    doc = DocIds(t.numpy().astype(np.int64))
     if isinstance(ids, torch.Tensor):
         _segment_cache.put(key, (weakref.ref(ids), ids._version, doc))
     return doc
 
 
-def resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk) -> MaskSpec:
-    """Single MaskSpec for the closures, the ``causal`` flag and ``segment_ids`` (AND of all)."""
+def segment_doc_ids(segment_ids):
+    """(q ids, kv ids or None) of a ``segment_ids`` argument: one id array for both sides (1-D, or [B, S] with
+    equal rows), or an object with ``.q`` / ``.kv`` arrays (the reference's SegmentIds, jax_exp.py:37-51),
+    which may differ and need not be sorted."""
+    if hasattr(segment_ids, "q") and hasattr(segment_ids, "kv") and not isinstance(segment_ids, DocIds):
+        dq = _doc_ids_of(segment_ids.q)
+        dk = dq if segment_ids.kv is segment_ids.q else _doc_ids_of(segment_ids.kv)
+        return dq, (None if dk == dq else dk)
+    return _doc_ids_of(segment_ids), None
+
+
+def resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk, Sq_pad=None, Sk_pad=None) -> MaskSpec:
+    """Single MaskSpec for the closures, the ``causal`` flag and ``segment_ids`` (AND of all).  ``Sq_pad`` /
+    ``Sk_pad``: the lengths the tensors are padded to for the kernels (ragged lengths).  Padded keys must
+    receive no probability: they get a document id of their own (the document mask is switched on for
+    the call if it was not), so that the kernels need no separate length bound."""
+    Sq_pad, Sk_pad = Sq_pad or Sq, Sk_pad or Sk
     spec = spec_of(mask_fn, block_mask_fn)
     if causal:
         spec = spec.combine(MaskSpec(flags=_lib.MASK_CAUSAL))
     if segment_ids is not None:
-        doc = segment_doc_ids(segment_ids)
-        if len(doc) != Sq or Sq != Sk:
-            raise ValueError("segment_ids must have one id per position of a self-attention sequence")
-        spec = spec.combine(MaskSpec(flags=_lib.MASK_DOC, doc_ids=doc))
+        dq, dk = segment_doc_ids(segment_ids)
+        if len(dq) != Sq or len(dk if dk is not None else dq) != Sk:
+            raise ValueError(f"segment_ids must have one id per position ({Sq} q, {Sk} kv); give an object with "
+                             ".q / .kv arrays when the two lengths differ")
+        spec = spec.combine(MaskSpec(flags=_lib.MASK_DOC, doc_ids=dq, doc_ids_k=dk))
+    if Sq_pad != Sq or Sk_pad != Sk:
+        if spec.flags & _lib.MASK_DOC:
+            ids_q = spec.doc_ids.array
+            ids_k = (spec.doc_ids_k if spec.doc_ids_k is not None else spec.doc_ids).array
+            if len(ids_q) < Sq or len(ids_k) < Sk:
+                raise ValueError(f"document ids cover {len(ids_q)} q / {len(ids_k)} kv positions, need {Sq} / {Sk}")
+            ids_q, ids_k = ids_q[:Sq], ids_k[:Sk]
+        else:
+            ids_q, ids_k = np.zeros(Sq, np.int32), np.zeros(Sk, np.int32)
+        pad_id = int(max(ids_q.max(initial=0), ids_k.max(initial=0))) + 1    # an id no query carries
+        dq_p = DocIds(np.pad(ids_q, (0, Sq_pad - Sq), mode="edge"))
+        dk_p = DocIds(np.pad(ids_k, (0, Sk_pad - Sk), constant_values=pad_id))
+        spec = MaskSpec(spec.flags | _lib.MASK_DOC, spec.window, spec.stride, dq_p, spec.custom, None if dk_p == dq_p else dk_p)
     return spec
+
+
+SEQ_ALIGN = 128   # every kernel's tiles divide it
+
+
+def padded_len(n: int) -> int:
+    return (n + SEQ_ALIGN - 1) // SEQ_ALIGN * SEQ_ALIGN
+
+
+def pad_seq(t: torch.Tensor, n: int, dim: int = 2) -> torch.Tensor:
+    """`t` zero-padded to n positions along `dim` (a copy only when padding is needed)."""
+    have = t.shape[dim]
+    if have == n:
+        return t
+    shape = list(t.shape)
+    shape[dim] = n
+    out = t.new_zeros(shape)
+    out.narrow(dim, 0, have).copy_(t)
+    return out
 
 
 def score_spec_c(score_fn: Optional[Callable], Hq: int, device, mod_q: int, mod_k: int, sm_scale=None) -> _lib.ScoreSpecC:

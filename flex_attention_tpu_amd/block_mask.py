@@ -99,15 +99,17 @@ def doc_ids_on(doc: Optional[DocIds], device) -> Optional[torch.Tensor]:
 
 
 def mask_spec_c(spec: MaskSpec, Sq: int, Sk: int, device) -> _lib.MaskSpecC:
-    """C view of a MaskSpec; validates the document array length."""
-    doc_ptr = None
+    """C view of a MaskSpec; validates the document array lengths."""
+    doc_q = doc_k = None
     if spec.flags & _lib.MASK_DOC:
         if spec.doc_ids is None:
             raise ValueError("document mask without document ids")
-        if len(spec.doc_ids) < max(Sq, Sk):
-            raise ValueError(f"document ids cover {len(spec.doc_ids)} positions, need {max(Sq, Sk)}")
-        doc_ptr = doc_ids_on(spec.doc_ids, device).data_ptr()
-    return _lib.MaskSpecC(spec.flags, spec.window, spec.stride, 0, doc_ptr, doc_ptr)
+        ids_k = spec.doc_ids_k if spec.doc_ids_k is not None else spec.doc_ids
+        if len(spec.doc_ids) < Sq or len(ids_k) < Sk:
+            raise ValueError(f"document ids cover {len(spec.doc_ids)} q / {len(ids_k)} kv positions, need {Sq} / {Sk}")
+        doc_q = doc_ids_on(spec.doc_ids, device).data_ptr()
+        doc_k = doc_ids_on(ids_k, device).data_ptr()
+    return _lib.MaskSpecC(spec.flags, spec.window, spec.stride, 0, doc_q, doc_k)
 
 
 def build_block_map(spec: MaskSpec, Sq: int, Sk: int, block_q: int, block_k: int, device,

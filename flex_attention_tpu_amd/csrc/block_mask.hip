@@ -11,7 +11,7 @@ namespace fa {
 // With a compiled mask predicate (FLEXATTN_MASK_CUSTOM) there is no closed form: the element predicate is
 // evaluated on every element of the tile, run = any kept, full = all kept, which is what the Python block
 // closure of a compiled mask returns (any(mask_fn over the tile)).
-__device__ __forceinline__ int tile_state(const MaskArgs& mk, int qb, int kb, int bq, int bk) {
+__device__ __forceinline__ int tile_state(const MaskArgs& mk, int qb, int kb, int bq, int bk, bool sorted_ids) {
   const int q_start = qb * bq, q_end = q_start + bq - 1;
   const int k_start = kb * bk, k_end = k_start + bk - 1;
 #if FLEXATTN_CUSTOM_HAS_MASK
@@ -44,8 +44,22 @@ __device__ __forceinline__ int tile_state(const MaskArgs& mk, int qb, int kb, in
     }
   }
   if (mk.flags & FLEXATTN_MASK_DOC) {
-    const int qmin = mk.doc_q[q_start], qmax = mk.doc_q[q_end];
-    const int kmin = mk.doc_k[k_start], kmax = mk.doc_k[k_end];
+    // smallest and largest id of each block: read at the block ends when the ids are sorted (what the
+    // reference's closure does, masks.py:113-139), by a scan of the block otherwise
+    int qmin = mk.doc_q[q_start], qmax = mk.doc_q[q_end];
+    int kmin = mk.doc_k[k_start], kmax = mk.doc_k[k_end];
+    if (!sorted_ids) {
+      for (int i = q_start; i <= q_end; ++i) {
+        const int d = mk.doc_q[i];
+        qmin = d < qmin ? d : qmin;
+        qmax = d > qmax ? d : qmax;
+      }
+      for (int j = k_start; j <= k_end; ++j) {
+        const int d = mk.doc_k[j];
+        kmin = d < kmin ? d : kmin;
+        kmax = d > kmax ? d : kmax;
+      }
+    }
     const int lo = qmin > kmin ? qmin : kmin;
     const int hi = qmax < kmax ? qmax : kmax;
     run = run && (lo <= hi);
@@ -60,6 +74,15 @@ __global__ __launch_bounds__(64) void block_mask_kernel(MaskArgs mk, int nq, int
                                                         uint8_t* state, int* kv_cnt, int* kv_idx,
                                                         int* q_cnt, int* q_idx) {
   const int lane = threadIdx.x;
+  // Are the document ids non-decreasing on both sides?  Every work-group checks for itself (the arrays are
+  // a few KB): the block ends then bound a block's ids.
+  bool sorted_ids = true;
+  if (mk.flags & FLEXATTN_MASK_DOC) {
+    bool ok = true;
+    for (int i = lane + 1; i < nq * bq; i += 64) ok = ok && (mk.doc_q[i - 1] <= mk.doc_q[i]);
+    for (int j = lane + 1; j < nk * bk; j += 64) ok = ok && (mk.doc_k[j - 1] <= mk.doc_k[j]);
+    sorted_ids = __ballot(!ok) == 0ull;
+  }
   const bool is_row = (int)blockIdx.x < nq;
   const int major = is_row ? blockIdx.x : blockIdx.x - nq;
   const int n_minor = is_row ? nk : nq;
@@ -70,7 +93,7 @@ __global__ __launch_bounds__(64) void block_mask_kernel(MaskArgs mk, int nq, int
     const int minor = base + lane;
     int st = 0;
     if (minor < n_minor) {
-      st = is_row ? tile_state(mk, major, minor, bq, bk) : tile_state(mk, minor, major, bq, bk);
+      st = is_row ? tile_state(mk, major, minor, bq, bk, sorted_ids) : tile_state(mk, minor, major, bq, bk, sorted_ids);
       if (is_row) state[(size_t)major * nk + minor] = (uint8_t)st;
     }
     const unsigned long long ballot = __ballot(st != 0);

@@ -8,7 +8,8 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import check_blocks, check_qkv, check_rows, kernel_block_map, library_for, resolve_mask, stream_of
+from ._common import (check_blocks, check_qkv, check_rows, kernel_block_map, library_for, pad_seq, padded_len,
+                      resolve_mask, stream_of)
 from .flex_attention_dq_bwd import bwd_params
 
 
@@ -27,8 +28,12 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
         check_rows(name, t, B, Hq, Sq, q.device)
     check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k,
                  block_q_major=block_q_major)
-    spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk)
-    bm = kernel_block_map(_lib.PASS_DKV, spec, q, Sq, Sk, D, score_fn)
+    # ragged lengths: zero-padded to the kernels' tiles (padded rows carry l = 0 and dO = 0: they add nothing)
+    Sq_p, Sk_p = padded_len(Sq), padded_len(Sk)
+    spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk, Sq_p, Sk_p)
+    q, do, k, v = pad_seq(q, Sq_p), pad_seq(do, Sq_p), pad_seq(k, Sk_p), pad_seq(v, Sk_p)
+    l, m, di = pad_seq(l, Sq_p), pad_seq(m, Sq_p), pad_seq(di, Sq_p)
+    bm = kernel_block_map(_lib.PASS_DKV, spec, q, Sq_p, Sk_p, D, score_fn)
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)
     p = bwd_params(q, k, v, l, m, do, di, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dk=dk, dv=dv,
@@ -36,4 +41,6 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     with torch.cuda.device(q.device):
         lib = library_for(score_fn, spec)
         _lib.check(lib.flexattn_bwd_dkv(C.byref(p), stream_of(q)), lib)
+    if Sk_p != Sk:
+        dk, dv = dk[:, :, :Sk].contiguous(), dv[:, :, :Sk].contiguous()
     return dk, dv

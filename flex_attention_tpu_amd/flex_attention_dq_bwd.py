@@ -7,8 +7,8 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (check_blocks, check_qkv, check_rows, dtype_code, kernel_block_map, library_for,
-                      resolve_mask, score_spec_c, stream_of)
+from ._common import (check_blocks, check_qkv, check_rows, dtype_code, kernel_block_map, library_for, pad_seq,
+                      padded_len, resolve_mask, score_spec_c, stream_of)
 from .block_mask import mask_spec_c
 
 
@@ -53,12 +53,18 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     for name, t in (("l", l), ("m", m), ("d", d)):
         check_rows(name, t, B, Hq, Sq, q.device)
     check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k)
-    spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk)
-    bm = kernel_block_map(_lib.PASS_DQ, spec, q, Sq, Sk, D, score_fn)
+    # ragged lengths: zero-padded to the kernels' tiles (padded rows carry l = 0: their probabilities vanish)
+    Sq_p, Sk_p = padded_len(Sq), padded_len(Sk)
+    spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk, Sq_p, Sk_p)
+    q, do, k, v = pad_seq(q, Sq_p), pad_seq(do, Sq_p), pad_seq(k, Sk_p), pad_seq(v, Sk_p)
+    l, m, d = pad_seq(l, Sq_p), pad_seq(m, Sq_p), pad_seq(d, Sq_p)
+    bm = kernel_block_map(_lib.PASS_DQ, spec, q, Sq_p, Sk_p, D, score_fn)
     dq = torch.empty_like(q)
     p = bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dq=dq,
                    compiled_loop=compiled_loop)
     with torch.cuda.device(q.device):
         lib = library_for(score_fn, spec)
         _lib.check(lib.flexattn_bwd_dq(C.byref(p), stream_of(q)), lib)
+    if Sq_p != Sq:
+        dq = dq[:, :, :Sq].contiguous()
     return dq

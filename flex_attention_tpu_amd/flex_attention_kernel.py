@@ -12,8 +12,8 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (check_blocks, check_qkv, dtype_code, kernel_block_map, library_for, resolve_mask,
-                      score_spec_c, stream_of)
+from ._common import (check_blocks, check_qkv, dtype_code, kernel_block_map, library_for, pad_seq, padded_len,
+                      resolve_mask, score_spec_c, stream_of)
 from .block_mask import mask_spec_c
 
 
@@ -32,22 +32,30 @@ def _flex_attention_impl(q, k, v, ab, segment_ids, save_residuals, causal, sm_sc
         raise NotImplementedError("additive bias `ab` is not supported")
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v)
     check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k)
-    spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk)
-    bm = kernel_block_map(_lib.PASS_FWD, spec, q, Sq, Sk, D, score_fn)
+    # ragged lengths: the tensors are zero-padded to the kernels' tiles, a key bound drops the padded keys
+    # and the padded query rows are cut off again
+    Sq_p, Sk_p = padded_len(Sq), padded_len(Sk)
+    spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk, Sq_p, Sk_p)
+    q, k, v = pad_seq(q, Sq_p), pad_seq(k, Sk_p), pad_seq(v, Sk_p)
+    bm = kernel_block_map(_lib.PASS_FWD, spec, q, Sq_p, Sk_p, D, score_fn)
     o = torch.empty_like(q)
     l = m = None
     if save_residuals:
-        l = torch.empty(B, Hq, Sq, dtype=torch.float32, device=q.device)
-        m = torch.empty(B, Hq, Sq, dtype=torch.float32, device=q.device)
+        l = torch.empty(B, Hq, Sq_p, dtype=torch.float32, device=q.device)
+        m = torch.empty(B, Hq, Sq_p, dtype=torch.float32, device=q.device)
     p = _lib.FwdParamsC(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
         l.data_ptr() if l is not None else None, m.data_ptr() if m is not None else None,
-        B, Hq, Hkv, Sq, Sk, D, dtype_code(q), float(sm_scale), _lib.FLAG_COMPILED_LOOP if compiled_loop else 0, 0,
+        B, Hq, Hkv, Sq_p, Sk_p, D, dtype_code(q), float(sm_scale), _lib.FLAG_COMPILED_LOOP if compiled_loop else 0, 0,
         score_spec_c(score_fn, Hq, q.device, block_q or 1, block_k or 1, sm_scale),
-        mask_spec_c(spec, Sq, Sk, q.device), bm.as_c())
+        mask_spec_c(spec, Sq_p, Sk_p, q.device), bm.as_c())
     with torch.cuda.device(q.device):
         lib = library_for(score_fn, spec)
         _lib.check(lib.flexattn_fwd(C.byref(p), stream_of(q)), lib)
+    if Sq_p != Sq:
+        o = o[:, :, :Sq].contiguous()
+        if save_residuals:
+            l, m = l[:, :, :Sq].contiguous(), m[:, :, :Sq].contiguous()
     if debug:
         print(f"[flexattn_fwd] B={B} Hq={Hq} Hkv={Hkv} Sq={Sq} Sk={Sk} D={D} dtype={q.dtype} "
               f"mask_flags={spec.flags} tiles_run={int((bm.state != 0).sum())}/{bm.nq * bm.nk}")

@@ -21,7 +21,7 @@ from . import _lib
 
 
 class DocIds:
-    """Immutable per-position document ids (int32, non-decreasing) with a precomputed hash."""
+    """Immutable per-position document ids (int32) with a precomputed hash."""
     __slots__ = ("array", "_key", "_hash")
 
     def __init__(self, ids):
@@ -48,8 +48,9 @@ class MaskSpec:
     flags: int = 0
     window: int = 0
     stride: int = 0
-    doc_ids: Optional[DocIds] = None
-    custom: Optional[object] = None   # compiler.CustomCode of a compiled mask closure (flag MASK_CUSTOM)
+    doc_ids: Optional[DocIds] = None      # ids of the q positions (and of the kv positions unless doc_ids_k is given)
+    custom: Optional[object] = None       # compiler.CustomCode of a compiled mask closure (flag MASK_CUSTOM)
+    doc_ids_k: Optional[DocIds] = None    # ids of the kv positions where they differ from the q side
 
     def combine(self, other: "MaskSpec") -> "MaskSpec":
         """Spec of the AND of two masks."""
@@ -57,10 +58,13 @@ class MaskSpec:
             raise NotImplementedError("two different compiled mask functions cannot be combined; AND them in one function")
         custom = self.custom if self.custom is not None else other.custom
         out = self._combine_builtin(other)
-        return MaskSpec(out.flags, out.window, out.stride, out.doc_ids, custom)
+        flags = out.flags | ((self.flags | other.flags) & _lib.MASK_CUSTOM)
+        doc_k = self.doc_ids_k if self.doc_ids is not None else other.doc_ids_k
+        return MaskSpec(flags, out.window, out.stride, out.doc_ids, custom, doc_k)
 
     def _combine_builtin(self, other: "MaskSpec") -> "MaskSpec":
-        if self.doc_ids is not None and other.doc_ids is not None and self.doc_ids != other.doc_ids:
+        if self.doc_ids is not None and other.doc_ids is not None and \
+                (self.doc_ids != other.doc_ids or self.doc_ids_k != other.doc_ids_k):
             raise NotImplementedError("two different document masks cannot be combined")
         doc = self.doc_ids if self.doc_ids is not None else other.doc_ids
         if (self.flags | other.flags) & _lib.MASK_S2:

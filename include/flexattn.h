@@ -71,7 +71,7 @@ typedef struct flexattn_mask_spec {
   int32_t window;
   int32_t stride;
   int32_t reserved;
-  const int32_t* doc_q; /* DOC: device int32 [Sq] */
+  const int32_t* doc_q; /* DOC: device int32 [Sq]: any ids (they need not be sorted) */
   const int32_t* doc_k; /* DOC: device int32 [Sk] (may equal doc_q) */
 } flexattn_mask_spec;
 

@@ -455,10 +455,97 @@ def test_autograd_function_end_to_end(F, case):
     assert torch.equal(qg.grad, dq) and kg.grad is None
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+@pytest.mark.parametrize("case", ["plain_200x300", "causal_1000", "softcap_causal_window_700", "alibi_causal_333",
+                                  "documents_900", "gqa_causal_130"])
+def test_ragged_sequence_lengths(F, case, dtype):
+    """Lengths that are no multiple of the kernels' tiles (the reference's drivers use Sk = 25600 with
+    1024-blocks, bwd_dq.py:389-390): the entry points pad to the tile, padded keys get no probability, and
+    every output has the caller's lengths."""
+    from flex_attention_tpu_amd import masks, scores
+    sc = 1 / math.sqrt(128)
+    B, Hq, Hkv, mf, sfn, okw, sid = 1, 2, 2, (None, None), None, {}, None
+    if case == "plain_200x300":
+        Sq, Sk = 200, 300
+    elif case == "causal_1000":
+        Sq = Sk = 1000
+        mf, okw = masks.make_causal_mask_fns(128, 128), dict(causal=True)
+    elif case == "softcap_causal_window_700":
+        Sq = Sk = 700
+        mf, sfn = masks.make_causal_sliding_window_mask_fns(128, 128, 200), scores.make_softcap_score_fn(10.0)
+        okw = dict(causal=True, window_size=200, score_mod=O.score_mod_softcap(10.0))
+    elif case == "alibi_causal_333":
+        Sq = Sk = 333
+        mf, sfn = masks.make_causal_mask_fns(128, 128), scores.make_alibi_global_score_fn(2)
+        okw = dict(causal=True, score_mod=O.score_mod_alibi_global(O.alibi_slopes(2)))
+    elif case == "documents_900":
+        Sq = Sk = 900
+        sid = O.doc_ids_from_lengths([250, 130, 400, 120])
+        okw = dict(causal=True, segment_ids=sid)
+    else:
+        B, Hq, Hkv, Sq, Sk = 2, 4, 2, 130, 130
+        mf, okw = masks.make_causal_mask_fns(128, 128), dict(causal=True)
+    q, k, v, do = O.make_inputs(B, Hq, Hkv, Sq, Sk, 128, dtype=dtype, seed=83)
+    ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, **okw)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, sm_scale=sc, **okw)
+    qg, kg, vg, dog = [x.to(DEV) for x in (q, k, v, do)]
+    causal_flag = case == "documents_900"
+    o, l, m = F._flex_attention_impl(qg, kg, vg, None, sid, True, causal_flag, sc, 1, 128, 128, 128, False, mf[1], mf[0], sfn)
+    assert o.shape == q.shape and l.shape == (B, Hq, Sq) and o.is_contiguous()
+    assert_close("o", o, ro, dtype)
+    assert_close("lse", m + l.log(), rm + rl.log(), dtype)
+    d = F.compute_delta(o, dog)
+    dq = F.flex_attention_bwd_dq(qg, kg, vg, None, sid, l, m, o, dog, d, block_b=1, block_q=128, block_k_major=128,
+                                 block_k=128, sm_scale=sc, debug=False, score_fn=sfn, mask_fn=mf[0], block_mask_fn=mf[1],
+                                 causal=causal_flag)
+    dk, dv = F.flash_attention_bwd_dkv(kg, vg, qg, None, sid, l, m, d, dog, block_b=1, block_q=128, block_q_major=128,
+                                       block_k_major=128, block_k=128, sm_scale=sc, causal=causal_flag, debug=False,
+                                       score_fn=sfn, mask_fn=mf[0], block_mask_fn=mf[1])
+    assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+    _check_grads((dq, dk, dv), (rdq, rdk, rdv), q, k, v, do, o, l, m, dtype, dict(sm_scale=sc, **okw))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+def test_distinct_unsorted_segment_ids(F, dtype):
+    """q and kv positions with ids of their own (the reference's SegmentIds with .q / .kv, jax_exp.py:37-51),
+    not sorted along the sequence, different lengths on the two sides: keep = same id (and causal)."""
+    import types
+    sc = 1 / math.sqrt(128)
+    Sq, Sk = 384, 640
+    g = torch.Generator().manual_seed(5)
+    ids_q = torch.randint(0, 3, (Sq // 32,), generator=g).repeat_interleave(32)    # runs of 32, ids recur
+    ids_k = torch.randint(0, 3, (Sk // 16,), generator=g).repeat_interleave(16)
+    ids_k[:16] = ids_q[0]                                                            # (every query keeps a key)
+    for v_ in range(3):
+        ids_k[16 * (v_ + 1): 16 * (v_ + 2)] = v_
+    keep = ids_q[:, None] == ids_k[None, :]
+    q, k, v, do = O.make_inputs(1, 2, 2, Sq, Sk, 128, dtype=dtype, seed=89)
+    okw = dict(sm_scale=sc, mask=keep)
+    ro, rl, rm = O.mha_reference(q, k, v, save_residuals=True, **okw)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, **okw)
+    sid = types.SimpleNamespace(q=ids_q, kv=ids_k)
+    qg, kg, vg, dog = [x.to(DEV) for x in (q, k, v, do)]
+    o, l, m = F._flex_attention_impl(qg, kg, vg, None, sid, True, False, sc, 1, 128, 128, 128, False, None, None, None)
+    assert_close("o", o, ro, dtype)
+    d = F.compute_delta(o, dog)
+    dq = F.flex_attention_bwd_dq(qg, kg, vg, None, sid, l, m, o, dog, d, block_b=1, block_q=128, block_k_major=128,
+                                 block_k=128, sm_scale=sc, debug=False)
+    dk, dv = F.flash_attention_bwd_dkv(kg, vg, qg, None, sid, l, m, d, dog, block_b=1, block_q=128, block_q_major=128,
+                                       block_k_major=128, block_k=128, sm_scale=sc, causal=False, debug=False)
+    _check_grads((dq, dk, dv), (rdq, rdk, rdv), q, k, v, do, o, l, m, dtype, okw)
+    # the builder's map for unsorted ids: never skips a tile with a kept element, never calls a tile full that is not
+    from flex_attention_tpu_amd import _common, block_mask
+    spec = _common.resolve_mask(None, None, False, sid, Sq, Sk)
+    bm = block_mask.build_block_map(spec, Sq, Sk, 128, 64, DEV)
+    brute = O.block_map_bruteforce(keep, 128, 64)
+    st = bm.state.cpu()
+    assert bool(((st == 0) <= (brute == 0)).all()) and bool(((st == 2) <= (brute == 2)).all())
+
+
 def test_entry_points_reject_bad_arguments_on_gpu(F):
-    q = torch.zeros(1, 2, 192, 128, dtype=torch.bfloat16, device=DEV)
-    with pytest.raises(ValueError):  # 192 is not a multiple of the 128-row q tile
-        F._flex_attention_impl(q, q, q, None, None, False, False, 1.0, 1, 64, 64, 64, False, None, None, None)
+    q = torch.zeros(1, 2, 256, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError):  # block_q must divide the sequence length
+        F._flex_attention_impl(q, q, q, None, None, False, False, 1.0, 1, 96, 64, 64, False, None, None, None)
     q = torch.zeros(1, 2, 256, 64, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(NotImplementedError):  # bf16 kernels exist for head dim 128 only
         F._flex_attention_impl(q, q, q, None, None, False, False, 1.0, 1, 128, 128, 128, False, None, None, None)

@@ -222,9 +222,18 @@ def test_host_caches_are_bounded():
     assert block_mask._map_cache.maxsize == block_mask.MAP_CACHE_SIZE
     # a segment-id tensor is turned into host ids once per tensor object and version
     ids = torch.tensor([0, 0, 1, 1, 2, 2, 2, 2], dtype=torch.int32)
-    d1 = _common.segment_doc_ids(ids)
-    assert _common.segment_doc_ids(ids) is d1
+    d1, none = _common.segment_doc_ids(ids)
+    assert none is None and _common.segment_doc_ids(ids)[0] is d1
     ids[4] = 1
-    d2 = _common.segment_doc_ids(ids)
+    d2 = _common.segment_doc_ids(ids)[0]
     assert d2 is not d1 and d2.array.tolist() == [0, 0, 1, 1, 1, 2, 2, 2]
-    assert _common.segment_doc_ids(d2) is d2
+    assert _common.segment_doc_ids(d2)[0] is d2
+    # distinct, unsorted q / kv ids (the reference's SegmentIds) come back as a pair
+    import types
+    pair = types.SimpleNamespace(q=torch.tensor([3, 1, 1, 2]), kv=torch.tensor([1, 1, 2, 3, 3, 0]))
+    dq, dk = _common.segment_doc_ids(pair)
+    assert dq.array.tolist() == [3, 1, 1, 2] and dk.array.tolist() == [1, 1, 2, 3, 3, 0]
+    # ragged lengths: padded keys get an id no query carries
+    spec = _common.resolve_mask(None, None, True, None, 200, 300, 256, 384)
+    assert spec.flags == _lib.MASK_CAUSAL | _lib.MASK_DOC
+    assert spec.doc_ids.array.tolist() == [0] * 256 and spec.doc_ids_k.array.tolist() == [0] * 300 + [1] * 84
