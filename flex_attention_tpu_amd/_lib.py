@@ -117,6 +117,7 @@ EXPORTS = (
     "flexattn_tile_shape",
     "flexattn_build_block_mask",
     "flexattn_fwd",
+    "flexattn_fwd_noalloc",
     "flexattn_bwd_delta",
     "flexattn_bwd_dq",
     "flexattn_bwd_dkv",
@@ -136,10 +137,11 @@ def _bind(lib: C.CDLL) -> C.CDLL:
         C.POINTER(MaskSpecC), C.c_int32, C.c_int32, C.c_int32, C.c_int32,
         C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
     lib.flexattn_fwd.argtypes = [C.POINTER(FwdParamsC), C.c_void_p]
+    lib.flexattn_fwd_noalloc.argtypes = [C.POINTER(FwdParamsC), C.c_void_p]
     lib.flexattn_bwd_delta.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
     lib.flexattn_bwd_dq.argtypes = [C.POINTER(BwdParamsC), C.c_void_p]
     lib.flexattn_bwd_dkv.argtypes = [C.POINTER(BwdParamsC), C.c_void_p]
-    for name in ("flexattn_tile_shape", "flexattn_build_block_mask", "flexattn_fwd", "flexattn_bwd_delta",
+    for name in ("flexattn_tile_shape", "flexattn_build_block_mask", "flexattn_fwd", "flexattn_fwd_noalloc", "flexattn_bwd_delta",
                  "flexattn_bwd_dq", "flexattn_bwd_dkv"):
         getattr(lib, name).restype = C.c_int
     return lib

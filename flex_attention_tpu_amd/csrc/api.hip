@@ -1,6 +1,7 @@
 // C ABI of libflexattn.so: argument validation and dispatch to the gfx950 kernels.
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 
 #include "fa_common.hpp"
 #include "launch.hpp"
@@ -166,6 +167,62 @@ static int to_bwd_args(const flexattn_bwd_params* p, int pass, BwdArgs* a) {
   return FLEXATTN_OK;
 }
 
+
+static int fwd_with_map(const flexattn_fwd_params* p, const flexattn_block_map& map, hipStream_t s) {
+  if (!p->q || !p->k || !p->v || !p->o) return set_error(FLEXATTN_EINVAL, "q, k, v or o is NULL");
+  if ((p->l == nullptr) != (p->m == nullptr)) return set_error(FLEXATTN_EINVAL, "l and m must both be given or both NULL");
+  int rc = check_shape(FLEXATTN_PASS_FWD, p->B, p->Hq, p->Hkv, p->Sq, p->Sk, p->D, p->dtype, map);
+  if (rc != FLEXATTN_OK) return rc;
+  if ((rc = check_scale_flags(p->sm_scale, p->flags)) != FLEXATTN_OK) return rc;
+  if ((rc = check_score(p->score)) != FLEXATTN_OK) return rc;
+  if ((rc = check_mask(p->mask)) != FLEXATTN_OK) return rc;
+  FwdArgs a;
+  a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.l = p->l; a.m = p->m;
+  a.B = p->B; a.Hq = p->Hq; a.Hkv = p->Hkv; a.Sq = p->Sq; a.Sk = p->Sk;
+  a.sm_scale = p->sm_scale;
+  a.flags = p->flags;
+  a.score = to_args(p->score);
+  a.mask = to_args(p->mask);
+  a.map = row_view(map);
+  if (p->dtype == FLEXATTN_BF16) return fwd_bf16_d128(a, s);
+  return fwd_f32(a, p->D, s);
+}
+
+// ---- resident block map of flexattn_fwd_noalloc ---------------------------------------------------------
+// The forward walks a block map (tile states, per-row counts and kv lists) that flexattn_fwd's caller
+// allocates.  flexattn_fwd_noalloc keeps one in this file-scope device array instead: every GPU the library
+// runs on holds its own copy (kScratchBytes, about 340 KB) until the process ends.  The array's name is only a
+// host-side handle; its device address is looked up once per device and kept here.
+constexpr int kScratchMaxRows = 4096;       // q tiles
+constexpr int kScratchMaxTiles = 65536;     // q tiles x kv tiles (e.g. 32768 x 32768 tokens at 128 x 128)
+constexpr size_t kScratchStateOff = 0;
+constexpr size_t kScratchCntOff = kScratchStateOff + kScratchMaxTiles;
+constexpr size_t kScratchIdxOff = kScratchCntOff + (size_t)kScratchMaxRows * 4;
+constexpr size_t kScratchBytes = kScratchIdxOff + (size_t)kScratchMaxTiles * 4;
+static_assert(kScratchCntOff % 256 == 0 && kScratchIdxOff % 256 == 0, "sub-arrays stay 256-byte aligned");
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static unsigned char* g_scratch_ptr[kMaxDevices] = {};
+
+static int scratch_of_current_device(unsigned char** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return set_error(FLEXATTN_ENOTSUP, "device ordinal %d outside [0, %d)", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      return set_error(FLEXATTN_ELAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = static_cast<unsigned char*>(ptr);
+  }
+  *out = g_scratch_ptr[dev];
+  return FLEXATTN_OK;
+}
+
 }  // namespace fa
 
 using namespace fa;
@@ -207,24 +264,43 @@ int flexattn_build_block_mask(const flexattn_mask_spec* mask, int32_t Sq, int32_
 
 int flexattn_fwd(const flexattn_fwd_params* p, void* stream) {
   if (p == nullptr) return set_error(FLEXATTN_EINVAL, "params is NULL");
-  if (!p->q || !p->k || !p->v || !p->o) return set_error(FLEXATTN_EINVAL, "q, k, v or o is NULL");
-  if ((p->l == nullptr) != (p->m == nullptr)) return set_error(FLEXATTN_EINVAL, "l and m must both be given or both NULL");
-  int rc = check_shape(FLEXATTN_PASS_FWD, p->B, p->Hq, p->Hkv, p->Sq, p->Sk, p->D, p->dtype, p->map);
+  return fwd_with_map(p, p->map, static_cast<hipStream_t>(stream));
+}
+
+int flexattn_fwd_noalloc(const flexattn_fwd_params* p, void* stream) {
+  if (p == nullptr) return set_error(FLEXATTN_EINVAL, "params is NULL");
+  if (p->B <= 0 || p->Hq <= 0 || p->Hkv <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->D <= 0)
+    return set_error(FLEXATTN_EINVAL, "non-positive dimension (B=%d Hq=%d Hkv=%d Sq=%d Sk=%d D=%d)", p->B, p->Hq, p->Hkv,
+                     p->Sq, p->Sk, p->D);
+  int bq = 0, bk = 0;
+  int rc = tile_shape(FLEXATTN_PASS_FWD, p->dtype, p->D, &bq, &bk);
   if (rc != FLEXATTN_OK) return rc;
-  if ((rc = check_scale_flags(p->sm_scale, p->flags)) != FLEXATTN_OK) return rc;
-  if ((rc = check_score(p->score)) != FLEXATTN_OK) return rc;
+  if (p->Sq % bq != 0) return set_error(FLEXATTN_EINVAL, "Sq=%d is not a multiple of the q tile %d", p->Sq, bq);
+  if (p->Sk % bk != 0) return set_error(FLEXATTN_EINVAL, "Sk=%d is not a multiple of the kv tile %d", p->Sk, bk);
+  const int nq = p->Sq / bq, nk = p->Sk / bk;
+  if (nq > kScratchMaxRows || (long long)nq * nk > kScratchMaxTiles)
+    return set_error(FLEXATTN_EINVAL,
+                     "flexattn_fwd_noalloc: %d x %d tiles exceed the resident block map (at most %d q tiles and %d tiles "
+                     "in all); build a map with flexattn_build_block_mask and call flexattn_fwd",
+                     nq, nk, kScratchMaxRows, kScratchMaxTiles);
   if ((rc = check_mask(p->mask)) != FLEXATTN_OK) return rc;
-  FwdArgs a;
-  a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.l = p->l; a.m = p->m;
-  a.B = p->B; a.Hq = p->Hq; a.Hkv = p->Hkv; a.Sq = p->Sq; a.Sk = p->Sk;
-  a.sm_scale = p->sm_scale;
-  a.flags = p->flags;
-  a.score = to_args(p->score);
-  a.mask = to_args(p->mask);
-  a.map = row_view(p->map);
+  unsigned char* base = nullptr;
+  if ((rc = scratch_of_current_device(&base)) != FLEXATTN_OK) return rc;
+  flexattn_block_map map;
+  map.state = base + kScratchStateOff;
+  map.kv_cnt = reinterpret_cast<const int32_t*>(base + kScratchCntOff);
+  map.kv_idx = reinterpret_cast<const int32_t*>(base + kScratchIdxOff);
+  map.q_cnt = nullptr;
+  map.q_idx = nullptr;
+  map.nq = nq; map.nk = nk; map.block_q = bq; map.block_k = bk;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (p->dtype == FLEXATTN_BF16) return fwd_bf16_d128(a, s);
-  return fwd_f32(a, p->D, s);
+  // every state, every count and every list entry below its count is rewritten by the builder: nothing of
+  // an earlier call is read, nothing needs clearing
+  rc = build_block_mask(to_args(p->mask), p->Sq, p->Sk, bq, bk, base + kScratchStateOff,
+                        reinterpret_cast<int*>(base + kScratchCntOff), reinterpret_cast<int*>(base + kScratchIdxOff),
+                        nullptr, nullptr, s);
+  if (rc != FLEXATTN_OK) return rc;
+  return fwd_with_map(p, map, s);
 }
 
 int flexattn_bwd_delta(const void* o, const void* dout, float* delta, int64_t rows, int32_t D, int32_t dtype,

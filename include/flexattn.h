@@ -13,7 +13,8 @@
  *  - Every function returns FLEXATTN_OK or a negative error code, never throws or aborts, and
  *    records a message readable with flexattn_last_error_string() (thread-local).
  *  - Launches are asynchronous on `stream` (a hipStream_t passed as void*; NULL = default stream).
- *  - Entry points are re-entrant and keep no mutable global state.
+ *  - Entry points are re-entrant and keep no mutable global state (flexattn_fwd_noalloc excepted: it owns one
+ *    device array per GPU, see there).
  */
 #ifndef FLEXATTN_H_
 #define FLEXATTN_H_
@@ -156,6 +157,19 @@ int flexattn_build_block_mask(const flexattn_mask_spec* mask, int32_t Sq, int32_
 
 /* Forward.  Replaces the pallas_call in _flex_attention_impl (flex_attention_kernel.py:173-187). */
 int flexattn_fwd(const flexattn_fwd_params* p, void* stream);
+
+/* Forward without any allocation.  No counterpart in the reference; for callers that cannot allocate
+ * device memory around the call: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  Same request and same results as flexattn_fwd, except that p->map is ignored: the block map of
+ * p->mask is built by the builder kernel into a device array that the library holds per GPU (about 340 KB,
+ * from library load to process end) and the forward walks it there, both launched on `stream`.  Limits:
+ * Sq / block_q <= 4096 q tiles and (Sq / block_q) * (Sk / block_k) <= 65536 tiles at the granularity of
+ * flexattn_tile_shape(FLEXATTN_PASS_FWD, ...) (e.g. 32768 x 32768 tokens); larger requests return
+ * FLEXATTN_EINVAL.  Calls no hipMalloc / hipFree; the first call on a device looks up the array's address
+ * (make that call outside graph capture).  Every call on a GPU uses that GPU's one array: calls whose
+ * execution may overlap on one GPU (different streams, graphs replayed concurrently) race and must be
+ * serialised by the caller. */
+int flexattn_fwd_noalloc(const flexattn_fwd_params* p, void* stream);
 
 /* delta_i = sum_c o_ic * do_ic in float32.  Replaces the caller-side reduction at
  * flex_attention_dq_bwd.py:932 and flash_attention_dkv_bwd.py:925.  rows = B*Hq*Sq. */
