@@ -758,12 +758,13 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
 #pragma unroll
       for (int x = 0; x < 2; ++x) {
         const float l_tot = half_sum(L[x]);
+        const float mt_row = half_max(Mt[x]);  // (the streams keep the running maximum per lane)
         inv[x] = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
         if (2 * qb2 + x < nQ && a.l != nullptr && lane_here < 32) {
           const size_t r = (size_t)bh * a.Sq + q_idx[x];
           // sums were taken against the reference maximum M: move them to the true maximum M + Mt
-          a.l[r] = (l_tot > 0.f) ? l_tot * fast_exp2(-Mt[x]) : 0.f;
-          a.m[r] = (l_tot > 0.f) ? (M[x] + Mt[x]) * kLn2 : kNegInf;  // natural units
+          a.l[r] = (l_tot > 0.f) ? l_tot * fast_exp2(-mt_row) : 0.f;
+          a.m[r] = (l_tot > 0.f) ? (M[x] + mt_row) * kLn2 : kNegInf;  // natural units
         }
       }
 #define FA_GET(T, SRC, REG)                                                                                        \

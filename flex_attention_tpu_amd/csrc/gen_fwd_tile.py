@@ -298,22 +298,30 @@ def build(masked, alibi=False):
         ops.append(valu(f"v_max3_f32 {vr(T[0])}, {vr(T[0])}, {vr(T[1])}, {vr(T[2])}", vset(T[0]), vset(T[0]) | vset(T[1]) | vset(T[2])))
         ops.append(valu(f"v_max3_f32 {vr(T[3])}, {vr(T[3])}, {vr(T[4])}, {vr(s + 15)}", vset(T[3]), vset(T[3]) | vset(T[4]) | vset(s + 15)))
         ops.append(valu(f"v_max_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[3])}", vset(T[0]), vset(T[0]) | vset(T[3])))
-        ops.append(valu(f"v_mov_b32_e32 {vr(T[1])}, {vr(T[0])}", vset(T[1]), vset(T[0])))
-
-        def swap(e):
-            e.raw("s_nop 1")
-            if "valu" not in DROP:
-                e.valu(f"v_permlane32_swap_b32 {vr(T[0])}, {vr(T[1])}", vset(T[0]) | vset(T[1]), vset(T[0]) | vset(T[1]))
-            e.raw("s_nop 1")
-        ops.append(Op(swap, cost=3))
-        ops.append(valu(f"v_max_f32_e32 {vr(T[0])}, {vr(T[0])}, {vr(T[1])}", vset(T[0]), vset(T[0]) | vset(T[1])))
+        # Mt is the running maximum of the lane's own 16 of the row's 32 scores per block (the two half-waves
+        # that share a q row meet in the block below and in the kernel's epilogue): the common path needs no
+        # exchange between lanes.
         ops.append(valu(f"v_max_f32_e32 {Mt}, {Mt}, {vr(T[0])}", kMt, kMt | vset(T[0])))
-        # does the running maximum leave [-TAU, TAU] (and is it finite: rows that kept nothing so far stay put)?
-        rare = [("valu", f"v_cmp_gt_f32_e64 vcc, |{Mt}|, {vr(V_TAU)}", set(), kMt | vset(V_TAU), False)]
-        if masked:
-            rare.append(("valu", f"v_cmp_neq_f32_e64 s[86:87], {Mt}, {vr(V_NEGINF)}", set(), kMt | vset(V_NEGINF), False))
-            rare.append(("raw", "s_and_b64 vcc, vcc, s[86:87]"))
+
+        # does a running maximum leave [-TAU, TAU] (and is it finite: lanes that kept nothing so far stay put)?
+        def leaves():
+            t = [("valu", f"v_cmp_gt_f32_e64 vcc, |{Mt}|, {vr(V_TAU)}", set(), kMt | vset(V_TAU), False)]
+            if masked:
+                t.append(("valu", f"v_cmp_neq_f32_e64 s[86:87], {Mt}, {vr(V_NEGINF)}", set(), kMt | vset(V_NEGINF), False))
+                t.append(("raw", "s_and_b64 vcc, vcc, s[86:87]"))
+            return t
+        rare = leaves()
         rare += [("raw", f"s_cbranch_vccz .Lfa_fwd_{tag}_keep{c}{q}_%="), ("skip_begin",), ("raw", "s_nop 3"),
+                 # some lane's maximum left the band: the row's maximum into both of its lanes, then the test
+                 # again, now the same for both (a lane whose half of the keys lags behind the other's gets
+                 # here once and carries the row's maximum from then on)
+                 ("valu", f"v_mov_b32_e32 {vr(T[0])}, {Mt}", vset(T[0]), kMt, False),
+                 ("valu", f"v_mov_b32_e32 {vr(T[1])}, {Mt}", vset(T[1]), kMt, False),
+                 ("raw", "s_nop 1"),
+                 ("valu", f"v_permlane32_swap_b32 {vr(T[0])}, {vr(T[1])}", vset(T[0]) | vset(T[1]), vset(T[0]) | vset(T[1]), False),
+                 ("raw", "s_nop 1"),
+                 ("valu", f"v_max_f32_e32 {Mt}, {vr(T[0])}, {vr(T[1])}", kMt, vset(T[0]) | vset(T[1]), False)]
+        rare += leaves() + [("raw", "s_nop 3"),
                  ("valu", f"v_cndmask_b32_e32 {vr(D)}, 0, {Mt}, vcc", vset(D), kMt, False),                 # the lane's shift
                  # (2^-shift, the shift held above -126: what was summed against a reference more than 2^126 too
                  # high has been flushed to zero and must stay zero, not become 0 x inf)
@@ -432,6 +440,31 @@ def build(masked, alibi=False):
     return em
 
 
+OUT_OF_LINE = True  # blocks that are skipped unless needed go behind the loop: the common path falls through
+
+
+def out_of_line(lines):
+    """Splits a stream into the common path and the skipped-unless-needed blocks.  Every `branch over the
+    block / block / label` group becomes an inverted branch into the block's copy behind the loop, which
+    jumps back: the common path then takes no branch and the loop body shrinks to what it executes."""
+    inverse = {"s_cbranch_vccz": "s_cbranch_vccnz", "s_cbranch_scc1": "s_cbranch_scc0"}
+    hot, cold = [], []
+    i = 0
+    while i < len(lines):
+        parts = lines[i].split()
+        if len(parts) == 2 and parts[0] in inverse and ("_late" in parts[1] or "_keep" in parts[1]):
+            label = parts[1]
+            j = lines.index(label + ":", i)
+            there = label.replace(".Lfa_fwd_", ".Lfa_fwd_x")
+            hot += [f"{inverse[parts[0]]} {there}", label + ":"]
+            cold += [there + ":"] + lines[i + 1:j] + [f"s_branch {label}"]
+            i = j + 1
+        else:
+            hot.append(lines[i])
+            i += 1
+    return hot, cold
+
+
 def run_loop(full, masked, alibi=False):
     """One asm statement: a run of consecutive steps [it, it_end) of one work item, all full or a
     single partial one.  At entry the step's K / V tiles are resident in LDS buffer %[buf]."""
@@ -495,6 +528,11 @@ def run_loop(full, masked, alibi=False):
     tail += [f"v_xor_b32_e32 %[t{i}], 0x10000, %[t{i}]" for i in range(8)]
     tail += [f"s_cmp_lt_u32 {S['it']}, {S['it_end']}", "s_cbranch_scc1 .Lfa_fwd_loop_%="]
     tail += [f"v_mov_b32_e32 %[{n}], {S[n]}" for n in STATE_IO]
+    if OUT_OF_LINE:
+        m_hot, m_cold = out_of_line(masked.out)
+        f_hot, f_cold = out_of_line(full.out)
+        return (top + m_hot + ["s_branch .Lfa_fwd_tail_%=", ".Lfa_fwd_full_%=:"] + f_hot + tail
+                + ["s_branch .Lfa_fwd_end_%="] + m_cold + f_cold + [".Lfa_fwd_end_%=:"])
     return top + masked.out + ["s_branch .Lfa_fwd_tail_%=", ".Lfa_fwd_full_%=:"] + full.out + tail
 
 

@@ -362,3 +362,42 @@ def test_dataflow_check_catches_an_early_overwrite():
     with pytest.raises(AssertionError):
         check_dataflow(moved, 1, 4)
 
+
+
+def test_fwd_out_of_line_blocks_are_the_inline_ones():
+    """gen_fwd_tile.out_of_line moves the skipped-unless-needed blocks behind the loop: putting every moved
+    block back where its branch is gives the stream the hazard checks above ran on, line for line, and the
+    common path that is left holds no branch that is normally taken."""
+    import gen_fwd_tile as g
+    direct = {"s_cbranch_vccnz": "s_cbranch_vccz", "s_cbranch_scc0": "s_cbranch_scc1"}
+    for masked in (False, True):
+        lines = g.build(masked).out
+        hot, cold = g.out_of_line(lines)
+        assert len(hot) + len(cold) == len(lines) + 2 * sum(1 for l in cold if l.startswith("s_branch"))
+        blocks = {}
+        cur = None
+        for l in cold:
+            if cur is None:
+                assert l.endswith(":")
+                cur = l[:-1]
+                blocks[cur] = []
+            elif l.startswith("s_branch"):
+                blocks[cur].append(l.split()[1])  # where it returns to
+                cur = None
+            else:
+                blocks[cur].append(l)
+        assert cur is None and len(blocks) == 14   # 8 blocks that move M, 6 late corrections
+        back = []
+        i = 0
+        while i < len(hot):
+            parts = hot[i].split()
+            if len(parts) == 2 and parts[1] in blocks:
+                body = blocks[parts[1]]
+                assert hot[i + 1] == body[-1] + ":", "the block returns to the instruction behind its branch"
+                back += [f"{direct[parts[0]]} {body[-1]}"] + body[:-1] + [hot[i + 1]]
+                i += 2
+            else:
+                assert not hot[i].startswith(("s_cbranch", "s_branch")), hot[i]
+                back.append(hot[i])
+                i += 1
+        assert back == lines

@@ -246,6 +246,28 @@ def test_single_key_rows(F):
     assert float(dq[:, :, 0, :].float().abs().max()) <= 2e-2
 
 
+@pytest.mark.parametrize("mask", ["none", "causal"])
+def test_growing_scores_move_the_reference_maximum(F, mask):
+    """Keys whose norm grows along the sequence and a large logit scale: the running row maximum keeps
+    rising by tens of log2 units, so the forward stream's reference maximum moves many times per row (the
+    blocks it normally skips, and the correction of the chain in flight).  Forward against the oracle."""
+    from flex_attention_tpu_amd import masks
+    B, H, S, D = 2, 4, 2048, 128
+    q, k, v, _ = O.make_inputs(B, H, H, S, S, D, dtype=torch.bfloat16, seed=41)
+    k = (k.float() * torch.linspace(0.1, 3.0, S).view(1, 1, S, 1)).to(torch.bfloat16)
+    # (sm_scale * log2(e) = 0.5 exactly: the streams fold that factor into their bf16 copy of Q, which
+    # then rounds nothing; with logits this large any other scale would test that rounding instead)
+    sc = 0.5 * math.log(2.0)
+    causal = mask == "causal"
+    mf, bf = masks.make_causal_mask_fns(128, 128) if causal else (None, None)
+    ro, rl, rm = O.mha_reference(q, k, v, save_residuals=True, sm_scale=sc, causal=causal)
+    o, l, m = _fwd(F, q.to(DEV), k.to(DEV), v.to(DEV), sc, mf, bf, None)
+    assert_close(f"o[{mask}]", o, ro, torch.bfloat16)
+    lse, rlse = m + torch.log(l), rm + torch.log(rl)
+    assert float((lse.cpu().double() - rlse.double()).abs().max()) <= 2e-2 + 2.0 ** -8 * float(rlse.abs().max())
+    assert float((m.cpu().double() - rm.double()).abs().max()) <= 2.0 ** -7 * float(rm.abs().max())
+
+
 @pytest.mark.parametrize("shape", [(1, 1, 1, 128, 128), (1, 2, 1, 384, 384), (2, 3, 3, 640, 640), (1, 4, 2, 1152, 1152),
                                    (2, 16, 16, 2048, 2048), (3, 16, 4, 2048, 2048), (8, 32, 32, 1024, 1024),
                                    (1, 2, 2, 256, 1280), (1, 2, 2, 1280, 256)], ids=lambda s: "x".join(map(str, s)))
