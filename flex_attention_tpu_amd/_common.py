@@ -95,8 +95,9 @@ def _doc_ids_of(ids) -> DocIds:
             return hit[2]
     t = torch.as_tensor(ids).detach().cpu()
     if t.ndim == 2:
+        # (rows that differ are split into one call per batch entry before they get here: per_batch_segments)
         if not bool((t == t[:1]).all()):
-            raise NotImplementedError("per-batch segment ids are not supported (every batch entry must carry the same ids)")
+            raise ValueError("segment ids differ between batch entries")
         t = t[0]
     if t.ndim != 1:
         raise ValueError("segment_ids must be a 1-D (or [B, S]) array of ids")
@@ -115,6 +116,68 @@ def segment_doc_ids(segment_ids):
         dk = dq if segment_ids.kv is segment_ids.q else _doc_ids_of(segment_ids.kv)
         return dq, (None if dk == dq else dk)
     return _doc_ids_of(segment_ids), None
+
+
+class _Segments:
+    """q / kv id arrays of one batch entry (same attributes as the reference's SegmentIds, jax_exp.py:37-51)."""
+
+    def __init__(self, q, kv):
+        self.q, self.kv = q, kv
+
+
+def per_batch_segments(segment_ids, B: int):
+    """None when one mask serves the whole batch; else a list with the ``segment_ids`` argument of every batch
+    entry.  The reference accepts ids of shape [B, S] (mha_reference.py:65-73); the kernels take one id array
+    per launch, so a batch whose entries carry different ids runs as one launch per entry."""
+    if segment_ids is None or isinstance(segment_ids, DocIds):
+        return None
+
+    def rows_of(x):
+        if isinstance(x, DocIds):
+            return None
+        t = torch.as_tensor(x)
+        if t.ndim != 2 or t.shape[0] == 1:
+            return None
+        if t.shape[0] != B:
+            raise ValueError(f"segment ids have {t.shape[0]} rows for a batch of {B}")
+        t = t.detach().cpu()
+        return None if bool((t == t[:1]).all()) else t
+
+    if hasattr(segment_ids, "q") and hasattr(segment_ids, "kv"):
+        rq, rk = rows_of(segment_ids.q), rows_of(segment_ids.kv)
+        if rq is None and rk is None:
+            return None
+        return [_Segments(rq[b] if rq is not None else segment_ids.q, rk[b] if rk is not None else segment_ids.kv)
+                for b in range(B)]
+    rows = rows_of(segment_ids)
+    return None if rows is None else [rows[b] for b in range(B)]
+
+
+def batch_entry(t, b: int):
+    """Batch entry b of a tensor argument as a batch of one (None and batch-broadcast tensors pass through)."""
+    if t is None or t.shape[0] == 1:
+        return t
+    return t[b:b + 1]
+
+
+def bias_c(ab, B: int, Hq: int, Sq: int, Sk: int, Sq_p: int, Sk_p: int, device):
+    """(BiasC, tensor to keep alive) of the additive bias ``ab``: [B or 1, Hq or 1, Sq, Sk], float32 or
+    bfloat16, added to the logits behind the score function (mha_reference.py:50-51).  Zero-padded along with
+    q and k when the lengths are ragged (padded keys are masked anyway)."""
+    if ab is None:
+        return _lib.BiasC(), None
+    if not isinstance(ab, torch.Tensor) or ab.ndim != 4:
+        raise ValueError("ab must be a 4-D tensor [B or 1, H or 1, Sq, Sk]")
+    if ab.shape[0] not in (1, B) or ab.shape[1] not in (1, Hq) or tuple(ab.shape[2:]) != (Sq, Sk):
+        raise ValueError(f"ab has shape {tuple(ab.shape)}, expected [{B} or 1, {Hq} or 1, {Sq}, {Sk}]")
+    if ab.dtype not in (torch.float32, torch.bfloat16):
+        raise NotImplementedError(f"ab dtype {ab.dtype} is not supported (float32 or bfloat16)")
+    if ab.device != device:
+        raise ValueError("ab must live on the device of q")
+    ab = pad_seq(pad_seq(ab, Sq_p, dim=2), Sk_p, dim=3).contiguous()
+    sb = 0 if ab.shape[0] == 1 else ab.stride(0)
+    sh = 0 if ab.shape[1] == 1 else ab.stride(1)
+    return _lib.BiasC(ab.data_ptr(), sb, sh, _lib.F32 if ab.dtype == torch.float32 else _lib.BF16, 0), ab
 
 
 def resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk, Sq_pad=None, Sk_pad=None) -> MaskSpec:

@@ -76,6 +76,16 @@ class BlockMapC(C.Structure):
     ]
 
 
+class BiasC(C.Structure):
+    _fields_ = [
+        ("ptr", C.c_void_p),
+        ("stride_b", C.c_int64),
+        ("stride_h", C.c_int64),
+        ("dtype", C.c_int32),
+        ("reserved", C.c_int32),
+    ]
+
+
 class FwdParamsC(C.Structure):
     _fields_ = [
         ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p),
@@ -90,6 +100,7 @@ class FwdParamsC(C.Structure):
         ("score", ScoreSpecC),
         ("mask", MaskSpecC),
         ("map", BlockMapC),
+        ("ab", BiasC),
     ]
 
 
@@ -108,6 +119,7 @@ class BwdParamsC(C.Structure):
         ("score", ScoreSpecC),
         ("mask", MaskSpecC),
         ("map", BlockMapC),
+        ("ab", BiasC),
     ]
 
 

@@ -24,7 +24,7 @@ int check_launch(const char* what) {
   return FLEXATTN_OK;
 }
 
-static ScoreArgs to_args(const flexattn_score_spec& s) {
+static ScoreArgs to_args(const flexattn_score_spec& s, const flexattn_bias& ab, int Sk) {
   ScoreArgs r;
   r.kind = s.kind;
   r.cap = s.cap;
@@ -32,7 +32,24 @@ static ScoreArgs to_args(const flexattn_score_spec& s) {
   r.mod_q = s.mod_q;
   r.mod_k = s.mod_k;
   r.slopes = s.slopes;
+  r.ab = ab.ptr;
+  r.ab_sb_rows = ab.ptr ? (int)(ab.stride_b / Sk) : 0;
+  r.ab_sh_rows = ab.ptr ? (int)(ab.stride_h / Sk) : 0;
+  r.ab_ld = Sk;
+  r.ab_f32 = ab.dtype == FLEXATTN_F32 ? 1 : 0;
   return r;
+}
+
+static int check_bias(const flexattn_bias& ab, int B, int Hq, int Sq, int Sk) {
+  if (ab.ptr == nullptr) return FLEXATTN_OK;
+  if (ab.dtype != FLEXATTN_F32 && ab.dtype != FLEXATTN_BF16) return set_error(FLEXATTN_EINVAL, "unknown bias dtype %d", ab.dtype);
+  if (ab.stride_b < 0 || ab.stride_h < 0) return set_error(FLEXATTN_EINVAL, "negative bias stride");
+  if (Sk <= 0 || ab.stride_b % Sk != 0 || ab.stride_h % Sk != 0)
+    return set_error(FLEXATTN_EINVAL, "bias strides (%lld, %lld) must be multiples of the row length Sk=%d",
+                     (long long)ab.stride_b, (long long)ab.stride_h, Sk);
+  const long long rows = (long long)(B - 1) * (ab.stride_b / Sk) + (long long)(Hq - 1) * (ab.stride_h / Sk) + Sq;
+  if (rows >= (1ll << 31)) return set_error(FLEXATTN_ENOTSUP, "bias spans %lld rows, at most 2^31 - 1 are addressed", rows);
+  return FLEXATTN_OK;
 }
 
 static MaskArgs to_args(const flexattn_mask_spec& m) {
@@ -155,13 +172,14 @@ static int to_bwd_args(const flexattn_bwd_params* p, int pass, BwdArgs* a) {
   if ((rc = check_scale_flags(p->sm_scale, p->flags)) != FLEXATTN_OK) return rc;
   if ((rc = check_score(p->score)) != FLEXATTN_OK) return rc;
   if ((rc = check_mask(p->mask)) != FLEXATTN_OK) return rc;
+  if ((rc = check_bias(p->ab, p->B, p->Hq, p->Sq, p->Sk)) != FLEXATTN_OK) return rc;
   a->q = p->q; a->k = p->k; a->v = p->v; a->dout = p->dout;
   a->l = p->l; a->m = p->m; a->delta = p->delta;
   a->dq = p->dq; a->dk = p->dk; a->dv = p->dv;
   a->B = p->B; a->Hq = p->Hq; a->Hkv = p->Hkv; a->Sq = p->Sq; a->Sk = p->Sk;
   a->sm_scale = p->sm_scale;
   a->flags = p->flags;
-  a->score = to_args(p->score);
+  a->score = to_args(p->score, p->ab, p->Sk);
   a->mask = to_args(p->mask);
   a->map = (pass == FLEXATTN_PASS_DKV) ? col_view(p->map) : row_view(p->map);
   return FLEXATTN_OK;
@@ -176,12 +194,13 @@ static int fwd_with_map(const flexattn_fwd_params* p, const flexattn_block_map& 
   if ((rc = check_scale_flags(p->sm_scale, p->flags)) != FLEXATTN_OK) return rc;
   if ((rc = check_score(p->score)) != FLEXATTN_OK) return rc;
   if ((rc = check_mask(p->mask)) != FLEXATTN_OK) return rc;
+  if ((rc = check_bias(p->ab, p->B, p->Hq, p->Sq, p->Sk)) != FLEXATTN_OK) return rc;
   FwdArgs a;
   a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.l = p->l; a.m = p->m;
   a.B = p->B; a.Hq = p->Hq; a.Hkv = p->Hkv; a.Sq = p->Sq; a.Sk = p->Sk;
   a.sm_scale = p->sm_scale;
   a.flags = p->flags;
-  a.score = to_args(p->score);
+  a.score = to_args(p->score, p->ab, p->Sk);
   a.mask = to_args(p->mask);
   a.map = row_view(map);
   if (p->dtype == FLEXATTN_BF16) return fwd_bf16_d128(a, s);

@@ -126,7 +126,7 @@ __global__ __launch_bounds__(256) void fwd_f32_kernel(FwdArgs a) {
       for (int jj = 0; jj < CH; ++jj) {
         const int j = kb * BK + j0 + jj;
         float s = quad_sum(dot_slice<NV>(qv, sK + (j0 + jj) * D, sub));
-        float x = sm.to_log2(s, q_idx, j);
+        float x = sm.to_log2(s, q_idx, j) + sm.bias2(q_idx, j);
         if (partial) {
           const int doc_j = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_k[j] : 0;
           if (!keep_elem(a.mask, q_idx, j, doc_i, doc_j)) x = kNegInf;
@@ -209,13 +209,14 @@ __global__ __launch_bounds__(256) void bwd_dq_f32_kernel(BwdArgs a) {
       const int j = kb * BK + jj;
       const float s = quad_sum(dot_slice<NV>(qv, sK + jj * D, sub));
       const float dp = quad_sum(dot_slice<NV>(dov, sV + jj * D, sub));
-      float x = sm.to_log2(s, q_idx, j);
+      const float tv = sm.to_log2(s, q_idx, j);  // (the score function's value: what its derivative is taken from)
+      float x = tv + sm.bias2(q_idx, j);
       if (partial) {
         const int doc_j = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_k[j] : 0;
         if (!keep_elem(a.mask, q_idx, j, doc_i, doc_j)) x = kNegInf;
       }
       const float p = exp2f(x - lse2);
-      const float ds = (x == kNegInf) ? 0.f : p * (dp - dl) * sm.dfactor(x, s, q_idx, j);
+      const float ds = (x == kNegInf) ? 0.f : p * (dp - dl) * sm.dfactor(tv, s, q_idx, j);
       axpy_slice<NV>(acc, ds, sK + jj * D, sub);
     }
   }
@@ -287,13 +288,14 @@ __global__ __launch_bounds__(256) void bwd_dkv_f32_kernel(BwdArgs a) {
         const int i = qb * BQ + ii;
         const float s = quad_sum(dot_slice<NV>(kv, sQ + ii * D, sub));
         const float dp = quad_sum(dot_slice<NV>(vv, sDO + ii * D, sub));
-        float x = sm.to_log2(s, i, k_idx);
+        const float tv = sm.to_log2(s, i, k_idx);
+        float x = tv + sm.bias2(i, k_idx);
         if (partial) {
           const int doc_i = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[i] : 0;
           if (!keep_elem(a.mask, i, k_idx, doc_i, doc_j)) x = kNegInf;
         }
         const float p = exp2f(x - sLse[ii]);
-        const float ds = (x == kNegInf) ? 0.f : p * (dp - sDl[ii]) * sm.dfactor(x, s, i, k_idx);
+        const float ds = (x == kNegInf) ? 0.f : p * (dp - sDl[ii]) * sm.dfactor(tv, s, i, k_idx);
         axpy_slice<NV>(dv_t, p, sDO + ii * D, sub);
         axpy_slice<NV>(dk_t, ds, sQ + ii * D, sub);
       }

@@ -249,7 +249,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
             const int e = 4 * g4 + u;
             const int i = q0 + r0 + u;
             const float tv = sm.to_log2(s_acc[e], i, k_idx);
-            float pe = fast_exp2(tv - lse4[u]);
+            float pe = fast_exp2(tv + sm.bias2(i, k_idx) - lse4[u]);
             float gd = pe * (dp_acc[e] - dl4[u]) * sm.dfactor(tv, s_acc[e], i, k_idx);
             if (MASKED) {
               const bool keep = keep_elem(a.mask, i, k_idx, di[u], doc_j);
@@ -785,7 +785,8 @@ int bwd_dkv_bf16_d128(const BwdArgs& a, hipStream_t stream) {
   return set_error(FLEXATTN_ENOTSUP, "this functor library holds the plain and the compiled score function only (kind %d asked)", a.score.kind);
 #else
   // (the generated-stream kernel caches the q tile list in LDS)
-  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nq <= dkv_cfg::MAX_LIST;
+  // (and has no additive bias)
+  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nq <= dkv_cfg::MAX_LIST && a.score.ab == nullptr;
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
       return stream_ok ? launch_dkv_plain<FLEXATTN_SCORE_NONE>(a, stream) : launch_dkv<FLEXATTN_SCORE_NONE>(a, stream);

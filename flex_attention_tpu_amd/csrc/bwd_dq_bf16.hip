@@ -217,7 +217,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
           for (int u = 0; u < 4; ++u) {
             const int e = 4 * g + u;
             const float tv = sm.to_log2(s_acc[e], q_idx, j0 + u);
-            const float pe = fast_exp2(tv - lse2);
+            const float pe = fast_exp2(tv + sm.bias2(q_idx, j0 + u) - lse2);
             float gd = pe * (dp_acc[e] - delta) * sm.dfactor(tv, s_acc[e], q_idx, j0 + u);
             if (MASKED) gd = keep_elem(a.mask, q_idx, j0 + u, doc_i, dj[u]) ? gd : 0.f;
             dsv[u] = gd;
@@ -686,7 +686,8 @@ int bwd_dq_bf16_d128(const BwdArgs& a, hipStream_t stream) {
   return set_error(FLEXATTN_ENOTSUP, "this functor library holds the plain and the compiled score function only (kind %d asked)", a.score.kind);
 #else
   // (the generated-stream kernel caches the kv list in LDS)
-  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= dq_cfg::MAX_LIST;
+  // (and has no additive bias)
+  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= dq_cfg::MAX_LIST && a.score.ab == nullptr;
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
       return stream_ok ? launch_dq_plain<false>(a, stream) : launch_dq<FLEXATTN_SCORE_NONE>(a, stream);

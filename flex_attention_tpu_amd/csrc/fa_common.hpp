@@ -44,6 +44,13 @@ struct ScoreArgs {
   float slope;
   int mod_q, mod_k;
   const float* slopes;
+  // additive bias on the modified logits (the reference's `ab`): element (b, h, i, j) at
+  // ab + ((b ab_sb_rows + h ab_sh_rows + i) ab_ld + j) elements, float32 or bf16; NULL = none
+  // (strides in rows of ab_ld elements, so that the (batch, head) offset stays in 32-bit scalar arithmetic)
+  const void* ab;
+  int ab_sb_rows, ab_sh_rows;
+  int ab_ld;
+  int ab_f32;
 };
 struct MaskArgs {
   int flags;
@@ -287,6 +294,11 @@ __device__ __forceinline__ unsigned keep_bits32_staged(const MaskArgs& mk, int f
 // log2(e) so that probabilities are exp2(t - lse2).  dfactor() returns d(s')/d(raw) given the
 // already transformed logit t (log2 domain).
 // ------------------------------------------------------------------------------------------
+// Internal kind: no score function, but an additive bias.  (The forward with a compiled loop keeps its
+// running maximum on the raw dot products when there is no score function at all; with a bias it must
+// take the log2-domain route of the score functions.)
+constexpr int kScoreBiasOnly = 100;
+
 template <int KIND>
 struct ScoreMod {
   float c2;      // sm_scale * log2e
@@ -294,6 +306,9 @@ struct ScoreMod {
   float a0, a1;  // kind-specific
   int mod_q, mod_k;
   int bb, hh_;   // batch and head (custom functors)
+  const char* ab_base;  // the additive bias, or NULL
+  int ab_row0;          // first row of the (batch, head) plane
+  int ab_ld, ab_f32;
 
   __device__ __forceinline__ void init(const ScoreArgs& s, float sm_scale, int head, int batch = 0) {
     bb = batch;
@@ -302,6 +317,10 @@ struct ScoreMod {
     c2 = sm_scale * kLog2e;
     mod_q = s.mod_q;
     mod_k = s.mod_k;
+    ab_ld = s.ab_ld;
+    ab_f32 = s.ab_f32;
+    ab_base = static_cast<const char*>(s.ab);
+    ab_row0 = batch * s.ab_sb_rows + head * s.ab_sh_rows;
     if (KIND == FLEXATTN_SCORE_ALIBI) {
       a0 = s.slopes[head] * kLog2e;
     } else if (KIND == FLEXATTN_SCORE_ALIBI_TILE) {
@@ -313,7 +332,7 @@ struct ScoreMod {
   }
 
   __device__ __forceinline__ float to_log2(float raw, int i, int j) const {
-    if (KIND == FLEXATTN_SCORE_NONE) {
+    if (KIND == FLEXATTN_SCORE_NONE || KIND == kScoreBiasOnly) {
       return raw * c2;
     } else if (KIND == FLEXATTN_SCORE_ALIBI) {
       return __builtin_fmaf(raw, c2, a0 * (float)(j - i));
@@ -329,6 +348,18 @@ struct ScoreMod {
       float r = fast_rcp(1.0f + e);
       return __builtin_fmaf(-2.0f * a1, r, a1);
     }
+  }
+
+  // The additive bias of element (i, j) in the log2 domain (0 without one).  It is added to to_log2()'s
+  // result by the kernels, which keep the sum apart from the value they hand to dfactor(): the bias does not
+  // depend on the dot product (mha_reference.py:50-51 adds it behind the score function).
+  __device__ __forceinline__ bool has_bias() const { return ab_base != nullptr; }
+  __device__ __forceinline__ float bias2(int i, int j) const {
+    if (ab_base == nullptr) return 0.f;
+    const unsigned long long at = (unsigned long long)(unsigned)(ab_row0 + i) * (unsigned)ab_ld + (unsigned)j;
+    const float v = ab_f32 ? reinterpret_cast<const float*>(ab_base)[at]
+                           : __builtin_bit_cast(float, (unsigned)reinterpret_cast<const unsigned short*>(ab_base)[at] << 16);
+    return v * kLog2e;
   }
 
   // d(s')/d(raw) in natural units, from the log2-domain modified logit t.

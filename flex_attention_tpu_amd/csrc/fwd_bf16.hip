@@ -228,7 +228,10 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
       for (int c = 0; c < 2; ++c) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          if (!kPlain) s_acc[c][e] = sm.to_log2(s_acc[c][e], q_idx, kv0 + 32 * c + acc_row(e, hh));
+          if (!kPlain) {
+            const int j = kv0 + 32 * c + acc_row(e, hh);
+            s_acc[c][e] = sm.to_log2(s_acc[c][e], q_idx, j) + sm.bias2(q_idx, j);
+          }
           m_tile = fmaxf(m_tile, s_acc[c][e]);
         }
       }
@@ -248,7 +251,7 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
             const int e = 4 * g + u;
-            float tv = kPlain ? s_acc[c][e] : sm.to_log2(s_acc[c][e], q_idx, j0 + u);
+            float tv = kPlain ? s_acc[c][e] : sm.to_log2(s_acc[c][e], q_idx, j0 + u) + sm.bias2(q_idx, j0 + u);
             tv = keep_elem(a.mask, q_idx, j0 + u, doc_i, dj[u]) ? tv : kNegInf;
             s_acc[c][e] = tv;
             m_tile = fmaxf(m_tile, tv);
@@ -836,16 +839,19 @@ int fwd_bf16_d128(const FwdArgs& a, hipStream_t stream) {
 #ifdef FLEXATTN_CUSTOM_ONLY
   // functor library of a compiled score function: the kernels with a compiled main loop only
   switch (a.score.kind) {
-    case FLEXATTN_SCORE_NONE: return launch_fwd<FLEXATTN_SCORE_NONE>(a, stream);
+    case FLEXATTN_SCORE_NONE:
+      return a.score.ab ? launch_fwd<kScoreBiasOnly>(a, stream) : launch_fwd<FLEXATTN_SCORE_NONE>(a, stream);
     case FLEXATTN_SCORE_CUSTOM: return launch_fwd<FLEXATTN_SCORE_CUSTOM>(a, stream);
   }
   return set_error(FLEXATTN_ENOTSUP, "this functor library holds the plain and the compiled score function only (kind %d asked)", a.score.kind);
 #else
   // The generated-stream kernel (one wave per SIMD, 64 q rows per wave) keeps the state rows and the
   // merged kv list in LDS, hence the bound on the list length.
-  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= fwd_cfg::MAX_LIST;
+  // and has no additive bias.
+  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= fwd_cfg::MAX_LIST && a.score.ab == nullptr;
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
+      if (a.score.ab != nullptr) return launch_fwd<kScoreBiasOnly>(a, stream);
       return stream_ok ? launch_fwd_plain<false>(a, stream) : launch_fwd<FLEXATTN_SCORE_NONE>(a, stream);
     case FLEXATTN_SCORE_ALIBI:
       return stream_ok ? launch_fwd_plain<true>(a, stream) : launch_fwd<FLEXATTN_SCORE_ALIBI>(a, stream);

@@ -61,7 +61,8 @@ struct TileLoader {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(goff[i]), "s"(g_tile), "s"(dst)
-                 : "memory", "m0");
+                 : "memory", "m0", "vcc");  // (vcc: else the allocator may hand it out for the address pair,
+                                            // which the instruction cannot take as its scalar base)
   }
 };
 

@@ -25,9 +25,9 @@ class _FlexAttention(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, opts):
-        score_fn, mask_fn, block_mask_fn, segment_ids, causal, sm_scale, block_q, block_k = opts
+        score_fn, mask_fn, block_mask_fn, segment_ids, causal, sm_scale, block_q, block_k, ab = opts
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        o, l, m = _flex_attention_impl(q, k, v, None, segment_ids, True, causal, sm_scale, 1, block_q, block_k, block_k,
+        o, l, m = _flex_attention_impl(q, k, v, ab, segment_ids, True, causal, sm_scale, 1, block_q, block_k, block_k,
                                        False, block_mask_fn, mask_fn, score_fn)
         ctx.save_for_backward(q, k, v, o, l, m)
         ctx.opts = opts
@@ -36,17 +36,17 @@ class _FlexAttention(torch.autograd.Function):
     @staticmethod
     def backward(ctx, do):
         q, k, v, o, l, m = ctx.saved_tensors
-        score_fn, mask_fn, block_mask_fn, segment_ids, causal, sm_scale, block_q, block_k = ctx.opts
+        score_fn, mask_fn, block_mask_fn, segment_ids, causal, sm_scale, block_q, block_k, ab = ctx.opts
         do = do.contiguous()
         di = compute_delta(o, do)  # float32 [B, H, Sq]  (jax_exp.py:276-278)
         dq = dk = dv = None
         if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
-            dk, dv = flash_attention_bwd_dkv(k, v, q, None, segment_ids, l, m, di, do, block_b=1, block_q=block_q,
+            dk, dv = flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, block_b=1, block_q=block_q,
                                              block_q_major=block_q, block_k_major=block_k, block_k=block_k,
                                              sm_scale=sm_scale, causal=causal, debug=False, score_fn=score_fn,
                                              mask_fn=mask_fn, block_mask_fn=block_mask_fn)
         if ctx.needs_input_grad[0]:
-            dq = flex_attention_bwd_dq(q, k, v, None, segment_ids, l, m, o, do, di, block_b=1, block_q=block_q,
+            dq = flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, di, block_b=1, block_q=block_q,
                                        block_k_major=block_k, block_k=block_k, sm_scale=sm_scale, debug=False,
                                        score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn, causal=causal)
         return dq, dk, dv, None
@@ -54,18 +54,22 @@ class _FlexAttention(torch.autograd.Function):
 
 def flex_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, score_fn: Optional[Callable] = None,
                    mask_fns: Optional[Tuple[Callable, Callable]] = None, *, segment_ids=None, causal: bool = False,
-                   sm_scale: Optional[float] = None, block_q: int = 128, block_k: int = 128) -> torch.Tensor:
+                   sm_scale: Optional[float] = None, block_q: int = 128, block_k: int = 128,
+                   ab: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Differentiable flex attention on ``[B, H, S, D]`` GPU tensors (k, v may have fewer heads: GQA).
 
     ``score_fn``   closure from ``scores`` (or ``util.make_jax_score_fn``), or None
     ``mask_fns``   ``(mask_fn, block_mask_fn)`` pair from ``masks``, or None
     ``segment_ids`` / ``causal``   as in the three entry points (ANDed with ``mask_fns``)
     ``sm_scale``   default 1 / sqrt(D)
+    ``ab``         additive bias on the logits, [B or 1, H or 1, Sq, Sk]; it receives no gradient (the reference's
+                   flex backward kernels produce none: flex_attention_dq_bwd.py:109-110 keeps `dab = ds` commented out)
     Gradients flow to q, k and v (``torch.autograd.grad`` / ``.backward()``); higher-order
     differentiation is not supported, as in the reference (jax_exp.py:243-244).
     """
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(q.shape[-1])
     mask_fn, block_mask_fn = mask_fns if mask_fns is not None else (None, None)
-    opts = (score_fn, mask_fn, block_mask_fn, segment_ids, bool(causal), float(sm_scale), int(block_q), int(block_k))
+    opts = (score_fn, mask_fn, block_mask_fn, segment_ids, bool(causal), float(sm_scale), int(block_q), int(block_k),
+            ab.detach() if ab is not None else None)
     return _FlexAttention.apply(q, k, v, opts)

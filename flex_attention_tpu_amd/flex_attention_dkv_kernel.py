@@ -8,8 +8,8 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (check_blocks, check_qkv, check_rows, kernel_block_map, library_for, pad_seq, padded_len,
-                      resolve_mask, stream_of)
+from ._common import (batch_entry, bias_c, check_blocks, check_qkv, check_rows, kernel_block_map, library_for, pad_seq,
+                      padded_len, per_batch_segments, resolve_mask, stream_of)
 from .flex_attention_dq_bwd import bwd_params
 
 
@@ -21,9 +21,15 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     of all query heads of a group are summed inside the kernel.  ``causal`` is honoured
     (the reference's north-star file ignores it; its mask-aware twin gets the same effect from
     ``mask_fn``)."""
-    if ab is not None:
-        raise NotImplementedError("additive bias `ab` is not supported")
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v, do)
+    rows = per_batch_segments(segment_ids, B)
+    if rows is not None:  # ids differ between batch entries: one launch per entry
+        outs = [flash_attention_bwd_dkv(
+            k[b:b + 1], v[b:b + 1], q[b:b + 1], batch_entry(ab, b), rows[b], l[b:b + 1], m[b:b + 1], di[b:b + 1], do[b:b + 1],
+            block_b=block_b, block_q=block_q, block_q_major=block_q_major, block_k_major=block_k_major, block_k=block_k,
+            sm_scale=sm_scale, causal=causal, debug=debug, score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn,
+            compiled_loop=compiled_loop) for b in range(B)]
+        return torch.cat([x[0] for x in outs], 0), torch.cat([x[1] for x in outs], 0)
     for name, t in (("l", l), ("m", m), ("di", di)):
         check_rows(name, t, B, Hq, Sq, q.device)
     check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k,
@@ -36,8 +42,9 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     bm = kernel_block_map(_lib.PASS_DKV, spec, q, Sq_p, Sk_p, D, score_fn)
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)
+    ab_c, ab_keep = bias_c(ab, B, Hq, Sq, Sk, Sq_p, Sk_p, q.device)
     p = bwd_params(q, k, v, l, m, do, di, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dk=dk, dv=dv,
-                   compiled_loop=compiled_loop)
+                   compiled_loop=compiled_loop, ab_c=ab_c)
     with torch.cuda.device(q.device):
         lib = library_for(score_fn, spec)
         _lib.check(lib.flexattn_bwd_dkv(C.byref(p), stream_of(q)), lib)

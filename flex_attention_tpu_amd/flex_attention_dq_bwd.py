@@ -7,8 +7,8 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (check_blocks, check_qkv, check_rows, dtype_code, kernel_block_map, library_for, pad_seq,
-                      padded_len, resolve_mask, score_spec_c, stream_of)
+from ._common import (batch_entry, bias_c, check_blocks, check_qkv, check_rows, dtype_code, kernel_block_map, library_for,
+                      pad_seq, padded_len, per_batch_segments, resolve_mask, score_spec_c, stream_of)
 from .block_mask import mask_spec_c
 
 
@@ -28,7 +28,7 @@ def compute_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
 
 
 def bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, mod_q, mod_k, dq=None, dk=None, dv=None,
-               compiled_loop=False):
+               compiled_loop=False, ab_c=None):
     B, Hq, Sq, D = q.shape
     _, Hkv, Sk, _ = k.shape
     return _lib.BwdParamsC(
@@ -36,7 +36,8 @@ def bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, mod_q, mod_k,
         dq.data_ptr() if dq is not None else None,
         dk.data_ptr() if dk is not None else None, dv.data_ptr() if dv is not None else None,
         B, Hq, Hkv, Sq, Sk, D, dtype_code(q), float(sm_scale), _lib.FLAG_COMPILED_LOOP if compiled_loop else 0, 0,
-        score_spec_c(score_fn, Hq, q.device, mod_q, mod_k, sm_scale), mask_spec_c(spec, Sq, Sk, q.device), bm.as_c())
+        score_spec_c(score_fn, Hq, q.device, mod_q, mod_k, sm_scale), mask_spec_c(spec, Sq, Sk, q.device), bm.as_c(),
+        ab_c if ab_c is not None else _lib.BiasC())
 
 
 def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, block_q, block_k_major,
@@ -45,9 +46,14 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     """dq = sum_j dS_ij * d(score)/dq, with P_ij = exp(S_ij - m_i) / l_i recomputed from the saved
     statistics, dP = do v^T, dS = P (dP - d) (flex_attention_dq_bwd.py:340-378).  ``o`` is only
     shape-checked, as in the reference (:163); ``d`` is the caller's delta (see compute_delta)."""
-    if ab is not None:
-        raise NotImplementedError("additive bias `ab` is not supported")
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v, do)
+    rows = per_batch_segments(segment_ids, B)
+    if rows is not None:  # ids differ between batch entries: one launch per entry
+        return torch.cat([flex_attention_bwd_dq(
+            q[b:b + 1], k[b:b + 1], v[b:b + 1], batch_entry(ab, b), rows[b], l[b:b + 1], m[b:b + 1], batch_entry(o, b),
+            do[b:b + 1], d[b:b + 1], block_b=block_b, block_q=block_q, block_k_major=block_k_major, block_k=block_k,
+            sm_scale=sm_scale, debug=debug, score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn, causal=causal,
+            compiled_loop=compiled_loop) for b in range(B)], 0)
     if o is not None and tuple(o.shape) != tuple(q.shape):
         raise ValueError(f"o has shape {tuple(o.shape)}, expected {tuple(q.shape)}")
     for name, t in (("l", l), ("m", m), ("d", d)):
@@ -60,8 +66,9 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     l, m, d = pad_seq(l, Sq_p), pad_seq(m, Sq_p), pad_seq(d, Sq_p)
     bm = kernel_block_map(_lib.PASS_DQ, spec, q, Sq_p, Sk_p, D, score_fn)
     dq = torch.empty_like(q)
+    ab_c, ab_keep = bias_c(ab, B, Hq, Sq, Sk, Sq_p, Sk_p, q.device)
     p = bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dq=dq,
-                   compiled_loop=compiled_loop)
+                   compiled_loop=compiled_loop, ab_c=ab_c)
     with torch.cuda.device(q.device):
         lib = library_for(score_fn, spec)
         _lib.check(lib.flexattn_bwd_dq(C.byref(p), stream_of(q)), lib)

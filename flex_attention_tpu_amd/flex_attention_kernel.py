@@ -12,8 +12,8 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (check_blocks, check_qkv, dtype_code, kernel_block_map, library_for, pad_seq, padded_len,
-                      resolve_mask, score_spec_c, stream_of)
+from ._common import (batch_entry, bias_c, check_blocks, check_qkv, dtype_code, kernel_block_map, library_for, pad_seq,
+                      padded_len, per_batch_segments, resolve_mask, score_spec_c, stream_of)
 from .block_mask import mask_spec_c
 
 
@@ -21,23 +21,30 @@ def _flex_attention_impl(q, k, v, ab, segment_ids, save_residuals, causal, sm_sc
                          block_k_major, block_k, debug, block_mask_fn, mask_fn, score_fn, *, compiled_loop=False):
     """Returns ``o`` (q.dtype) or ``(o, l, m)`` with float32 ``l, m`` of shape [B, H, Sq].
 
-    Semantics (flex_attention_kernel.py:248-319): S = score_mod(sm_scale * q k^T); masked
+    Semantics (flex_attention_kernel.py:248-319): S = score_mod(sm_scale * q k^T) + ab; masked
     positions are excluded; m = rowmax S, l = sum exp(S - m), o = exp(S - m) v / l.
     Unlike the reference's flex forward, ``causal=True`` is honoured (ANDed with ``mask_fn``), as
     flash_attention_fwd_ref.py:78-86 and the dense reference do.  ``compiled_loop=True`` (not in the
     reference) selects the bf16 kernel with a compiled main loop instead of the generated instruction
     stream, for comparisons.
     """
-    if ab is not None:
-        raise NotImplementedError("additive bias `ab` is not supported")
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v)
     check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k)
+    rows = per_batch_segments(segment_ids, B)
+    if rows is not None:  # ids differ between batch entries: one launch per entry
+        outs = [_flex_attention_impl(q[b:b + 1], k[b:b + 1], v[b:b + 1], batch_entry(ab, b), rows[b], save_residuals, causal,
+                                     sm_scale, block_b, block_q, block_k_major, block_k, debug, block_mask_fn, mask_fn,
+                                     score_fn, compiled_loop=compiled_loop) for b in range(B)]
+        if not save_residuals:
+            return torch.cat(outs, 0)
+        return tuple(torch.cat([o[i] for o in outs], 0) for i in range(3))
     # ragged lengths: the tensors are zero-padded to the kernels' tiles, a key bound drops the padded keys
     # and the padded query rows are cut off again
     Sq_p, Sk_p = padded_len(Sq), padded_len(Sk)
     spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk, Sq_p, Sk_p)
     q, k, v = pad_seq(q, Sq_p), pad_seq(k, Sk_p), pad_seq(v, Sk_p)
     bm = kernel_block_map(_lib.PASS_FWD, spec, q, Sq_p, Sk_p, D, score_fn)
+    ab_c, ab_keep = bias_c(ab, B, Hq, Sq, Sk, Sq_p, Sk_p, q.device)
     o = torch.empty_like(q)
     l = m = None
     if save_residuals:
@@ -48,7 +55,7 @@ def _flex_attention_impl(q, k, v, ab, segment_ids, save_residuals, causal, sm_sc
         l.data_ptr() if l is not None else None, m.data_ptr() if m is not None else None,
         B, Hq, Hkv, Sq_p, Sk_p, D, dtype_code(q), float(sm_scale), _lib.FLAG_COMPILED_LOOP if compiled_loop else 0, 0,
         score_spec_c(score_fn, Hq, q.device, block_q or 1, block_k or 1, sm_scale),
-        mask_spec_c(spec, Sq_p, Sk_p, q.device), bm.as_c())
+        mask_spec_c(spec, Sq_p, Sk_p, q.device), bm.as_c(), ab_c)
     with torch.cuda.device(q.device):
         lib = library_for(score_fn, spec)
         _lib.check(lib.flexattn_fwd(C.byref(p), stream_of(q)), lib)

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FLEXATTN_VERSION 100 /* major*10000 + minor*100 + patch */
+#define FLEXATTN_VERSION 101 /* major*10000 + minor*100 + patch */
 
 /* status codes */
 #define FLEXATTN_OK 0
@@ -89,6 +89,18 @@ typedef struct flexattn_block_map {
   int32_t nq, nk, block_q, block_k;
 } flexattn_block_map;
 
+/* Additive bias on the logits, the reference's `ab` argument (flex_attention_kernel.py:262-266,
+ * flash_attention_dkv_bwd.py:261-263, mha_reference.py:50-51): logits = score_mod(sm_scale <q, k>) + ab,
+ * then the mask.  Element (b, h, i, j) lies at ptr + b stride_b + h stride_h + i Sk + j (in elements;
+ * a stride of 0 broadcasts over that dimension; strides must be multiples of Sk).  ptr NULL = no bias.  Calls with a bias run the kernels
+ * with a compiled main loop.  No gradient of the bias is produced (the reference computes none either). */
+typedef struct flexattn_bias {
+  const void* ptr;
+  int64_t stride_b, stride_h;
+  int32_t dtype; /* FLEXATTN_F32 or FLEXATTN_BF16 */
+  int32_t reserved;
+} flexattn_bias;
+
 /* Call flags.  The bf16 kernels exist twice: with a generated, hand-scheduled instruction stream as
  * main loop (the default wherever one exists for the request) and with a compiled loop (every
  * score kind and list length).  Both meet the stated tolerances; the flag selects the compiled one
@@ -107,6 +119,7 @@ typedef struct flexattn_fwd_params {
   flexattn_score_spec score;
   flexattn_mask_spec mask;
   flexattn_block_map map; /* granularity must equal flexattn_tile_shape(FLEXATTN_PASS_FWD, ...) */
+  flexattn_bias ab;
 } flexattn_fwd_params;
 
 typedef struct flexattn_bwd_params {
@@ -122,6 +135,7 @@ typedef struct flexattn_bwd_params {
   flexattn_score_spec score;
   flexattn_mask_spec mask;
   flexattn_block_map map; /* granularity of the pass being launched */
+  flexattn_bias ab;
 } flexattn_bwd_params;
 
 #define FLEXATTN_PASS_FWD 0

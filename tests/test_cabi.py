@@ -35,8 +35,9 @@ def test_struct_sizes_follow_c_layout():
     assert C.sizeof(_lib.ScoreSpecC) == 32
     assert C.sizeof(_lib.MaskSpecC) == 32
     assert C.sizeof(_lib.BlockMapC) == 56
-    assert C.sizeof(_lib.FwdParamsC) == 6 * 8 + 10 * 4 + 32 + 32 + 56
-    assert C.sizeof(_lib.BwdParamsC) == 10 * 8 + 10 * 4 + 32 + 32 + 56
+    assert C.sizeof(_lib.BiasC) == 32
+    assert C.sizeof(_lib.FwdParamsC) == 6 * 8 + 10 * 4 + 32 + 32 + 56 + 32
+    assert C.sizeof(_lib.BwdParamsC) == 10 * 8 + 10 * 4 + 32 + 32 + 56 + 32
 
 
 def test_tile_shapes(lib):

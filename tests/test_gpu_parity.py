@@ -187,6 +187,80 @@ def test_causal_flag_and_segment_ids_arguments(F):
     assert torch.equal(o2, o)
 
 
+def _all_passes_with(F, q, k, v, do, ab, sid, sc, mask_pair, score_fn, causal):
+    mf, bf = mask_pair if mask_pair else (None, None)
+    o, l, m = F._flex_attention_impl(q, k, v, ab, sid, True, causal, sc, 1, 128, 128, 128, False, bf, mf, score_fn)
+    d = F.compute_delta(o, do)
+    dq = F.flex_attention_bwd_dq(q, k, v, ab, sid, l, m, o, do, d, block_b=1, block_q=128, block_k_major=128,
+                                 block_k=128, sm_scale=sc, debug=False, score_fn=score_fn, mask_fn=mf, block_mask_fn=bf,
+                                 causal=causal)
+    dk, dv = F.flash_attention_bwd_dkv(k, v, q, ab, sid, l, m, d, do, block_b=1, block_q=128, block_q_major=128,
+                                       block_k_major=128, block_k=128, sm_scale=sc, causal=causal, debug=False,
+                                       score_fn=score_fn, mask_fn=mf, block_mask_fn=bf)
+    return o, l, m, dq, dk, dv
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+@pytest.mark.parametrize("case", ["plain", "softcap_causal_gqa", "ragged_bf16_bias"])
+def test_additive_bias(F, case, dtype):
+    """`ab` is added to the logits behind the score function and in front of the mask (mha_reference.py:50-51,
+    flex_attention_kernel.py:262-266, flash_attention_dkv_bwd.py:261-263) in all three passes: full [B, H, Sq, Sk],
+    broadcast over heads and batch, bfloat16 bias, ragged lengths."""
+    from flex_attention_tpu_amd import masks, scores
+    sc = 1 / math.sqrt(128)
+    g = torch.Generator().manual_seed(3)
+    if case == "plain":
+        B, Hq, Hkv, Sq, Sk = 2, 2, 2, 256, 384
+        ab = torch.randn(B, Hq, Sq, Sk, generator=g) * 2
+        mask_pair, score_fn, okw, causal = None, None, {}, False
+    elif case == "softcap_causal_gqa":
+        B, Hq, Hkv, Sq, Sk = 2, 4, 2, 512, 512
+        ab = torch.randn(B, 1, Sq, Sk, generator=g)            # one plane per batch entry, shared by the heads
+        mask_pair, score_fn = masks.make_causal_mask_fns(128, 128), scores.make_softcap_score_fn(5.0)
+        okw, causal = dict(causal=True, score_mod=O.score_mod_softcap(5.0)), False
+    else:
+        B, Hq, Hkv, Sq, Sk = 1, 2, 2, 200, 333
+        ab = (torch.randn(1, 1, Sq, Sk, generator=g) * 3).to(torch.bfloat16)
+        mask_pair, score_fn, okw, causal = None, None, dict(causal=True), True
+    q, k, v, do = O.make_inputs(B, Hq, Hkv, Sq, Sk, 128, dtype=dtype, seed=61)
+    ab_full = ab.float().expand(B, Hq, Sq, Sk)
+    ro, rl, rm = O.mha_reference(q, k, v, ab_full, sm_scale=sc, save_residuals=True, **okw)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, ab_full, sm_scale=sc, **okw)
+    qg, kg, vg, dog = [x.to(DEV) for x in (q, k, v, do)]
+    o, l, m, dq, dk, dv = _all_passes_with(F, qg, kg, vg, dog, ab.to(DEV), None, sc, mask_pair, score_fn, causal)
+    assert_close("o", o, ro, dtype)
+    assert_close("lse", m + l.log(), rm + rl.log(), dtype)
+    tol = dict(sm_scale=sc, **okw)
+    ma = O.mha_bwd_reference(q, k, v, o.float().cpu(), do, l.cpu(), m.cpu(), ab_full, **tol)
+    for name, t, r, chain in (("dq", dq, ma[0], rdq), ("dk", dk, ma[1], rdk), ("dv", dv, ma[2], rdv)):
+        assert_close(name, t, r, dtype)
+        assert_close(name + " chain", t, chain, dtype, chain=True)
+    # without the bias the result differs (the argument is not ignored)
+    o0 = F._flex_attention_impl(qg, kg, vg, None, None, False, causal, sc, 1, 128, 128, 128, False,
+                                mask_pair[1] if mask_pair else None, mask_pair[0] if mask_pair else None, score_fn)
+    assert float((o0.float() - o.float()).abs().max()) > 0.05
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+def test_segment_ids_per_batch_entry(F, dtype):
+    """Segment ids of shape [B, S] whose rows differ (mha_reference.py:65-73 takes them): every batch entry is
+    masked by its own documents."""
+    sc = 1 / math.sqrt(128)
+    B, S = 3, 512
+    sid = torch.stack([O.doc_ids_from_lengths(l) for l in ([100, 412], [256, 256], [512])])
+    q, k, v, do = O.make_inputs(B, 4, 2, S, S, 128, dtype=dtype, seed=67)
+    okw = dict(sm_scale=sc, causal=True, segment_ids=sid)
+    ro, rl, rm = O.mha_reference(q, k, v, save_residuals=True, **okw)
+    qg, kg, vg, dog = [x.to(DEV) for x in (q, k, v, do)]
+    o, l, m, dq, dk, dv = _all_passes_with(F, qg, kg, vg, dog, None, sid, sc, None, None, True)
+    assert o.shape == q.shape and l.shape == (B, 4, S) and dk.shape == k.shape
+    assert_close("o", o, ro, dtype)
+    assert_close("lse", m + l.log(), rm + rl.log(), dtype)
+    ma = O.mha_bwd_reference(q, k, v, o.float().cpu(), do, l.cpu(), m.cpu(), **okw)
+    for name, t, r in (("dq", dq, ma[0]), ("dk", dk, ma[1]), ("dv", dv, ma[2])):
+        assert_close(name, t, r, dtype)
+
+
 def test_compiled_loop_kernels_on_request(F):
     """bf16 calls run the generated-stream kernels wherever one exists (covered by every other test
     here); `compiled_loop=True` (FLEXATTN_FLAG_COMPILED_LOOP) routes a call to the kernels with a

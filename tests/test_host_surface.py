@@ -137,8 +137,22 @@ def test_entry_points_validate_arguments_without_gpu():
     q = torch.zeros(1, 2, 128, 128, dtype=torch.bfloat16)
     with pytest.raises(ValueError, match="GPU"):
         F._flex_attention_impl(q, q, q, None, None, False, False, 1.0, 1, 128, 128, 128, False, None, None, None)
-    with pytest.raises(NotImplementedError, match="ab"):
-        F._flex_attention_impl(q, q, q, q, None, False, False, 1.0, 1, 128, 128, 128, False, None, None, None)
+    # the additive bias is checked against the shapes of q and k before anything is launched
+    from flex_attention_tpu_amd._common import bias_c, per_batch_segments
+    for bad in (torch.zeros(1, 2, 128, 64), torch.zeros(3, 2, 128, 128), torch.zeros(2, 128, 128)):
+        with pytest.raises(ValueError, match="ab"):
+            bias_c(bad, 1, 2, 128, 128, 128, 128, torch.device("cpu"))
+    with pytest.raises(NotImplementedError, match="dtype"):
+        bias_c(torch.zeros(1, 2, 128, 128, dtype=torch.float16), 1, 2, 128, 128, 128, 128, torch.device("cpu"))
+    c, keep = bias_c(torch.zeros(1, 1, 100, 120), 2, 2, 100, 120, 128, 128, torch.device("cpu"))
+    assert tuple(keep.shape) == (1, 1, 128, 128) and c.stride_b == 0 and c.stride_h == 0 and c.ptr == keep.data_ptr()
+    # segment ids per batch entry: split only when the rows differ
+    same = torch.zeros(2, 128, dtype=torch.int32)
+    assert per_batch_segments(same, 2) is None and per_batch_segments(None, 2) is None
+    rows = per_batch_segments(torch.stack([torch.zeros(128), torch.ones(128)]), 2)
+    assert len(rows) == 2 and int(rows[1][0]) == 1
+    with pytest.raises(ValueError, match="rows"):
+        per_batch_segments(torch.zeros(3, 128), 2)
     with pytest.raises(NotImplementedError):
         block_mask.spec_of(lambda a, b: a[:, None] >= b[None, :], None)
     from flex_attention_tpu_amd._common import check_blocks, score_spec_c
