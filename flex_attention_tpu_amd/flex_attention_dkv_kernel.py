@@ -8,7 +8,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (batch_entry, bias_c, check_blocks, check_qkv, check_rows, kernel_block_map, library_for, pad_seq,
+from ._common import (batch_entry, bias_c, check_blocks, check_qkv, check_rows, kernel_block_map, kernel_head_dim, library_for, pad_seq,
                       padded_len, per_batch_segments, resolve_mask, stream_of)
 from .flex_attention_dq_bwd import bwd_params
 
@@ -39,6 +39,8 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk, Sq_p, Sk_p)
     q, do, k, v = pad_seq(q, Sq_p), pad_seq(do, Sq_p), pad_seq(k, Sk_p), pad_seq(v, Sk_p)
     l, m, di = pad_seq(l, Sq_p), pad_seq(m, Sq_p), pad_seq(di, Sq_p)
+    D_user, D = D, kernel_head_dim(D, q.dtype)   # smaller head dimensions: zero-padded columns
+    q, do, k, v = pad_seq(q, D, 3), pad_seq(do, D, 3), pad_seq(k, D, 3), pad_seq(v, D, 3)
     bm = kernel_block_map(_lib.PASS_DKV, spec, q, Sq_p, Sk_p, D, score_fn)
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)
@@ -48,6 +50,6 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     with torch.cuda.device(q.device):
         lib = library_for(score_fn, spec)
         _lib.check(lib.flexattn_bwd_dkv(C.byref(p), stream_of(q)), lib)
-    if Sk_p != Sk:
-        dk, dv = dk[:, :, :Sk].contiguous(), dv[:, :, :Sk].contiguous()
+    if Sk_p != Sk or D != D_user:
+        dk, dv = dk[:, :, :Sk, :D_user].contiguous(), dv[:, :, :Sk, :D_user].contiguous()
     return dk, dv

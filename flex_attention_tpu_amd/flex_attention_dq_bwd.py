@@ -7,7 +7,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (batch_entry, bias_c, check_blocks, check_qkv, check_rows, dtype_code, kernel_block_map, library_for,
+from ._common import (batch_entry, bias_c, check_blocks, check_qkv, check_rows, dtype_code, kernel_block_map, kernel_head_dim, library_for,
                       pad_seq, padded_len, per_batch_segments, resolve_mask, score_spec_c, stream_of)
 from .block_mask import mask_spec_c
 
@@ -20,6 +20,9 @@ def compute_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
     if not (o.is_cuda and o.is_contiguous() and do.is_contiguous()):
         raise ValueError("o and do must be contiguous GPU tensors")
     B, H, S, D = o.shape
+    if D not in (64, 128):   # (zero columns add nothing to the sum)
+        D = kernel_head_dim(D, o.dtype)
+        o, do = pad_seq(o, D, 3), pad_seq(do, D, 3)
     d = torch.empty(B, H, S, dtype=torch.float32, device=o.device)
     with torch.cuda.device(o.device):
         _lib.check(_lib.load().flexattn_bwd_delta(o.data_ptr(), do.data_ptr(), d.data_ptr(), B * H * S, D,
@@ -64,6 +67,8 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk, Sq_p, Sk_p)
     q, do, k, v = pad_seq(q, Sq_p), pad_seq(do, Sq_p), pad_seq(k, Sk_p), pad_seq(v, Sk_p)
     l, m, d = pad_seq(l, Sq_p), pad_seq(m, Sq_p), pad_seq(d, Sq_p)
+    D_user, D = D, kernel_head_dim(D, q.dtype)   # smaller head dimensions: zero-padded columns
+    q, do, k, v = pad_seq(q, D, 3), pad_seq(do, D, 3), pad_seq(k, D, 3), pad_seq(v, D, 3)
     bm = kernel_block_map(_lib.PASS_DQ, spec, q, Sq_p, Sk_p, D, score_fn)
     dq = torch.empty_like(q)
     ab_c, ab_keep = bias_c(ab, B, Hq, Sq, Sk, Sq_p, Sk_p, q.device)
@@ -72,6 +77,6 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     with torch.cuda.device(q.device):
         lib = library_for(score_fn, spec)
         _lib.check(lib.flexattn_bwd_dq(C.byref(p), stream_of(q)), lib)
-    if Sq_p != Sq:
-        dq = dq[:, :, :Sq].contiguous()
+    if Sq_p != Sq or D != D_user:
+        dq = dq[:, :, :Sq, :D_user].contiguous()
     return dq

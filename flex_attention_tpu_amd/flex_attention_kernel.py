@@ -12,7 +12,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (batch_entry, bias_c, check_blocks, check_qkv, dtype_code, kernel_block_map, library_for, pad_seq,
+from ._common import (batch_entry, bias_c, check_blocks, check_qkv, dtype_code, kernel_block_map, kernel_head_dim, library_for, pad_seq,
                       padded_len, per_batch_segments, resolve_mask, score_spec_c, stream_of)
 from .block_mask import mask_spec_c
 
@@ -43,6 +43,8 @@ def _flex_attention_impl(q, k, v, ab, segment_ids, save_residuals, causal, sm_sc
     Sq_p, Sk_p = padded_len(Sq), padded_len(Sk)
     spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk, Sq_p, Sk_p)
     q, k, v = pad_seq(q, Sq_p), pad_seq(k, Sk_p), pad_seq(v, Sk_p)
+    D_user, D = D, kernel_head_dim(D, q.dtype)   # smaller head dimensions: zero-padded columns
+    q, k, v = pad_seq(q, D, 3), pad_seq(k, D, 3), pad_seq(v, D, 3)
     bm = kernel_block_map(_lib.PASS_FWD, spec, q, Sq_p, Sk_p, D, score_fn)
     ab_c, ab_keep = bias_c(ab, B, Hq, Sq, Sk, Sq_p, Sk_p, q.device)
     o = torch.empty_like(q)
@@ -59,8 +61,8 @@ def _flex_attention_impl(q, k, v, ab, segment_ids, save_residuals, causal, sm_sc
     with torch.cuda.device(q.device):
         lib = library_for(score_fn, spec)
         _lib.check(lib.flexattn_fwd(C.byref(p), stream_of(q)), lib)
-    if Sq_p != Sq:
-        o = o[:, :, :Sq].contiguous()
+    if Sq_p != Sq or D != D_user:
+        o = o[:, :, :Sq, :D_user].contiguous()
         if save_residuals:
             l, m = l[:, :, :Sq].contiguous(), m[:, :, :Sq].contiguous()
     if debug:

@@ -261,6 +261,26 @@ def test_segment_ids_per_batch_entry(F, dtype):
         assert_close(name, t, r, dtype)
 
 
+@pytest.mark.parametrize("D,dtype", [(64, torch.bfloat16), (96, torch.bfloat16), (32, torch.float32), (80, torch.float32)],
+                         ids=["bf16-64", "bf16-96", "fp32-32", "fp32-80"])
+def test_small_head_dimensions(F, D, dtype):
+    """Head dimensions below the kernels' own (bf16 128, fp32 64 / 128) run zero-padded: all passes against the
+    oracle at the caller's head dimension, causal, grouped kv heads."""
+    from flex_attention_tpu_amd import masks
+    sc = 1 / math.sqrt(D)
+    q, k, v, do = O.make_inputs(1, 4, 2, 384, 384, D, dtype=dtype, seed=71)
+    okw = dict(sm_scale=sc, causal=True)
+    ro, rl, rm = O.mha_reference(q, k, v, save_residuals=True, **okw)
+    qg, kg, vg, dog = [x.to(DEV) for x in (q, k, v, do)]
+    o, l, m, dq, dk, dv = _all_passes_with(F, qg, kg, vg, dog, None, None, sc, masks.make_causal_mask_fns(128, 128), None, False)
+    assert o.shape == q.shape and dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+    assert_close("o", o, ro, dtype)
+    assert_close("lse", m + l.log(), rm + rl.log(), dtype)
+    ma = O.mha_bwd_reference(q, k, v, o.float().cpu(), do, l.cpu(), m.cpu(), **okw)
+    for name, t, r in (("dq", dq, ma[0]), ("dk", dk, ma[1]), ("dv", dv, ma[2])):
+        assert_close(name, t, r, dtype)
+
+
 def test_compiled_loop_kernels_on_request(F):
     """bf16 calls run the generated-stream kernels wherever one exists (covered by every other test
     here); `compiled_loop=True` (FLEXATTN_FLAG_COMPILED_LOOP) routes a call to the kernels with a
