@@ -51,7 +51,7 @@ import os
 import sys
 
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
-from gfx950_stream import Emitter, Op, ar, aset, schedule, vr, vset  # noqa: E402
+from gfx950_stream import Emitter, Op, ar, aset, address_flips, schedule, vr, vset  # noqa: E402
 
 NSLOT = 8        # staging slots of 8 registers
 MIN_AHEAD = 2    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
@@ -266,10 +266,15 @@ def build(masked, alibi=False, softcap=False):
     # operand fragments of the MFMA pairs, in the order of their use: not before the pair that had
     # the staging slot has been issued, at least MIN_AHEAD pairs before their own
     reads = []
+    read_texts = []
     for k in range(len(pairs)):
         for text, dst in pair_loads(k):
             reads.append(lds(text, dst, earliest=max(0, 2 * (k - NSLOT) + 2), deadline=max(0, 2 * (k - MIN_AHEAD))))
+            read_texts.append((text, max(0, 2 * (k - MIN_AHEAD))))
     chains.append(reads)
+    # the operand addresses move to the other step buffer behind their last read of the step
+    chains.append(address_flips(read_texts, lambda name, at: valu(
+        f"v_xor_b32_e32 %[{name}], 0x10000, %[{name}]", {("op", name)}, {("op", name)}, earliest=at)))
     # -lse and -delta of block c: behind the first MFMAs of A(c - 1), which read the registers, and
     # well before the first MFMAs of A(c)
     rows = []
@@ -289,11 +294,14 @@ def build(masked, alibi=False, softcap=False):
     # (issued back to back they hold the wave for about a thousand cycles: one CU moves 64 B / clk)
     state = {"direct": 0}
 
-    def direct(lds_imm, goff, gbase):
+    # (M0 of load k + 1 is written behind load k; the loop top writes the first one's)
+    def direct(k, goff, gbase):
+        nxt = None if k == 15 else ((k + 1) // 4) * TILE + ((k + 1) % 4) * 1024
+
         def emit(e):
             if "vmem" in DROP:
                 return
-            e.lds_direct_load(lds_imm, goff, gbase, S_LDSN)
+            e.lds_direct_load_chained(goff, gbase, nxt, S_LDSN)
             state["direct"] += 1
         return emit
 
@@ -302,7 +310,7 @@ def build(masked, alibi=False, softcap=False):
     for t, gbase in enumerate((S_GQ0, S_GQ1, S_GD0, S_GD1)):  # half tiles in LDS order
         for i in range(4):
             at = LOAD_FIRST + LOAD_EVERY * k
-            vm.append(Op(direct(t * TILE + i * 1024, "%[g1v]" if i == 1 else f"%[g{i}]", gbase), cost=LOAD_COST, earliest=at, deadline=at + 12))
+            vm.append(Op(direct(k, "%[g1v]" if i == 1 else f"%[g{i}]", gbase), cost=LOAD_COST, earliest=at, deadline=at + 12))
             k += 1
     chains.append(vm)
 
@@ -403,6 +411,7 @@ def run_loop(full, masked, alibi=False, softcap=False):
         f"s_xor_b32 {t1}, s81, 1",
         f"s_lshl_b32 {t1}, {t1}, 16",
         f"s_add_u32 {S_LDSN}, {t1}, s63",
+        f"s_mov_b32 m0, {S_LDSN}",   # LDS destination of the step's first copy (the streams write the others)
         # q block of the step after the next one (the list position wraps inside the list: always valid)
         # (a vector load: an open scalar load would disturb the streams' lgkmcnt bookkeeping)
         f"s_lshl_b32 {t1}, s79, 2",
@@ -429,8 +438,6 @@ def run_loop(full, masked, alibi=False, softcap=False):
         "s_cselect_b32 s79, 0, s79",
         "s_xor_b32 s81, s81, 1",
     ]
-    tail += [f"v_xor_b32_e32 %[r{i}], 0x10000, %[r{i}]" for i in range(8)]
-    tail += [f"v_xor_b32_e32 %[t{i}], 0x10000, %[t{i}]" for i in range(8)]
     tail += ["v_xor_b32_e32 %[la], 0x200, %[la]", "v_xor_b32_e32 %[lw], 0x200, %[lw]",
              "s_cmp_lt_u32 s76, s82", "s_cbranch_scc1 .Lfa_dkv_loop_%="]
     tail += [f"v_mov_b32_e32 %[{n}], {SREG[n]}" for n in STATE_IO]

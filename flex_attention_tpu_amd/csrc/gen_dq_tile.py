@@ -41,7 +41,7 @@ import os
 import sys
 
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
-from gfx950_stream import Emitter, Op, ar, aset, schedule, vr, vset  # noqa: E402
+from gfx950_stream import Emitter, Op, address_flips, ar, aset, schedule, vr, vset  # noqa: E402
 
 NSLOT = 8        # staging slots of 8 registers
 MIN_AHEAD = 3    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
@@ -212,11 +212,16 @@ def build(masked, alibi=False):
     # ---- LDS reads of the MFMA pairs, in the order of their use: not before the pair that had the
     # staging slot has been issued, at least MIN_AHEAD pairs before their own
     reads = []
+    read_texts = []
     for k in range(len(pairs)):
         for text, dst in pair_loads(k):
             reads.append(Op((lambda e, t=text, d=dst: e.lds_read(t, d)) if "lds" not in DROP else (lambda e: None),
                             earliest=max(0, 2 * (k - NSLOT) + 2), deadline=max(0, 2 * (k - MIN_AHEAD))))
+            read_texts.append((text, max(0, 2 * (k - MIN_AHEAD))))
     chains.append(reads)
+    # the operand addresses move to the other step buffer behind their last read of the step
+    chains.append(address_flips(read_texts, lambda name, at: valu(
+        f"v_xor_b32_e32 %[{name}], 0x10000, %[{name}]", {("op", name)}, {("op", name)}, earliest=at)))
 
     # ---- next step's K / V tiles: 16 LDS-direct loads per wave spread over the stream ------------
     vm = []
@@ -225,9 +230,12 @@ def build(masked, alibi=False):
         for i in range(4):
             at = LOAD_FIRST + LOAD_EVERY * k
 
-            def emit(e, imm=t * TILE + i * 1024, goff="%[g1v]" if i == 1 else f"%[g{i}]", gb=gbase):
+            # (M0 of load k + 1 is written behind load k; the loop top writes the first one's)
+            nxt = None if k == 15 else ((k + 1) // 4) * TILE + ((k + 1) % 4) * 1024
+
+            def emit(e, nxt=nxt, goff="%[g1v]" if i == 1 else f"%[g{i}]", gb=gbase):
                 if "vmem" not in DROP:
-                    e.lds_direct_load(imm, goff, gb, S_LDSN)
+                    e.lds_direct_load_chained(goff, gb, nxt, S_LDSN)
             vm.append(Op(emit, cost=LOAD_COST, earliest=at, deadline=at + 12))
             k += 1
     chains.append(vm)
@@ -285,6 +293,7 @@ def run_loop(full, masked, alibi=False):
         f"s_xor_b32 {t1}, {S['buf']}, 1",
         f"s_lshl_b32 {t1}, {t1}, 16",
         f"s_add_u32 {S_LDSN}, {t1}, {S['w4k']}",
+        f"s_mov_b32 m0, {S_LDSN}",   # LDS destination of the step's first copy (the streams write the others)
         # list entries of the step after the next one, clamped into the list: a second half past its
         # end repeats the last tile (finite data; its keep bits are zero)
         f"s_add_u32 {t0}, {S['it']}, 2",
@@ -313,8 +322,6 @@ def run_loop(full, masked, alibi=False):
     ]
     if alibi:
         tail += [f"s_mov_b32 {S_CUR[0]}, {ka}", f"s_mov_b32 {S_CUR[1]}, {kb_}"]
-    tail += [f"v_xor_b32_e32 %[r{i}], 0x10000, %[r{i}]" for i in range(8)]
-    tail += [f"v_xor_b32_e32 %[t{i}], 0x10000, %[t{i}]" for i in range(8)]
     tail += [f"s_cmp_lt_u32 {S['it']}, {S['it_end']}", "s_cbranch_scc1 .Lfa_dq_loop_%="]
     tail += [f"v_mov_b32_e32 %[{n}], {S[n]}" for n in STATE_IO]
     return top + masked.out + ["s_branch .Lfa_dq_tail_%=", ".Lfa_dq_full_%=:"] + full.out + tail

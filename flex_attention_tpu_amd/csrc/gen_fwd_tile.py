@@ -54,7 +54,7 @@ import os
 import sys
 
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
-from gfx950_stream import Emitter, Op, ar, aset, schedule, vr, vset  # noqa: E402
+from gfx950_stream import Emitter, Op, address_flips, ar, aset, schedule, vr, vset  # noqa: E402
 
 MIN_AHEAD = 2    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
 WAIT_OLD = 20    # a wait for LDS data also covers younger reads issued at least this many instructions ago
@@ -200,6 +200,7 @@ def build(masked, alibi=False):
                   cost=TRANS_COST if trans else 1, **kw)
 
     reads = []
+    read_texts = []
     for k, (kind, c, x) in enumerate(pairs):
         if kind == "A":
             ia = a_index[k]
@@ -207,6 +208,7 @@ def build(masked, alibi=False):
             earliest = 2 * a_pairs[ia - 8] + 2 if ia >= 8 else 0
             reads.append((2 * k, Op((lambda e, t=text, d=dst: e.lds_read(t, d)) if "lds" not in DROP else (lambda e: None),
                                     earliest=earliest, deadline=max(0, 2 * (k - MIN_AHEAD)))))
+            read_texts.append((text, max(0, 2 * (k - MIN_AHEAD))))
         elif x[0] == 0:
             q, u, j = x
             off = 2 * TILE + half_off(c) + u * 4096
@@ -221,6 +223,7 @@ def build(masked, alibi=False):
                             e.lds_read(t, d)
                     earliest = b_last(c - 1, 1, u) + 1 if c > 0 else 0
                     reads.append((2 * k, Op(emit, earliest=earliest, deadline=2 * (k - MIN_AHEAD))))
+                    read_texts.append((text, 2 * (k - MIN_AHEAD)))
     reads.sort(key=lambda r: r[0])  # (stable: in the order of their use)
 
     def mfma_of(k, j):
@@ -414,6 +417,9 @@ def build(masked, alibi=False):
         for q in range(2):
             soft.extend(softmax_chain(c, q))
     chains = [soft, [op for _, op in reads]]
+    # the operand addresses move to the other step buffer behind their last read of the step
+    chains.append(address_flips(read_texts, lambda name, at: valu(
+        f"v_xor_b32_e32 %[{name}], 0x10000, %[{name}]", {("op", name)}, {("op", name)}, earliest=at)))
     if alibi:
         # chain (1, q): behind the first MFMA of chain (0, q) and before this step's first softmax
         chains.append([Op(lambda e, q=q: bias_ops(e, 1, q, S_CUR[0]), cost=CAP, earliest=2 + q, deadline=a_mfma(1, 0, q) - 6)
@@ -426,9 +432,12 @@ def build(masked, alibi=False):
         for i in range(4):
             at = LOAD_FIRST + LOAD_EVERY * k
 
-            def emit(e, imm=t * TILE + i * 1024, goff="%[g1v]" if i == 1 else f"%[g{i}]", gb=gbase):
+            # (M0 of load k + 1 is written behind load k; the loop top writes the first one's)
+            nxt = None if k == 15 else ((k + 1) // 4) * TILE + ((k + 1) % 4) * 1024
+
+            def emit(e, nxt=nxt, goff="%[g1v]" if i == 1 else f"%[g{i}]", gb=gbase):
                 if "vmem" not in DROP:
-                    e.lds_direct_load(imm, goff, gb, S_LDSN)
+                    e.lds_direct_load_chained(goff, gb, nxt, S_LDSN)
             vm.append(Op(emit, cost=LOAD_COST, earliest=at, deadline=at + 12))
             k += 1
     chains.append(vm)
@@ -497,6 +506,7 @@ def run_loop(full, masked, alibi=False):
         top += [f"s_lshl_b32 {t2}, {kb}, 14", f"s_lshr_b32 {t3}, {kb}, 18",  # 64 rows x 256 bytes per kv tile
                 f"s_add_u32 s{n}, {blo}, {t2}", f"s_addc_u32 s{n + 1}, {bhi}, {t3}"]
     top += [f"s_xor_b32 {t1}, {S['buf']}, 1", f"s_lshl_b32 {t1}, {t1}, 16", f"s_add_u32 {S_LDSN}, {t1}, {S['w4k']}",
+            f"s_mov_b32 m0, {S_LDSN}",   # LDS destination of the step's first copy (the streams write the others)
             f"s_cmp_eq_u32 {S['partial']}, 0", "s_cbranch_scc1 .Lfa_fwd_full_%="]
     tail = [
         ".Lfa_fwd_tail_%=:",
@@ -524,8 +534,6 @@ def run_loop(full, masked, alibi=False):
     ]
     if alibi:
         tail += [f"s_mov_b32 {S_CUR[0]}, {ka}", f"s_mov_b32 {S_CUR[1]}, {kb_}"]
-    tail += [f"v_xor_b32_e32 %[r{i}], 0x10000, %[r{i}]" for i in range(8)]
-    tail += [f"v_xor_b32_e32 %[t{i}], 0x10000, %[t{i}]" for i in range(8)]
     tail += [f"s_cmp_lt_u32 {S['it']}, {S['it_end']}", "s_cbranch_scc1 .Lfa_fwd_loop_%="]
     tail += [f"v_mov_b32_e32 %[{n}], {S[n]}" for n in STATE_IO]
     if OUT_OF_LINE:

@@ -50,6 +50,7 @@ class Emitter:
         self.lds_time = []         # ... and when each was issued
         self.wait_old = None       # a wait also covers younger reads issued at least this long ago
         self.stats = {"nop": 0, "wait": 0, "mfma": 0, "valu": 0, "lds": 0}
+        self._m0_t = None
 
     def _raw(self, text, states=1):
         self.out.append(text)
@@ -187,6 +188,16 @@ class Emitter:
         self._raw(f"global_load_lds_dwordx4 {goff}, {gbase}")
         self.stats["vmem"] = self.stats.get("vmem", 0) + 1
 
+    def lds_direct_load_chained(self, goff, gbase, next_imm, ldsn="%[ldsn]"):
+        """An LDS-direct load whose M0 was written behind the previous one (the first one's by the code in
+        front of the stream), followed by the M0 write of the next one: no wait state is spent between the
+        write and its load."""
+        if getattr(self, "_m0_t", None) is None:
+            self._m0_t = -(1 << 20)   # written before the stream
+        self.lds_direct_issue(goff, gbase)
+        if next_imm is not None:
+            self.lds_direct_dest(next_imm, ldsn)
+
     def lds_write(self, text, src_regs):
         """An LDS store: takes a place in the in-order LDS queue like a read."""
         self._wait_lds(src_regs)
@@ -236,6 +247,19 @@ class Op:
 
     def __init__(self, emit, cost=1, earliest=0, deadline=None):
         self.emit, self.cost, self.earliest, self.deadline = emit, cost, earliest, deadline
+
+
+def address_flips(reads, make_op, pattern=r"%\[([rt]\d)\]"):
+    """Chain of operations that flip the LDS operand addresses between the two step buffers (XOR with
+    0x10000), each placed behind the last read of the step that uses the address: in the stream they hide
+    in the gaps between MFMAs, behind the loop's barrier nothing hides them.  `reads`: (text, deadline) of
+    every LDS read of the step; `make_op(name, earliest)` builds the flip of operand `name`."""
+    import re
+    last = {}
+    for text, deadline in reads:
+        for name in re.findall(pattern, text):
+            last[name] = max(last.get(name, 0), deadline)
+    return [make_op(name, at + 1) for name, at in sorted(last.items(), key=lambda kv: kv[1])]
 
 
 def schedule(em, mfmas, chains, cap):
