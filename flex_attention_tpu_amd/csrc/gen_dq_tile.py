@@ -47,8 +47,8 @@ NSLOT = 8        # staging slots of 8 registers
 MIN_AHEAD = 3    # MFMA pairs at least between the LDS reads of a pair and its MFMAs
 WAIT_OLD = 20    # a wait for LDS data also covers younger reads issued at least this many instructions ago
 CAP = 6          # instructions the scheduler puts between two MFMAs unless deadlines force more
-LOAD_FIRST = 2   # MFMA gap from which the first LDS-direct load of the next step may go out
-LOAD_EVERY = 2   # gaps between two of them
+LOAD_FIRST = 0   # MFMA gap from which the first LDS-direct load of the next step may go out
+LOAD_EVERY = 3   # gaps between two of them
 LOAD_COST = 3    # share of an MFMA gap one of them takes
 TRANS_COST = 2   # share of an MFMA gap a transcendental takes (it holds the wave's issue for two slots)
 DROP = ()        # instruction classes left out (--drop, timing studies only)

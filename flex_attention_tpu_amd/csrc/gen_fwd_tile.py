@@ -66,6 +66,7 @@ TAU = "0x40c00000"  # 6.0: M moves when the running maximum relative to it leave
 TRANS_COST = 2   # share of an MFMA gap a transcendental takes (it holds the wave's issue for two slots)
 ROUNDED_SUM = False  # row sums add the bf16-rounded probabilities (v_dot2c on the packed pairs) instead of the fp32 ones
 DROP = ()        # instruction classes left out (--drop, timing studies only)
+SEQUENTIAL = True  # (plain scores) the S chains of the two q blocks one after the other instead of alternating
 
 TILE = 16384
 # No scalar operands: constants come from a per-wave table in LDS, loop state from VGPR operands.
@@ -152,20 +153,37 @@ def build(masked, alibi=False):
             for j in range(2):
                 pairs.append(("B", c, (q, u, j)))
 
-    add_A(0, 0, 8)
-    for c in range(4):
-        for q in range(2):
-            if c < 3:
-                add_A(c + 1, 4 * q, 4 * q + 4)
-            if q == 1:
-                add_B(c, 0)
-            elif c > 0:
-                add_B(c - 1, 1)
-    add_B(3, 1)
+    # Without a position bias the S chains of the two q blocks run one after the other (a chain's eight
+    # MFMAs issue back to back at full rate): the first chain of a kv block is finished eight MFMAs earlier
+    # than when the two alternate, its softmax starts that much earlier, and the softmax work spreads over
+    # the step instead of crowding behind A(0).  A pair is then two k-steps of one chain.
+    sequential = SEQUENTIAL and not alibi
+
+    def add_S(c, q):
+        for j in range(4):
+            pairs.append(("A", c, (q, j)))
+
+    if sequential:
+        for kind, c, q in (("S", 0, 0), ("S", 0, 1), ("S", 1, 0), ("B", 0, 0), ("S", 1, 1), ("B", 0, 1), ("S", 2, 0), ("B", 1, 0),
+                           ("S", 2, 1), ("B", 1, 1), ("S", 3, 0), ("B", 2, 0), ("S", 3, 1), ("B", 2, 1), ("B", 3, 0), ("B", 3, 1)):
+            (add_S if kind == "S" else add_B)(c, q)
+    else:
+        add_A(0, 0, 8)
+        for c in range(4):
+            for q in range(2):
+                if c < 3:
+                    add_A(c + 1, 4 * q, 4 * q + 4)
+                if q == 1:
+                    add_B(c, 0)
+                elif c > 0:
+                    add_B(c - 1, 1)
+        add_B(3, 1)
     idx = {key: 2 * k for k, key in enumerate(pairs)}  # number of the pair's first MFMA
     n_mfma = 2 * len(pairs)
 
     def a_mfma(c, ks, q):     # S chain of q block q: MFMA number of k-step ks
+        if sequential:
+            return idx[("A", c, (q, ks >> 1))] + (ks & 1)
         return idx[("A", c, ks)] + q
 
     def b_first(c, q, u):
@@ -190,6 +208,9 @@ def build(masked, alibi=False):
     def k_slot(k):
         return A_STG + 32 + 4 * (a_index[k] % 8)
 
+    def ks_slot(ks):          # (sequential chains: the fragment of k-step ks has its own slot, read once for both chains)
+        return A_STG + 32 + 4 * ks
+
     def v_place(u, db):
         return A_STG + 4 * (4 * u + db)
 
@@ -202,7 +223,15 @@ def build(masked, alibi=False):
     reads = []
     read_texts = []
     for k, (kind, c, x) in enumerate(pairs):
-        if kind == "A":
+        if kind == "A" and sequential:
+            q, j = x
+            for ks in (2 * j, 2 * j + 1) if q == 0 else ():
+                text, dst = f"ds_read_b128 {ar(ks_slot(ks), 4)}, %[r{ks}] offset:{half_off(c)}", aset(ks_slot(ks), 4)
+                earliest = a_mfma(c - 1, ks, 1) + 1 if c > 0 else 0   # (the slot's last user: the second chain of block c - 1)
+                reads.append((2 * k, Op((lambda e, t=text, d=dst: e.lds_read(t, d)) if "lds" not in DROP else (lambda e: None),
+                                        earliest=earliest, deadline=max(0, 2 * (k - MIN_AHEAD)))))
+                read_texts.append((text, max(0, 2 * (k - MIN_AHEAD))))
+        elif kind == "A":
             ia = a_index[k]
             text, dst = f"ds_read_b128 {ar(k_slot(k), 4)}, %[r{x}] offset:{half_off(c)}", aset(k_slot(k), 4)
             earliest = 2 * a_pairs[ia - 8] + 2 if ia >= 8 else 0
@@ -229,11 +258,16 @@ def build(masked, alibi=False):
     def mfma_of(k, j):
         kind, c, x = pairs[k]
         if kind == "A":
-            ks, q = x, j
+            if sequential:
+                q, ks = x[0], 2 * x[1] + j
+                slot = ks_slot(ks)
+            else:
+                ks, q = x, j
+                slot = k_slot(k)
             s = v_s(c, q)
             # the chain starts from -M: its result is the score relative to the reference maximum
             cin = V_NEGM + 16 * q if ks == 0 else s
-            return (vr(s, 16), ar(k_slot(k), 4), ar(A_Q + 32 * q + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(k_slot(k), 4),
+            return (vr(s, 16), ar(slot, 4), ar(A_Q + 32 * q + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(slot, 4),
                     aset(A_Q + 32 * q + 4 * ks, 4), vset(cin, 16))
         q, u, jj = x
         db = 2 * jj + j
@@ -271,6 +305,8 @@ def build(masked, alibi=False):
                     e.valu(*op[1:])
         return Op(emit, cost=2, **kw)
 
+    late_sums = []
+
     def softmax_chain(c, q):
         """Online softmax of the lane's 16 scores (relative to M) of q block q in kv block c."""
         s = v_s(c, q)
@@ -279,7 +315,7 @@ def build(masked, alibi=False):
         D, AL, negm = V_D + q, V_AL + q, V_NEGM + 16 * q
         ops = []
 
-        if c > 0:
+        if c > 0 and not sequential:
             # M moved while this block's chain was in flight with the old -M: apply the shift now
             late = [("raw", f"s_cmp_eq_u32 {S_PEND[q]}, 0"), ("raw", f"s_cbranch_scc1 .Lfa_fwd_{tag}_late{c}{q}_%="), ("skip_begin",)]
             for e in range(16):
@@ -349,15 +385,20 @@ def build(masked, alibi=False):
             rare += [("raw", "s_mov_b32 s86, -1"), ("raw", "s_mov_b32 s87, 0"),
                      ("valu", f"v_cndmask_b32_e64 {vr(T[5])}, 0, {vr(D)}, s[86:87]", vset(T[5]), vset(D), False),
                      ("valu", f"v_sub_f32_e32 %[addv{q}], %[addv{q}], {vr(T[5])}", kA, kA | vset(T[5]), False)]
-        if c < 3:
+        if c < 3 and not sequential:
             rare.append(("raw", f"s_mov_b32 {S_PEND[q]}, 1"))  # (kv block c + 1 of this step is in flight; block 0 of the next step is not)
         rare += [("skip_end",), ("label", f".Lfa_fwd_{tag}_keep{c}{q}_%=:")]
         # The block rescales O^T: every B(c - 1, q) MFMA is out, no B(c, q) MFMA is; and the chain of
         # kv block c + 1 has started (it carries the old -M and is corrected by its own "late" block).
         rare_earliest = 0
+        rare_deadline = None
         if c > 0:
             rare_earliest = b_last(c - 1, q, 1) + 1
-        if c < 3:
+        if c < 3 and sequential:
+            # (sequential chains: the chain of kv block c + 1 starts behind this block and takes the corrected
+            # -M registers as they are; nothing is ever in flight with the old ones)
+            rare_deadline = a_mfma(c + 1, 0, q) - 1
+        elif c < 3:
             rare_earliest = max(rare_earliest, a_mfma(c + 1, 0, q) + 1)
         if alibi and c < 3:
             # The accumulator input of chain (c + 2, q) (block 0 of the next step for c = 2) right in front
@@ -367,7 +408,7 @@ def build(masked, alibi=False):
             tile = S_CUR[1] if cn < 4 else S_SEL[0]
             ops.append(Op(lambda e: bias_ops(e, cn & 3, q, tile), cost=CAP, earliest=rare_earliest,
                           deadline=a_mfma(cn, 0, q) - 6 if cn < 4 else None))
-        ops.append(block(rare, earliest=rare_earliest))
+        ops.append(block(rare, earliest=rare_earliest, deadline=rare_deadline))
 
         # p = 2^(score - M), packed to bf16 B operands.  The row sum adds the fp32 values: l is then the
         # softmax denominator of the logits themselves, which is what the backward kernels divide their
@@ -391,6 +432,15 @@ def build(masked, alibi=False):
 
         # (one accumulator: splitting the chain over two registers measured slower)
         def dots(g):
+            if sequential and c == 3 and not ROUNDED_SUM:
+                # The last kv block's row sums wait until their B MFMAs are going out (the exponentials of group
+                # g are done by then: their packs feed B(3, q) half g >> 1): they fill the gaps of the step's
+                # last MFMAs, which have no softmax left to hide, instead of crowding the block's short window.
+                for u in range(4):
+                    e = 4 * g + u
+                    late_sums.append(valu(f"v_add_f32_e32 {L}, {L}, {vr(s + e)}", kL, kL | vset(s + e),
+                                          earliest=b_first(c, q, g >> 1)))
+                return
             if ROUNDED_SUM:
                 for h in range(2):
                     pr = v_p(c, q, g >> 1) + 2 * (g & 1) + h
@@ -417,6 +467,8 @@ def build(masked, alibi=False):
         for q in range(2):
             soft.extend(softmax_chain(c, q))
     chains = [soft, [op for _, op in reads]]
+    if late_sums:
+        chains.append(late_sums)
     # the operand addresses move to the other step buffer behind their last read of the step
     chains.append(address_flips(read_texts, lambda name, at: valu(
         f"v_xor_b32_e32 %[{name}], 0x10000, %[{name}]", {("op", name)}, {("op", name)}, earliest=at)))

@@ -386,7 +386,7 @@ def test_fwd_out_of_line_blocks_are_the_inline_ones():
                 cur = None
             else:
                 blocks[cur].append(l)
-        assert cur is None and len(blocks) == 14   # 8 blocks that move M, 6 late corrections
+        assert cur is None and len(blocks) == 8    # the blocks that move M (sequential chains need no late corrections)
         back = []
         i = 0
         while i < len(hot):
