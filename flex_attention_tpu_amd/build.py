@@ -17,6 +17,7 @@ SOURCES = [
     "block_mask.hip",
     "delta.hip",
     "attn_f32.hip",
+    "attn_f32_mfma.hip",
     "fwd_bf16.hip",
     "bwd_dq_bf16.hip",
     "bwd_dkv_bf16.hip",

@@ -204,7 +204,7 @@ static int fwd_with_map(const flexattn_fwd_params* p, const flexattn_block_map& 
   a.mask = to_args(p->mask);
   a.map = row_view(map);
   if (p->dtype == FLEXATTN_BF16) return fwd_bf16_d128(a, s);
-  return fwd_f32(a, p->D, s);
+  return (a.flags & FLEXATTN_FLAG_COMPILED_LOOP) ? fwd_f32(a, p->D, s) : fwd_f32_mfma(a, p->D, s);
 }
 
 // ---- resident block map of flexattn_fwd_noalloc ---------------------------------------------------------
@@ -335,7 +335,7 @@ int flexattn_bwd_dq(const flexattn_bwd_params* p, void* stream) {
   if (rc != FLEXATTN_OK) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (p->dtype == FLEXATTN_BF16) return bwd_dq_bf16_d128(a, s);
-  return bwd_dq_f32(a, p->D, s);
+  return (a.flags & FLEXATTN_FLAG_COMPILED_LOOP) ? bwd_dq_f32(a, p->D, s) : bwd_dq_f32_mfma(a, p->D, s);
 }
 
 int flexattn_bwd_dkv(const flexattn_bwd_params* p, void* stream) {
@@ -344,7 +344,7 @@ int flexattn_bwd_dkv(const flexattn_bwd_params* p, void* stream) {
   if (rc != FLEXATTN_OK) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (p->dtype == FLEXATTN_BF16) return bwd_dkv_bf16_d128(a, s);
-  return bwd_dkv_f32(a, p->D, s);
+  return (a.flags & FLEXATTN_FLAG_COMPILED_LOOP) ? bwd_dkv_f32(a, p->D, s) : bwd_dkv_f32_mfma(a, p->D, s);
 }
 
 }  // extern "C"

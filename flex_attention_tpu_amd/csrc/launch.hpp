@@ -25,6 +25,10 @@ int fwd_f32(const FwdArgs& a, int D, hipStream_t stream);
 int bwd_dq_f32(const BwdArgs& a, int D, hipStream_t stream);
 int bwd_dkv_f32(const BwdArgs& a, int D, hipStream_t stream);
 void f32_tile(int* bq, int* bk);
+// the same on the fp32 matrix cores (the default; FLEXATTN_FLAG_COMPILED_LOOP selects the FMA kernels)
+int fwd_f32_mfma(const FwdArgs& a, int D, hipStream_t stream);
+int bwd_dq_f32_mfma(const BwdArgs& a, int D, hipStream_t stream);
+int bwd_dkv_f32_mfma(const BwdArgs& a, int D, hipStream_t stream);
 
 int bwd_delta(const void* o, const void* dout, float* delta, int64_t rows, int D, int dtype, hipStream_t stream);
 

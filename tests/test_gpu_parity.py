@@ -281,18 +281,20 @@ def test_small_head_dimensions(F, D, dtype):
         assert_close(name, t, r, dtype)
 
 
-def test_compiled_loop_kernels_on_request(F):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+def test_compiled_loop_kernels_on_request(F, dtype):
     """bf16 calls run the generated-stream kernels wherever one exists (covered by every other test
     here); `compiled_loop=True` (FLEXATTN_FLAG_COMPILED_LOOP) routes a call to the kernels with a
     compiled main loop, which must agree with the oracle as well, including rows whose tiles are
-    partly or entirely masked, and the global ALiBi bias with several q heads per kv head."""
+    partly or entirely masked, and the global ALiBi bias with several q heads per kv head.  For
+    float32 the flag selects the FMA kernels instead of the ones on the fp32 matrix cores."""
     from flex_attention_tpu_amd import masks, scores
-    cases = [c for c in _small_cases() if c[3] is None]
+    cases = [c for c in _small_cases() if c[3] is None or dtype == torch.float32]
     cases.append(("alibi_gqa", (1, 4, 2, 512, 512), masks.make_causal_mask_fns(128, 128), scores.make_alibi_global_score_fn(4),
                   dict(causal=True, score_mod=O.score_mod_alibi_global(O.alibi_slopes(4))), 1 / math.sqrt(128)))
     for name, shape, mask_pair, score_fn, okw, sc in cases:
         B, Hq, Hkv, Sq, Sk = shape
-        q, k, v, do = O.make_inputs(B, Hq, Hkv, Sq, Sk, 128, dtype=torch.bfloat16, seed=23)
+        q, k, v, do = O.make_inputs(B, Hq, Hkv, Sq, Sk, 128, dtype=dtype, seed=23)
         ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, **okw)
         rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, sm_scale=sc, **okw)
         qc, kc, vc, doc = q, k, v, do
@@ -300,8 +302,8 @@ def test_compiled_loop_kernels_on_request(F):
         mf, bf = mask_pair if mask_pair else (None, None)
         o, l, m = F._flex_attention_impl(q, k, v, None, None, True, False, sc, 1, 128, 128, 128, False, bf, mf, score_fn,
                                          compiled_loop=True)
-        assert_close(name + " o", o, ro, torch.bfloat16)
-        assert_close(name + " lse", m + l.log(), rm + rl.log(), torch.bfloat16)
+        assert_close(name + " o", o, ro, dtype)
+        assert_close(name + " lse", m + l.log(), rm + rl.log(), dtype)
         d = F.compute_delta(o, do)
         dq = F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=128, block_k_major=128,
                                      block_k=128, sm_scale=sc, debug=False, score_fn=score_fn, mask_fn=mf,
@@ -309,16 +311,16 @@ def test_compiled_loop_kernels_on_request(F):
         dk, dv = F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=128, block_q_major=128,
                                            block_k_major=128, block_k=128, sm_scale=sc, causal=False, debug=False,
                                            score_fn=score_fn, mask_fn=mf, block_mask_fn=bf, compiled_loop=True)
-        _check_grads((dq, dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, torch.bfloat16, dict(sm_scale=sc, **okw), name + " ")
+        _check_grads((dq, dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, dtype, dict(sm_scale=sc, **okw), name + " ")
         # the default (generated-stream) kernels on the same inputs: GQA with the bias takes the
         # stream forward and dq and the compiled dk/dv
         if name == "alibi_gqa":
             o2, l2, m2 = _fwd(F, q, k, v, sc, mf, bf, score_fn)
-            assert_close(name + " o", o2, ro, torch.bfloat16)
+            assert_close(name + " o", o2, ro, dtype)
             d2 = F.compute_delta(o2, do)
             dq2 = _dq(F, q, k, v, l2, m2, o2, do, d2, sc, mf, bf, score_fn)
             dk2, dv2 = _dkv(F, q, k, v, l2, m2, do, d2, sc, mf, bf, score_fn)
-            _check_grads((dq2, dk2, dv2), (rdq, rdk, rdv), qc, kc, vc, doc, o2, l2, m2, torch.bfloat16,
+            _check_grads((dq2, dk2, dv2), (rdq, rdk, rdv), qc, kc, vc, doc, o2, l2, m2, dtype,
                          dict(sm_scale=sc, **okw), name + " ")
 
 
