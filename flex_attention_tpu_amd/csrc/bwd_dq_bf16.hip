@@ -284,9 +284,16 @@ static int launch_dq(const BwdArgs& a, hipStream_t stream) {
 // S chain, slope' (j - i) - lse, with one fp32 MFMA per 32-key block (see gen_dq_tile.py).
 // DOCS: the mask compares document ids; a persistent work-group then takes its items from the longest-first
 // schedule (sorted_items).  (A template parameter: the code costs the other masks registers.)
-template <bool ALIBI, bool DOCS>
+// SOFTCAP: s' = cap tanh(s / cap).  Q goes in multiplied by 2 log2(e) sm_scale / cap, so that an S chain gives u
+// with e^(2 s / cap) = 2^u; the stream turns it into r = 1 / (2^u + 1) (tanh = 1 - 2 r), the exponent
+// cap' - lse - 2 cap' r (cap' = cap log2 e) and the derivative's r (1 - r); the factor 4 sm_scale that is left
+// goes onto dq in the epilogue.
+// KIND: 0 plain, 1 ALIBI, 2 SOFTCAP.
+template <int KIND, bool DOCS>
 __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs a) {
   using namespace dq_cfg;
+  constexpr bool ALIBI = KIND == 1;
+  constexpr bool SOFTCAP = KIND == 2;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   bf16_t* sT = reinterpret_cast<bf16_t*>(smem_raw);  // buffer b: K tile 0, K tile 1, V tile 0, V tile 1
   unsigned* sTbl = reinterpret_cast<unsigned*>(sT + 8 * kTileElems);
@@ -388,7 +395,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   };
   DqPinned st;
   // Q goes in multiplied by sm_scale * log2(e): the streams' scores are then in the log2 domain
-  const float c2 = a.sm_scale * kLog2e;
+  const float cap2 = SOFTCAP ? a.score.cap * kLog2e : 0.f;
+  const float c2 = SOFTCAP ? 2.0f * kLog2e * a.sm_scale / a.score.cap : a.sm_scale * kLog2e;
+  const float out_scale = SOFTCAP ? 4.0f * a.sm_scale : a.sm_scale;
   auto scaled = [c2](unsigned two) {
     const float lo = __builtin_bit_cast(float, two << 16) * c2;
     const float hi = __builtin_bit_cast(float, two & 0xffff0000u) * c2;
@@ -564,7 +573,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
         if (lane == 0) {
           tbl[0] = (unsigned)n_tiles;
           tbl[1] = base0 + (unsigned)w * 4096u;  // LDS address of the wave's first 1 KB block in buffer 0
-          tbl[2] = __builtin_bit_cast(unsigned, a.sm_scale * kLog2e);
+          tbl[2] = __builtin_bit_cast(unsigned, SOFTCAP ? -2.0f * cap2 : c2);
           tbl[3] = (unsigned)n_steps;
           tbl[4] = (unsigned)(size_t)tile_idx;
           tbl[5] = (unsigned)((size_t)tile_idx >> 32);
@@ -598,6 +607,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
 #define FA_DQ_ALIBI_CLOBBERS , "s101", "v184", "v185", "v186"
         FA_DQ_CALL(FA_DQ_RUN_ALIBI, FA_DQ_ALIBI_CLOBBERS, [aone] "v"(aone), [mulv] "v"(mulv), [addv] "v"(addv), [iq] "v"(q_idx), [ka0] "v"(ka0),
                    [kb0] "v"(kb0));
+      } else if constexpr (SOFTCAP) {
+        const float caplse = cap2 - lse2;
+        FA_DQ_CALL(FA_DQ_RUN_SOFTCAP, , [lse] "v"(caplse));
       } else {
         FA_DQ_CALL(FA_DQ_RUN, , [lse] "v"(lse2));
       }
@@ -631,9 +643,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
                    "=v"(x[15])                                                                                     \
                  : "{" REG "}"(SRC));                                                                              \
     _Pragma("unroll") for (int g = 0; g < 4; ++g) {                                                                \
-      /* the streams leave the constant sm_scale out of dS: apply it once */                                       \
-      const bf16x2 lo = pack_bf16(x[4 * g] * a.sm_scale, x[4 * g + 1] * a.sm_scale);                               \
-      const bf16x2 hi = pack_bf16(x[4 * g + 2] * a.sm_scale, x[4 * g + 3] * a.sm_scale);                           \
+      /* the streams leave the constant sm_scale (softcap: 4 sm_scale) out of dS: apply it once */                 \
+      const bf16x2 lo = pack_bf16(x[4 * g] * out_scale, x[4 * g + 1] * out_scale);                                 \
+      const bf16x2 hi = pack_bf16(x[4 * g + 2] * out_scale, x[4 * g + 3] * out_scale);                             \
       const bf16x4 out = {lo[0], lo[1], hi[0], hi[1]};                                                             \
       *reinterpret_cast<bf16x4*>(stage + wr + (unsigned)(((4 * T + g) ^ (row_here & 15)) << 4)) = out;             \
     }                                                                                                              \
@@ -655,10 +667,10 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   }  // work items
 }
 
-template <bool ALIBI, bool DOCS>
+template <int KIND, bool DOCS>
 static int launch_dq_plain_on(const BwdArgs& a, hipStream_t stream) {
   using namespace dq_cfg;
-  auto kern = bwd_dq_bf16_d128_plain_kernel<ALIBI, DOCS>;
+  auto kern = bwd_dq_bf16_d128_plain_kernel<KIND, DOCS>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, PLAIN_LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(dq): %s", hipGetErrorString(attr));
@@ -669,10 +681,10 @@ static int launch_dq_plain_on(const BwdArgs& a, hipStream_t stream) {
   return check_launch("flexattn_bwd_dq bf16");
 }
 
-template <bool ALIBI>
+template <int KIND>
 static int launch_dq_plain(const BwdArgs& a, hipStream_t stream) {
-  return (a.mask.flags & FLEXATTN_MASK_DOC) ? launch_dq_plain_on<ALIBI, true>(a, stream)
-                                            : launch_dq_plain_on<ALIBI, false>(a, stream);
+  return (a.mask.flags & FLEXATTN_MASK_DOC) ? launch_dq_plain_on<KIND, true>(a, stream)
+                                            : launch_dq_plain_on<KIND, false>(a, stream);
 }
 
 #endif  // FLEXATTN_CUSTOM_ONLY
@@ -690,10 +702,11 @@ int bwd_dq_bf16_d128(const BwdArgs& a, hipStream_t stream) {
   const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= dq_cfg::MAX_LIST && a.score.ab == nullptr;
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
-      return stream_ok ? launch_dq_plain<false>(a, stream) : launch_dq<FLEXATTN_SCORE_NONE>(a, stream);
+      return stream_ok ? launch_dq_plain<0>(a, stream) : launch_dq<FLEXATTN_SCORE_NONE>(a, stream);
     case FLEXATTN_SCORE_ALIBI:
-      return stream_ok ? launch_dq_plain<true>(a, stream) : launch_dq<FLEXATTN_SCORE_ALIBI>(a, stream);
-    case FLEXATTN_SCORE_SOFTCAP: return launch_dq<FLEXATTN_SCORE_SOFTCAP>(a, stream);
+      return stream_ok ? launch_dq_plain<1>(a, stream) : launch_dq<FLEXATTN_SCORE_ALIBI>(a, stream);
+    case FLEXATTN_SCORE_SOFTCAP:
+      return stream_ok ? launch_dq_plain<2>(a, stream) : launch_dq<FLEXATTN_SCORE_SOFTCAP>(a, stream);
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_dq<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);
   }
   return set_error(FLEXATTN_EINVAL, "unknown score kind %d", a.score.kind);

@@ -51,6 +51,8 @@ LOAD_FIRST = 0   # MFMA gap from which the first LDS-direct load of the next ste
 LOAD_EVERY = 3   # gaps between two of them
 LOAD_COST = 3    # share of an MFMA gap one of them takes
 TRANS_COST = 2   # share of an MFMA gap a transcendental takes (it holds the wave's issue for two slots)
+CAP_SOFTCAP = 8  # instructions per MFMA gap in the softcap variant (8 VALU ops per element instead of 2)
+S_K2 = "s62"     # (softcap variant) -2 cap log2(e): the table's c2 entry
 DROP = ()        # instruction classes left out (--drop, timing studies only)
 
 TILE = 16384
@@ -107,7 +109,7 @@ def bias_ops(e, block, tile, odd):
     e.mfma_f32x2(vr(V_NL, 16), "%[aone]", vr(b), vset(V_NL, 16), set(), vset(b))
 
 
-def build(masked, alibi=False):
+def build(masked, alibi=False, softcap=False):
     em = Emitter()
     em.wait_old = WAIT_OLD
     pairs = []
@@ -155,8 +157,11 @@ def build(masked, alibi=False):
             s, dp = V_S[c & 1], V_DP[c & 1]
             cin = V_NL if ks == 0 else s
             cdn = V_ND if ks == 0 else dp
-            return [(vr(s, 16), ar(base, 4), ar(A_Q + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(base, 4), aset(A_Q + 4 * ks, 4),
-                     vset(cin, 16)),
+            first = (vr(s, 16), ar(base, 4), ar(A_Q + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(base, 4), aset(A_Q + 4 * ks, 4),
+                     vset(cin, 16))
+            if softcap and ks == 0:   # (the chain's result is the exponent of e^(2 s / cap): nothing to start from)
+                first = (vr(s, 16), ar(base, 4), ar(A_Q + 4 * ks, 4), "0", vset(s, 16), aset(base, 4), aset(A_Q + 4 * ks, 4), set())
+            return [first,
                     (vr(dp, 16), ar(base + 4, 4), ar(A_DO + 4 * ks, 4), vr(cdn, 16), vset(dp, 16), aset(base + 4, 4),
                      aset(A_DO + 4 * ks, 4), vset(cdn, 16))]
         u, j = x
@@ -185,6 +190,26 @@ def build(masked, alibi=False):
             for u in range(4):
                 e = 4 * g + u
                 ops.append(valu(f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
+            if softcap:
+                # the chain gave u with e^(2 s / cap) = 2^u:  r = 1 / (2^u + 1), tanh = 1 - 2 r;  dP' r (1 - r) (the
+                # derivative's factor 4 goes into the epilogue's scale);  exponent (cap' - lse) - 2 cap' r -> P
+                kl = {("op", "lse")}
+                for text, trans in (("v_add_f32_e32 {s}, 1.0, {s}", False), ("v_rcp_f32_e32 {s}, {s}", True)):
+                    for u in range(4):
+                        e = 4 * g + u
+                        ops.append(valu(text.format(s=vr(s + e)), vset(s + e), vset(s + e), trans))
+                for u in range(4):
+                    e = 4 * g + u
+                    ops.append(valu(f"v_mul_f32_e32 {vr(dp + e)}, {vr(dp + e)}, {vr(s + e)}", vset(dp + e), vset(dp + e) | vset(s + e)))
+                for u in range(4):
+                    e = 4 * g + u
+                    ops.append(valu(f"v_fma_f32 {vr(dp + e)}, -{vr(dp + e)}, {vr(s + e)}, {vr(dp + e)}", vset(dp + e), vset(dp + e) | vset(s + e)))
+                for u in range(4):
+                    e = 4 * g + u
+                    ops.append(valu(f"v_fma_f32 {vr(s + e)}, {vr(s + e)}, {S_K2}, %[lse]", vset(s + e), vset(s + e) | kl))
+                for u in range(4):
+                    e = 4 * g + u
+                    ops.append(valu(f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
             if masked:
                 for u in range(4):
                     e = 4 * g + u
@@ -250,12 +275,12 @@ def build(masked, alibi=False):
                            deadline=first_A[c] - 6 if c < 4 else None))
         chains.append(bias)
 
-    schedule(em, mfmas, chains, CAP)
+    schedule(em, mfmas, chains, CAP_SOFTCAP if softcap else CAP)
     em.drain()
     return em
 
 
-def run_loop(full, masked, alibi=False):
+def run_loop(full, masked, alibi=False, softcap=False):
     """One asm statement: a run of consecutive steps [it, it_end) of one work item, at most one of
     them partial.  At entry the step's K / V tiles are resident in LDS buffer %[buf]; each pass
     computes the next step's addresses, streams the step (which copies the next step's tiles into the
@@ -272,7 +297,7 @@ def run_loop(full, masked, alibi=False):
         entry += [f"v_readfirstlane_b32 {S_CUR[0]}, %[ka0]", f"v_readfirstlane_b32 {S_CUR[1]}, %[kb0]"]
         bias_ops(pre, 0, S_CUR[0], 0)   # (used by the first MFMA of the loop, more than 20 instructions on)
         entry += pre.out
-    else:
+    elif not softcap:   # (softcap: %[lse] is cap' - lse and joins the exponent element by element)
         entry += [f"v_sub_f32_e32 {vr(V_NL + e)}, 0, %[lse]" for e in range(16)]
     entry += [f"v_sub_f32_e32 {vr(V_ND + e)}, 0, %[dl]" for e in range(16)]
     top = entry + [".Lfa_dq_loop_%=:"]
@@ -348,6 +373,7 @@ def main():
         full, masked = build(False), build(True)
         macro("FA_DQ_RUN", run_loop(full, masked))
         macro("FA_DQ_RUN_ALIBI", run_loop(build(False, True), build(True, True), True))
+        macro("FA_DQ_RUN_SOFTCAP", run_loop(build(False, softcap=True), build(True, softcap=True), softcap=True))
         for name, em in (("full", full), ("masked", masked)):
             print(f"{args.out}: {name}: {len(em.out)} instructions, {em.stats}", file=sys.stderr)
         macro("FA_DQ_ZERO_ACC", [f"v_accvgpr_write_b32 a{A_DQ + i}, 0" for i in range(64)])

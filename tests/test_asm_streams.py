@@ -251,6 +251,13 @@ def test_dq_tile_streams_respect_hazards():
         assert em.stats["mfma"] == 96 and em.stats["mfma32"] == 4
         assert n == em.stats["mfma"] + em.stats["mfma32"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
         scratch_ok(em.out, 66, 186, 191)
+        # softcap variant: eight element-wise operations per score instead of two, same MFMAs
+        em = g.build(masked, softcap=True)
+        n = check_stream(em.out)
+        assert em.stats["mfma"] == 96
+        assert n == em.stats["mfma"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
+        scratch_ok(em.out, 66, 183, 191)
+        check_dataflow(em.out, 1, 4)
 
 
 def test_fwd_tile_streams_respect_hazards():
