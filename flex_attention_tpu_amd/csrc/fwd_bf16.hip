@@ -359,9 +359,18 @@ static int launch_fwd(const FwdArgs& a, hipStream_t stream) {
 // S chain, slope' (j - i) - M, with one fp32 MFMA per chain (see gen_fwd_tile.py).
 // DOCS: the mask compares document ids; those of a partial step's kv tiles are staged through LDS
 // (stage_doc_ids).  (A template parameter: the staging code costs the other masks registers.)
-template <bool ALIBI, bool DOCS>
+// SOFTCAP: s' = cap tanh(s / cap) is bounded by the cap, so the reference maximum is the constant cap and the
+// streams track no maximum at all: Q goes in multiplied by 2 log2(e) sm_scale / cap, an S chain gives u with
+// e^(2 s / cap) = 2^u, and p = 2^(-2 cap' r), r = 1 / (2^u + 1), cap' = cap log2(e).  The residuals are returned
+// relative to that bound, m = cap and l = sum exp(s' - cap): m + log l is the row's logsumexp as always, which
+// is all the backward kernels take from them.  (Caps up to 50 / log2(e): beyond, p could leave the range of the
+// accumulation; the compiled kernel takes those.)
+// KIND: 0 plain, 1 ALIBI, 2 SOFTCAP.
+template <int KIND, bool DOCS>
 __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) {
   using namespace fwd_cfg;
+  constexpr bool ALIBI = KIND == 1;
+  constexpr bool SOFTCAP = KIND == 2;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   bf16_t* sT = reinterpret_cast<bf16_t*>(smem_raw);  // buffer b: K tile 0, K tile 1, V tile 0, V tile 1
   unsigned* sTbl = reinterpret_cast<unsigned*>(sT + 8 * kTileElems);
@@ -472,7 +481,8 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
   };
   FwdPinned st;
   // Q goes in multiplied by sm_scale * log2(e): the streams' scores are then in the log2 domain
-  const float c2 = a.sm_scale * kLog2e;
+  const float cap2 = SOFTCAP ? a.score.cap * kLog2e : 0.f;
+  const float c2 = SOFTCAP ? 2.0f * kLog2e * a.sm_scale / a.score.cap : a.sm_scale * kLog2e;
   auto scaled = [c2](unsigned two) {
     const float lo = __builtin_bit_cast(float, two << 16) * c2;
     const float hi = __builtin_bit_cast(float, two & 0xffff0000u) * c2;
@@ -550,7 +560,8 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
     const int q_idx[2] = {(2 * qb2) * BM + q_local, (2 * qb2 + 1) * BM + q_local};
     // softmax state of the lane's two q rows (log2 domain): reference maximum M, running maximum
     // relative to it, sum of 2^(score - M)
-    float M[2] = {0.f, 0.f}, Mt[2] = {kNegInf, kNegInf}, L[2] = {0.f, 0.f};
+    // (softcap: the reference is the constant cap and the streams leave M and Mt alone)
+    float M[2] = {cap2, cap2}, Mt[2] = {SOFTCAP ? 0.f : kNegInf, SOFTCAP ? 0.f : kNegInf}, L[2] = {0.f, 0.f};
     // operands of the fp32 MFMA that makes the S chains' accumulator input under a position bias
     // (addv: -M of the lane's q row in lanes 0-31, which the streams keep up to date; the slope in the others)
     const float a2 = ALIBI ? a.score.slopes[bh % a.Hq] * kLog2e : 0.f;
@@ -595,7 +606,7 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
       const int ka = entry(0), kbb = entry(1);
       tbl[0] = (unsigned)n_list;
       tbl[1] = base0 + (unsigned)w * 4096u;  // LDS address of the wave's first 1 KB block in buffer 0
-      tbl[2] = __builtin_bit_cast(unsigned, c2);
+      tbl[2] = __builtin_bit_cast(unsigned, SOFTCAP ? -2.0f * cap2 : c2);
       tbl[3] = (unsigned)n_steps;
       tbl[4] = (unsigned)(size_t)Kg;
       tbl[5] = (unsigned)((size_t)Kg >> 32);
@@ -733,6 +744,8 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
         const int kb0 = __builtin_amdgcn_readfirstlane(entry(2 * it + 1));
         FA_FWD_CALL(FA_FWD_RUN_ALIBI, FA_FWD_ADDV, FA_FWD_ALIBI_CLOBBERS, [aone] "v"(aone), [mulv] "v"(mulv), [iq] "v"(q_idx[0]), [ka0] "v"(ka0),
                     [kb0] "v"(kb0));
+      } else if constexpr (SOFTCAP) {
+        FA_FWD_CALL(FA_FWD_RUN_SOFTCAP, , );
       } else {
         FA_FWD_CALL(FA_FWD_RUN, , );
       }
@@ -811,10 +824,10 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
   }  // work items
 }
 
-template <bool ALIBI, bool DOCS>
+template <int KIND, bool DOCS>
 static int launch_fwd_plain_on(const FwdArgs& a, hipStream_t stream) {
   using namespace fwd_cfg;
-  auto kern = fwd_bf16_d128_plain_kernel<ALIBI, DOCS>;
+  auto kern = fwd_bf16_d128_plain_kernel<KIND, DOCS>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, PLAIN_LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(fwd): %s", hipGetErrorString(attr));
@@ -827,10 +840,10 @@ static int launch_fwd_plain_on(const FwdArgs& a, hipStream_t stream) {
   return check_launch("flexattn_fwd bf16");
 }
 
-template <bool ALIBI>
+template <int KIND>
 static int launch_fwd_plain(const FwdArgs& a, hipStream_t stream) {
-  return (a.mask.flags & FLEXATTN_MASK_DOC) ? launch_fwd_plain_on<ALIBI, true>(a, stream)
-                                            : launch_fwd_plain_on<ALIBI, false>(a, stream);
+  return (a.mask.flags & FLEXATTN_MASK_DOC) ? launch_fwd_plain_on<KIND, true>(a, stream)
+                                            : launch_fwd_plain_on<KIND, false>(a, stream);
 }
 
 #endif  // FLEXATTN_CUSTOM_ONLY
@@ -852,10 +865,11 @@ int fwd_bf16_d128(const FwdArgs& a, hipStream_t stream) {
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
       if (a.score.ab != nullptr) return launch_fwd<kScoreBiasOnly>(a, stream);
-      return stream_ok ? launch_fwd_plain<false>(a, stream) : launch_fwd<FLEXATTN_SCORE_NONE>(a, stream);
+      return stream_ok ? launch_fwd_plain<0>(a, stream) : launch_fwd<FLEXATTN_SCORE_NONE>(a, stream);
     case FLEXATTN_SCORE_ALIBI:
-      return stream_ok ? launch_fwd_plain<true>(a, stream) : launch_fwd<FLEXATTN_SCORE_ALIBI>(a, stream);
-    case FLEXATTN_SCORE_SOFTCAP: return launch_fwd<FLEXATTN_SCORE_SOFTCAP>(a, stream);
+      return stream_ok ? launch_fwd_plain<1>(a, stream) : launch_fwd<FLEXATTN_SCORE_ALIBI>(a, stream);
+    case FLEXATTN_SCORE_SOFTCAP:
+      return (stream_ok && a.score.cap * kLog2e <= 50.f) ? launch_fwd_plain<2>(a, stream) : launch_fwd<FLEXATTN_SCORE_SOFTCAP>(a, stream);
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_fwd<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);
   }
   return set_error(FLEXATTN_EINVAL, "unknown score kind %d", a.score.kind);

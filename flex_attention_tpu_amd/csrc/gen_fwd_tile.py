@@ -66,6 +66,8 @@ TAU = "0x40c00000"  # 6.0: M moves when the running maximum relative to it leave
 TRANS_COST = 2   # share of an MFMA gap a transcendental takes (it holds the wave's issue for two slots)
 ROUNDED_SUM = False  # row sums add the bf16-rounded probabilities (v_dot2c on the packed pairs) instead of the fp32 ones
 DROP = ()        # instruction classes left out (--drop, timing studies only)
+CAP_SOFTCAP = 8  # instructions per MFMA gap in the softcap variant (6.5 VALU ops per score instead of 2.5)
+S_K2 = "s62"     # (softcap variant) -2 cap log2(e): the table's c2 entry
 SEQUENTIAL = True  # (plain scores) the S chains of the two q blocks one after the other instead of alternating
 
 TILE = 16384
@@ -136,7 +138,7 @@ def v_p(c, x, u):
     return V_P0 + 8 * x + 4 * u
 
 
-def build(masked, alibi=False):
+def build(masked, alibi=False, softcap=False):
     em = Emitter()
     em.wait_old = WAIT_OLD
     # MFMA pairs (2 MFMAs each), in issue order.  The two q blocks of a kv block are processed half a
@@ -267,6 +269,9 @@ def build(masked, alibi=False):
             s = v_s(c, q)
             # the chain starts from -M: its result is the score relative to the reference maximum
             cin = V_NEGM + 16 * q if ks == 0 else s
+            if softcap and ks == 0:   # (softcap: the result is the exponent of e^(2 s / cap), nothing to start from)
+                return (vr(s, 16), ar(slot, 4), ar(A_Q + 32 * q + 4 * ks, 4), "0", vset(s, 16), aset(slot, 4),
+                        aset(A_Q + 32 * q + 4 * ks, 4), set())
             return (vr(s, 16), ar(slot, 4), ar(A_Q + 32 * q + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(slot, 4),
                     aset(A_Q + 32 * q + 4 * ks, 4), vset(cin, 16))
         q, u, jj = x
@@ -314,6 +319,41 @@ def build(masked, alibi=False):
         kM, kMt, kL = {("op", f"M{q}")}, {("op", f"Mt{q}")}, {("op", f"L{q}")}
         D, AL, negm = V_D + q, V_AL + q, V_NEGM + 16 * q
         ops = []
+
+        if softcap:
+            # Scores are bounded by the cap, so the reference maximum is the constant cap and nothing is tracked:
+            # the chain gave u with e^(2 s / cap) = 2^u; r = 1 / (2^u + 1), tanh = 1 - 2 r, and
+            # p = 2^(cap' tanh - cap') = 2^(-2 cap' r) with cap' = cap log2(e) (S_K2 holds -2 cap').
+            def packs_sc(g):
+                u2 = g >> 1
+                war = b_last(c - 1, q, u2) + 1 if c > 0 else 0   # the registers are those of block c - 1
+                for h in range(2):
+                    e = 4 * g + 2 * h
+                    pr = v_p(c, q, u2) + 2 * (g & 1) + h
+                    ops.append(valu(f"v_cvt_pk_bf16_f32 {vr(pr)}, {vr(s + e)}, {vr(s + e + 1)}", vset(pr), vset(s + e, 2),
+                                    earliest=war, deadline=b_first(c, q, u2) - 1))
+            for g in range(4):
+                for text, trans in (("v_exp_f32_e32 {s}, {s}", True), ("v_add_f32_e32 {s}, 1.0, {s}", False),
+                                    ("v_rcp_f32_e32 {s}, {s}", True), (f"v_mul_f32_e32 {{s}}, {S_K2}, {{s}}", False),
+                                    ("v_exp_f32_e32 {s}, {s}", True)):
+                    for u in range(4):
+                        e = 4 * g + u
+                        ops.append(valu(text.format(s=vr(s + e)), vset(s + e), vset(s + e), trans))
+                if masked:
+                    for u in range(4):
+                        e = 4 * g + u
+                        ops.append(valu(f"v_bfe_i32 {vr(V_MSK + u)}, %[m{2 * q + (c >> 1)}], {16 * (c & 1) + e}, 1", vset(V_MSK + u), set()))
+                    for u in range(4):
+                        e = 4 * g + u   # keep ? p : 0
+                        ops.append(valu(f"v_and_b32_e32 {vr(s + e)}, {vr(s + e)}, {vr(V_MSK + u)}", vset(s + e), vset(s + e) | vset(V_MSK + u)))
+                packs_sc(g)
+                for u in range(4):
+                    e = 4 * g + u
+                    ops.append(valu(f"v_add_f32_e32 {L}, {L}, {vr(s + e)}", kL, kL | vset(s + e)))
+            ops[0].earliest = max(ops[0].earliest, a_mfma(c, 7, q) + 4)   # the chain's last result needs 12 wait states
+            if c + 2 < 4:
+                ops[-1].deadline = min(ops[-1].deadline or (1 << 30), a_mfma(c + 2, 0, q))  # A(c + 2) writes the same S registers
+            return ops
 
         if c > 0 and not sequential:
             # M moved while this block's chain was in flight with the old -M: apply the shift now
@@ -496,7 +536,7 @@ def build(masked, alibi=False):
 
     if masked:
         em.valu(f"v_mov_b32_e32 {vr(V_NEGINF)}, 0xff800000", vset(V_NEGINF), set())
-    schedule(em, mfmas, chains, CAP)
+    schedule(em, mfmas, chains, CAP_SOFTCAP if softcap else CAP)
     em.drain()
     return em
 
@@ -526,7 +566,7 @@ def out_of_line(lines):
     return hot, cold
 
 
-def run_loop(full, masked, alibi=False):
+def run_loop(full, masked, alibi=False, softcap=False):
     """One asm statement: a run of consecutive steps [it, it_end) of one work item, all full or a
     single partial one.  At entry the step's K / V tiles are resident in LDS buffer %[buf]."""
     t0, t1, t2, t3 = S_T
@@ -542,7 +582,7 @@ def run_loop(full, masked, alibi=False):
         for q in range(2):
             bias_ops(pre, 0, q, S_CUR[0])   # (used by the first MFMAs of the loop, more than 20 instructions on)
         entry += pre.out
-    else:
+    elif not softcap:
         entry += [f"v_sub_f32_e32 {vr(V_NEGM + 16 * q + e)}, 0, %[M{q}]" for q in range(2) for e in range(16)]
     top = entry + [".Lfa_fwd_loop_%=:"]
     # on the item's last step the tiles copied "for the next step" are the first step of the next
@@ -617,6 +657,7 @@ def main():
         full, masked = build(False), build(True)
         macro("FA_FWD_RUN", run_loop(full, masked))
         macro("FA_FWD_RUN_ALIBI", run_loop(build(False, True), build(True, True), True))
+        macro("FA_FWD_RUN_SOFTCAP", run_loop(build(False, softcap=True), build(True, softcap=True), softcap=True))
         for name, em in (("full", full), ("masked", masked)):
             print(f"{args.out}: {name}: {len(em.out)} instructions, {em.stats}", file=sys.stderr)
         macro("FA_FWD_ZERO_ACC", [f"v_accvgpr_write_b32 a{A_O + i}, 0" for i in range(128)])

@@ -275,6 +275,13 @@ def test_fwd_tile_streams_respect_hazards():
         assert ab.stats["mfma"] == 128 and ab.stats["mfma32"] == 8
         assert nb == ab.stats["mfma"] + ab.stats["mfma32"] + ab.stats["valu"] + ab.stats["lds"] + ab.stats["vmem"]
         scratch_ok(ab.out, 66, 201, 255)
+        # softcap variant: no maximum is tracked, no branch at all, 6.5 element-wise operations per score
+        sc = g.build(masked, softcap=True)
+        ns = check_stream(sc.out)
+        assert sc.stats["mfma"] == 128 and not any(l.startswith(("s_cbranch", "s_branch")) for l in sc.out)
+        assert ns == sc.stats["mfma"] + sc.stats["valu"] + sc.stats["lds"] + sc.stats["vmem"]
+        scratch_ok(sc.out, 66, 199, 255)
+        check_dataflow(sc.out, 2, 4)
         # between a forward branch and its label there is only VALU / scalar work: a skipped MFMA,
         # LDS read or wait would break the stream's bookkeeping
         pending = None
