@@ -1,7 +1,9 @@
 """Benchmark of the flex-attention hot path on one MI355X.
 
 One step = one pass of the hot path over one batch of synthetic input resident in HBM:
-forward (saving l, m), delta pre-pass, dq backward, dk/dv backward.  The headline workload is
+forward (saving l, m), delta pre-pass, dk/dv backward, dq backward (the dk/dv pass hands its dS to the dq pass
+where the kernels of the configuration can: plain and softcap scores in bf16; the two passes without the
+hand-over are timed beside it).  The headline workload is
 benchmark configurations 2 + 3 (B=4, H=32, S=4096, D=128, bf16, causal); the other configurations
 (cfg1 fp32 small, cfg4 ALiBi + causal window, cfg5 GQA + soft-cap + documents) are measured in the
 same run and reported as sub-objects (`--config NAME` makes one of them the headline instead).
@@ -94,19 +96,21 @@ def measure(cfg, steps, warmup):
     def fwd():
         return F._flex_attention_impl(q, k, v, None, None, True, False, sc, 1, blk, blk, blk, False, bf, mf, sfn)
 
-    def dq_of(o, l, m, d):
+    def dq_of(o, l, m, d, ds=None):
         return F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=blk, block_k_major=blk,
-                                       block_k=blk, sm_scale=sc, debug=False, score_fn=sfn, mask_fn=mf, block_mask_fn=bf)
+                                       block_k=blk, sm_scale=sc, debug=False, score_fn=sfn, mask_fn=mf, block_mask_fn=bf,
+                                       ds=ds)
 
-    def dkv_of(l, m, d):
+    def dkv_of(l, m, d, return_ds=False):
         return F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=blk, block_q_major=blk,
                                          block_k_major=blk, block_k=blk, sm_scale=sc, causal=False, debug=False,
-                                         score_fn=sfn, mask_fn=mf, block_mask_fn=bf)
+                                         score_fn=sfn, mask_fn=mf, block_mask_fn=bf, return_ds=return_ds)
 
     def step():
         o, l, m = fwd()
         d = F.compute_delta(o, do)
-        return o, dq_of(o, l, m, d), dkv_of(l, m, d)
+        dk, dv, ds = dkv_of(l, m, d, True)   # (ds is None where the configuration's kernels exchange nothing)
+        return o, dq_of(o, l, m, d, ds), dk, dv
 
     for _ in range(warmup):
         step()
@@ -122,8 +126,11 @@ def measure(cfg, steps, warmup):
     # behind every launch of a second batch gives the launch-to-launch intervals for the quantiles.
     o, l, m = fwd()
     d = F.compute_delta(o, do)
-    launches = {"fwd": fwd, "delta": lambda: F.compute_delta(o, do), "dq": lambda: dq_of(o, l, m, d),
-                "dkv": lambda: dkv_of(l, m, d)}
+    ds = dkv_of(l, m, d, True)[2]
+    launches = {"fwd": fwd, "delta": lambda: F.compute_delta(o, do), "dq": lambda: dq_of(o, l, m, d, ds),
+                "dkv": lambda: dkv_of(l, m, d, True)}
+    if ds is not None:   # the two passes on their own, each recomputing S, dP and dS
+        launches.update(dq_recompute=lambda: dq_of(o, l, m, d), dkv_no_export=lambda: dkv_of(l, m, d))
     ms, quant = {}, {}
     for name, fn in launches.items():
         fn()
@@ -143,7 +150,7 @@ def measure(cfg, steps, warmup):
         torch.cuda.synchronize()
         quant[name] = quantiles([ev[i].elapsed_time(ev[i + 1]) for i in range(steps)])
     return {"ms_step": wall * 1e3 / steps, "ms": ms, "quantiles_ms": quant, "elem_bytes": q.element_size(),
-            "numel_q": q.numel(), "numel_k": k.numel()}
+            "numel_q": q.numel(), "numel_k": k.numel(), "ds_bytes": ds.buf.numel() if ds is not None else 0}
 
 
 def tf(fl, t_ms):
@@ -168,8 +175,13 @@ def summary(cfg, r):
         "bwd": {"ms": ms_bwd, "tflops": tf(2.5 * f_fwd, ms_bwd), "delta_ms": ms["delta"], "dq_ms": ms["dq"],
                 "dkv_ms": ms["dkv"], "delta_gbs": bytes_delta / (ms["delta"] * 1e-3) / 1e9,
                 "dq_quantiles_ms": r["quantiles_ms"]["dq"], "dkv_quantiles_ms": r["quantiles_ms"]["dkv"],
-                "delta_quantiles_ms": r["quantiles_ms"]["delta"]},
+                "delta_quantiles_ms": r["quantiles_ms"]["delta"], "ds_exchange": r["ds_bytes"] > 0},
     }
+    if r["ds_bytes"] > 0:
+        ms_split = ms["delta"] + ms["dq_recompute"] + ms["dkv_no_export"]
+        out["bwd"].update(ds_buffer_bytes=r["ds_bytes"], dq_recompute_ms=ms["dq_recompute"],
+                          dkv_no_export_ms=ms["dkv_no_export"], ms_without_exchange=ms_split,
+                          tflops_without_exchange=tf(2.5 * f_fwd, ms_split))
     if eb == 2:
         out["fwd"]["frac_of_peak"] = out["fwd"]["tflops"] / PEAK_BF16_TFLOPS
         out["bwd"]["frac_of_peak"] = out["bwd"]["tflops"] / PEAK_BF16_TFLOPS
@@ -226,8 +238,8 @@ def main():
     f_fwd = configs.flops_fwd(cfg)
     bf16 = r["elem_bytes"] == 2
     # roofline of the dominant kernel; algorithmic FLOPs of one launch:
-    #   fwd 2 matmuls = F_fwd, dq 3 matmuls = 1.5 F_fwd, dk/dv 4 matmuls = 2 F_fwd
-    algo = {"fwd": f_fwd, "dq": 1.5 * f_fwd, "dkv": 2.0 * f_fwd}
+    #   fwd 2 matmuls = F_fwd, dk/dv 4 matmuls = 2 F_fwd, dq 3 matmuls = 1.5 F_fwd (1 matmul from exchanged dS)
+    algo = {"fwd": f_fwd, "dq": (0.5 if r["ds_bytes"] > 0 else 1.5) * f_fwd, "dkv": 2.0 * f_fwd}
     dom = max(algo, key=lambda n: ms[n])
     traffic = counter_traffic(dom) if name == "cfg2" else None
     roofline = {
@@ -249,7 +261,7 @@ def main():
         "ms_per_step": r["ms_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if bf16 else "f32", "data": "synthetic",
-        "config": {"workload": f"{cfg.name}{'+cfg3' if name == 'cfg2' else ''}: fwd + delta + dq + dk/dv, B={cfg.B} "
+        "config": {"workload": f"{cfg.name}{'+cfg3' if name == 'cfg2' else ''}: fwd + delta + dk/dv + dq, B={cfg.B} "
                                f"Hq={cfg.Hq} Hkv={cfg.Hkv} S={cfg.S} D={cfg.D} {'bf16' if bf16 else 'fp32'}, "
                                f"mask={cfg.mask}, score={cfg.score}, sm_scale=1/sqrt(D)"},
         "fwd": head["fwd"], "bwd": head["bwd"],

@@ -120,6 +120,8 @@ class BwdParamsC(C.Structure):
         ("mask", MaskSpecC),
         ("map", BlockMapC),
         ("ab", BiasC),
+        ("ds", C.c_void_p),
+        ("ds_bytes", C.c_int64),
     ]
 
 
@@ -131,6 +133,7 @@ EXPORTS = (
     "flexattn_fwd",
     "flexattn_fwd_noalloc",
     "flexattn_bwd_delta",
+    "flexattn_bwd_ds_bytes",
     "flexattn_bwd_dq",
     "flexattn_bwd_dkv",
     "flexattn_custom_tag",
@@ -152,6 +155,8 @@ def _bind(lib: C.CDLL) -> C.CDLL:
     lib.flexattn_fwd_noalloc.argtypes = [C.POINTER(FwdParamsC), C.c_void_p]
     lib.flexattn_bwd_delta.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
     lib.flexattn_bwd_dq.argtypes = [C.POINTER(BwdParamsC), C.c_void_p]
+    lib.flexattn_bwd_ds_bytes.argtypes = [C.POINTER(BwdParamsC)]
+    lib.flexattn_bwd_ds_bytes.restype = C.c_int64
     lib.flexattn_bwd_dkv.argtypes = [C.POINTER(BwdParamsC), C.c_void_p]
     for name in ("flexattn_tile_shape", "flexattn_build_block_mask", "flexattn_fwd", "flexattn_fwd_noalloc", "flexattn_bwd_delta",
                  "flexattn_bwd_dq", "flexattn_bwd_dkv"):

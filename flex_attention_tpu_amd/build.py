@@ -21,6 +21,7 @@ SOURCES = [
     "fwd_bf16.hip",
     "bwd_dq_bf16.hip",
     "bwd_dkv_bf16.hip",
+    "bwd_dq_ds.hip",
 ]
 
 # instruction streams generated before compiling: (generator script, output it writes next to itself)

@@ -128,13 +128,15 @@ static int check_scale_flags(float sm_scale, int flags) {
   return FLEXATTN_OK;
 }
 
+// `tile_pass`: the pass whose tile granularity the map must have (the dq pass reads the dk/dv kernel's dS blocks at
+// that kernel's tiles)
 static int check_shape(int pass, int B, int Hq, int Hkv, int Sq, int Sk, int D, int dtype,
-                       const flexattn_block_map& map) {
+                       const flexattn_block_map& map, int tile_pass = -1) {
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || Sq <= 0 || Sk <= 0 || D <= 0)
     return set_error(FLEXATTN_EINVAL, "non-positive dimension (B=%d Hq=%d Hkv=%d Sq=%d Sk=%d D=%d)", B, Hq, Hkv, Sq, Sk, D);
   if (Hq % Hkv != 0) return set_error(FLEXATTN_EINVAL, "Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
   int bq = 0, bk = 0;
-  int rc = tile_shape(pass, dtype, D, &bq, &bk);
+  int rc = tile_shape(tile_pass >= 0 ? tile_pass : pass, dtype, D, &bq, &bk);
   if (rc != FLEXATTN_OK) return rc;
   if (Sq % bq != 0) return set_error(FLEXATTN_EINVAL, "Sq=%d is not a multiple of the q tile %d", Sq, bq);
   if (Sk % bk != 0) return set_error(FLEXATTN_EINVAL, "Sk=%d is not a multiple of the kv tile %d", Sk, bk);
@@ -161,18 +163,54 @@ static MapArgs col_view(const flexattn_block_map& m) {
   return r;
 }
 
+// Whether the bf16 dk/dv and dq kernels of this request can hand dS over through a buffer: the generated-stream
+// dk/dv kernels for plain and softcap scores write it (the position-bias streams keep the key's share of the
+// bias out of their dS, compiled-loop kernels have no export).  Looks at shapes, score and flags only.
+static bool ds_exchange_ok(const flexattn_bwd_params* p) {
+#ifdef FLEXATTN_CUSTOM_ONLY
+  (void)p;
+  return false;
+#else
+  if (p == nullptr || p->dtype != FLEXATTN_BF16 || p->D != 128) return false;
+  if ((p->flags & FLEXATTN_FLAG_COMPILED_LOOP) || p->ab.ptr != nullptr) return false;
+  if (p->score.kind != FLEXATTN_SCORE_NONE && p->score.kind != FLEXATTN_SCORE_SOFTCAP) return false;
+  if (p->B <= 0 || p->Hq <= 0 || p->Sq <= 0 || p->Sk <= 0) return false;
+  int bq = 0, bk = 0;
+  bwd_dkv_bf16_d128_tile(&bq, &bk);
+  if (p->Sq % bq != 0 || p->Sk % bk != 0) return false;
+  return p->Sq / bq <= 1024 && p->Sk / bk <= 1024;  // (both kernels cache a tile list in LDS)
+#endif
+}
+
+static int64_t ds_bytes_of(const flexattn_bwd_params* p) {
+  return (int64_t)p->B * p->Hq * (int64_t)p->Sq * (int64_t)p->Sk * 2;
+}
+
+static int check_ds(const flexattn_bwd_params* p) {
+  if (p->ds == nullptr) return FLEXATTN_OK;
+  if (!ds_exchange_ok(p))
+    return set_error(FLEXATTN_EINVAL, "ds given, but the kernels of this request exchange no dS (flexattn_bwd_ds_bytes is 0)");
+  if (p->ds_bytes < ds_bytes_of(p))
+    return set_error(FLEXATTN_EINVAL, "ds holds %lld bytes, the request needs %lld", (long long)p->ds_bytes,
+                     (long long)ds_bytes_of(p));
+  return FLEXATTN_OK;
+}
+
 static int to_bwd_args(const flexattn_bwd_params* p, int pass, BwdArgs* a) {
   if (p == nullptr) return set_error(FLEXATTN_EINVAL, "params is NULL");
   if (!p->q || !p->k || !p->v || !p->dout || !p->l || !p->m || !p->delta)
     return set_error(FLEXATTN_EINVAL, "a required input pointer is NULL");
   if (pass == FLEXATTN_PASS_DQ && !p->dq) return set_error(FLEXATTN_EINVAL, "dq is NULL");
   if (pass == FLEXATTN_PASS_DKV && (!p->dk || !p->dv)) return set_error(FLEXATTN_EINVAL, "dk or dv is NULL");
-  int rc = check_shape(pass, p->B, p->Hq, p->Hkv, p->Sq, p->Sk, p->D, p->dtype, p->map);
+  int rc = check_ds(p);
+  if (rc != FLEXATTN_OK) return rc;
+  rc = check_shape(pass, p->B, p->Hq, p->Hkv, p->Sq, p->Sk, p->D, p->dtype, p->map, p->ds ? FLEXATTN_PASS_DKV : -1);
   if (rc != FLEXATTN_OK) return rc;
   if ((rc = check_scale_flags(p->sm_scale, p->flags)) != FLEXATTN_OK) return rc;
   if ((rc = check_score(p->score)) != FLEXATTN_OK) return rc;
   if ((rc = check_mask(p->mask)) != FLEXATTN_OK) return rc;
   if ((rc = check_bias(p->ab, p->B, p->Hq, p->Sq, p->Sk)) != FLEXATTN_OK) return rc;
+  a->ds = p->ds;
   a->q = p->q; a->k = p->k; a->v = p->v; a->dout = p->dout;
   a->l = p->l; a->m = p->m; a->delta = p->delta;
   a->dq = p->dq; a->dk = p->dk; a->dv = p->dv;
@@ -329,11 +367,15 @@ int flexattn_bwd_delta(const void* o, const void* dout, float* delta, int64_t ro
   return bwd_delta(o, dout, delta, rows, D, dtype, static_cast<hipStream_t>(stream));
 }
 
+int64_t flexattn_bwd_ds_bytes(const flexattn_bwd_params* p) { return ds_exchange_ok(p) ? ds_bytes_of(p) : 0; }
+
 int flexattn_bwd_dq(const flexattn_bwd_params* p, void* stream) {
   BwdArgs a;
   int rc = to_bwd_args(p, FLEXATTN_PASS_DQ, &a);
   if (rc != FLEXATTN_OK) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (p->ds != nullptr)  // (checked: bf16 and a plain or softcap score; the softcap streams leave 4 out of dS)
+    return bwd_dq_from_ds(a, (p->score.kind == FLEXATTN_SCORE_SOFTCAP ? 4.f : 1.f) * p->sm_scale, s);
   if (p->dtype == FLEXATTN_BF16) return bwd_dq_bf16_d128(a, s);
   return (a.flags & FLEXATTN_FLAG_COMPILED_LOOP) ? bwd_dq_f32(a, p->D, s) : bwd_dq_f32_mfma(a, p->D, s);
 }

@@ -47,6 +47,7 @@ namespace fa {
 namespace dkv_cfg {
 constexpr int BNK = 128;  // kv rows per work-group
 constexpr int BQ = 128;   // q rows per step (two 64-row LDS tiles)
+constexpr size_t kDsBlockBytes = (size_t)BQ * BNK * 2;  // one exported dS block
 constexpr int D = 128;
 constexpr int MAX_LIST = 1024;  // longest q tile list the plain-score kernel caches in LDS
 // (Q, dO) x 2 buffers x 2 tiles, lse x2, delta x2, run-loop tables, cached q tile list and its partial flags
@@ -324,9 +325,14 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
 // goes into dk with sm_scale.
 // DOCS: the mask compares document ids; those of a partial q tile are staged through LDS (stage_doc_ids).
 // (A template parameter: the staging code in the kernel costs the other masks registers.)
-template <int SCORE, bool DOCS>
+// EXPORT: the streams also write the step's bf16 dS (without sm_scale, as the dk product takes it) to a.ds, one
+// 32 KB block per (query head, q tile, kv tile) at ((head nq + q tile) nk + kv tile) 32 KB; inside a block wave w
+// (kv columns 32 w + L % 32) writes 1 KB per (32-row q block c, 16-row half u) at 8192 w + 1024 (2 c + u), lane L
+// its 8 values (rows 8 (e / 4) + 4 (L / 32) + e % 4 of the half) at 16 (2 (L % 32) + L / 32).  bwd_dq_ds.hip reads it.
+template <int SCORE, bool DOCS, bool EXPORT = false>
 __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs a) {
   using namespace dkv_cfg;
+  static_assert(!(EXPORT && SCORE == FLEXATTN_SCORE_ALIBI), "the position-bias streams keep the key's share out of dS");
   constexpr bool ALIBI = SCORE == FLEXATTN_SCORE_ALIBI;
   constexpr bool SOFTCAP = SCORE == FLEXATTN_SCORE_SOFTCAP;
   const float cap2 = SOFTCAP ? a.score.cap * kLog2e : 0.f;
@@ -384,6 +390,10 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     return g;
   };
   auto kv_offset = [&](const Geometry& g) { return ((size_t)g.bhk * a.Sk + (size_t)g.kb * BNK) * D; };
+  // (EXPORT) dS block of the item's kv tile against q tile 0 of the group's first query head
+  auto ds_base = [&](const Geometry& g) {
+    return static_cast<char*>(a.ds) + (((size_t)g.bhk * group) * nQ * nKb + (size_t)g.kb) * kDsBlockBytes;
+  };
   // first row of the group's first query head: (b Hq + hk group) Sq with bhk = b Hkv + hk
   auto first_row = [&](const Geometry& g) { return (size_t)g.bhk * group * a.Sq; };
 
@@ -568,6 +578,13 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     tbl[13] = (unsigned)((size_t)rowa >> 32);
     tbl[14] = (unsigned)(size_t)rowb;
     tbl[15] = (unsigned)((size_t)rowb >> 32);
+    if (EXPORT) {
+      const size_t ds0 = (size_t)ds_base(geo);
+      tbl[28] = (unsigned)ds0;
+      tbl[29] = (unsigned)(ds0 >> 32);
+      tbl[30] = (unsigned)(nQ * nKb);
+      tbl[31] = (unsigned)nKb;
+    }
   }
   const unsigned tbl_addr = (unsigned)(size_t)tbl;
 
@@ -649,6 +666,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
             tbl[26] = __builtin_bit_cast(unsigned, pre.na2);
             tbl[27] = (unsigned)(geo_n.kb * BNK + BNK / 2);
           }
+          if (EXPORT) {
+            const size_t ds_n = (size_t)ds_base(geo_n);
+            tbl[26] = (unsigned)ds_n;
+            tbl[27] = (unsigned)(ds_n >> 32);
+          }
         }
         resident = true;
       }
@@ -666,7 +688,20 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
                  [m1] "v"(km[1]), [tid4] "v"(tid4), [c2v] "v"(c2), ##__VA_ARGS__                                                \
                : "memory", "scc", "vcc", "m0", FA_DKV_RUN_SGPRS, "v67", FA_DKV_TILE_CLOBBERS CLOB_MORE)
 #define FA_DKV_ALIBI_CLOBBERS , "s101"
-    if constexpr (ALIBI) {
+#define FA_DKV_DS_CLOBBERS , "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59"
+    if constexpr (EXPORT) {
+      // dS block of step `it` (head it / n_tiles of the group, q tile qb) and the lane's place in the wave's part
+      const size_t ds_cur = (size_t)ds_base(geo) + ((size_t)(it / n_tiles) * nQ + (size_t)qb) * nKb * kDsBlockBytes;
+      const unsigned dslo = (unsigned)ds_cur, dshi = (unsigned)(ds_cur >> 32);
+      const unsigned dsv = 8192u * (unsigned)w + 4096u + 16u * (unsigned)(2 * l32 + hh);
+      if constexpr (SOFTCAP) {
+        const float k2 = -2.f * cap2;
+        FA_DKV_CALL(FA_DKV_RUN_SOFTCAP_DS, FA_DKV_ALIBI_CLOBBERS FA_DKV_DS_CLOBBERS, [k2] "v"(k2), [dslo] "v"(dslo),
+                    [dshi] "v"(dshi), [dsv] "v"(dsv));
+      } else {
+        FA_DKV_CALL(FA_DKV_RUN_DS, FA_DKV_DS_CLOBBERS, [dslo] "v"(dslo), [dshi] "v"(dshi), [dsv] "v"(dsv));
+      }
+    } else if constexpr (ALIBI) {
       FA_DKV_CALL(FA_DKV_RUN_ALIBI, FA_DKV_ALIBI_CLOBBERS, [kc] "v"(kc));
     } else if constexpr (SOFTCAP) {
       const float k2 = -2.f * cap2;
@@ -675,6 +710,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
       FA_DKV_CALL(FA_DKV_RUN, );
     }
 #undef FA_DKV_CALL
+#undef FA_DKV_DS_CLOBBERS
 #undef FA_DKV_ALIBI_CLOBBERS
     it = __builtin_amdgcn_readfirstlane(it);
     p1 = __builtin_amdgcn_readfirstlane(p1);
@@ -752,10 +788,10 @@ static int launch_dkv(const BwdArgs& a, hipStream_t stream) {
 }
 
 #ifndef FLEXATTN_CUSTOM_ONLY
-template <int SCORE, bool DOCS>
+template <int SCORE, bool DOCS, bool EXPORT>
 static int launch_dkv_plain_on(const BwdArgs& a, hipStream_t stream) {
   using namespace dkv_cfg;
-  auto kern = bwd_dkv_bf16_d128_plain_kernel<SCORE, DOCS>;
+  auto kern = bwd_dkv_bf16_d128_plain_kernel<SCORE, DOCS, EXPORT>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(dkv): %s", hipGetErrorString(attr));
@@ -770,8 +806,13 @@ static int launch_dkv_plain_on(const BwdArgs& a, hipStream_t stream) {
 
 template <int SCORE>
 static int launch_dkv_plain(const BwdArgs& a, hipStream_t stream) {
-  return (a.mask.flags & FLEXATTN_MASK_DOC) ? launch_dkv_plain_on<SCORE, true>(a, stream)
-                                            : launch_dkv_plain_on<SCORE, false>(a, stream);
+  if constexpr (SCORE != FLEXATTN_SCORE_ALIBI) {
+    if (a.ds != nullptr)
+      return (a.mask.flags & FLEXATTN_MASK_DOC) ? launch_dkv_plain_on<SCORE, true, true>(a, stream)
+                                                : launch_dkv_plain_on<SCORE, false, true>(a, stream);
+  }
+  return (a.mask.flags & FLEXATTN_MASK_DOC) ? launch_dkv_plain_on<SCORE, true, false>(a, stream)
+                                            : launch_dkv_plain_on<SCORE, false, false>(a, stream);
 }
 
 #endif  // FLEXATTN_CUSTOM_ONLY

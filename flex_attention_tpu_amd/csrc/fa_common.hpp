@@ -83,6 +83,7 @@ struct BwdArgs {
   const void* q; const void* k; const void* v; const void* dout;
   const float* l; const float* m; const float* delta;
   void* dq; void* dk; void* dv;
+  void* ds;   // dS exchange buffer (bf16 kernels that can use one), or null
   int B, Hq, Hkv, Sq, Sk;
   float sm_scale;
   int flags;  // FLEXATTN_FLAG_*

@@ -63,6 +63,7 @@ LOAD_COST = 3    # share of an MFMA gap one of them takes
 LDS_COST = 1     # share of an MFMA gap an LDS read takes
 TRANS_COST = 2   # share of an MFMA gap a transcendental takes (it holds the wave's issue for two slots)
 DROP = ()        # instruction classes left out (--drop, timing studies only)
+DS_COST = 3      # share of an MFMA gap a dS store takes
 
 TILE = 16384
 # Scalar registers owned by the run loop (all clobbered).  The compiler hands scalars to an asm
@@ -89,6 +90,11 @@ S_KC = "s101"     # (position-bias variant) 128 kb + 64: the middle of the item'
 # ds'/ds = 1 - tanh^2 = 4 r (1 - r), whose factor 4 the epilogue applies to dk.
 S_CAP, S_K2 = "s64", "s101"
 CAP_SOFTCAP = 8   # instructions per MFMA gap in the softcap variant (8 VALU ops per element instead of 2)
+# dS export variant: the step's bf16 dS (the B operand registers of the dk product) also goes to a buffer in
+# global memory, one 32 KB block per (query head, q tile, kv tile), from which the dq pass takes it.  Block of
+# the step: item base + ((head inside the group) nq nk + (q tile) nk) 32 KB; wave w writes bytes [8192 w, + 8192),
+# 1 KB per (q block c, half u) at (2 c + u) 1024, lane L at 16 (2 (L % 32) + L / 32).
+S_DSB, S_NQNK, S_NK, S_DS, S_DSN = "s[52:53]", "s54", "s55", "s[56:57]", "s[58:59]"
 V_QB2 = 67      # q block index of the step after the next one, across the stream
 ROW_SLOT = 28   # MFMA slot at which the next step's lse / delta values are turned around
 V_ROW = 144     # 4 temporaries for that, inside pb[1] (first written by E(1), after ROW_SLOT)
@@ -103,7 +109,7 @@ V_TMP = 68    # 4 temporaries of the masked variant
 DL_OFFSET = 1024
 
 
-def build(masked, alibi=False, softcap=False):
+def build(masked, alibi=False, softcap=False, export=False):
     em = Emitter()
     em.wait_old = WAIT_OLD
 
@@ -187,6 +193,18 @@ def build(masked, alibi=False, softcap=False):
 
     chains = []
     e_chains = []
+    state = {"direct": 0, "stores_behind": 0}
+
+    def ds_store(c, u, reg):
+        # One 16-byte store per lane and 16-row half, once the half's second group is converted.  (Measured: a store
+        # costs the wave about 46 cycles of issue whatever its cache policy bits; two 8-byte stores per half cost more.)
+        def emit(e):
+            if "vmem" in DROP:
+                return
+            e.vmem_store(f"global_store_dwordx4 %[dsv], {vr(reg, 4)}, {S_DS} offset:{(2 * c + u) * 1024 - 4096}", vset(reg, 4))
+            state["direct"] += 1
+            state["stores_behind"] += 1
+        return Op(emit, cost=DS_COST, deadline=n_mfma)
 
     def lse_read(c, g):
         return lds(f"ds_read_b128 {vr(V_LSE + 4 * g, 4)}, %[la] offset:{(32 * c + 8 * g) * 4}", vset(V_LSE + 4 * g, 4))
@@ -255,9 +273,12 @@ def build(masked, alibi=False, softcap=False):
                                 earliest=war, deadline=first_B[(c, u2)] - 1))
                 ops.append(valu(f"v_cvt_pk_bf16_f32 {vr(dsb + h)}, {vr(dp + e)}, {vr(dp + e + 1)}", vset(dsb + h), vset(dp + e, 2),
                                 earliest=war, deadline=first_B[(c, u2)] - 1))
+            if export and (g & 1):
+                ops.append(ds_store(c, u2, V_DSB + 8 * (c & 1) + 4 * u2))
         ops[0].earliest = last_A[c] + 4            # the chains' last results need 12 wait states
         if c + 2 < 4:
-            ops[-1].deadline = min(ops[-1].deadline, first_A[c + 2])  # A(c + 2) writes the same S / dP registers
+            last_cvt = ops[-2] if export else ops[-1]
+            last_cvt.deadline = min(last_cvt.deadline, first_A[c + 2])  # A(c + 2) writes the same S / dP registers
         e_chains.append(ops)
     # one chain: block c + 1 must not read its row values before block c has put them there
     chains.append([op for ops in e_chains for op in ops])
@@ -292,7 +313,8 @@ def build(masked, alibi=False, softcap=False):
 
     # ---- next step's Q / dO tiles: 16 LDS-direct loads per wave spread over the stream ----------
     # (issued back to back they hold the wave for about a thousand cycles: one CU moves 64 B / clk)
-    state = {"direct": 0}
+    # (vector-memory operations complete in issue order: one count of those issued so far, and the text index of
+    # the last LDS-direct load, behind which only dS stores are open at the end of the stream)
 
     # (M0 of load k + 1 is written behind load k; the loop top writes the first one's)
     def direct(k, goff, gbase):
@@ -303,6 +325,7 @@ def build(masked, alibi=False, softcap=False):
                 return
             e.lds_direct_load_chained(goff, gbase, nxt, S_LDSN)
             state["direct"] += 1
+            state["stores_behind"] = 0
         return emit
 
     vm = []
@@ -353,10 +376,13 @@ def build(masked, alibi=False, softcap=False):
 
     schedule(em, mfmas, chains, CAP_SOFTCAP if softcap else CAP)
     em.drain()
+    if export:
+        # the step's copies have landed once only the stores issued behind the last of them are open
+        em.raw(f"s_waitcnt vmcnt({state['stores_behind']})")
     return em
 
 
-def run_loop(full, masked, alibi=False, softcap=False):
+def run_loop(full, masked, alibi=False, softcap=False, export=False):
     """One asm statement: a run of consecutive steps [it, it_end) of one work-group, all full or a
     single partial one.  At entry the step's Q / dO tiles and row values are resident in LDS buffer
     s81; each pass computes the next step's addresses, streams the tile (which copies the next
@@ -371,8 +397,21 @@ def run_loop(full, masked, alibi=False, softcap=False):
         entry += [f"v_readfirstlane_b32 {S_KC}, %[kc]"]
     if softcap:
         entry += [f"v_readfirstlane_b32 {S_K2}, %[k2]"]
-    switch = ([f"ds_read_b64 {vr(V_TBL + 10, 2)}, %[tbl] offset:104"] if alibi else [])
+    assert not (alibi and export)
+    switch = ([f"ds_read_b64 {vr(V_TBL + 10, 2)}, %[tbl] offset:104"] if alibi or export else [])
     switch_sgprs = ([f"v_readfirstlane_b32 s64, {vr(V_TBL + 10)}", f"v_readfirstlane_b32 {S_KC}, {vr(V_TBL + 11)}"] if alibi else [])
+    ds_next = []
+    if export:
+        # table dwords 28-31: the item's first dS block (two dwords), blocks per head nq nk, blocks per q tile nk;
+        # dwords 26, 27: the next item's first dS block; %[dslo], %[dshi]: the block of the run's first step
+        entry = ([f"ds_read_b128 {vr(V_TBL + 16, 4)}, %[tbl] offset:112"] + entry
+                 + [f"v_readfirstlane_b32 s{52 + i}, {vr(V_TBL + 16 + i)}" for i in range(4)]
+                 + ["v_readfirstlane_b32 s56, %[dslo]", "v_readfirstlane_b32 s57, %[dshi]"])
+        switch_sgprs = [f"v_readfirstlane_b32 s52, {vr(V_TBL + 10)}", f"v_readfirstlane_b32 s53, {vr(V_TBL + 11)}"]
+        # dS block of the next step: item base + (min(g1, gmax) nq nk + qb1 nk) 32 KB
+        ds_next = [f"s_min_u32 {t0}, s78, s61", f"s_mul_i32 {t0}, {t0}, {S_NQNK}", f"s_mul_i32 {t1}, s80, {S_NK}",
+                   f"s_add_u32 {t0}, {t0}, {t1}", f"s_lshl_b32 {t2}, {t0}, 15", f"s_lshr_b32 {t3}, {t0}, 17",
+                   f"s_add_u32 s58, s52, {t2}", f"s_addc_u32 s59, s53, {t3}"]
     top = entry + [
         ".Lfa_dkv_loop_%=:",
         # The last step of the run that ends an item (bit 1 of the flags) copies the next item's first
@@ -391,6 +430,7 @@ def run_loop(full, masked, alibi=False, softcap=False):
         f"v_readfirstlane_b32 s80, {vr(V_TBL + 8)}",
         "s_mov_b32 s78, 0",
         ".Lfa_dkv_same_%=:",
+    ] + ds_next + [
         # row of the next step relative to the first head of the group: min(g1, gmax) Sq + 128 qb1
         f"s_min_u32 {t0}, s78, s61",
         f"s_mul_i32 {t0}, {t0}, s62",
@@ -424,8 +464,10 @@ def run_loop(full, masked, alibi=False, softcap=False):
     ]
     tail = [
         ".Lfa_dkv_tail_%=:",
-        "s_waitcnt vmcnt(0) lgkmcnt(0)",
+        # (dS stores issued behind the step's last copy may stay open: the streams wait for the copies themselves)
+        "s_waitcnt lgkmcnt(0)" if export else "s_waitcnt vmcnt(0) lgkmcnt(0)",
         "s_barrier",
+    ] + (["s_mov_b64 s[56:57], s[58:59]"] if export else []) + [
         "s_add_u32 s76, s76, 1",
         f"v_readfirstlane_b32 s80, {vr(V_QB2)}",
         "s_add_u32 s77, s77, 1",
@@ -460,9 +502,10 @@ def main():
         # one statement for both kinds of tile: a second asm statement on another control-flow
         # path makes the compiler shuffle the pinned registers around each of them
         full, masked = build(False), build(True)
-        for name, alibi, softcap in (("FA_DKV_RUN", False, False), ("FA_DKV_RUN_ALIBI", True, False),
-                                     ("FA_DKV_RUN_SOFTCAP", False, True)):
-            lines = run_loop(build(False, alibi, softcap), build(True, alibi, softcap), alibi, softcap)
+        for name, alibi, softcap, export in (("FA_DKV_RUN", False, False, False), ("FA_DKV_RUN_ALIBI", True, False, False),
+                                             ("FA_DKV_RUN_SOFTCAP", False, True, False), ("FA_DKV_RUN_DS", False, False, True),
+                                             ("FA_DKV_RUN_SOFTCAP_DS", False, True, True)):
+            lines = run_loop(build(False, alibi, softcap, export), build(True, alibi, softcap, export), alibi, softcap, export)
             f.write(f"#define {name} \\\n")
             f.write(" \\\n".join(f'  "{line}\\n"' for line in lines))
             f.write("\n\n")

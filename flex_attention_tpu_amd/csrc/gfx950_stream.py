@@ -198,6 +198,15 @@ class Emitter:
         if next_imm is not None:
             self.lds_direct_dest(next_imm, ldsn)
 
+    def vmem_store(self, text, src_regs):
+        """A store to global memory from VGPRs (it joins the in-order vector-memory queue)."""
+        self._wait_lds(src_regs)
+        for r in src_regs:
+            if r in self.mfma_w:
+                self._need_gap(self.mfma_w[r], self.mfma_lat.get(r, 12))
+        self._raw(text)
+        self.stats["vmem"] = self.stats.get("vmem", 0) + 1
+
     def lds_write(self, text, src_regs):
         """An LDS store: takes a place in the in-order LDS queue like a read."""
         self._wait_lds(src_regs)

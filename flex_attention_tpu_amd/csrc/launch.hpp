@@ -19,6 +19,9 @@ int bwd_dq_bf16_d128(const BwdArgs& a, hipStream_t stream);
 void bwd_dq_bf16_d128_tile(int* bq, int* bk);
 int bwd_dkv_bf16_d128(const BwdArgs& a, hipStream_t stream);
 void bwd_dkv_bf16_d128_tile(int* bq, int* bk);
+// dq = out_scale dS K from the dS blocks that the dk/dv stream kernels wrote to a.ds (a.map: row lists at the
+// dk/dv tiles)
+int bwd_dq_from_ds(const BwdArgs& a, float out_scale, hipStream_t stream);
 
 // fp32, head dim 64 or 128 (FMA kernels, exact-arithmetic path)
 int fwd_f32(const FwdArgs& a, int D, hipStream_t stream);

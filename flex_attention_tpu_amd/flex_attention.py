@@ -20,6 +20,11 @@ from .flex_attention_dq_bwd import compute_delta, flex_attention_bwd_dq
 from .flex_attention_kernel import _flex_attention_impl
 
 
+# The backward hands dS from the dk/dv pass to the dq pass (DsBlocks in flex_attention_dq_bwd.py) when both
+# gradients are wanted and the buffer, B Hq Sq Sk bf16 values, stays below this many bytes.
+DS_EXCHANGE_MAX_BYTES = 32 << 30
+
+
 class _FlexAttention(torch.autograd.Function):
     """o = softmax(mask(score_mod(sm_scale q k^T))) v with the saved statistics (l, m) for the backward."""
 
@@ -39,16 +44,24 @@ class _FlexAttention(torch.autograd.Function):
         score_fn, mask_fn, block_mask_fn, segment_ids, causal, sm_scale, block_q, block_k, ab = ctx.opts
         do = do.contiguous()
         di = compute_delta(o, do)  # float32 [B, H, Sq]  (jax_exp.py:276-278)
-        dq = dk = dv = None
+        dq = dk = dv = ds = None
         if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
-            dk, dv = flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, block_b=1, block_q=block_q,
-                                             block_q_major=block_q, block_k_major=block_k, block_k=block_k,
-                                             sm_scale=sm_scale, causal=causal, debug=False, score_fn=score_fn,
-                                             mask_fn=mask_fn, block_mask_fn=block_mask_fn)
+            pad = lambda n: -(-n // 128) * 128
+            exchange = (ctx.needs_input_grad[0] and
+                        2 * q.shape[0] * q.shape[1] * pad(q.shape[2]) * pad(k.shape[2]) <= DS_EXCHANGE_MAX_BYTES)
+            dk, dv, ds = flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, block_b=1, block_q=block_q,
+                                                 block_q_major=block_q, block_k_major=block_k, block_k=block_k,
+                                                 sm_scale=sm_scale, causal=causal, debug=False, score_fn=score_fn,
+                                                 mask_fn=mask_fn, block_mask_fn=block_mask_fn, return_ds=True) \
+                if exchange else (*flash_attention_bwd_dkv(
+                    k, v, q, ab, segment_ids, l, m, di, do, block_b=1, block_q=block_q, block_q_major=block_q,
+                    block_k_major=block_k, block_k=block_k, sm_scale=sm_scale, causal=causal, debug=False,
+                    score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn), None)
         if ctx.needs_input_grad[0]:
             dq = flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, di, block_b=1, block_q=block_q,
                                        block_k_major=block_k, block_k=block_k, sm_scale=sm_scale, debug=False,
-                                       score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn, causal=causal)
+                                       score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn, causal=causal,
+                                       ds=ds)
         return dq, dk, dv, None
 
 

@@ -10,17 +10,19 @@ import torch
 from . import _lib
 from ._common import (batch_entry, bias_c, check_blocks, check_qkv, check_rows, kernel_block_map, kernel_head_dim, library_for, pad_seq,
                       padded_len, per_batch_segments, resolve_mask, stream_of)
-from .flex_attention_dq_bwd import bwd_params
+from .flex_attention_dq_bwd import DsBlocks, bwd_params
 
 
 def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=None, block_q, block_q_major,
                             block_k_major, block_k, sm_scale, causal, debug, score_fn=None, mask_fn=None,
-                            block_mask_fn=None, compiled_loop=False):
+                            block_mask_fn=None, compiled_loop=False, return_ds=False):
     """(dk, dv): dv = P^T do, dk = dS^T * d(score)/dk with P recomputed from (l, m) and
     dS = P (dP - di) (flex_attention_dkv_kernel.py:237-272).  With grouped KV heads the gradients
     of all query heads of a group are summed inside the kernel.  ``causal`` is honoured
     (the reference's north-star file ignores it; its mask-aware twin gets the same effect from
-    ``mask_fn``)."""
+    ``mask_fn``).  ``return_ds=True`` returns (dk, dv, ds): ds is the pass's dS as a DsBlocks for
+    ``flex_attention_bwd_dq(..., ds=ds)``, or None when the kernels of the call exchange nothing (fp32, position
+    biases, ``ab``, compiled score functions): the dq pass then recomputes as usual."""
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v, do)
     rows = per_batch_segments(segment_ids, B)
     if rows is not None:  # ids differ between batch entries: one launch per entry
@@ -28,8 +30,11 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
             k[b:b + 1], v[b:b + 1], q[b:b + 1], batch_entry(ab, b), rows[b], l[b:b + 1], m[b:b + 1], di[b:b + 1], do[b:b + 1],
             block_b=block_b, block_q=block_q, block_q_major=block_q_major, block_k_major=block_k_major, block_k=block_k,
             sm_scale=sm_scale, causal=causal, debug=debug, score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn,
-            compiled_loop=compiled_loop) for b in range(B)]
-        return torch.cat([x[0] for x in outs], 0), torch.cat([x[1] for x in outs], 0)
+            compiled_loop=compiled_loop, return_ds=return_ds) for b in range(B)]
+        dk, dv = torch.cat([x[0] for x in outs], 0), torch.cat([x[1] for x in outs], 0)
+        if not return_ds:
+            return dk, dv
+        return dk, dv, (DsBlocks(entries=[x[2] for x in outs]) if all(x[2] is not None for x in outs) else None)
     for name, t in (("l", l), ("m", m), ("di", di)):
         check_rows(name, t, B, Hq, Sq, q.device)
     check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k,
@@ -47,9 +52,15 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     ab_c, ab_keep = bias_c(ab, B, Hq, Sq, Sk, Sq_p, Sk_p, q.device)
     p = bwd_params(q, k, v, l, m, do, di, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dk=dk, dv=dv,
                    compiled_loop=compiled_loop, ab_c=ab_c)
+    ds = None
     with torch.cuda.device(q.device):
         lib = library_for(score_fn, spec)
+        if return_ds:
+            need = lib.flexattn_bwd_ds_bytes(C.byref(p))
+            if need > 0:
+                ds = DsBlocks(torch.empty(need, dtype=torch.uint8, device=q.device), (B, Hq, Sq_p, Sk_p))
+                p.ds, p.ds_bytes = ds.buf.data_ptr(), need
         _lib.check(lib.flexattn_bwd_dkv(C.byref(p), stream_of(q)), lib)
     if Sk_p != Sk or D != D_user:
         dk, dv = dk[:, :, :Sk, :D_user].contiguous(), dv[:, :, :Sk, :D_user].contiguous()
-    return dk, dv
+    return (dk, dv, ds) if return_ds else (dk, dv)

@@ -30,6 +30,16 @@ def compute_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
     return d
 
 
+class DsBlocks:
+    """dS of one dk/dv pass, as ``flash_attention_bwd_dkv(..., return_ds=True)`` leaves it for
+    ``flex_attention_bwd_dq(..., ds=...)``: bf16 values in the kernels' own block layout, opaque to callers.
+    The reference's two backward kernels each recompute S, dP and dS (flex_attention_dq_bwd.py:340-378,
+    flash_attention_dkv_bwd.py:232-302); handing dS over leaves the dq pass one contraction instead of three."""
+
+    def __init__(self, buf=None, shape=None, entries=None):
+        self.buf, self.shape, self.entries = buf, shape, entries
+
+
 def bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, mod_q, mod_k, dq=None, dk=None, dv=None,
                compiled_loop=False, ab_c=None):
     B, Hq, Sq, D = q.shape
@@ -45,18 +55,22 @@ def bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, mod_q, mod_k,
 
 def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, block_q, block_k_major,
                           block_k, sm_scale, debug, score_fn=None, mask_fn=None, block_mask_fn=None,
-                          causal=False, compiled_loop=False):
+                          causal=False, compiled_loop=False, ds=None):
     """dq = sum_j dS_ij * d(score)/dq, with P_ij = exp(S_ij - m_i) / l_i recomputed from the saved
     statistics, dP = do v^T, dS = P (dP - d) (flex_attention_dq_bwd.py:340-378).  ``o`` is only
-    shape-checked, as in the reference (:163); ``d`` is the caller's delta (see compute_delta)."""
+    shape-checked, as in the reference (:163); ``d`` is the caller's delta (see compute_delta).
+    ``ds``: the DsBlocks of the dk/dv pass of the same arguments, if that pass returned one: dq is then
+    sm_scale dS K, nothing is recomputed."""
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v, do)
     rows = per_batch_segments(segment_ids, B)
     if rows is not None:  # ids differ between batch entries: one launch per entry
+        if ds is not None and (ds.entries is None or len(ds.entries) != B):
+            raise ValueError("ds does not come from a dk/dv pass of these arguments")
         return torch.cat([flex_attention_bwd_dq(
             q[b:b + 1], k[b:b + 1], v[b:b + 1], batch_entry(ab, b), rows[b], l[b:b + 1], m[b:b + 1], batch_entry(o, b),
             do[b:b + 1], d[b:b + 1], block_b=block_b, block_q=block_q, block_k_major=block_k_major, block_k=block_k,
             sm_scale=sm_scale, debug=debug, score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn, causal=causal,
-            compiled_loop=compiled_loop) for b in range(B)], 0)
+            compiled_loop=compiled_loop, ds=ds.entries[b] if ds is not None else None) for b in range(B)], 0)
     if o is not None and tuple(o.shape) != tuple(q.shape):
         raise ValueError(f"o has shape {tuple(o.shape)}, expected {tuple(q.shape)}")
     for name, t in (("l", l), ("m", m), ("d", d)):
@@ -69,11 +83,16 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     l, m, d = pad_seq(l, Sq_p), pad_seq(m, Sq_p), pad_seq(d, Sq_p)
     D_user, D = D, kernel_head_dim(D, q.dtype)   # smaller head dimensions: zero-padded columns
     q, do, k, v = pad_seq(q, D, 3), pad_seq(do, D, 3), pad_seq(k, D, 3), pad_seq(v, D, 3)
-    bm = kernel_block_map(_lib.PASS_DQ, spec, q, Sq_p, Sk_p, D, score_fn)
+    if ds is not None and (ds.buf is None or ds.shape != (B, Hq, Sq_p, Sk_p) or ds.buf.device != q.device):
+        raise ValueError("ds does not come from a dk/dv pass of these arguments")
+    # (the dS blocks lie at the dk/dv kernel's tiles: the dq pass walks that map's row lists)
+    bm = kernel_block_map(_lib.PASS_DKV if ds is not None else _lib.PASS_DQ, spec, q, Sq_p, Sk_p, D, score_fn)
     dq = torch.empty_like(q)
     ab_c, ab_keep = bias_c(ab, B, Hq, Sq, Sk, Sq_p, Sk_p, q.device)
     p = bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dq=dq,
                    compiled_loop=compiled_loop, ab_c=ab_c)
+    if ds is not None:
+        p.ds, p.ds_bytes = ds.buf.data_ptr(), ds.buf.numel()
     with torch.cuda.device(q.device):
         lib = library_for(score_fn, spec)
         _lib.check(lib.flexattn_bwd_dq(C.byref(p), stream_of(q)), lib)

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FLEXATTN_VERSION 101 /* major*10000 + minor*100 + patch */
+#define FLEXATTN_VERSION 102 /* major*10000 + minor*100 + patch */
 
 /* status codes */
 #define FLEXATTN_OK 0
@@ -136,6 +136,9 @@ typedef struct flexattn_bwd_params {
   flexattn_mask_spec mask;
   flexattn_block_map map; /* granularity of the pass being launched */
   flexattn_bias ab;
+  /* dS exchange buffer, or NULL (see flexattn_bwd_ds_bytes): written by flexattn_bwd_dkv, read by flexattn_bwd_dq */
+  void* ds;
+  int64_t ds_bytes;
 } flexattn_bwd_params;
 
 #define FLEXATTN_PASS_FWD 0
@@ -189,6 +192,18 @@ int flexattn_fwd_noalloc(const flexattn_fwd_params* p, void* stream);
  * flex_attention_dq_bwd.py:932 and flash_attention_dkv_bwd.py:925.  rows = B*Hq*Sq. */
 int flexattn_bwd_delta(const void* o, const void* dout, float* delta, int64_t rows, int32_t D,
                        int32_t dtype, void* stream);
+
+/* dS exchange between the two backward passes.  The reference's dq and dk/dv kernels each recompute S, dP and dS
+ * (flex_attention_dq_bwd.py:340-378, flash_attention_dkv_bwd.py:232-302).  Here the dk/dv pass can leave its
+ * bf16 dS in a caller-allocated device buffer `ds`, and a dq pass that is given the same buffer computes
+ * dq = sm_scale dS K from it, one contraction instead of three.  Returns the bytes `ds` must hold for the request
+ * described by p (B Hq Sq Sk 2; only shapes, dtype, D, flags, score and ab are looked at), or 0 when the
+ * kernels of the request exchange nothing (fp32, position biases, an additive bias, compiled score functions,
+ * FLEXATTN_FLAG_COMPILED_LOOP, more than 1024 tiles along a sequence): then ds must stay NULL.
+ * Order: flexattn_bwd_dkv with p->ds set, then flexattn_bwd_dq with the same p->ds on the same stream (or
+ * ordered behind it); for that dq call p->map is the map at the granularity of FLEXATTN_PASS_DKV with its
+ * kv_cnt / kv_idx lists.  With ds == NULL both passes work on their own as before. */
+int64_t flexattn_bwd_ds_bytes(const flexattn_bwd_params* p);
 
 /* dq backward.  Replaces the pallas_call in flex_attention_bwd_dq (flex_attention_dq_bwd.py:251-265). */
 int flexattn_bwd_dq(const flexattn_bwd_params* p, void* stream);

@@ -222,7 +222,7 @@ def test_compiler_keeps_out_of_the_pinned_registers(tmp_path):
                         "-o", str(asm)], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr
     text = asm.read_text().split("\n")
-    start = next(i for i, l in enumerate(text) if l.startswith("_ZN2fa30bwd_dkv_bf16_d128_plain_kernelILi0ELb0E"))  # (the plain-score instantiation)
+    start = next(i for i, l in enumerate(text) if l.startswith("_ZN2fa30bwd_dkv_bf16_d128_plain_kernelILi0ELb0ELb0E"))  # (plain score, no document ids, no dS export)
     end = next(i for i, l in enumerate(text) if i > start and l.strip() == "s_endpgm")
     in_asm = False
     for line in text[start:end]:

@@ -37,7 +37,7 @@ def test_struct_sizes_follow_c_layout():
     assert C.sizeof(_lib.BlockMapC) == 56
     assert C.sizeof(_lib.BiasC) == 32
     assert C.sizeof(_lib.FwdParamsC) == 6 * 8 + 10 * 4 + 32 + 32 + 56 + 32
-    assert C.sizeof(_lib.BwdParamsC) == 10 * 8 + 10 * 4 + 32 + 32 + 56 + 32
+    assert C.sizeof(_lib.BwdParamsC) == 10 * 8 + 10 * 4 + 32 + 32 + 56 + 32 + 16
 
 
 def test_tile_shapes(lib):
@@ -79,3 +79,37 @@ def test_error_codes_and_messages(lib):
         _lib.check(_lib.ENOTSUP)
     with pytest.raises(ValueError):
         _lib.check(_lib.EINVAL)
+
+
+def test_ds_exchange_sizes_and_argument_checks(lib):
+    """flexattn_bwd_ds_bytes looks at shapes, dtype, score and flags only; a dS buffer on a request whose kernels
+    exchange nothing, or one that is too small, is refused before any launch."""
+    dummy = C.create_string_buffer(64)
+    p = _lib.BwdParamsC()
+    p.B, p.Hq, p.Hkv, p.Sq, p.Sk, p.D, p.dtype, p.sm_scale = 2, 4, 2, 256, 384, 128, _lib.BF16, 0.125
+    assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 2 * 4 * 256 * 384 * 2
+    p.score.kind = _lib.SCORE_SOFTCAP
+    assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 2 * 4 * 256 * 384 * 2
+    for kind in (_lib.SCORE_ALIBI, _lib.SCORE_ALIBI_TILE):
+        p.score.kind = kind
+        assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 0
+    p.score.kind = _lib.SCORE_NONE
+    p.flags = _lib.FLAG_COMPILED_LOOP
+    assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 0
+    p.flags, p.dtype = 0, _lib.F32
+    assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 0
+    p.dtype, p.Sq = _lib.BF16, 200          # not a multiple of the dk/dv tile
+    assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 0
+    p.Sq = 1025 * 128                       # more than 1024 tiles along a sequence
+    assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 0
+    assert lib.flexattn_bwd_ds_bytes(None) == 0
+    # a buffer where none is exchanged, and one that is too small
+    p.Sq, p.dtype = 256, _lib.F32
+    for f in ("q", "k", "v", "dout", "l", "m", "delta", "dq", "dk", "dv", "ds"):
+        setattr(p, f, C.addressof(dummy))
+    p.ds_bytes = 1 << 40
+    for call in (lib.flexattn_bwd_dq, lib.flexattn_bwd_dkv):
+        assert call(C.byref(p), None) == _lib.EINVAL and b"exchange no dS" in lib.flexattn_last_error_string()
+    p.dtype, p.ds_bytes = _lib.BF16, 2 * 4 * 256 * 384 * 2 - 1
+    for call in (lib.flexattn_bwd_dq, lib.flexattn_bwd_dkv):
+        assert call(C.byref(p), None) == _lib.EINVAL and b"needs" in lib.flexattn_last_error_string()

@@ -36,16 +36,28 @@ def _fwd(F, q, k, v, sc, mf, bf, score_fn, causal=False, blk=128):
     return F._flex_attention_impl(q, k, v, None, None, True, causal, sc, 1, blk, blk, blk, False, bf, mf, score_fn)
 
 
-def _dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, score_fn, causal=False, blk=128):
-    return F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=blk, block_k_major=blk,
+def _dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, score_fn, causal=False, blk=128, ds=None, sid=None):
+    return F.flex_attention_bwd_dq(q, k, v, None, sid, l, m, o, do, d, block_b=1, block_q=blk, block_k_major=blk,
                                    block_k=blk, sm_scale=sc, debug=False, score_fn=score_fn, mask_fn=mf,
-                                   block_mask_fn=bf, causal=causal)
+                                   block_mask_fn=bf, causal=causal, ds=ds)
 
 
-def _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, score_fn, causal=False, blk=128):
-    return F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=blk, block_q_major=blk,
+def _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, score_fn, causal=False, blk=128, return_ds=False, sid=None):
+    return F.flash_attention_bwd_dkv(k, v, q, None, sid, l, m, d, do, block_b=1, block_q=blk, block_q_major=blk,
                                      block_k_major=blk, block_k=blk, sm_scale=sc, causal=causal, debug=False,
-                                     score_fn=score_fn, mask_fn=mf, block_mask_fn=bf)
+                                     score_fn=score_fn, mask_fn=mf, block_mask_fn=bf, return_ds=return_ds)
+
+
+def _exchanged_dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, score_fn, dk, dv, expect, causal=False, sid=None):
+    """The backward with dS handed from the dk/dv pass to the dq pass: dk, dv must be the bits of the pass
+    without the export; returns that dq (None where the kernels of the call exchange nothing, which
+    must be exactly where `expect` says so)."""
+    dk2, dv2, ds = _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, score_fn, causal=causal, return_ds=True, sid=sid)
+    assert torch.equal(dk2, dk) and torch.equal(dv2, dv), "dk, dv change when dS is exported"
+    assert (ds is not None) == expect, "dS exchange offered" if ds is not None else "no dS exchange offered"
+    if ds is None:
+        return None
+    return _dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, score_fn, causal=causal, ds=ds, sid=sid)
 
 
 def _check_grads(got, chain_ref, q, k, v, do, o, l, m, dtype, okw, tag=""):
@@ -161,6 +173,11 @@ def test_small_shapes_all_passes(F, case, dtype):
     dq = _dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, score_fn)
     dk, dv = _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, score_fn)
     _check_grads((dq, dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, dtype, dict(sm_scale=sc, **okw))
+    # dS exchange: the bf16 stream kernels of plain and softcap scores offer it
+    dqx = _exchanged_dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, score_fn, dk, dv,
+                        expect=dtype == torch.bfloat16 and not name.startswith("alibi"))
+    if dqx is not None:
+        _check_grads((dqx, dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, dtype, dict(sm_scale=sc, **okw), tag="exchange ")
 
 
 def test_causal_flag_and_segment_ids_arguments(F):
@@ -259,6 +276,12 @@ def test_segment_ids_per_batch_entry(F, dtype):
     ma = O.mha_bwd_reference(q, k, v, o.float().cpu(), do, l.cpu(), m.cpu(), **okw)
     for name, t, r in (("dq", dq, ma[0]), ("dk", dk, ma[1]), ("dv", dv, ma[2])):
         assert_close(name, t, r, dtype)
+    # (the dS exchange goes entry by entry as well)
+    d = F.compute_delta(o, dog)
+    dqx = _exchanged_dq(F, qg, kg, vg, l, m, o, dog, d, sc, None, None, None, dk, dv, expect=dtype == torch.bfloat16,
+                        causal=True, sid=sid)
+    if dqx is not None:
+        assert_close("exchange dq", dqx, ma[0], dtype)
 
 
 @pytest.mark.parametrize("D,dtype", [(64, torch.bfloat16), (96, torch.bfloat16), (32, torch.float32), (80, torch.float32)],
@@ -570,7 +593,13 @@ def test_autograd_function_end_to_end(F, case):
     # .backward() accumulates into .grad; gradients only where asked for
     o2 = F.flex_attention(qg, kg.detach(), vg.detach(), sfn, mf, sm_scale=sc)
     o2.backward(do.to(DEV))
-    assert torch.equal(qg.grad, dq) and kg.grad is None
+    assert kg.grad is None
+    # (dq alone is recomputed by the dq kernel; with dk / dv wanted as well it comes from the dk/dv pass's dS where
+    # the kernels exchange it: not the same bits, the same bound)
+    sdq = same_residual_grads(q, k, v, do, o_, l_, m_, sm_scale=sc, **okw)[0]
+    assert_close("dq alone", qg.grad, sdq, dtype)
+    if case in ("alibi_window", "fp32_plain"):
+        assert torch.equal(qg.grad, dq)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
@@ -621,6 +650,11 @@ def test_ragged_sequence_lengths(F, case, dtype):
                                        score_fn=sfn, mask_fn=mf[0], block_mask_fn=mf[1])
     assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
     _check_grads((dq, dk, dv), (rdq, rdk, rdv), q, k, v, do, o, l, m, dtype, dict(sm_scale=sc, **okw))
+    dqx = _exchanged_dq(F, qg, kg, vg, l, m, o, dog, d, sc, mf[0], mf[1], sfn, dk, dv,
+                        expect=dtype == torch.bfloat16 and not case.startswith("alibi"), causal=causal_flag, sid=sid)
+    if dqx is not None:
+        assert dqx.shape == q.shape
+        _check_grads((dqx, dk, dv), (rdq, rdk, rdv), q, k, v, do, o, l, m, dtype, dict(sm_scale=sc, **okw), tag="exchange ")
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
@@ -729,6 +763,8 @@ def _full_config_check(F, name, n_rows, heads_q, dense_group):
     dk, dv = _dkv(F, qg, kg, vg, l, m, dog, d, sc, mf, bf, sfn)
     d_s = F.compute_delta(o, dosg)
     dk_s, dv_s = _dkv(F, qg, kg, vg, l, m, dosg, d_s, sc, mf, bf, sfn)
+    # the same backward with dS handed from the dk/dv pass to the dq pass (plain and softcap scores)
+    dqx = _exchanged_dq(F, qg, kg, vg, l, m, o, dog, d, sc, mf, bf, sfn, dk, dv, expect=cfg.score in ("none", "softcap"))
     torch.cuda.synchronize()
     # the oracle's backward from the kernels' own residuals on the sampled rows (identical inputs)
     sdq, sdk_s, sdv_s = same_residual_grads(q, k, v, do, o, l, m, sm_scale=sc, q_rows=rows, heads=heads, **okw)
@@ -739,6 +775,8 @@ def _full_config_check(F, name, n_rows, heads_q, dense_group):
         assert_close(f"lse[{b},{h}]", (m + l.log())[b, h, rows.to(DEV)], (rm + rl.log())[b, h], cfg.dtype)
         assert_close(f"dq[{b},{h}]", dq[b, h, rows.to(DEV)], sdq[b, h], cfg.dtype)
         assert_close(f"dq[{b},{h}] chain", dq[b, h, rows.to(DEV)], rdq[b, h], cfg.dtype, chain=True)
+        if dqx is not None:
+            assert_close(f"exchange dq[{b},{h}]", dqx[b, h, rows.to(DEV)], sdq[b, h], cfg.dtype)
     kv_heads = sorted({(b, h // group) for (b, h) in heads})
     for (b, hk) in kv_heads:
         assert all((b, hk * group + gq) in heads for gq in range(group)), "sample whole KV groups"
@@ -766,6 +804,8 @@ def _full_config_check(F, name, n_rows, heads_q, dense_group):
         assert_close(f"o[{b},{h}] whole", o[b, h], wo[b, h], cfg.dtype)
         assert_close(f"lse[{b},{h}] whole", lse[b, h], wlse[b, h], cfg.dtype)
         assert_close(f"dq[{b},{h}] whole", dq[b, h], wdq[b, h], cfg.dtype)
+        if dqx is not None:
+            assert_close(f"exchange dq[{b},{h}] whole", dqx[b, h], wdq[b, h], cfg.dtype)
     assert_close(f"dk[{b},{hk}] whole", dk[b, hk], wdk[b, hk], cfg.dtype)
     assert_close(f"dv[{b},{hk}] whole", dv[b, hk], wdv[b, hk], cfg.dtype)
     return dict(o=o, l=l, m=m, dq=dq, dk=dk, dv=dv)
