@@ -1,9 +1,9 @@
 """Benchmark of the flex-attention hot path on one MI355X.
 
 One step = one pass of the hot path over one batch of synthetic input resident in HBM:
-forward (saving l, m), delta pre-pass, dk/dv backward, dq backward (the dk/dv pass hands its dS to the dq pass
-where the kernels of the configuration can: plain and softcap scores in bf16; the two passes without the
-hand-over are timed beside it).  The headline workload is
+forward (saving l, m), delta pre-pass, dq backward, dk/dv backward (where the package's own backward does so,
+softcap scores, the dk/dv pass hands its dS to the dq pass; where the kernels can run either way the other way
+is timed beside it).  The headline workload is
 benchmark configurations 2 + 3 (B=4, H=32, S=4096, D=128, bf16, causal); the other configurations
 (cfg1 fp32 small, cfg4 ALiBi + causal window, cfg5 GQA + soft-cap + documents) are measured in the
 same run and reported as sub-objects (`--config NAME` makes one of them the headline instead).
@@ -106,9 +106,15 @@ def measure(cfg, steps, warmup):
                                          block_k_major=blk, block_k=blk, sm_scale=sc, causal=False, debug=False,
                                          score_fn=sfn, mask_fn=mf, block_mask_fn=bf, return_ds=return_ds)
 
+    # the step hands dS over where the package's own backward (flex_attention) would: ds_exchange_pays
+    from flex_attention_tpu_amd.flex_attention_dq_bwd import ds_exchange_pays
+    exchange = ds_exchange_pays(sfn)
+
     def step():
         o, l, m = fwd()
         d = F.compute_delta(o, do)
+        if not exchange:
+            return o, dq_of(o, l, m, d), dkv_of(l, m, d)
         dk, dv, ds = dkv_of(l, m, d, True)   # (ds is None where the configuration's kernels exchange nothing)
         return o, dq_of(o, l, m, d, ds), dk, dv
 
@@ -126,11 +132,14 @@ def measure(cfg, steps, warmup):
     # behind every launch of a second batch gives the launch-to-launch intervals for the quantiles.
     o, l, m = fwd()
     d = F.compute_delta(o, do)
-    ds = dkv_of(l, m, d, True)[2]
-    launches = {"fwd": fwd, "delta": lambda: F.compute_delta(o, do), "dq": lambda: dq_of(o, l, m, d, ds),
-                "dkv": lambda: dkv_of(l, m, d, True)}
-    if ds is not None:   # the two passes on their own, each recomputing S, dP and dS
-        launches.update(dq_recompute=lambda: dq_of(o, l, m, d), dkv_no_export=lambda: dkv_of(l, m, d))
+    ds = dkv_of(l, m, d, True)[2]   # (None where the configuration's kernels exchange nothing)
+    used = exchange and ds is not None
+    launches = {"fwd": fwd, "delta": lambda: F.compute_delta(o, do),
+                "dq": (lambda: dq_of(o, l, m, d, ds)) if used else (lambda: dq_of(o, l, m, d)),
+                "dkv": (lambda: dkv_of(l, m, d, True)) if used else (lambda: dkv_of(l, m, d))}
+    if ds is not None:   # the other way of running the two passes, for comparison
+        launches.update(dq_other=(lambda: dq_of(o, l, m, d)) if used else (lambda: dq_of(o, l, m, d, ds)),
+                        dkv_other=(lambda: dkv_of(l, m, d)) if used else (lambda: dkv_of(l, m, d, True)))
     ms, quant = {}, {}
     for name, fn in launches.items():
         fn()
@@ -150,7 +159,8 @@ def measure(cfg, steps, warmup):
         torch.cuda.synchronize()
         quant[name] = quantiles([ev[i].elapsed_time(ev[i + 1]) for i in range(steps)])
     return {"ms_step": wall * 1e3 / steps, "ms": ms, "quantiles_ms": quant, "elem_bytes": q.element_size(),
-            "numel_q": q.numel(), "numel_k": k.numel(), "ds_bytes": ds.buf.numel() if ds is not None else 0}
+            "numel_q": q.numel(), "numel_k": k.numel(), "ds_bytes": ds.buf.numel() if ds is not None else 0,
+            "ds_used": used}
 
 
 def tf(fl, t_ms):
@@ -175,13 +185,13 @@ def summary(cfg, r):
         "bwd": {"ms": ms_bwd, "tflops": tf(2.5 * f_fwd, ms_bwd), "delta_ms": ms["delta"], "dq_ms": ms["dq"],
                 "dkv_ms": ms["dkv"], "delta_gbs": bytes_delta / (ms["delta"] * 1e-3) / 1e9,
                 "dq_quantiles_ms": r["quantiles_ms"]["dq"], "dkv_quantiles_ms": r["quantiles_ms"]["dkv"],
-                "delta_quantiles_ms": r["quantiles_ms"]["delta"], "ds_exchange": r["ds_bytes"] > 0},
+                "delta_quantiles_ms": r["quantiles_ms"]["delta"], "ds_exchange": r["ds_used"]},
     }
-    if r["ds_bytes"] > 0:
-        ms_split = ms["delta"] + ms["dq_recompute"] + ms["dkv_no_export"]
-        out["bwd"].update(ds_buffer_bytes=r["ds_bytes"], dq_recompute_ms=ms["dq_recompute"],
-                          dkv_no_export_ms=ms["dkv_no_export"], ms_without_exchange=ms_split,
-                          tflops_without_exchange=tf(2.5 * f_fwd, ms_split))
+    if r["ds_bytes"] > 0:   # the backward run the other way (with the dS hand-over if the step runs without, and vice versa)
+        ms_other = ms["delta"] + ms["dq_other"] + ms["dkv_other"]
+        tag = "without_exchange" if r["ds_used"] else "with_exchange"
+        out["bwd"].update({"ds_buffer_bytes": r["ds_bytes"], f"dq_ms_{tag}": ms["dq_other"], f"dkv_ms_{tag}": ms["dkv_other"],
+                           f"ms_{tag}": ms_other, f"tflops_{tag}": tf(2.5 * f_fwd, ms_other)})
     if eb == 2:
         out["fwd"]["frac_of_peak"] = out["fwd"]["tflops"] / PEAK_BF16_TFLOPS
         out["bwd"]["frac_of_peak"] = out["bwd"]["tflops"] / PEAK_BF16_TFLOPS
@@ -239,7 +249,7 @@ def main():
     bf16 = r["elem_bytes"] == 2
     # roofline of the dominant kernel; algorithmic FLOPs of one launch:
     #   fwd 2 matmuls = F_fwd, dk/dv 4 matmuls = 2 F_fwd, dq 3 matmuls = 1.5 F_fwd (1 matmul from exchanged dS)
-    algo = {"fwd": f_fwd, "dq": (0.5 if r["ds_bytes"] > 0 else 1.5) * f_fwd, "dkv": 2.0 * f_fwd}
+    algo = {"fwd": f_fwd, "dq": (0.5 if r["ds_used"] else 1.5) * f_fwd, "dkv": 2.0 * f_fwd}
     dom = max(algo, key=lambda n: ms[n])
     traffic = counter_traffic(dom) if name == "cfg2" else None
     roofline = {

@@ -16,12 +16,13 @@ from typing import Callable, Optional, Tuple
 import torch
 
 from .flex_attention_dkv_kernel import flash_attention_bwd_dkv
-from .flex_attention_dq_bwd import compute_delta, flex_attention_bwd_dq
+from .flex_attention_dq_bwd import compute_delta, ds_exchange_pays, flex_attention_bwd_dq
 from .flex_attention_kernel import _flex_attention_impl
 
 
 # The backward hands dS from the dk/dv pass to the dq pass (DsBlocks in flex_attention_dq_bwd.py) when both
-# gradients are wanted and the buffer, B Hq Sq Sk bf16 values, stays below this many bytes.
+# gradients are wanted, the hand-over is expected to pay (ds_exchange_pays) and the buffer, B Hq Sq Sk bf16
+# values, stays below this many bytes.
 DS_EXCHANGE_MAX_BYTES = 32 << 30
 
 
@@ -47,7 +48,7 @@ class _FlexAttention(torch.autograd.Function):
         dq = dk = dv = ds = None
         if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
             pad = lambda n: -(-n // 128) * 128
-            exchange = (ctx.needs_input_grad[0] and
+            exchange = (ctx.needs_input_grad[0] and ds_exchange_pays(score_fn) and
                         2 * q.shape[0] * q.shape[1] * pad(q.shape[2]) * pad(k.shape[2]) <= DS_EXCHANGE_MAX_BYTES)
             dk, dv, ds = flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, block_b=1, block_q=block_q,
                                                  block_q_major=block_q, block_k_major=block_k, block_k=block_k,

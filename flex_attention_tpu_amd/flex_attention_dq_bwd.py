@@ -40,6 +40,16 @@ class DsBlocks:
         self.buf, self.shape, self.entries = buf, shape, entries
 
 
+def ds_exchange_pays(score_fn) -> bool:
+    """Whether handing dS from the dk/dv pass to the dq pass is expected to shorten the backward.  Measured on
+    MI355X: with the softcap score (eight element-wise operations per score in the recomputing dq kernel) the
+    backward of a 16k-token GQA document batch went from 1.92 to 1.45 ms; with plain scores at B=4, H=32, S=4096
+    the export slows the dk/dv pass (writing S^2-sized dS costs it clock under the power limit) by as much as the
+    dq pass gains, 1.70 against 1.68 ms, so there the passes stay on their own."""
+    spec = getattr(score_fn, "spec", None)
+    return getattr(spec, "kind", None) == _lib.SCORE_SOFTCAP
+
+
 def bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, mod_q, mod_k, dq=None, dk=None, dv=None,
                compiled_loop=False, ab_c=None):
     B, Hq, Sq, D = q.shape
