@@ -31,7 +31,7 @@ def regs_of(token):
 
 def split_operands(line):
     op, _, rest = line.partition(" ")
-    rest = re.sub(r"offset:\d+", "", rest)
+    rest = re.sub(r"offset:-?\d+", "", rest)
     return op, [t.strip() for t in rest.split(",")] if rest.strip() else []
 
 
@@ -116,6 +116,11 @@ def check_stream(lines):
             fifo.append(dst)
         elif op.startswith("global_load_lds"):
             pass  # operands come from the compiler; the destination is LDS through M0
+        elif op.startswith("global_store"):
+            src = regs_of(ops[1])  # (the address operands come from the compiler and the run loop)
+            assert not lds_pending(src), f"store of a register with an LDS read in flight: {line}"
+            for r in src:
+                assert mfma_done(r), f"store of a fresh MFMA result: {line}"
         elif op.startswith("ds_write"):
             src = regs_of(ops[1])
             assert not lds_pending(src), f"LDS store of a register with an LDS read in flight: {line}"
@@ -179,6 +184,55 @@ def test_dkv_tile_streams_respect_hazards():
             assert v.stats["mfma"] == 128
             assert nv == v.stats["mfma"] + v.stats["valu"] + v.stats["lds"] + v.stats["vmem"]
             scratch_ok(v.out, 68, 199, 255)
+
+
+def test_dkv_export_streams_store_the_dk_operand_and_count_their_waits():
+    """dS export variants of the dk/dv streams: every (q block, half) is stored once, from the registers its
+    conversions wrote last; the wait of the row values' turn-around counts every vector-memory operation in front
+    of it (the two row loads precede the stream), the closing wait the stores behind the last LDS-direct copy."""
+    import gen_dkv_tile as g
+
+    for softcap in (False, True):
+        for masked in (False, True):
+            em = g.build(masked, False, softcap, True)
+            n = check_stream(em.out)
+            assert em.stats["mfma"] == 128 and em.stats["vmem"] == 24
+            assert n == em.stats["mfma"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
+            scratch_ok(em.out, 68, 199, 255)
+            last_writer, offsets, vmem, waits, last_load = {}, [], 0, [], -1
+            for i, line in enumerate(em.out):
+                op, ops = split_operands(line)
+                if op.startswith("global_store"):
+                    assert op == "global_store_dwordx4" and ops[0] == "%[dsv]" and ops[2] == "s[56:57]", line
+                    src = regs_of(ops[1])
+                    assert len(src) == 4 and all(last_writer.get(r, "").startswith("v_cvt_pk_bf16_f32") for r in src), line
+                    offsets.append(int(re.search(r"offset:(-?\d+)", line).group(1)))
+                    vmem += 1
+                elif op.startswith("global_load_lds"):
+                    vmem += 1
+                    last_load = vmem
+                elif op == "s_waitcnt" and "vmcnt" in line:
+                    waits.append((int(re.search(r"vmcnt\((\d+)\)", line).group(1)), vmem))
+                elif op.startswith("v_") and ops:
+                    for r in regs_of(ops[0]):
+                        last_writer[r] = op
+            assert sorted(offsets) == [1024 * k - 4096 for k in range(8)]
+            # the stored registers are the B operands of the dk MFMAs (dk accumulators a[64:127])
+            dk_b = set()
+            for line in em.out:
+                op, ops = split_operands(line)
+                if op.startswith("v_mfma") and regs_of(ops[0]) <= {("a", i) for i in range(64, 128)}:
+                    dk_b |= regs_of(ops[2])
+            stored = set()
+            for line in em.out:
+                op, ops = split_operands(line)
+                if op.startswith("global_store"):
+                    stored |= regs_of(ops[1])
+            assert stored == dk_b
+            assert len(waits) == 2
+            (n_turn, at_turn), (n_end, at_end) = waits
+            assert n_turn == at_turn, "the turn-around must wait for exactly the operations in front of it"
+            assert at_end == vmem == 24 and n_end == vmem - last_load, "the closing wait leaves only stores behind the last copy open"
 
 
 def test_hazard_checker_catches_a_bad_stream():
