@@ -7,8 +7,11 @@
 // global -> LDS (global_load_lds_dwordx4, no registers in between) through rings of stages, and reads both
 // operands with transposing LDS reads: computed transposed, dq^T[d, i] += sum_j K^T[d, j] dS^T[j, i], the lane
 // that owned kv column j in the dk/dv kernel wrote 8 q rows of it contiguously, which is what
-// ds_read_b64_tr_b16 turns into "lane owns q row i, 4 consecutive j".  The kernel moves 32 KB of dS per 16 MFMAs
-// and wave: it is bound by HBM, not by the matrix pipe.
+// ds_read_b64_tr_b16 turns into "lane owns q row i, 4 consecutive j".  The kernel moves 32 KB of dS and 32 KB of K
+// per 32 MFMAs and wave; the matrix pipe is busy a quarter of the time.  Measured with cycle stamps per 32-column
+// stage and wave: waiting for the copies 180-255, barrier 100-140, issuing the wave's four copies 700 (an
+// LDS-direct copy of 1 KB holds the issuing wave about 175 cycles when all eight waves of the CU copy at once),
+// LDS reads and MFMAs 410.
 //
 // Layout of a dS block (written by the dk/dv kernel): kv columns 32 w' + jj (w' = 0..3), q rows 32 c + 16 u + ii:
 // byte 8192 w' + 1024 (2 c + u) + 16 (2 jj + hi) + 8 g + 2 e holds row ii = 8 g + 4 hi + e.
