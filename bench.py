@@ -2,8 +2,8 @@
 
 One step = one pass of the hot path over one batch of synthetic input resident in HBM:
 forward (saving l, m), delta pre-pass, dq backward, dk/dv backward (where the package's own backward does so,
-softcap scores, the dk/dv pass hands its dS to the dq pass; where the kernels can run either way the other way
-is timed beside it).  The headline workload is
+softcap scores and masks with many partial tiles, the dk/dv pass hands its dS to the dq pass; where the kernels
+can run either way the other way is timed beside it).  The headline workload is
 benchmark configurations 2 + 3 (B=4, H=32, S=4096, D=128, bf16, causal); the other configurations
 (cfg1 fp32 small, cfg4 ALiBi + causal window, cfg5 GQA + soft-cap + documents) are measured in the
 same run and reported as sub-objects (`--config NAME` makes one of them the headline instead).
@@ -108,7 +108,7 @@ def measure(cfg, steps, warmup):
 
     # the step hands dS over where the package's own backward (flex_attention) would: ds_exchange_pays
     from flex_attention_tpu_amd.flex_attention_dq_bwd import ds_exchange_pays
-    exchange = ds_exchange_pays(sfn)
+    exchange = ds_exchange_pays(sfn, mf)
 
     def step():
         o, l, m = fwd()

@@ -48,7 +48,7 @@ class _FlexAttention(torch.autograd.Function):
         dq = dk = dv = ds = None
         if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
             pad = lambda n: -(-n // 128) * 128
-            exchange = (ctx.needs_input_grad[0] and ds_exchange_pays(score_fn) and
+            exchange = (ctx.needs_input_grad[0] and ds_exchange_pays(score_fn, mask_fn, segment_ids) and
                         2 * q.shape[0] * q.shape[1] * pad(q.shape[2]) * pad(k.shape[2]) <= DS_EXCHANGE_MAX_BYTES)
             dk, dv, ds = flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, block_b=1, block_q=block_q,
                                                  block_q_major=block_q, block_k_major=block_k, block_k=block_k,

@@ -40,14 +40,22 @@ class DsBlocks:
         self.buf, self.shape, self.entries = buf, shape, entries
 
 
-def ds_exchange_pays(score_fn) -> bool:
-    """Whether handing dS from the dk/dv pass to the dq pass is expected to shorten the backward.  Measured on
-    MI355X: with the softcap score (eight element-wise operations per score in the recomputing dq kernel) the
-    backward of a 16k-token GQA document batch went from 1.92 to 1.45 ms; with plain scores at B=4, H=32, S=4096
-    the export slows the dk/dv pass (writing S^2-sized dS costs it clock under the power limit) by as much as the
-    dq pass gains, 1.70 against 1.68 ms, so there the passes stay on their own."""
-    spec = getattr(score_fn, "spec", None)
-    return getattr(spec, "kind", None) == _lib.SCORE_SOFTCAP
+def ds_exchange_pays(score_fn, mask_fn=None, segment_ids=None) -> bool:
+    """Whether handing dS from the dk/dv pass to the dq pass is expected to shorten the backward: yes with the
+    softcap score (eight element-wise operations per score in the recomputing dq kernel) and with masks that
+    leave many partial tiles (documents, windows: the dq pass from dS does no mask work at all); no with plain
+    scores under no mask or a plain causal one, where the export slows the dk/dv pass (writing S^2-sized dS costs
+    it clock under the power limit) by as much as the dq pass gains.  Measured on MI355X, dq + dk/dv in ms,
+    recomputing -> exchanging: softcap + documents, 16k tokens, GQA 4:1: 1.93 -> 1.47; documents, plain scores, same
+    shape: 1.75 -> 1.34; five documents in B=4, H=32, S=4096: 1.09 -> 0.91; causal window 1025, B=2, H=16, S=8192:
+    0.56 -> 0.49; softcap, causal, B=4, H=32, S=4096: 2.08 -> 1.86; plain causal, same shape: 1.67 -> 1.68; plain
+    causal GQA 4:1, B=2, Hq=32, S=8192: 3.09 -> 3.17."""
+    if getattr(getattr(score_fn, "spec", None), "kind", None) == _lib.SCORE_SOFTCAP:
+        return True
+    if segment_ids is not None:
+        return True
+    flags = getattr(getattr(mask_fn, "spec", None), "flags", 0)
+    return bool(flags & (_lib.MASK_WINDOW | _lib.MASK_DOC | _lib.MASK_S2))
 
 
 def bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, mod_q, mod_k, dq=None, dk=None, dv=None,

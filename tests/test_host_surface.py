@@ -251,3 +251,18 @@ def test_host_caches_are_bounded():
     spec = _common.resolve_mask(None, None, True, None, 200, 300, 256, 384)
     assert spec.flags == _lib.MASK_CAUSAL | _lib.MASK_DOC
     assert spec.doc_ids.array.tolist() == [0] * 256 and spec.doc_ids_k.array.tolist() == [0] * 300 + [1] * 84
+
+
+def test_ds_exchange_policy():
+    """The backward hands dS from the dk/dv pass to the dq pass for softcap scores and for masks that leave many
+    partial tiles, not for plain scores under no mask or a plain causal one."""
+    from flex_attention_tpu_amd import masks, scores
+    from flex_attention_tpu_amd.flex_attention_dq_bwd import ds_exchange_pays
+    causal = masks.make_causal_mask_fns(128, 128)[0]
+    assert not ds_exchange_pays(None) and not ds_exchange_pays(None, causal)
+    assert not ds_exchange_pays(scores.make_alibi_global_score_fn(4), causal)
+    assert ds_exchange_pays(scores.make_softcap_score_fn(30.0), causal)
+    assert ds_exchange_pays(None, masks.make_causal_sliding_window_mask_fns(128, 128, 300)[0])
+    assert ds_exchange_pays(None, masks.make_jagged_mask_fns(128, 128, [100, 156])[0])
+    assert ds_exchange_pays(None, None, segment_ids=[0] * 128 + [1] * 128)
+
