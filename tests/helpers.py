@@ -6,6 +6,9 @@ from oracle import mha_oracle as O
 # north-star tolerances, asserted as written: bf16 max-abs <= 2e-2 and rel-L2 <= 1e-2; fp32 1e-5
 BF16_ABS, BF16_REL = 2e-2, 1e-2
 F32_ABS, F32_REL = 1e-5, 1e-5
+# whole-chain gradients (kernel forward -> delta -> kernel backward against oracle forward -> oracle backward) may
+# exceed the element-wise bound by the share that comes from the forward's rounded output, see assert_close
+CHAIN_SLACK = 1.5
 
 # (test, name, max|ref|, max-abs, rel-L2, worst error / bound) of every comparison of the session, printed by conftest's
 # terminal summary so that the strict numbers of each configuration are in the pytest output
@@ -29,15 +32,19 @@ def assert_close(name, test, ref, dtype, chain=False):
     The strict max-abs of every comparison goes into REPORT and the terminal summary.
 
     `chain=True` marks a comparison of gradients taken through the whole chain (kernel forward ->
-    delta -> kernel backward against oracle forward -> oracle backward): rel-L2 is asserted, the
-    max-abs figure is reported only.  There the two backward passes start from different residuals:
-    the kernels' delta = sum(o * do) is taken of the forward's bf16 output, as the interface demands
-    (o is returned in q.dtype), the oracle's of its own float64 o, and that difference (up to 2^-8
-    relative per element of o, times |do|, summed over the head dimension) is not a property of the
-    backward kernels.  They are held to the bound by the comparison on identical residuals
-    (same_residual_grads), which is how the reference checks its own backward kernels
-    (flex_attention_dq_bwd.py:920-946, flash_attention_dkv_bwd.py:913-940: the same o, l, m, d go to
-    the kernels and to mha_bwd_reference)."""
+    delta -> kernel backward against oracle forward -> oracle backward): rel-L2 is asserted as
+    written and the element-wise bound with the factor CHAIN_SLACK = 1.5.  There the two backward
+    passes start from different residuals: the kernels' delta = sum(o * do) is taken of the forward's
+    bf16 output, as the interface demands (o is returned in q.dtype), the oracle's of its own float64
+    o, and that difference (up to 2^-9 relative per element of o, times |do|, summed over the head
+    dimension: about 0.03 per row at head dimension 128 with unit-variance inputs, times P times
+    |k| or |q| in dq and dk) is not a property of the backward kernels.  The largest whole-chain
+    figures measured on the benchmark configurations are 1.09 (dk, ALiBi + window) and 1.37 (dk,
+    softcap + documents + grouped heads) times the element-wise bound, so 1.5 leaves the chain no room
+    to drift unnoticed.  The backward kernels themselves are held to the bound proper by the
+    comparison on identical residuals (same_residual_grads), which is how the reference checks its
+    own backward kernels (flex_attention_dq_bwd.py:920-946, flash_attention_dkv_bwd.py:913-940: the
+    same o, l, m, d go to the kernels and to mha_bwd_reference)."""
     test, ref = test.detach().cpu().double(), ref.detach().cpu().double()
     ma, rl = O.max_abs(test, ref), O.rel_l2(test, ref)
     ref_max = float(ref.abs().max())
@@ -50,8 +57,9 @@ def assert_close(name, test, ref, dtype, chain=False):
         rel_tol = F32_REL
     REPORT.append((CURRENT, name, ref_max, ma, rl, ratio))
     assert rl <= rel_tol, f"{name}: rel-L2 {rl:.3e} > {rel_tol:.1e} (max-abs {ma:.3e})"
-    assert chain or ratio <= 1.0, (f"{name}: max-abs {ma:.3e}, {ratio:.2f} x the element-wise bound "
-                          f"(rel-L2 {rl:.3e}, max|ref| {ref_max:.3f})")
+    limit = CHAIN_SLACK if (chain and dtype == torch.bfloat16) else 1.0
+    assert ratio <= limit, (f"{name}: max-abs {ma:.3e}, {ratio:.2f} x the element-wise bound (limit {limit}; "
+                            f"rel-L2 {rl:.3e}, max|ref| {ref_max:.3f})")
     return ma, rl
 
 

@@ -469,3 +469,125 @@ def test_fwd_out_of_line_blocks_are_the_inline_ones():
                 back.append(hot[i])
                 i += 1
         assert back == lines
+
+
+# ---------------------------------------------------------------------------------------------------
+# vector-memory queue of the run loops: no load into registers may be open when control leaves the asm
+# ---------------------------------------------------------------------------------------------------
+def check_vmem_queue(lines):
+    """Walks every control-flow path of an asm region (forward and backward branches, both outcomes of
+    every conditional one) and replays the in-order vector-memory queue: loads into VGPRs, LDS-direct
+    loads and stores enter it, `s_waitcnt vmcnt(N)` retires all but the N youngest.  Asserts that
+
+      * no instruction names a VGPR that a load still in the queue will write (the value is not there
+        yet; and if the compiler or the stream reused the register, the late load would overwrite it);
+      * at every `s_barrier` no load of either kind is open (the barrier tells the other waves that
+        this wave's copies have landed);
+      * where control leaves the region (falls off its end) only stores are open: the compiler, which
+        does not know of the region's loads, is free to reuse every register behind it.
+
+    Returns the number of (instruction, queue state) pairs visited."""
+    labels = {l[:-1]: i for i, l in enumerate(lines) if l.endswith(":")}
+    seen = set()
+    work = [(0, ())]
+    while work:
+        pc, q = work.pop()
+        while True:
+            if (pc, q) in seen:
+                break
+            seen.add((pc, q))
+            if pc == len(lines):
+                open_loads = [e for e in q if e[0] != "store"]
+                assert not open_loads, f"region ends with loads in flight: {open_loads}"
+                break
+            line = lines[pc]
+            op, ops = split_operands(line)
+            pending = set().union(*[set(e[1]) for e in q]) if q else set()
+            if op.endswith(":"):
+                pc += 1
+                continue
+            if op == "s_waitcnt":
+                m = re.search(r"vmcnt\((\d+)\)", line)
+                if m:
+                    n = int(m.group(1))
+                    q = q[len(q) - n:] if n < len(q) else q
+                    if n == 0:
+                        q = ()
+                pc += 1
+                continue
+            if op == "s_barrier":
+                open_loads = [e for e in q if e[0] != "store"]
+                assert not open_loads, f"s_barrier with loads in flight: {open_loads}"
+                pc += 1
+                continue
+            if op == "s_branch":
+                pc = labels[ops[0]]
+                continue
+            if op.startswith("s_cbranch"):
+                work.append((labels[ops[0]], q))
+                pc += 1
+                continue
+            named = regs_of(line)
+            assert not (named & pending), f"register of a load in flight is used: {line}"
+            if op.startswith("global_load_lds"):
+                q = q + (("lds", ()),)
+            elif op.startswith("global_load") or op.startswith("buffer_load"):
+                q = q + (("load", tuple(sorted(regs_of(ops[0])))),)
+            elif op.startswith("global_store") or op.startswith("buffer_store"):
+                q = q + (("store", ()),)
+            pc += 1
+    return len(seen)
+
+
+def _run_loops():
+    import gen_dkv_tile, gen_dq_tile, gen_fwd_tile
+    for alibi, softcap, export in ((False, False, False), (True, False, False), (False, True, False), (False, False, True),
+                                   (False, True, True)):
+        g = gen_dkv_tile
+        yield f"dkv alibi={alibi} softcap={softcap} export={export}", g.run_loop(
+            g.build(False, alibi, softcap, export), g.build(True, alibi, softcap, export), alibi, softcap, export)
+    for g, name in ((gen_dq_tile, "dq"), (gen_fwd_tile, "fwd")):
+        for alibi, softcap in ((False, False), (True, False), (False, True)):
+            yield f"{name} alibi={alibi} softcap={softcap}", g.run_loop(
+                g.build(False, alibi, softcap), g.build(True, alibi, softcap), alibi, softcap)
+
+
+def test_run_loops_leave_no_load_in_flight():
+    """Every generated run loop (the dq and dk/dv ones are the only asm regions of the library that load
+    from global memory into registers; every other asm load, the forward loop's included, has LDS as its
+    destination and is waited for with vmcnt(0) in front of the work-group barrier): on every path through the region the loads into registers have been waited
+    for before their registers are named again and before control leaves the region, and all copies into
+    LDS before each barrier.  The dS-exporting loops may leave stores open, nothing else."""
+    n_loops = 0
+    for name, lines in _run_loops():
+        # (the check is not vacuous: every loop copies into LDS, the backward loops also load into registers)
+        assert any(l.startswith("global_load_lds") for l in lines), name
+        assert name.startswith("fwd") or any(l.startswith("global_load_dword") for l in lines), name
+        assert check_vmem_queue(lines) > len(lines), name
+        n_loops += 1
+    assert n_loops == 11
+
+
+def test_vmem_queue_checker_catches_open_loads():
+    # a load into a register that is still open where the region ends
+    bad = ["global_load_dword v66, v66, s[66:67]", "v_mov_b32_e32 v70, 0"]
+    with pytest.raises(AssertionError, match="ends with loads in flight"):
+        check_vmem_queue(bad)
+    check_vmem_queue(bad + ["s_waitcnt vmcnt(0)"])
+    # ... open on one of two paths only (the wait is skipped by a branch)
+    bad = ["global_load_dword v66, v66, s[66:67]", "s_cbranch_scc1 .Lskip", "s_waitcnt vmcnt(0)", ".Lskip:", "s_nop 0"]
+    with pytest.raises(AssertionError, match="ends with loads in flight"):
+        check_vmem_queue(bad)
+    # a store behind the load may stay open, the load may not: vmcnt(1) retires the load, vmcnt(2) does not
+    ok = ["global_load_dword v66, v66, s[66:67]", "global_store_dwordx4 v80, v[72:75], s[56:57]", "s_waitcnt vmcnt(1)"]
+    check_vmem_queue(ok)
+    with pytest.raises(AssertionError, match="ends with loads in flight"):
+        check_vmem_queue(ok[:2] + ["s_waitcnt vmcnt(2)"])
+    # the destination is read before the wait
+    bad = ["global_load_dword v66, v66, s[66:67]", "v_readfirstlane_b32 s80, v66", "s_waitcnt vmcnt(0)"]
+    with pytest.raises(AssertionError, match="register of a load in flight"):
+        check_vmem_queue(bad)
+    # a copy into LDS still open at the barrier, across a loop back-edge
+    bad = [".Ltop:", "s_barrier", "global_load_lds_dwordx4 v70, s[20:21]", "s_cbranch_scc1 .Ltop", "s_waitcnt vmcnt(0)"]
+    with pytest.raises(AssertionError, match="s_barrier with loads in flight"):
+        check_vmem_queue(bad)

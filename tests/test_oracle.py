@@ -202,3 +202,93 @@ def test_golden_vectors():
     dq, dk, dv = O.mha_bwd_reference(q, k, v, o, do, l, m, **kw)
     for name, t in (("o", o), ("l", l), ("m", m), ("dq", dq), ("dk", dk), ("dv", dv)):
         assert np.allclose(t.numpy(), g[name], rtol=0, atol=1e-12), name
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_additive_bias_branch_matches_sdpa_float_mask(causal):
+    """`ab=` (mha_reference.py:50-51: added behind the score function, in front of the masks) against
+    SDPA with a float ``attn_mask`` (added to the scaled logits), forward and autograd backward; under
+    `causal` the float mask carries -inf above the diagonal.  A bias that was dropped, scaled by sm_scale
+    or added behind the mask fails here."""
+    q, k, v, do = O.make_inputs(2, 3, 3, 40, 56, 16, dtype=torch.float64, seed=13)
+    g = torch.Generator().manual_seed(14)
+    ab = torch.randn(2, 3, 40, 56, generator=g, dtype=torch.float64) * 2
+    kw = dict(sm_scale=0.3, causal=causal)
+    o, l, m = O.mha_reference(q, k, v, ab, save_residuals=True, **kw)
+    dq, dk, dv = O.mha_bwd_reference(q, k, v, o, do, l, m, ab, **kw)
+    bias = ab.clone()
+    if causal:
+        bias = bias.masked_fill(torch.arange(56)[None, :] > torch.arange(40)[:, None], float("-inf"))
+    qd, kd, vd = [x.clone().requires_grad_() for x in (q, k, v)]
+    r = torch.nn.functional.scaled_dot_product_attention(qd, kd, vd, attn_mask=bias, scale=0.3)
+    assert (o - r).abs().max() < 1e-12
+    s = torch.einsum("bhqc,bhkc->bhqk", q, k) * 0.3 + bias
+    assert ((m + l.log()) - torch.logsumexp(s, -1)).abs().max() < 1e-12
+    gq, gk, gv = torch.autograd.grad(r, (qd, kd, vd), do)
+    for a, b in ((dq, gq), (dk, gk), (dv, gv)):
+        assert (a - b).abs().max() < 1e-11
+
+
+def test_additive_bias_with_score_mod_and_gqa_matches_autograd():
+    """`ab=` next to a score function and grouped kv heads: the bias is added to the *modified* logits
+    (softcap first, then + ab) -- against autograd of an independently written dense softmax."""
+    q, k, v, do = O.make_inputs(1, 4, 2, 24, 24, 8, dtype=torch.float64, seed=15)
+    ab = torch.randn(1, 4, 24, 24, generator=torch.Generator().manual_seed(16), dtype=torch.float64)
+    kw = dict(sm_scale=0.6, causal=True, score_mod=O.score_mod_softcap(2.5))
+    o, l, m = O.mha_reference(q, k, v, ab, save_residuals=True, **kw)
+    dq, dk, dv = O.mha_bwd_reference(q, k, v, o, do, l, m, ab, **kw)
+    qd, kd, vd = [x.clone().requires_grad_() for x in (q, k, v)]
+    outs = []
+    for h in range(4):
+        s = 2.5 * torch.tanh((qd[0, h] @ kd[0, h // 2].T) * 0.6 / 2.5) + ab[0, h]
+        s = s.masked_fill(torch.arange(24)[None, :] > torch.arange(24)[:, None], float("-inf"))
+        outs.append(torch.softmax(s, -1) @ vd[0, h // 2])
+    r = torch.stack(outs)[None]
+    assert (r - o).abs().max() < 1e-12
+    gq, gk, gv = torch.autograd.grad(r, (qd, kd, vd), do)
+    for a, b in ((dq, gq), (dk, gk), (dv, gv)):
+        assert (a - b).abs().max() < 1e-11
+
+
+@pytest.mark.parametrize("per_batch", [False, True])
+def test_dense_mask_branch_matches_sdpa_bool_mask(per_batch):
+    """`mask=` (an arbitrary boolean keep mask, [Sq, Sk] or one per batch entry) against SDPA with a boolean
+    ``attn_mask`` (True = attend), forward and autograd backward.  Every row keeps at least one key."""
+    B, H, Sq, Sk = 2, 2, 32, 48
+    q, k, v, do = O.make_inputs(B, H, H, Sq, Sk, 16, dtype=torch.float64, seed=17)
+    g = torch.Generator().manual_seed(18)
+    keep = torch.rand((B, Sq, Sk) if per_batch else (Sq, Sk), generator=g) < 0.4
+    keep[..., 0] = True
+    kw = dict(sm_scale=0.35, mask=keep)
+    o, l, m = O.mha_reference(q, k, v, save_residuals=True, **kw)
+    dq, dk, dv = O.mha_bwd_reference(q, k, v, o, do, l, m, **kw)
+    qd, kd, vd = [x.clone().requires_grad_() for x in (q, k, v)]
+    am = keep[:, None] if per_batch else keep
+    r = torch.nn.functional.scaled_dot_product_attention(qd, kd, vd, attn_mask=am, scale=0.35)
+    assert (o - r).abs().max() < 1e-12
+    gq, gk, gv = torch.autograd.grad(r, (qd, kd, vd), do)
+    for a, b in ((dq, gq), (dk, gk), (dv, gv)):
+        assert (a - b).abs().max() < 1e-11
+    # the mask composes with the keyword masks by AND
+    o2 = O.mha_reference(q, k, v, causal=True, **kw)
+    both = am & (torch.arange(Sk)[None, :] <= torch.arange(Sq)[:, None])
+    r2 = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=both, scale=0.35)
+    assert (o2 - r2).abs().max() < 1e-12
+
+
+def test_legacy_alibi_slope_branch_matches_sdpa_float_mask():
+    """`alibi_slope=` (the tile-local bias the reference's dense code mimics with `% 1024` / `% 512`,
+    mha_reference.py:35-41): logits - slope |i % mod_q - j % mod_k|, here as a float attn_mask of SDPA."""
+    S = 40
+    q, k, v, do = O.make_inputs(1, 2, 2, S, S, 8, dtype=torch.float64, seed=19)
+    kw = dict(sm_scale=0.5, alibi_slope=0.7, alibi_mods=(16, 8))
+    o, l, m = O.mha_reference(q, k, v, save_residuals=True, **kw)
+    dq, dk, dv = O.mha_bwd_reference(q, k, v, o, do, l, m, **kw)
+    i, j = torch.arange(S)[:, None], torch.arange(S)[None, :]
+    bias = -0.7 * ((i % 16) - (j % 8)).abs().to(torch.float64)
+    qd, kd, vd = [x.clone().requires_grad_() for x in (q, k, v)]
+    r = torch.nn.functional.scaled_dot_product_attention(qd, kd, vd, attn_mask=bias, scale=0.5)
+    assert (o - r).abs().max() < 1e-12
+    gq, gk, gv = torch.autograd.grad(r, (qd, kd, vd), do)
+    for a, b in ((dq, gq), (dk, gk), (dv, gv)):
+        assert (a - b).abs().max() < 1e-11
