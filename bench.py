@@ -27,18 +27,39 @@ PEAK_HBM_GBS = 8000.0
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_cfg2_hbm_traffic.txt")
 
 
+def kernel_sources_digest():
+    """sha256 (first 16 hex digits) over the kernel sources of libflexattn.so: the HIP files, their headers and
+    the stream generators, in name order.  The counter summary under profiles/ records the digest of the
+    sources it was measured on; a different digest here means the kernels changed since."""
+    import hashlib
+    csrc = os.path.join(ROOT, "flex_attention_tpu_amd", "csrc")
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".hpp", ".py")):
+            h.update(name.encode())
+            h.update(open(os.path.join(csrc, name), "rb").read())
+    return h.hexdigest()[:16]
+
+
 def counter_traffic(kernel):
-    """HBM bytes per launch of `kernel` on cfg2 from the committed rocprofv3 counter summary (FETCH_SIZE
-    and WRITE_SIZE runs of this script, scaled by the 256 MiB device copy main() ends with), or None.
-    Counter-derived in a separate profiler run, not measured in this run."""
+    """(HBM bytes per launch of `kernel` on cfg2, stale) from the committed rocprofv3 counter summary
+    (FETCH_SIZE and WRITE_SIZE runs of this script, scaled by the 256 MiB device copy main() ends with), or
+    (None, None).  Counter-derived in a separate profiler run, not measured in this run: `stale` says whether
+    the kernel sources have changed since that run (the summary names the digest it was measured on)."""
+    value, digest = None, None
     try:
         for line in open(TRAFFIC_PROFILE):
             f = line.split()
             if len(f) >= 6 and f[0] == kernel and re.fullmatch(r"[0-9.]+", f[5]):
-                return int(float(f[5]) * 1e6)
+                value = int(float(f[5]) * 1e6)
+            m = re.match(r"kernel sources digest: ([0-9a-f]{16})", line)
+            if m:
+                digest = m.group(1)
     except OSError:
         pass
-    return None
+    if value is None:
+        return None, None
+    return value, digest != kernel_sources_digest()
 
 
 def cpu_baseline(cfg, budget_s=12.0):
@@ -251,13 +272,14 @@ def main():
     #   fwd 2 matmuls = F_fwd, dk/dv 4 matmuls = 2 F_fwd, dq 3 matmuls = 1.5 F_fwd (1 matmul from exchanged dS)
     algo = {"fwd": f_fwd, "dq": (0.5 if r["ds_used"] else 1.5) * f_fwd, "dkv": 2.0 * f_fwd}
     dom = max(algo, key=lambda n: ms[n])
-    traffic = counter_traffic(dom) if name == "cfg2" else None
+    traffic, stale = counter_traffic(dom) if name == "cfg2" else (None, None)
     roofline = {
         "kernel": dom, "bound": "mfma", "achieved": tf(algo[dom], ms[dom]), "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s", "frac": tf(algo[dom], ms[dom]) / PEAK_BF16_TFLOPS,
         "traffic": traffic,
         "traffic_source": "profiles/bench_cfg2_hbm_traffic.txt (rocprofv3 --pmc runs of this script, not this run)"
                           if traffic is not None else None,
+        "traffic_stale": stale,   # True: the kernel sources changed since the counter runs behind `traffic`
         "launch_ms": ms[dom], "launch_quantiles_ms": r["quantiles_ms"][dom],
     }
     if not bf16:

@@ -86,6 +86,14 @@ class BiasC(C.Structure):
     ]
 
 
+class DsIndexC(C.Structure):
+    _fields_ = [
+        ("col", C.c_void_p),
+        ("rank", C.c_void_p),
+        ("pairs", C.c_int64),
+    ]
+
+
 class FwdParamsC(C.Structure):
     _fields_ = [
         ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p),
@@ -122,6 +130,7 @@ class BwdParamsC(C.Structure):
         ("ab", BiasC),
         ("ds", C.c_void_p),
         ("ds_bytes", C.c_int64),
+        ("ds_index", DsIndexC),
     ]
 
 
@@ -130,6 +139,7 @@ EXPORTS = (
     "flexattn_last_error_string",
     "flexattn_tile_shape",
     "flexattn_build_block_mask",
+    "flexattn_build_ds_index",
     "flexattn_fwd",
     "flexattn_fwd_noalloc",
     "flexattn_bwd_delta",
@@ -151,6 +161,7 @@ def _bind(lib: C.CDLL) -> C.CDLL:
     lib.flexattn_build_block_mask.argtypes = [
         C.POINTER(MaskSpecC), C.c_int32, C.c_int32, C.c_int32, C.c_int32,
         C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.flexattn_build_ds_index.argtypes = [C.POINTER(BlockMapC), C.c_void_p, C.c_void_p, C.c_void_p]
     lib.flexattn_fwd.argtypes = [C.POINTER(FwdParamsC), C.c_void_p]
     lib.flexattn_fwd_noalloc.argtypes = [C.POINTER(FwdParamsC), C.c_void_p]
     lib.flexattn_bwd_delta.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
@@ -158,7 +169,7 @@ def _bind(lib: C.CDLL) -> C.CDLL:
     lib.flexattn_bwd_ds_bytes.argtypes = [C.POINTER(BwdParamsC)]
     lib.flexattn_bwd_ds_bytes.restype = C.c_int64
     lib.flexattn_bwd_dkv.argtypes = [C.POINTER(BwdParamsC), C.c_void_p]
-    for name in ("flexattn_tile_shape", "flexattn_build_block_mask", "flexattn_fwd", "flexattn_fwd_noalloc", "flexattn_bwd_delta",
+    for name in ("flexattn_tile_shape", "flexattn_build_block_mask", "flexattn_build_ds_index", "flexattn_fwd", "flexattn_fwd_noalloc", "flexattn_bwd_delta",
                  "flexattn_bwd_dq", "flexattn_bwd_dkv"):
         getattr(lib, name).restype = C.c_int
     return lib

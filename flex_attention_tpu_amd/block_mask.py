@@ -62,12 +62,45 @@ class BlockMap:
         self.q_idx = torch.empty(self.nk, self.nq, dtype=torch.int32, device=device)
         self.built_on = None   # stream the builder kernel was launched on
         self.ready = None      # event recorded behind it
+        self._ds_index = None  # (col, rank, pairs) of the dS exchange buffer, built at first use
+
+    def _tensors(self):
+        t = [self.state, self.kv_cnt, self.kv_idx, self.q_cnt, self.q_idx]
+        if self._ds_index is not None:
+            t += [self._ds_index[0], self._ds_index[1]]
+        return t
 
     def wait_ready(self, device) -> None:
-        """Makes the current stream wait for the builder kernel if that ran on another stream."""
+        """Makes the current stream wait for the builder kernel if that ran on another stream, and tells the
+        caching allocator that the map is in use on this stream too (a map evicted from the cache must not be
+        handed out again while a kernel on this stream still walks it)."""
         cur = torch.cuda.current_stream(device)
         if self.ready is not None and cur.cuda_stream != self.built_on:
             cur.wait_event(self.ready)
+            for t in self._tensors():
+                t.record_stream(cur)
+
+    def ds_index(self):
+        """(col int32 [nk + 1], rank int32 [nq, nk], pairs) of flexattn_build_ds_index for this map: the order of
+        the dS exchange buffer's blocks over the kept tile pairs.  Built once per map (one 4-byte copy to the
+        host for the number of pairs)."""
+        if self._ds_index is None:
+            dev = self.state.device
+            col = torch.empty(self.nk + 1, dtype=torch.int32, device=dev)
+            rank = torch.empty(self.nq, self.nk, dtype=torch.int32, device=dev)
+            lib = _lib.load()
+            with torch.cuda.device(dev):
+                self.wait_ready(dev)
+                cmap = self.as_c()
+                _lib.check(lib.flexattn_build_ds_index(C.byref(cmap), col.data_ptr(), rank.data_ptr(),
+                                                       torch.cuda.current_stream(dev).cuda_stream), lib)
+                pairs = int(col[-1].item())
+            self._ds_index = (col, rank, pairs)
+        return self._ds_index
+
+    def ds_index_c(self) -> _lib.DsIndexC:
+        col, rank, pairs = self.ds_index()
+        return _lib.DsIndexC(col.data_ptr(), rank.data_ptr(), pairs)
 
     def as_c(self) -> _lib.BlockMapC:
         return _lib.BlockMapC(self.state.data_ptr(), self.kv_cnt.data_ptr(), self.kv_idx.data_ptr(),
@@ -107,8 +140,11 @@ def mask_spec_c(spec: MaskSpec, Sq: int, Sk: int, device) -> _lib.MaskSpecC:
         ids_k = spec.doc_ids_k if spec.doc_ids_k is not None else spec.doc_ids
         if len(spec.doc_ids) < Sq or len(ids_k) < Sk:
             raise ValueError(f"document ids cover {len(spec.doc_ids)} q / {len(ids_k)} kv positions, need {Sq} / {Sk}")
-        doc_q = doc_ids_on(spec.doc_ids, device).data_ptr()
-        doc_k = doc_ids_on(ids_k, device).data_ptr()
+        tq, tk = doc_ids_on(spec.doc_ids, device), doc_ids_on(ids_k, device)
+        cur = torch.cuda.current_stream(device)
+        tq.record_stream(cur)   # (cached arrays may be evicted while a kernel on this stream still reads them)
+        tk.record_stream(cur)
+        doc_q, doc_k = tq.data_ptr(), tk.data_ptr()
     return _lib.MaskSpecC(spec.flags, spec.window, spec.stride, 0, doc_q, doc_k)
 
 

@@ -178,18 +178,24 @@ static bool ds_exchange_ok(const flexattn_bwd_params* p) {
   int bq = 0, bk = 0;
   bwd_dkv_bf16_d128_tile(&bq, &bk);
   if (p->Sq % bq != 0 || p->Sk % bk != 0) return false;
+  if (p->ds_index.pairs <= 0 || p->ds_index.pairs > (int64_t)(p->Sq / bq) * (p->Sk / bk)) return false;
   return p->Sq / bq <= 1024 && p->Sk / bk <= 1024;  // (both kernels cache a tile list in LDS)
 #endif
 }
 
+// one block of block_q x block_k bf16 values per (query head, kept tile pair)
 static int64_t ds_bytes_of(const flexattn_bwd_params* p) {
-  return (int64_t)p->B * p->Hq * (int64_t)p->Sq * (int64_t)p->Sk * 2;
+  int bq = 0, bk = 0;
+  bwd_dkv_bf16_d128_tile(&bq, &bk);
+  return (int64_t)p->B * p->Hq * p->ds_index.pairs * bq * bk * 2;
 }
 
 static int check_ds(const flexattn_bwd_params* p) {
   if (p->ds == nullptr) return FLEXATTN_OK;
   if (!ds_exchange_ok(p))
     return set_error(FLEXATTN_EINVAL, "ds given, but the kernels of this request exchange no dS (flexattn_bwd_ds_bytes is 0)");
+  if (p->ds_index.col == nullptr || p->ds_index.rank == nullptr)
+    return set_error(FLEXATTN_EINVAL, "ds given without ds_index.col / ds_index.rank (flexattn_build_ds_index)");
   if (p->ds_bytes < ds_bytes_of(p))
     return set_error(FLEXATTN_EINVAL, "ds holds %lld bytes, the request needs %lld", (long long)p->ds_bytes,
                      (long long)ds_bytes_of(p));
@@ -211,6 +217,9 @@ static int to_bwd_args(const flexattn_bwd_params* p, int pass, BwdArgs* a) {
   if ((rc = check_mask(p->mask)) != FLEXATTN_OK) return rc;
   if ((rc = check_bias(p->ab, p->B, p->Hq, p->Sq, p->Sk)) != FLEXATTN_OK) return rc;
   a->ds = p->ds;
+  a->ds_col = p->ds_index.col;
+  a->ds_rank = p->ds_index.rank;
+  a->ds_pairs = p->ds_index.pairs;
   a->q = p->q; a->k = p->k; a->v = p->v; a->dout = p->dout;
   a->l = p->l; a->m = p->m; a->delta = p->delta;
   a->dq = p->dq; a->dk = p->dk; a->dv = p->dv;
@@ -317,6 +326,14 @@ int flexattn_build_block_mask(const flexattn_mask_spec* mask, int32_t Sq, int32_
   if (rc != FLEXATTN_OK) return rc;
   return build_block_mask(to_args(*mask), Sq, Sk, block_q, block_k, state, kv_cnt, kv_idx, q_cnt, q_idx,
                           static_cast<hipStream_t>(stream));
+}
+
+int flexattn_build_ds_index(const flexattn_block_map* map, int32_t* col, int32_t* rank, void* stream) {
+  if (map == nullptr || col == nullptr || rank == nullptr) return set_error(FLEXATTN_EINVAL, "map, col or rank is NULL");
+  if (map->state == nullptr || map->q_cnt == nullptr || map->q_idx == nullptr)
+    return set_error(FLEXATTN_EINVAL, "block map lacks state or q_cnt/q_idx");
+  if (map->nq <= 0 || map->nk <= 0) return set_error(FLEXATTN_EINVAL, "block map of %d x %d tiles", map->nq, map->nk);
+  return build_ds_index(map->state, map->q_cnt, map->q_idx, map->nq, map->nk, col, rank, static_cast<hipStream_t>(stream));
 }
 
 int flexattn_fwd(const flexattn_fwd_params* p, void* stream) {

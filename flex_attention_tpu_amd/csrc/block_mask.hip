@@ -106,6 +106,38 @@ __global__ __launch_bounds__(64) void block_mask_kernel(MaskArgs mk, int nq, int
   if (cnt != nullptr && lane == 0) cnt[major] = total;
 }
 
+// Index of the dS exchange buffer over the kept tile pairs of a block map, counted kv tile by kv tile:
+// col[kb] = kept pairs in the kv tiles before kb (col[nk] = all of them), rank[qb, kb] = col[kb] + position of
+// qb in kb's q list, -1 for skipped pairs.  Work-group kb < nk owns column kb; work-group nk writes the total.
+__global__ __launch_bounds__(256) void ds_index_kernel(const uint8_t* state, const int* q_cnt, const int* q_idx, int nq,
+                                                       int nk, int* col, int* rank) {
+  __shared__ int part[256];
+  const int kb = blockIdx.x;
+  const int tid = threadIdx.x;
+  int sum = 0;
+  for (int k = tid; k < kb; k += 256) sum += q_cnt[k];
+  part[tid] = sum;
+  __syncthreads();
+  for (int step = 128; step > 0; step >>= 1) {
+    if (tid < step) part[tid] += part[tid + step];
+    __syncthreads();
+  }
+  const int first = part[0];
+  if (tid == 0) col[kb] = first;
+  if (kb == nk) return;
+  // (skipped pairs and kept pairs are written by disjoint threads: a pair is in the list exactly when its state is not 0)
+  for (int qb = tid; qb < nq; qb += 256)
+    if (state[(size_t)qb * nk + kb] == 0) rank[(size_t)qb * nk + kb] = -1;
+  const int n = q_cnt[kb];
+  for (int t = tid; t < n; t += 256) rank[(size_t)q_idx[(size_t)kb * nq + t] * nk + kb] = first + t;
+}
+
+int build_ds_index(const uint8_t* state, const int* q_cnt, const int* q_idx, int nq, int nk, int* col, int* rank,
+                   hipStream_t stream) {
+  hipLaunchKernelGGL(ds_index_kernel, dim3(nk + 1), dim3(256), 0, stream, state, q_cnt, q_idx, nq, nk, col, rank);
+  return check_launch("flexattn_build_ds_index");
+}
+
 int build_block_mask(const MaskArgs& mask, int Sq, int Sk, int block_q, int block_k, uint8_t* state,
                      int* kv_cnt, int* kv_idx, int* q_cnt, int* q_idx, hipStream_t stream) {
   const int nq = Sq / block_q, nk = Sk / block_k;

@@ -326,7 +326,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
 // DOCS: the mask compares document ids; those of a partial q tile are staged through LDS (stage_doc_ids).
 // (A template parameter: the staging code in the kernel costs the other masks registers.)
 // EXPORT: the streams also write the step's bf16 dS (without sm_scale, as the dk product takes it) to a.ds, one
-// 32 KB block per (query head, q tile, kv tile) at ((head nq + q tile) nk + kv tile) 32 KB; inside a block wave w
+// 32 KB block per (query head, kept tile pair) at (head a.ds_pairs + a.ds_col[kv tile] + place of the q tile in the
+// kv tile's list) 32 KB (the index of flexattn_build_ds_index: skipped pairs take no room); inside a block wave w
 // (kv columns 32 w + L % 32) writes 1 KB per (32-row q block c, 16-row half u) at 8192 w + 1024 (2 c + u), lane L
 // its 8 values (rows 8 (e / 4) + 4 (L / 32) + e % 4 of the half) at 16 (2 (L % 32) + L / 32).  bwd_dq_ds.hip reads it.
 template <int SCORE, bool DOCS, bool EXPORT = false>
@@ -390,9 +391,12 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     return g;
   };
   auto kv_offset = [&](const Geometry& g) { return ((size_t)g.bhk * a.Sk + (size_t)g.kb * BNK) * D; };
-  // (EXPORT) dS block of the item's kv tile against q tile 0 of the group's first query head
+  // (EXPORT) dS block of the item's kv tile against the first q tile of its list, for the group's first query
+  // head: the blocks of a head are ordered kv tile by kv tile (a.ds_col[kb] pairs lie before kv tile kb), and
+  // along each kv tile's q list
   auto ds_base = [&](const Geometry& g) {
-    return static_cast<char*>(a.ds) + (((size_t)g.bhk * group) * nQ * nKb + (size_t)g.kb) * kDsBlockBytes;
+    const int first = __builtin_amdgcn_readfirstlane(a.ds_col[g.kb]);
+    return static_cast<char*>(a.ds) + (((size_t)g.bhk * group) * (size_t)a.ds_pairs + (size_t)first) * kDsBlockBytes;
   };
   // first row of the group's first query head: (b Hq + hk group) Sq with bhk = b Hkv + hk
   auto first_row = [&](const Geometry& g) { return (size_t)g.bhk * group * a.Sq; };
@@ -557,6 +561,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   fetch(geo_n, pre);
 
   const unsigned tid4 = (unsigned)row * 4u;
+  // (EXPORT) first dS block of this item and of the next one
+  const size_t ds_item = EXPORT ? (size_t)ds_base(geo) : 0;
+  const size_t ds_item_n = EXPORT ? (size_t)ds_base(geo_n) : 0;
   // Work-group constants of the run loop, one 32-dword table per wave behind the row values
   // (order: TABLE in gen_dkv_tile.py; the second half names the next item's first step, see below).
   // Written and read by the same wave: no barrier needed.
@@ -579,11 +586,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     tbl[14] = (unsigned)(size_t)rowb;
     tbl[15] = (unsigned)((size_t)rowb >> 32);
     if (EXPORT) {
-      const size_t ds0 = (size_t)ds_base(geo);
+      const size_t ds0 = ds_item;
       tbl[28] = (unsigned)ds0;
       tbl[29] = (unsigned)(ds0 >> 32);
-      tbl[30] = (unsigned)(nQ * nKb);
-      tbl[31] = (unsigned)nKb;
+      tbl[30] = (unsigned)a.ds_pairs;   // blocks per query head
+      tbl[31] = 0u;
     }
   }
   const unsigned tbl_addr = (unsigned)(size_t)tbl;
@@ -667,7 +674,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
             tbl[27] = (unsigned)(geo_n.kb * BNK + BNK / 2);
           }
           if (EXPORT) {
-            const size_t ds_n = (size_t)ds_base(geo_n);
+            const size_t ds_n = ds_item_n;
             tbl[26] = (unsigned)ds_n;
             tbl[27] = (unsigned)(ds_n >> 32);
           }
@@ -690,8 +697,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
 #define FA_DKV_ALIBI_CLOBBERS , "s101"
 #define FA_DKV_DS_CLOBBERS , "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59"
     if constexpr (EXPORT) {
-      // dS block of step `it` (head it / n_tiles of the group, q tile qb) and the lane's place in the wave's part
-      const size_t ds_cur = (size_t)ds_base(geo) + ((size_t)(it / n_tiles) * nQ + (size_t)qb) * nKb * kDsBlockBytes;
+      // dS block of step `it` (head it / n_tiles of the group, place p0 in the q list) and the lane's place in
+      // the wave's part
+      const size_t ds_cur = ds_item + ((size_t)(it / n_tiles) * (size_t)a.ds_pairs + (size_t)p0) * kDsBlockBytes;
       const unsigned dslo = (unsigned)ds_cur, dshi = (unsigned)(ds_cur >> 32);
       const unsigned dsv = 8192u * (unsigned)w + 4096u + 16u * (unsigned)(2 * l32 + hh);
       if constexpr (SOFTCAP) {

@@ -2,8 +2,9 @@
 // instead of the three of the recomputing dq kernel (S = Q K^T, dP = dO V^T, dq += dS K).
 //
 // The dk/dv stream kernel (bwd_dkv_bf16.hip, EXPORT) leaves every step's bf16 dS in a buffer of 32 KB blocks, one
-// per (query head, 128-row q tile, 128-column kv tile) in the register layout it has there (a lane owns one kv
-// column).  This kernel walks a q tile's row list of the same 128 x 128 block map, copies dS blocks and K tiles
+// per (query head, kept pair of a 128-row q tile and a 128-column kv tile) in the register layout it has there (a
+// lane owns one kv column); block of pair (qb, kb) of head bh: bh ds_pairs + ds_rank[qb nk + kb].
+// This kernel walks a q tile's row list of the same 128 x 128 block map, copies dS blocks and K tiles
 // global -> LDS (global_load_lds_dwordx4, no registers in between) through rings of stages, and reads both
 // operands with transposing LDS reads: computed transposed, dq^T[d, i] += sum_j K^T[d, j] dS^T[j, i], the lane
 // that owned kv column j in the dk/dv kernel wrote 8 q rows of it contiguously, which is what
@@ -46,6 +47,7 @@ constexpr size_t kDsBlockBytes = (size_t)BQ * BNK * 2;
 static_assert(NK >= 2 && NDS >= 2 && NDS <= 17 && NK <= 10, "the wait counts are written for up to 15 stages behind");
 static_assert(LDS_BYTES <= 160 * 1024 / OCC, "the rings must fit the CU's LDS");
 static_assert(NDS * DS_STAGE_BYTES >= 4 * 8192, "the epilogue stages 8 KB per wave in the dS ring");
+static_assert(MAX_LIST == 1024, "a list entry packs the kv tile into 10 bits");
 }  // namespace dqds_cfg
 
 #ifndef FLEXATTN_CUSTOM_ONLY
@@ -76,12 +78,17 @@ __global__ __launch_bounds__(256, dqds_cfg::OCC) void bwd_dq_from_ds_kernel(BwdA
   const int group = a.Hq / a.Hkv;
   const int bhk = (bh / a.Hq) * a.Hkv + (bh % a.Hq) / group;
 
+  // the q tile's list in LDS: kv tile (10 bits, nk <= 1024) and the dS block of the pair (22 bits: at most 2^20 pairs)
   const int n_list = a.map.cnt[qb];
   const int* list = a.map.idx + (size_t)qb * nK;
-  for (int t = tid; t < n_list; t += 256) sIdx[t] = list[t];
+  const int* rank = a.ds_rank + (size_t)qb * nK;
+  for (int t = tid; t < n_list; t += 256) {
+    const int kb = list[t];
+    sIdx[t] = kb | (rank[kb] << 10);
+  }
   __syncthreads();
 
-  const char* ds_row = static_cast<const char*>(a.ds) + ((size_t)bh * nQ + qb) * nK * kDsBlockBytes;
+  const char* ds_row = static_cast<const char*>(a.ds) + (size_t)bh * (size_t)a.ds_pairs * kDsBlockBytes;
   const bf16_t* Kg = static_cast<const bf16_t*>(a.k) + (size_t)bhk * a.Sk * D;
   const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char*)(smem_raw);
   const unsigned lane16 = (unsigned)lane * 16u;
@@ -100,13 +107,14 @@ __global__ __launch_bounds__(256, dqds_cfg::OCC) void bwd_dq_from_ds_kernel(BwdA
   // rows.  A wave's copies complete in issue order, so a copy from the L2 issued behind copies from HBM would
   // wait for those: waves 0, 1 copy only dS (four pieces each), waves 2, 3 only K, and each kind runs as far ahead
   // as its ring allows.
-  auto tile_of = [&](int s) { return __builtin_amdgcn_readfirstlane(sIdx[s / PARTS]); };
+  auto tile_of = [&](int s) { return __builtin_amdgcn_readfirstlane(sIdx[s / PARTS] & 1023); };
+  auto block_of = [&](int s) { return __builtin_amdgcn_readfirstlane((int)((unsigned)sIdx[s / PARTS] >> 10)); };
   const bool ds_wave = w < 2;
   auto issue = [&](int s) {
     const char* src;
     unsigned dst;
     if (ds_wave) {
-      src = ds_row + (size_t)tile_of(s) * kDsBlockBytes + (size_t)(s % PARTS) * DS_STAGE_BYTES;
+      src = ds_row + (size_t)block_of(s) * kDsBlockBytes + (size_t)(s % PARTS) * DS_STAGE_BYTES;
       dst = lds0 + (unsigned)(s % NDS) * DS_STAGE_BYTES + (unsigned)w * 4096u;
     } else {
       src = reinterpret_cast<const char*>(Kg + ((size_t)tile_of(s) * BNK + (size_t)(s % PARTS) * STAGE_KV) * D);
@@ -241,6 +249,8 @@ int bwd_dq_from_ds(const BwdArgs& a, float out_scale, hipStream_t stream) {
 #else
   using namespace dqds_cfg;
   if (a.map.nk > MAX_LIST) return set_error(FLEXATTN_ENOTSUP, "dq from dS: %d kv tiles, at most %d", a.map.nk, MAX_LIST);
+  if (a.ds_rank == nullptr || a.ds_pairs <= 0 || a.ds_pairs > (1ll << 20))
+    return set_error(FLEXATTN_EINVAL, "dq from dS: no index of the dS blocks (or more than 2^20 kept tile pairs)");
   auto kern = bwd_dq_from_ds_kernel;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);

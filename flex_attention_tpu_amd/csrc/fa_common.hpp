@@ -84,6 +84,11 @@ struct BwdArgs {
   const float* l; const float* m; const float* delta;
   void* dq; void* dk; void* dv;
   void* ds;   // dS exchange buffer (bf16 kernels that can use one), or null
+  // its index over the kept tile pairs of the dk/dv kernel's block map: block of pair (q head bh, q tile qb,
+  // kv tile kb) = bh ds_pairs + ds_rank[qb nk + kb], with ds_rank = ds_col[kb] + position of qb in kb's q list
+  const int* ds_col;
+  const int* ds_rank;
+  long long ds_pairs;
   int B, Hq, Hkv, Sq, Sk;
   float sm_scale;
   int flags;  // FLEXATTN_FLAG_*

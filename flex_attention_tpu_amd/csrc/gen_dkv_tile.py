@@ -91,10 +91,11 @@ S_KC = "s101"     # (position-bias variant) 128 kb + 64: the middle of the item'
 S_CAP, S_K2 = "s64", "s101"
 CAP_SOFTCAP = 8   # instructions per MFMA gap in the softcap variant (8 VALU ops per element instead of 2)
 # dS export variant: the step's bf16 dS (the B operand registers of the dk product) also goes to a buffer in
-# global memory, one 32 KB block per (query head, q tile, kv tile), from which the dq pass takes it.  Block of
-# the step: item base + ((head inside the group) nq nk + (q tile) nk) 32 KB; wave w writes bytes [8192 w, + 8192),
+# global memory, one 32 KB block per (query head, kept tile pair), from which the dq pass takes it.  The blocks of
+# a head are ordered kv tile by kv tile and along each kv tile's q list.  Block of the step: item base + ((head
+# inside the group) pairs + (place in the q list)) 32 KB; wave w writes bytes [8192 w, + 8192),
 # 1 KB per (q block c, half u) at (2 c + u) 1024, lane L at 16 (2 (L % 32) + L / 32).
-S_DSB, S_NQNK, S_NK, S_DS, S_DSN = "s[52:53]", "s54", "s55", "s[56:57]", "s[58:59]"
+S_DSB, S_PAIRS, S_DS, S_DSN = "s[52:53]", "s54", "s[56:57]", "s[58:59]"
 V_QB2 = 67      # q block index of the step after the next one, across the stream
 ROW_SLOT = 28   # MFMA slot at which the next step's lse / delta values are turned around
 V_ROW = 144     # 4 temporaries for that, inside pb[1] (first written by E(1), after ROW_SLOT)
@@ -402,15 +403,17 @@ def run_loop(full, masked, alibi=False, softcap=False, export=False):
     switch_sgprs = ([f"v_readfirstlane_b32 s64, {vr(V_TBL + 10)}", f"v_readfirstlane_b32 {S_KC}, {vr(V_TBL + 11)}"] if alibi else [])
     ds_next = []
     if export:
-        # table dwords 28-31: the item's first dS block (two dwords), blocks per head nq nk, blocks per q tile nk;
-        # dwords 26, 27: the next item's first dS block; %[dslo], %[dshi]: the block of the run's first step
+        # table dwords 28-30: the item's first dS block (two dwords: first query head of the group, first entry of the
+        # kv tile's q list), blocks per head (the kept tile pairs of the map); dwords 26, 27: the next item's first dS
+        # block; %[dslo], %[dshi]: the block of the run's first step
         entry = ([f"ds_read_b128 {vr(V_TBL + 16, 4)}, %[tbl] offset:112"] + entry
                  + [f"v_readfirstlane_b32 s{52 + i}, {vr(V_TBL + 16 + i)}" for i in range(4)]
                  + ["v_readfirstlane_b32 s56, %[dslo]", "v_readfirstlane_b32 s57, %[dshi]"])
         switch_sgprs = [f"v_readfirstlane_b32 s52, {vr(V_TBL + 10)}", f"v_readfirstlane_b32 s53, {vr(V_TBL + 11)}"]
-        # dS block of the next step: item base + (min(g1, gmax) nq nk + qb1 nk) 32 KB
-        ds_next = [f"s_min_u32 {t0}, s78, s61", f"s_mul_i32 {t0}, {t0}, {S_NQNK}", f"s_mul_i32 {t1}, s80, {S_NK}",
-                   f"s_add_u32 {t0}, {t0}, {t1}", f"s_lshl_b32 {t2}, {t0}, 15", f"s_lshr_b32 {t3}, {t0}, 17",
+        # dS block of the next step: item base + (min(g1, gmax) pairs + p1) 32 KB: the blocks of a kv tile follow its
+        # q list (p1 = the next step's place in it; 0 where the next step is the next item's first)
+        ds_next = [f"s_min_u32 {t0}, s78, s61", f"s_mul_i32 {t0}, {t0}, {S_PAIRS}",
+                   f"s_add_u32 {t0}, {t0}, s77", f"s_lshl_b32 {t2}, {t0}, 15", f"s_lshr_b32 {t3}, {t0}, 17",
                    f"s_add_u32 s58, s52, {t2}", f"s_addc_u32 s59, s53, {t3}"]
     top = entry + [
         ".Lfa_dkv_loop_%=:",

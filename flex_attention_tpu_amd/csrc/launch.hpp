@@ -38,4 +38,7 @@ int bwd_delta(const void* o, const void* dout, float* delta, int64_t rows, int D
 int build_block_mask(const MaskArgs& mask, int Sq, int Sk, int block_q, int block_k, uint8_t* state,
                      int* kv_cnt, int* kv_idx, int* q_cnt, int* q_idx, hipStream_t stream);
 
+int build_ds_index(const uint8_t* state, const int* q_cnt, const int* q_idx, int nq, int nk, int* col, int* rank,
+                   hipStream_t stream);
+
 }  // namespace fa

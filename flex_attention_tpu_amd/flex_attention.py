@@ -21,9 +21,9 @@ from .flex_attention_kernel import _flex_attention_impl
 
 
 # The backward hands dS from the dk/dv pass to the dq pass (DsBlocks in flex_attention_dq_bwd.py) when both
-# gradients are wanted, the hand-over is expected to pay (ds_exchange_pays) and the buffer, B Hq Sq Sk bf16
-# values, stays below this many bytes.
-DS_EXCHANGE_MAX_BYTES = 32 << 30
+# gradients are wanted and the hand-over is expected to pay (ds_exchange_pays).  The buffer holds one 32 KB block
+# per query head and kept pair of 128 x 128 tiles (what the mask skips takes no room); the dk/dv entry point
+# declines it, and the dq pass recomputes, when it would take more than half of the free device memory.
 
 
 class _FlexAttention(torch.autograd.Function):
@@ -47,9 +47,7 @@ class _FlexAttention(torch.autograd.Function):
         di = compute_delta(o, do)  # float32 [B, H, Sq]  (jax_exp.py:276-278)
         dq = dk = dv = ds = None
         if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
-            pad = lambda n: -(-n // 128) * 128
-            exchange = (ctx.needs_input_grad[0] and ds_exchange_pays(score_fn, mask_fn, segment_ids) and
-                        2 * q.shape[0] * q.shape[1] * pad(q.shape[2]) * pad(k.shape[2]) <= DS_EXCHANGE_MAX_BYTES)
+            exchange = ctx.needs_input_grad[0] and ds_exchange_pays(score_fn, mask_fn, segment_ids)
             dk, dv, ds = flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, block_b=1, block_q=block_q,
                                                  block_q_major=block_q, block_k_major=block_k, block_k=block_k,
                                                  sm_scale=sm_scale, causal=causal, debug=False, score_fn=score_fn,

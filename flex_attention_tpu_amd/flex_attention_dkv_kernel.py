@@ -10,7 +10,7 @@ import torch
 from . import _lib
 from ._common import (batch_entry, bias_c, check_blocks, check_qkv, check_rows, kernel_block_map, kernel_head_dim, library_for, pad_seq,
                       padded_len, per_batch_segments, resolve_mask, stream_of)
-from .flex_attention_dq_bwd import DsBlocks, bwd_params
+from .flex_attention_dq_bwd import DsBlocks, alloc_ds, bwd_params
 
 
 def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=None, block_q, block_q_major,
@@ -22,7 +22,8 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     (the reference's north-star file ignores it; its mask-aware twin gets the same effect from
     ``mask_fn``).  ``return_ds=True`` returns (dk, dv, ds): ds is the pass's dS as a DsBlocks for
     ``flex_attention_bwd_dq(..., ds=ds)``, or None when the kernels of the call exchange nothing (fp32, position
-    biases, ``ab``, compiled score functions): the dq pass then recomputes as usual."""
+    biases, ``ab``, compiled score functions) or the device has too little free memory for the buffer (one 32 KB
+    block per query head and kept pair of 128 x 128 tiles): the dq pass then recomputes as usual."""
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v, do)
     rows = per_batch_segments(segment_ids, B)
     if rows is not None:  # ids differ between batch entries: one launch per entry
@@ -56,10 +57,16 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     with torch.cuda.device(q.device):
         lib = library_for(score_fn, spec)
         if return_ds:
-            need = lib.flexattn_bwd_ds_bytes(C.byref(p))
-            if need > 0:
-                ds = DsBlocks(torch.empty(need, dtype=torch.uint8, device=q.device), (B, Hq, Sq_p, Sk_p))
-                p.ds, p.ds_bytes = ds.buf.data_ptr(), need
+            p.ds_index.pairs = 1   # (asks whether the kernels of the call exchange at all, before the index is built)
+            if lib.flexattn_bwd_ds_bytes(C.byref(p)) > 0:
+                p.ds_index = bm.ds_index_c()
+                need = lib.flexattn_bwd_ds_bytes(C.byref(p))
+                buf = alloc_ds(need, q.device)
+                if buf is not None:
+                    ds = DsBlocks(buf, (B, Hq, Sq_p, Sk_p), index=bm.ds_index())
+                    p.ds, p.ds_bytes = buf.data_ptr(), need
+            if ds is None:
+                p.ds_index = _lib.DsIndexC()
         _lib.check(lib.flexattn_bwd_dkv(C.byref(p), stream_of(q)), lib)
     if Sk_p != Sk or D != D_user:
         dk, dv = dk[:, :, :Sk, :D_user].contiguous(), dv[:, :, :Sk, :D_user].contiguous()

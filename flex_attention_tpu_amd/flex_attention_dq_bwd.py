@@ -36,8 +36,27 @@ class DsBlocks:
     The reference's two backward kernels each recompute S, dP and dS (flex_attention_dq_bwd.py:340-378,
     flash_attention_dkv_bwd.py:232-302); handing dS over leaves the dq pass one contraction instead of three."""
 
-    def __init__(self, buf=None, shape=None, entries=None):
-        self.buf, self.shape, self.entries = buf, shape, entries
+    def __init__(self, buf=None, shape=None, entries=None, index=None):
+        self.buf, self.shape, self.entries, self.index = buf, shape, entries, index
+
+
+# The dS buffer is never allowed to take more than this share of the device memory that is free when it is
+# asked for: the backward must not fail for want of memory where the recomputing dq pass would have worked.
+DS_FREE_MEMORY_SHARE = 0.5
+
+
+def alloc_ds(nbytes: int, device):
+    """The dS exchange buffer, or None when it does not fit comfortably: more than DS_FREE_MEMORY_SHARE of the
+    memory that is free (the driver's figure plus what torch's allocator holds unused), or an out-of-memory error
+    from the allocator all the same.  The caller then runs the two recomputing passes."""
+    free, _ = torch.cuda.mem_get_info(device)
+    cached = torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)
+    if nbytes > DS_FREE_MEMORY_SHARE * (free + cached):
+        return None
+    try:
+        return torch.empty(nbytes, dtype=torch.uint8, device=device)
+    except torch.cuda.OutOfMemoryError:
+        return None
 
 
 def ds_exchange_pays(score_fn, mask_fn=None, segment_ids=None) -> bool:
@@ -101,7 +120,7 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     l, m, d = pad_seq(l, Sq_p), pad_seq(m, Sq_p), pad_seq(d, Sq_p)
     D_user, D = D, kernel_head_dim(D, q.dtype)   # smaller head dimensions: zero-padded columns
     q, do, k, v = pad_seq(q, D, 3), pad_seq(do, D, 3), pad_seq(k, D, 3), pad_seq(v, D, 3)
-    if ds is not None and (ds.buf is None or ds.shape != (B, Hq, Sq_p, Sk_p) or ds.buf.device != q.device):
+    if ds is not None and (ds.buf is None or ds.index is None or ds.shape != (B, Hq, Sq_p, Sk_p) or ds.buf.device != q.device):
         raise ValueError("ds does not come from a dk/dv pass of these arguments")
     # (the dS blocks lie at the dk/dv kernel's tiles: the dq pass walks that map's row lists)
     bm = kernel_block_map(_lib.PASS_DKV if ds is not None else _lib.PASS_DQ, spec, q, Sq_p, Sk_p, D, score_fn)
@@ -111,6 +130,8 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
                    compiled_loop=compiled_loop, ab_c=ab_c)
     if ds is not None:
         p.ds, p.ds_bytes = ds.buf.data_ptr(), ds.buf.numel()
+        col, rank, pairs = ds.index   # (the index the dk/dv pass wrote the blocks by)
+        p.ds_index = _lib.DsIndexC(col.data_ptr(), rank.data_ptr(), pairs)
     with torch.cuda.device(q.device):
         lib = library_for(score_fn, spec)
         _lib.check(lib.flexattn_bwd_dq(C.byref(p), stream_of(q)), lib)

@@ -7,6 +7,7 @@ sequence length and pass.  FLOPs and bytes follow the reference's conventions: c
 S^2 / 2 pairs; forward 4 D per pair, dq 6 D, dk/dv 8 D; bytes = every operand and result moved once.
 
     python -m flex_attention_tpu_amd.roofline --out roofline_mi355x.csv [--max-seq 65536] [--plot roofline.png]
+    python -m flex_attention_tpu_amd.roofline --from-csv roofline_mi355x.csv --plot roofline.png   # plot only, no GPU
 """
 from __future__ import annotations
 
@@ -80,6 +81,13 @@ def write_csv(rows, path):
             w.writerow(r)
 
 
+def read_csv(path):
+    """Rows of a CSV written by write_csv (numbers parsed back)."""
+    with open(path, newline="") as f:
+        return [{k: (v if k == "Pass" else (int(v) if k == "SeqLen" else float(v))) for k, v in r.items()}
+                for r in csv.DictReader(f)]
+
+
 def plot(rows, path):
     """Log-log roofline (memory slope and MFMA ceiling) with the measured points; needs matplotlib."""
     import matplotlib
@@ -91,8 +99,12 @@ def plot(rows, path):
     for name, mark in (("fwd", "o"), ("dq", "s"), ("dkv", "^")):
         pts = [r for r in rows if r["Pass"] == name]
         plt.loglog([r["Intensity"] for r in pts], [r["TFLOPs"] for r in pts], mark + "-", label=name)
+    fwd = [r for r in rows if r["Pass"] == "fwd"]
+    for r in (fwd[0], fwd[-1]) if fwd else ():
+        plt.annotate(f"S={r['SeqLen']}", (r["Intensity"], r["TFLOPs"]), textcoords="offset points", xytext=(4, -12), fontsize=7)
     plt.xlabel("arithmetic intensity (FLOP / byte)")
     plt.ylabel("TFLOP/s")
+    plt.title("flex attention on MI355X: bf16, causal, B=1, H=8, D=128, S = 1k ... 256k", fontsize=9)
     plt.legend()
     plt.grid(True, which="both", alpha=0.3)
     plt.tight_layout()
@@ -107,9 +119,13 @@ def main():
     ap.add_argument("--heads", type=int, default=8)
     ap.add_argument("--iters", type=int, default=10)
     ap.add_argument("--plot", default=None, help="also write a roofline plot (PNG; needs matplotlib)")
+    ap.add_argument("--from-csv", default=None, help="plot the rows of this CSV instead of measuring (no GPU needed)")
     args = ap.parse_args()
-    rows = sweep(args.max_seq, args.min_seq, args.heads, args.iters)
-    write_csv(rows, args.out)
+    if args.from_csv:
+        rows = read_csv(args.from_csv)
+    else:
+        rows = sweep(args.max_seq, args.min_seq, args.heads, args.iters)
+        write_csv(rows, args.out)
     if args.plot:
         plot(rows, args.plot)
 

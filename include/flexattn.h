@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FLEXATTN_VERSION 102 /* major*10000 + minor*100 + patch */
+#define FLEXATTN_VERSION 103 /* major*10000 + minor*100 + patch */
 
 /* status codes */
 #define FLEXATTN_OK 0
@@ -122,6 +122,17 @@ typedef struct flexattn_fwd_params {
   flexattn_bias ab;
 } flexattn_fwd_params;
 
+/* Index of the dS exchange buffer (see flexattn_bwd_ds_bytes) over the kept tile pairs of the dk/dv pass's block
+ * map, as produced by flexattn_build_ds_index: the buffer holds one 32 KB block per (query head, kept pair),
+ * block of (head bh, q tile qb, kv tile kb) = bh * pairs + rank[qb * nk + kb].  The reference's tiled backward
+ * kernels keep O(block) state (flex_attention_dq_bwd.py:325-380); this buffer is the one O(kept tiles) object of
+ * the build, and it is only as large as the mask leaves it. */
+typedef struct flexattn_ds_index {
+  const int32_t* col;  /* device [nk + 1]: kept pairs in the kv tiles before kb; col[nk] = pairs */
+  const int32_t* rank; /* device [nq, nk]: col[kb] + position of qb in kb's q list; -1 for skipped pairs */
+  int64_t pairs;       /* number of kept pairs (the caller reads col[nk] back once per map) */
+} flexattn_ds_index;
+
 typedef struct flexattn_bwd_params {
   const void* q; const void* k; const void* v; const void* dout;
   const float* l; const float* m; const float* delta; /* [B,Hq,Sq] */
@@ -139,6 +150,7 @@ typedef struct flexattn_bwd_params {
   /* dS exchange buffer, or NULL (see flexattn_bwd_ds_bytes): written by flexattn_bwd_dkv, read by flexattn_bwd_dq */
   void* ds;
   int64_t ds_bytes;
+  flexattn_ds_index ds_index; /* needed with ds; for the map at the granularity of FLEXATTN_PASS_DKV */
 } flexattn_bwd_params;
 
 #define FLEXATTN_PASS_FWD 0
@@ -193,13 +205,19 @@ int flexattn_fwd_noalloc(const flexattn_fwd_params* p, void* stream);
 int flexattn_bwd_delta(const void* o, const void* dout, float* delta, int64_t rows, int32_t D,
                        int32_t dtype, void* stream);
 
+/* Builds the index of the dS exchange buffer for a block map at the granularity of FLEXATTN_PASS_DKV (state, q_cnt
+ * and q_idx are read): col [nk + 1] and rank [nq * nk] are caller-allocated device int32 arrays.  No counterpart
+ * in the reference (its backward kernels exchange nothing). */
+int flexattn_build_ds_index(const flexattn_block_map* map, int32_t* col, int32_t* rank, void* stream);
+
 /* dS exchange between the two backward passes.  The reference's dq and dk/dv kernels each recompute S, dP and dS
  * (flex_attention_dq_bwd.py:340-378, flash_attention_dkv_bwd.py:232-302).  Here the dk/dv pass can leave its
  * bf16 dS in a caller-allocated device buffer `ds`, and a dq pass that is given the same buffer computes
  * dq = sm_scale dS K from it, one contraction instead of three.  Returns the bytes `ds` must hold for the request
- * described by p (B Hq Sq Sk 2; only shapes, dtype, D, flags, score and ab are looked at), or 0 when the
- * kernels of the request exchange nothing (fp32, position biases, an additive bias, compiled score functions,
- * FLEXATTN_FLAG_COMPILED_LOOP, more than 1024 tiles along a sequence): then ds must stay NULL.
+ * described by p (B Hq ds_index.pairs 32 KB: one block per query head and kept tile pair; only shapes, dtype, D,
+ * flags, score, ab and ds_index.pairs are looked at), or 0 when the kernels of the request exchange nothing
+ * (fp32, position biases, an additive bias, compiled score functions, FLEXATTN_FLAG_COMPILED_LOOP, more than
+ * 1024 tiles along a sequence, ds_index.pairs <= 0): then ds must stay NULL.
  * Order: flexattn_bwd_dkv with p->ds set, then flexattn_bwd_dq with the same p->ds on the same stream (or
  * ordered behind it); for that dq call p->map is the map at the granularity of FLEXATTN_PASS_DKV with its
  * kv_cnt / kv_idx lists.  With ds == NULL both passes work on their own as before. */

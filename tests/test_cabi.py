@@ -37,7 +37,8 @@ def test_struct_sizes_follow_c_layout():
     assert C.sizeof(_lib.BlockMapC) == 56
     assert C.sizeof(_lib.BiasC) == 32
     assert C.sizeof(_lib.FwdParamsC) == 6 * 8 + 10 * 4 + 32 + 32 + 56 + 32
-    assert C.sizeof(_lib.BwdParamsC) == 10 * 8 + 10 * 4 + 32 + 32 + 56 + 32 + 16
+    assert C.sizeof(_lib.DsIndexC) == 24
+    assert C.sizeof(_lib.BwdParamsC) == 10 * 8 + 10 * 4 + 32 + 32 + 56 + 32 + 16 + 24
 
 
 def test_tile_shapes(lib):
@@ -82,12 +83,19 @@ def test_error_codes_and_messages(lib):
 
 
 def test_ds_exchange_sizes_and_argument_checks(lib):
-    """flexattn_bwd_ds_bytes looks at shapes, dtype, score and flags only; a dS buffer on a request whose kernels
-    exchange nothing, or one that is too small, is refused before any launch."""
+    """flexattn_bwd_ds_bytes looks at shapes, dtype, score, flags and the number of kept tile pairs only (one 32 KB
+    block per query head and pair); a dS buffer on a request whose kernels exchange nothing, one without its
+    index, or one that is too small, is refused before any launch."""
     dummy = C.create_string_buffer(64)
     p = _lib.BwdParamsC()
     p.B, p.Hq, p.Hkv, p.Sq, p.Sk, p.D, p.dtype, p.sm_scale = 2, 4, 2, 256, 384, 128, _lib.BF16, 0.125
-    assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 2 * 4 * 256 * 384 * 2
+    assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 0          # no kept pairs named
+    p.ds_index.pairs = 5
+    assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 2 * 4 * 5 * 128 * 128 * 2
+    p.ds_index.pairs = 2 * 3 + 1                                # more pairs than the 2 x 3 tiles of the shape
+    assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 0
+    p.ds_index.pairs = 6
+    assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 2 * 4 * 256 * 384 * 2   # every pair kept: the dense size
     p.score.kind = _lib.SCORE_SOFTCAP
     assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 2 * 4 * 256 * 384 * 2
     for kind in (_lib.SCORE_ALIBI, _lib.SCORE_ALIBI_TILE):
@@ -103,13 +111,21 @@ def test_ds_exchange_sizes_and_argument_checks(lib):
     p.Sq = 1025 * 128                       # more than 1024 tiles along a sequence
     assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 0
     assert lib.flexattn_bwd_ds_bytes(None) == 0
-    # a buffer where none is exchanged, and one that is too small
+    # a buffer where none is exchanged, one without its index, and one that is too small
     p.Sq, p.dtype = 256, _lib.F32
     for f in ("q", "k", "v", "dout", "l", "m", "delta", "dq", "dk", "dv", "ds"):
         setattr(p, f, C.addressof(dummy))
     p.ds_bytes = 1 << 40
     for call in (lib.flexattn_bwd_dq, lib.flexattn_bwd_dkv):
         assert call(C.byref(p), None) == _lib.EINVAL and b"exchange no dS" in lib.flexattn_last_error_string()
-    p.dtype, p.ds_bytes = _lib.BF16, 2 * 4 * 256 * 384 * 2 - 1
+    p.dtype = _lib.BF16
+    for call in (lib.flexattn_bwd_dq, lib.flexattn_bwd_dkv):
+        assert call(C.byref(p), None) == _lib.EINVAL and b"ds_index" in lib.flexattn_last_error_string()
+    p.ds_index.col = p.ds_index.rank = C.addressof(dummy)
+    p.ds_bytes = 2 * 4 * 256 * 384 * 2 - 1
     for call in (lib.flexattn_bwd_dq, lib.flexattn_bwd_dkv):
         assert call(C.byref(p), None) == _lib.EINVAL and b"needs" in lib.flexattn_last_error_string()
+    # the index builder checks its arguments
+    assert lib.flexattn_build_ds_index(None, None, None, None) == _lib.EINVAL
+    m = _lib.BlockMapC()
+    assert lib.flexattn_build_ds_index(C.byref(m), C.addressof(dummy), C.addressof(dummy), None) == _lib.EINVAL

@@ -126,6 +126,50 @@ def test_block_mask_builder_matches_config_fixtures(F):
             assert torch.equal(run, gold), name
 
 
+def test_ds_index_builder_bit_exact(F):
+    """flexattn_build_ds_index: the blocks of the dS exchange buffer follow the kept tile pairs kv tile by kv tile
+    and along each kv tile's q list; skipped pairs get -1 and take no room.  Against a host enumeration."""
+    from flex_attention_tpu_amd import block_mask
+    S = 2048
+    for name, (mf, bf), _ in _mask_cases(S, 128, 128):
+        bm = block_mask.create_block_mask((mf, bf), S, S, 128, 128, DEV)
+        col, rank, pairs = bm.ds_index()
+        run = bm.run_mask().cpu().numpy()
+        nq, nk = run.shape
+        want_col = np.concatenate([[0], np.cumsum(run.sum(axis=0))]).astype(np.int32)
+        want_rank = np.full((nq, nk), -1, np.int32)
+        for kb in range(nk):
+            qs = np.nonzero(run[:, kb])[0]
+            want_rank[qs, kb] = want_col[kb] + np.arange(len(qs))
+        assert pairs == int(run.sum()), name
+        assert np.array_equal(col.cpu().numpy(), want_col), name
+        assert np.array_equal(rank.cpu().numpy(), want_rank), name
+
+
+def test_ds_buffer_holds_the_kept_pairs_only(F):
+    """The exchange buffer of a masked call is as large as the mask leaves it: 32 KB per query head and kept pair
+    of 128 x 128 tiles (a causal window of 300 over 4096 tokens keeps 122 of 1024 pairs)."""
+    from flex_attention_tpu_amd import masks
+    S, W = 4096, 300
+    sc = 1 / math.sqrt(128)
+    g = torch.Generator().manual_seed(3)
+    q, k, v, do = (torch.randn(1, 2, S, 128, generator=g).to(torch.bfloat16).to(DEV) for _ in range(4))
+    mf, bf = masks.make_causal_sliding_window_mask_fns(128, 128, W)
+    o, l, m = _fwd(F, q, k, v, sc, mf, bf, None)
+    d = F.compute_delta(o, do)
+    dk, dv, ds = _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, None, return_ds=True)
+    kept = sum(1 for qb in range(32) for kb in range(32) if kb <= qb and 128 * qb - (128 * kb + 127) < W)
+    assert ds is not None and ds.buf.numel() == 2 * kept * 128 * 128 * 2 and kept == 122
+    # a device without room for the buffer: the pass declines the exchange, the dq pass then recomputes
+    from flex_attention_tpu_amd import flex_attention_dq_bwd as dqmod
+    share, dqmod.DS_FREE_MEMORY_SHARE = dqmod.DS_FREE_MEMORY_SHARE, 0.0
+    try:
+        dk2, dv2, ds2 = _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, None, return_ds=True)
+    finally:
+        dqmod.DS_FREE_MEMORY_SHARE = share
+    assert ds2 is None and torch.equal(dk2, dk) and torch.equal(dv2, dv)
+
+
 # ------------------------------------------------------------------------------------------------
 # small-shape parity matrix (oracle runs whole tensors in float64)
 # ------------------------------------------------------------------------------------------------
@@ -504,6 +548,93 @@ def test_document_masks_longest_first_schedule(F):
     ref = all_passes(q.float(), k.float(), v.float(), do.float())
     for name, a, b in zip(("o", "lse", "dq", "dk", "dv"), got, ref):
         assert O.rel_l2(a.float().cpu(), b.cpu()) <= 1e-2, name
+
+
+def _sampled_oracle_check(F, q, k, v, do, sc, mf, bf, sfn, okw, n_rows, heads, dtype=torch.bfloat16, tag="", **call_kw):
+    """All passes of one call on the GPU against the oracle on `n_rows` sampled q rows of the (batch, q head)
+    pairs `heads` (whole kv groups): o, lse and dq on those rows; dk, dv with dO zeroed outside the sampled rows
+    (the gradients are linear in dO, so every kv position is exercised at full length).  The backward against the
+    oracle's backward from the kernels' own residuals.  `call_kw` goes to the three entry points (compiled_loop)."""
+    B, Hq, Sq, _ = q.shape
+    Hkv = k.shape[1]
+    g = torch.Generator().manual_seed(7)
+    rows = torch.sort(torch.randperm(Sq, generator=g)[:n_rows]).values
+    rows[0], rows[-1] = 0, Sq - 1
+    ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, q_rows=rows, heads=heads,
+                                 compute_dtype=torch.float32, **okw)
+    do_s = torch.zeros_like(do)
+    do_s[:, :, rows] = do[:, :, rows]
+    qg, kg, vg, dog = [x.to(DEV) for x in (q, k, v, do_s)]
+    o, l, m = F._flex_attention_impl(qg, kg, vg, None, None, True, False, sc, 1, 128, 128, 128, False, bf, mf, sfn, **call_kw)
+    d = F.compute_delta(o, dog)
+    dq = F.flex_attention_bwd_dq(qg, kg, vg, None, None, l, m, o, dog, d, block_b=1, block_q=128, block_k_major=128,
+                                 block_k=128, sm_scale=sc, debug=False, score_fn=sfn, mask_fn=mf, block_mask_fn=bf, **call_kw)
+    dk, dv = F.flash_attention_bwd_dkv(kg, vg, qg, None, None, l, m, d, dog, block_b=1, block_q=128, block_q_major=128,
+                                       block_k_major=128, block_k=128, sm_scale=sc, causal=False, debug=False,
+                                       score_fn=sfn, mask_fn=mf, block_mask_fn=bf, **call_kw)
+    torch.cuda.synchronize()
+    sdq, sdk, sdv = same_residual_grads(q, k, v, do_s, o, l, m, sm_scale=sc, q_rows=rows, heads=heads,
+                                        compute_dtype=torch.float32, **okw)
+    dr = rows.to(DEV)
+    group = Hq // Hkv
+    for (b, h) in heads:
+        assert_close(f"{tag}o[{b},{h}]", o[b, h, dr], ro[b, h], dtype)
+        assert_close(f"{tag}lse[{b},{h}]", (m + l.log())[b, h, dr], (rm + rl.log())[b, h], dtype)
+        assert_close(f"{tag}dq[{b},{h}]", dq[b, h, dr], sdq[b, h], dtype)
+    for (b, hk) in sorted({(b, h // group) for (b, h) in heads}):
+        assert all((b, hk * group + gq) in heads for gq in range(group)), "sample whole KV groups"
+        assert_close(f"{tag}dk[{b},{hk}]", dk[b, hk], sdk[b, hk], dtype)
+        assert_close(f"{tag}dv[{b},{hk}]", dv[b, hk], sdv[b, hk], dtype)
+
+
+@pytest.mark.parametrize("compiled_loop", [False, True], ids=["default", "compiled_loop"])
+def test_long_tile_lists_s131072(F, compiled_loop):
+    """One head of 131072 tokens under the causal mask (the reference's own sweep goes to 262144,
+    roofline_data_flex.csv:10): 2048 kv tiles of 64 rows in a row's list, 1024 q tiles of 128 rows in a column's,
+    i.e. lists beyond what the generated-stream forward caches (it hands over to the kernel with a compiled
+    loop) and at the limit of the backward streams; and the same with every pass on its compiled-loop kernel.
+    Sampled rows against the oracle."""
+    from flex_attention_tpu_amd import masks
+    S = 131072
+    sc = 1 / math.sqrt(128)
+    q, k, v, do = O.make_inputs(1, 1, 1, S, S, 128, dtype=torch.bfloat16, seed=131)
+    mf, bf = masks.make_causal_mask_fns(128, 128)
+    _sampled_oracle_check(F, q, k, v, do, sc, mf, bf, None, dict(causal=True), 192, [(0, 0)], compiled_loop=compiled_loop)
+
+
+@pytest.mark.parametrize("case", ["persistent_mha_b8_h32_s1024", "gqa_4to1_s2048", "documents_longest_first",
+                                  "alibi_b8_h32_s1024", "softcap_gqa_s2048"])
+def test_schedule_edges_against_the_oracle(F, case):
+    """Shapes at the edges of the work schedules (the persistent grid of one work-group per CU with several heads
+    per work-group, grouped kv heads at 2048 tokens, the longest-first schedule that document masks get with
+    eight items per work-group) and the position-bias and softcap streams on such grids: sampled rows of a few
+    heads of the full launch against the oracle."""
+    from flex_attention_tpu_amd import masks, scores
+    sc = 1 / math.sqrt(128)
+    mf, bf, sfn = None, None, None
+    if case == "persistent_mha_b8_h32_s1024":
+        B, Hq, Hkv, S, heads = 8, 32, 32, 1024, [(0, 0), (5, 17), (7, 31)]
+        (mf, bf), okw = masks.make_causal_mask_fns(128, 128), dict(causal=True)
+    elif case == "gqa_4to1_s2048":
+        B, Hq, Hkv, S, heads = 3, 16, 4, 2048, [(0, 0), (0, 1), (0, 2), (0, 3), (2, 12), (2, 13), (2, 14), (2, 15)]
+        (mf, bf), okw = masks.make_causal_sliding_window_mask_fns(128, 128, 300), dict(causal=True, window_size=300)
+    elif case == "documents_longest_first":
+        B, Hq, Hkv, S, heads = 16, 32, 32, 1024, [(0, 0), (9, 30), (15, 31)]
+        lens = [100, 412, 212, 300]
+        (mf, bf), okw = masks.make_jagged_mask_fns(128, 128, lens), dict(causal=True, segment_ids=O.doc_ids_from_lengths(lens))
+    elif case == "alibi_b8_h32_s1024":
+        B, Hq, Hkv, S, heads = 8, 32, 32, 1024, [(0, 0), (3, 8), (7, 31)]
+        (mf, bf), sfn = masks.make_causal_mask_fns(128, 128), scores.make_alibi_global_score_fn(32)
+        okw = dict(causal=True, score_mod=O.score_mod_alibi_global(O.alibi_slopes(32)))
+    else:
+        B, Hq, Hkv, S, heads = 1, 16, 4, 2048, [(0, 4), (0, 5), (0, 6), (0, 7)]
+        lens = [700, 900, 448]
+        (mf, bf), sfn = masks.make_jagged_mask_fns(128, 128, lens), scores.make_softcap_score_fn(2.0)
+        okw = dict(causal=True, segment_ids=O.doc_ids_from_lengths(lens), score_mod=O.score_mod_softcap(2.0))
+    q, k, v, do = O.make_inputs(B, Hq, Hkv, S, S, 128, dtype=torch.bfloat16, seed=137)
+    if case == "softcap_gqa_s2048":
+        q = (q.float() * 3).to(torch.bfloat16)   # (scores of several caps: the tanh saturates)
+    _sampled_oracle_check(F, q, k, v, do, sc, mf, bf, sfn, okw, 160, heads)
 
 
 def test_integration_doc_binding_runs_verbatim(F):
