@@ -131,6 +131,7 @@ class BwdParamsC(C.Structure):
         ("ds", C.c_void_p),
         ("ds_bytes", C.c_int64),
         ("ds_index", DsIndexC),
+        ("dab", C.c_void_p),
     ]
 
 

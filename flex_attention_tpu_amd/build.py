@@ -62,21 +62,37 @@ def _compile(src: str, force: bool, build_dir: str = BUILD_DIR, extra_flags=()) 
     return obj
 
 
-def build_library(force: bool = True, jobs: int = 8, out_path: str = LIB_PATH, build_dir: str = BUILD_DIR,
-                  extra_flags=()) -> str:
-    """Compiles every HIP source for gfx950 and links libflexattn.so next to the package (or, with
-    `out_path` / `build_dir` / `extra_flags`, a functor library of compiler.py against its generated header)."""
-    os.makedirs(build_dir, exist_ok=True)
+def generate_streams(out_dir: str = CSRC) -> None:
+    """Runs the stream generators; each writes its include file into `out_dir` (written under a temporary name
+    and moved into place, so that a compiler running in another process never reads half a file)."""
     for gen, out in GENERATED:
-        r = subprocess.run([sys.executable, os.path.join(CSRC, gen), os.path.join(CSRC, out)], capture_output=True, text=True)
+        final = os.path.join(out_dir, out)
+        tmp = f"{final}.{os.getpid()}.tmp"
+        r = subprocess.run([sys.executable, os.path.join(CSRC, gen), tmp], capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"{gen} failed:\n{r.stdout}\n{r.stderr}")
+        os.replace(tmp, final)
+
+
+def build_library(force: bool = True, jobs: int = 8, out_path: str = LIB_PATH, build_dir: str = BUILD_DIR,
+                  extra_flags=(), include_dir: str = CSRC) -> str:
+    """Compiles every HIP source for gfx950 and links libflexattn.so next to the package (or, with
+    `out_path` / `build_dir` / `extra_flags`, a functor library of compiler.py against its generated header).
+    `include_dir`: where the generated streams go (a functor library writes its copy into its own build
+    directory and nothing into the package; the compiler takes the package's copy, the same text, where one
+    lies next to the sources, and this one otherwise).  The library is linked under a temporary name
+    and moved into place: a process that finds the file finds a complete one."""
+    os.makedirs(build_dir, exist_ok=True)
+    generate_streams(include_dir)
+    inc = (f"-I{include_dir}",) if include_dir != CSRC else ()
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(lambda s: _compile(s, force, build_dir, tuple(extra_flags)), SOURCES))
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out_path]
+        objs = list(ex.map(lambda s: _compile(s, force, build_dir, inc + tuple(extra_flags)), SOURCES))
+    tmp = f"{out_path}.{os.getpid()}.tmp"
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
+    os.replace(tmp, out_path)
     return out_path
 
 

@@ -773,18 +773,31 @@ def library_path(score: Optional[CustomCode], mask: Optional[CustomCode]) -> str
 def build_functor_library(score: Optional[CustomCode], mask: Optional[CustomCode], force: bool = False) -> str:
     """Compiles (hipcc, gfx950) the library of a functor pair unless it is cached; returns its path."""
     from . import build as B
+    import fcntl
     path = library_path(score, mask)
     if os.path.exists(path) and not force:
         return path
     d = os.path.dirname(path)
     os.makedirs(d, exist_ok=True)
-    header = os.path.join(d, "custom_functor.hpp")
-    with open(header, "w") as f:
-        f.write(header_text(score, mask))
-    flags = [f'-DFLEXATTN_CUSTOM_HEADER="{header}"']
-    if score is not None:
-        flags.append("-DFLEXATTN_CUSTOM_ONLY")   # a custom score runs the compiled-loop kernels: skip the generated streams
-    B.build_library(force=True, out_path=path, build_dir=os.path.join(d, "obj"), extra_flags=flags)
+    # one builder per functor pair at a time (processes that compile the same closures at once: ranks of a job,
+    # test workers); everything is written inside the pair's own directory, the library under a temporary name
+    with open(os.path.join(d, ".lock"), "w") as lock:
+        fcntl.flock(lock, fcntl.LOCK_EX)
+        try:
+            if os.path.exists(path) and not force:   # (another process built it while this one waited)
+                return path
+            header = os.path.join(d, "custom_functor.hpp")
+            tmp = f"{header}.{os.getpid()}.tmp"
+            with open(tmp, "w") as f:
+                f.write(header_text(score, mask))
+            os.replace(tmp, header)
+            flags = [f'-DFLEXATTN_CUSTOM_HEADER="{header}"']
+            if score is not None:
+                flags.append("-DFLEXATTN_CUSTOM_ONLY")   # a custom score runs the compiled-loop kernels: skip the generated streams
+            obj = os.path.join(d, "obj")
+            B.build_library(force=True, out_path=path, build_dir=obj, extra_flags=flags, include_dir=obj)
+        finally:
+            fcntl.flock(lock, fcntl.LOCK_UN)
     return path
 
 

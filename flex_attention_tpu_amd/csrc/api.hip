@@ -216,6 +216,11 @@ static int to_bwd_args(const flexattn_bwd_params* p, int pass, BwdArgs* a) {
   if ((rc = check_score(p->score)) != FLEXATTN_OK) return rc;
   if ((rc = check_mask(p->mask)) != FLEXATTN_OK) return rc;
   if ((rc = check_bias(p->ab, p->B, p->Hq, p->Sq, p->Sk)) != FLEXATTN_OK) return rc;
+  if (p->dab != nullptr) {
+    if (pass != FLEXATTN_PASS_DQ) return set_error(FLEXATTN_EINVAL, "dab is an output of flexattn_bwd_dq");
+    if (p->ds != nullptr) return set_error(FLEXATTN_EINVAL, "dab and ds exclude each other (the dq pass from dS recomputes nothing)");
+  }
+  a->dab = p->dab;
   a->ds = p->ds;
   a->ds_col = p->ds_index.col;
   a->ds_rank = p->ds_index.rank;
@@ -393,7 +398,10 @@ int flexattn_bwd_dq(const flexattn_bwd_params* p, void* stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (p->ds != nullptr)  // (checked: bf16 and a plain or softcap score; the softcap streams leave 4 out of dS)
     return bwd_dq_from_ds(a, (p->score.kind == FLEXATTN_SCORE_SOFTCAP ? 4.f : 1.f) * p->sm_scale, s);
-  if (p->dtype == FLEXATTN_BF16) return bwd_dq_bf16_d128(a, s);
+  if (p->dtype == FLEXATTN_BF16) {
+    if (a.dab != nullptr) a.flags |= FLEXATTN_FLAG_COMPILED_LOOP;  // (the generated streams store no bias gradient)
+    return bwd_dq_bf16_d128(a, s);
+  }
   return (a.flags & FLEXATTN_FLAG_COMPILED_LOOP) ? bwd_dq_f32(a, p->D, s) : bwd_dq_f32_mfma(a, p->D, s);
 }
 

@@ -216,7 +216,9 @@ __global__ __launch_bounds__(256) void bwd_dq_f32_kernel(BwdArgs a) {
         if (!keep_elem(a.mask, q_idx, j, doc_i, doc_j)) x = kNegInf;
       }
       const float p = exp2f(x - lse2);
-      const float ds = (x == kNegInf) ? 0.f : p * (dp - dl) * sm.dfactor(tv, s, q_idx, j);
+      const float gl = (x == kNegInf) ? 0.f : p * (dp - dl);   // gradient with respect to the logit (the bias's share)
+      if (a.dab != nullptr && sub == 0) a.dab[row * (size_t)a.Sk + j] = gl;
+      const float ds = (x == kNegInf) ? 0.f : gl * sm.dfactor(tv, s, q_idx, j);
       axpy_slice<NV>(acc, ds, sK + jj * D, sub);
     }
   }

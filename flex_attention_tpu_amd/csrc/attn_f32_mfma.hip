@@ -260,7 +260,9 @@ __global__ __launch_bounds__(256) void bwd_dq_f32_mfma_kernel(BwdArgs a) {
           if (!keep_elem(a.mask, q_idx, j, doc_i, doc_j)) x = kNegInf;
         }
         const float pe = exp2f(x - lse2);
-        ds[i] = (x == kNegInf) ? 0.f : pe * (dp[i] - dl) * sm.dfactor(tv, s[i], q_idx, j);
+        const float gl = (x == kNegInf) ? 0.f : pe * (dp[i] - dl);   // gradient with respect to the logit (the bias's share)
+        if (a.dab != nullptr) a.dab[row * (size_t)a.Sk + j] = gl;
+        ds[i] = (x == kNegInf) ? 0.f : gl * sm.dfactor(tv, s[i], q_idx, j);
       }
       accumulate_rows<D>(acc, Kg + (size_t)j0 * D, ds, l32, half);
     }

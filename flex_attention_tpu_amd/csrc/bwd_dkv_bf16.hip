@@ -375,7 +375,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   const bool sorted = DOCS && gridDim.x != (unsigned)n_wg;
   int* sItems = reinterpret_cast<int*>(sPart + MAX_LIST) + 4 * 128;
   if (DOCS && sorted)
-    sorted_items([&](int t) { return a.map.cnt[t]; }, nKb, n_wg / nKb, (int)blockIdx.x, n_items, tid,
+    sorted_items([&](int t) { return a.map.cnt[t]; }, nKb, n_wg / nKb, 1, (int)blockIdx.x, n_items, tid,
                  reinterpret_cast<int*>(smem_raw), sItems);
   auto geometry = [&](int item) {
     Geometry g;

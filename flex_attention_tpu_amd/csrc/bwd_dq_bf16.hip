@@ -111,6 +111,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
   const uint8_t* tile_state = a.map.state + (size_t)qb * nK;
   int doc_i = 0;
   if (a.mask.flags & FLEXATTN_MASK_DOC) doc_i = a.mask.doc_q[q_idx];
+  float* dab_row = a.dab != nullptr ? a.dab + row * (size_t)a.Sk : nullptr;  // this lane's row of the bias gradient
 
   f32x16 dq_acc[4];
 #pragma unroll
@@ -213,15 +214,23 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
             dj[0] = d4[0]; dj[1] = d4[1]; dj[2] = d4[2]; dj[3] = d4[3];
           }
           float dsv[4];
+          f32x4 gb;   // the gradient with respect to the logits themselves: what an additive bias receives
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
             const int e = 4 * g + u;
             const float tv = sm.to_log2(s_acc[e], q_idx, j0 + u);
             const float pe = fast_exp2(tv + sm.bias2(q_idx, j0 + u) - lse2);
-            float gd = pe * (dp_acc[e] - delta) * sm.dfactor(tv, s_acc[e], q_idx, j0 + u);
-            if (MASKED) gd = keep_elem(a.mask, q_idx, j0 + u, doc_i, dj[u]) ? gd : 0.f;
+            float gl = pe * (dp_acc[e] - delta);
+            float gd = gl * sm.dfactor(tv, s_acc[e], q_idx, j0 + u);
+            if (MASKED) {   // (selected, not multiplied: a score function may return anything at a dropped element)
+              const bool keep = keep_elem(a.mask, q_idx, j0 + u, doc_i, dj[u]);
+              gl = keep ? gl : 0.f;
+              gd = keep ? gd : 0.f;
+            }
+            gb[u] = gl;
             dsv[u] = gd;
           }
+          if (dab_row != nullptr) *reinterpret_cast<f32x4*>(dab_row + j0) = gb;
           const bf16x2 d01 = pack_bf16(dsv[0], dsv[1]), d23 = pack_bf16(dsv[2], dsv[3]);
           const int o = 4 * (g & 1);
           ds[g >> 1][o] = d01[0]; ds[g >> 1][o + 1] = d01[1]; ds[g >> 1][o + 2] = d23[0]; ds[g >> 1][o + 3] = d23[1];
@@ -337,7 +346,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   const bool sorted = DOCS && gridDim.x != (unsigned)n_wg;
   int* sItems = reinterpret_cast<int*>(sSt + MAX_LIST) + 4 * 128;
   if (DOCS && sorted)
-    sorted_items([&](int t) { return a.map.cnt[t]; }, nQ, n_wg / nQ, (int)blockIdx.x, n_items, tid,
+    sorted_items([&](int t) { return a.map.cnt[t]; }, nQ, n_wg / nQ, group, (int)blockIdx.x, n_items, tid,
                  reinterpret_cast<int*>(smem_raw), sItems);
   auto geometry = [&](int item, int& bh, int& qb) {
     if (DOCS && sorted) {

@@ -434,7 +434,7 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
   int* sItems = reinterpret_cast<int*>(sStB + MAX_LIST) + 4 * 128;
   if (DOCS && sorted)
     sorted_items([&](int t) { return a.map.cnt[2 * t] + (2 * t + 1 < nQ ? a.map.cnt[2 * t + 1] : 0); }, nQ2, n_wg / nQ2,
-                 (int)blockIdx.x, n_items, tid, reinterpret_cast<int*>(smem_raw), sItems);
+                 group, (int)blockIdx.x, n_items, tid, reinterpret_cast<int*>(smem_raw), sItems);
   auto geometry = [&](int item, int& bh, int& qb2) {
     if (DOCS && sorted) {
       const int v = sItems[item];

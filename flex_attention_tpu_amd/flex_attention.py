@@ -30,22 +30,24 @@ class _FlexAttention(torch.autograd.Function):
     """o = softmax(mask(score_mod(sm_scale q k^T))) v with the saved statistics (l, m) for the backward."""
 
     @staticmethod
-    def forward(ctx, q, k, v, opts):
-        score_fn, mask_fn, block_mask_fn, segment_ids, causal, sm_scale, block_q, block_k, ab = opts
+    def forward(ctx, q, k, v, ab, opts):
+        score_fn, mask_fn, block_mask_fn, segment_ids, causal, sm_scale, block_q, block_k = opts
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         o, l, m = _flex_attention_impl(q, k, v, ab, segment_ids, True, causal, sm_scale, 1, block_q, block_k, block_k,
                                        False, block_mask_fn, mask_fn, score_fn)
-        ctx.save_for_backward(q, k, v, o, l, m)
+        ctx.save_for_backward(q, k, v, o, l, m, *([ab] if ab is not None else []))
         ctx.opts = opts
         return o
 
     @staticmethod
     def backward(ctx, do):
-        q, k, v, o, l, m = ctx.saved_tensors
-        score_fn, mask_fn, block_mask_fn, segment_ids, causal, sm_scale, block_q, block_k, ab = ctx.opts
+        q, k, v, o, l, m, *rest = ctx.saved_tensors
+        ab = rest[0] if rest else None
+        score_fn, mask_fn, block_mask_fn, segment_ids, causal, sm_scale, block_q, block_k = ctx.opts
+        want_dab = ab is not None and ctx.needs_input_grad[3]
         do = do.contiguous()
         di = compute_delta(o, do)  # float32 [B, H, Sq]  (jax_exp.py:276-278)
-        dq = dk = dv = ds = None
+        dq = dk = dv = ds = dab = None
         if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
             exchange = ctx.needs_input_grad[0] and ds_exchange_pays(score_fn, mask_fn, segment_ids)
             dk, dv, ds = flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, block_b=1, block_q=block_q,
@@ -56,12 +58,14 @@ class _FlexAttention(torch.autograd.Function):
                     k, v, q, ab, segment_ids, l, m, di, do, block_b=1, block_q=block_q, block_q_major=block_q,
                     block_k_major=block_k, block_k=block_k, sm_scale=sm_scale, causal=causal, debug=False,
                     score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn), None)
-        if ctx.needs_input_grad[0]:
+        if ctx.needs_input_grad[0] or want_dab:   # (the bias gradient is an output of the dq pass)
             dq = flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, di, block_b=1, block_q=block_q,
                                        block_k_major=block_k, block_k=block_k, sm_scale=sm_scale, debug=False,
                                        score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn, causal=causal,
-                                       ds=ds)
-        return dq, dk, dv, None
+                                       ds=ds, return_dab=want_dab)
+            if want_dab:
+                dq, dab = dq
+        return dq if ctx.needs_input_grad[0] else None, dk, dv, dab, None
 
 
 def flex_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, score_fn: Optional[Callable] = None,
@@ -74,14 +78,14 @@ def flex_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, score_fn: 
     ``mask_fns``   ``(mask_fn, block_mask_fn)`` pair from ``masks``, or None
     ``segment_ids`` / ``causal``   as in the three entry points (ANDed with ``mask_fns``)
     ``sm_scale``   default 1 / sqrt(D)
-    ``ab``         additive bias on the logits, [B or 1, H or 1, Sq, Sk]; it receives no gradient (the reference's
-                   flex backward kernels produce none: flex_attention_dq_bwd.py:109-110 keeps `dab = ds` commented out)
-    Gradients flow to q, k and v (``torch.autograd.grad`` / ``.backward()``); higher-order
+    ``ab``         additive bias on the logits, [B or 1, H or 1, Sq, Sk]; a bias that requires grad receives
+                   dab = P (dP - delta), summed over the dimensions it broadcasts (the output the reference declares
+                   next to dk, dv, flash_attention_dkv_bwd.py:103-107,130-138)
+    Gradients flow to q, k, v and ab (``torch.autograd.grad`` / ``.backward()``); higher-order
     differentiation is not supported, as in the reference (jax_exp.py:243-244).
     """
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(q.shape[-1])
     mask_fn, block_mask_fn = mask_fns if mask_fns is not None else (None, None)
-    opts = (score_fn, mask_fn, block_mask_fn, segment_ids, bool(causal), float(sm_scale), int(block_q), int(block_k),
-            ab.detach() if ab is not None else None)
-    return _FlexAttention.apply(q, k, v, opts)
+    opts = (score_fn, mask_fn, block_mask_fn, segment_ids, bool(causal), float(sm_scale), int(block_q), int(block_k))
+    return _FlexAttention.apply(q, k, v, ab, opts)

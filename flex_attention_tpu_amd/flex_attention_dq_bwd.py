@@ -92,17 +92,23 @@ def bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, mod_q, mod_k,
 
 def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, block_q, block_k_major,
                           block_k, sm_scale, debug, score_fn=None, mask_fn=None, block_mask_fn=None,
-                          causal=False, compiled_loop=False, ds=None):
+                          causal=False, compiled_loop=False, ds=None, return_dab=False):
     """dq = sum_j dS_ij * d(score)/dq, with P_ij = exp(S_ij - m_i) / l_i recomputed from the saved
     statistics, dP = do v^T, dS = P (dP - d) (flex_attention_dq_bwd.py:340-378).  ``o`` is only
     shape-checked, as in the reference (:163); ``d`` is the caller's delta (see compute_delta).
     ``ds``: the DsBlocks of the dk/dv pass of the same arguments, if that pass returned one: dq is then
-    sm_scale dS K, nothing is recomputed."""
+    sm_scale dS K, nothing is recomputed.
+    ``return_dab=True`` (needs ``ab``; excludes ``ds``) returns (dq, dab): the gradient of the additive bias in
+    ab's shape and dtype, dab = P (dP - d) summed over the dimensions ``ab`` broadcasts -- the output the
+    reference declares next to dk, dv (flash_attention_dkv_bwd.py:103-107,130-138) and its upstream dq kernel
+    writes (jax_exp.py:1252-1255; there multiplied by sm_scale)."""
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v, do)
     rows = per_batch_segments(segment_ids, B)
     if rows is not None:  # ids differ between batch entries: one launch per entry
         if ds is not None and (ds.entries is None or len(ds.entries) != B):
             raise ValueError("ds does not come from a dk/dv pass of these arguments")
+        if return_dab:
+            raise NotImplementedError("return_dab with segment ids that differ between batch entries")
         return torch.cat([flex_attention_bwd_dq(
             q[b:b + 1], k[b:b + 1], v[b:b + 1], batch_entry(ab, b), rows[b], l[b:b + 1], m[b:b + 1], batch_entry(o, b),
             do[b:b + 1], d[b:b + 1], block_b=block_b, block_q=block_q, block_k_major=block_k_major, block_k=block_k,
@@ -128,6 +134,13 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     ab_c, ab_keep = bias_c(ab, B, Hq, Sq, Sk, Sq_p, Sk_p, q.device)
     p = bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dq=dq,
                    compiled_loop=compiled_loop, ab_c=ab_c)
+    dab_full = None
+    if return_dab:
+        if ab is None or ds is not None:
+            raise ValueError("return_dab needs the additive bias `ab` and excludes `ds`")
+        # (only the tiles the block map visits are written: masked-out pairs have no gradient)
+        dab_full = torch.zeros(B, Hq, Sq_p, Sk_p, dtype=torch.float32, device=q.device)
+        p.dab = dab_full.data_ptr()
     if ds is not None:
         p.ds, p.ds_bytes = ds.buf.data_ptr(), ds.buf.numel()
         col, rank, pairs = ds.index   # (the index the dk/dv pass wrote the blocks by)
@@ -137,4 +150,11 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
         _lib.check(lib.flexattn_bwd_dq(C.byref(p), stream_of(q)), lib)
     if Sq_p != Sq or D != D_user:
         dq = dq[:, :, :Sq, :D_user].contiguous()
-    return dq
+    if not return_dab:
+        return dq
+    dab = dab_full[:, :, :Sq, :Sk]
+    if ab.shape[0] == 1 and B > 1:
+        dab = dab.sum(0, keepdim=True)
+    if ab.shape[1] == 1 and Hq > 1:
+        dab = dab.sum(1, keepdim=True)
+    return dq, dab.to(ab.dtype).contiguous()

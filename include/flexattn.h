@@ -93,7 +93,7 @@ typedef struct flexattn_block_map {
  * flash_attention_dkv_bwd.py:261-263, mha_reference.py:50-51): logits = score_mod(sm_scale <q, k>) + ab,
  * then the mask.  Element (b, h, i, j) lies at ptr + b stride_b + h stride_h + i Sk + j (in elements;
  * a stride of 0 broadcasts over that dimension; strides must be multiples of Sk).  ptr NULL = no bias.  Calls with a bias run the kernels
- * with a compiled main loop.  No gradient of the bias is produced (the reference computes none either). */
+ * with a compiled main loop.  flexattn_bwd_dq can return the gradient of the bias (flexattn_bwd_params.dab). */
 typedef struct flexattn_bias {
   const void* ptr;
   int64_t stride_b, stride_h;
@@ -151,6 +151,12 @@ typedef struct flexattn_bwd_params {
   void* ds;
   int64_t ds_bytes;
   flexattn_ds_index ds_index; /* needed with ds; for the map at the granularity of FLEXATTN_PASS_DKV */
+  /* Gradient of the additive bias, or NULL: out of flexattn_bwd_dq, float32 [B, Hq, Sq, Sk] (full shape: the caller
+   * sums over the dimensions its bias broadcasts).  dab = P (dP - delta), the gradient with respect to the logits
+   * (the reference declares this output next to dk, dv, flash_attention_dkv_bwd.py:103-107,130-138, and its upstream
+   * dq kernel writes it, jax_exp.py:1252-1255, there multiplied by sm_scale).  Only the tiles the block map visits
+   * are written: clear the buffer first.  A call with dab runs the dq kernel with a compiled main loop; it excludes ds. */
+  float* dab;
 } flexattn_bwd_params;
 
 #define FLEXATTN_PASS_FWD 0

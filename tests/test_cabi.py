@@ -38,7 +38,7 @@ def test_struct_sizes_follow_c_layout():
     assert C.sizeof(_lib.BiasC) == 32
     assert C.sizeof(_lib.FwdParamsC) == 6 * 8 + 10 * 4 + 32 + 32 + 56 + 32
     assert C.sizeof(_lib.DsIndexC) == 24
-    assert C.sizeof(_lib.BwdParamsC) == 10 * 8 + 10 * 4 + 32 + 32 + 56 + 32 + 16 + 24
+    assert C.sizeof(_lib.BwdParamsC) == 10 * 8 + 10 * 4 + 32 + 32 + 56 + 32 + 16 + 24 + 8
 
 
 def test_tile_shapes(lib):

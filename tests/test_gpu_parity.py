@@ -292,10 +292,37 @@ def test_additive_bias(F, case, dtype):
     assert_close("o", o, ro, dtype)
     assert_close("lse", m + l.log(), rm + rl.log(), dtype)
     tol = dict(sm_scale=sc, **okw)
-    ma = O.mha_bwd_reference(q, k, v, o.float().cpu(), do, l.cpu(), m.cpu(), ab_full, **tol)
+    ma = O.mha_bwd_reference(q, k, v, o.float().cpu(), do, l.cpu(), m.cpu(), ab_full, return_dab=True, **tol)
     for name, t, r, chain in (("dq", dq, ma[0], rdq), ("dk", dk, ma[1], rdk), ("dv", dv, ma[2], rdv)):
         assert_close(name, t, r, dtype)
         assert_close(name + " chain", t, chain, dtype, chain=True)
+    # the gradient of the bias (an output of the dq pass), in the bias's own shape and dtype: summed over the
+    # dimensions it broadcasts
+    mf_, bf_ = mask_pair if mask_pair else (None, None)
+    d = F.compute_delta(o, dog)
+    dq2, dab = F.flex_attention_bwd_dq(qg, kg, vg, ab.to(DEV), None, l, m, o, dog, d, block_b=1, block_q=128,
+                                       block_k_major=128, block_k=128, sm_scale=sc, debug=False, score_fn=score_fn,
+                                       mask_fn=mf_, block_mask_fn=bf_, causal=causal, return_dab=True)
+    rdab = ma[3]
+    for dim in (0, 1):
+        if ab.shape[dim] == 1:
+            rdab = rdab.sum(dim, keepdim=True)
+    assert dab.shape == ab.shape and dab.dtype == ab.dtype
+    assert_close("dq with dab", dq2, ma[0], dtype)
+    if dtype == torch.bfloat16 or ab.dtype == torch.bfloat16:
+        assert_close("dab", dab, rdab, torch.bfloat16)
+    else:
+        # float32: 1e-5 relative to the value where that exceeds 1 (dab is P (dP - delta), not normalised like the
+        # other gradients: entries reach 8 here, where float32 round-off alone is 1e-6 per operation)
+        err = (dab.cpu().double() - rdab).abs()
+        assert O.rel_l2(dab, rdab) <= 1e-5 and bool((err <= 1e-5 * rdab.abs().clamp(min=1.0)).all()), float(err.max())
+    assert float(rdab.abs().max()) > 1e-3
+    # ... and through the differentiable op
+    abg = ab.to(DEV).requires_grad_(True)
+    qa = qg.clone().requires_grad_(True)
+    og = F.flex_attention(qa, kg, vg, score_fn, mask_pair, causal=causal, sm_scale=sc, ab=abg)
+    gq, gab = torch.autograd.grad(og, (qa, abg), dog)
+    assert torch.equal(gab, dab) and gq.shape == q.shape
     # without the bias the result differs (the argument is not ignored)
     o0 = F._flex_attention_impl(qg, kg, vg, None, None, False, causal, sc, 1, 128, 128, 128, False,
                                 mask_pair[1] if mask_pair else None, mask_pair[0] if mask_pair else None, score_fn)

@@ -292,3 +292,30 @@ def test_legacy_alibi_slope_branch_matches_sdpa_float_mask():
     gq, gk, gv = torch.autograd.grad(r, (qd, kd, vd), do)
     for a, b in ((dq, gq), (dk, gk), (dv, gv)):
         assert (a - b).abs().max() < 1e-11
+
+
+def test_bias_gradient_matches_autograd_of_sdpa():
+    """`return_dab`: the gradient of the additive bias is ds = p (dp - delta), neither scaled by sm_scale nor by
+    the score function's derivative -- against autograd through SDPA with a float ``attn_mask`` that requires
+    grad (causal folded into the mask as -inf, whose entries receive no gradient), and with a softcap score
+    through an independently written softmax."""
+    B, H, Sq, Sk = 2, 2, 24, 40
+    q, k, v, do = O.make_inputs(B, H, H, Sq, Sk, 8, dtype=torch.float64, seed=21)
+    ab = torch.randn(B, H, Sq, Sk, generator=torch.Generator().manual_seed(22), dtype=torch.float64)
+    kw = dict(sm_scale=0.37, causal=True)
+    o, l, m = O.mha_reference(q, k, v, ab, save_residuals=True, **kw)
+    dq, dk, dv, dab = O.mha_bwd_reference(q, k, v, o, do, l, m, ab, return_dab=True, **kw)
+    above = torch.arange(Sk)[None, :] > torch.arange(Sq)[:, None]
+    abd = ab.clone().requires_grad_()
+    r = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=abd.masked_fill(above, float("-inf")), scale=0.37)
+    (g,) = torch.autograd.grad(r, abd, do)
+    assert (dab - g).abs().max() < 1e-12 and float(g.abs().max()) > 1e-3
+    assert float(dab[..., above].abs().max()) == 0.0
+    # softcap in front of the bias: d logits / d ab is still 1
+    kw = dict(sm_scale=0.5, score_mod=O.score_mod_softcap(1.5))
+    o, l, m = O.mha_reference(q, k, v, ab, save_residuals=True, **kw)
+    dab = O.mha_bwd_reference(q, k, v, o, do, l, m, ab, return_dab=True, **kw)[3]
+    abd = ab.clone().requires_grad_()
+    s = 1.5 * torch.tanh(torch.einsum("bhqc,bhkc->bhqk", q, k) * 0.5 / 1.5) + abd
+    (g,) = torch.autograd.grad(torch.softmax(s, -1) @ v, abd, do)
+    assert (dab - g).abs().max() < 1e-12
