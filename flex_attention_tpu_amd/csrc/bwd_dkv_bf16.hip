@@ -49,7 +49,8 @@ constexpr int BNK = 128;  // kv rows per work-group
 constexpr int BQ = 128;   // q rows per step (two 64-row LDS tiles)
 constexpr size_t kDsBlockBytes = (size_t)BQ * BNK * 2;  // one exported dS block
 constexpr int D = 128;
-constexpr int MAX_LIST = 1024;  // longest q tile list the plain-score kernel caches in LDS
+constexpr int MAX_LIST = 2048;       // longest q tile list the plain-score kernel caches in LDS (262144 tokens)
+constexpr int PREFETCH_LIST = 1024;  // of which an item's prefetch carries this many in registers; the rest is read when the item starts
 // (Q, dO) x 2 buffers x 2 tiles, lse x2, delta x2, run-loop tables, cached q tile list and its partial flags
 constexpr int LDS_BYTES = 8 * kTileElems * 2 + 4 * BQ * 4 + 4 * 32 * 4 + MAX_LIST * 5 + kDocStageBytes + kMaxSortedItems * 4;
 }  // namespace dkv_cfg
@@ -404,7 +405,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   // Everything an item needs from global memory before its first step is fetched while the previous
   // item runs: plain loads whose values are not touched until that item's last step is done.  (They
   // live in v[192:255] and the low registers, which the run loop leaves alone.)
-  constexpr int kListRegs = MAX_LIST / 256;
+  constexpr int kListRegs = PREFETCH_LIST / 256;
   struct ItemRegs {
     RowBlock k, v;                 // the wave's 32 K / V rows (full-row layout, see rows_load)
     int doc, n_tiles, qb0;         // list length and its first entry
@@ -529,6 +530,14 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     if (t < nQ) {
       sIdx[t] = cur.idx[j];
       sPart[t] = cur.part[j] == 1 ? 1 : 0;
+    }
+  }
+  if (nQ > PREFETCH_LIST) {
+    // columns longer than the prefetched part (more than 131072 tokens): the rest straight from global memory
+    // (an item is then thousands of steps long: the wait does not show)
+    for (int t = PREFETCH_LIST + tid_p; t < nQ; t += 256) {
+      sIdx[t] = tile_idx[t];
+      sPart[t] = a.map.state[(size_t)t * a.map.nk + kb] == 1 ? 1 : 0;
     }
   }
   if (n_iter > 0 && !resident) {

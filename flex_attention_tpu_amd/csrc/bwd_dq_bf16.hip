@@ -41,7 +41,8 @@ constexpr int BN = 64;
 constexpr int D = 128;
 constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2
 // plain-score kernel: steps of two kv tiles, (K, K, V, V) x 2 buffers, per-wave tables, cached kv list + states
-constexpr int MAX_LIST = 2048;
+constexpr int MAX_LIST = 4096;       // kv tiles of a row whose list and states the kernel caches in LDS (262144 tokens)
+constexpr int PREFETCH_LIST = 2048;  // of which an item's prefetch carries this many in registers; the rest is read when the item starts
 constexpr int PLAIN_LDS_BYTES = 8 * kTileElems * 2 + 4 * 16 * 4 + MAX_LIST * 5 + kDocStageBytes + kMaxSortedItems * 4;
 }  // namespace dq_cfg
 
@@ -330,7 +331,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   // Everything an item needs from global memory before its first step.  It is fetched while the
   // previous item runs (plain loads whose values are not touched until then), so that an item
   // starts after one memory round trip (its first kv tiles) instead of a chain of dependent ones.
-  constexpr int kListRegs = MAX_LIST / 256;
+  constexpr int kListRegs = PREFETCH_LIST / 256;
   struct ItemRegs {
     RowBlock q, d;       // the wave's 32 Q / dO rows (full-row layout, see rows_load)
     float l, m, delta;
@@ -468,6 +469,15 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
       if (t < nK) {
         sIdx[t] = cur.idx[j];
         sSt[t] = cur.st[j];
+      }
+    }
+    if (nK > PREFETCH_LIST) {
+      // rows longer than the prefetched part (more than 131072 tokens): the rest straight from global memory
+      // (an item is then thousands of steps long: the wait does not show)
+      const uint8_t* state_row = a.map.state + (size_t)qb * nK;
+      for (int t = PREFETCH_LIST + tid_p; t < nK; t += 256) {
+        sIdx[t] = tile_idx[t];
+        sSt[t] = state_row[t];
       }
     }
 

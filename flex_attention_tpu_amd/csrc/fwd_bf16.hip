@@ -43,7 +43,8 @@ constexpr int D = 128;
 constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2
 // plain-score kernel: 256 q rows per work item, steps of two kv tiles: (K, K, V, V) x 2 buffers, per-wave
 // tables, wave counters, merged kv list, the two state rows
-constexpr int MAX_LIST = 1024;
+constexpr int MAX_LIST = 4096;       // kv tiles of a row that the merged list and the state rows in LDS hold (262144 tokens)
+constexpr int PREFETCH_LIST = 1024;  // of which an item's prefetch carries this many in registers; the rest is read when the item starts
 constexpr int PLAIN_LDS_BYTES = 8 * kTileElems * 2 + 4 * 16 * 4 + 16 + MAX_LIST * 4 + 2 * MAX_LIST + kDocStageBytes + kMaxSortedItems * 4;
 }  // namespace fwd_cfg
 
@@ -417,7 +418,7 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
   };
   // Everything an item needs from global memory before its first step, fetched while the previous
   // item runs (plain loads whose values are not touched until that item's last run).
-  constexpr int kListRegs = MAX_LIST / 256;
+  constexpr int kListRegs = PREFETCH_LIST / 256;
   static_assert(kListRegs <= 4, "the packed state words hold four tiles per lane");
   struct ItemRegs {
     RowBlock q[2];      // the wave's 32 Q rows of each q tile (full-row layout, see rows_load)
@@ -532,22 +533,43 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
       }
     }
     int n_list = 0;
+    auto append = [&](bool present, int t) {   // tiles t of all 256 threads, in thread order, behind the list so far
+      const unsigned long long mask = __ballot(present);
+      if (lane == 0) sCnt[w] = __builtin_popcountll(mask);
+      __syncthreads();
+      int off = n_list;
+      for (int ww = 0; ww < 4; ++ww) {
+        const int cw = sCnt[ww];
+        if (ww < w) off += cw;
+        n_list += cw;
+      }
+      if (present) sList[off + __builtin_popcountll(mask & ((1ull << lane) - 1ull))] = t;
+      __syncthreads();
+    };
 #pragma unroll
     for (int j = 0; j < kListRegs; ++j) {
       if (256 * j < nK) {
         const int t = tid_p + 256 * j;
-        const bool present = t < nK && (((cur.sa | cur.sb) >> (8 * j)) & 0xffu) != 0u;
-        const unsigned long long mask = __ballot(present);
-        if (lane == 0) sCnt[w] = __builtin_popcountll(mask);
-        __syncthreads();
-        int off = n_list;
-        for (int ww = 0; ww < 4; ++ww) {
-          const int cw = sCnt[ww];
-          if (ww < w) off += cw;
-          n_list += cw;
+        append(t < nK && (((cur.sa | cur.sb) >> (8 * j)) & 0xffu) != 0u, t);
+      }
+    }
+    if (nK > PREFETCH_LIST) {
+      // rows longer than the prefetched part (more than 65536 tokens): the rest of the two state rows straight
+      // from global memory (an item is then thousands of steps long: the wait does not show)
+      const int qa = min(2 * qb2, nQ - 1), qb_ = min(2 * qb2 + 1, nQ - 1);
+      const bool valid_b = 2 * qb2 + 1 < nQ;
+      const uint8_t* row_a = a.map.state + (size_t)qa * nK;
+      const uint8_t* row_b = a.map.state + (size_t)qb_ * nK;
+      for (int base = PREFETCH_LIST; base < nK; base += 256) {
+        const int t = base + tid_p;
+        unsigned sa = 0u, sb = 0u;
+        if (t < nK) {
+          sa = row_a[t];
+          sb = valid_b ? row_b[t] : 0u;
+          sStA[t] = (unsigned char)sa;
+          sStB[t] = (unsigned char)sb;
         }
-        if (present) sList[off + __builtin_popcountll(mask & ((1ull << lane) - 1ull))] = t;
-        __syncthreads();
+        append((sa | sb) != 0u, t);
       }
     }
     n_list = __builtin_amdgcn_readfirstlane(n_list);
@@ -680,14 +702,18 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
         if constexpr (ALIBI) {
           // the next item's list is walked from its end: its last two tiles, from the packed state words
           // (lane tid of the work-group holds tiles tid + 256 j), wave maxima exchanged through LDS
+          // (rows longer than the prefetched part: the end of the list is not among the fetched states; the next
+          // item then loads its first step itself)
           int top1 = -1, top2 = -1;
+          if (nK <= PREFETCH_LIST) {
 #pragma unroll
-          for (int j = 0; j < kListRegs; ++j) {
-            unsigned long long m = __ballot((((pre.sa | pre.sb) >> (8 * j)) & 0xffu) != 0u && tid + 256 * j < nK);
-            while (m != 0ull && top2 < w * 64 + 256 * j) {  // (tiles of a later j are larger: they replace both)
-              const int t = w * 64 + 256 * j + 63 - __builtin_clzll(m);
-              m &= ~(1ull << (63 - __builtin_clzll(m)));
-              if (t > top1) { top2 = top1; top1 = t; } else if (t > top2) { top2 = t; }
+            for (int j = 0; j < kListRegs; ++j) {
+              unsigned long long m = __ballot((((pre.sa | pre.sb) >> (8 * j)) & 0xffu) != 0u && tid + 256 * j < nK);
+              while (m != 0ull && top2 < w * 64 + 256 * j) {  // (tiles of a later j are larger: they replace both)
+                const int t = w * 64 + 256 * j + 63 - __builtin_clzll(m);
+                m &= ~(1ull << (63 - __builtin_clzll(m)));
+                if (t > top1) { top2 = top1; top1 = t; } else if (t > top2) { top2 = t; }
+              }
             }
           }
           if (lane == 0) sCnt[w] = (top1 & 0xffff) | (top2 << 16);

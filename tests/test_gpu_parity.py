@@ -614,19 +614,33 @@ def _sampled_oracle_check(F, q, k, v, do, sc, mf, bf, sfn, okw, n_rows, heads, d
         assert_close(f"{tag}dv[{b},{hk}]", dv[b, hk], sdv[b, hk], dtype)
 
 
-@pytest.mark.parametrize("compiled_loop", [False, True], ids=["default", "compiled_loop"])
-def test_long_tile_lists_s131072(F, compiled_loop):
-    """One head of 131072 tokens under the causal mask (the reference's own sweep goes to 262144,
-    roofline_data_flex.csv:10): 2048 kv tiles of 64 rows in a row's list, 1024 q tiles of 128 rows in a column's,
-    i.e. lists beyond what the generated-stream forward caches (it hands over to the kernel with a compiled
-    loop) and at the limit of the backward streams; and the same with every pass on its compiled-loop kernel.
-    Sampled rows against the oracle."""
+@pytest.mark.parametrize("S,compiled_loop", [(131072, False), (131072, True), (262144, False)],
+                         ids=["131072-default", "131072-compiled_loop", "262144-default"])
+def test_long_tile_lists(F, S, compiled_loop):
+    """One head of 131072 and of 262144 tokens under the causal mask (the reference's own sweep goes to 262144,
+    roofline_data_flex.csv:10): up to 4096 kv tiles of 64 rows in a row's list and 2048 q tiles of 128 rows in a
+    column's.  The generated-stream kernels prefetch the first 1024 (dq: 2048) list entries of an item in
+    registers and read the rest of a longer list when the item starts; and the same with every pass on its
+    compiled-loop kernel.  Sampled rows against the oracle."""
     from flex_attention_tpu_amd import masks
-    S = 131072
     sc = 1 / math.sqrt(128)
     q, k, v, do = O.make_inputs(1, 1, 1, S, S, 128, dtype=torch.bfloat16, seed=131)
     mf, bf = masks.make_causal_mask_fns(128, 128)
-    _sampled_oracle_check(F, q, k, v, do, sc, mf, bf, None, dict(causal=True), 192, [(0, 0)], compiled_loop=compiled_loop)
+    _sampled_oracle_check(F, q, k, v, do, sc, mf, bf, None, dict(causal=True), 160, [(0, 0)], compiled_loop=compiled_loop)
+
+
+def test_long_tile_lists_position_bias_and_window(F):
+    """Lists beyond the prefetched part under the other stream variants: the position bias (whose forward walks
+    the list from its end) with a causal window at 131072 tokens (rows of 2048 kv tiles, of which a window of 5000
+    tokens keeps about 80), two heads."""
+    from flex_attention_tpu_amd import masks, scores
+    S = 131072
+    sc = 1 / math.sqrt(128)
+    q, k, v, do = O.make_inputs(1, 2, 2, S, S, 128, dtype=torch.bfloat16, seed=133)
+    mf, bf = masks.make_causal_sliding_window_mask_fns(128, 128, 5000)
+    sfn = scores.make_alibi_global_score_fn(2)
+    okw = dict(causal=True, window_size=5000, score_mod=O.score_mod_alibi_global(O.alibi_slopes(2)))
+    _sampled_oracle_check(F, q, k, v, do, sc, mf, bf, sfn, okw, 128, [(0, 0), (0, 1)])
 
 
 @pytest.mark.parametrize("case", ["persistent_mha_b8_h32_s1024", "gqa_4to1_s2048", "documents_longest_first",
