@@ -59,6 +59,8 @@ class MaskSpecC(C.Structure):
         ("reserved", C.c_int32),
         ("doc_q", C.c_void_p),
         ("doc_k", C.c_void_p),
+        ("doc_q_range", C.c_void_p),
+        ("doc_k_range", C.c_void_p),
     ]
 
 

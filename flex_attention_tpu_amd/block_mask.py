@@ -131,9 +131,23 @@ def doc_ids_on(doc: Optional[DocIds], device) -> Optional[torch.Tensor]:
     return t
 
 
+_range_cache = LRU(DOC_CACHE_SIZE)  # (DocIds, DocIds of the other side, device) -> int32 [n, 2] device array or False
+
+
+def doc_ranges_on(doc: DocIds, other: DocIds, device) -> Optional[torch.Tensor]:
+    """Device copy of ``doc.ranges_in(other)`` (cached per device), or None when ``other`` is not sorted."""
+    key = (doc, other, str(device))
+    t = _range_cache.get(key)
+    if t is None:
+        r = doc.ranges_in(other)
+        t = torch.from_numpy(r).to(device) if r is not None else False
+        _range_cache.put(key, t)
+    return t if t is not False else None
+
+
 def mask_spec_c(spec: MaskSpec, Sq: int, Sk: int, device) -> _lib.MaskSpecC:
     """C view of a MaskSpec; validates the document array lengths."""
-    doc_q = doc_k = None
+    doc_q = doc_k = range_q = range_k = None
     if spec.flags & _lib.MASK_DOC:
         if spec.doc_ids is None:
             raise ValueError("document mask without document ids")
@@ -145,7 +159,17 @@ def mask_spec_c(spec: MaskSpec, Sq: int, Sk: int, device) -> _lib.MaskSpecC:
         tq.record_stream(cur)   # (cached arrays may be evicted while a kernel on this stream still reads them)
         tk.record_stream(cur)
         doc_q, doc_k = tq.data_ptr(), tk.data_ptr()
-    return _lib.MaskSpecC(spec.flags, spec.window, spec.stride, 0, doc_q, doc_k)
+        # sorted ids (the usual case: documents packed one after the other): the interval of the other side's
+        # positions with a position's id, from which the kernels mask partial tiles without comparing ids
+        if len(spec.doc_ids) == Sq and len(ids_k) == Sk:
+            rq, rk = doc_ranges_on(spec.doc_ids, ids_k, device), doc_ranges_on(ids_k, spec.doc_ids, device)
+            if rq is not None:
+                rq.record_stream(cur)
+                range_q = rq.data_ptr()
+            if rk is not None:
+                rk.record_stream(cur)
+                range_k = rk.data_ptr()
+    return _lib.MaskSpecC(spec.flags, spec.window, spec.stride, 0, doc_q, doc_k, range_q, range_k)
 
 
 def build_block_map(spec: MaskSpec, Sq: int, Sk: int, block_q: int, block_k: int, device,

@@ -59,6 +59,8 @@ static MaskArgs to_args(const flexattn_mask_spec& m) {
   r.stride = m.stride;
   r.doc_q = m.doc_q;
   r.doc_k = m.doc_k;
+  r.doc_q_range = m.doc_q_range;
+  r.doc_k_range = m.doc_k_range;
   return r;
 }
 

@@ -409,6 +409,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   struct ItemRegs {
     RowBlock k, v;                 // the wave's 32 K / V rows (full-row layout, see rows_load)
     int doc, n_tiles, qb0;         // list length and its first entry
+    int qlo, qhi;                  // (DOCS) first and last q position that carries the column's document id, where known
     float na2;                     // -slopes[head] log2(e) (ALIBI)
     int idx[kListRegs];            // q list entries tid + 256 j
     unsigned char part[kListRegs]; // state of q tile tid + 256 j against this kv tile
@@ -426,6 +427,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     rows_load(r.k, Kg + (size_t)(tid_here >> 6) * 32 * D, tid_here & 63);
     rows_load(r.v, Vg + (size_t)(tid_here >> 6) * 32 * D, tid_here & 63);
     r.doc = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_k[g.kb * BNK + kv_local] : 0;
+    if constexpr (DOCS) {
+      const bool have = a.mask.doc_k_range != nullptr;
+      r.qlo = have ? a.mask.doc_k_range[2 * (g.kb * BNK + kv_local)] : 0;
+      r.qhi = have ? a.mask.doc_k_range[2 * (g.kb * BNK + kv_local) + 1] : 0;
+    }
     const int* tile_idx = a.map.idx + (size_t)g.kb * nQ;
     r.n_tiles = a.map.cnt[g.kb];
     r.qb0 = tile_idx[0];  // (nQ >= 1: always readable; used only if the list is not empty)
@@ -439,7 +445,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   };
   // What is left of an item's fetched values once its K / V fragments sit in their registers.
   struct ItemHead {
-    int doc, n_tiles, qb0;
+    int doc, n_tiles, qb0, qlo, qhi;
     float na2;
     int idx[kListRegs];
     unsigned char part[kListRegs];
@@ -466,6 +472,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     FA_PUT(6, "a[152:155]", "a[184:187]") FA_PUT(7, "a[156:159]", "a[188:191]")
 #undef FA_PUT
     c.doc = r.doc;
+    if constexpr (DOCS) { c.qlo = r.qlo; c.qhi = r.qhi; }
     c.n_tiles = __builtin_amdgcn_readfirstlane(r.n_tiles);
     c.qb0 = __builtin_amdgcn_readfirstlane(r.qb0);
     c.na2 = ALIBI ? __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, r.na2))) : 0.f;
@@ -510,6 +517,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
   const float* rowa = (lse_wave ? a.l : a.delta) + rows0;
   const float* rowb = (lse_wave ? a.m : a.delta) + rows0;
   const int doc_j = cur.doc;
+  // (DOCS) with sorted q ids the queries of the column's document are one interval: the keep bits of a partial tile
+  // then have a closed form (keep_bits32_range) and no ids are read
+  const bool ranged = DOCS && a.mask.doc_k_range != nullptr && keep_bits_have_range(a.mask);
   const int* tile_idx = a.map.idx + (size_t)kb * nQ;
   const int n_tiles = cur.n_tiles;
   const int n_iter = n_tiles * group;
@@ -625,10 +635,16 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
       const int q0 = qb * BQ;
       if constexpr (DOCS) {
         int* sDoc = reinterpret_cast<int*>(sPart + MAX_LIST) + w * 128;  // the wave's stage for document ids
-        stage_doc_ids(a.mask.doc_q, q0, q0 + 64, lane, sDoc);
+        if (ranged) {
 #pragma unroll
-        for (int half = 0; half < 2; ++half)
-          km[half] = keep_bits32_staged<false>(a.mask, k_idx, q0 + 64 * half + 4 * hh, doc_j, sDoc + 64 * half + 4 * hh);
+          for (int half = 0; half < 2; ++half)
+            km[half] = keep_bits32_range<false>(a.mask, k_idx, q0 + 64 * half + 4 * hh, cur.qlo, cur.qhi);
+        } else {
+          stage_doc_ids(a.mask.doc_q, q0, q0 + 64, lane, sDoc);
+#pragma unroll
+          for (int half = 0; half < 2; ++half)
+            km[half] = keep_bits32_staged<false>(a.mask, k_idx, q0 + 64 * half + 4 * hh, doc_j, sDoc + 64 * half + 4 * hh);
+        }
       } else {
 #pragma unroll
         for (int half = 0; half < 2; ++half)

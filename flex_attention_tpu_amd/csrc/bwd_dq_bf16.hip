@@ -336,6 +336,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
     RowBlock q, d;       // the wave's 32 Q / dO rows (full-row layout, see rows_load)
     float l, m, delta;
     int doc;
+    int klo, khi;                  // (DOCS) first and last kv position that carries the row's document id, where known
     int n_tiles, kb0, kb1;         // list length and its first two entries
     int idx[kListRegs];            // kv list entries tid + 256 j
     unsigned char st[kListRegs];   // state of kv tile tid + 256 j in the q tile's state row
@@ -372,6 +373,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
     r.m = a.m[row];
     r.delta = a.delta[row];
     r.doc = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[qb * BM + q_local] : 0;
+    if constexpr (DOCS) {
+      const bool have = a.mask.doc_q_range != nullptr;
+      r.klo = have ? a.mask.doc_q_range[2 * (qb * BM + q_local)] : 0;
+      r.khi = have ? a.mask.doc_q_range[2 * (qb * BM + q_local) + 1] : 0;
+    }
     r.n_tiles = a.map.cnt[qb];
     const int* tile_idx = a.map.idx + (size_t)qb * nK;
     r.kb0 = tile_idx[0];                // (nK >= 1: always readable; meaningful only if the list is not empty)
@@ -399,7 +405,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   // What is left of an item's fetched values once its Q^T / dO^T fragments sit in their registers.
   struct ItemHead {
     float l, m, delta;
-    int doc, n_tiles, kb0, kb1;
+    int doc, klo, khi, n_tiles, kb0, kb1;
     int idx[kListRegs];
     unsigned char st[kListRegs];
   };
@@ -428,6 +434,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
     FA_PUT(6, "a[88:91]", "a[120:123]") FA_PUT(7, "a[92:95]", "a[124:127]")
 #undef FA_PUT
     c.l = r.l; c.m = r.m; c.delta = r.delta; c.doc = r.doc;
+    if constexpr (DOCS) { c.klo = r.klo; c.khi = r.khi; }
     c.n_tiles = __builtin_amdgcn_readfirstlane(r.n_tiles);
     c.kb0 = __builtin_amdgcn_readfirstlane(r.kb0);
     c.kb1 = __builtin_amdgcn_readfirstlane(r.kb1);
@@ -491,6 +498,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
     const float mulv = hh ? 0.f : a2;
     const float addv = hh ? a2 : -lse2;
     const int doc_i = cur.doc;
+    // (DOCS) with sorted kv ids the keys of the row's document are one interval: the keep bits of a partial tile
+    // then have a closed form (keep_bits32_range) and no ids are read
+    const bool ranged = DOCS && a.mask.doc_q_range != nullptr && keep_bits_have_range(a.mask);
     const int kb_first = cur.kb0;
     const int kb_second = (n_tiles > 1) ? cur.kb1 : kb_first;
     if (n_tiles > 0 && !resident) {
@@ -556,7 +566,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
       if (it_part < n_steps) {
         // the lane's keep bits: element e of kv block c sits at bit 16 (c & 1) + e of km[c >> 1]
         int* sDoc = reinterpret_cast<int*>(sSt + MAX_LIST) + w * 128;  // the wave's stage for document ids
-        if (a.mask.flags & FLEXATTN_MASK_DOC) {
+        if ((a.mask.flags & FLEXATTN_MASK_DOC) && !ranged) {
           const int e1 = 2 * it_part + 1 < n_tiles ? 2 * it_part + 1 : 2 * it_part;
           stage_doc_ids(a.mask.doc_k, __builtin_amdgcn_readfirstlane(sIdx[2 * it_part]) * BN,
                         __builtin_amdgcn_readfirstlane(sIdx[e1]) * BN, lane, sDoc);
@@ -569,6 +579,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
           const int state = __builtin_amdgcn_readfirstlane((int)sSt[kt]);
           if (state == 2) {
             km[hx] = 0xffffffffu;
+          } else if (DOCS && ranged) {
+            km[hx] = keep_bits32_range<true>(a.mask, q_idx, kt * BN + 4 * hh, cur.klo, cur.khi);
           } else if (a.mask.flags & FLEXATTN_MASK_DOC) {
             km[hx] = keep_bits32_staged<true>(a.mask, q_idx, kt * BN + 4 * hh, doc_i, sDoc + 64 * hx + 4 * hh);
           } else {

@@ -58,6 +58,10 @@ struct MaskArgs {
   int stride;
   const int* doc_q;
   const int* doc_k;
+  // For masks whose document ids are sorted on the other side, the positions of the other side that carry a
+  // position's id form one interval: (first, last) per position, first > last if there is none; null = unknown.
+  const int* doc_q_range;  // [Sq, 2]: kv positions with the id of q position i
+  const int* doc_k_range;  // [Sk, 2]: q positions with the id of kv position j
 };
 // One direction of the block map: for "major" block r, idx[r*n_minor + t], t < cnt[r], are the
 // minor blocks to visit; state is always indexed [q block][kv block].
@@ -274,6 +278,38 @@ __host__ __device__ __forceinline__ unsigned keep_bits32(const MaskArgs& mk, int
     }
   }
   return bits;
+}
+
+// keep_bits32 for causal / window / document masks when the positions of the varying side that carry the fixed
+// index's document id are known to form the interval [rlo, rhi] (MaskArgs::doc_q_range / doc_k_range; empty:
+// rlo > rhi): together with the causal and window bounds the kept offsets are still one interval, so a partial
+// tile of a document mask costs a dozen integer operations instead of 32 id compares behind a load.
+__host__ __device__ __forceinline__ bool keep_bits_have_range(const MaskArgs& mk) {
+  return (mk.flags & FLEXATTN_MASK_DOC) != 0 &&
+         (mk.flags & ~(FLEXATTN_MASK_CAUSAL | FLEXATTN_MASK_WINDOW | FLEXATTN_MASK_DOC)) == 0;
+}
+template <bool KEYS>
+__host__ __device__ __forceinline__ unsigned keep_bits32_range(const MaskArgs& mk, int fixed, int base, int rlo, int rhi) {
+  const int d = fixed - base;
+  const bool causal = (mk.flags & FLEXATTN_MASK_CAUSAL) != 0;
+  const bool window = (mk.flags & FLEXATTN_MASK_WINDOW) != 0;
+  const int width = mk.window < (1 << 28) ? mk.window : (1 << 28);
+  int lo, hi;
+  if (KEYS) {
+    lo = window ? d - width + 1 : 0;
+    hi = causal ? d : 63;
+  } else {
+    lo = causal ? d : 0;
+    hi = window ? width + d - 1 : 63;
+  }
+  const int a = rlo - base, b = rhi - base;
+  if (lo < a) lo = a;
+  if (hi > b) hi = b;
+  if (lo < 0) lo = 0;
+  if (hi > 63) hi = 63;
+  if (lo > hi) return 0u;
+  const unsigned long long upto = hi == 63 ? ~0ull : ((2ull << hi) - 1ull);
+  return compress_even_nibbles(upto & ~((1ull << lo) - 1ull));
 }
 
 // keep_bits32 for masks with document ids, the strip's ids staged in LDS (stage_doc_ids): `ids` points at

@@ -423,6 +423,7 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
   struct ItemRegs {
     RowBlock q[2];      // the wave's 32 Q rows of each q tile (full-row layout, see rows_load)
     int doc[2];
+    int klo[2], khi[2]; // (DOCS) first and last kv position that carries the row's document id, where known
     unsigned sa, sb;    // byte j: state of kv tile tid + 256 j in the state row of q tile 0 / 1
     unsigned head;      // states of kv tile `lane` in both rows: where the merged list starts
   };
@@ -461,6 +462,11 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
       const int qb = min(2 * qb2 + x, nQ - 1);  // (a missing second tile repeats the first; nothing of it is stored)
       rows_load(r.q[x], static_cast<const bf16_t*>(a.q) + ((size_t)bh * a.Sq + (size_t)qb * BM + w_here * 32) * D, lane_here);
       r.doc[x] = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[qb * BM + row_here] : 0;
+      if constexpr (DOCS) {
+        const bool ranged = a.mask.doc_q_range != nullptr;
+        r.klo[x] = ranged ? a.mask.doc_q_range[2 * (qb * BM + row_here)] : 0;
+        r.khi[x] = ranged ? a.mask.doc_q_range[2 * (qb * BM + row_here) + 1] : 0;
+      }
       const uint8_t* row = a.map.state + (size_t)qb * nK;
       const bool valid = 2 * qb2 + x < nQ;
       unsigned packed = 0u;
@@ -478,6 +484,7 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
   // What is left of an item's fetched values once its Q^T fragments sit in their registers.
   struct ItemHead {
     int doc[2];
+    int klo[2], khi[2];
     unsigned sa, sb;
   };
   FwdPinned st;
@@ -506,6 +513,10 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
 #undef FA_PUT
     c.doc[0] = r.doc[0];
     c.doc[1] = r.doc[1];
+    if constexpr (DOCS) {
+      c.klo[0] = r.klo[0]; c.klo[1] = r.klo[1];
+      c.khi[0] = r.khi[0]; c.khi[1] = r.khi[1];
+    }
     c.sa = r.sa;
     c.sb = r.sb;
   };
@@ -579,6 +590,9 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
                  : "={a[0:15]}"(st.o[0]), "={a[16:31]}"(st.o[1]), "={a[32:47]}"(st.o[2]), "={a[48:63]}"(st.o[3]),
                    "={a[64:79]}"(st.o[4]), "={a[80:95]}"(st.o[5]), "={a[96:111]}"(st.o[6]), "={a[112:127]}"(st.o[7]));
     const int doc_i[2] = {cur.doc[0], cur.doc[1]};
+    // (DOCS) with sorted kv ids the keys of a row's document are one interval: the keep bits of a partial tile
+    // then have a closed form (keep_bits32_range) and no ids are read
+    const bool ranged = DOCS && a.mask.doc_q_range != nullptr && keep_bits_have_range(a.mask);
     const int q_idx[2] = {(2 * qb2) * BM + q_local, (2 * qb2 + 1) * BM + q_local};
     // softmax state of the lane's two q rows (log2 domain): reference maximum M, running maximum
     // relative to it, sum of 2^(score - M)
@@ -656,9 +670,11 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
       unsigned km[4] = {0u, 0u, 0u, 0u};  // keep bits of q block x, kv tile hx of the step: km[2 x + hx]
       if (partial) {
         int* sDoc = reinterpret_cast<int*>(sStB + MAX_LIST) + w * 128;  // the wave's stage for document ids
-        if constexpr (DOCS)
-          stage_doc_ids(a.mask.doc_k, __builtin_amdgcn_readfirstlane(entry(2 * it)) * BN,
-                        __builtin_amdgcn_readfirstlane(entry(2 * it + 1)) * BN, lane, sDoc);
+        if constexpr (DOCS) {
+          if (!ranged)
+            stage_doc_ids(a.mask.doc_k, __builtin_amdgcn_readfirstlane(entry(2 * it)) * BN,
+                          __builtin_amdgcn_readfirstlane(entry(2 * it + 1)) * BN, lane, sDoc);
+        }
 #pragma unroll
         for (int hx = 0; hx < 2; ++hx) {
           const int e = 2 * it + hx;
@@ -671,7 +687,8 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
               km[2 * x + hx] = 0xffffffffu;
             } else if (state == 1) {
               if constexpr (DOCS)
-                km[2 * x + hx] = keep_bits32_staged<true>(a.mask, q_idx[x], k * BN + 4 * hh, doc_i[x], sDoc + 64 * hx + 4 * hh);
+                km[2 * x + hx] = ranged ? keep_bits32_range<true>(a.mask, q_idx[x], k * BN + 4 * hh, cur.klo[x], cur.khi[x])
+                                        : keep_bits32_staged<true>(a.mask, q_idx[x], k * BN + 4 * hh, doc_i[x], sDoc + 64 * hx + 4 * hh);
               else
                 km[2 * x + hx] = keep_bits32<true>(a.mask, q_idx[x], k * BN + 4 * hh, doc_i[x], a.mask.doc_k);
             }

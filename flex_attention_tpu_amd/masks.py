@@ -40,6 +40,21 @@ class DocIds:
     def __len__(self):
         return self.array.shape[0]
 
+    def is_sorted(self) -> bool:
+        """Whether the ids are non-decreasing along the sequence (the reference's jagged mask: masks.py:88-103)."""
+        a = self.array
+        return bool(a.shape[0] < 2 or (a[1:] >= a[:-1]).all())
+
+    def ranges_in(self, other: "DocIds"):
+        """int32 [len(self), 2]: for every position of this array the first and last position of ``other`` that
+        carries the same id (first > last where there is none), or None when ``other`` is not sorted (the positions
+        then form no interval).  The kernels mask partial tiles of a document mask from these bounds."""
+        if not other.is_sorted():
+            return None
+        lo = np.searchsorted(other.array, self.array, side="left")
+        hi = np.searchsorted(other.array, self.array, side="right") - 1
+        return np.ascontiguousarray(np.stack([lo, hi], axis=1).astype(np.int32))
+
 
 @dataclass(frozen=True)
 class MaskSpec:

@@ -74,6 +74,14 @@ typedef struct flexattn_mask_spec {
   int32_t reserved;
   const int32_t* doc_q; /* DOC: device int32 [Sq]: any ids (they need not be sorted) */
   const int32_t* doc_k; /* DOC: device int32 [Sk] (may equal doc_q) */
+  /* DOC, optional (NULL = not known): where the ids of the OTHER side are non-decreasing, the positions there that
+   * carry a position's id form one interval, and the kernels then mask partial tiles from these bounds instead of
+   * comparing ids element by element (the reference's jagged mask has sorted ids: masks.py:88-110).
+   * doc_q_range: device int32 [Sq, 2], for q position i the first and last kv position j with doc_k[j] == doc_q[i]
+   * (first > last if there is none); needs doc_k non-decreasing.  doc_k_range: device int32 [Sk, 2], likewise the
+   * q positions with the id of kv position j; needs doc_q non-decreasing.  Wrong bounds give wrong results. */
+  const int32_t* doc_q_range;
+  const int32_t* doc_k_range;
 } flexattn_mask_spec;
 
 /* Block-sparsity map at (block_q x block_k) granularity, as produced by

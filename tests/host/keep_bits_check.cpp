@@ -1,6 +1,7 @@
 // Host-side check of the keep-bit closed forms in fa_common.hpp (compiled by tests/test_keep_bits.py with
 // `hipcc --cuda-host-only`, runs on the CPU): keep_bits32 against the element-wise predicate keep_elem
-// for every mask flag combination, on both sides (keys varying / queries varying).
+// for every mask flag combination, on both sides (keys varying / queries varying); and keep_bits32_range, the
+// interval form for document masks with sorted ids, likewise.
 #include <cstdio>
 #include <cstdlib>
 #include <vector>
@@ -63,6 +64,22 @@ int main() {
         return 1;
       }
       checked += 2;
+      if (keep_bits_have_range(mk)) {
+        // the interval form: positions that carry the fixed index's id (the ids are sorted: one run)
+        int rlo = fixed, rhi = fixed;
+        while (rlo > 0 && doc[rlo - 1] == doc[fixed]) --rlo;
+        while (rhi + 1 < S && doc[rhi + 1] == doc[fixed]) ++rhi;
+        const unsigned kr = keep_bits32_range<true>(mk, fixed, b, rlo, rhi);
+        const unsigned qr = keep_bits32_range<false>(mk, fixed, b, rlo, rhi);
+        if (kr != k1 || qr != q1) {
+          std::printf("MISMATCH (range) flags=%d window=%d fixed=%d base=%d keys %08x/%08x queries %08x/%08x\n", flags,
+                      mk.window, fixed, b, kr, k1, qr, q1);
+          return 1;
+        }
+        // an id that the other side does not carry at all: nothing is kept
+        if (keep_bits32_range<true>(mk, fixed, b, 5, 4) != 0u || keep_bits32_range<false>(mk, fixed, b, 5, 4) != 0u) return 1;
+        checked += 2;
+      }
     }
   }
   std::printf("ok %ld\n", checked);

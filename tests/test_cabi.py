@@ -33,12 +33,12 @@ def test_version_matches_header(lib):
 def test_struct_sizes_follow_c_layout():
     # pointers 8-byte aligned, no surprises in the ctypes mirrors
     assert C.sizeof(_lib.ScoreSpecC) == 32
-    assert C.sizeof(_lib.MaskSpecC) == 32
+    assert C.sizeof(_lib.MaskSpecC) == 48
     assert C.sizeof(_lib.BlockMapC) == 56
     assert C.sizeof(_lib.BiasC) == 32
-    assert C.sizeof(_lib.FwdParamsC) == 6 * 8 + 10 * 4 + 32 + 32 + 56 + 32
+    assert C.sizeof(_lib.FwdParamsC) == 6 * 8 + 10 * 4 + 32 + 48 + 56 + 32
     assert C.sizeof(_lib.DsIndexC) == 24
-    assert C.sizeof(_lib.BwdParamsC) == 10 * 8 + 10 * 4 + 32 + 32 + 56 + 32 + 16 + 24 + 8
+    assert C.sizeof(_lib.BwdParamsC) == 10 * 8 + 10 * 4 + 32 + 48 + 56 + 32 + 16 + 24 + 8
 
 
 def test_tile_shapes(lib):
