@@ -118,9 +118,10 @@ def measure(cfg, steps, warmup):
         return F._flex_attention_impl(q, k, v, None, None, True, False, sc, 1, blk, blk, blk, False, bf, mf, sfn)
 
     def dq_of(o, l, m, d, ds=None):
+        # d=None: the dq pass takes delta = sum(o * do) itself and returns it next to dq
         return F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=blk, block_k_major=blk,
                                        block_k=blk, sm_scale=sc, debug=False, score_fn=sfn, mask_fn=mf, block_mask_fn=bf,
-                                       ds=ds)
+                                       ds=ds, return_delta=d is None)
 
     def dkv_of(l, m, d, return_ds=False):
         return F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=blk, block_q_major=blk,
@@ -129,13 +130,14 @@ def measure(cfg, steps, warmup):
 
     # the step hands dS over where the package's own backward (flex_attention) would: ds_exchange_pays
     from flex_attention_tpu_amd.flex_attention_dq_bwd import ds_exchange_pays
-    exchange = ds_exchange_pays(sfn, mf)
+    exchange = ds_exchange_pays(sfn, mf) and q.dtype == torch.bfloat16
 
     def step():
         o, l, m = fwd()
+        if not exchange:   # delta, dq and dk/dv from one call (flexattn_bwd), as the package's own backward runs them
+            return (o,) + F.flex_attention_bwd(q, k, v, None, None, l, m, o, do, block_q=blk, block_k=blk, sm_scale=sc,
+                                               score_fn=sfn, mask_fn=mf, block_mask_fn=bf)
         d = F.compute_delta(o, do)
-        if not exchange:
-            return o, dq_of(o, l, m, d), dkv_of(l, m, d)
         dk, dv, ds = dkv_of(l, m, d, True)   # (ds is None where the configuration's kernels exchange nothing)
         return o, dq_of(o, l, m, d, ds), dk, dv
 
@@ -155,15 +157,20 @@ def measure(cfg, steps, warmup):
     d = F.compute_delta(o, do)
     ds = dkv_of(l, m, d, True)[2]   # (None where the configuration's kernels exchange nothing)
     used = exchange and ds is not None
+    fused = not exchange   # the dq call launches the delta kernel itself (d=None): the step makes no delta call
     launches = {"fwd": fwd, "delta": lambda: F.compute_delta(o, do),
-                "dq": (lambda: dq_of(o, l, m, d, ds)) if used else (lambda: dq_of(o, l, m, d)),
+                "dq": (lambda: dq_of(o, l, m, d, ds)) if used else (lambda: dq_of(o, l, m, None if fused else d)),
                 "dkv": (lambda: dkv_of(l, m, d, True)) if used else (lambda: dkv_of(l, m, d))}
+    if fused:
+        launches["dq_given_delta"] = lambda: dq_of(o, l, m, d)   # the dq pass alone, delta from its own launch
     if ds is not None:   # the other way of running the two passes, for comparison
-        launches.update(dq_other=(lambda: dq_of(o, l, m, d)) if used else (lambda: dq_of(o, l, m, d, ds)),
+        launches.update(dq_other=(lambda: dq_of(o, l, m, None)) if used else (lambda: dq_of(o, l, m, d, ds)),
                         dkv_other=(lambda: dkv_of(l, m, d)) if used else (lambda: dkv_of(l, m, d, True)))
     ms, quant = {}, {}
     for name, fn in launches.items():
-        fn()
+        for _ in range(3):   # (buffers a launch allocates for the first time are slow on first touch)
+            fn()
+        torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(steps):
@@ -181,7 +188,7 @@ def measure(cfg, steps, warmup):
         quant[name] = quantiles([ev[i].elapsed_time(ev[i + 1]) for i in range(steps)])
     return {"ms_step": wall * 1e3 / steps, "ms": ms, "quantiles_ms": quant, "elem_bytes": q.element_size(),
             "numel_q": q.numel(), "numel_k": k.numel(), "ds_bytes": ds.buf.numel() if ds is not None else 0,
-            "ds_used": used}
+            "ds_used": used, "delta_fused": fused}
 
 
 def tf(fl, t_ms):
@@ -194,7 +201,8 @@ def summary(cfg, r):
     from flex_attention_tpu_amd import configs
     ms = r["ms"]
     f_fwd = configs.flops_fwd(cfg)
-    ms_bwd = ms["delta"] + ms["dq"] + ms["dkv"]
+    fused = r["delta_fused"]   # ms["dq"] is then the dq call that launches the delta kernel and the dq kernel
+    ms_bwd = (0.0 if fused else ms["delta"]) + ms["dq"] + ms["dkv"]
     eb, nq, nk = r["elem_bytes"], r["numel_q"], r["numel_k"]
     rows = 4 * cfg.B * cfg.Hq * cfg.S
     bytes_delta = 2 * nq * eb + rows
@@ -206,10 +214,15 @@ def summary(cfg, r):
         "bwd": {"ms": ms_bwd, "tflops": tf(2.5 * f_fwd, ms_bwd), "delta_ms": ms["delta"], "dq_ms": ms["dq"],
                 "dkv_ms": ms["dkv"], "delta_gbs": bytes_delta / (ms["delta"] * 1e-3) / 1e9,
                 "dq_quantiles_ms": r["quantiles_ms"]["dq"], "dkv_quantiles_ms": r["quantiles_ms"]["dkv"],
-                "delta_quantiles_ms": r["quantiles_ms"]["delta"], "ds_exchange": r["ds_used"]},
+                "delta_quantiles_ms": r["quantiles_ms"]["delta"], "ds_exchange": r["ds_used"],
+                "delta_launched_by_dq_call": fused},
     }
+    if fused:   # (dq_ms covers the delta kernel and the dq kernel; delta_ms and the dq kernel alone beside it)
+        out["bwd"].update(dq_kernel_ms=ms["dq_given_delta"],
+                          ms_with_separate_delta_call=ms["delta"] + ms["dq_given_delta"] + ms["dkv"])
     if r["ds_bytes"] > 0:   # the backward run the other way (with the dS hand-over if the step runs without, and vice versa)
-        ms_other = ms["delta"] + ms["dq_other"] + ms["dkv_other"]
+        # (the hand-over needs delta before the dk/dv pass: its own launch; the recomputing way takes it in the dq pass)
+        ms_other = (0.0 if r["ds_used"] else ms["delta"]) + ms["dq_other"] + ms["dkv_other"]
         tag = "without_exchange" if r["ds_used"] else "with_exchange"
         out["bwd"].update({"ds_buffer_bytes": r["ds_bytes"], f"dq_ms_{tag}": ms["dq_other"], f"dkv_ms_{tag}": ms["dkv_other"],
                            f"ms_{tag}": ms_other, f"tflops_{tag}": tf(2.5 * f_fwd, ms_other)})
@@ -271,6 +284,9 @@ def main():
     # roofline of the dominant kernel; algorithmic FLOPs of one launch:
     #   fwd 2 matmuls = F_fwd, dk/dv 4 matmuls = 2 F_fwd, dq 3 matmuls = 1.5 F_fwd (1 matmul from exchanged dS)
     algo = {"fwd": f_fwd, "dq": (0.5 if r["ds_used"] else 1.5) * f_fwd, "dkv": 2.0 * f_fwd}
+    ms = dict(ms)
+    if r["delta_fused"]:
+        ms["dq"] = ms["dq_given_delta"]   # (the roofline object is about single kernels: the dq kernel without the delta kernel)
     dom = max(algo, key=lambda n: ms[n])
     traffic, stale = counter_traffic(dom) if name == "cfg2" else (None, None)
     roofline = {

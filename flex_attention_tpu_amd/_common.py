@@ -295,3 +295,22 @@ def library_for(score_fn, spec: MaskSpec):
 
 def stream_of(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_no_switch = _NoSwitch()
+
+
+def on_device(device):
+    """Context that makes `device` the current one for the launch; nothing to enter when it already is (the
+    usual case: switching costs the launch path several microseconds, which small problems are bound by)."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _no_switch
+    return torch.cuda.device(device)

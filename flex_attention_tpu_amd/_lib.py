@@ -134,6 +134,8 @@ class BwdParamsC(C.Structure):
         ("ds_bytes", C.c_int64),
         ("ds_index", DsIndexC),
         ("dab", C.c_void_p),
+        ("o", C.c_void_p),
+        ("delta_out", C.c_void_p),
     ]
 
 
@@ -149,6 +151,7 @@ EXPORTS = (
     "flexattn_bwd_ds_bytes",
     "flexattn_bwd_dq",
     "flexattn_bwd_dkv",
+    "flexattn_bwd",
     "flexattn_custom_tag",
 )
 
@@ -172,8 +175,9 @@ def _bind(lib: C.CDLL) -> C.CDLL:
     lib.flexattn_bwd_ds_bytes.argtypes = [C.POINTER(BwdParamsC)]
     lib.flexattn_bwd_ds_bytes.restype = C.c_int64
     lib.flexattn_bwd_dkv.argtypes = [C.POINTER(BwdParamsC), C.c_void_p]
+    lib.flexattn_bwd.argtypes = [C.POINTER(BwdParamsC), C.POINTER(BwdParamsC), C.c_void_p]
     for name in ("flexattn_tile_shape", "flexattn_build_block_mask", "flexattn_build_ds_index", "flexattn_fwd", "flexattn_fwd_noalloc", "flexattn_bwd_delta",
-                 "flexattn_bwd_dq", "flexattn_bwd_dkv"):
+                 "flexattn_bwd_dq", "flexattn_bwd_dkv", "flexattn_bwd"):
         getattr(lib, name).restype = C.c_int
     return lib
 

@@ -206,8 +206,14 @@ static int check_ds(const flexattn_bwd_params* p) {
 
 static int to_bwd_args(const flexattn_bwd_params* p, int pass, BwdArgs* a) {
   if (p == nullptr) return set_error(FLEXATTN_EINVAL, "params is NULL");
-  if (!p->q || !p->k || !p->v || !p->dout || !p->l || !p->m || !p->delta)
+  if (!p->q || !p->k || !p->v || !p->dout || !p->l || !p->m)
     return set_error(FLEXATTN_EINVAL, "a required input pointer is NULL");
+  if (p->o != nullptr) {
+    if (p->delta_out == nullptr) return set_error(FLEXATTN_EINVAL, "o given without delta_out");
+    if (p->ds != nullptr) return set_error(FLEXATTN_EINVAL, "o (delta computed by the call) and ds exclude each other");
+  } else if (!p->delta) {
+    return set_error(FLEXATTN_EINVAL, "delta is NULL (give delta, or o and delta_out)");
+  }
   if (pass == FLEXATTN_PASS_DQ && !p->dq) return set_error(FLEXATTN_EINVAL, "dq is NULL");
   if (pass == FLEXATTN_PASS_DKV && (!p->dk || !p->dv)) return set_error(FLEXATTN_EINVAL, "dk or dv is NULL");
   int rc = check_ds(p);
@@ -223,6 +229,8 @@ static int to_bwd_args(const flexattn_bwd_params* p, int pass, BwdArgs* a) {
     if (p->ds != nullptr) return set_error(FLEXATTN_EINVAL, "dab and ds exclude each other (the dq pass from dS recomputes nothing)");
   }
   a->dab = p->dab;
+  a->o = p->o;
+  a->delta_out = p->delta_out;
   a->ds = p->ds;
   a->ds_col = p->ds_index.col;
   a->ds_rank = p->ds_index.rank;
@@ -239,6 +247,18 @@ static int to_bwd_args(const flexattn_bwd_params* p, int pass, BwdArgs* a) {
   return FLEXATTN_OK;
 }
 
+
+// With `o` given the call computes delta itself: the delta kernel runs in front of the pass, on the same stream.
+// (Folding the sum into the dq stream kernel was measured and is not done: fetching an item's 32 rows of o along
+// with those of Q and dO an item ahead lengthened the dq launch by 0.067 ms on B=4, H=32, S=4096, where the delta
+// kernel takes 0.038 ms: the burst of row loads at an item's start is what the CU cannot keep in flight.)
+static int delta_first(BwdArgs* a, int D, int dtype, hipStream_t s) {
+  if (a->o == nullptr) return FLEXATTN_OK;
+  const int rc = bwd_delta(a->o, a->dout, a->delta_out, (int64_t)a->B * a->Hq * a->Sq, D, dtype, s);
+  a->delta = a->delta_out;
+  a->o = nullptr;
+  return rc;
+}
 
 static int fwd_with_map(const flexattn_fwd_params* p, const flexattn_block_map& map, hipStream_t s) {
   if (!p->q || !p->k || !p->v || !p->o) return set_error(FLEXATTN_EINVAL, "q, k, v or o is NULL");
@@ -391,15 +411,8 @@ int flexattn_bwd_delta(const void* o, const void* dout, float* delta, int64_t ro
   return bwd_delta(o, dout, delta, rows, D, dtype, static_cast<hipStream_t>(stream));
 }
 
-int64_t flexattn_bwd_ds_bytes(const flexattn_bwd_params* p) { return ds_exchange_ok(p) ? ds_bytes_of(p) : 0; }
-
-int flexattn_bwd_dq(const flexattn_bwd_params* p, void* stream) {
-  BwdArgs a;
-  int rc = to_bwd_args(p, FLEXATTN_PASS_DQ, &a);
-  if (rc != FLEXATTN_OK) return rc;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (p->ds != nullptr)  // (checked: bf16 and a plain or softcap score; the softcap streams leave 4 out of dS)
-    return bwd_dq_from_ds(a, (p->score.kind == FLEXATTN_SCORE_SOFTCAP ? 4.f : 1.f) * p->sm_scale, s);
+static int launch_dq(const flexattn_bwd_params* p, BwdArgs a, hipStream_t s) {
+  if (p->ds != nullptr) return bwd_dq_from_ds(a, (p->score.kind == FLEXATTN_SCORE_SOFTCAP ? 4.f : 1.f) * p->sm_scale, s);
   if (p->dtype == FLEXATTN_BF16) {
     if (a.dab != nullptr) a.flags |= FLEXATTN_FLAG_COMPILED_LOOP;  // (the generated streams store no bias gradient)
     return bwd_dq_bf16_d128(a, s);
@@ -407,13 +420,58 @@ int flexattn_bwd_dq(const flexattn_bwd_params* p, void* stream) {
   return (a.flags & FLEXATTN_FLAG_COMPILED_LOOP) ? bwd_dq_f32(a, p->D, s) : bwd_dq_f32_mfma(a, p->D, s);
 }
 
+static int launch_dkv(const flexattn_bwd_params* p, const BwdArgs& a, hipStream_t s) {
+  if (p->dtype == FLEXATTN_BF16) return bwd_dkv_bf16_d128(a, s);
+  return (a.flags & FLEXATTN_FLAG_COMPILED_LOOP) ? bwd_dkv_f32(a, p->D, s) : bwd_dkv_f32_mfma(a, p->D, s);
+}
+
+int flexattn_bwd(const flexattn_bwd_params* pq, const flexattn_bwd_params* pkv, void* stream) {
+  BwdArgs aq, akv;
+  int rc = to_bwd_args(pq, FLEXATTN_PASS_DQ, &aq);
+  if (rc != FLEXATTN_OK) return rc;
+  if ((rc = to_bwd_args(pkv, FLEXATTN_PASS_DKV, &akv)) != FLEXATTN_OK) return rc;
+  if (pq->ds != nullptr || pkv->ds != nullptr)
+    return set_error(FLEXATTN_EINVAL, "flexattn_bwd runs the two passes side by side: no dS hand-over (call flexattn_bwd_dkv, then flexattn_bwd_dq)");
+  if (pq->B != pkv->B || pq->Hq != pkv->Hq || pq->Hkv != pkv->Hkv || pq->Sq != pkv->Sq || pq->Sk != pkv->Sk || pq->D != pkv->D ||
+      pq->dtype != pkv->dtype || pq->q != pkv->q || pq->k != pkv->k || pq->v != pkv->v || pq->dout != pkv->dout)
+    return set_error(FLEXATTN_EINVAL, "flexattn_bwd: the two parameter blocks describe different problems");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // delta once, for both passes
+  if (pq->o != nullptr) {
+    if (pkv->o == nullptr && pkv->delta != pq->delta_out)
+      return set_error(FLEXATTN_EINVAL, "flexattn_bwd: the dk/dv block must read the delta that the dq block's call computes");
+    if ((rc = delta_first(&aq, pq->D, pq->dtype, s)) != FLEXATTN_OK) return rc;
+    akv.delta = aq.delta;
+    akv.o = nullptr;
+  } else if ((rc = delta_first(&akv, pkv->D, pkv->dtype, s)) != FLEXATTN_OK) {
+    return rc;
+  }
+  // (The two passes do not depend on each other, but running them side by side on two streams does not pay where it
+  // could, on problems too small to fill the GPU: those are bound by the host's launch path, and the event record /
+  // wait pairs of a fork and a join cost it more than the overlap saves: measured on B=1, H=4, S=512, fp32: 110 us
+  // per backward against 65 us for the three launches in a row.)
+  if ((rc = launch_dq(pq, aq, s)) != FLEXATTN_OK) return rc;
+  return launch_dkv(pkv, akv, s);
+}
+
+int64_t flexattn_bwd_ds_bytes(const flexattn_bwd_params* p) { return ds_exchange_ok(p) ? ds_bytes_of(p) : 0; }
+
+int flexattn_bwd_dq(const flexattn_bwd_params* p, void* stream) {
+  BwdArgs a;
+  int rc = to_bwd_args(p, FLEXATTN_PASS_DQ, &a);
+  if (rc != FLEXATTN_OK) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if ((rc = delta_first(&a, p->D, p->dtype, s)) != FLEXATTN_OK) return rc;
+  return launch_dq(p, a, s);   // (ds: checked to be bf16 and a plain or softcap score; the softcap streams leave 4 out of dS)
+}
+
 int flexattn_bwd_dkv(const flexattn_bwd_params* p, void* stream) {
   BwdArgs a;
   int rc = to_bwd_args(p, FLEXATTN_PASS_DKV, &a);
   if (rc != FLEXATTN_OK) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (p->dtype == FLEXATTN_BF16) return bwd_dkv_bf16_d128(a, s);
-  return (a.flags & FLEXATTN_FLAG_COMPILED_LOOP) ? bwd_dkv_f32(a, p->D, s) : bwd_dkv_f32_mfma(a, p->D, s);
+  if ((rc = delta_first(&a, p->D, p->dtype, s)) != FLEXATTN_OK) return rc;
+  return launch_dkv(p, a, s);
 }
 
 }  // extern "C"

@@ -96,6 +96,10 @@ struct BwdArgs {
   // gradient of the additive bias, float32 [B, Hq, Sq, Sk], or null: the dq kernels with a compiled loop store
   // P (dP - delta) of every element of the tiles they visit (0 where the element mask drops it)
   float* dab;
+  // delta computed by the call: with `o` set, the delta kernel runs in front of the pass and writes delta_out
+  // (the entry points resolve this before a kernel sees the arguments)
+  const void* o;
+  float* delta_out;
   int B, Hq, Hkv, Sq, Sk;
   float sm_scale;
   int flags;  // FLEXATTN_FLAG_*

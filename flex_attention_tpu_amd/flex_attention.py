@@ -26,6 +26,38 @@ from .flex_attention_kernel import _flex_attention_impl
 # declines it, and the dq pass recomputes, when it would take more than half of the free device memory.
 
 
+def flex_attention_bwd(q, k, v, ab, segment_ids, l, m, o, do, *, block_q, block_k, sm_scale, causal=False, score_fn=None,
+                       mask_fn=None, block_mask_fn=None, compiled_loop=False):
+    """(dq, dk, dv) of one backward: delta = sum(o * do), the dq pass and the dk/dv pass (the sequence of the
+    reference's custom_vjp wiring, jax_exp.py:276-321) from one call through the C ABI (flexattn_bwd): small
+    problems are bound by the host's path to a launch.  No dS hand-over (see flash_attention_bwd_dkv(return_ds=True) for that) and no bias
+    gradient (flex_attention_bwd_dq(return_dab=True))."""
+    import ctypes as C
+    from . import _lib
+    from ._common import on_device, stream_of
+    kw = dict(sm_scale=sm_scale, debug=False, score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn,
+              compiled_loop=compiled_loop)
+    dq_call = flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, None, block_b=1, block_q=block_q,
+                                    block_k_major=block_k, block_k=block_k, causal=causal, return_delta=True, _defer=True, **kw)
+    dkv_call = None
+    if dq_call is not None and dq_call["delta"] is not None:
+        dkv_call = flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, dq_call["delta"], do, block_b=1, block_q=block_q,
+                                           block_q_major=block_q, block_k_major=block_k, block_k=block_k, causal=causal,
+                                           _defer=True, **kw)
+    if dkv_call is None:   # (padded shapes, ids per batch entry: the passes one after the other)
+        dq, di = flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, None, block_b=1, block_q=block_q,
+                                       block_k_major=block_k, block_k=block_k, causal=causal, return_delta=True, **kw)
+        dk, dv = flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, block_b=1, block_q=block_q,
+                                         block_q_major=block_q, block_k_major=block_k, block_k=block_k, causal=causal, **kw)
+        return dq, dk, dv
+    lib = dq_call["lib"]
+    with on_device(q.device):
+        _lib.check(lib.flexattn_bwd(C.byref(dq_call["params"]), C.byref(dkv_call["params"]), stream_of(q)), lib)
+    dq, _ = dq_call["finish"]()
+    dk, dv = dkv_call["finish"]()
+    return dq, dk, dv
+
+
 class _FlexAttention(torch.autograd.Function):
     """o = softmax(mask(score_mod(sm_scale q k^T))) v with the saved statistics (l, m) for the backward."""
 
@@ -46,10 +78,31 @@ class _FlexAttention(torch.autograd.Function):
         score_fn, mask_fn, block_mask_fn, segment_ids, causal, sm_scale, block_q, block_k = ctx.opts
         want_dab = ab is not None and ctx.needs_input_grad[3]
         do = do.contiguous()
-        di = compute_delta(o, do)  # float32 [B, H, Sq]  (jax_exp.py:276-278)
         dq = dk = dv = ds = dab = None
-        if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
-            exchange = ctx.needs_input_grad[0] and ds_exchange_pays(score_fn, mask_fn, segment_ids)
+        want_dkv = ctx.needs_input_grad[1] or ctx.needs_input_grad[2]
+        want_dq = ctx.needs_input_grad[0] or want_dab
+        exchange = (want_dkv and ctx.needs_input_grad[0] and ab is None and q.dtype == torch.bfloat16 and
+                    ds_exchange_pays(score_fn, mask_fn, segment_ids))
+        # di = sum(o * do), float32 [B, H, Sq] (jax_exp.py:276-278): taken by the dq pass itself where that pass runs
+        # first (no dS hand-over), else by its own launch
+        di = None
+        if want_dkv and ctx.needs_input_grad[0] and not want_dab and not exchange:
+            dq, dk, dv = flex_attention_bwd(q, k, v, ab, segment_ids, l, m, o, do, block_q=block_q, block_k=block_k,
+                                            sm_scale=sm_scale, causal=causal, score_fn=score_fn, mask_fn=mask_fn,
+                                            block_mask_fn=block_mask_fn)
+            return dq, dk, dv, None, None
+        if want_dq and not exchange:
+            dq = flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, None, block_b=1, block_q=block_q,
+                                       block_k_major=block_k, block_k=block_k, sm_scale=sm_scale, debug=False,
+                                       score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn, causal=causal,
+                                       return_dab=want_dab, return_delta=not want_dab)
+            if want_dab:
+                dq, dab = dq
+            else:
+                dq, di = dq
+        if di is None and want_dkv:
+            di = compute_delta(o, do)
+        if want_dkv:
             dk, dv, ds = flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, block_b=1, block_q=block_q,
                                                  block_q_major=block_q, block_k_major=block_k, block_k=block_k,
                                                  sm_scale=sm_scale, causal=causal, debug=False, score_fn=score_fn,
@@ -58,13 +111,11 @@ class _FlexAttention(torch.autograd.Function):
                     k, v, q, ab, segment_ids, l, m, di, do, block_b=1, block_q=block_q, block_q_major=block_q,
                     block_k_major=block_k, block_k=block_k, sm_scale=sm_scale, causal=causal, debug=False,
                     score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn), None)
-        if ctx.needs_input_grad[0] or want_dab:   # (the bias gradient is an output of the dq pass)
+        if want_dq and exchange:
             dq = flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, di, block_b=1, block_q=block_q,
                                        block_k_major=block_k, block_k=block_k, sm_scale=sm_scale, debug=False,
                                        score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn, causal=causal,
-                                       ds=ds, return_dab=want_dab)
-            if want_dab:
-                dq, dab = dq
+                                       ds=ds)
         return dq if ctx.needs_input_grad[0] else None, dk, dv, dab, None
 
 

@@ -8,14 +8,14 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (batch_entry, bias_c, check_blocks, check_qkv, check_rows, kernel_block_map, kernel_head_dim, library_for, pad_seq,
+from ._common import (on_device, batch_entry, bias_c, check_blocks, check_qkv, check_rows, kernel_block_map, kernel_head_dim, library_for, pad_seq,
                       padded_len, per_batch_segments, resolve_mask, stream_of)
 from .flex_attention_dq_bwd import DsBlocks, alloc_ds, bwd_params
 
 
 def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=None, block_q, block_q_major,
                             block_k_major, block_k, sm_scale, causal, debug, score_fn=None, mask_fn=None,
-                            block_mask_fn=None, compiled_loop=False, return_ds=False):
+                            block_mask_fn=None, compiled_loop=False, return_ds=False, _defer=False):
     """(dk, dv): dv = P^T do, dk = dS^T * d(score)/dk with P recomputed from (l, m) and
     dS = P (dP - di) (flex_attention_dkv_kernel.py:237-272).  With grouped KV heads the gradients
     of all query heads of a group are summed inside the kernel.  ``causal`` is honoured
@@ -26,6 +26,8 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     block per query head and kept pair of 128 x 128 tiles): the dq pass then recomputes as usual."""
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v, do)
     rows = per_batch_segments(segment_ids, B)
+    if rows is not None and _defer:
+        return None
     if rows is not None:  # ids differ between batch entries: one launch per entry
         outs = [flash_attention_bwd_dkv(
             k[b:b + 1], v[b:b + 1], q[b:b + 1], batch_entry(ab, b), rows[b], l[b:b + 1], m[b:b + 1], di[b:b + 1], do[b:b + 1],
@@ -54,8 +56,12 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     p = bwd_params(q, k, v, l, m, do, di, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dk=dk, dv=dv,
                    compiled_loop=compiled_loop, ab_c=ab_c)
     ds = None
-    with torch.cuda.device(q.device):
-        lib = library_for(score_fn, spec)
+    lib = library_for(score_fn, spec)
+    if _defer:   # (flex_attention_bwd launches this pass together with the dq pass: whole tiles only, no hand-over)
+        if Sk_p != Sk or Sq_p != Sq or D != D_user or return_ds:
+            return None
+        return {"params": p, "lib": lib, "finish": lambda: (dk, dv), "keep": (q, k, v, do, l, m, di, ab_keep, bm)}
+    with on_device(q.device):
         if return_ds:
             p.ds_index.pairs = 1   # (asks whether the kernels of the call exchange at all, before the index is built)
             if lib.flexattn_bwd_ds_bytes(C.byref(p)) > 0:

@@ -7,7 +7,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (batch_entry, bias_c, check_blocks, check_qkv, check_rows, dtype_code, kernel_block_map, kernel_head_dim, library_for,
+from ._common import (on_device, batch_entry, bias_c, check_blocks, check_qkv, check_rows, dtype_code, kernel_block_map, kernel_head_dim, library_for,
                       pad_seq, padded_len, per_batch_segments, resolve_mask, score_spec_c, stream_of)
 from .block_mask import mask_spec_c
 
@@ -24,7 +24,7 @@ def compute_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
         D = kernel_head_dim(D, o.dtype)
         o, do = pad_seq(o, D, 3), pad_seq(do, D, 3)
     d = torch.empty(B, H, S, dtype=torch.float32, device=o.device)
-    with torch.cuda.device(o.device):
+    with on_device(o.device):
         _lib.check(_lib.load().flexattn_bwd_delta(o.data_ptr(), do.data_ptr(), d.data_ptr(), B * H * S, D,
                                                   dtype_code(o), stream_of(o)))
     return d
@@ -40,21 +40,24 @@ class DsBlocks:
         self.buf, self.shape, self.entries, self.index = buf, shape, entries, index
 
 
-# The dS buffer is never allowed to take more than this share of the device memory that is free when it is
-# asked for: the backward must not fail for want of memory where the recomputing dq pass would have worked.
-DS_FREE_MEMORY_SHARE = 0.5
+# The dS buffer is never allowed to take more than this share of the device's memory, and an out-of-memory error of
+# the allocator is caught: the backward must not fail for want of memory where the recomputing dq pass would have worked.
+DS_MEMORY_SHARE = 0.25
+_total_memory = {}
 
 
 def alloc_ds(nbytes: int, device):
-    """The dS exchange buffer, or None when it does not fit comfortably: more than DS_FREE_MEMORY_SHARE of the
-    memory that is free (the driver's figure plus what torch's allocator holds unused), or an out-of-memory error
-    from the allocator all the same.  The caller then runs the two recomputing passes."""
-    free, _ = torch.cuda.mem_get_info(device)
-    cached = torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)
-    if nbytes > DS_FREE_MEMORY_SHARE * (free + cached):
+    """The dS exchange buffer, or None when it does not fit comfortably: more than DS_MEMORY_SHARE of the device's
+    memory, or an out-of-memory error from the allocator.  The caller then runs the two recomputing passes.  (The
+    driver's figure of free memory is not asked per call: the query takes 0.2 ms and holds the launch path up.)"""
+    dev = torch.device(device)
+    total = _total_memory.get(dev)
+    if total is None:
+        total = _total_memory[dev] = torch.cuda.get_device_properties(dev).total_memory
+    if nbytes > DS_MEMORY_SHARE * total:
         return None
     try:
-        return torch.empty(nbytes, dtype=torch.uint8, device=device)
+        return torch.empty(nbytes, dtype=torch.uint8, device=dev)
     except torch.cuda.OutOfMemoryError:
         return None
 
@@ -69,7 +72,10 @@ def ds_exchange_pays(score_fn, mask_fn=None, segment_ids=None) -> bool:
     shape: 1.75 -> 1.34; five documents in B=4, H=32, S=4096: 1.09 -> 0.91; causal window 1025, B=2, H=16, S=8192:
     0.56 -> 0.49; softcap, causal, B=4, H=32, S=4096: 2.08 -> 1.86; plain causal, same shape: 1.67 -> 1.68; plain
     causal GQA 4:1, B=2, Hq=32, S=8192: 3.09 -> 3.17."""
-    if getattr(getattr(score_fn, "spec", None), "kind", None) == _lib.SCORE_SOFTCAP:
+    kind = getattr(getattr(score_fn, "spec", None), "kind", _lib.SCORE_NONE if score_fn is None else None)
+    if kind not in (_lib.SCORE_NONE, _lib.SCORE_SOFTCAP):
+        return False   # (position biases and compiled score functions: their kernels exchange nothing)
+    if kind == _lib.SCORE_SOFTCAP:
         return True
     if segment_ids is not None:
         return True
@@ -92,12 +98,15 @@ def bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, mod_q, mod_k,
 
 def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, block_q, block_k_major,
                           block_k, sm_scale, debug, score_fn=None, mask_fn=None, block_mask_fn=None,
-                          causal=False, compiled_loop=False, ds=None, return_dab=False):
+                          causal=False, compiled_loop=False, ds=None, return_dab=False, return_delta=False, _defer=False):
     """dq = sum_j dS_ij * d(score)/dq, with P_ij = exp(S_ij - m_i) / l_i recomputed from the saved
     statistics, dP = do v^T, dS = P (dP - d) (flex_attention_dq_bwd.py:340-378).  ``o`` is only
     shape-checked, as in the reference (:163); ``d`` is the caller's delta (see compute_delta).
     ``ds``: the DsBlocks of the dk/dv pass of the same arguments, if that pass returned one: dq is then
     sm_scale dS K, nothing is recomputed.
+    ``d=None``: the call takes delta = sum(o * do) itself (the reference hands ``o`` to this function without using
+    it, :163): the delta kernel runs in front of the dq kernel, one call through the C ABI instead of two;
+    ``return_delta=True`` then returns (dq, d) so that the dk/dv pass can be given the same d.
     ``return_dab=True`` (needs ``ab``; excludes ``ds``) returns (dq, dab): the gradient of the additive bias in
     ab's shape and dtype, dab = P (dP - d) summed over the dimensions ``ab`` broadcasts -- the output the
     reference declares next to dk, dv (flash_attention_dkv_bwd.py:103-107,130-138) and its upstream dq kernel
@@ -109,13 +118,25 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
             raise ValueError("ds does not come from a dk/dv pass of these arguments")
         if return_dab:
             raise NotImplementedError("return_dab with segment ids that differ between batch entries")
-        return torch.cat([flex_attention_bwd_dq(
+        if _defer:
+            return None
+        if d is None:
+            d = compute_delta(o, do)
+        out = torch.cat([flex_attention_bwd_dq(
             q[b:b + 1], k[b:b + 1], v[b:b + 1], batch_entry(ab, b), rows[b], l[b:b + 1], m[b:b + 1], batch_entry(o, b),
             do[b:b + 1], d[b:b + 1], block_b=block_b, block_q=block_q, block_k_major=block_k_major, block_k=block_k,
             sm_scale=sm_scale, debug=debug, score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn, causal=causal,
             compiled_loop=compiled_loop, ds=ds.entries[b] if ds is not None else None) for b in range(B)], 0)
+        return (out, d) if return_delta else out
     if o is not None and tuple(o.shape) != tuple(q.shape):
         raise ValueError(f"o has shape {tuple(o.shape)}, expected {tuple(q.shape)}")
+    fuse_delta = d is None
+    if fuse_delta:
+        if o is None or ds is not None:
+            raise ValueError("d=None needs `o` (delta is then taken of o and do) and excludes `ds`")
+        if o.dtype != q.dtype or not o.is_contiguous() or o.device != q.device:
+            raise ValueError("o must be a contiguous tensor of q's dtype on q's device")
+        d = torch.empty(B, Hq, Sq, dtype=torch.float32, device=q.device)
     for name, t in (("l", l), ("m", m), ("d", d)):
         check_rows(name, t, B, Hq, Sq, q.device)
     check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k)
@@ -123,17 +144,20 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     Sq_p, Sk_p = padded_len(Sq), padded_len(Sk)
     spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk, Sq_p, Sk_p)
     q, do, k, v = pad_seq(q, Sq_p), pad_seq(do, Sq_p), pad_seq(k, Sk_p), pad_seq(v, Sk_p)
-    l, m, d = pad_seq(l, Sq_p), pad_seq(m, Sq_p), pad_seq(d, Sq_p)
+    l, m, d_p = pad_seq(l, Sq_p), pad_seq(m, Sq_p), pad_seq(d, Sq_p)
     D_user, D = D, kernel_head_dim(D, q.dtype)   # smaller head dimensions: zero-padded columns
     q, do, k, v = pad_seq(q, D, 3), pad_seq(do, D, 3), pad_seq(k, D, 3), pad_seq(v, D, 3)
+    o_p = pad_seq(pad_seq(o, Sq_p), D, 3) if fuse_delta else None
     if ds is not None and (ds.buf is None or ds.index is None or ds.shape != (B, Hq, Sq_p, Sk_p) or ds.buf.device != q.device):
         raise ValueError("ds does not come from a dk/dv pass of these arguments")
     # (the dS blocks lie at the dk/dv kernel's tiles: the dq pass walks that map's row lists)
     bm = kernel_block_map(_lib.PASS_DKV if ds is not None else _lib.PASS_DQ, spec, q, Sq_p, Sk_p, D, score_fn)
     dq = torch.empty_like(q)
     ab_c, ab_keep = bias_c(ab, B, Hq, Sq, Sk, Sq_p, Sk_p, q.device)
-    p = bwd_params(q, k, v, l, m, do, d, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dq=dq,
+    p = bwd_params(q, k, v, l, m, do, d_p, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dq=dq,
                    compiled_loop=compiled_loop, ab_c=ab_c)
+    if fuse_delta:
+        p.delta, p.o, p.delta_out = None, o_p.data_ptr(), d_p.data_ptr()
     dab_full = None
     if return_dab:
         if ab is None or ds is not None:
@@ -145,16 +169,29 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
         p.ds, p.ds_bytes = ds.buf.data_ptr(), ds.buf.numel()
         col, rank, pairs = ds.index   # (the index the dk/dv pass wrote the blocks by)
         p.ds_index = _lib.DsIndexC(col.data_ptr(), rank.data_ptr(), pairs)
-    with torch.cuda.device(q.device):
-        lib = library_for(score_fn, spec)
+    if return_delta and return_dab:
+        raise ValueError("return_delta and return_dab exclude each other")
+    lib = library_for(score_fn, spec)
+    keep = (q, k, v, do, l, m, d_p, o_p, ab_keep, bm, dab_full)   # what the parameter block points at
+
+    def finish():
+        """The call's results from the kernels' output buffers (cuts padding off, reduces the bias gradient)."""
+        out, d_out = dq, d
+        if Sq_p != Sq or D != D_user:
+            out = out[:, :, :Sq, :D_user].contiguous()
+        if fuse_delta and d_p is not d:
+            d_out = d_p[:, :, :Sq].contiguous()
+        if not return_dab:
+            return (out, d_out) if return_delta else out
+        dab = dab_full[:, :, :Sq, :Sk]
+        if ab.shape[0] == 1 and B > 1:
+            dab = dab.sum(0, keepdim=True)
+        if ab.shape[1] == 1 and Hq > 1:
+            dab = dab.sum(1, keepdim=True)
+        return out, dab.to(ab.dtype).contiguous()
+
+    if _defer:   # (flex_attention_bwd launches this pass together with the dk/dv pass)
+        return {"params": p, "lib": lib, "finish": finish, "keep": keep, "delta": d if d_p is d else None}
+    with on_device(q.device):
         _lib.check(lib.flexattn_bwd_dq(C.byref(p), stream_of(q)), lib)
-    if Sq_p != Sq or D != D_user:
-        dq = dq[:, :, :Sq, :D_user].contiguous()
-    if not return_dab:
-        return dq
-    dab = dab_full[:, :, :Sq, :Sk]
-    if ab.shape[0] == 1 and B > 1:
-        dab = dab.sum(0, keepdim=True)
-    if ab.shape[1] == 1 and Hq > 1:
-        dab = dab.sum(1, keepdim=True)
-    return dq, dab.to(ab.dtype).contiguous()
+    return finish()

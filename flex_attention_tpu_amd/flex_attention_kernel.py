@@ -12,7 +12,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (batch_entry, bias_c, check_blocks, check_qkv, dtype_code, kernel_block_map, kernel_head_dim, library_for, pad_seq,
+from ._common import (on_device, batch_entry, bias_c, check_blocks, check_qkv, dtype_code, kernel_block_map, kernel_head_dim, library_for, pad_seq,
                       padded_len, per_batch_segments, resolve_mask, score_spec_c, stream_of)
 from .block_mask import mask_spec_c
 
@@ -58,7 +58,7 @@ def _flex_attention_impl(q, k, v, ab, segment_ids, save_residuals, causal, sm_sc
         B, Hq, Hkv, Sq_p, Sk_p, D, dtype_code(q), float(sm_scale), _lib.FLAG_COMPILED_LOOP if compiled_loop else 0, 0,
         score_spec_c(score_fn, Hq, q.device, block_q or 1, block_k or 1, sm_scale),
         mask_spec_c(spec, Sq_p, Sk_p, q.device), bm.as_c(), ab_c)
-    with torch.cuda.device(q.device):
+    with on_device(q.device):
         lib = library_for(score_fn, spec)
         _lib.check(lib.flexattn_fwd(C.byref(p), stream_of(q)), lib)
     if Sq_p != Sq or D != D_user:

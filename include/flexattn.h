@@ -165,6 +165,14 @@ typedef struct flexattn_bwd_params {
    * dq kernel writes it, jax_exp.py:1252-1255, there multiplied by sm_scale).  Only the tiles the block map visits
    * are written: clear the buffer first.  A call with dab runs the dq kernel with a compiled main loop; it excludes ds. */
   float* dab;
+  /* delta computed by the call, optional: with o ([B,Hq,Sq,D], the forward's output) and delta_out ([B,Hq,Sq]
+   * float32) set, `delta` is ignored: delta = sum(o * dout) is taken by the call and written to delta_out (the
+   * reference leaves the reduction to its callers, flex_attention_dq_bwd.py:932, and hands `o` to its dq entry
+   * point without using it, :163): the delta kernel is launched in front of the pass on the same stream, one call
+   * across the boundary instead of two.  A dk/dv call of the same backward then reads delta_out as its `delta`.
+   * Excludes ds. */
+  const void* o;
+  float* delta_out;
 } flexattn_bwd_params;
 
 #define FLEXATTN_PASS_FWD 0
@@ -243,6 +251,13 @@ int flexattn_bwd_dq(const flexattn_bwd_params* p, void* stream);
 /* dk/dv backward.  Replaces the pallas_call in flash_attention_bwd_dkv
  * (flex_attention_dkv_kernel.py:158-172; mask-aware twin flash_attention_dkv_bwd.py:164-178). */
 int flexattn_bwd_dkv(const flexattn_bwd_params* p, void* stream);
+
+/* The whole backward from one call: delta (when the dq block names `o` and `delta_out`), the dq pass of `dq` and the
+ * dk/dv pass of `dkv` (the two blocks describe the same problem, each with the block map of its pass; no dS hand-over),
+ * launched one after the other on `stream`.  Replaces the sequence the reference's custom_vjp wiring runs
+ * (jax_exp.py:276-321: di, then the dk/dv and the dq kernels) by one call across the boundary: small problems are
+ * bound by the host's path to a launch, not by the kernels. */
+int flexattn_bwd(const flexattn_bwd_params* dq, const flexattn_bwd_params* dkv, void* stream);
 
 #ifdef __cplusplus
 }

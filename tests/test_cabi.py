@@ -38,7 +38,7 @@ def test_struct_sizes_follow_c_layout():
     assert C.sizeof(_lib.BiasC) == 32
     assert C.sizeof(_lib.FwdParamsC) == 6 * 8 + 10 * 4 + 32 + 48 + 56 + 32
     assert C.sizeof(_lib.DsIndexC) == 24
-    assert C.sizeof(_lib.BwdParamsC) == 10 * 8 + 10 * 4 + 32 + 48 + 56 + 32 + 16 + 24 + 8
+    assert C.sizeof(_lib.BwdParamsC) == 10 * 8 + 10 * 4 + 32 + 48 + 56 + 32 + 16 + 24 + 8 + 16
 
 
 def test_tile_shapes(lib):
@@ -125,6 +125,8 @@ def test_ds_exchange_sizes_and_argument_checks(lib):
     p.ds_bytes = 2 * 4 * 256 * 384 * 2 - 1
     for call in (lib.flexattn_bwd_dq, lib.flexattn_bwd_dkv):
         assert call(C.byref(p), None) == _lib.EINVAL and b"needs" in lib.flexattn_last_error_string()
+    # the whole backward from one call: both blocks are checked, and they must describe the same problem
+    assert lib.flexattn_bwd(None, None, None) == _lib.EINVAL
     # the index builder checks its arguments
     assert lib.flexattn_build_ds_index(None, None, None, None) == _lib.EINVAL
     m = _lib.BlockMapC()

@@ -162,11 +162,11 @@ def test_ds_buffer_holds_the_kept_pairs_only(F):
     assert ds is not None and ds.buf.numel() == 2 * kept * 128 * 128 * 2 and kept == 122
     # a device without room for the buffer: the pass declines the exchange, the dq pass then recomputes
     from flex_attention_tpu_amd import flex_attention_dq_bwd as dqmod
-    share, dqmod.DS_FREE_MEMORY_SHARE = dqmod.DS_FREE_MEMORY_SHARE, 0.0
+    share, dqmod.DS_MEMORY_SHARE = dqmod.DS_MEMORY_SHARE, 0.0
     try:
         dk2, dv2, ds2 = _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, None, return_ds=True)
     finally:
-        dqmod.DS_FREE_MEMORY_SHARE = share
+        dqmod.DS_MEMORY_SHARE = share
     assert ds2 is None and torch.equal(dk2, dk) and torch.equal(dv2, dv)
 
 
@@ -217,11 +217,38 @@ def test_small_shapes_all_passes(F, case, dtype):
     dq = _dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, score_fn)
     dk, dv = _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, score_fn)
     _check_grads((dq, dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, dtype, dict(sm_scale=sc, **okw))
+    # d=None: the dq pass takes delta itself (the bf16 stream kernels while they fetch an item's rows, the others
+    # through the delta kernel): the same delta and the same dq, bit for bit
+    dq_f, d_f = F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, None, block_b=1, block_q=128, block_k_major=128,
+                                        block_k=128, sm_scale=sc, debug=False, score_fn=score_fn, mask_fn=mf,
+                                        block_mask_fn=bf, return_delta=True)
+    assert torch.equal(d_f, d) and torch.equal(dq_f, dq), "delta taken by the dq pass differs from the delta kernel's"
     # dS exchange: the bf16 stream kernels of plain and softcap scores offer it
     dqx = _exchanged_dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, score_fn, dk, dv,
                         expect=dtype == torch.bfloat16 and not name.startswith("alibi"))
     if dqx is not None:
         _check_grads((dqx, dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, dtype, dict(sm_scale=sc, **okw), tag="exchange ")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+def test_whole_backward_from_one_call(F, dtype):
+    """flex_attention_bwd (flexattn_bwd: delta, dq and dk/dv from one call) gives the bits of the three separate
+    calls: a small problem (twice in a row), a larger one, and a ragged one (which falls back to the separate
+    calls)."""
+    from flex_attention_tpu_amd import masks, scores
+    sc = 1 / math.sqrt(128)
+    for (B, Hq, Hkv, S), repeat in (((1, 4, 2, 512), 2), ((2, 8, 8, 2048), 1), ((1, 2, 2, 300), 1)):
+        q, k, v, do = (x.to(DEV) for x in O.make_inputs(B, Hq, Hkv, S, S, 128, dtype=dtype, seed=97))
+        mf, bf = masks.make_causal_mask_fns(128, 128)
+        sfn = scores.make_softcap_score_fn(20.0)
+        o, l, m = _fwd(F, q, k, v, sc, mf, bf, sfn)
+        d = F.compute_delta(o, do)
+        dq = _dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, sfn)
+        dk, dv = _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, sfn)
+        for _ in range(repeat):
+            dq2, dk2, dv2 = F.flex_attention_bwd(q, k, v, None, None, l, m, o, do, block_q=128, block_k=128, sm_scale=sc,
+                                                 score_fn=sfn, mask_fn=mf, block_mask_fn=bf)
+            assert torch.equal(dq2, dq) and torch.equal(dk2, dk) and torch.equal(dv2, dv), (B, Hq, S)
 
 
 def test_causal_flag_and_segment_ids_arguments(F):
@@ -933,6 +960,11 @@ def _full_config_check(F, name, n_rows, heads_q, dense_group):
     d = F.compute_delta(o, dog)
     dq = _dq(F, qg, kg, vg, l, m, o, dog, d, sc, mf, bf, sfn)
     dk, dv = _dkv(F, qg, kg, vg, l, m, dog, d, sc, mf, bf, sfn)
+    # (the same dq pass taking delta itself, as the package's backward runs it: the same bits)
+    dq_f, d_f = F.flex_attention_bwd_dq(qg, kg, vg, None, None, l, m, o, dog, None, block_b=1, block_q=128, block_k_major=128,
+                                        block_k=128, sm_scale=sc, debug=False, score_fn=sfn, mask_fn=mf, block_mask_fn=bf,
+                                        return_delta=True)
+    assert torch.equal(d_f, d) and torch.equal(dq_f, dq), "delta taken by the dq pass differs from the delta kernel's"
     d_s = F.compute_delta(o, dosg)
     dk_s, dv_s = _dkv(F, qg, kg, vg, l, m, dosg, d_s, sc, mf, bf, sfn)
     # the same backward with dS handed from the dk/dv pass to the dq pass (plain and softcap scores)
