@@ -20,8 +20,9 @@ PEAK_HBM_GBS = 8000.0
 
 
 def sweep(max_seq: int = 65536, min_seq: int = 1024, heads: int = 8, iters: int = 10, causal: bool = True, device="cuda:0"):
-    """Rows (dict) of the sweep.  Sequences longer than the generated-stream kernels' list cache (64k at
-    the forward's 64-row kv tiles) run the kernels with a compiled main loop."""
+    """Rows (dict) of the sweep.  Every length up to 262144 runs the generated-stream kernels (their list cache holds
+    4096 kv tiles of 64 rows resp. 2048 q tiles of 128); longer sequences would take the kernels with a compiled
+    main loop."""
     import torch
     import flex_attention_tpu_amd as F
     from flex_attention_tpu_amd import masks
