@@ -730,7 +730,10 @@ int bwd_dq_bf16_d128(const BwdArgs& a, hipStream_t stream) {
 #else
   // (the generated-stream kernel caches the kv list in LDS)
   // (and has no additive bias)
-  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= dq_cfg::MAX_LIST && a.score.ab == nullptr;
+  // (and folds its scale into bf16 Q: folded_scale_ok)
+  const float fold = a.score.kind == FLEXATTN_SCORE_SOFTCAP ? 2.0f * kLog2e * a.sm_scale / a.score.cap : a.sm_scale * kLog2e;
+  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= dq_cfg::MAX_LIST && a.score.ab == nullptr &&
+                         folded_scale_ok(fold, a.sm_scale, 128);
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
       return stream_ok ? launch_dq_plain<0>(a, stream) : launch_dq<FLEXATTN_SCORE_NONE>(a, stream);

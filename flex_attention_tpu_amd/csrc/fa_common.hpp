@@ -37,6 +37,21 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kNegInf = -__builtin_huge_valf();
 
+// The generated-stream kernels of the forward and dq fold their scale (sm_scale log2 e; softcap: 2 log2 e sm_scale /
+// cap) into the bf16 copy of Q they keep in registers, so every logit carries that product's rounding: about
+// 2^-9 / sqrt(3) * fold * sqrt(sum_i (q_i k_i)^2) in the exponent, i.e. 0.0011 fold sqrt(D) for unit-variance
+// operands.  At the usual sm_scale = 1 / sqrt(D) that is 0.0016, below the 2^-9 the probabilities lose anyway when
+// they are rounded to bf16 for the second product.  With sm_scale = 1 on such operands (the reference's own
+// drivers) it is 0.018: probabilities off by 1.3 %, lse by 0.06, dq by 2 % in relative L2.  Such calls take the
+// kernels with a compiled main loop, which scale the fp32 product.  A power of two folds exactly.  (Softcap: the
+// exponent moves by at most cap log2 e / 2 per unit of the chain's result, so the rounding of its fold weighs what
+// the plain fold sm_scale log2 e would: the same bound on sm_scale serves.)
+inline bool folded_scale_ok(float fold, float sm_scale, int D) {
+  int e;
+  const float mant = __builtin_frexpf(fold, &e);
+  return mant == 0.5f || sm_scale * kLog2e * __builtin_sqrtf((float)D) <= 2.9f;
+}
+
 // Kernel-side views of the C ABI structs (pointers already typed).
 struct ScoreArgs {
   int kind;

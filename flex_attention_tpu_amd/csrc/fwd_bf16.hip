@@ -904,7 +904,10 @@ int fwd_bf16_d128(const FwdArgs& a, hipStream_t stream) {
   // The generated-stream kernel (one wave per SIMD, 64 q rows per wave) keeps the state rows and the
   // merged kv list in LDS, hence the bound on the list length.
   // and has no additive bias.
-  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= fwd_cfg::MAX_LIST && a.score.ab == nullptr;
+  // and whose scale, folded into bf16 Q, must not cost the logits their accuracy (folded_scale_ok).
+  const float fold = a.score.kind == FLEXATTN_SCORE_SOFTCAP ? 2.0f * kLog2e * a.sm_scale / a.score.cap : a.sm_scale * kLog2e;
+  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= fwd_cfg::MAX_LIST && a.score.ab == nullptr &&
+                         folded_scale_ok(fold, a.sm_scale, 128);
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
       if (a.score.ab != nullptr) return launch_fwd<kScoreBiasOnly>(a, stream);

@@ -21,8 +21,14 @@ def oracle_kwargs(cfg):
     return O.kwargs_for_config(cfg)
 
 
-def assert_close(name, test, ref, dtype, chain=False):
+def assert_close(name, test, ref, dtype, chain=False, tensor_scale=False):
     """rel-L2 (benchmark_fwd.py:81-83 of the reference) and max-abs against the tolerance of the dtype.
+
+    `tensor_scale=True` (bf16 gradients whose magnitude is far above 1, as with the reference drivers' sm_scale = 1:
+    dq and dk reach 40 there) takes the absolute bound of the tensor's largest magnitude for every element,
+    max(2e-2, 2^-7 max|ref|), instead of each element's own: an element of dq = sum_j dS_ij k_j carries the rounding
+    of the dS and k terms it sums (dS is rounded to bf16 for the product, in the reference's kernels as here), whose
+    size is the row's, not the element's.  For tensors up to 2.56 in magnitude that is the literal 2e-2.
 
     float32: max-abs <= 1e-5 and rel-L2 <= 1e-5, as written.
     bfloat16: rel-L2 <= 1e-2 and, element by element, |test - ref| <= max(2e-2, 2^-7 |ref|).  The
@@ -49,7 +55,7 @@ def assert_close(name, test, ref, dtype, chain=False):
     ma, rl = O.max_abs(test, ref), O.rel_l2(test, ref)
     ref_max = float(ref.abs().max())
     if dtype == torch.bfloat16:
-        bound = torch.clamp(ref.abs() * 2.0 ** -7, min=BF16_ABS)
+        bound = torch.clamp((ref.abs().max() if tensor_scale else ref.abs()) * 2.0 ** -7, min=BF16_ABS)
         ratio = float(((test - ref).abs() / bound).max())
         rel_tol = BF16_REL
     else:

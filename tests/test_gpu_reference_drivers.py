@@ -1,0 +1,152 @@
+"""GPU parity on the workloads of the reference's own driver scripts, with their arguments.
+
+The reference has no test suite: each of its drivers builds one workload, runs the kernels and the dense
+reference and prints a relative L2 error (main.py:44-177 forward; flex_attention_dq_bwd.py:788-946 dq;
+flash_attention_dkv_bwd.py:772-940 dk/dv).  These tests run the same workloads through this package's entry
+points with the drivers' keyword arguments -- sm_scale = 1.0 on unit-variance bf16 inputs of head dimension
+128 (logits of standard deviation 11: softmax rows dominated by one or two keys, a harder regime than the
+1/sqrt(D) of the benchmark configurations), blocks of 1024, batch 1 -- and compare with the oracle on sampled
+rows at the stated tolerances (helpers.assert_close): rel-L2 <= 1e-2 for every tensor; o, lse and dv element by
+element; dq and dk, which reach magnitudes of 25 to 40 here, against the bound of the tensor's largest magnitude
+(`tensor_scale`).  Inputs come from this build's seeded generator (the reference's JAX PRNG streams are not
+reproducible without JAX).
+
+At this scale the library runs the forward and dq on the kernels that scale the fp32 product (the generated-stream
+kernels fold the scale into their bf16 copy of Q, which costs logits of this size their accuracy: o off by 0.06, dq
+by 2 % in relative L2 when measured), so these tests also pin that choice: they fail on the stream kernels.
+
+Differences from the drivers, on purpose: the backward takes the residuals of the forward under the same mask
+(the drivers feed the residuals of an unmasked forward to masked backward kernels; the one test of that habit
+below is test_backward_from_the_residuals_of_an_unmasked_forward), and the position-bias case is compared with
+the oracle's tile-local bias, which is what the reference's score function computes on a tile
+(scores.py:3-11), not with the global bias of its dense reference.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_close, same_residual_grads
+from oracle import mha_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+BLOCK = 1024      # block_q = block_k_major = block_k of the drivers
+SM_SCALE = 1.0
+
+
+@pytest.fixture(scope="module")
+def F():
+    import flex_attention_tpu_amd as F
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return F
+
+
+def driver_doc_lengths(total_len, num_docs, seed):
+    """Document lengths as the dk/dv driver draws them (flash_attention_dkv_bwd.py:747-770): num_docs - 1 distinct
+    cut points from numpy's legacy generator."""
+    np.random.seed(seed)
+    cuts = np.sort(np.random.choice(range(1, total_len), num_docs - 1, replace=False))
+    return [int(n) for n in np.diff(np.concatenate(([0], cuts, [total_len])))]
+
+
+def _driver_cases(S):
+    """(name, (mask_fn, block_mask_fn), score_fn, oracle keywords) of the drivers' case lists."""
+    from flex_attention_tpu_amd import masks, scores
+    lens = driver_doc_lengths(S, 5, 42)
+    return {
+        "causal": (masks.make_causal_mask_fns(BLOCK, BLOCK), None, dict(causal=True)),
+        "sliding_window_1024": (masks.make_sliding_window_mask_fns(BLOCK, BLOCK, 1024), None, dict(window_size=1024)),
+        "jagged_5_docs": (masks.make_jagged_mask_fns(BLOCK, BLOCK, lens), None,
+                          dict(causal=True, segment_ids=O.doc_ids_from_lengths(lens))),
+        "alibi_0.5": ((None, None), scores.make_alibi_score_fn(slope=0.5),
+                      dict(score_mod=O.score_mod_alibi_tile_local(0.5, BLOCK, BLOCK))),
+        "tanh_30": ((None, None), scores.make_softcap_score_fn(cap=30.0), dict(score_mod=O.score_mod_softcap(30.0))),
+    }
+
+
+def _run_all(F, q, k, v, do, mf, bf, sfn, fwd_masks=None):
+    """Forward, delta, dq and dk/dv with the drivers' keyword arguments.  `fwd_masks`: another mask pair for the
+    forward than for the backward."""
+    fm, fb = (mf, bf) if fwd_masks is None else fwd_masks
+    o, l, m = F._flex_attention_impl(q, k, v, None, None, True, False, SM_SCALE, 1, BLOCK, BLOCK, BLOCK, False, fb, fm, sfn)
+    d = F.compute_delta(o, do)
+    dq = F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=BLOCK, block_k_major=BLOCK,
+                                 block_k=BLOCK, sm_scale=SM_SCALE, debug=False, score_fn=sfn, mask_fn=mf, block_mask_fn=bf)
+    dk, dv = F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=BLOCK, block_q_major=BLOCK,
+                                       block_k_major=BLOCK, block_k=BLOCK, sm_scale=SM_SCALE, causal=False, debug=False,
+                                       score_fn=sfn, mask_fn=mf, block_mask_fn=bf)
+    torch.cuda.synchronize()
+    return o, l, m, dq, dk, dv
+
+
+def _sample_rows(S, n):
+    g = torch.Generator().manual_seed(11)
+    rows = torch.sort(torch.randperm(S, generator=g)[:n]).values
+    rows[0], rows[-1] = 0, S - 1
+    return rows
+
+
+def test_forward_driver_workload(F):
+    """main.py:44-177: bf16, B = 1, H = 1, S = 16384, D = 128, blocks 1024, the place-holder mask (the only live
+    case of the list), sm_scale = 1.0 (main.py:155)."""
+    from flex_attention_tpu_amd import masks
+    S = 16384
+    q, k, v, _ = O.make_inputs(1, 1, 1, S, S, 128, dtype=torch.bfloat16, seed=0)
+    mf, bf = masks.place_holder(BLOCK, BLOCK)
+    rows = _sample_rows(S, 256)
+    ro, rl, rm = O.mha_reference(q, k, v, sm_scale=SM_SCALE, save_residuals=True, q_rows=rows, compute_dtype=torch.float32)
+    o, l, m = F._flex_attention_impl(q.to(DEV), k.to(DEV), v.to(DEV), None, None, True, False, SM_SCALE, 1, BLOCK, BLOCK,
+                                     BLOCK, False, bf, mf, None)
+    dr = rows.to(DEV)
+    assert_close("o", o[:, :, dr], ro, torch.bfloat16)
+    assert_close("lse", (m + l.log())[:, :, dr], rm + rl.log(), torch.bfloat16)
+
+
+@pytest.mark.parametrize("case", ["causal", "sliding_window_1024", "jagged_5_docs", "alibi_0.5", "tanh_30"])
+def test_backward_driver_workloads(F, case):
+    """flex_attention_dq_bwd.py:788-946 and flash_attention_dkv_bwd.py:772-940: bf16, B = 1, H = 8, S = 4096,
+    D = 128, blocks 1024, sm_scale = 1.0; cases causal, sliding window 1024 (one-sided, no causal bound), five
+    documents drawn with seed 42 (the dk/dv driver's), the tile-local position bias of slope 0.5 and softcap 30,
+    the last two without a mask.  All passes on two heads' sampled rows against the oracle."""
+    S, H = 4096, 8
+    (mf, bf), sfn, okw = _driver_cases(S)[case]
+    q, k, v, do = O.make_inputs(1, H, H, S, S, 128, dtype=torch.bfloat16, seed=0)
+    rows = _sample_rows(S, 192)
+    heads = [(0, 0), (0, 7)]
+    ro, rl, rm = O.mha_reference(q, k, v, sm_scale=SM_SCALE, save_residuals=True, q_rows=rows, heads=heads,
+                                 compute_dtype=torch.float32, **okw)
+    do_s = torch.zeros_like(do)   # (dk, dv are linear in dO: rows outside the sample contribute nothing)
+    do_s[:, :, rows] = do[:, :, rows]
+    o, l, m, dq, dk, dv = _run_all(F, q.to(DEV), k.to(DEV), v.to(DEV), do_s.to(DEV), mf, bf, sfn)
+    sdq, sdk, sdv = same_residual_grads(q, k, v, do_s, o, l, m, sm_scale=SM_SCALE, q_rows=rows, heads=heads,
+                                        compute_dtype=torch.float32, **okw)
+    dr = rows.to(DEV)
+    for (b, h) in heads:
+        assert_close(f"o[{h}]", o[b, h, dr], ro[b, h], torch.bfloat16)
+        assert_close(f"lse[{h}]", (m + l.log())[b, h, dr], (rm + rl.log())[b, h], torch.bfloat16)
+        assert_close(f"dq[{h}]", dq[b, h, dr], sdq[b, h], torch.bfloat16, tensor_scale=True)
+        assert_close(f"dk[{h}]", dk[b, h], sdk[b, h], torch.bfloat16, tensor_scale=True)
+        assert_close(f"dv[{h}]", dv[b, h], sdv[b, h], torch.bfloat16)
+
+
+def test_backward_from_the_residuals_of_an_unmasked_forward(F):
+    """The drivers hand (o, l, m) of an unmasked forward to backward kernels that run under the causal mask
+    (flex_attention_dq_bwd.py:920-926, flash_attention_dkv_bwd.py:913-919): P is then no softmax, but the
+    backward kernels are functions of (l, m, delta) as given, and the dense reference gets the same ones."""
+    from flex_attention_tpu_amd import masks
+    S, H = 4096, 8
+    (mf, bf), _, okw = _driver_cases(S)["causal"]
+    q, k, v, do = O.make_inputs(1, H, H, S, S, 128, dtype=torch.bfloat16, seed=0)
+    rows = _sample_rows(S, 192)
+    heads = [(0, 3)]
+    do_s = torch.zeros_like(do)
+    do_s[:, :, rows] = do[:, :, rows]
+    o, l, m, dq, dk, dv = _run_all(F, q.to(DEV), k.to(DEV), v.to(DEV), do_s.to(DEV), mf, bf, None,
+                                   fwd_masks=masks.place_holder(BLOCK, BLOCK))
+    sdq, sdk, sdv = same_residual_grads(q, k, v, do_s, o, l, m, sm_scale=SM_SCALE, q_rows=rows, heads=heads,
+                                        compute_dtype=torch.float32, **okw)
+    dr = rows.to(DEV)
+    assert_close("dq", dq[0, 3, dr], sdq[0, 3], torch.bfloat16, tensor_scale=True)
+    assert_close("dk", dk[0, 3], sdk[0, 3], torch.bfloat16, tensor_scale=True)
+    assert_close("dv", dv[0, 3], sdv[0, 3], torch.bfloat16)
