@@ -2,7 +2,8 @@
 
 The reference has no test suite: each of its drivers builds one workload, runs the kernels and the dense
 reference and prints a relative L2 error (main.py:44-177 forward; flex_attention_dq_bwd.py:788-946 dq;
-flash_attention_dkv_bwd.py:772-940 dk/dv).  These tests run the same workloads through this package's entry
+flash_attention_dkv_bwd.py:772-940 dk/dv; the early float32 drivers reference_bwd_test.py:744-812 and
+bwd_dq.py:385-478, at the end of this file, run at 1/sqrt(D)).  These tests run the same workloads through this package's entry
 points with the drivers' keyword arguments -- sm_scale = 1.0 on unit-variance bf16 inputs of head dimension
 128 (logits of standard deviation 11: softmax rows dominated by one or two keys, a harder regime than the
 1/sqrt(D) of the benchmark configurations), blocks of 1024, batch 1 -- and compare with the oracle on sampled
@@ -150,3 +151,47 @@ def test_backward_from_the_residuals_of_an_unmasked_forward(F):
     assert_close("dq", dq[0, 3, dr], sdq[0, 3], torch.bfloat16, tensor_scale=True)
     assert_close("dk", dk[0, 3], sdk[0, 3], torch.bfloat16, tensor_scale=True)
     assert_close("dv", dv[0, 3], sdv[0, 3], torch.bfloat16)
+
+
+def _fp32_all(F, q, k, v, do, bq, bkm, bk):
+    sc = 1.0 / float(np.sqrt(np.float32(128)))
+    o, l, m = F._flex_attention_impl(q, k, v, None, None, True, False, sc, 1, bq, bkm, bk, False, None, None, None)
+    d = F.compute_delta(o, do)
+    dq = F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=bq, block_k_major=bkm,
+                                 block_k=bk, sm_scale=sc, debug=False)
+    dk, dv = F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=bq, block_q_major=bq,
+                                       block_k_major=bkm, block_k=bk, sm_scale=sc, causal=False, debug=False)
+    torch.cuda.synchronize()
+    return sc, o, l, m, dq, dk, dv
+
+
+def test_fp32_cross_attention_driver_workload(F):
+    """bwd_dq.py:385-478: float32, B = H = 1, 128 queries against 25600 keys, D = 128, sm_scale = 1/sqrt(D), no mask,
+    block_q 128, block_k 256.  Every element against the float64 oracle at 1e-5."""
+    q, k, v, do = O.make_inputs(1, 1, 1, 128, 25600, 128, dtype=torch.float32, seed=0)
+    sc, o, l, m, dq, dk, dv = _fp32_all(F, q.to(DEV), k.to(DEV), v.to(DEV), do.to(DEV), 128, 256, 256)
+    ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, sm_scale=sc)
+    assert_close("o", o, ro, torch.float32)
+    assert_close("lse", m + l.log(), rm + rl.log(), torch.float32)
+    for name, t, r in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+        assert_close(name, t, r, torch.float32, chain=True)
+
+
+def test_fp32_long_sequence_driver_workload(F):
+    """reference_bwd_test.py:744-812: float32, B = H = 1, S = 16384, D = 128, sm_scale = 1/sqrt(D), no mask, block_q
+    128, block_k 128.  Sampled rows against the float64 oracle at 1e-5 (dk, dv with dO zeroed outside the sample)."""
+    S = 16384
+    q, k, v, do = O.make_inputs(1, 1, 1, S, S, 128, dtype=torch.float32, seed=0)
+    rows = _sample_rows(S, 192)
+    do_s = torch.zeros_like(do)
+    do_s[:, :, rows] = do[:, :, rows]
+    sc, o, l, m, dq, dk, dv = _fp32_all(F, q.to(DEV), k.to(DEV), v.to(DEV), do_s.to(DEV), 128, 128, 128)
+    ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, q_rows=rows)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do_s[:, :, rows], rl, rm, sm_scale=sc, q_rows=rows)
+    dr = rows.to(DEV)
+    assert_close("o", o[:, :, dr], ro, torch.float32)
+    assert_close("lse", (m + l.log())[:, :, dr], rm + rl.log(), torch.float32)
+    assert_close("dq", dq[:, :, dr], rdq, torch.float32, chain=True)
+    assert_close("dk", dk, rdk, torch.float32, chain=True)
+    assert_close("dv", dv, rdv, torch.float32, chain=True)
