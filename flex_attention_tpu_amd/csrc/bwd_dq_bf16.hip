@@ -298,12 +298,15 @@ static int launch_dq(const BwdArgs& a, hipStream_t stream) {
 // with e^(2 s / cap) = 2^u; the stream turns it into r = 1 / (2^u + 1) (tanh = 1 - 2 r), the exponent
 // cap' - lse - 2 cap' r (cap' = cap log2 e) and the derivative's r (1 - r); the factor 4 sm_scale that is left
 // goes onto dq in the epilogue.
-// KIND: 0 plain, 1 ALIBI, 2 SOFTCAP.
+// EXACT: plain scores with Q unscaled in its registers; the stream turns the raw product into the exponent with one
+// fma per element (c2 <q, k> - lse).  For scales too large to fold into bf16 Q (folded_scale_ok).
+// KIND: 0 plain, 1 ALIBI, 2 SOFTCAP, 3 EXACT.
 template <int KIND, bool DOCS>
 __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs a) {
   using namespace dq_cfg;
   constexpr bool ALIBI = KIND == 1;
   constexpr bool SOFTCAP = KIND == 2;
+  constexpr bool EXACT = KIND == 3;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   bf16_t* sT = reinterpret_cast<bf16_t*>(smem_raw);  // buffer b: K tile 0, K tile 1, V tile 0, V tile 1
   unsigned* sTbl = reinterpret_cast<unsigned*>(sT + 8 * kTileElems);
@@ -414,9 +417,10 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   const float cap2 = SOFTCAP ? a.score.cap * kLog2e : 0.f;
   const float c2 = SOFTCAP ? 2.0f * kLog2e * a.sm_scale / a.score.cap : a.sm_scale * kLog2e;
   const float out_scale = SOFTCAP ? 4.0f * a.sm_scale : a.sm_scale;
-  auto scaled = [c2](unsigned two) {
-    const float lo = __builtin_bit_cast(float, two << 16) * c2;
-    const float hi = __builtin_bit_cast(float, two & 0xffff0000u) * c2;
+  const float q_mul = EXACT ? 1.0f : c2;   // (EXACT: Q stays as it is; the stream scales the fp32 product)
+  auto scaled = [q_mul](unsigned two) {
+    const float lo = __builtin_bit_cast(float, two << 16) * q_mul;
+    const float hi = __builtin_bit_cast(float, two & 0xffff0000u) * q_mul;
     return __builtin_bit_cast(unsigned, pack_bf16(lo, hi));
   };
   // (`stage`: the wave's 16 KB of a free LDS step buffer)
@@ -641,6 +645,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
       } else if constexpr (SOFTCAP) {
         const float caplse = cap2 - lse2;
         FA_DQ_CALL(FA_DQ_RUN_SOFTCAP, , [lse] "v"(caplse));
+      } else if constexpr (EXACT) {
+        FA_DQ_CALL(FA_DQ_RUN_EXACT, , [lse] "v"(lse2));
       } else {
         FA_DQ_CALL(FA_DQ_RUN, , [lse] "v"(lse2));
       }
@@ -730,17 +736,19 @@ int bwd_dq_bf16_d128(const BwdArgs& a, hipStream_t stream) {
 #else
   // (the generated-stream kernel caches the kv list in LDS)
   // (and has no additive bias)
-  // (and folds its scale into bf16 Q: folded_scale_ok)
+  // (and folds its scale into bf16 Q where that is harmless, folded_scale_ok; plain scores have a variant that does
+  // not fold, the position-bias and softcap streams do not)
   const float fold = a.score.kind == FLEXATTN_SCORE_SOFTCAP ? 2.0f * kLog2e * a.sm_scale / a.score.cap : a.sm_scale * kLog2e;
-  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= dq_cfg::MAX_LIST && a.score.ab == nullptr &&
-                         folded_scale_ok(fold, a.sm_scale, 128);
+  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nk <= dq_cfg::MAX_LIST && a.score.ab == nullptr;
+  const bool fold_ok = folded_scale_ok(fold, a.sm_scale, 128);
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
-      return stream_ok ? launch_dq_plain<0>(a, stream) : launch_dq<FLEXATTN_SCORE_NONE>(a, stream);
+      if (stream_ok) return fold_ok ? launch_dq_plain<0>(a, stream) : launch_dq_plain<3>(a, stream);
+      return launch_dq<FLEXATTN_SCORE_NONE>(a, stream);
     case FLEXATTN_SCORE_ALIBI:
-      return stream_ok ? launch_dq_plain<1>(a, stream) : launch_dq<FLEXATTN_SCORE_ALIBI>(a, stream);
+      return stream_ok && fold_ok ? launch_dq_plain<1>(a, stream) : launch_dq<FLEXATTN_SCORE_ALIBI>(a, stream);
     case FLEXATTN_SCORE_SOFTCAP:
-      return stream_ok ? launch_dq_plain<2>(a, stream) : launch_dq<FLEXATTN_SCORE_SOFTCAP>(a, stream);
+      return stream_ok && fold_ok ? launch_dq_plain<2>(a, stream) : launch_dq<FLEXATTN_SCORE_SOFTCAP>(a, stream);
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_dq<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);
   }
   return set_error(FLEXATTN_EINVAL, "unknown score kind %d", a.score.kind);

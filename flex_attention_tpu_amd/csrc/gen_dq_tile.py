@@ -58,7 +58,7 @@ DROP = ()        # instruction classes left out (--drop, timing studies only)
 TILE = 16384
 # No scalar operands: constants come from a per-wave table in LDS, loop state from VGPR operands
 # (the compiler may print a VGPR for an "s" operand once many uniform values are live).
-TABLE = ["n_tiles", "w4k", "c2", "n_steps",  # (c2: unused; its register holds a tile index in the position-bias variant)
+TABLE = ["n_tiles", "w4k", "c2", "n_steps",  # (c2: softcap and exact-scale variants; its register holds a tile index in the position-bias variant)
          "idx_lo", "idx_hi", "kg_lo", "kg_hi", "vg_lo", "vg_hi", "kban", "kbbn",
          "kgn_lo", "kgn_hi", "vgn_lo", "vgn_hi"]
 SREG = {"n_tiles": "s60", "w4k": "s61", "c2": "s62", "n_steps": "s63", "idx_lo": "s64", "idx_hi": "s65",
@@ -109,7 +109,7 @@ def bias_ops(e, block, tile, odd):
     e.mfma_f32x2(vr(V_NL, 16), "%[aone]", vr(b), vset(V_NL, 16), set(), vset(b))
 
 
-def build(masked, alibi=False, softcap=False):
+def build(masked, alibi=False, softcap=False, exact=False):
     em = Emitter()
     em.wait_old = WAIT_OLD
     pairs = []
@@ -159,7 +159,8 @@ def build(masked, alibi=False, softcap=False):
             cdn = V_ND if ks == 0 else dp
             first = (vr(s, 16), ar(base, 4), ar(A_Q + 4 * ks, 4), vr(cin, 16), vset(s, 16), aset(base, 4), aset(A_Q + 4 * ks, 4),
                      vset(cin, 16))
-            if softcap and ks == 0:   # (the chain's result is the exponent of e^(2 s / cap): nothing to start from)
+            if (softcap or exact) and ks == 0:   # (softcap: the chain's result is the exponent of e^(2 s / cap), nothing to
+                # start from; exact scale: the raw product, scaled and shifted by one fma per element below)
                 first = (vr(s, 16), ar(base, 4), ar(A_Q + 4 * ks, 4), "0", vset(s, 16), aset(base, 4), aset(A_Q + 4 * ks, 4), set())
             return [first,
                     (vr(dp, 16), ar(base + 4, 4), ar(A_DO + 4 * ks, 4), vr(cdn, 16), vset(dp, 16), aset(base + 4, 4),
@@ -187,6 +188,12 @@ def build(masked, alibi=False, softcap=False):
         s, dp = V_S[c & 1], V_DP[c & 1]
         ops = []
         for g in range(4):
+            if exact:
+                # exponent = c2 <q, k> - lse from the raw product: Q went in unscaled, so the logit carries no rounding
+                # of a pre-scaled operand (calls whose scale is too large to fold into bf16 Q, see folded_scale_ok)
+                for u in range(4):
+                    e = 4 * g + u
+                    ops.append(valu(f"v_fma_f32 {vr(s + e)}, {vr(s + e)}, {S_K2}, -%[lse]", vset(s + e), vset(s + e) | {("op", "lse")}))
             for u in range(4):
                 e = 4 * g + u
                 ops.append(valu(f"v_exp_f32_e32 {vr(s + e)}, {vr(s + e)}", vset(s + e), vset(s + e), True))
@@ -280,7 +287,7 @@ def build(masked, alibi=False, softcap=False):
     return em
 
 
-def run_loop(full, masked, alibi=False, softcap=False):
+def run_loop(full, masked, alibi=False, softcap=False, exact=False):
     """One asm statement: a run of consecutive steps [it, it_end) of one work item, at most one of
     them partial.  At entry the step's K / V tiles are resident in LDS buffer %[buf]; each pass
     computes the next step's addresses, streams the step (which copies the next step's tiles into the
@@ -297,7 +304,7 @@ def run_loop(full, masked, alibi=False, softcap=False):
         entry += [f"v_readfirstlane_b32 {S_CUR[0]}, %[ka0]", f"v_readfirstlane_b32 {S_CUR[1]}, %[kb0]"]
         bias_ops(pre, 0, S_CUR[0], 0)   # (used by the first MFMA of the loop, more than 20 instructions on)
         entry += pre.out
-    elif not softcap:   # (softcap: %[lse] is cap' - lse and joins the exponent element by element)
+    elif not softcap and not exact:   # (softcap: %[lse] is cap' - lse and joins the exponent element by element; exact: lse)
         entry += [f"v_sub_f32_e32 {vr(V_NL + e)}, 0, %[lse]" for e in range(16)]
     entry += [f"v_sub_f32_e32 {vr(V_ND + e)}, 0, %[dl]" for e in range(16)]
     top = entry + [".Lfa_dq_loop_%=:"]
@@ -374,6 +381,7 @@ def main():
         macro("FA_DQ_RUN", run_loop(full, masked))
         macro("FA_DQ_RUN_ALIBI", run_loop(build(False, True), build(True, True), True))
         macro("FA_DQ_RUN_SOFTCAP", run_loop(build(False, softcap=True), build(True, softcap=True), softcap=True))
+        macro("FA_DQ_RUN_EXACT", run_loop(build(False, exact=True), build(True, exact=True), exact=True))
         for name, em in (("full", full), ("masked", masked)):
             print(f"{args.out}: {name}: {len(em.out)} instructions, {em.stats}", file=sys.stderr)
         macro("FA_DQ_ZERO_ACC", [f"v_accvgpr_write_b32 a{A_DQ + i}, 0" for i in range(64)])

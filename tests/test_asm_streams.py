@@ -324,6 +324,13 @@ def test_dq_tile_streams_respect_hazards():
         assert n == em.stats["mfma"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
         scratch_ok(em.out, 66, 183, 191)
         check_dataflow(em.out, 1, 4)
+        # exact-scale variant: Q unscaled, one fma per score turns the raw product into the exponent
+        em = g.build(masked, exact=True)
+        n = check_stream(em.out)
+        assert em.stats["mfma"] == 96 and sum("v_fma_f32" in l for l in em.out) == 64
+        assert n == em.stats["mfma"] + em.stats["valu"] + em.stats["lds"] + em.stats["vmem"]
+        scratch_ok(em.out, 66, 183, 191)
+        check_dataflow(em.out, 1, 4)
 
 
 def test_fwd_tile_streams_respect_hazards():
@@ -562,6 +569,7 @@ def _run_loops():
         for alibi, softcap in ((False, False), (True, False), (False, True)):
             yield f"{name} alibi={alibi} softcap={softcap}", g.run_loop(
                 g.build(False, alibi, softcap), g.build(True, alibi, softcap), alibi, softcap)
+    yield "dq exact", gen_dq_tile.run_loop(gen_dq_tile.build(False, exact=True), gen_dq_tile.build(True, exact=True), exact=True)
 
 
 def test_run_loops_leave_no_load_in_flight():
@@ -577,7 +585,7 @@ def test_run_loops_leave_no_load_in_flight():
         assert name.startswith("fwd") or any(l.startswith("global_load_dword") for l in lines), name
         assert check_vmem_queue(lines) > len(lines), name
         n_loops += 1
-    assert n_loops == 11
+    assert n_loops == 12
 
 
 def test_vmem_queue_checker_catches_open_loads():

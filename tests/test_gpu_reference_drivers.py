@@ -12,9 +12,11 @@ element; dq and dk, which reach magnitudes of 25 to 40 here, against the bound o
 (`tensor_scale`).  Inputs come from this build's seeded generator (the reference's JAX PRNG streams are not
 reproducible without JAX).
 
-At this scale the library runs the forward and dq on the kernels that scale the fp32 product (the generated-stream
-kernels fold the scale into their bf16 copy of Q, which costs logits of this size their accuracy: o off by 0.06, dq
-by 2 % in relative L2 when measured), so these tests also pin that choice: they fail on the stream kernels.
+At this scale the library runs the forward and dq on kernels that scale the fp32 product (dq with plain scores: the
+exact-scale variant of its generated stream; the forward, and dq under the position bias and softcap: the kernels
+with a compiled main loop):
+the ordinary streams fold the scale into their bf16 copy of Q, which costs logits of this size their accuracy (o off
+by 0.06, dq by 2 % in relative L2 when measured), so these tests also pin that choice: they fail on those.
 
 Differences from the drivers, on purpose: the backward takes the residuals of the forward under the same mask
 (the drivers feed the residuals of an unmasked forward to masked backward kernels; the one test of that habit
@@ -66,7 +68,7 @@ def _driver_cases(S):
     }
 
 
-def _run_all(F, q, k, v, do, mf, bf, sfn, fwd_masks=None):
+def _run_all(F, q, k, v, do, mf, bf, sfn, fwd_masks=None, BLOCK=BLOCK):
     """Forward, delta, dq and dk/dv with the drivers' keyword arguments.  `fwd_masks`: another mask pair for the
     forward than for the backward."""
     fm, fb = (mf, bf) if fwd_masks is None else fwd_masks
@@ -86,6 +88,29 @@ def _sample_rows(S, n):
     rows = torch.sort(torch.randperm(S, generator=g)[:n]).values
     rows[0], rows[-1] = 0, S - 1
     return rows
+
+
+@pytest.mark.parametrize("case", ["causal", "jagged_5_docs"])
+def test_unit_scale_small_shapes(F, case):
+    """sm_scale = 1.0 at a size where every element is compared: B = 2, H = 2, S = 512 (the exact-scale variant of the
+    dq stream kernel, which serves plain scores at this scale, on single- and multi-step items with partial
+    tiles)."""
+    from flex_attention_tpu_amd import masks
+    S = 512
+    if case == "causal":
+        (mf, bf), okw = masks.make_causal_mask_fns(128, 128), dict(causal=True)
+    else:
+        lens = driver_doc_lengths(S, 5, 42)
+        (mf, bf), okw = masks.make_jagged_mask_fns(128, 128, lens), dict(causal=True, segment_ids=O.doc_ids_from_lengths(lens))
+    q, k, v, do = O.make_inputs(2, 2, 2, S, S, 128, dtype=torch.bfloat16, seed=3)
+    ro, rl, rm = O.mha_reference(q, k, v, sm_scale=SM_SCALE, save_residuals=True, **okw)
+    o, l, m, dq, dk, dv = _run_all(F, q.to(DEV), k.to(DEV), v.to(DEV), do.to(DEV), mf, bf, None, BLOCK=128)
+    sdq, sdk, sdv = same_residual_grads(q, k, v, do, o, l, m, sm_scale=SM_SCALE, **okw)
+    assert_close("o", o, ro, torch.bfloat16)
+    assert_close("lse", m + l.log(), rm + rl.log(), torch.bfloat16)
+    assert_close("dq", dq, sdq, torch.bfloat16, tensor_scale=True)
+    assert_close("dk", dk, sdk, torch.bfloat16, tensor_scale=True)
+    assert_close("dv", dv, sdv, torch.bfloat16)
 
 
 def test_forward_driver_workload(F):
