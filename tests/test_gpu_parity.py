@@ -8,6 +8,13 @@ The forward is compared with the oracle's forward; the backward kernels with the
 from identical residuals (the reference's own method) and, in rel-L2, with the oracle's whole chain.
 Full-size configurations are checked against the oracle on sampled q rows, on whole heads of the
 dense launch and through size-independent invariants.
+
+Cases that combine a score function with sm_scale != 1 (the position-bias and softcap cases here, configurations
+4 and 5) are pinned to this build's definition, logits = score_mod(sm_scale <q, k>), which the oracle restates:
+the reference does not agree with itself there (its forward ignores sm_scale next to a score function,
+flex_attention_kernel.py:249-255, its backward kernels multiply the score function's result by it,
+flex_attention_dq_bwd.py:340-345), and its drivers only ever pass sm_scale = 1 with score functions, where all
+conventions coincide (those workloads: test_gpu_reference_drivers.py).
 """
 import math
 import os
