@@ -2,9 +2,11 @@
 // genuine fp32 products and fp32 accumulation, 64 cycles per 32 x 32 x 2 block), head dim 64 or 128.
 // The small fp32 problems this path serves (configuration 1: 2 MB of operands, 0.27 GFLOP) are bound by
 // how long the longest chain of dependent work is, not by bandwidth: a work-group owns 32 "owner" rows
-// (q rows for forward and dq, kv rows for dk/dv), and its four waves split the streamed side between them
-// (wave w takes entries w, w + 4, ... of the owner tile's list in the block map) and merge their partial
-// results through LDS at the end.  Operands go from global memory (L2-resident at these sizes) straight
+// (q rows for forward and dq, kv rows for dk/dv), and its NW waves split the streamed side between them in
+// units of 32 rows (wave w takes units w, w + NW, ... of the owner tile's list in the block map) and merge
+// their partial results through LDS at the end.  NW = 4 (one wave per SIMD) in general; head dim 64 on a grid
+// that leaves CUs idle takes NW = 8: the two waves of a SIMD hide each other's operand loads, which nothing
+// prefetches (208 registers per lane at head dim 64 allow two waves; head dim 128 needs 304).  Operands go from global memory (L2-resident at these sizes) straight
 // into MFMA operand registers: no LDS staging, no barriers in the main loop.
 //
 // MFMA operand layout (32x32x2 fp32): lane L supplies A[L % 32][L / 32] and B[L / 32][L % 32] (one float
@@ -63,14 +65,14 @@ __device__ __forceinline__ void accumulate_rows(f32x16 (&acc)[D / 32], const flo
 // ------------------------------------------------------------------------------------------
 // forward: lane = q column of S^T = K Q^T; O^T accumulates V^T P^T
 // ------------------------------------------------------------------------------------------
-template <int D, int SCORE>
-__global__ __launch_bounds__(256) void fwd_f32_mfma_kernel(FwdArgs a) {
+template <int D, int SCORE, int NW>
+__global__ __launch_bounds__(64 * NW) void fwd_f32_mfma_kernel(FwdArgs a) {
   using namespace f32m;
   constexpr int ND = D / 32;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   float (*sO)[BO][D + 1] = reinterpret_cast<float (*)[BO][D + 1]>(smem_raw);   // [wave][row][d]
-  float (*sM)[BO] = reinterpret_cast<float (*)[BO]>(smem_raw + sizeof(float) * 4 * BO * (D + 1));
-  float (*sL)[BO] = sM + 4;
+  float (*sM)[BO] = reinterpret_cast<float (*)[BO]>(smem_raw + sizeof(float) * NW * BO * (D + 1));
+  float (*sL)[BO] = sM + NW;
 
   const int nO = a.Sq / BO, nK = a.map.nk;
   const int wg = blockIdx.x;
@@ -102,12 +104,12 @@ __global__ __launch_bounds__(256) void fwd_f32_mfma_kernel(FwdArgs a) {
   const int* tile_idx = a.map.idx + (size_t)qb * nK;
   const uint8_t* tile_state = a.map.state + (size_t)qb * nK;
 
-  for (int t = w; t < n_tiles; t += 4) {
-    const int kb = tile_idx[t];
+  static_assert(BT == 64, "a list entry is two units of 32 rows");
+  for (int u = w; u < 2 * n_tiles; u += NW) {
+    const int kb = tile_idx[u >> 1];
     const bool partial = tile_state[kb] == 1;
-#pragma unroll 1
-    for (int blk = 0; blk < BT / 32; ++blk) {
-      const int j0 = kb * BT + 32 * blk;
+    {
+      const int j0 = kb * BT + 32 * (u & 1);
       const f32x16 s = dot_block<D>(Kg + (size_t)(j0 + l32) * D, qf, half);
       float x[16];
       float m_blk = kNegInf;
@@ -142,7 +144,7 @@ __global__ __launch_bounds__(256) void fwd_f32_mfma_kernel(FwdArgs a) {
     }
   }
 
-  // ---- the four waves' partial results (each relative to its own maximum) into one ----
+  // ---- the waves' partial results (each relative to its own maximum) into one ----
   const float l_wave = half_sum(l_run);
   if (half == 0) {
     sM[w][l32] = m_run;
@@ -153,35 +155,36 @@ __global__ __launch_bounds__(256) void fwd_f32_mfma_kernel(FwdArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) sO[w][l32][32 * db + acc_row(i, half)] = acc[db][i];
   __syncthreads();
-  const int r = tid >> 3, c0 = (tid & 7) * (D / 8);
+  constexpr int TPR = 2 * NW, CPT = D / TPR;   // threads per owner row, columns per thread
+  const int r = tid / TPR, c0 = (tid % TPR) * CPT;
   float m_all = kNegInf;
 #pragma unroll
-  for (int ww = 0; ww < 4; ++ww) m_all = fmaxf(m_all, sM[ww][r]);
+  for (int ww = 0; ww < NW; ++ww) m_all = fmaxf(m_all, sM[ww][r]);
   const float m_safe = (m_all == kNegInf) ? 0.f : m_all;
-  float f[4], l_all = 0.f;
+  float f[NW], l_all = 0.f;
 #pragma unroll
-  for (int ww = 0; ww < 4; ++ww) {
+  for (int ww = 0; ww < NW; ++ww) {
     f[ww] = exp2f(sM[ww][r] - m_safe);   // (0 for a wave that kept nothing)
     l_all += sL[ww][r] * f[ww];
   }
   const float inv = (l_all > 0.f) ? 1.0f / l_all : 0.f;
   float* Og = static_cast<float*>(a.o) + ((size_t)bh * a.Sq + ob * BO + r) * D + c0;
 #pragma unroll
-  for (int c = 0; c < D / 8; ++c) {
+  for (int c = 0; c < CPT; ++c) {
     float o = 0.f;
 #pragma unroll
-    for (int ww = 0; ww < 4; ++ww) o = __builtin_fmaf(sO[ww][r][c0 + c], f[ww], o);
+    for (int ww = 0; ww < NW; ++ww) o = __builtin_fmaf(sO[ww][r][c0 + c], f[ww], o);
     Og[c] = o * inv;
   }
-  if (a.l != nullptr && (tid & 7) == 0) {
+  if (a.l != nullptr && (tid % TPR) == 0) {
     a.l[(size_t)bh * a.Sq + ob * BO + r] = l_all;
     a.m[(size_t)bh * a.Sq + ob * BO + r] = m_all * kLn2;
   }
 }
 
-// Sum of the four waves' accumulators (each [ND][16] in MFMA layout: column = the lane's owner row) through
-// LDS, written out as rows of D floats: thread tid takes row tid / 8, columns (tid % 8) D / 8 ...
-template <int D>
+// Sum of the waves' accumulators (each [ND][16] in MFMA layout: column = the lane's owner row) through
+// LDS, written out as rows of D floats: 2 NW threads per row, D / (2 NW) consecutive columns each.
+template <int D, int NW>
 __device__ __forceinline__ void merge_and_store(const f32x16 (&acc)[D / 32], float (*stage)[f32m::BO][D + 1], float* out_rows,
                                                 float mul, int tid) {
   const int w = tid >> 6, l32 = tid & 31, half = (tid >> 5) & 1;
@@ -190,10 +193,15 @@ __device__ __forceinline__ void merge_and_store(const f32x16 (&acc)[D / 32], flo
 #pragma unroll
     for (int i = 0; i < 16; ++i) stage[w][l32][32 * db + acc_row(i, half)] = acc[db][i];
   __syncthreads();
-  const int r = tid >> 3, c0 = (tid & 7) * (D / 8);
+  constexpr int TPR = 2 * NW, CPT = D / TPR;
+  const int r = tid / TPR, c0 = (tid % TPR) * CPT;
 #pragma unroll
-  for (int c = 0; c < D / 8; ++c)
-    out_rows[(size_t)r * D + c0 + c] = (stage[0][r][c0 + c] + stage[1][r][c0 + c] + stage[2][r][c0 + c] + stage[3][r][c0 + c]) * mul;
+  for (int c = 0; c < CPT; ++c) {
+    float x = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < NW; ++ww) x += stage[ww][r][c0 + c];
+    out_rows[(size_t)r * D + c0 + c] = x * mul;
+  }
 }
 
 __device__ __forceinline__ float lse2_from(float l, float m) {
@@ -203,8 +211,8 @@ __device__ __forceinline__ float lse2_from(float l, float m) {
 // ------------------------------------------------------------------------------------------
 // dq: lane = q column; S^T = K Q^T, dP^T = V dO^T, dq^T += K^T dS^T
 // ------------------------------------------------------------------------------------------
-template <int D, int SCORE>
-__global__ __launch_bounds__(256) void bwd_dq_f32_mfma_kernel(BwdArgs a) {
+template <int D, int SCORE, int NW>
+__global__ __launch_bounds__(64 * NW) void bwd_dq_f32_mfma_kernel(BwdArgs a) {
   using namespace f32m;
   constexpr int ND = D / 32;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
@@ -241,12 +249,11 @@ __global__ __launch_bounds__(256) void bwd_dq_f32_mfma_kernel(BwdArgs a) {
   const int n_tiles = a.map.cnt[qb];
   const int* tile_idx = a.map.idx + (size_t)qb * nK;
   const uint8_t* tile_state = a.map.state + (size_t)qb * nK;
-  for (int t = w; t < n_tiles; t += 4) {
-    const int kb = tile_idx[t];
+  for (int u = w; u < 2 * n_tiles; u += NW) {
+    const int kb = tile_idx[u >> 1];
     const bool partial = tile_state[kb] == 1;
-#pragma unroll 1
-    for (int blk = 0; blk < BT / 32; ++blk) {
-      const int j0 = kb * BT + 32 * blk;
+    {
+      const int j0 = kb * BT + 32 * (u & 1);
       const f32x16 s = dot_block<D>(Kg + (size_t)(j0 + l32) * D, qf, half);
       const f32x16 dp = dot_block<D>(Vg + (size_t)(j0 + l32) * D, dof, half);
       float ds[16];
@@ -267,20 +274,19 @@ __global__ __launch_bounds__(256) void bwd_dq_f32_mfma_kernel(BwdArgs a) {
       accumulate_rows<D>(acc, Kg + (size_t)j0 * D, ds, l32, half);
     }
   }
-  merge_and_store<D>(acc, sA, static_cast<float*>(a.dq) + ((size_t)bh * a.Sq + ob * BO) * D, 1.0f, tid);
+  merge_and_store<D, NW>(acc, sA, static_cast<float*>(a.dq) + ((size_t)bh * a.Sq + ob * BO) * D, 1.0f, tid);
 }
 
 // ------------------------------------------------------------------------------------------
 // dk/dv: lane = kv column; S = Q K^T, dP = dO V^T, dv^T += dO^T P, dk^T += Q^T dS, over the q tiles of the
 // kv block's list and the q heads of its kv head
 // ------------------------------------------------------------------------------------------
-template <int D, int SCORE>
-__global__ __launch_bounds__(256) void bwd_dkv_f32_mfma_kernel(BwdArgs a) {
+template <int D, int SCORE, int NW>
+__global__ __launch_bounds__(64 * NW) void bwd_dkv_f32_mfma_kernel(BwdArgs a) {
   using namespace f32m;
   constexpr int ND = D / 32;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  float (*sA)[BO][D + 1] = reinterpret_cast<float (*)[BO][D + 1]>(smem_raw);
-  float (*sB)[BO][D + 1] = sA + 4;
+  float (*sA)[BO][D + 1] = reinterpret_cast<float (*)[BO][D + 1]>(smem_raw);   // (dk, then dv)
 
   const int nO = a.Sk / BO, nQ = a.map.nq;
   const int wg = blockIdx.x;
@@ -305,7 +311,8 @@ __global__ __launch_bounds__(256) void bwd_dkv_f32_mfma_kernel(BwdArgs a) {
   const int n_tiles = a.map.cnt[kb];
   const int* tile_idx = a.map.idx + (size_t)kb * nQ;
   const uint8_t* state = a.map.state;
-  for (int it = w; it < group * n_tiles; it += 4) {
+  for (int u = w; u < 2 * group * n_tiles; u += NW) {
+    const int it = u >> 1;
     const int g = it / n_tiles, qb = tile_idx[it - g * n_tiles];
     const int h = hk * group + g;
     const size_t head_row = (size_t)(b * a.Hq + h) * a.Sq;
@@ -314,9 +321,8 @@ __global__ __launch_bounds__(256) void bwd_dkv_f32_mfma_kernel(BwdArgs a) {
     ScoreMod<SCORE> sm;
     sm.init(a.score, a.sm_scale, h, b);
     const bool partial = state[(size_t)qb * a.map.nk + kb] == 1;
-#pragma unroll 1
-    for (int blk = 0; blk < BT / 32; ++blk) {
-      const int i0 = qb * BT + 32 * blk;
+    {
+      const int i0 = qb * BT + 32 * (u & 1);
       const f32x16 s = dot_block<D>(Qg + (size_t)(i0 + l32) * D, kf, half);
       const f32x16 dp = dot_block<D>(dOg + (size_t)(i0 + l32) * D, vf, half);
       float pv[16], ds[16];
@@ -337,62 +343,71 @@ __global__ __launch_bounds__(256) void bwd_dkv_f32_mfma_kernel(BwdArgs a) {
       accumulate_rows<D>(dk_acc, Qg + (size_t)i0 * D, ds, l32, half);
     }
   }
-  merge_and_store<D>(dk_acc, sA, static_cast<float*>(a.dk) + ((size_t)bhk * a.Sk + ob * BO) * D, 1.0f, tid);
-  merge_and_store<D>(dv_acc, sB, static_cast<float*>(a.dv) + ((size_t)bhk * a.Sk + ob * BO) * D, 1.0f, tid);
+  merge_and_store<D, NW>(dk_acc, sA, static_cast<float*>(a.dk) + ((size_t)bhk * a.Sk + ob * BO) * D, 1.0f, tid);
+  __syncthreads();  // (the stage is read by other threads than wrote it: all of dk is out before dv goes in)
+  merge_and_store<D, NW>(dv_acc, sA, static_cast<float*>(a.dv) + ((size_t)bhk * a.Sk + ob * BO) * D, 1.0f, tid);
 }
 
 template <typename Kern, typename Args>
-static int launch_mfma(Kern kern, int grid, int lds, const Args& a, hipStream_t stream, const char* what) {
+static int launch_mfma(Kern kern, int grid, int waves, int lds, const Args& a, hipStream_t stream, const char* what) {
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(%s): %s", what, hipGetErrorString(e));
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, stream, a);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * waves), lds, stream, a);
   return check_launch(what);
 }
 
-#define FA_F32M_DISPATCH(KERNEL, GRID, LDS, ARGS, WHAT)                                                                       \
-  switch ((ARGS).score.kind) {                                                                                           \
-    case FLEXATTN_SCORE_NONE: return launch_mfma(KERNEL<DD, FLEXATTN_SCORE_NONE>, GRID, LDS, ARGS, stream, WHAT);             \
-    case FLEXATTN_SCORE_ALIBI: return launch_mfma(KERNEL<DD, FLEXATTN_SCORE_ALIBI>, GRID, LDS, ARGS, stream, WHAT);           \
-    case FLEXATTN_SCORE_SOFTCAP: return launch_mfma(KERNEL<DD, FLEXATTN_SCORE_SOFTCAP>, GRID, LDS, ARGS, stream, WHAT);       \
-    case FLEXATTN_SCORE_ALIBI_TILE: return launch_mfma(KERNEL<DD, FLEXATTN_SCORE_ALIBI_TILE>, GRID, LDS, ARGS, stream, WHAT); \
-    case FLEXATTN_SCORE_CUSTOM: return launch_mfma(KERNEL<DD, FLEXATTN_SCORE_CUSTOM>, GRID, LDS, ARGS, stream, WHAT);         \
-  }                                                                                                                      \
+#define FA_F32M_DISPATCH(KERNEL, GRID, LDS, ARGS, WHAT)                                                                            \
+  switch ((ARGS).score.kind) {                                                                                                \
+    case FLEXATTN_SCORE_NONE: return launch_mfma(KERNEL<DD, FLEXATTN_SCORE_NONE, NWW>, GRID, NWW, LDS, ARGS, stream, WHAT);             \
+    case FLEXATTN_SCORE_ALIBI: return launch_mfma(KERNEL<DD, FLEXATTN_SCORE_ALIBI, NWW>, GRID, NWW, LDS, ARGS, stream, WHAT);           \
+    case FLEXATTN_SCORE_SOFTCAP: return launch_mfma(KERNEL<DD, FLEXATTN_SCORE_SOFTCAP, NWW>, GRID, NWW, LDS, ARGS, stream, WHAT);       \
+    case FLEXATTN_SCORE_ALIBI_TILE: return launch_mfma(KERNEL<DD, FLEXATTN_SCORE_ALIBI_TILE, NWW>, GRID, NWW, LDS, ARGS, stream, WHAT); \
+    case FLEXATTN_SCORE_CUSTOM: return launch_mfma(KERNEL<DD, FLEXATTN_SCORE_CUSTOM, NWW>, GRID, NWW, LDS, ARGS, stream, WHAT);         \
+  }                                                                                                                           \
   return set_error(FLEXATTN_EINVAL, "unknown score kind %d", (ARGS).score.kind);
 
-template <int DD>
+// Eight waves per work-group where two fit a SIMD (head dim 64) and the grid is small enough to leave CUs idle
+// (at most two work-groups per CU): the extra waves then cost nothing and hide the operand loads.
+static bool wide_groups(int D, int grid) { return D == 64 && grid <= 512; }
+
+template <int DD, int NWW>
 static int fwd_f32_mfma_d(const FwdArgs& a, hipStream_t stream) {
   const int grid = a.B * a.Hq * (a.Sq / f32m::BO);
-  const int lds = 4 * (4 * f32m::BO * (DD + 1) + 2 * 4 * f32m::BO);
+  const int lds = 4 * (NWW * f32m::BO * (DD + 1) + 2 * NWW * f32m::BO);
   FA_F32M_DISPATCH(fwd_f32_mfma_kernel, grid, lds, a, "flexattn_fwd f32")
 }
 
-template <int DD>
+template <int DD, int NWW>
 static int bwd_dq_f32_mfma_d(const BwdArgs& a, hipStream_t stream) {
   const int grid = a.B * a.Hq * (a.Sq / f32m::BO);
-  const int lds = 4 * 4 * f32m::BO * (DD + 1);
+  const int lds = 4 * NWW * f32m::BO * (DD + 1);
   FA_F32M_DISPATCH(bwd_dq_f32_mfma_kernel, grid, lds, a, "flexattn_bwd_dq f32")
 }
-template <int DD>
+template <int DD, int NWW>
 static int bwd_dkv_f32_mfma_d(const BwdArgs& a, hipStream_t stream) {
   const int grid = a.B * a.Hkv * (a.Sk / f32m::BO);
-  const int lds = 2 * 4 * 4 * f32m::BO * (DD + 1);
+  const int lds = 4 * NWW * f32m::BO * (DD + 1);
   FA_F32M_DISPATCH(bwd_dkv_f32_mfma_kernel, grid, lds, a, "flexattn_bwd_dkv f32")
 }
 
 int bwd_dq_f32_mfma(const BwdArgs& a, int D, hipStream_t stream) {
-  if (D == 64) return bwd_dq_f32_mfma_d<64>(a, stream);
-  if (D == 128) return bwd_dq_f32_mfma_d<128>(a, stream);
+  if (D == 64)
+    return wide_groups(D, a.B * a.Hq * (a.Sq / f32m::BO)) ? bwd_dq_f32_mfma_d<64, 8>(a, stream) : bwd_dq_f32_mfma_d<64, 4>(a, stream);
+  if (D == 128) return bwd_dq_f32_mfma_d<128, 4>(a, stream);
   return set_error(FLEXATTN_ENOTSUP, "fp32 dq: head dim %d not in {64, 128}", D);
 }
 int bwd_dkv_f32_mfma(const BwdArgs& a, int D, hipStream_t stream) {
-  if (D == 64) return bwd_dkv_f32_mfma_d<64>(a, stream);
-  if (D == 128) return bwd_dkv_f32_mfma_d<128>(a, stream);
+  if (D == 64)
+    return wide_groups(D, a.B * a.Hkv * (a.Sk / f32m::BO)) ? bwd_dkv_f32_mfma_d<64, 8>(a, stream)
+                                                          : bwd_dkv_f32_mfma_d<64, 4>(a, stream);
+  if (D == 128) return bwd_dkv_f32_mfma_d<128, 4>(a, stream);
   return set_error(FLEXATTN_ENOTSUP, "fp32 dk/dv: head dim %d not in {64, 128}", D);
 }
 
 int fwd_f32_mfma(const FwdArgs& a, int D, hipStream_t stream) {
-  if (D == 64) return fwd_f32_mfma_d<64>(a, stream);
-  if (D == 128) return fwd_f32_mfma_d<128>(a, stream);
+  if (D == 64)
+    return wide_groups(D, a.B * a.Hq * (a.Sq / f32m::BO)) ? fwd_f32_mfma_d<64, 8>(a, stream) : fwd_f32_mfma_d<64, 4>(a, stream);
+  if (D == 128) return fwd_f32_mfma_d<128, 4>(a, stream);
   return set_error(FLEXATTN_ENOTSUP, "fp32 forward: head dim %d not in {64, 128}", D);
 }
 
