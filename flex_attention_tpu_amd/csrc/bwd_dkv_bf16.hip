@@ -562,6 +562,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     const int row_p = tid_p & (BQ - 1);
     const float x = rowa[r0 + row_p], y = rowb[r0 + row_p];
     if (lse_wave) {  // (the streams want -lse: it is the accumulator input of the S chain)
+      // (one fused multiply-add, as the streams' turn-around rounds the row values of every later step: an item's
+      // results then do not depend on whether its first step was set up here or by the last step of the item before it)
       float neg_lse = (x > 0.f) ? -__builtin_fmaf(y, kLog2e, log2f(x)) : -__builtin_huge_valf();
       if (ALIBI) neg_lse = __builtin_fmaf((float)((int)r0 + row_p - kc), na2, neg_lse);
       if (SOFTCAP) neg_lse += cap2;

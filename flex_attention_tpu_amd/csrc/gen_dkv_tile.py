@@ -347,10 +347,12 @@ def build(masked, alibi=False, softcap=False, export=False):
         # l = 0; waves 2, 3: -delta (%[lsew] is non-zero resp. zero).  One LDS store into the next buffer.
         ra_, rb_, rt_, inf_ = V_ROW, V_ROW + 1, V_ROW + 2, V_ROW + 3
         e.raw(f"s_waitcnt vmcnt({state['direct']})")
+        # (-lse by one fused multiply-add, m (-log2 e) - log2 l: the same rounding as the kernel's own set-up of an
+        # item's first step, so that a step's row values do not depend on who prepared them)
         e.valu(f"v_log_f32_e32 {vr(rt_)}, {vr(ra_)}", vset(rt_), vset(ra_), True)
-        e.valu(f"v_mul_f32_e32 {vr(rb_)}, 0xbfb8aa3b, {vr(rb_)}", vset(rb_), vset(rb_))
+        e.raw(f"s_mov_b32 {S_T[1]}, 0xbfb8aa3b")
         e.valu(f"v_mov_b32_e32 {vr(inf_)}, 0xff800000", vset(inf_), set())
-        e.valu(f"v_sub_f32_e32 {vr(rt_)}, {vr(rb_)}, {vr(rt_)}", vset(rt_), vset(rt_) | vset(rb_))
+        e.valu(f"v_fma_f32 {vr(rt_)}, {vr(rb_)}, {S_T[1]}, -{vr(rt_)}", vset(rt_), vset(rt_) | vset(rb_))
         e.valu(f"v_cmp_lt_f32_e32 vcc, 0, {vr(ra_)}", set(), vset(ra_))
         e.valu(f"v_cndmask_b32_e32 {vr(rt_)}, {vr(inf_)}, {vr(rt_)}, vcc", vset(rt_), vset(rt_) | vset(inf_))
         if softcap:

@@ -1,0 +1,115 @@
+"""Size-independent properties of the kernels at the full sizes of the benchmark configurations, where the oracle
+only reaches sampled rows and single heads: every output element of the full launch takes part, bit for bit.
+
+* Determinism: the same call twice gives the same bits (every output tile has one writer and a fixed order of
+  accumulation; nothing depends on which work-group runs an item, or when).
+* Equivariance: permuting the batch entries (and, where the score function does not depend on the head, the kv
+  groups of heads) permutes the outputs and changes no bit.  The persistent work-groups then run the same items in
+  another order, next to other items and with other prefetched neighbours: state that leaks from one item into
+  the next, or a schedule that visits an item twice or not at all, shows here on every element.
+* Homogeneity: scaling dO (or v) by two doubles dq, dk, dv (or o) exactly: delta, dP and dS double without rounding
+  (powers of two), so the bf16 results are the doubled bf16 results.
+* No gradient without dO: dO = 0 gives dq = dk = dv = 0.
+"""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def F():
+    import flex_attention_tpu_amd as F
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return F
+
+
+def _calls(F, cfg):
+    from flex_attention_tpu_amd import configs
+    import warnings
+    warnings.filterwarnings("ignore", message="score_fn with sm_scale")
+    mf, bf = configs.mask_fns(cfg)
+    sfn = configs.score_fn(cfg)
+    sc = cfg.sm_scale
+
+    def fwd(q, k, v):
+        return F._flex_attention_impl(q, k, v, None, None, True, False, sc, 1, 128, 128, 128, False, bf, mf, sfn)
+
+    def bwd(q, k, v, o, l, m, do):
+        return F.flex_attention_bwd(q, k, v, None, None, l, m, o, do, block_q=128, block_k=128, sm_scale=sc, score_fn=sfn,
+                                    mask_fn=mf, block_mask_fn=bf)
+
+    def bwd_exchanging(q, k, v, o, l, m, do):
+        """The backward with dS handed from the dk/dv pass to the dq pass (None where nothing is exchanged)."""
+        d = F.compute_delta(o, do)
+        dk, dv, ds = F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=128, block_q_major=128,
+                                               block_k_major=128, block_k=128, sm_scale=sc, causal=False, debug=False,
+                                               score_fn=sfn, mask_fn=mf, block_mask_fn=bf, return_ds=True)
+        if ds is None:
+            return None
+        dq = F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=128, block_k_major=128,
+                                     block_k=128, sm_scale=sc, debug=False, score_fn=sfn, mask_fn=mf, block_mask_fn=bf, ds=ds)
+        return dq, dk, dv
+    return fwd, bwd, bwd_exchanging
+
+
+def _same(name, a, b):
+    assert torch.equal(a, b), f"{name}: {int((a != b).sum())} of {a.numel()} elements differ"
+
+
+@pytest.mark.parametrize("name", ["cfg1", "cfg2", "cfg4", "cfg5"])
+def test_full_size_properties(F, name):
+    from flex_attention_tpu_amd import configs
+    cfg = configs.CONFIGS[name]
+    fwd, bwd, bwd_x = _calls(F, cfg)
+    q, k, v, do = [x.to(DEV) for x in configs.make_inputs(cfg)]
+    group = cfg.Hq // cfg.Hkv
+
+    o, l, m = fwd(q, k, v)
+    grads = bwd(q, k, v, o, l, m, do)
+
+    # determinism
+    o2, l2, m2 = fwd(q, k, v)
+    for n, a, b in zip(("o", "l", "m"), (o, l, m), (o2, l2, m2)):
+        _same(f"{n} of a second run", a, b)
+    for n, a, b in zip(("dq", "dk", "dv"), grads, bwd(q, k, v, o, l, m, do)):
+        _same(f"{n} of a second run", a, b)
+
+    # equivariance under a permutation of the batch entries and, unless the score depends on the head, of the kv groups
+    g = torch.Generator().manual_seed(5)
+    pb = torch.randperm(cfg.B, generator=g).to(DEV)
+    pk = (torch.randperm(cfg.Hkv, generator=g) if cfg.score != "alibi" else torch.arange(cfg.Hkv)).to(DEV)
+    pq = (pk[:, None] * group + torch.arange(group, device=DEV)[None, :]).reshape(-1)   # q heads follow their kv head
+
+    def perm_q(x):
+        return x[pb][:, pq].contiguous()
+
+    def perm_k(x):
+        return x[pb][:, pk].contiguous()
+    op, lp, mp = fwd(perm_q(q), perm_k(k), perm_k(v))
+    _same("o under a permutation of batch entries and kv groups", op, perm_q(o))
+    _same("l under a permutation", lp, perm_q(l))
+    _same("m under a permutation", mp, perm_q(m))
+    dqp, dkp, dvp = bwd(perm_q(q), perm_k(k), perm_k(v), op, lp, mp, perm_q(do))
+    _same("dq under a permutation", dqp, perm_q(grads[0]))
+    _same("dk under a permutation", dkp, perm_k(grads[1]))
+    _same("dv under a permutation", dvp, perm_k(grads[2]))
+
+    # homogeneity: powers of two go through every product and sum without rounding
+    o_v2 = fwd(q, k, v * 2)[0]
+    _same("o of 2 v", o_v2, o * 2)
+    for n, a, b in zip(("dq", "dk", "dv"), bwd(q, k, v, o, l, m, do * 2), grads):
+        _same(f"{n} of 2 dO", a, b * 2)
+    for n, a in zip(("dq", "dk", "dv"), bwd(q, k, v, o, l, m, torch.zeros_like(do))):
+        assert not a.any(), f"{n} of dO = 0 is not zero"
+
+    # the backward that hands dS over: the same dk, dv; dq deterministic, equivariant and homogeneous as well
+    gx = bwd_x(q, k, v, o, l, m, do)
+    if gx is not None:
+        _same("dk with the dS hand-over", gx[1], grads[1])
+        _same("dv with the dS hand-over", gx[2], grads[2])
+        _same("dq from dS, second run", bwd_x(q, k, v, o, l, m, do)[0], gx[0])
+        _same("dq from dS under a permutation", bwd_x(perm_q(q), perm_k(k), perm_k(v), op, lp, mp, perm_q(do))[0], perm_q(gx[0]))
+        _same("dq from dS of 2 dO", bwd_x(q, k, v, o, l, m, do * 2)[0], gx[0] * 2)
