@@ -10,6 +10,9 @@ only reaches sampled rows and single heads: every output element of the full lau
 * Homogeneity: scaling dO (or v) by two doubles dq, dk, dv (or o) exactly: delta, dP and dS double without rounding
   (powers of two), so the bf16 results are the doubled bf16 results.
 * No gradient without dO: dO = 0 gives dq = dk = dv = 0.
+* Locality: a (batch entry, kv group) launched alone gives its bits of the full launch (one item per work-group
+  against the persistent schedule); under a causal mask the first half of the tokens alone gives the first half of
+  o, l, m and dq.
 """
 import pytest
 import torch
@@ -113,3 +116,61 @@ def test_full_size_properties(F, name):
         _same("dq from dS, second run", bwd_x(q, k, v, o, l, m, do)[0], gx[0])
         _same("dq from dS under a permutation", bwd_x(perm_q(q), perm_k(k), perm_k(v), op, lp, mp, perm_q(do))[0], perm_q(gx[0]))
         _same("dq from dS of 2 dO", bwd_x(q, k, v, o, l, m, do * 2)[0], gx[0] * 2)
+
+
+@pytest.mark.parametrize("name", ["cfg1", "cfg2", "cfg4", "cfg5"])
+def test_a_part_launched_alone_equals_its_part_of_the_full_launch(F, name):
+    """One (batch entry, kv group) launched on its own gives the bits it has in the full launch: the small launch
+    runs one work item per work-group, handed out by the hardware, the full one the persistent schedule with
+    several items per work-group and the next item's first step copied during the last step of the one before.
+    (The position bias takes its slopes from the head's index and the number of heads of the call: that
+    configuration launches a whole batch entry instead.)"""
+    from flex_attention_tpu_amd import configs
+    cfg = configs.CONFIGS[name]
+    fwd, bwd, bwd_x = _calls(F, cfg)
+    q, k, v, do = [x.to(DEV) for x in configs.make_inputs(cfg)]
+    group = cfg.Hq // cfg.Hkv
+    b = cfg.B - 1
+    kv_heads = slice(0, cfg.Hkv) if cfg.score == "alibi" else slice(cfg.Hkv - 1, cfg.Hkv)
+    q_heads = slice(kv_heads.start * group, kv_heads.stop * group)
+
+    def part_q(x):
+        return x[b:b + 1, q_heads].contiguous()
+
+    def part_k(x):
+        return x[b:b + 1, kv_heads].contiguous()
+    o, l, m = fwd(q, k, v)
+    grads = bwd(q, k, v, o, l, m, do)
+    os_, ls_, ms_ = fwd(part_q(q), part_k(k), part_k(v))
+    _same("o", os_, part_q(o))
+    _same("l", ls_, part_q(l))
+    _same("m", ms_, part_q(m))
+    dqs, dks, dvs = bwd(part_q(q), part_k(k), part_k(v), os_, ls_, ms_, part_q(do))
+    _same("dq", dqs, part_q(grads[0]))
+    _same("dk", dks, part_k(grads[1]))
+    _same("dv", dvs, part_k(grads[2]))
+    gx = bwd_x(q, k, v, o, l, m, do)
+    if gx is not None:
+        _same("dq from dS", bwd_x(part_q(q), part_k(k), part_k(v), os_, ls_, ms_, part_q(do))[0], part_q(gx[0]))
+
+
+@pytest.mark.parametrize("name", ["cfg2", "cfg4"])
+def test_causal_prefix(F, name):
+    """Under a causal mask the first half of the rows does not see the second: the forward and dq of the first
+    S / 2 tokens alone give the bits of the first S / 2 rows of the full launch (another number of tiles, other lists,
+    another schedule; the same arithmetic per row)."""
+    from flex_attention_tpu_amd import configs
+    cfg = configs.CONFIGS[name]
+    fwd, bwd, _ = _calls(F, cfg)
+    q, k, v, do = [x.to(DEV) for x in configs.make_inputs(cfg)]
+    n = cfg.S // 2
+    o, l, m = fwd(q, k, v)
+    dq = bwd(q, k, v, o, l, m, do)[0]
+
+    def head(x):
+        return x[:, :, :n].contiguous()
+    oh, lh, mh = fwd(head(q), head(k), head(v))
+    _same("o of the first half", oh, head(o))
+    _same("l of the first half", lh, head(l))
+    _same("m of the first half", mh, head(m))
+    _same("dq of the first half", bwd(head(q), head(k), head(v), oh, lh, mh, head(do))[0], head(dq))
