@@ -174,3 +174,74 @@ def test_causal_prefix(F, name):
     _same("l of the first half", lh, head(l))
     _same("m of the first half", mh, head(m))
     _same("dq of the first half", bwd(head(q), head(k), head(v), oh, lh, mh, head(do))[0], head(dq))
+
+
+def _random_case(rng, it):
+    """A random shape, mask, score function, dtype and kernel family (seeded): (tag, tensors, call arguments)."""
+    import math
+    from flex_attention_tpu_amd import masks, scores
+    B, Hkv, g = rng.choice([2, 3, 4, 8]), rng.choice([2, 4, 8, 16]), rng.choice([1, 1, 2, 4])
+    S = 128 * rng.choice([2, 4, 7, 8, 13, 16, 24, 32])
+    mk = rng.choice(["none", "causal", "window", "causal_window", "documents"])
+    sk = rng.choice(["none", "none", "alibi", "softcap"])
+    dt = rng.choice([torch.bfloat16, torch.bfloat16, torch.bfloat16, torch.float32])
+    compiled_loop = rng.random() < 0.2
+    if dt == torch.float32 and S > 2048:
+        S = 1024
+    if mk == "none":
+        mf, bf = None, None
+    elif mk == "causal":
+        mf, bf = masks.make_causal_mask_fns(128, 128)
+    elif mk == "window":
+        mf, bf = masks.make_sliding_window_mask_fns(128, 128, rng.randint(100, 900))
+    elif mk == "causal_window":
+        mf, bf = masks.make_causal_sliding_window_mask_fns(128, 128, rng.randint(1, 700))
+    else:
+        lens, left = [], S
+        while left > 0:
+            lens.append(min(left, rng.randint(1, 700)))
+            left -= lens[-1]
+        mf, bf = masks.make_jagged_mask_fns(128, 128, lens)
+    sfn = {"none": None, "alibi": scores.make_alibi_global_score_fn(Hkv * g),
+           "softcap": scores.make_softcap_score_fn(rng.choice([2.0, 30.0]))}[sk]
+    sc = rng.choice([1.0, 1.0, 3.0]) / math.sqrt(128)
+    gen = torch.Generator().manual_seed(7000 + it)
+    q, k, v, do = [torch.randn(B, h, S, 128, generator=gen).to(dt).to(DEV) for h in (Hkv * g, Hkv, Hkv, Hkv * g)]
+    tag = f"B={B} Hq={Hkv * g} Hkv={Hkv} S={S} mask={mk} score={sk} scale={sc:.3f} {str(dt)[6:]} compiled_loop={compiled_loop}"
+    return tag, (q, k, v, do), (sc, mf, bf, sfn, compiled_loop), mk
+
+
+def _all_passes(F, q, k, v, do, sc, mf, bf, sfn, compiled_loop):
+    o, l, m = F._flex_attention_impl(q, k, v, None, None, True, False, sc, 1, 128, 128, 128, False, bf, mf, sfn,
+                                     compiled_loop=compiled_loop)
+    d = F.compute_delta(o, do)
+    kw = dict(sm_scale=sc, debug=False, score_fn=sfn, mask_fn=mf, block_mask_fn=bf, compiled_loop=compiled_loop)
+    dq = F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=128, block_k_major=128, block_k=128, **kw)
+    dk, dv, ds = F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_b=1, block_q=128, block_q_major=128,
+                                           block_k_major=128, block_k=128, causal=False, return_ds=True, **kw)
+    dqx = dq if ds is None else F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, block_b=1, block_q=128,
+                                                        block_k_major=128, block_k=128, ds=ds, **kw)
+    return o, l, m, dq, dk, dv, dqx
+
+
+def test_random_shapes_locality(F):
+    """The locality properties above on 24 random shapes (2 to 32 tiles, 2 to 64 heads, grouped kv heads), masks,
+    score functions, scales, both dtypes and both kernel families: one batch entry alone against its part of the
+    full launch, every output and the dq from handed-over dS, and under causal masks a prefix of the tokens against
+    the prefix of o, l, m, dq.  Bit for bit."""
+    import random
+    import warnings
+    warnings.filterwarnings("ignore", message="score_fn with sm_scale")
+    rng = random.Random(20)
+    for it in range(24):
+        tag, (q, k, v, do), args, mk = _random_case(rng, it)
+        full = _all_passes(F, q, k, v, do, *args)
+        b = rng.randrange(q.shape[0])
+        part = _all_passes(F, *[x[b:b + 1].contiguous() for x in (q, k, v, do)], *args)
+        for name, a, r in zip(("o", "l", "m", "dq", "dk", "dv", "dq from dS"), part, full):
+            _same(f"{tag}: {name} of batch entry {b} alone", a, r[b:b + 1])
+        if mk in ("causal", "causal_window") and q.shape[2] >= 512:
+            n = 128 * rng.randrange(1, q.shape[2] // 128)
+            pre = _all_passes(F, *[x[:, :, :n].contiguous() for x in (q, k, v, do)], *args)
+            for name, a, r in zip(("o", "l", "m", "dq"), pre[:4], full[:4]):
+                _same(f"{tag}: {name} of the first {n} tokens alone", a, r[:, :, :n])
