@@ -13,6 +13,7 @@ only reaches sampled rows and single heads: every output element of the full lau
 * Locality: a (batch entry, kv group) launched alone gives its bits of the full launch (one item per work-group
   against the persistent schedule); under a causal mask the first half of the tokens alone gives the first half of
   o, l, m and dq.
+* Grouped kv heads give, per query head, the bits of the same call with the kv heads repeated.
 """
 import pytest
 import torch
@@ -245,3 +246,33 @@ def test_random_shapes_locality(F):
             pre = _all_passes(F, *[x[:, :, :n].contiguous() for x in (q, k, v, do)], *args)
             for name, a, r in zip(("o", "l", "m", "dq"), pre[:4], full[:4]):
                 _same(f"{tag}: {name} of the first {n} tokens alone", a, r[:, :, :n])
+
+
+def test_grouped_kv_heads_equal_repeated_kv_heads(F):
+    """Grouped kv heads against the same call with every kv head repeated for its query heads (on 12 seeded random
+    shapes, masks and score functions): o, l, m and dq bit for bit (a query head's rows do not care how the kv heads
+    are stored; the schedules differ); dk, dv, which the grouped kernels sum over the group in fp32 inside one work
+    item, against the sum of the repeated heads' bf16 results in relative L2."""
+    import random
+    import warnings
+    warnings.filterwarnings("ignore", message="score_fn with sm_scale")
+    rng = random.Random(21)
+    done = 0
+    it = 0
+    while done < 12:
+        it += 1
+        tag, (q, k, v, do), args, _ = _random_case(rng, 100 + it)
+        g = q.shape[1] // k.shape[1]
+        if g == 1:
+            continue
+        done += 1
+        a = _all_passes(F, q, k, v, do, *args)
+        ke, ve = k.repeat_interleave(g, 1).contiguous(), v.repeat_interleave(g, 1).contiguous()
+        e = _all_passes(F, q, ke, ve, do, *args)
+        for name, x, y in zip(("o", "l", "m", "dq"), a[:4], e[:4]):
+            _same(f"{tag}: {name} with repeated kv heads", y, x)
+        B, Hkv, S, D = k.shape
+        for name, x, y in zip(("dk", "dv"), a[4:6], e[4:6]):
+            ys = y.float().view(B, Hkv, g, S, D).sum(2)
+            rel = float((x.float() - ys).norm() / (ys.norm() + 1e-9))
+            assert rel <= 6e-3, f"{tag}: {name} of the group against the sum over repeated heads: rel-L2 {rel:.2e}"
