@@ -713,8 +713,8 @@ def test_schedule_edges_against_the_oracle(F, case):
 
 
 def test_integration_doc_binding_runs_verbatim(F):
-    """The ctypes binding printed in INTEGRATION.md, executed as it stands (only the library path is
-    filled in), against the oracle: the struct layouts of the document and of the header agree."""
+    """The ctypes binding printed in the integration notes at the repository root, executed as it stands (only the
+    library path is filled in), against the oracle: the struct layouts of the document and of the header agree."""
     import re
     from flex_attention_tpu_amd import _lib
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
