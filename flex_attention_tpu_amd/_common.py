@@ -9,7 +9,7 @@ import numpy as np
 import torch
 
 from . import _lib
-from .block_mask import LRU, BlockMap, build_block_map, mask_spec_c, spec_of
+from .block_mask import LRU, BlockMap, build_block_map, mask_spec_c, raw_stream, spec_of
 from .masks import DocIds, MaskSpec
 from .scores import ScoreSpec
 
@@ -294,7 +294,7 @@ def library_for(score_fn, spec: MaskSpec):
 
 
 def stream_of(t: torch.Tensor) -> int:
-    return torch.cuda.current_stream(t.device).cuda_stream
+    return raw_stream(t.device)
 
 
 class _NoSwitch:

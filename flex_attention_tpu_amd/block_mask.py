@@ -17,6 +17,17 @@ import torch
 from . import _lib
 from .masks import DocIds, MaskSpec
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def raw_stream(device) -> int:
+    """Handle of the current stream of `device` (the lookup that builds no Stream object where torch has one: the
+    launch path of a small call is a few tens of microseconds in all)."""
+    if _raw_stream is not None:
+        idx = device.index
+        return _raw_stream(torch.cuda.current_device() if idx is None else idx)
+    return torch.cuda.current_stream(device).cuda_stream
+
 
 class LRU:
     """Small least-recently-used cache: holds at most ``maxsize`` entries (each may pin device
@@ -74,8 +85,10 @@ class BlockMap:
         """Makes the current stream wait for the builder kernel if that ran on another stream, and tells the
         caching allocator that the map is in use on this stream too (a map evicted from the cache must not be
         handed out again while a kernel on this stream still walks it)."""
+        if self.ready is None or raw_stream(device) == self.built_on:
+            return
         cur = torch.cuda.current_stream(device)
-        if self.ready is not None and cur.cuda_stream != self.built_on:
+        if cur.cuda_stream != self.built_on:
             cur.wait_event(self.ready)
             for t in self._tensors():
                 t.record_stream(cur)
