@@ -226,7 +226,15 @@ def check(rc: int, lib=None) -> None:
     raise RuntimeError(f"flexattn error {rc}: {msg}")
 
 
+_tile_shapes = {}
+
+
 def tile_shape(pass_id: int, dtype: int, D: int):
-    bq, bk = C.c_int32(0), C.c_int32(0)
-    check(load().flexattn_tile_shape(pass_id, dtype, D, C.byref(bq), C.byref(bk)))
-    return bq.value, bk.value
+    """(block_q, block_k) of the kernels of a pass (a property of the library: asked once per combination)."""
+    key = (pass_id, dtype, D)
+    hit = _tile_shapes.get(key)
+    if hit is None:
+        bq, bk = C.c_int32(0), C.c_int32(0)
+        check(load().flexattn_tile_shape(pass_id, dtype, D, C.byref(bq), C.byref(bk)))
+        hit = _tile_shapes[key] = (bq.value, bk.value)
+    return hit
