@@ -100,7 +100,11 @@ __global__ __launch_bounds__(256, dqds_cfg::OCC) void bwd_dq_from_ds_kernel(BwdA
   for (int i = 0; i < 4; ++i) {
     const int piece = 4 * (w & 1) + i;
     const int row = piece * 4 + (lane >> 4);
-    goff[i] = w < 2 ? (unsigned)piece * 1024u + lane16 : (unsigned)(row * kTileD + (((lane & 15) ^ swz(row)) << 3)) * 2u;
+    // (dS pieces of the odd halves u = piece & 1 go into LDS with their 128-byte halves of every 256 bytes swapped:
+    // the two 16-lane groups of a half-wave read pieces u = 0 and u = 1 at the same offset, which would be the same
+    // banks; the swap puts them on the two halves of the banks)
+    goff[i] = w < 2 ? (unsigned)piece * 1024u + (lane16 ^ (128u * (unsigned)(piece & 1)))
+                    : (unsigned)(row * kTileD + (((lane & 15) ^ swz(row)) << 3)) * 2u;
   }
 
   // stage s = part s % PARTS of the list's kv tile s / PARTS: that part's dS as it lies in the block and its 32 K
@@ -143,8 +147,11 @@ __global__ __launch_bounds__(256, dqds_cfg::OCC) void bwd_dq_from_ds_kernel(BwdA
   // (a wave computes 64 q rows x 64 head columns: q blocks 2 (w >> 1) + qi, column blocks 2 (w & 1) + di; with
   // 32 x 128 per wave every MFMA would take 2.5 operand reads from LDS instead of 2, and the LDS reads bound the loop)
   const int wq = w >> 1, wd = w & 1;
-  const unsigned ds_off = 1024u * (unsigned)(4 * wq + ((lane & 31) >> 4))
-                          + 32u * (unsigned)(8 * hh + (l16 >> 2)) + 16u * (unsigned)(l16 & 1) + 8u * (unsigned)((l16 & 3) >> 1);
+  const unsigned ds_u = (unsigned)((lane & 31) >> 4);
+  const unsigned ds_in = 32u * (unsigned)(8 * hh + (l16 >> 2)) + 16u * (unsigned)(l16 & 1) + 8u * (unsigned)((l16 & 3) >> 1);
+  // (the lane's two reads per fragment, 128 bytes apart; swapped in the pieces of the odd halves, see goff)
+  const unsigned ds_off = 1024u * (unsigned)(4 * wq) + 1024u * ds_u + (ds_in ^ (128u * ds_u));
+  const unsigned ds_off2 = 1024u * (unsigned)(4 * wq) + 1024u * ds_u + ((ds_in + 128u) ^ (128u * ds_u));
   // K^T fragment: rows 16 ks + 8 hh + (l16 >> 2) (+ 4), columns 32 db + 16 ((lane & 31) >> 4) + 4 (l16 & 3) .. + 4
   const int k_row = 8 * hh + (l16 >> 2);
   const int k_chunk = 2 * ((lane & 31) >> 4) + ((l16 & 3) >> 1);
@@ -191,7 +198,7 @@ __global__ __launch_bounds__(256, dqds_cfg::OCC) void bwd_dq_from_ds_kernel(BwdA
       for (int qi = 0; qi < 2; ++qi) {
         const char* dsp = st + 8192 * (ks >> 1) + 512 * (ks & 1) + 2048 * qi + ds_off;
         const s16x4 b0 = lds_read_tr16(reinterpret_cast<const bf16_t*>(dsp));
-        const s16x4 b1 = lds_read_tr16(reinterpret_cast<const bf16_t*>(dsp + 128));
+        const s16x4 b1 = lds_read_tr16(reinterpret_cast<const bf16_t*>(dsp - ds_off + ds_off2));
         bfrag[qi] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7));
       }
 #pragma unroll

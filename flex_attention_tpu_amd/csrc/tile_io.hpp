@@ -1,10 +1,14 @@
 // LDS tile layout and asynchronous global -> LDS tile loads shared by the bf16 kernels.
 //
 // A tile is 64 rows x 128 bf16 = 64 rows x 16 chunks of 16 bytes, 16 KB, stored unpadded.  Chunk c
-// of row r sits at chunk position c ^ swz(r).  swz takes 16 distinct values over any 16
-// consecutive rows, so a b128 read of one chunk column over 16 rows is bank-conflict free, and
-// over 4 consecutive rows it moves a pair of adjacent chunks to 4 distinct pairs, so the
-// transposing 8-byte reads (4 rows x 32 bytes per 16 lanes) are conflict free as well.
+// of row r sits at chunk position c ^ swz(r).  swz permutes the bits of r & 15, so it takes 16 distinct values
+// over any 16 consecutive rows and a b128 read of one chunk column over 16 rows (16 lanes, 256 bytes, one LDS
+// cycle) is bank-conflict free.  The transposing 8-byte reads take, per half-wave of 32 lanes, 4 consecutive rows
+// x two adjacent pairs of chunks (2 x 32 bytes per row): the rows' swizzles differ in bits 2-3 only, so a pair
+// of chunks moves by a multiple of two pairs and the eight 32-byte pieces fall on the eight distinct pairs of
+// a row, 256 bytes over all 64 banks.  (With the row's low bits in bits 1-2 of the swizzle instead, the two
+// pairs of a half-wave fell on the same four positions: every transposing read took two LDS cycles, the 25-32 %
+// bank-conflict cycles the counters showed.)
 #pragma once
 #include "fa_common.hpp"
 
@@ -14,7 +18,9 @@ constexpr int kTileRows = 64;
 constexpr int kTileD = 128;
 constexpr int kTileElems = kTileRows * kTileD;  // 8192 bf16 = 16 KB
 
-__device__ __forceinline__ constexpr int swz(int row) { return ((row & 7) << 1) | ((row >> 3) & 1); }
+__device__ __forceinline__ constexpr int swz(int row) {
+  return ((row & 3) << 2) | (((row >> 2) & 1) << 1) | ((row >> 3) & 1);
+}
 
 // Element offset of (row, 16-byte chunk) inside a tile.
 __device__ __forceinline__ constexpr int tile_off(int row, int chunk) {
