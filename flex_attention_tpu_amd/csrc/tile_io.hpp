@@ -18,12 +18,12 @@ constexpr int kTileRows = 64;
 constexpr int kTileD = 128;
 constexpr int kTileElems = kTileRows * kTileD;  // 8192 bf16 = 16 KB
 
-__device__ __forceinline__ constexpr int swz(int row) {
+__host__ __device__ __forceinline__ constexpr int swz(int row) {
   return ((row & 3) << 2) | (((row >> 2) & 1) << 1) | ((row >> 3) & 1);
 }
 
 // Element offset of (row, 16-byte chunk) inside a tile.
-__device__ __forceinline__ constexpr int tile_off(int row, int chunk) {
+__host__ __device__ __forceinline__ constexpr int tile_off(int row, int chunk) {
   return row * kTileD + ((chunk ^ swz(row)) << 3);
 }
 
