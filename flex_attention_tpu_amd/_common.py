@@ -219,16 +219,18 @@ def padded_len(n: int) -> int:
 
 
 def kernel_head_dim(D: int, dtype) -> int:
-    """Head dimension the kernels run a call of head dimension D at: bf16 128, fp32 64 or 128.  Smaller ones
-    are zero-padded (dot products and the output columns that are kept do not change); the reference itself
-    refuses head dimensions that are not multiples of 128 (flex_attention_kernel.py:302-306)."""
+    """Head dimension the kernels run a call of head dimension D at: bf16 128 or 256, fp32 64 or 128.  Others
+    are zero-padded to the next of these (dot products and the output columns that are kept do not change); the
+    reference itself refuses head dimensions that are not multiples of 128 (flex_attention_kernel.py:302-306)."""
     if D <= 0:
         raise ValueError(f"head_dim must be positive, got {D}")
-    if D > 128:
-        raise NotImplementedError(f"head_dim {D} is not supported (at most 128)")
-    if dtype == torch.float32 and D <= 64:
-        return 64
-    return 128
+    if dtype == torch.float32:
+        if D > 128:
+            raise NotImplementedError(f"float32 head_dim {D} is not supported (at most 128)")
+        return 64 if D <= 64 else 128
+    if D > 256:
+        raise NotImplementedError(f"head_dim {D} is not supported (at most 256)")
+    return 128 if D <= 128 else 256
 
 
 def pad_seq(t: torch.Tensor, n: int, dim: int = 2) -> torch.Tensor:

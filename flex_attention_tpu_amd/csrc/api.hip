@@ -110,8 +110,8 @@ static int tile_shape(int pass, int dtype, int D, int* bq, int* bk) {
     return FLEXATTN_OK;
   }
   if (dtype == FLEXATTN_BF16) {
-    if (D != 128) return set_error(FLEXATTN_ENOTSUP, "bf16: head dim %d not supported (128 only)", D);
-    switch (pass) {
+    if (D != 128 && D != 256) return set_error(FLEXATTN_ENOTSUP, "bf16: head dim %d not in {128, 256}", D);
+    switch (pass) {   // (head dim 256 runs on the tiles of head dim 128)
       case FLEXATTN_PASS_FWD: fwd_bf16_d128_tile(bq, bk); return FLEXATTN_OK;
       case FLEXATTN_PASS_DQ: bwd_dq_bf16_d128_tile(bq, bk); return FLEXATTN_OK;
       case FLEXATTN_PASS_DKV: bwd_dkv_bf16_d128_tile(bq, bk); return FLEXATTN_OK;
@@ -277,7 +277,7 @@ static int fwd_with_map(const flexattn_fwd_params* p, const flexattn_block_map& 
   a.score = to_args(p->score, p->ab, p->Sk);
   a.mask = to_args(p->mask);
   a.map = row_view(map);
-  if (p->dtype == FLEXATTN_BF16) return fwd_bf16_d128(a, s);
+  if (p->dtype == FLEXATTN_BF16) return p->D == 256 ? fwd_bf16_d256(a, s) : fwd_bf16_d128(a, s);
   return (a.flags & FLEXATTN_FLAG_COMPILED_LOOP) ? fwd_f32(a, p->D, s) : fwd_f32_mfma(a, p->D, s);
 }
 
@@ -415,13 +415,13 @@ static int launch_dq(const flexattn_bwd_params* p, BwdArgs a, hipStream_t s) {
   if (p->ds != nullptr) return bwd_dq_from_ds(a, (p->score.kind == FLEXATTN_SCORE_SOFTCAP ? 4.f : 1.f) * p->sm_scale, s);
   if (p->dtype == FLEXATTN_BF16) {
     if (a.dab != nullptr) a.flags |= FLEXATTN_FLAG_COMPILED_LOOP;  // (the generated streams store no bias gradient)
-    return bwd_dq_bf16_d128(a, s);
+    return p->D == 256 ? bwd_dq_bf16_d256(a, s) : bwd_dq_bf16_d128(a, s);
   }
   return (a.flags & FLEXATTN_FLAG_COMPILED_LOOP) ? bwd_dq_f32(a, p->D, s) : bwd_dq_f32_mfma(a, p->D, s);
 }
 
 static int launch_dkv(const flexattn_bwd_params* p, const BwdArgs& a, hipStream_t s) {
-  if (p->dtype == FLEXATTN_BF16) return bwd_dkv_bf16_d128(a, s);
+  if (p->dtype == FLEXATTN_BF16) return p->D == 256 ? bwd_dkv_bf16_d256(a, s) : bwd_dkv_bf16_d128(a, s);
   return (a.flags & FLEXATTN_FLAG_COMPILED_LOOP) ? bwd_dkv_f32(a, p->D, s) : bwd_dkv_f32_mfma(a, p->D, s);
 }
 

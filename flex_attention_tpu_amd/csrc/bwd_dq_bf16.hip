@@ -39,7 +39,7 @@ namespace dq_cfg {
 constexpr int BM = 128;
 constexpr int BN = 64;
 constexpr int D = 128;
-constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2
+constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2, per 128 columns of the head dimension
 // plain-score kernel: steps of two kv tiles, (K, K, V, V) x 2 buffers, per-wave tables, cached kv list + states
 constexpr int MAX_LIST = 4096;       // kv tiles of a row whose list and states the kernel caches in LDS (262144 tokens)
 constexpr int PREFETCH_LIST = 2048;  // of which an item's prefetch carries this many in registers; the rest is read when the item starts
@@ -60,12 +60,17 @@ struct DqPinned {
       "+{a[96:99]}"(st.d[0]), "+{a[100:103]}"(st.d[1]), "+{a[104:107]}"(st.d[2]), "+{a[108:111]}"(st.d[3]),   \
       "+{a[112:115]}"(st.d[4]), "+{a[116:119]}"(st.d[5]), "+{a[120:123]}"(st.d[6]), "+{a[124:127]}"(st.d[7])
 
-template <int SCORE>
-__global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
+// Head dimension 128 NP: a row of K or V is NP panels of 128 columns, each panel of a 64-row tile one LDS tile
+// (tile_io.hpp) at [buffer][panel]; the contractions of S and dP run over the panels, dq^T has four accumulators
+// per panel.
+template <int SCORE, int NP>
+__global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void bwd_dq_bf16_kernel(BwdArgs a) {
   using namespace dq_cfg;
+  constexpr int D = 128 * NP;
+  constexpr int kPanel = kTileElems * 2;   // bytes
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   bf16_t* sK = reinterpret_cast<bf16_t*>(smem_raw);
-  bf16_t* sV = sK + 2 * kTileElems;
+  bf16_t* sV = sK + 2 * NP * kTileElems;
 
   const int nQ = a.Sq / BM;
   const int nK = a.map.nk;
@@ -97,9 +102,9 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
   ScoreMod<SCORE> sm;
   sm.init(a.score, a.sm_scale, h, b);
 
-  bf16x8 qreg[8], doreg[8];
+  bf16x8 qreg[8 * NP], doreg[8 * NP];
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) {
+  for (int ks = 0; ks < 8 * NP; ++ks) {
     qreg[ks] = *reinterpret_cast<const bf16x8*>(Qg + (size_t)q_local * D + ks * 16 + hh * 8);
     doreg[ks] = *reinterpret_cast<const bf16x8*>(dOg + (size_t)q_local * D + ks * 16 + hh * 8);
   }
@@ -114,9 +119,9 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
   if (a.mask.flags & FLEXATTN_MASK_DOC) doc_i = a.mask.doc_q[q_idx];
   float* dab_row = a.dab != nullptr ? a.dab + row * (size_t)a.Sk : nullptr;  // this lane's row of the bias gradient
 
-  f32x16 dq_acc[4];
+  f32x16 dq_acc[4 * NP];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 4 * NP; ++i)
 #pragma unroll
     for (int e = 0; e < 16; ++e) dq_acc[i][e] = 0.f;
 
@@ -128,12 +133,15 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
   if (n_tiles > 2) kb_n2 = tile_idx[2];
   if (n_tiles > 0) st_cur = tile_state[kb_cur];
   if (n_tiles > 1) st_nxt = tile_state[kb_nxt];
-  TileLoader<4> loader;
+  TileLoader<4, D> loader;
   loader.init(w, lane);
   if (n_tiles > 0) {
     const int kb0 = __builtin_amdgcn_readfirstlane(kb_cur);
-    loader.load(Kg + (size_t)kb0 * BN * D, sK);
-    loader.load(Vg + (size_t)kb0 * BN * D, sV);
+#pragma unroll
+    for (int pn = 0; pn < NP; ++pn) {
+      loader.load(Kg + (size_t)kb0 * BN * D + 128 * pn, sK + pn * kTileElems);
+      loader.load(Vg + (size_t)kb0 * BN * D + 128 * pn, sV + pn * kTileElems);
+    }
   }
   wait_vmem_all();
   __syncthreads();
@@ -160,12 +168,15 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
     const int st_n2 = (t + 2 < n_tiles) ? tile_state[kb_n2] : 0;
     if (t + 1 < n_tiles) {
       const int kbn = __builtin_amdgcn_readfirstlane(kb_nxt);
-      loader.load(Kg + (size_t)kbn * BN * D, sK + (buf ^ 1) * kTileElems);
-      loader.load(Vg + (size_t)kbn * BN * D, sV + (buf ^ 1) * kTileElems);
+#pragma unroll
+      for (int pn = 0; pn < NP; ++pn) {
+        loader.load(Kg + (size_t)kbn * BN * D + 128 * pn, sK + ((buf ^ 1) * NP + pn) * kTileElems);
+        loader.load(Vg + (size_t)kbn * BN * D + 128 * pn, sV + ((buf ^ 1) * NP + pn) * kTileElems);
+      }
     }
     const int kv0 = kb * BN;
-    const char* kt = reinterpret_cast<const char*>(sK + buf * kTileElems);
-    const char* vt = reinterpret_cast<const char*>(sV + buf * kTileElems);
+    const char* kt = reinterpret_cast<const char*>(sK + buf * NP * kTileElems);
+    const char* vt = reinterpret_cast<const char*>(sV + buf * NP * kTileElems);
 
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
@@ -176,28 +187,30 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
         s_acc[e] = 0.f;
         dp_acc[e] = 0.f;
       }
-      {
+#pragma unroll
+      for (int pn = 0; pn < NP; ++pn) {
         bf16x8 kf[8];
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) kf[ks] = *reinterpret_cast<const bf16x8*>(kt + r_off[ks] + c * 32 * kTileD * 2);
+        for (int ks = 0; ks < 8; ++ks) kf[ks] = *reinterpret_cast<const bf16x8*>(kt + pn * kPanel + r_off[ks] + c * 32 * kTileD * 2);
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) s_acc = mfma32(kf[ks], qreg[ks], s_acc);
+        for (int ks = 0; ks < 8; ++ks) s_acc = mfma32(kf[ks], qreg[8 * pn + ks], s_acc);
       }
-      {
+#pragma unroll
+      for (int pn = 0; pn < NP; ++pn) {
         bf16x8 vf[8];
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) vf[ks] = *reinterpret_cast<const bf16x8*>(vt + r_off[ks] + c * 32 * kTileD * 2);
+        for (int ks = 0; ks < 8; ++ks) vf[ks] = *reinterpret_cast<const bf16x8*>(vt + pn * kPanel + r_off[ks] + c * 32 * kTileD * 2);
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) dp_acc = mfma32(vf[ks], doreg[ks], dp_acc);
+        for (int ks = 0; ks < 8; ++ks) dp_acc = mfma32(vf[ks], doreg[8 * pn + ks], dp_acc);
       }
       // K^T fragments for the dq product
-      s16x4 klo[2][4], khi[2][4];
+      s16x4 klo[2][4 * NP], khi[2][4 * NP];
       auto read_kt = [&](int u) {
 #pragma unroll
-        for (int db = 0; db < 4; ++db) {
-          const int off = (32 * c + 16 * u) * kTileD * 2;
-          klo[u][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(kt + t_off[db][0] + off));
-          khi[u][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(kt + t_off[db][1] + off));
+        for (int db = 0; db < 4 * NP; ++db) {
+          const int off = (32 * c + 16 * u) * kTileD * 2 + (db >> 2) * kPanel;
+          klo[u][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(kt + t_off[db & 3][0] + off));
+          khi[u][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(kt + t_off[db & 3][1] + off));
         }
       };
 
@@ -249,7 +262,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int db = 0; db < 4; ++db) dq_acc[db] = mfma32(join_tr(klo[u][db], khi[u][db]), ds[u], dq_acc[db]);
+        for (int db = 0; db < 4 * NP; ++db) dq_acc[db] = mfma32(join_tr(klo[u][db], khi[u][db]), ds[u], dq_acc[db]);
     }
 
     kb_cur = kb_nxt; kb_nxt = kb_n2; kb_n2 = kb_n3;
@@ -259,7 +272,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
   }
 
 #pragma unroll
-  for (int db = 0; db < 4; ++db) {
+  for (int db = 0; db < 4 * NP; ++db) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       bf16x2 lo = pack_bf16(dq_acc[db][4 * g], dq_acc[db][4 * g + 1]);
@@ -270,15 +283,15 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_bf16_d128_kernel(BwdArgs a) {
   }
 }
 
-template <int SCORE>
+template <int SCORE, int NP = 1>
 static int launch_dq(const BwdArgs& a, hipStream_t stream) {
   using namespace dq_cfg;
-  auto kern = bwd_dq_bf16_d128_kernel<SCORE>;
+  auto kern = bwd_dq_bf16_kernel<SCORE, NP>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, NP * LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(dq): %s", hipGetErrorString(attr));
   const int n_wg = a.B * a.Hq * (a.Sq / BM);
-  hipLaunchKernelGGL(kern, dim3(n_wg), dim3(256), LDS_BYTES, stream, a);
+  hipLaunchKernelGGL(kern, dim3(n_wg), dim3(256), NP * LDS_BYTES, stream, a);
   return check_launch("flexattn_bwd_dq bf16");
 }
 
@@ -753,6 +766,21 @@ int bwd_dq_bf16_d128(const BwdArgs& a, hipStream_t stream) {
   }
   return set_error(FLEXATTN_EINVAL, "unknown score kind %d", a.score.kind);
 #endif
+}
+
+// Head dim 256: the kernels with a compiled main loop (two 128-column panels per row), every score kind.
+int bwd_dq_bf16_d256(const BwdArgs& a, hipStream_t stream) {
+  switch (a.score.kind) {
+    case FLEXATTN_SCORE_NONE: return launch_dq<FLEXATTN_SCORE_NONE, 2>(a, stream);
+#ifdef FLEXATTN_CUSTOM_ONLY
+    case FLEXATTN_SCORE_CUSTOM: return launch_dq<FLEXATTN_SCORE_CUSTOM, 2>(a, stream);
+#else
+    case FLEXATTN_SCORE_ALIBI: return launch_dq<FLEXATTN_SCORE_ALIBI, 2>(a, stream);
+    case FLEXATTN_SCORE_SOFTCAP: return launch_dq<FLEXATTN_SCORE_SOFTCAP, 2>(a, stream);
+    case FLEXATTN_SCORE_ALIBI_TILE: return launch_dq<FLEXATTN_SCORE_ALIBI_TILE, 2>(a, stream);
+#endif
+  }
+  return set_error(FLEXATTN_ENOTSUP, "score kind %d is not in this library", a.score.kind);
 }
 
 void bwd_dq_bf16_d128_tile(int* bq, int* bk) {

@@ -52,6 +52,7 @@ static int launch_delta(const void* o, const void* dout, float* delta, int64_t r
 
 int bwd_delta(const void* o, const void* dout, float* delta, int64_t rows, int D, int dtype, hipStream_t stream) {
   if (dtype == FLEXATTN_BF16 && D == 128) return launch_delta<bf16_t, 128>(o, dout, delta, rows, stream);
+  if (dtype == FLEXATTN_BF16 && D == 256) return launch_delta<bf16_t, 256>(o, dout, delta, rows, stream);
   if (dtype == FLEXATTN_BF16 && D == 64) return launch_delta<bf16_t, 64>(o, dout, delta, rows, stream);
   if (dtype == FLEXATTN_F32 && D == 128) return launch_delta<float, 128>(o, dout, delta, rows, stream);
   if (dtype == FLEXATTN_F32 && D == 64) return launch_delta<float, 64>(o, dout, delta, rows, stream);

@@ -1,4 +1,4 @@
-// Flex-attention forward, bf16, head dim 128, gfx950.
+// Flex-attention forward, bf16, head dim 128 (generated streams and compiled loop) and 256 (compiled loop), gfx950.
 //
 // One work-group = 4 waves = one 128-row Q tile of one (batch, head); each wave owns 32 q rows.
 // The kernel works on S^T = K Q^T so that one lane holds one q row's scores: softmax statistics
@@ -40,7 +40,7 @@ namespace fwd_cfg {
 constexpr int BM = 128;  // q rows per work-group
 constexpr int BN = 64;   // kv rows per step
 constexpr int D = 128;
-constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2
+constexpr int LDS_BYTES = 4 * kTileElems * 2;  // K x2, V x2, per 128 columns of the head dimension
 // plain-score kernel: 256 q rows per work item, steps of two kv tiles: (K, K, V, V) x 2 buffers, per-wave
 // tables, wave counters, merged kv list, the two state rows
 constexpr int MAX_LIST = 4096;       // kv tiles of a row that the merged list and the state rows in LDS hold (262144 tokens)
@@ -63,12 +63,15 @@ struct FwdPinned {
       "+{a[160:163]}"(st.q[8]), "+{a[164:167]}"(st.q[9]), "+{a[168:171]}"(st.q[10]), "+{a[172:175]}"(st.q[11]), \
       "+{a[176:179]}"(st.q[12]), "+{a[180:183]}"(st.q[13]), "+{a[184:187]}"(st.q[14]), "+{a[188:191]}"(st.q[15])
 
-template <int SCORE>
-__global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
+// Head dimension 128 NP: a row of K or V is NP panels of 128 columns, each panel of a 64-row tile one LDS tile
+// (tile_io.hpp) at [buffer][panel]; the contraction of S runs over the panels, O^T has four accumulators per panel.
+template <int SCORE, int NP>
+__global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void fwd_bf16_kernel(FwdArgs a) {
   using namespace fwd_cfg;
+  constexpr int D = 128 * NP;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   bf16_t* sK = reinterpret_cast<bf16_t*>(smem_raw);
-  bf16_t* sV = sK + 2 * kTileElems;
+  bf16_t* sV = sK + 2 * NP * kTileElems;
 
   const int nQ = a.Sq / BM;
   const int nK = a.map.nk;
@@ -98,9 +101,9 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
   sm.init(a.score, a.sm_scale, h, b);
 
   // Q^T as B operand: lane holds q row l32, 8 consecutive d per k-step.
-  bf16x8 qreg[8];
+  bf16x8 qreg[8 * NP];
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks)
+  for (int ks = 0; ks < 8 * NP; ++ks)
     qreg[ks] = *reinterpret_cast<const bf16x8*>(Qg + (size_t)q_local * D + ks * 16 + hh * 8);
 
   const int n_tiles = a.map.cnt[qb];
@@ -110,9 +113,9 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
   int doc_i = 0;
   if (a.mask.flags & FLEXATTN_MASK_DOC) doc_i = a.mask.doc_q[q_idx];
 
-  f32x16 o_acc[4];
+  f32x16 o_acc[4 * NP];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 4 * NP; ++i)
 #pragma unroll
     for (int e = 0; e < 16; ++e) o_acc[i][e] = 0.f;
   float m_run = kNegInf;  // running max: raw dot-product units (plain score) or log2-domain logits
@@ -126,12 +129,15 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
   if (n_tiles > 2) kb_n2 = tile_idx[2];
   if (n_tiles > 0) st_cur = tile_state[kb_cur];
   if (n_tiles > 1) st_nxt = tile_state[kb_nxt];
-  TileLoader<4> loader;
+  TileLoader<4, D> loader;
   loader.init(__builtin_amdgcn_readfirstlane(w), lane);
   if (n_tiles > 0) {
     const int kb0 = __builtin_amdgcn_readfirstlane(kb_cur);
-    loader.load(Kg + (size_t)kb0 * BN * D, sK);
-    loader.load(Vg + (size_t)kb0 * BN * D, sV);
+#pragma unroll
+    for (int pn = 0; pn < NP; ++pn) {
+      loader.load(Kg + (size_t)kb0 * BN * D + 128 * pn, sK + pn * kTileElems);
+      loader.load(Vg + (size_t)kb0 * BN * D + 128 * pn, sV + pn * kTileElems);
+    }
   }
   wait_vmem_all();
   __syncthreads();
@@ -174,20 +180,23 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
     // pipe and the matrix pipe overlap inside the wave; sched_barrier fences the stages.  The
     // first half of V^T is fetched before the softmax, whose VALU work hides that latency.
     f32x16 s_acc[2];
-    const char* kt = reinterpret_cast<const char*>(sK + buf * kTileElems);
-    const char* vt = reinterpret_cast<const char*>(sV + buf * kTileElems);
-    bf16x8 kf[4][4];             // [2c + ks/4][ks%4]
-    s16x4 vlo[4][4], vhi[4][4];  // [tt][db]
+    const char* kt = reinterpret_cast<const char*>(sK + buf * NP * kTileElems);
+    const char* vt = reinterpret_cast<const char*>(sV + buf * NP * kTileElems);
+    constexpr int NG = 4 * NP;        // stages of four MFMAs of S: g = (2 NP) c + 2 panel + half of the panel's k-steps
+    constexpr int kPanel = kTileElems * 2;   // bytes
+    bf16x8 kf[NG][4];
+    s16x4 vlo[4][4 * NP], vhi[4][4 * NP];  // [tt][db]
     auto read_k = [&](int g) {
+      const int c = g / (2 * NP), pn = (g % (2 * NP)) >> 1;
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        kf[g][i] = *reinterpret_cast<const bf16x8*>(kt + k_off[4 * (g & 1) + i] + (g >> 1) * 32 * kTileD * 2);
+        kf[g][i] = *reinterpret_cast<const bf16x8*>(kt + pn * kPanel + k_off[4 * (g & 1) + i] + c * 32 * kTileD * 2);
     };
     auto read_v = [&](int tt) {
 #pragma unroll
-      for (int db = 0; db < 4; ++db) {
-        vlo[tt][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(vt + v_off[db][0] + tt * 16 * kTileD * 2));
-        vhi[tt][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(vt + v_off[db][1] + tt * 16 * kTileD * 2));
+      for (int db = 0; db < 4 * NP; ++db) {
+        vlo[tt][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(vt + (db >> 2) * kPanel + v_off[db & 3][0] + tt * 16 * kTileD * 2));
+        vhi[tt][db] = lds_read_tr16(reinterpret_cast<const bf16_t*>(vt + (db >> 2) * kPanel + v_off[db & 3][1] + tt * 16 * kTileD * 2));
       }
     };
 #pragma unroll
@@ -197,23 +206,24 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
     read_k(0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      if (g < 3) {
+    for (int g = 0; g < NG; ++g) {
+      if (g < NG - 1) {
         read_k(g + 1);
       } else {
         read_v(0);
       }
+      const int c = g / (2 * NP), pn = (g % (2 * NP)) >> 1;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) s_acc[g >> 1] = mfma32(kf[g][i], qreg[4 * (g & 1) + i], s_acc[g >> 1]);
-      if (g < 3) {
+      for (int i = 0; i < 4; ++i) s_acc[c] = mfma32(kf[g][i], qreg[8 * pn + 4 * (g & 1) + i], s_acc[c]);
+      if (g < NG - 1) {
         FA_INTERLEAVE(4, 1)
       } else {
-        FA_INTERLEAVE(4, 2)
+        FA_INTERLEAVE(4, 2 * NP)
       }
       __builtin_amdgcn_sched_barrier(0);
-      if (prefetch) {
-        loader.load_block(k_next, sK + (buf ^ 1) * kTileElems, g);
-        loader.load_block(v_next, sV + (buf ^ 1) * kTileElems, g);
+      if (prefetch) {   // (stage g copies block g % 4 of panel g / 4 of the next K and V tiles)
+        loader.load_block(k_next + 128 * (g >> 2), sK + ((buf ^ 1) * NP + (g >> 2)) * kTileElems, g & 3);
+        loader.load_block(v_next + 128 * (g >> 2), sV + ((buf ^ 1) * NP + (g >> 2)) * kTileElems, g & 3);
       }
     }
     read_v(1);
@@ -269,7 +279,7 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
       const float alpha = fast_exp2((m_run - m_safe) * e_scale);
       l_run *= alpha;
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+      for (int db = 0; db < 4 * NP; ++db)
 #pragma unroll
         for (int e = 0; e < 16; ++e) o_acc[db][e] *= alpha;
       m_run = m_new;
@@ -303,8 +313,8 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
     for (int tt = 0; tt < 4; ++tt) {
       if (tt < 2) read_v(tt + 2);
 #pragma unroll
-      for (int db = 0; db < 4; ++db) o_acc[db] = mfma32(join_tr(vlo[tt][db], vhi[tt][db]), p[tt], o_acc[db]);
-      if (tt < 2) { FA_INTERLEAVE(4, 2) }
+      for (int db = 0; db < 4 * NP; ++db) o_acc[db] = mfma32(join_tr(vlo[tt][db], vhi[tt][db]), p[tt], o_acc[db]);
+      if (tt < 2) { FA_INTERLEAVE(4 * NP, 2) }
       __builtin_amdgcn_sched_barrier(0);
     }
 
@@ -318,7 +328,7 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
   const float l_tot = half_sum(l_run);
   const float inv = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
 #pragma unroll
-  for (int db = 0; db < 4; ++db) {
+  for (int db = 0; db < 4 * NP; ++db) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       bf16x2 lo = pack_bf16(o_acc[db][4 * g] * inv, o_acc[db][4 * g + 1] * inv);
@@ -334,15 +344,15 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_d128_kernel(FwdArgs a) {
   }
 }
 
-template <int SCORE>
+template <int SCORE, int NP = 1>
 static int launch_fwd(const FwdArgs& a, hipStream_t stream) {
   using namespace fwd_cfg;
-  auto kern = fwd_bf16_d128_kernel<SCORE>;
+  auto kern = fwd_bf16_kernel<SCORE, NP>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, NP * LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(fwd): %s", hipGetErrorString(attr));
   const int n_wg = a.B * a.Hq * (a.Sq / BM);
-  hipLaunchKernelGGL(kern, dim3(n_wg), dim3(256), LDS_BYTES, stream, a);
+  hipLaunchKernelGGL(kern, dim3(n_wg), dim3(256), NP * LDS_BYTES, stream, a);
   return check_launch("flexattn_fwd bf16");
 }
 
@@ -924,6 +934,22 @@ int fwd_bf16_d128(const FwdArgs& a, hipStream_t stream) {
   }
   return set_error(FLEXATTN_EINVAL, "unknown score kind %d", a.score.kind);
 #endif
+}
+
+// Head dim 256: the kernels with a compiled main loop (two 128-column panels per row), every score kind.
+int fwd_bf16_d256(const FwdArgs& a, hipStream_t stream) {
+  switch (a.score.kind) {
+    case FLEXATTN_SCORE_NONE:
+      return a.score.ab ? launch_fwd<kScoreBiasOnly, 2>(a, stream) : launch_fwd<FLEXATTN_SCORE_NONE, 2>(a, stream);
+#ifdef FLEXATTN_CUSTOM_ONLY
+    case FLEXATTN_SCORE_CUSTOM: return launch_fwd<FLEXATTN_SCORE_CUSTOM, 2>(a, stream);
+#else
+    case FLEXATTN_SCORE_ALIBI: return launch_fwd<FLEXATTN_SCORE_ALIBI, 2>(a, stream);
+    case FLEXATTN_SCORE_SOFTCAP: return launch_fwd<FLEXATTN_SCORE_SOFTCAP, 2>(a, stream);
+    case FLEXATTN_SCORE_ALIBI_TILE: return launch_fwd<FLEXATTN_SCORE_ALIBI_TILE, 2>(a, stream);
+#endif
+  }
+  return set_error(FLEXATTN_ENOTSUP, "score kind %d is not in this library", a.score.kind);
 }
 
 void fwd_bf16_d128_tile(int* bq, int* bk) {

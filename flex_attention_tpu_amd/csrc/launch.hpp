@@ -14,10 +14,13 @@ int check_launch(const char* what);
 
 // bf16, head dim 128 (MFMA kernels)
 int fwd_bf16_d128(const FwdArgs& a, hipStream_t stream);
+int fwd_bf16_d256(const FwdArgs& a, hipStream_t stream);   // (same tiles as head dim 128)
 void fwd_bf16_d128_tile(int* bq, int* bk);
 int bwd_dq_bf16_d128(const BwdArgs& a, hipStream_t stream);
+int bwd_dq_bf16_d256(const BwdArgs& a, hipStream_t stream);
 void bwd_dq_bf16_d128_tile(int* bq, int* bk);
 int bwd_dkv_bf16_d128(const BwdArgs& a, hipStream_t stream);
+int bwd_dkv_bf16_d256(const BwdArgs& a, hipStream_t stream);
 void bwd_dkv_bf16_d128_tile(int* bq, int* bk);
 // dq = out_scale dS K from the dS blocks that the dk/dv stream kernels wrote to a.ds (a.map: row lists at the
 // dk/dv tiles)

@@ -27,13 +27,14 @@ __host__ __device__ __forceinline__ constexpr int tile_off(int row, int chunk) {
   return row * kTileD + ((chunk ^ swz(row)) << 3);
 }
 
-// Asynchronous copy of a 64 x 128 bf16 tile (global row stride 128 elements) into LDS with
+// Asynchronous copy of a 64 x 128 bf16 tile (global row stride ROW elements: 128, or the head dimension where a
+// tile is one 128-column panel of wider rows) into LDS with
 // global_load_lds_dwordx4: the data never passes through registers.  Each instruction fills one
 // contiguous 1 KB block (4 tile rows); lane L's 16 bytes land at block + 16*L, so the swizzle is
 // applied on the global side.  The NWAVES waves of a work-group each copy 16/NWAVES blocks.  The
 // lane-dependent global offsets are loop invariant and are computed once (TileLoader::init); per
 // tile only the uniform base pointers change.  Completion = vmcnt(0) on every wave + barrier.
-template <int NWAVES>
+template <int NWAVES, int ROW = kTileD>
 struct TileLoader {
   static constexpr int kBlocks = 16 / NWAVES;  // 1 KB blocks copied per wave
   unsigned goff[kBlocks];  // byte offset of this lane's 16 bytes inside the global tile, per block
@@ -45,7 +46,7 @@ struct TileLoader {
     for (int i = 0; i < kBlocks; ++i) {
       const int row = (wave * kBlocks + i) * 4 + (lane >> 4);
       const int chunk = (lane & 15) ^ swz(row);
-      goff[i] = (unsigned)(row * kTileD + chunk * 8) * 2u;
+      goff[i] = (unsigned)(row * ROW + chunk * 8) * 2u;
     }
   }
 

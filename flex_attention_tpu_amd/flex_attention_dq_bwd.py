@@ -20,7 +20,7 @@ def compute_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
     if not (o.is_cuda and o.is_contiguous() and do.is_contiguous()):
         raise ValueError("o and do must be contiguous GPU tensors")
     B, H, S, D = o.shape
-    if D not in (64, 128):   # (zero columns add nothing to the sum)
+    if D not in (64, 128) and not (D == 256 and o.dtype == torch.bfloat16):   # (zero columns add nothing to the sum)
         D = kernel_head_dim(D, o.dtype)
         o, do = pad_seq(o, D, 3), pad_seq(do, D, 3)
     d = torch.empty(B, H, S, dtype=torch.float32, device=o.device)
@@ -116,17 +116,25 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     if rows is not None:  # ids differ between batch entries: one launch per entry
         if ds is not None and (ds.entries is None or len(ds.entries) != B):
             raise ValueError("ds does not come from a dk/dv pass of these arguments")
-        if return_dab:
-            raise NotImplementedError("return_dab with segment ids that differ between batch entries")
+        if return_dab and (ab is None or ds is not None or return_delta):
+            raise ValueError("return_dab needs the additive bias `ab` and excludes `ds` and return_delta")
         if _defer:
             return None
         if d is None:
             d = compute_delta(o, do)
-        out = torch.cat([flex_attention_bwd_dq(
+        parts = [flex_attention_bwd_dq(
             q[b:b + 1], k[b:b + 1], v[b:b + 1], batch_entry(ab, b), rows[b], l[b:b + 1], m[b:b + 1], batch_entry(o, b),
             do[b:b + 1], d[b:b + 1], block_b=block_b, block_q=block_q, block_k_major=block_k_major, block_k=block_k,
             sm_scale=sm_scale, debug=debug, score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn, causal=causal,
-            compiled_loop=compiled_loop, ds=ds.entries[b] if ds is not None else None) for b in range(B)], 0)
+            compiled_loop=compiled_loop, ds=ds.entries[b] if ds is not None else None, return_dab=return_dab)
+            for b in range(B)]
+        if return_dab:
+            # a bias shared by the batch entries collects the sum of their gradients (added in float32; the
+            # entries' own planes were rounded to the bias's dtype once already)
+            dabs = [x[1] for x in parts]
+            dab = torch.cat(dabs, 0) if ab.shape[0] != 1 else torch.stack([x.float() for x in dabs]).sum(0).to(ab.dtype)
+            return torch.cat([x[0] for x in parts], 0), dab
+        out = torch.cat(parts, 0)
         return (out, d) if return_delta else out
     if o is not None and tuple(o.shape) != tuple(q.shape):
         raise ValueError(f"o has shape {tuple(o.shape)}, expected {tuple(q.shape)}")

@@ -5,6 +5,7 @@ import os
 import re
 
 import pytest
+import torch
 
 from flex_attention_tpu_amd import _lib
 
@@ -48,6 +49,18 @@ def test_tile_shapes(lib):
         assert bq > 0 and bk > 0
     with pytest.raises(NotImplementedError):
         _lib.tile_shape(_lib.PASS_FWD, _lib.BF16, 96)
+    # bf16 head dimension 256 runs on the tiles of 128; beyond that, and float32 beyond 128, there is no kernel
+    for p in (_lib.PASS_FWD, _lib.PASS_DQ, _lib.PASS_DKV):
+        assert _lib.tile_shape(p, _lib.BF16, 256) == _lib.tile_shape(p, _lib.BF16, 128)
+    for dtype, D in ((_lib.BF16, 384), (_lib.F32, 256)):
+        with pytest.raises(NotImplementedError):
+            _lib.tile_shape(_lib.PASS_FWD, dtype, D)
+    from flex_attention_tpu_amd._common import kernel_head_dim
+    assert [kernel_head_dim(D, torch.bfloat16) for D in (1, 64, 128, 129, 192, 256)] == [128, 128, 128, 256, 256, 256]
+    assert [kernel_head_dim(D, torch.float32) for D in (1, 64, 65, 128)] == [64, 64, 128, 128]
+    for dtype, D in ((torch.bfloat16, 257), (torch.float32, 129)):
+        with pytest.raises(NotImplementedError):
+            kernel_head_dim(D, dtype)
     with pytest.raises(ValueError):
         _lib.tile_shape(7, _lib.BF16, 128)
 

@@ -46,10 +46,20 @@ def _oracle_kwargs(name, Sq, Sk):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
 @pytest.mark.parametrize("name", ["alibi_mod", "softcap_mod", "mixed_mod", "prefix_lm", "checker", "mixed_mod+prefix_lm"])
 def test_compiled_closures_all_passes(F, compiled, name, dtype):
+    _closures_all_passes(F, compiled, name, dtype, 128)
+
+
+@pytest.mark.parametrize("name", ["alibi_mod", "mixed_mod+prefix_lm"])
+def test_compiled_closures_head_dimension_256(F, compiled, name):
+    """The functor libraries hold the bf16 kernels of head dimension 256 as well."""
+    _closures_all_passes(F, compiled, name, torch.bfloat16, 256)
+
+
+def _closures_all_passes(F, compiled, name, dtype, D):
     score_fn, mask_pair = compiled[name]
     B, Hq, Hkv, S = 2, 4, 2, 512
-    sc = 1 / math.sqrt(128)
-    q, k, v, do = O.make_inputs(B, Hq, Hkv, S, S, 128, dtype=dtype, seed=61)
+    sc = 1 / math.sqrt(D)
+    q, k, v, do = O.make_inputs(B, Hq, Hkv, S, S, D, dtype=dtype, seed=61)
     from flex_attention_tpu_amd import masks
     okw = dict(sm_scale=sc, causal=(name == "alibi_mod"), **_oracle_kwargs(name, S, S))
     ro, rl, rm = O.mha_reference(q, k, v, save_residuals=True, **okw)

@@ -409,6 +409,60 @@ def test_small_head_dimensions(F, D, dtype):
         assert_close(name, t, r, dtype)
 
 
+@pytest.mark.parametrize("case", _small_cases(), ids=lambda c: c[0])
+def test_head_dimension_256(F, case):
+    """bf16 at head dimension 256 (the reference takes any multiple of 128, flex_attention_kernel.py:302-306): rows
+    of two 128-column panels through the kernels with a compiled main loop, every mask and score of the small
+    matrix, all passes against the oracle.  These kernels exchange no dS."""
+    name, (B, Hq, Hkv, Sq, Sk), mask_pair, score_fn, okw, _ = case
+    D, dtype = 256, torch.bfloat16
+    sc = 1 / math.sqrt(D)
+    q, k, v, do = O.make_inputs(B, Hq, Hkv, Sq, Sk, D, dtype=dtype, seed=83)
+    ro, rl, rm = O.mha_reference(q, k, v, sm_scale=sc, save_residuals=True, **okw)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, sm_scale=sc, **okw)
+    qc, kc, vc, doc = q, k, v, do
+    q, k, v, do = [x.to(DEV) for x in (q, k, v, do)]
+    mf, bf = mask_pair if mask_pair else (None, None)
+    o, l, m = _fwd(F, q, k, v, sc, mf, bf, score_fn)
+    assert o.shape == q.shape
+    assert_close("o", o, ro, dtype)
+    assert_close("lse", m + l.log(), rm + rl.log(), dtype)
+    d = F.compute_delta(o, do)
+    assert_close("delta", d, O.delta(o.cpu(), do.cpu()), torch.float32)
+    dq = _dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, score_fn)
+    dk, dv = _dkv(F, q, k, v, l, m, do, d, sc, mf, bf, score_fn)
+    assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+    _check_grads((dq, dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, dtype, dict(sm_scale=sc, **okw))
+    assert _exchanged_dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, score_fn, dk, dv, expect=False) is None
+
+
+def test_head_dimensions_between_128_and_256(F):
+    """A bf16 head dimension of 192 runs zero-padded to 256; with an additive bias and its gradient, grouped kv
+    heads, a ragged length and per-entry segment ids (the host-side paths around the kernels at the wider rows)."""
+    D, dtype = 192, torch.bfloat16
+    sc = 1 / math.sqrt(D)
+    B, Hq, Hkv, S = 2, 4, 2, 300
+    q, k, v, do = O.make_inputs(B, Hq, Hkv, S, S, D, dtype=dtype, seed=89)
+    g = torch.Generator().manual_seed(97)
+    ab = torch.randn(1, Hq, S, S, generator=g)
+    sid = torch.stack([O.doc_ids_from_lengths(x) for x in ([100, 200], [300])])
+    okw = dict(sm_scale=sc, causal=True, segment_ids=sid)
+    ab_full = ab.expand(B, Hq, S, S)
+    ro, rl, rm = O.mha_reference(q, k, v, ab_full, save_residuals=True, **okw)
+    qg, kg, vg, dog, abg = [x.to(DEV) for x in (q, k, v, do, ab)]
+    o, l, m, dq, dk, dv = _all_passes_with(F, qg, kg, vg, dog, abg, sid, sc, None, None, True)
+    assert o.shape == q.shape and dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+    assert_close("o", o, ro, dtype)
+    assert_close("lse", m + l.log(), rm + rl.log(), dtype)
+    ma = O.mha_bwd_reference(q, k, v, o.float().cpu(), do, l.cpu(), m.cpu(), ab_full, return_dab=True, **okw)
+    for name, t, r in (("dq", dq, ma[0]), ("dk", dk, ma[1]), ("dv", dv, ma[2])):
+        assert_close(name, t, r, dtype)
+    dq2, dab = F.flex_attention_bwd_dq(qg, kg, vg, abg, sid, l, m, o, dog, F.compute_delta(o, dog), block_b=1, block_q=128,
+                                       block_k_major=128, block_k=128, sm_scale=sc, debug=False, causal=True, return_dab=True)
+    assert dab.shape == ab.shape and torch.equal(dq2, dq)
+    assert_close("dab", dab, ma[3].sum(0, keepdim=True), dtype)   # (summed over the batch entries the bias is shared by)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
 def test_compiled_loop_kernels_on_request(F, dtype):
     """bf16 calls run the generated-stream kernels wherever one exists (covered by every other test
@@ -904,8 +958,11 @@ def test_entry_points_reject_bad_arguments_on_gpu(F):
     q = torch.zeros(1, 2, 256, 128, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ValueError):  # block_q must divide the sequence length
         F._flex_attention_impl(q, q, q, None, None, False, False, 1.0, 1, 96, 64, 64, False, None, None, None)
-    q = torch.zeros(1, 2, 256, 192, dtype=torch.bfloat16, device=DEV)
-    with pytest.raises(NotImplementedError):  # head dimensions above 128 have no kernel (smaller ones are padded)
+    q = torch.zeros(1, 2, 256, 384, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(NotImplementedError):  # bf16 head dimensions above 256 have no kernel (others are padded to 128 or 256)
+        F._flex_attention_impl(q, q, q, None, None, False, False, 1.0, 1, 128, 128, 128, False, None, None, None)
+    q = torch.zeros(1, 2, 256, 192, dtype=torch.float32, device=DEV)
+    with pytest.raises(NotImplementedError):  # float32: above 128
         F._flex_attention_impl(q, q, q, None, None, False, False, 1.0, 1, 128, 128, 128, False, None, None, None)
     q = torch.zeros(1, 2, 256, 128, dtype=torch.float16, device=DEV)
     with pytest.raises(NotImplementedError):
