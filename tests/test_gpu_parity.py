@@ -463,6 +463,25 @@ def test_head_dimensions_between_128_and_256(F):
     assert_close("dab", dab, ma[3].sum(0, keepdim=True), dtype)   # (summed over the batch entries the bias is shared by)
 
 
+@pytest.mark.parametrize("case", ["causal_gqa", "softcap_documents"])
+def test_head_dimension_256_at_4096_tokens(F, case):
+    """Head dimension 256 at the sequence length of the benchmark configurations (B=2, 8 q heads on 2 kv heads,
+    S=4096): 64 kv tiles in a row's list, 32 q tiles times 4 heads in a column's.  Sampled rows of two whole kv
+    groups against the oracle."""
+    from flex_attention_tpu_amd import masks, scores
+    D, S = 256, 4096
+    sc = 1 / math.sqrt(D)
+    q, k, v, do = O.make_inputs(2, 8, 2, S, S, D, dtype=torch.bfloat16, seed=137)
+    if case == "causal_gqa":
+        (mf, bf), sfn, okw = masks.make_causal_mask_fns(128, 128), None, dict(causal=True)
+    else:
+        lens = [1000, 24, 2000, 1072]
+        (mf, bf), sfn = masks.make_jagged_mask_fns(128, 128, lens), scores.make_softcap_score_fn(30.0)
+        okw = dict(causal=True, segment_ids=O.doc_ids_from_lengths(lens), score_mod=O.score_mod_softcap(30.0))
+    heads = [(0, h) for h in range(4)] + [(1, h) for h in range(4, 8)]
+    _sampled_oracle_check(F, q, k, v, do, sc, mf, bf, sfn, okw, 96, heads)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
 def test_compiled_loop_kernels_on_request(F, dtype):
     """bf16 calls run the generated-stream kernels wherever one exists (covered by every other test

@@ -177,8 +177,9 @@ def test_causal_prefix(F, name):
     _same("dq of the first half", bwd(head(q), head(k), head(v), oh, lh, mh, head(do))[0], head(dq))
 
 
-def _random_case(rng, it):
-    """A random shape, mask, score function, dtype and kernel family (seeded): (tag, tensors, call arguments)."""
+def _random_case(rng, it, D=128):
+    """A random shape, mask, score function, dtype and kernel family (seeded): (tag, tensors, call arguments).
+    Head dimension D; 256 is bf16 only."""
     import math
     from flex_attention_tpu_amd import masks, scores
     B, Hkv, g = rng.choice([2, 3, 4, 8]), rng.choice([2, 4, 8, 16]), rng.choice([1, 1, 2, 4])
@@ -187,6 +188,8 @@ def _random_case(rng, it):
     sk = rng.choice(["none", "none", "alibi", "softcap"])
     dt = rng.choice([torch.bfloat16, torch.bfloat16, torch.bfloat16, torch.float32])
     compiled_loop = rng.random() < 0.2
+    if D > 128:
+        dt = torch.bfloat16
     if dt == torch.float32 and S > 2048:
         S = 1024
     if mk == "none":
@@ -205,10 +208,10 @@ def _random_case(rng, it):
         mf, bf = masks.make_jagged_mask_fns(128, 128, lens)
     sfn = {"none": None, "alibi": scores.make_alibi_global_score_fn(Hkv * g),
            "softcap": scores.make_softcap_score_fn(rng.choice([2.0, 30.0]))}[sk]
-    sc = rng.choice([1.0, 1.0, 3.0]) / math.sqrt(128)
+    sc = rng.choice([1.0, 1.0, 3.0]) / math.sqrt(D)
     gen = torch.Generator().manual_seed(7000 + it)
-    q, k, v, do = [torch.randn(B, h, S, 128, generator=gen).to(dt).to(DEV) for h in (Hkv * g, Hkv, Hkv, Hkv * g)]
-    tag = f"B={B} Hq={Hkv * g} Hkv={Hkv} S={S} mask={mk} score={sk} scale={sc:.3f} {str(dt)[6:]} compiled_loop={compiled_loop}"
+    q, k, v, do = [torch.randn(B, h, S, D, generator=gen).to(dt).to(DEV) for h in (Hkv * g, Hkv, Hkv, Hkv * g)]
+    tag = f"B={B} Hq={Hkv * g} Hkv={Hkv} S={S} D={D} mask={mk} score={sk} scale={sc:.3f} {str(dt)[6:]} compiled_loop={compiled_loop}"
     return tag, (q, k, v, do), (sc, mf, bf, sfn, compiled_loop), mk
 
 
@@ -225,17 +228,18 @@ def _all_passes(F, q, k, v, do, sc, mf, bf, sfn, compiled_loop):
     return o, l, m, dq, dk, dv, dqx
 
 
-def test_random_shapes_locality(F):
-    """The locality properties above on 24 random shapes (2 to 32 tiles, 2 to 64 heads, grouped kv heads), masks,
-    score functions, scales, both dtypes and both kernel families: one batch entry alone against its part of the
-    full launch, every output and the dq from handed-over dS, and under causal masks a prefix of the tokens against
-    the prefix of o, l, m, dq.  Bit for bit."""
+@pytest.mark.parametrize("D,n_cases,seed", [(128, 24, 20), (256, 10, 22)], ids=["d128", "d256"])
+def test_random_shapes_locality(F, D, n_cases, seed):
+    """The locality properties above on random shapes (2 to 32 tiles, 2 to 64 heads, grouped kv heads), masks,
+    score functions, scales, both dtypes and both kernel families (24 cases at head dimension 128, 10 at 256): one
+    batch entry alone against its part of the full launch, every output and the dq from handed-over dS, and under
+    causal masks a prefix of the tokens against the prefix of o, l, m, dq.  Bit for bit."""
     import random
     import warnings
     warnings.filterwarnings("ignore", message="score_fn with sm_scale")
-    rng = random.Random(20)
-    for it in range(24):
-        tag, (q, k, v, do), args, mk = _random_case(rng, it)
+    rng = random.Random(seed)
+    for it in range(n_cases):
+        tag, (q, k, v, do), args, mk = _random_case(rng, it, D)
         full = _all_passes(F, q, k, v, do, *args)
         b = rng.randrange(q.shape[0])
         part = _all_passes(F, *[x[b:b + 1].contiguous() for x in (q, k, v, do)], *args)
@@ -248,20 +252,21 @@ def test_random_shapes_locality(F):
                 _same(f"{tag}: {name} of the first {n} tokens alone", a, r[:, :, :n])
 
 
-def test_grouped_kv_heads_equal_repeated_kv_heads(F):
+@pytest.mark.parametrize("D,n_cases,seed", [(128, 12, 21), (256, 6, 23)], ids=["d128", "d256"])
+def test_grouped_kv_heads_equal_repeated_kv_heads(F, D, n_cases, seed):
     """Grouped kv heads against the same call with every kv head repeated for its query heads (on 12 seeded random
-    shapes, masks and score functions): o, l, m and dq bit for bit (a query head's rows do not care how the kv heads
+    shapes, masks and score functions at head dimension 128, 6 at 256): o, l, m and dq bit for bit (a query head's rows do not care how the kv heads
     are stored; the schedules differ); dk, dv, which the grouped kernels sum over the group in fp32 inside one work
     item, against the sum of the repeated heads' bf16 results in relative L2."""
     import random
     import warnings
     warnings.filterwarnings("ignore", message="score_fn with sm_scale")
-    rng = random.Random(21)
+    rng = random.Random(seed)
     done = 0
     it = 0
-    while done < 12:
+    while done < n_cases:
         it += 1
-        tag, (q, k, v, do), args, _ = _random_case(rng, 100 + it)
+        tag, (q, k, v, do), args, _ = _random_case(rng, 100 + it, D)
         g = q.shape[1] // k.shape[1]
         if g == 1:
             continue
@@ -271,7 +276,7 @@ def test_grouped_kv_heads_equal_repeated_kv_heads(F):
         e = _all_passes(F, q, ke, ve, do, *args)
         for name, x, y in zip(("o", "l", "m", "dq"), a[:4], e[:4]):
             _same(f"{tag}: {name} with repeated kv heads", y, x)
-        B, Hkv, S, D = k.shape
+        B, Hkv, S, _ = k.shape
         for name, x, y in zip(("dk", "dv"), a[4:6], e[4:6]):
             ys = y.float().view(B, Hkv, g, S, D).sum(2)
             rel = float((x.float() - ys).norm() / (ys.norm() + 1e-9))
