@@ -8,6 +8,7 @@
  *
  * Conventions
  *  - All tensors are contiguous row-major [B, H, S, D] device memory owned by the caller.
+ *    Head dimension D: 128 or 256 for bf16, 64 or 128 for float32 (anything else: FLEXATTN_ENOTSUP).
  *    q/o/do/dq have Hq heads, k/v/dk/dv have Hkv heads, Hq % Hkv == 0 (kv head = h / (Hq/Hkv)).
  *  - l, m, delta are float32 [B, Hq, Sq].
  *  - Every function returns FLEXATTN_OK or a negative error code, never throws or aborts, and
@@ -26,7 +27,7 @@
 extern "C" {
 #endif
 
-#define FLEXATTN_VERSION 103 /* major*10000 + minor*100 + patch */
+#define FLEXATTN_VERSION 104 /* major*10000 + minor*100 + patch */
 
 /* status codes */
 #define FLEXATTN_OK 0
@@ -192,7 +193,7 @@ const char* flexattn_last_error_string(void);
 const char* flexattn_custom_tag(void);
 
 /* Tile granularity (block_q, block_k) the kernels of `pass` expect of the block map for this
- * dtype and head dimension. */
+ * dtype and head dimension (bf16 head dimension 256 runs on the tiles of 128). */
 int flexattn_tile_shape(int32_t pass, int32_t dtype, int32_t D, int32_t* block_q, int32_t* block_k);
 
 /* Block-mask builder.  Replaces the per-grid-step evaluation of the `block_mask_fn` closures
