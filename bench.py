@@ -5,7 +5,8 @@ forward (saving l, m), delta pre-pass, dq backward, dk/dv backward (where the pa
 softcap scores and masks with many partial tiles, the dk/dv pass hands its dS to the dq pass; where the kernels
 can run either way the other way is timed beside it).  The headline workload is
 benchmark configurations 2 + 3 (B=4, H=32, S=4096, D=128, bf16, causal); the other configurations
-(cfg1 fp32 small, cfg4 ALiBi + causal window, cfg5 GQA + soft-cap + documents) are measured in the
+(cfg1 fp32 small, cfg4 ALiBi + causal window, cfg5 GQA + soft-cap + documents; and d256, cfg2's FLOPs at head
+dimension 256, which is not one of the reference's configurations) are measured in the
 same run and reported as sub-objects (`--config NAME` makes one of them the headline instead).
 Prints ONE JSON line: whole-step algorithmic TFLOP/s, per-pass TFLOP/s and fraction of the bf16
 MFMA peak, launch-time quantiles, a roofline object for the dominant kernel and the CPU oracle
@@ -264,9 +265,9 @@ def main():
     head = summary(cfg, r)
     others = {}
     if not args.only:
-        for other in ("cfg1", "cfg2", "cfg4", "cfg5"):
+        for other in ("cfg1", "cfg2", "cfg4", "cfg5", "d256"):
             if other != name:
-                c = configs.CONFIGS[other]
+                c = configs.CONFIGS.get(other) or configs.EXTRA_CONFIGS[other]
                 others[other] = summary(c, measure(c, args.steps, args.warmup))
                 torch.cuda.empty_cache()
 

@@ -94,12 +94,9 @@ def _doc_ids_of(ids) -> DocIds:
         if hit is not None and hit[0]() is ids and hit[1] == ids._version:
             return hit[2]
     t = torch.as_tensor(ids).detach().cpu()
-    if t.ndim == 2:
-        # (rows that differ are split into one call per batch entry before they get here: per_batch_segments)
-        if not bool((t == t[:1]).all()):
-            raise ValueError("segment ids differ between batch entries")
-        t = t[0]
-    if t.ndim != 1:
+    if t.ndim == 2 and bool((t == t[:1]).all()):
+        t = t[0]   # (equal rows: one row serves the batch)
+    if t.ndim not in (1, 2):
         raise ValueError("segment_ids must be a 1-D (or [B, S]) array of ids")
     doc = DocIds(t.numpy().astype(np.int64))
     if isinstance(ids, torch.Tensor):
@@ -108,9 +105,9 @@ def _doc_ids_of(ids) -> DocIds:
 
 
 def segment_doc_ids(segment_ids):
-    """(q ids, kv ids or None) of a ``segment_ids`` argument: one id array for both sides (1-D, or [B, S] with
-    equal rows), or an object with ``.q`` / ``.kv`` arrays (the reference's SegmentIds, jax_exp.py:37-51),
-    which may differ and need not be sorted."""
+    """(q ids, kv ids or None) of a ``segment_ids`` argument: one id array for both sides (1-D, or [B, S]: a row
+    per batch entry, mha_reference.py:65-73), or an object with ``.q`` / ``.kv`` arrays (the reference's
+    SegmentIds, jax_exp.py:37-51), which may differ and need not be sorted."""
     if hasattr(segment_ids, "q") and hasattr(segment_ids, "kv") and not isinstance(segment_ids, DocIds):
         dq = _doc_ids_of(segment_ids.q)
         dk = dq if segment_ids.kv is segment_ids.q else _doc_ids_of(segment_ids.kv)
@@ -118,46 +115,11 @@ def segment_doc_ids(segment_ids):
     return _doc_ids_of(segment_ids), None
 
 
-class _Segments:
-    """q / kv id arrays of one batch entry (same attributes as the reference's SegmentIds, jax_exp.py:37-51)."""
-
-    def __init__(self, q, kv):
-        self.q, self.kv = q, kv
-
-
-def per_batch_segments(segment_ids, B: int):
-    """None when one mask serves the whole batch; else a list with the ``segment_ids`` argument of every batch
-    entry.  The reference accepts ids of shape [B, S] (mha_reference.py:65-73); the kernels take one id array
-    per launch, so a batch whose entries carry different ids runs as one launch per entry."""
-    if segment_ids is None or isinstance(segment_ids, DocIds):
-        return None
-
-    def rows_of(x):
-        if isinstance(x, DocIds):
-            return None
-        t = torch.as_tensor(x)
-        if t.ndim != 2 or t.shape[0] == 1:
-            return None
-        if t.shape[0] != B:
-            raise ValueError(f"segment ids have {t.shape[0]} rows for a batch of {B}")
-        t = t.detach().cpu()
-        return None if bool((t == t[:1]).all()) else t
-
-    if hasattr(segment_ids, "q") and hasattr(segment_ids, "kv"):
-        rq, rk = rows_of(segment_ids.q), rows_of(segment_ids.kv)
-        if rq is None and rk is None:
-            return None
-        return [_Segments(rq[b] if rq is not None else segment_ids.q, rk[b] if rk is not None else segment_ids.kv)
-                for b in range(B)]
-    rows = rows_of(segment_ids)
-    return None if rows is None else [rows[b] for b in range(B)]
-
-
-def batch_entry(t, b: int):
-    """Batch entry b of a tensor argument as a batch of one (None and batch-broadcast tensors pass through)."""
-    if t is None or t.shape[0] == 1:
-        return t
-    return t[b:b + 1]
+def check_doc_batches(spec: MaskSpec, B: int) -> None:
+    """Document ids with a row per batch entry must have one for every entry of the call."""
+    for d in (spec.doc_ids, spec.doc_ids_k):
+        if d is not None and d.batches not in (1, B):
+            raise ValueError(f"segment ids have {d.batches} rows for a batch of {B}")
 
 
 def bias_c(ab, B: int, Hq: int, Sq: int, Sk: int, Sq_p: int, Sk_p: int, device):
@@ -199,14 +161,17 @@ def resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk, Sq_pad=Non
         if spec.flags & _lib.MASK_DOC:
             ids_q = spec.doc_ids.array
             ids_k = (spec.doc_ids_k if spec.doc_ids_k is not None else spec.doc_ids).array
-            if len(ids_q) < Sq or len(ids_k) < Sk:
-                raise ValueError(f"document ids cover {len(ids_q)} q / {len(ids_k)} kv positions, need {Sq} / {Sk}")
-            ids_q, ids_k = ids_q[:Sq], ids_k[:Sk]
+            if ids_q.shape[-1] < Sq or ids_k.shape[-1] < Sk:
+                raise ValueError(f"document ids cover {ids_q.shape[-1]} q / {ids_k.shape[-1]} kv positions, need {Sq} / {Sk}")
+            ids_q, ids_k = ids_q[..., :Sq], ids_k[..., :Sk]
         else:
             ids_q, ids_k = np.zeros(Sq, np.int32), np.zeros(Sk, np.int32)
         pad_id = int(max(ids_q.max(initial=0), ids_k.max(initial=0))) + 1    # an id no query carries
-        dq_p = DocIds(np.pad(ids_q, (0, Sq_pad - Sq), mode="edge"))
-        dk_p = DocIds(np.pad(ids_k, (0, Sk_pad - Sk), constant_values=pad_id))
+
+        def tail(a, n):   # (pad widths of the sequence axis; rows per batch entry keep their axis)
+            return [(0, 0)] * (a.ndim - 1) + [(0, n)]
+        dq_p = DocIds(np.pad(ids_q, tail(ids_q, Sq_pad - Sq), mode="edge"))
+        dk_p = DocIds(np.pad(ids_k, tail(ids_k, Sk_pad - Sk), constant_values=pad_id))
         spec = MaskSpec(spec.flags | _lib.MASK_DOC, spec.window, spec.stride, dq_p, spec.custom, None if dk_p == dq_p else dk_p)
     return spec
 

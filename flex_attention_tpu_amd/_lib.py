@@ -56,7 +56,7 @@ class MaskSpecC(C.Structure):
         ("flags", C.c_int32),
         ("window", C.c_int32),
         ("stride", C.c_int32),
-        ("reserved", C.c_int32),
+        ("doc_batches", C.c_int32),
         ("doc_q", C.c_void_p),
         ("doc_k", C.c_void_p),
         ("doc_q_range", C.c_void_p),

@@ -144,6 +144,21 @@ def doc_ids_on(doc: Optional[DocIds], device) -> Optional[torch.Tensor]:
     return t
 
 
+_rows_cache = LRU(DOC_CACHE_SIZE)   # (DocIds, B) -> DocIds with B rows
+
+
+def _rows_of(doc: DocIds, B: int) -> DocIds:
+    """`doc` with one row per batch entry (a shared row repeated; cached)."""
+    if doc.batches == B and doc.array.ndim == 2:
+        return doc
+    key = (doc, B)
+    d = _rows_cache.get(key)
+    if d is None:
+        d = DocIds(doc.rows(B))
+        _rows_cache.put(key, d)
+    return d
+
+
 _range_cache = LRU(DOC_CACHE_SIZE)  # (DocIds, DocIds of the other side, device) -> int32 [n, 2] device array or False
 
 
@@ -161,28 +176,37 @@ def doc_ranges_on(doc: DocIds, other: DocIds, device) -> Optional[torch.Tensor]:
 def mask_spec_c(spec: MaskSpec, Sq: int, Sk: int, device) -> _lib.MaskSpecC:
     """C view of a MaskSpec; validates the document array lengths."""
     doc_q = doc_k = range_q = range_k = None
+    doc_batches = 0
     if spec.flags & _lib.MASK_DOC:
         if spec.doc_ids is None:
             raise ValueError("document mask without document ids")
         ids_k = spec.doc_ids_k if spec.doc_ids_k is not None else spec.doc_ids
         if len(spec.doc_ids) < Sq or len(ids_k) < Sk:
             raise ValueError(f"document ids cover {len(spec.doc_ids)} q / {len(ids_k)} kv positions, need {Sq} / {Sk}")
-        tq, tk = doc_ids_on(spec.doc_ids, device), doc_ids_on(ids_k, device)
+        # a row per batch entry on either side: both sides go to the kernels as [B, S] (doc_batches = B)
+        batches = max(spec.doc_ids.batches, ids_k.batches)
+        ids_q = spec.doc_ids
+        if batches > 1:
+            if len(ids_q) != Sq or len(ids_k) != Sk:   # (the kernels step from row to row by the sequence lengths)
+                raise ValueError(f"document ids per batch entry must have exactly {Sq} q / {Sk} kv positions")
+            ids_q, ids_k = _rows_of(ids_q, batches), _rows_of(ids_k, batches)
+        tq, tk = doc_ids_on(ids_q, device), doc_ids_on(ids_k, device)
         cur = torch.cuda.current_stream(device)
         tq.record_stream(cur)   # (cached arrays may be evicted while a kernel on this stream still reads them)
         tk.record_stream(cur)
         doc_q, doc_k = tq.data_ptr(), tk.data_ptr()
         # sorted ids (the usual case: documents packed one after the other): the interval of the other side's
         # positions with a position's id, from which the kernels mask partial tiles without comparing ids
-        if len(spec.doc_ids) == Sq and len(ids_k) == Sk:
-            rq, rk = doc_ranges_on(spec.doc_ids, ids_k, device), doc_ranges_on(ids_k, spec.doc_ids, device)
+        if len(ids_q) == Sq and len(ids_k) == Sk:
+            rq, rk = doc_ranges_on(ids_q, ids_k, device), doc_ranges_on(ids_k, ids_q, device)
             if rq is not None:
                 rq.record_stream(cur)
                 range_q = rq.data_ptr()
             if rk is not None:
                 rk.record_stream(cur)
                 range_k = rk.data_ptr()
-    return _lib.MaskSpecC(spec.flags, spec.window, spec.stride, 0, doc_q, doc_k, range_q, range_k)
+        doc_batches = batches
+    return _lib.MaskSpecC(spec.flags, spec.window, spec.stride, doc_batches, doc_q, doc_k, range_q, range_k)
 
 
 def build_block_map(spec: MaskSpec, Sq: int, Sk: int, block_q: int, block_k: int, device,

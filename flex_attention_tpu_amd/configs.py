@@ -45,6 +45,13 @@ CONFIGS: Dict[str, AttnConfig] = {
     "cfg5": AttnConfig("cfg5", torch.bfloat16, 1, 32, 8, 16384, 128, mask="document", score="softcap", cap=30.0),
 }
 
+# Not one of the reference's configurations: the FLOPs of cfg2 at head dimension 256 (half the heads), which the
+# reference's kernels accept (flex_attention_kernel.py:302-306) and none of its drivers runs.  bench.py reports it
+# next to the others.
+EXTRA_CONFIGS: Dict[str, AttnConfig] = {
+    "d256": AttnConfig("d256", torch.bfloat16, 4, 16, 16, 4096, 256, mask="causal"),
+}
+
 
 def make_inputs(cfg: AttnConfig, device="cpu"):
     g = torch.Generator(device="cpu").manual_seed(cfg.seed)

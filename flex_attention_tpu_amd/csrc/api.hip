@@ -61,7 +61,17 @@ static MaskArgs to_args(const flexattn_mask_spec& m) {
   r.doc_k = m.doc_k;
   r.doc_q_range = m.doc_q_range;
   r.doc_k_range = m.doc_k_range;
+  r.doc_batched = ((m.flags & FLEXATTN_MASK_DOC) && m.doc_batches > 1) ? 1 : 0;
   return r;
+}
+
+// Document arrays given per batch entry must cover the call's batch.
+static int check_doc_batches(const flexattn_mask_spec& m, int B) {
+  if (!(m.flags & FLEXATTN_MASK_DOC)) return FLEXATTN_OK;
+  if (m.doc_batches < 0 || (m.doc_batches > 1 && m.doc_batches != B))
+    return set_error(FLEXATTN_EINVAL, "mask DOC: doc_batches=%d, must be 0 or 1 (one row of ids for all) or the batch size %d",
+                     m.doc_batches, B);
+  return FLEXATTN_OK;
 }
 
 static int check_score(const flexattn_score_spec& s) {
@@ -223,6 +233,7 @@ static int to_bwd_args(const flexattn_bwd_params* p, int pass, BwdArgs* a) {
   if ((rc = check_scale_flags(p->sm_scale, p->flags)) != FLEXATTN_OK) return rc;
   if ((rc = check_score(p->score)) != FLEXATTN_OK) return rc;
   if ((rc = check_mask(p->mask)) != FLEXATTN_OK) return rc;
+  if ((rc = check_doc_batches(p->mask, p->B)) != FLEXATTN_OK) return rc;
   if ((rc = check_bias(p->ab, p->B, p->Hq, p->Sq, p->Sk)) != FLEXATTN_OK) return rc;
   if (p->dab != nullptr) {
     if (pass != FLEXATTN_PASS_DQ) return set_error(FLEXATTN_EINVAL, "dab is an output of flexattn_bwd_dq");
@@ -268,6 +279,7 @@ static int fwd_with_map(const flexattn_fwd_params* p, const flexattn_block_map& 
   if ((rc = check_scale_flags(p->sm_scale, p->flags)) != FLEXATTN_OK) return rc;
   if ((rc = check_score(p->score)) != FLEXATTN_OK) return rc;
   if ((rc = check_mask(p->mask)) != FLEXATTN_OK) return rc;
+  if ((rc = check_doc_batches(p->mask, p->B)) != FLEXATTN_OK) return rc;
   if ((rc = check_bias(p->ab, p->B, p->Hq, p->Sq, p->Sk)) != FLEXATTN_OK) return rc;
   FwdArgs a;
   a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.l = p->l; a.m = p->m;
@@ -351,7 +363,9 @@ int flexattn_build_block_mask(const flexattn_mask_spec* mask, int32_t Sq, int32_
     return set_error(FLEXATTN_EINVAL, "count and index arrays must be given in pairs");
   int rc = check_mask(*mask);
   if (rc != FLEXATTN_OK) return rc;
-  return build_block_mask(to_args(*mask), Sq, Sk, block_q, block_k, state, kv_cnt, kv_idx, q_cnt, q_idx,
+  if ((mask->flags & FLEXATTN_MASK_DOC) && mask->doc_batches < 0)
+    return set_error(FLEXATTN_EINVAL, "mask DOC: doc_batches=%d is negative", mask->doc_batches);
+  return build_block_mask(to_args(*mask), mask->doc_batches, Sq, Sk, block_q, block_k, state, kv_cnt, kv_idx, q_cnt, q_idx,
                           static_cast<hipStream_t>(stream));
 }
 
@@ -397,7 +411,8 @@ int flexattn_fwd_noalloc(const flexattn_fwd_params* p, void* stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   // every state, every count and every list entry below its count is rewritten by the builder: nothing of
   // an earlier call is read, nothing needs clearing
-  rc = build_block_mask(to_args(p->mask), p->Sq, p->Sk, bq, bk, base + kScratchStateOff,
+  if ((rc = check_doc_batches(p->mask, p->B)) != FLEXATTN_OK) return rc;
+  rc = build_block_mask(to_args(p->mask), p->mask.doc_batches, p->Sq, p->Sk, bq, bk, base + kScratchStateOff,
                         reinterpret_cast<int*>(base + kScratchCntOff), reinterpret_cast<int*>(base + kScratchIdxOff),
                         nullptr, nullptr, s);
   if (rc != FLEXATTN_OK) return rc;

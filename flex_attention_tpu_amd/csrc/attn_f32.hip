@@ -91,6 +91,7 @@ __global__ __launch_bounds__(256) void fwd_f32_kernel(FwdArgs a) {
   const int wg = blockIdx.x;
   const int bh = wg / nQ, qb = nQ - 1 - (wg % nQ);
   const int b = bh / a.Hq, h = bh % a.Hq, hk = h / (a.Hq / a.Hkv);
+  const MaskArgs mk = mask_of_batch(a.mask, b, a.Sq, a.Sk);
   const int tid = threadIdx.x, sub = tid & 3, r = tid >> 2;
   const int q_idx = qb * BQ + r;
 
@@ -100,7 +101,7 @@ __global__ __launch_bounds__(256) void fwd_f32_kernel(FwdArgs a) {
 
   ScoreMod<SCORE> sm;
   sm.init(a.score, a.sm_scale, h, b);
-  const int doc_i = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[q_idx] : 0;
+  const int doc_i = (mk.flags & FLEXATTN_MASK_DOC) ? mk.doc_q[q_idx] : 0;
 
   f32x4 qv[NV], acc[NV];
   load_slice<NV>(qv, Qg, sub);
@@ -128,8 +129,8 @@ __global__ __launch_bounds__(256) void fwd_f32_kernel(FwdArgs a) {
         float s = quad_sum(dot_slice<NV>(qv, sK + (j0 + jj) * D, sub));
         float x = sm.to_log2(s, q_idx, j) + sm.bias2(q_idx, j);
         if (partial) {
-          const int doc_j = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_k[j] : 0;
-          if (!keep_elem(a.mask, q_idx, j, doc_i, doc_j)) x = kNegInf;
+          const int doc_j = (mk.flags & FLEXATTN_MASK_DOC) ? mk.doc_k[j] : 0;
+          if (!keep_elem(mk, q_idx, j, doc_i, doc_j)) x = kNegInf;
         }
         tv[jj] = x;
         m_new = fmaxf(m_new, x);
@@ -175,6 +176,7 @@ __global__ __launch_bounds__(256) void bwd_dq_f32_kernel(BwdArgs a) {
   const int wg = blockIdx.x;
   const int bh = wg / nQ, qb = nQ - 1 - (wg % nQ);
   const int b = bh / a.Hq, h = bh % a.Hq, hk = h / (a.Hq / a.Hkv);
+  const MaskArgs mk = mask_of_batch(a.mask, b, a.Sq, a.Sk);
   const int tid = threadIdx.x, sub = tid & 3, r = tid >> 2;
   const int q_idx = qb * BQ + r;
   const size_t row = (size_t)bh * a.Sq + q_idx;
@@ -184,7 +186,7 @@ __global__ __launch_bounds__(256) void bwd_dq_f32_kernel(BwdArgs a) {
 
   ScoreMod<SCORE> sm;
   sm.init(a.score, a.sm_scale, h, b);
-  const int doc_i = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[q_idx] : 0;
+  const int doc_i = (mk.flags & FLEXATTN_MASK_DOC) ? mk.doc_q[q_idx] : 0;
 
   f32x4 qv[NV], dov[NV], acc[NV];
   load_slice<NV>(qv, static_cast<const float*>(a.q) + row * D, sub);
@@ -212,8 +214,8 @@ __global__ __launch_bounds__(256) void bwd_dq_f32_kernel(BwdArgs a) {
       const float tv = sm.to_log2(s, q_idx, j);  // (the score function's value: what its derivative is taken from)
       float x = tv + sm.bias2(q_idx, j);
       if (partial) {
-        const int doc_j = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_k[j] : 0;
-        if (!keep_elem(a.mask, q_idx, j, doc_i, doc_j)) x = kNegInf;
+        const int doc_j = (mk.flags & FLEXATTN_MASK_DOC) ? mk.doc_k[j] : 0;
+        if (!keep_elem(mk, q_idx, j, doc_i, doc_j)) x = kNegInf;
       }
       const float p = exp2f(x - lse2);
       const float gl = (x == kNegInf) ? 0.f : p * (dp - dl);   // gradient with respect to the logit (the bias's share)
@@ -242,6 +244,7 @@ __global__ __launch_bounds__(256) void bwd_dkv_f32_kernel(BwdArgs a) {
   const int wg = blockIdx.x;
   const int bhk = wg / nKb, kb = wg % nKb;
   const int b = bhk / a.Hkv, hk = bhk % a.Hkv;
+  const MaskArgs mk = mask_of_batch(a.mask, b, a.Sq, a.Sk);
   const int group = a.Hq / a.Hkv;
   const int tid = threadIdx.x, sub = tid & 3, r = tid >> 2;
   const int k_idx = kb * BK + r;
@@ -255,7 +258,7 @@ __global__ __launch_bounds__(256) void bwd_dkv_f32_kernel(BwdArgs a) {
     dk_acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
     dv_acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  const int doc_j = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_k[k_idx] : 0;
+  const int doc_j = (mk.flags & FLEXATTN_MASK_DOC) ? mk.doc_k[k_idx] : 0;
 
   const int n_tiles = a.map.cnt[kb];
   const int* tile_idx = a.map.idx + (size_t)kb * nQ;
@@ -293,8 +296,8 @@ __global__ __launch_bounds__(256) void bwd_dkv_f32_kernel(BwdArgs a) {
         const float tv = sm.to_log2(s, i, k_idx);
         float x = tv + sm.bias2(i, k_idx);
         if (partial) {
-          const int doc_i = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[i] : 0;
-          if (!keep_elem(a.mask, i, k_idx, doc_i, doc_j)) x = kNegInf;
+          const int doc_i = (mk.flags & FLEXATTN_MASK_DOC) ? mk.doc_q[i] : 0;
+          if (!keep_elem(mk, i, k_idx, doc_i, doc_j)) x = kNegInf;
         }
         const float p = exp2f(x - sLse[ii]);
         const float ds = (x == kNegInf) ? 0.f : p * (dp - sDl[ii]) * sm.dfactor(tv, s, i, k_idx);

@@ -79,6 +79,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_f32_mfma_kernel(FwdArgs a) {
   const int bh = wg / nO, ob = nO - 1 - (wg % nO);
   const int qb = ob / (BT / BO);
   const int b = bh / a.Hq, h = bh % a.Hq, hk = h / (a.Hq / a.Hkv);
+  const MaskArgs mk = mask_of_batch(a.mask, b, a.Sq, a.Sk);
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, l32 = lane & 31, half = lane >> 5;
   const int q_idx = ob * BO + l32;
 
@@ -88,8 +89,8 @@ __global__ __launch_bounds__(64 * NW) void fwd_f32_mfma_kernel(FwdArgs a) {
 
   ScoreMod<SCORE> sm;
   sm.init(a.score, a.sm_scale, h, b);
-  const bool has_doc = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
-  const int doc_i = has_doc ? a.mask.doc_q[q_idx] : 0;
+  const bool has_doc = (mk.flags & FLEXATTN_MASK_DOC) != 0;
+  const int doc_i = has_doc ? mk.doc_q[q_idx] : 0;
 
   f32x4 qf[D / 8];
   load_operand_row<D>(qf, Qg, half);
@@ -118,8 +119,8 @@ __global__ __launch_bounds__(64 * NW) void fwd_f32_mfma_kernel(FwdArgs a) {
         const int j = j0 + acc_row(i, half);
         float v = sm.to_log2(s[i], q_idx, j) + sm.bias2(q_idx, j);
         if (partial) {
-          const int doc_j = has_doc ? a.mask.doc_k[j] : 0;
-          if (!keep_elem(a.mask, q_idx, j, doc_i, doc_j)) v = kNegInf;
+          const int doc_j = has_doc ? mk.doc_k[j] : 0;
+          if (!keep_elem(mk, q_idx, j, doc_i, doc_j)) v = kNegInf;
         }
         x[i] = v;
         m_blk = fmaxf(m_blk, v);
@@ -223,6 +224,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_f32_mfma_kernel(BwdArgs a) {
   const int bh = wg / nO, ob = nO - 1 - (wg % nO);
   const int qb = ob / (BT / BO);
   const int b = bh / a.Hq, h = bh % a.Hq, hk = h / (a.Hq / a.Hkv);
+  const MaskArgs mk = mask_of_batch(a.mask, b, a.Sq, a.Sk);
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, l32 = lane & 31, half = lane >> 5;
   const int q_idx = ob * BO + l32;
   const size_t row = (size_t)bh * a.Sq + q_idx;
@@ -232,8 +234,8 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_f32_mfma_kernel(BwdArgs a) {
 
   ScoreMod<SCORE> sm;
   sm.init(a.score, a.sm_scale, h, b);
-  const bool has_doc = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
-  const int doc_i = has_doc ? a.mask.doc_q[q_idx] : 0;
+  const bool has_doc = (mk.flags & FLEXATTN_MASK_DOC) != 0;
+  const int doc_i = has_doc ? mk.doc_q[q_idx] : 0;
 
   f32x4 qf[D / 8], dof[D / 8];
   load_operand_row<D>(qf, static_cast<const float*>(a.q) + row * D, half);
@@ -263,8 +265,8 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_f32_mfma_kernel(BwdArgs a) {
         const float tv = sm.to_log2(s[i], q_idx, j);   // (the score function's value: what its derivative is taken from)
         float x = tv + sm.bias2(q_idx, j);
         if (partial) {
-          const int doc_j = has_doc ? a.mask.doc_k[j] : 0;
-          if (!keep_elem(a.mask, q_idx, j, doc_i, doc_j)) x = kNegInf;
+          const int doc_j = has_doc ? mk.doc_k[j] : 0;
+          if (!keep_elem(mk, q_idx, j, doc_i, doc_j)) x = kNegInf;
         }
         const float pe = exp2f(x - lse2);
         const float gl = (x == kNegInf) ? 0.f : pe * (dp[i] - dl);   // gradient with respect to the logit (the bias's share)
@@ -293,12 +295,13 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_f32_mfma_kernel(BwdArgs a) {
   const int bhk = wg / nO, ob = wg % nO;
   const int kb = ob / (BT / BO);
   const int b = bhk / a.Hkv, hk = bhk % a.Hkv, group = a.Hq / a.Hkv;
+  const MaskArgs mk = mask_of_batch(a.mask, b, a.Sq, a.Sk);
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, l32 = lane & 31, half = lane >> 5;
   const int k_idx = ob * BO + l32;
   const size_t krow = (size_t)bhk * a.Sk + k_idx;
 
-  const bool has_doc = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
-  const int doc_j = has_doc ? a.mask.doc_k[k_idx] : 0;
+  const bool has_doc = (mk.flags & FLEXATTN_MASK_DOC) != 0;
+  const int doc_j = has_doc ? mk.doc_k[k_idx] : 0;
   f32x4 kf[D / 8], vf[D / 8];
   load_operand_row<D>(kf, static_cast<const float*>(a.k) + krow * D, half);
   load_operand_row<D>(vf, static_cast<const float*>(a.v) + krow * D, half);
@@ -332,8 +335,8 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_f32_mfma_kernel(BwdArgs a) {
         const float tv = sm.to_log2(s[e], i, k_idx);
         float x = tv + sm.bias2(i, k_idx);
         if (partial) {
-          const int doc_i = has_doc ? a.mask.doc_q[i] : 0;
-          if (!keep_elem(a.mask, i, k_idx, doc_i, doc_j)) x = kNegInf;
+          const int doc_i = has_doc ? mk.doc_q[i] : 0;
+          if (!keep_elem(mk, i, k_idx, doc_i, doc_j)) x = kNegInf;
         }
         const float pe = exp2f(x - lse2_from(a.l[head_row + i], a.m[head_row + i]));
         pv[e] = pe;

@@ -70,19 +70,33 @@ __device__ __forceinline__ int tile_state(const MaskArgs& mk, int qb, int kb, in
 
 // Work-groups [0, nq) own one q-block row each: write its states and its ascending kv list.
 // Work-groups [nq, nq + nk) own one kv-block column each: write its ascending q list.
-__global__ __launch_bounds__(64) void block_mask_kernel(MaskArgs mk, int nq, int nk, int bq, int bk,
+// `batches`: number of batch entries the document arrays hold a row for (1: one row for all).  The map is then the
+// union over the entries: a tile runs if it runs for any entry and is full only if it is full for every entry (an
+// entry that keeps nothing of a tile it visits masks every element of it).
+__global__ __launch_bounds__(64) void block_mask_kernel(MaskArgs mk, int batches, int nq, int nk, int bq, int bk,
                                                         uint8_t* state, int* kv_cnt, int* kv_idx,
                                                         int* q_cnt, int* q_idx) {
   const int lane = threadIdx.x;
-  // Are the document ids non-decreasing on both sides?  Every work-group checks for itself (the arrays are
-  // a few KB): the block ends then bound a block's ids.
+  // Are the document ids non-decreasing on both sides (of every entry)?  Every work-group checks for itself (the
+  // arrays are a few KB): the block ends then bound a block's ids.
   bool sorted_ids = true;
   if (mk.flags & FLEXATTN_MASK_DOC) {
     bool ok = true;
-    for (int i = lane + 1; i < nq * bq; i += 64) ok = ok && (mk.doc_q[i - 1] <= mk.doc_q[i]);
-    for (int j = lane + 1; j < nk * bk; j += 64) ok = ok && (mk.doc_k[j - 1] <= mk.doc_k[j]);
+    for (int e = 0; e < batches; ++e) {
+      const MaskArgs me = mask_of_batch(mk, e, nq * bq, nk * bk);
+      for (int i = lane + 1; i < nq * bq; i += 64) ok = ok && (me.doc_q[i - 1] <= me.doc_q[i]);
+      for (int j = lane + 1; j < nk * bk; j += 64) ok = ok && (me.doc_k[j - 1] <= me.doc_k[j]);
+    }
     sorted_ids = __ballot(!ok) == 0ull;
   }
+  auto tile_state_all = [&](int qb, int kb) {
+    int st = tile_state(mk, qb, kb, bq, bk, sorted_ids);
+    for (int e = 1; e < batches; ++e) {
+      const int se = tile_state(mask_of_batch(mk, e, nq * bq, nk * bk), qb, kb, bq, bk, sorted_ids);
+      st = (st == 0 && se == 0) ? 0 : ((st == 2 && se == 2) ? 2 : 1);
+    }
+    return st;
+  };
   const bool is_row = (int)blockIdx.x < nq;
   const int major = is_row ? blockIdx.x : blockIdx.x - nq;
   const int n_minor = is_row ? nk : nq;
@@ -93,7 +107,7 @@ __global__ __launch_bounds__(64) void block_mask_kernel(MaskArgs mk, int nq, int
     const int minor = base + lane;
     int st = 0;
     if (minor < n_minor) {
-      st = is_row ? tile_state(mk, major, minor, bq, bk, sorted_ids) : tile_state(mk, minor, major, bq, bk, sorted_ids);
+      st = is_row ? tile_state_all(major, minor) : tile_state_all(minor, major);
       if (is_row) state[(size_t)major * nk + minor] = (uint8_t)st;
     }
     const unsigned long long ballot = __ballot(st != 0);
@@ -138,12 +152,12 @@ int build_ds_index(const uint8_t* state, const int* q_cnt, const int* q_idx, int
   return check_launch("flexattn_build_ds_index");
 }
 
-int build_block_mask(const MaskArgs& mask, int Sq, int Sk, int block_q, int block_k, uint8_t* state,
+int build_block_mask(const MaskArgs& mask, int doc_batches, int Sq, int Sk, int block_q, int block_k, uint8_t* state,
                      int* kv_cnt, int* kv_idx, int* q_cnt, int* q_idx, hipStream_t stream) {
   const int nq = Sq / block_q, nk = Sk / block_k;
   const bool want_cols = q_cnt != nullptr;
   const int grid = nq + (want_cols ? nk : 0);
-  hipLaunchKernelGGL(block_mask_kernel, dim3(grid), dim3(64), 0, stream, mask, nq, nk, block_q, block_k,
+  hipLaunchKernelGGL(block_mask_kernel, dim3(grid), dim3(64), 0, stream, mask, doc_batches > 1 ? doc_batches : 1, nq, nk, block_q, block_k,
                      state, kv_cnt, kv_idx, q_cnt, q_idx);
   return check_launch("flexattn_build_block_mask");
 }

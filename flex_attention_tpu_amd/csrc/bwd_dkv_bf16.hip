@@ -88,6 +88,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
   const int bhk = wg / nKb;
   const int kb = wg % nKb;  // low kv tiles have the most q tiles under causal masks: they go first
   const int b = bhk / a.Hkv;
+  const MaskArgs mk = mask_of_batch(a.mask, b, a.Sq, a.Sk);
   const int hk = bhk % a.Hkv;
   const int group = a.Hq / a.Hkv;
 
@@ -112,7 +113,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
     vreg[ks] = *reinterpret_cast<const bf16x8*>(Vg + (size_t)kv_local * D + ks * 16 + hh * 8);
   }
   int doc_j = 0;
-  if (a.mask.flags & FLEXATTN_MASK_DOC) doc_j = a.mask.doc_k[k_idx];
+  if (mk.flags & FLEXATTN_MASK_DOC) doc_j = mk.doc_k[k_idx];
 
   f32x16 dk_acc[4], dv_acc[4];
 #pragma unroll
@@ -234,7 +235,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
       bf16x8 pb[2], dsb[2];
       auto elementwise = [&](auto masked) {
         constexpr bool MASKED = decltype(masked)::value;
-        const bool has_doc = MASKED && (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
+        const bool has_doc = MASKED && (mk.flags & FLEXATTN_MASK_DOC) != 0;
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
           const int r0 = 32 * cc + 8 * g4 + 4 * hh;  // the lane's q rows come in runs of 4
@@ -242,7 +243,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
           const f32x4 dl4 = *reinterpret_cast<const f32x4*>(sDl + buf * BQ + r0);
           int di[4] = {0, 0, 0, 0};
           if (MASKED && has_doc) {
-            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_q + q0 + r0);
+            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(mk.doc_q + q0 + r0);
             di[0] = d4[0]; di[1] = d4[1]; di[2] = d4[2]; di[3] = d4[3];
           }
           float pv[4], dsv[4];
@@ -254,7 +255,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
             float pe = fast_exp2(tv + sm.bias2(i, k_idx) - lse4[u]);
             float gd = pe * (dp_acc[e] - dl4[u]) * sm.dfactor(tv, s_acc[e], i, k_idx);
             if (MASKED) {
-              const bool keep = keep_elem(a.mask, i, k_idx, di[u], doc_j);
+              const bool keep = keep_elem(mk, i, k_idx, di[u], doc_j);
               pe = keep ? pe : 0.f;
               gd = keep ? gd : 0.f;
             }
@@ -332,6 +333,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_wide_kernel(BwdArgs a) {
   const int bhk = wg / nKb;
   const int kb = wg % nKb;
   const int b = bhk / a.Hkv;
+  const MaskArgs mk = mask_of_batch(a.mask, b, a.Sq, a.Sk);
   const int hk = bhk % a.Hkv;
   const int group = a.Hq / a.Hkv;
 
@@ -356,7 +358,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_wide_kernel(BwdArgs a) {
     vreg[ks] = *reinterpret_cast<const bf16x8*>(Vg + (size_t)kv_local * D + ks * 16 + hh * 8);
   }
   int doc_j = 0;
-  if (a.mask.flags & FLEXATTN_MASK_DOC) doc_j = a.mask.doc_k[k_idx];
+  if (mk.flags & FLEXATTN_MASK_DOC) doc_j = mk.doc_k[k_idx];
 
   f32x16 dk_acc[4 * NP], dv_acc[4 * NP];
 #pragma unroll
@@ -467,7 +469,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_wide_kernel(BwdArgs a) {
       bf16x8 pb[2], dsb[2];
       auto elementwise = [&](auto masked) {
         constexpr bool MASKED = decltype(masked)::value;
-        const bool has_doc = MASKED && (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
+        const bool has_doc = MASKED && (mk.flags & FLEXATTN_MASK_DOC) != 0;
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
           const int r0 = 32 * c + 8 * g4 + 4 * hh;  // the lane's q rows come in runs of 4
@@ -475,7 +477,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_wide_kernel(BwdArgs a) {
           const f32x4 dl4 = *reinterpret_cast<const f32x4*>(sDl + buf * HQ + r0);
           int di[4] = {0, 0, 0, 0};
           if (MASKED && has_doc) {
-            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_q + q0 + r0);
+            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(mk.doc_q + q0 + r0);
             di[0] = d4[0]; di[1] = d4[1]; di[2] = d4[2]; di[3] = d4[3];
           }
           float pv[4], dsv[4];
@@ -487,7 +489,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_wide_kernel(BwdArgs a) {
             float pe = fast_exp2(tv + sm.bias2(i, k_idx) - lse4[u]);
             float gd = pe * (dp_acc[e] - dl4[u]) * sm.dfactor(tv, s_acc[e], i, k_idx);
             if (MASKED) {
-              const bool keep = keep_elem(a.mask, i, k_idx, di[u], doc_j);
+              const bool keep = keep_elem(mk, i, k_idx, di[u], doc_j);
               pe = keep ? pe : 0.f;
               gd = keep ? gd : 0.f;
             }
@@ -652,6 +654,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     return g;
   };
   auto kv_offset = [&](const Geometry& g) { return ((size_t)g.bhk * a.Sk + (size_t)g.kb * BNK) * D; };
+  // (DOCS) document arrays given per batch entry: the rows of the entry of a (batch, kv head) pair
+  auto doc_rows = [&](int bhk, int S) { return (DOCS && a.mask.doc_batched) ? (size_t)(bhk / a.Hkv) * (size_t)S : (size_t)0; };
   // (EXPORT) dS block of the item's kv tile against the first q tile of its list, for the group's first query
   // head: the blocks of a head are ordered kv tile by kv tile (a.ds_col[kb] pairs lie before kv tile kb), and
   // along each kv tile's q list
@@ -686,11 +690,12 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
     const bf16_t* Vg = static_cast<const bf16_t*>(a.v) + kv_offset(g);
     rows_load(r.k, Kg + (size_t)(tid_here >> 6) * 32 * D, tid_here & 63);
     rows_load(r.v, Vg + (size_t)(tid_here >> 6) * 32 * D, tid_here & 63);
-    r.doc = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_k[g.kb * BNK + kv_local] : 0;
+    const size_t dk_rows = doc_rows(g.bhk, a.Sk);
+    r.doc = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_k[dk_rows + g.kb * BNK + kv_local] : 0;
     if constexpr (DOCS) {
       const bool have = a.mask.doc_k_range != nullptr;
-      r.qlo = have ? a.mask.doc_k_range[2 * (g.kb * BNK + kv_local)] : 0;
-      r.qhi = have ? a.mask.doc_k_range[2 * (g.kb * BNK + kv_local) + 1] : 0;
+      r.qlo = have ? a.mask.doc_k_range[2 * (dk_rows + g.kb * BNK + kv_local)] : 0;
+      r.qhi = have ? a.mask.doc_k_range[2 * (dk_rows + g.kb * BNK + kv_local) + 1] : 0;
     }
     const int* tile_idx = a.map.idx + (size_t)g.kb * nQ;
     r.n_tiles = a.map.cnt[g.kb];
@@ -902,7 +907,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
           for (int half = 0; half < 2; ++half)
             km[half] = keep_bits32_range<false>(a.mask, k_idx, q0 + 64 * half + 4 * hh, cur.qlo, cur.qhi);
         } else {
-          stage_doc_ids(a.mask.doc_q, q0, q0 + 64, lane, sDoc);
+          stage_doc_ids(a.mask.doc_q + doc_rows(geo.bhk, a.Sq), q0, q0 + 64, lane, sDoc);
 #pragma unroll
           for (int half = 0; half < 2; ++half)
             km[half] = keep_bits32_staged<false>(a.mask, k_idx, q0 + 64 * half + 4 * hh, doc_j, sDoc + 64 * half + 4 * hh);

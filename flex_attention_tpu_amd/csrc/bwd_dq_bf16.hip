@@ -79,6 +79,7 @@ __global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void bwd_dq_bf16_kernel(BwdAr
   const int bh = wg / nQ;
   const int qb = nQ - 1 - (wg % nQ);
   const int b = bh / a.Hq;
+  const MaskArgs mk = mask_of_batch(a.mask, b, a.Sq, a.Sk);
   const int h = bh % a.Hq;
   const int hk = h / (a.Hq / a.Hkv);
 
@@ -116,7 +117,7 @@ __global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void bwd_dq_bf16_kernel(BwdAr
   const int* tile_idx = a.map.idx + (size_t)qb * nK;
   const uint8_t* tile_state = a.map.state + (size_t)qb * nK;
   int doc_i = 0;
-  if (a.mask.flags & FLEXATTN_MASK_DOC) doc_i = a.mask.doc_q[q_idx];
+  if (mk.flags & FLEXATTN_MASK_DOC) doc_i = mk.doc_q[q_idx];
   float* dab_row = a.dab != nullptr ? a.dab + row * (size_t)a.Sk : nullptr;  // this lane's row of the bias gradient
 
   f32x16 dq_acc[4 * NP];
@@ -218,13 +219,13 @@ __global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void bwd_dq_bf16_kernel(BwdAr
       bf16x8 ds[2];
       auto elementwise = [&](auto masked) {
         constexpr bool MASKED = decltype(masked)::value;
-        const bool has_doc = MASKED && (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
+        const bool has_doc = MASKED && (mk.flags & FLEXATTN_MASK_DOC) != 0;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const int j0 = kv0 + 32 * c + 8 * g + 4 * hh;
           int dj[4] = {0, 0, 0, 0};
           if (MASKED && has_doc) {
-            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_k + j0);
+            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(mk.doc_k + j0);
             dj[0] = d4[0]; dj[1] = d4[1]; dj[2] = d4[2]; dj[3] = d4[3];
           }
           float dsv[4];
@@ -237,7 +238,7 @@ __global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void bwd_dq_bf16_kernel(BwdAr
             float gl = pe * (dp_acc[e] - delta);
             float gd = gl * sm.dfactor(tv, s_acc[e], q_idx, j0 + u);
             if (MASKED) {   // (selected, not multiplied: a score function may return anything at a dropped element)
-              const bool keep = keep_elem(a.mask, q_idx, j0 + u, doc_i, dj[u]);
+              const bool keep = keep_elem(mk, q_idx, j0 + u, doc_i, dj[u]);
               gl = keep ? gl : 0.f;
               gd = keep ? gd : 0.f;
             }
@@ -378,6 +379,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
   };
   // (batch, kv head) pair of a (batch, q head) pair: bh / group, exact for the small numbers involved
   auto kv_pair = [&](int bh) { return group == 1 ? bh : (int)(((float)bh + 0.5f) * inv_group); };
+  // (DOCS) document arrays given per batch entry: the rows of the entry of a (batch, q head) pair
+  auto doc_rows = [&](int bh, int S) { return (DOCS && a.mask.doc_batched) ? (size_t)(bh / a.Hq) * (size_t)S : (size_t)0; };
   auto fetch = [&](int item, ItemRegs& r) {
     int bh, qb;
     geometry(item, bh, qb);
@@ -388,11 +391,12 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
     r.l = a.l[row];
     r.m = a.m[row];
     r.delta = a.delta[row];
-    r.doc = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[qb * BM + q_local] : 0;
+    const size_t dq_rows = doc_rows(bh, a.Sq);
+    r.doc = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[dq_rows + qb * BM + q_local] : 0;
     if constexpr (DOCS) {
       const bool have = a.mask.doc_q_range != nullptr;
-      r.klo = have ? a.mask.doc_q_range[2 * (qb * BM + q_local)] : 0;
-      r.khi = have ? a.mask.doc_q_range[2 * (qb * BM + q_local) + 1] : 0;
+      r.klo = have ? a.mask.doc_q_range[2 * (dq_rows + qb * BM + q_local)] : 0;
+      r.khi = have ? a.mask.doc_q_range[2 * (dq_rows + qb * BM + q_local) + 1] : 0;
     }
     r.n_tiles = a.map.cnt[qb];
     const int* tile_idx = a.map.idx + (size_t)qb * nK;
@@ -585,7 +589,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_bf16_d128_plain_kernel(BwdArgs 
         int* sDoc = reinterpret_cast<int*>(sSt + MAX_LIST) + w * 128;  // the wave's stage for document ids
         if ((a.mask.flags & FLEXATTN_MASK_DOC) && !ranged) {
           const int e1 = 2 * it_part + 1 < n_tiles ? 2 * it_part + 1 : 2 * it_part;
-          stage_doc_ids(a.mask.doc_k, __builtin_amdgcn_readfirstlane(sIdx[2 * it_part]) * BN,
+          stage_doc_ids(a.mask.doc_k + doc_rows(bh, a.Sk), __builtin_amdgcn_readfirstlane(sIdx[2 * it_part]) * BN,
                         __builtin_amdgcn_readfirstlane(sIdx[e1]) * BN, lane, sDoc);
         }
 #pragma unroll

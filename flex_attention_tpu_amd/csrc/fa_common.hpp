@@ -77,7 +77,22 @@ struct MaskArgs {
   // position's id form one interval: (first, last) per position, first > last if there is none; null = unknown.
   const int* doc_q_range;  // [Sq, 2]: kv positions with the id of q position i
   const int* doc_k_range;  // [Sk, 2]: q positions with the id of kv position j
+  // Nonzero: the four arrays hold one row per batch entry ([B, Sq], [B, Sk], [B, Sq, 2], [B, Sk, 2]); a kernel
+  // masks a batch entry with that entry's rows (mask_of_batch) and the block map is the union over the entries.
+  int doc_batched;
 };
+
+// The mask of batch entry b: the document arrays advanced to the entry's rows where they are given per entry.
+__host__ __device__ __forceinline__ MaskArgs mask_of_batch(const MaskArgs& m, int b, int Sq, int Sk) {
+  MaskArgs r = m;
+  if (m.doc_batched) {
+    r.doc_q += (size_t)b * Sq;
+    r.doc_k += (size_t)b * Sk;
+    if (r.doc_q_range != nullptr) r.doc_q_range += (size_t)b * Sq * 2;
+    if (r.doc_k_range != nullptr) r.doc_k_range += (size_t)b * Sk * 2;
+  }
+  return r;
+}
 // One direction of the block map: for "major" block r, idx[r*n_minor + t], t < cnt[r], are the
 // minor blocks to visit; state is always indexed [q block][kv block].
 struct MapArgs {

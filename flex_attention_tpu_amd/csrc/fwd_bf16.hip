@@ -80,6 +80,7 @@ __global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void fwd_bf16_kernel(FwdArgs 
   const int bh = wg / nQ;
   const int qb = nQ - 1 - (wg % nQ);  // longest rows first under causal masks
   const int b = bh / a.Hq;
+  const MaskArgs mk = mask_of_batch(a.mask, b, a.Sq, a.Sk);
   const int h = bh % a.Hq;
   const int hk = h / (a.Hq / a.Hkv);
 
@@ -111,7 +112,7 @@ __global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void fwd_bf16_kernel(FwdArgs 
   const uint8_t* tile_state = a.map.state + (size_t)qb * nK;
 
   int doc_i = 0;
-  if (a.mask.flags & FLEXATTN_MASK_DOC) doc_i = a.mask.doc_q[q_idx];
+  if (mk.flags & FLEXATTN_MASK_DOC) doc_i = mk.doc_q[q_idx];
 
   f32x16 o_acc[4 * NP];
 #pragma unroll
@@ -248,7 +249,7 @@ __global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void fwd_bf16_kernel(FwdArgs 
       }
     } else {
       // the lane's kv indices come in runs of 4: kv0 + 32c + 8g + 4hh + {0..3}
-      const bool has_doc = (a.mask.flags & FLEXATTN_MASK_DOC) != 0;
+      const bool has_doc = (mk.flags & FLEXATTN_MASK_DOC) != 0;
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
 #pragma unroll
@@ -256,14 +257,14 @@ __global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void fwd_bf16_kernel(FwdArgs 
           const int j0 = kv0 + 32 * c + 8 * g + 4 * hh;
           int dj[4] = {0, 0, 0, 0};
           if (has_doc) {
-            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(a.mask.doc_k + j0);
+            const auto d4 = *reinterpret_cast<const int __attribute__((ext_vector_type(4)))*>(mk.doc_k + j0);
             dj[0] = d4[0]; dj[1] = d4[1]; dj[2] = d4[2]; dj[3] = d4[3];
           }
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
             const int e = 4 * g + u;
             float tv = kPlain ? s_acc[c][e] : sm.to_log2(s_acc[c][e], q_idx, j0 + u) + sm.bias2(q_idx, j0 + u);
-            tv = keep_elem(a.mask, q_idx, j0 + u, doc_i, dj[u]) ? tv : kNegInf;
+            tv = keep_elem(mk, q_idx, j0 + u, doc_i, dj[u]) ? tv : kNegInf;
             s_acc[c][e] = tv;
             m_tile = fmaxf(m_tile, tv);
           }
@@ -459,9 +460,12 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
   };
   // (batch, kv head) pair of a (batch, q head) pair: bh / group, exact for the small numbers involved
   auto kv_pair = [&](int bh) { return group == 1 ? bh : (int)(((float)bh + 0.5f) * inv_group); };
+  // (DOCS) document arrays given per batch entry: the rows of the entry of a (batch, q head) pair
+  auto doc_rows = [&](int bh, int S) { return (DOCS && a.mask.doc_batched) ? (size_t)(bh / a.Hq) * (size_t)S : (size_t)0; };
   auto fetch = [&](int item, ItemRegs& r) {
     int bh, qb2;
     geometry(item, bh, qb2);
+    const size_t dq_rows = doc_rows(bh, a.Sq);
     const int tid_here = opaque(tid);
     const int lane_here = tid_here & 63;
     const int row_here = (tid_here >> 6) * 32 + (lane_here & 31);
@@ -471,11 +475,11 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
     for (int x = 0; x < 2; ++x) {
       const int qb = min(2 * qb2 + x, nQ - 1);  // (a missing second tile repeats the first; nothing of it is stored)
       rows_load(r.q[x], static_cast<const bf16_t*>(a.q) + ((size_t)bh * a.Sq + (size_t)qb * BM + w_here * 32) * D, lane_here);
-      r.doc[x] = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[qb * BM + row_here] : 0;
+      r.doc[x] = (a.mask.flags & FLEXATTN_MASK_DOC) ? a.mask.doc_q[dq_rows + qb * BM + row_here] : 0;
       if constexpr (DOCS) {
         const bool ranged = a.mask.doc_q_range != nullptr;
-        r.klo[x] = ranged ? a.mask.doc_q_range[2 * (qb * BM + row_here)] : 0;
-        r.khi[x] = ranged ? a.mask.doc_q_range[2 * (qb * BM + row_here) + 1] : 0;
+        r.klo[x] = ranged ? a.mask.doc_q_range[2 * (dq_rows + qb * BM + row_here)] : 0;
+        r.khi[x] = ranged ? a.mask.doc_q_range[2 * (dq_rows + qb * BM + row_here) + 1] : 0;
       }
       const uint8_t* row = a.map.state + (size_t)qb * nK;
       const bool valid = 2 * qb2 + x < nQ;
@@ -682,7 +686,7 @@ __global__ __launch_bounds__(256, 1) void fwd_bf16_d128_plain_kernel(FwdArgs a) 
         int* sDoc = reinterpret_cast<int*>(sStB + MAX_LIST) + w * 128;  // the wave's stage for document ids
         if constexpr (DOCS) {
           if (!ranged)
-            stage_doc_ids(a.mask.doc_k, __builtin_amdgcn_readfirstlane(entry(2 * it)) * BN,
+            stage_doc_ids(a.mask.doc_k + doc_rows(bh, a.Sk), __builtin_amdgcn_readfirstlane(entry(2 * it)) * BN,
                           __builtin_amdgcn_readfirstlane(entry(2 * it + 1)) * BN, lane, sDoc);
         }
 #pragma unroll

@@ -38,7 +38,8 @@ int bwd_dkv_f32_mfma(const BwdArgs& a, int D, hipStream_t stream);
 
 int bwd_delta(const void* o, const void* dout, float* delta, int64_t rows, int D, int dtype, hipStream_t stream);
 
-int build_block_mask(const MaskArgs& mask, int Sq, int Sk, int block_q, int block_k, uint8_t* state,
+// (doc_batches: batch entries the mask's document arrays hold a row for; the map is the union over them)
+int build_block_mask(const MaskArgs& mask, int doc_batches, int Sq, int Sk, int block_q, int block_k, uint8_t* state,
                      int* kv_cnt, int* kv_idx, int* q_cnt, int* q_idx, hipStream_t stream);
 
 int build_ds_index(const uint8_t* state, const int* q_cnt, const int* q_idx, int nq, int nk, int* col, int* rank,

@@ -8,8 +8,8 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (on_device, batch_entry, bias_c, check_blocks, check_qkv, check_rows, kernel_block_map, kernel_head_dim, library_for, pad_seq,
-                      padded_len, per_batch_segments, resolve_mask, stream_of)
+from ._common import (on_device, bias_c, check_blocks, check_doc_batches, check_qkv, check_rows, kernel_block_map, kernel_head_dim, library_for, pad_seq,
+                      padded_len, resolve_mask, stream_of)
 from .flex_attention_dq_bwd import DsBlocks, alloc_ds, bwd_params
 
 
@@ -25,19 +25,6 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     biases, ``ab``, compiled score functions) or the device has too little free memory for the buffer (one 32 KB
     block per query head and kept pair of 128 x 128 tiles): the dq pass then recomputes as usual."""
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v, do)
-    rows = per_batch_segments(segment_ids, B)
-    if rows is not None and _defer:
-        return None
-    if rows is not None:  # ids differ between batch entries: one launch per entry
-        outs = [flash_attention_bwd_dkv(
-            k[b:b + 1], v[b:b + 1], q[b:b + 1], batch_entry(ab, b), rows[b], l[b:b + 1], m[b:b + 1], di[b:b + 1], do[b:b + 1],
-            block_b=block_b, block_q=block_q, block_q_major=block_q_major, block_k_major=block_k_major, block_k=block_k,
-            sm_scale=sm_scale, causal=causal, debug=debug, score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn,
-            compiled_loop=compiled_loop, return_ds=return_ds) for b in range(B)]
-        dk, dv = torch.cat([x[0] for x in outs], 0), torch.cat([x[1] for x in outs], 0)
-        if not return_ds:
-            return dk, dv
-        return dk, dv, (DsBlocks(entries=[x[2] for x in outs]) if all(x[2] is not None for x in outs) else None)
     for name, t in (("l", l), ("m", m), ("di", di)):
         check_rows(name, t, B, Hq, Sq, q.device)
     check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k,
@@ -45,6 +32,7 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     # ragged lengths: zero-padded to the kernels' tiles (padded rows carry l = 0 and dO = 0: they add nothing)
     Sq_p, Sk_p = padded_len(Sq), padded_len(Sk)
     spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk, Sq_p, Sk_p)
+    check_doc_batches(spec, B)   # (ids of shape [B, S]: the kernels mask every batch entry by its own row)
     q, do, k, v = pad_seq(q, Sq_p), pad_seq(do, Sq_p), pad_seq(k, Sk_p), pad_seq(v, Sk_p)
     l, m, di = pad_seq(l, Sq_p), pad_seq(m, Sq_p), pad_seq(di, Sq_p)
     D_user, D = D, kernel_head_dim(D, q.dtype)   # smaller head dimensions: zero-padded columns

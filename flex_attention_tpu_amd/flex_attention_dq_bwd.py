@@ -7,8 +7,8 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (on_device, batch_entry, bias_c, check_blocks, check_qkv, check_rows, dtype_code, kernel_block_map, kernel_head_dim, library_for,
-                      pad_seq, padded_len, per_batch_segments, resolve_mask, score_spec_c, stream_of)
+from ._common import (on_device, bias_c, check_blocks, check_doc_batches, check_qkv, check_rows, dtype_code, kernel_block_map, kernel_head_dim, library_for,
+                      pad_seq, padded_len, resolve_mask, score_spec_c, stream_of)
 from .block_mask import mask_spec_c
 
 
@@ -36,8 +36,8 @@ class DsBlocks:
     The reference's two backward kernels each recompute S, dP and dS (flex_attention_dq_bwd.py:340-378,
     flash_attention_dkv_bwd.py:232-302); handing dS over leaves the dq pass one contraction instead of three."""
 
-    def __init__(self, buf=None, shape=None, entries=None, index=None):
-        self.buf, self.shape, self.entries, self.index = buf, shape, entries, index
+    def __init__(self, buf=None, shape=None, index=None):
+        self.buf, self.shape, self.index = buf, shape, index
 
 
 # The dS buffer is never allowed to take more than this share of the device's memory, and an out-of-memory error of
@@ -112,30 +112,6 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     reference declares next to dk, dv (flash_attention_dkv_bwd.py:103-107,130-138) and its upstream dq kernel
     writes (jax_exp.py:1252-1255; there multiplied by sm_scale)."""
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v, do)
-    rows = per_batch_segments(segment_ids, B)
-    if rows is not None:  # ids differ between batch entries: one launch per entry
-        if ds is not None and (ds.entries is None or len(ds.entries) != B):
-            raise ValueError("ds does not come from a dk/dv pass of these arguments")
-        if return_dab and (ab is None or ds is not None or return_delta):
-            raise ValueError("return_dab needs the additive bias `ab` and excludes `ds` and return_delta")
-        if _defer:
-            return None
-        if d is None:
-            d = compute_delta(o, do)
-        parts = [flex_attention_bwd_dq(
-            q[b:b + 1], k[b:b + 1], v[b:b + 1], batch_entry(ab, b), rows[b], l[b:b + 1], m[b:b + 1], batch_entry(o, b),
-            do[b:b + 1], d[b:b + 1], block_b=block_b, block_q=block_q, block_k_major=block_k_major, block_k=block_k,
-            sm_scale=sm_scale, debug=debug, score_fn=score_fn, mask_fn=mask_fn, block_mask_fn=block_mask_fn, causal=causal,
-            compiled_loop=compiled_loop, ds=ds.entries[b] if ds is not None else None, return_dab=return_dab)
-            for b in range(B)]
-        if return_dab:
-            # a bias shared by the batch entries collects the sum of their gradients (added in float32; the
-            # entries' own planes were rounded to the bias's dtype once already)
-            dabs = [x[1] for x in parts]
-            dab = torch.cat(dabs, 0) if ab.shape[0] != 1 else torch.stack([x.float() for x in dabs]).sum(0).to(ab.dtype)
-            return torch.cat([x[0] for x in parts], 0), dab
-        out = torch.cat(parts, 0)
-        return (out, d) if return_delta else out
     if o is not None and tuple(o.shape) != tuple(q.shape):
         raise ValueError(f"o has shape {tuple(o.shape)}, expected {tuple(q.shape)}")
     fuse_delta = d is None
@@ -151,6 +127,7 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     # ragged lengths: zero-padded to the kernels' tiles (padded rows carry l = 0: their probabilities vanish)
     Sq_p, Sk_p = padded_len(Sq), padded_len(Sk)
     spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk, Sq_p, Sk_p)
+    check_doc_batches(spec, B)   # (ids of shape [B, S]: the kernels mask every batch entry by its own row)
     q, do, k, v = pad_seq(q, Sq_p), pad_seq(do, Sq_p), pad_seq(k, Sk_p), pad_seq(v, Sk_p)
     l, m, d_p = pad_seq(l, Sq_p), pad_seq(m, Sq_p), pad_seq(d, Sq_p)
     D_user, D = D, kernel_head_dim(D, q.dtype)   # smaller head dimensions: zero-padded columns

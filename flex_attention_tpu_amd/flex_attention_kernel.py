@@ -12,8 +12,8 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._common import (on_device, batch_entry, bias_c, check_blocks, check_qkv, dtype_code, kernel_block_map, kernel_head_dim, library_for, pad_seq,
-                      padded_len, per_batch_segments, resolve_mask, score_spec_c, stream_of)
+from ._common import (on_device, bias_c, check_blocks, check_doc_batches, check_qkv, dtype_code, kernel_block_map, kernel_head_dim, library_for, pad_seq,
+                      padded_len, resolve_mask, score_spec_c, stream_of)
 from .block_mask import mask_spec_c
 
 
@@ -30,18 +30,11 @@ def _flex_attention_impl(q, k, v, ab, segment_ids, save_residuals, causal, sm_sc
     """
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v)
     check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k)
-    rows = per_batch_segments(segment_ids, B)
-    if rows is not None:  # ids differ between batch entries: one launch per entry
-        outs = [_flex_attention_impl(q[b:b + 1], k[b:b + 1], v[b:b + 1], batch_entry(ab, b), rows[b], save_residuals, causal,
-                                     sm_scale, block_b, block_q, block_k_major, block_k, debug, block_mask_fn, mask_fn,
-                                     score_fn, compiled_loop=compiled_loop) for b in range(B)]
-        if not save_residuals:
-            return torch.cat(outs, 0)
-        return tuple(torch.cat([o[i] for o in outs], 0) for i in range(3))
     # ragged lengths: the tensors are zero-padded to the kernels' tiles, a key bound drops the padded keys
     # and the padded query rows are cut off again
     Sq_p, Sk_p = padded_len(Sq), padded_len(Sk)
     spec = resolve_mask(mask_fn, block_mask_fn, causal, segment_ids, Sq, Sk, Sq_p, Sk_p)
+    check_doc_batches(spec, B)   # (ids of shape [B, S]: the kernels mask every batch entry by its own row)
     q, k, v = pad_seq(q, Sq_p), pad_seq(k, Sk_p), pad_seq(v, Sk_p)
     D_user, D = D, kernel_head_dim(D, q.dtype)   # smaller head dimensions: zero-padded columns
     q, k, v = pad_seq(q, D, 3), pad_seq(k, D, 3), pad_seq(v, D, 3)

@@ -21,15 +21,30 @@ from . import _lib
 
 
 class DocIds:
-    """Immutable per-position document ids (int32) with a precomputed hash."""
+    """Immutable per-position document ids (int32) with a precomputed hash: one row [S] for every batch entry, or
+    one row per entry, [B, S] (the reference's segment ids of shape [B, S], mha_reference.py:65-73)."""
     __slots__ = ("array", "_key", "_hash")
 
     def __init__(self, ids):
         arr = np.ascontiguousarray(np.asarray(ids, dtype=np.int32))
+        if arr.ndim not in (1, 2):
+            raise ValueError("document ids must be a 1-D (or [B, S]) array")
         arr.setflags(write=False)
         self.array = arr
-        self._key = arr.tobytes()
+        self._key = (arr.shape, arr.tobytes())
         self._hash = hash(self._key)
+
+    @property
+    def batches(self) -> int:
+        """Rows of ids: 1 when all batch entries share them."""
+        return 1 if self.array.ndim == 1 else self.array.shape[0]
+
+    def rows(self, B: int) -> np.ndarray:
+        """The ids as [B, S] (a shared row repeated)."""
+        a = self.array if self.array.ndim == 2 else self.array[None, :]
+        if a.shape[0] not in (1, B):
+            raise ValueError(f"document ids have {a.shape[0]} rows for a batch of {B}")
+        return np.ascontiguousarray(np.broadcast_to(a, (B, a.shape[1])))
 
     def __hash__(self):
         return self._hash
@@ -38,22 +53,31 @@ class DocIds:
         return isinstance(other, DocIds) and self._key == other._key
 
     def __len__(self):
-        return self.array.shape[0]
+        return self.array.shape[-1]
 
     def is_sorted(self) -> bool:
-        """Whether the ids are non-decreasing along the sequence (the reference's jagged mask: masks.py:88-103)."""
+        """Whether the ids are non-decreasing along the sequence (the reference's jagged mask: masks.py:88-103),
+        in every row."""
         a = self.array
-        return bool(a.shape[0] < 2 or (a[1:] >= a[:-1]).all())
+        return bool(a.shape[-1] < 2 or (a[..., 1:] >= a[..., :-1]).all())
 
     def ranges_in(self, other: "DocIds"):
-        """int32 [len(self), 2]: for every position of this array the first and last position of ``other`` that
-        carries the same id (first > last where there is none), or None when ``other`` is not sorted (the positions
-        then form no interval).  The kernels mask partial tiles of a document mask from these bounds."""
+        """int32 [len(self), 2] (with rows per batch entry on either side: [B, len(self), 2]): for every position of
+        this array the first and last position of ``other`` (of the same batch entry) that carries the same id
+        (first > last where there is none), or None when ``other`` is not sorted (the positions then form no
+        interval).  The kernels mask partial tiles of a document mask from these bounds."""
         if not other.is_sorted():
             return None
-        lo = np.searchsorted(other.array, self.array, side="left")
-        hi = np.searchsorted(other.array, self.array, side="right") - 1
-        return np.ascontiguousarray(np.stack([lo, hi], axis=1).astype(np.int32))
+
+        def one(mine, theirs):
+            lo = np.searchsorted(theirs, mine, side="left")
+            hi = np.searchsorted(theirs, mine, side="right") - 1
+            return np.stack([lo, hi], axis=1).astype(np.int32)
+        if self.batches == 1 and other.batches == 1:
+            return np.ascontiguousarray(one(self.array.reshape(-1), other.array.reshape(-1)))
+        B = max(self.batches, other.batches)
+        mine, theirs = self.rows(B), other.rows(B)
+        return np.ascontiguousarray(np.stack([one(mine[b], theirs[b]) for b in range(B)], axis=0))
 
 
 @dataclass(frozen=True)

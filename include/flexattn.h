@@ -72,7 +72,11 @@ typedef struct flexattn_mask_spec {
   int32_t flags;
   int32_t window;
   int32_t stride;
-  int32_t reserved;
+  /* DOC: 0 or 1: the arrays below hold one row, shared by all batch entries.  B (the call's batch size): they hold
+   * one row per batch entry, [B, Sq], [B, Sk], [B, Sq, 2], [B, Sk, 2] (the reference's segment ids of shape [B, S],
+   * mha_reference.py:65-73): every entry is masked by its own row; the block map built from such a specification is
+   * the union over the entries (a tile runs if it runs for any entry). */
+  int32_t doc_batches;
   const int32_t* doc_q; /* DOC: device int32 [Sq]: any ids (they need not be sorted) */
   const int32_t* doc_k; /* DOC: device int32 [Sk] (may equal doc_q) */
   /* DOC, optional (NULL = not known): where the ids of the OTHER side are non-decreasing, the positions there that

@@ -381,12 +381,75 @@ def test_segment_ids_per_batch_entry(F, dtype):
     ma = O.mha_bwd_reference(q, k, v, o.float().cpu(), do, l.cpu(), m.cpu(), **okw)
     for name, t, r in (("dq", dq, ma[0]), ("dk", dk, ma[1]), ("dv", dv, ma[2])):
         assert_close(name, t, r, dtype)
-    # (the dS exchange goes entry by entry as well)
+    # (the dS exchange works from the union map as well)
     d = F.compute_delta(o, dog)
     dqx = _exchanged_dq(F, qg, kg, vg, l, m, o, dog, d, sc, None, None, None, dk, dv, expect=dtype == torch.bfloat16,
                         causal=True, sid=sid)
     if dqx is not None:
         assert_close("exchange dq", dqx, ma[0], dtype)
+
+
+@pytest.mark.parametrize("ids_kind", ["sorted", "one_entry_unsorted", "q_and_kv_differ"])
+def test_segment_ids_per_batch_entry_on_the_persistent_schedule(F, ids_kind):
+    """Rows of ids that differ between the batch entries at a size where the stream kernels run their persistent
+    longest-first schedule (B=8, 16 q heads on 8 kv heads, S=1024: 512 forward items): one launch per pass, every
+    entry masked by its own row (the kernels step through the id arrays with a batch stride), the block map the
+    union over the entries.  Entry 0 is one document, entry 1 many short ones (most tiles it visits keep nothing
+    of it), entry 2 documents that end inside tiles, entry 3 the first again, entries 4-7 the same in another order.  `one_entry_unsorted`: ids that
+    recur, so the kernels compare staged ids instead of intervals; `q_and_kv_differ`: an object with .q / .kv.
+    Against the oracle, the block map against the union of the entries' brute-force maps, and every entry against
+    the same entry launched alone with its own row of ids and its own map: bit for bit (the tiles the union adds
+    to an entry's lists keep nothing of it and add exact zeros)."""
+    import types
+    from flex_attention_tpu_amd import _common, block_mask
+    sc = 1 / math.sqrt(128)
+    B, Hq, Hkv, S = 8, 16, 8, 1024
+    rows = [O.doc_ids_from_lengths(x) for x in ([1024], [60] * 17 + [4], [300, 212, 500, 12], [1024])]
+    if ids_kind == "one_entry_unsorted":
+        rows[2] = torch.arange(S) // 96 % 3            # ids 0, 1, 2, 0, 1, 2, ... in runs of 96
+    rows = rows + [rows[2], rows[0], rows[1], rows[2]]
+    sid = torch.stack([r.to(torch.int32) for r in rows])
+    sid_arg = sid
+    causal = ids_kind != "q_and_kv_differ"
+    if not causal:   # (no causal term: the documents of the kv side begin elsewhere, every q id occurs among them;
+        # one q head per kv head: without the causal term a key's gradient sums several times the terms)
+        Hkv = Hq
+        sid_kv = sid.clone()
+        sid_kv[1] = sid_kv[6] = O.doc_ids_from_lengths([30] * 17 + [514])
+        sid_kv[2] = sid_kv[4] = sid_kv[7] = O.doc_ids_from_lengths([500, 12, 212, 300])
+        sid_arg = types.SimpleNamespace(q=sid, kv=sid_kv)
+    q, k, v, do = O.make_inputs(B, Hq, Hkv, S, S, 128, dtype=torch.bfloat16, seed=139)
+    if not causal:
+        keep = sid[:, :, None] == sid_kv[:, None, :]
+        okw = dict(sm_scale=sc, mask=keep)
+    else:
+        keep = (sid[:, :, None] == sid[:, None, :]) & (torch.arange(S)[:, None] >= torch.arange(S)[None, :])
+        okw = dict(sm_scale=sc, causal=True, segment_ids=sid)
+    ro, rl, rm = O.mha_reference(q, k, v, save_residuals=True, compute_dtype=torch.float32, **okw)
+    qg, kg, vg, dog = [x.to(DEV) for x in (q, k, v, do)]
+    o, l, m, dq, dk, dv = _all_passes_with(F, qg, kg, vg, dog, None, sid_arg, sc, None, None, causal)
+    rows_kept = keep.any(-1)                              # (a query without a key has no defined output)
+    rk = rows_kept[:, None, :, None]
+    assert_close("o", torch.where(rk.to(DEV), o, torch.zeros_like(o)), torch.where(rk, ro, torch.zeros_like(ro)), torch.bfloat16)
+    ma = O.mha_bwd_reference(q, k, v, o.float().cpu(), do, l.cpu(), m.cpu(), compute_dtype=torch.float32, **okw)
+    for name, t, r in (("dq", dq, ma[0]), ("dk", dk, ma[1]), ("dv", dv, ma[2])):
+        assert_close(name, t, r, torch.bfloat16)
+    # the map: the union of the entries' maps
+    spec = _common.resolve_mask(None, None, causal, sid_arg, S, S)
+    bm = block_mask.build_block_map(spec, S, S, 128, 64, DEV)
+    brute = torch.stack([O.block_map_bruteforce(keep[b], 128, 64) for b in range(B)])
+    union = torch.where((brute == 0).all(0), 0, torch.where((brute == 2).all(0), 2, 1))
+    st = bm.state.cpu()
+    if ids_kind == "sorted":
+        assert torch.equal(st.to(union.dtype), union)
+    else:   # (ids that recur: the builder may keep a tile that holds no pair, never the other way round)
+        assert bool(((st == 0) <= (union == 0)).all()) and bool(((st == 2) <= (union == 2)).all())
+    # every entry alone (its own row of ids, its own map)
+    for b in range(B):
+        one = sid[b] if causal else types.SimpleNamespace(q=sid[b], kv=sid_kv[b])
+        part = _all_passes_with(F, *[x[b:b + 1].contiguous() for x in (qg, kg, vg, dog)], None, one, sc, None, None, causal)
+        for name, t, r in zip(("o", "l", "m", "dq", "dk", "dv"), part, (o, l, m, dq, dk, dv)):
+            assert torch.equal(t[0], r[b]), f"{name} of entry {b} alone: {int((t[0] != r[b]).sum())} elements differ"
 
 
 @pytest.mark.parametrize("D,dtype", [(64, torch.bfloat16), (96, torch.bfloat16), (32, torch.float32), (80, torch.float32)],

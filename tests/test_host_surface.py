@@ -138,7 +138,7 @@ def test_entry_points_validate_arguments_without_gpu():
     with pytest.raises(ValueError, match="GPU"):
         F._flex_attention_impl(q, q, q, None, None, False, False, 1.0, 1, 128, 128, 128, False, None, None, None)
     # the additive bias is checked against the shapes of q and k before anything is launched
-    from flex_attention_tpu_amd._common import bias_c, per_batch_segments
+    from flex_attention_tpu_amd._common import bias_c, check_doc_batches, resolve_mask, segment_doc_ids
     for bad in (torch.zeros(1, 2, 128, 64), torch.zeros(3, 2, 128, 128), torch.zeros(2, 128, 128)):
         with pytest.raises(ValueError, match="ab"):
             bias_c(bad, 1, 2, 128, 128, 128, 128, torch.device("cpu"))
@@ -146,13 +146,21 @@ def test_entry_points_validate_arguments_without_gpu():
         bias_c(torch.zeros(1, 2, 128, 128, dtype=torch.float16), 1, 2, 128, 128, 128, 128, torch.device("cpu"))
     c, keep = bias_c(torch.zeros(1, 1, 100, 120), 2, 2, 100, 120, 128, 128, torch.device("cpu"))
     assert tuple(keep.shape) == (1, 1, 128, 128) and c.stride_b == 0 and c.stride_h == 0 and c.ptr == keep.data_ptr()
-    # segment ids per batch entry: split only when the rows differ
+    # segment ids per batch entry: equal rows collapse into one, rows that differ stay rows of the specification
+    # (the kernels take them with a batch stride), ragged lengths pad every row, and the rows must match the batch
     same = torch.zeros(2, 128, dtype=torch.int32)
-    assert per_batch_segments(same, 2) is None and per_batch_segments(None, 2) is None
-    rows = per_batch_segments(torch.stack([torch.zeros(128), torch.ones(128)]), 2)
-    assert len(rows) == 2 and int(rows[1][0]) == 1
+    assert segment_doc_ids(same)[0].batches == 1
+    ids = torch.stack([torch.zeros(100), torch.cat([torch.zeros(40), torch.ones(60)])]).to(torch.int32)
+    dq, dk = segment_doc_ids(ids)
+    assert dq.batches == 2 and dk is None and len(dq) == 100 and dq.is_sorted()
+    r = dq.ranges_in(dq)
+    assert r.shape == (2, 100, 2) and r[0, 5].tolist() == [0, 99] and r[1, 5].tolist() == [0, 39] and r[1, 50].tolist() == [40, 99]
+    spec = resolve_mask(None, None, True, ids, 100, 100, 128, 128)
+    assert spec.doc_ids.array.shape == (2, 128) and spec.doc_ids_k.array.shape == (2, 128)
+    assert spec.doc_ids.array[1, -1] == 1 and (spec.doc_ids_k.array[:, 100:] == 2).all()   # padded keys: an id of their own
+    check_doc_batches(spec, 2)
     with pytest.raises(ValueError, match="rows"):
-        per_batch_segments(torch.zeros(3, 128), 2)
+        check_doc_batches(spec, 3)
     with pytest.raises(NotImplementedError):
         block_mask.spec_of(lambda a, b: a[:, None] >= b[None, :], None)
     from flex_attention_tpu_amd._common import check_blocks, score_spec_c
