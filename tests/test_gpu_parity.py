@@ -1049,6 +1049,10 @@ def test_entry_points_reject_bad_arguments_on_gpu(F):
     q = torch.zeros(1, 2, 256, 128, dtype=torch.float16, device=DEV)
     with pytest.raises(NotImplementedError):
         F._flex_attention_impl(q, q, q, None, None, False, False, 1.0, 1, 128, 128, 128, False, None, None, None)
+    q = torch.zeros(2, 2, 256, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError, match="rows"):  # ids per batch entry: one row for every entry of the call
+        F._flex_attention_impl(q, q, q, None, torch.arange(3)[:, None].expand(3, 256), False, False, 1.0, 1, 128, 128, 128,
+                               False, None, None, None)
 
 
 # ------------------------------------------------------------------------------------------------

@@ -14,6 +14,8 @@ only reaches sampled rows and single heads: every output element of the full lau
   against the persistent schedule); under a causal mask the first half of the tokens alone gives the first half of
   o, l, m and dq.
 * Grouped kv heads give, per query head, the bits of the same call with the kv heads repeated.
+* Segment ids with a row per batch entry: permuting the entries together with their rows permutes the outputs, and
+  an entry launched alone with its row gives its bits of the batch.
 """
 import pytest
 import torch
@@ -281,3 +283,53 @@ def test_grouped_kv_heads_equal_repeated_kv_heads(F, D, n_cases, seed):
             ys = y.float().view(B, Hkv, g, S, D).sum(2)
             rel = float((x.float() - ys).norm() / (ys.norm() + 1e-9))
             assert rel <= 6e-3, f"{tag}: {name} of the group against the sum over repeated heads: rel-L2 {rel:.2e}"
+
+
+def test_segment_ids_per_batch_entry_properties(F):
+    """Rows of segment ids that differ between the batch entries, at 4096 tokens (B=4, 16 q heads on 4 kv heads,
+    softcap scores, random documents per entry, one entry with ids that recur): one launch per pass on the union
+    map.  Determinism, equivariance under a permutation of the entries with their rows, and every entry alone
+    with its own row and its own map: bit for bit, all outputs and the dq from handed-over dS."""
+    import math
+    import random
+    import warnings
+    from flex_attention_tpu_amd import scores
+    warnings.filterwarnings("ignore", message="score_fn with sm_scale")
+    B, Hq, Hkv, S, D = 4, 16, 4, 4096, 128
+    rng = random.Random(31)
+    rows = []
+    for b in range(B):
+        lens, left = [], S
+        while left > 0:
+            lens.append(min(left, rng.randint(1, 1500)))
+            left -= lens[-1]
+        ids = torch.repeat_interleave(torch.arange(len(lens)), torch.tensor(lens))
+        rows.append(ids % 3 if b == 2 else ids)      # (entry 2: ids recur, no intervals)
+    sid = torch.stack(rows).to(torch.int32)
+    gen = torch.Generator().manual_seed(9000)
+    q, k, v, do = [torch.randn(B, h, S, D, generator=gen).to(torch.bfloat16).to(DEV) for h in (Hq, Hkv, Hkv, Hq)]
+    sc, sfn = 1 / math.sqrt(D), scores.make_softcap_score_fn(30.0)
+
+    def passes(q, k, v, do, sid):
+        o, l, m = F._flex_attention_impl(q, k, v, None, sid, True, True, sc, 1, 128, 128, 128, False, None, None, sfn)
+        d = F.compute_delta(o, do)
+        kw = dict(sm_scale=sc, debug=False, score_fn=sfn, causal=True)
+        dq = F.flex_attention_bwd_dq(q, k, v, None, sid, l, m, o, do, d, block_b=1, block_q=128, block_k_major=128, block_k=128, **kw)
+        dk, dv, ds = F.flash_attention_bwd_dkv(k, v, q, None, sid, l, m, d, do, block_b=1, block_q=128, block_q_major=128,
+                                               block_k_major=128, block_k=128, return_ds=True, **kw)
+        assert ds is not None
+        dqx = F.flex_attention_bwd_dq(q, k, v, None, sid, l, m, o, do, d, block_b=1, block_q=128, block_k_major=128,
+                                      block_k=128, ds=ds, **kw)
+        return o, l, m, dq, dk, dv, dqx
+    names = ("o", "l", "m", "dq", "dk", "dv", "dq from dS")
+    full = passes(q, k, v, do, sid)
+    for n, a, b_ in zip(names, passes(q, k, v, do, sid), full):
+        _same(f"{n} of a second run", a, b_)
+    pb = torch.tensor([2, 0, 3, 1])
+    perm = passes(*[x[pb.to(DEV)].contiguous() for x in (q, k, v, do)], sid[pb])
+    for n, a, b_ in zip(names, perm, full):
+        _same(f"{n} under a permutation of the batch entries and their rows of ids", a, b_[pb.to(DEV)])
+    for b in range(B):
+        part = passes(*[x[b:b + 1].contiguous() for x in (q, k, v, do)], sid[b])
+        for n, a, b_ in zip(names, part, full):
+            _same(f"{n} of entry {b} alone", a, b_[b:b + 1])
