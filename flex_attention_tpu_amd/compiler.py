@@ -43,7 +43,7 @@ import torch
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 JIT_DIR = os.path.join(PKG_DIR, "_jit")
-CODEGEN_VERSION = 1
+CODEGEN_VERSION = 2
 
 
 # ------------------------------------------------------------------------------------------------
@@ -302,10 +302,10 @@ class Select(Node):
 
 # name -> (C function, torch function, derivative rule f(x, dx, y) with y = the call itself)
 FUNCS = {
-    "tanh": ("tanhf", torch.tanh, lambda x, dx, y: mul(dx, sub(Const(1.0), mul(y, y)))),
-    "exp": ("expf", torch.exp, lambda x, dx, y: mul(dx, y)),
-    "log": ("logf", torch.log, lambda x, dx, y: div(dx, x)),
-    "sqrt": ("sqrtf", torch.sqrt, lambda x, dx, y: div(dx, mul(Const(2.0), y))),
+    "tanh": ("fa_tanh", torch.tanh, lambda x, dx, y: mul(dx, sub(Const(1.0), mul(y, y)))),
+    "exp": ("fa_exp", torch.exp, lambda x, dx, y: mul(dx, y)),
+    "log": ("fa_log", torch.log, lambda x, dx, y: div(dx, x)),
+    "sqrt": ("fa_sqrt", torch.sqrt, lambda x, dx, y: div(dx, mul(Const(2.0), y))),
     "abs": ("fabsf", torch.abs, lambda x, dx, y: mul(dx, Select(Bin("<", x, Const(0.0)), Const(-1.0), Const(1.0)))),
     "sigmoid": ("fa_sigmoid", torch.sigmoid, lambda x, dx, y: mul(dx, mul(y, sub(Const(1.0), y)))),
 }
@@ -717,10 +717,59 @@ HEADER_PRELUDE = """// Generated by flex_attention_tpu_amd.compiler; do not edit
 #pragma once
 #include <math.h>
 namespace fa {
-__host__ __device__ inline int fa_py_mod(int a, int b) { const int r = a % b; return (r != 0 && ((r < 0) != (b < 0))) ? r + b : r; }
-__host__ __device__ inline int fa_py_floordiv(int a, int b) { const int q = a / b; return ((a % b != 0) && ((a < 0) != (b < 0))) ? q - 1 : q; }
+// Python's % and // on integers.  A divisor that is a power of two (tile sizes, which reach a tile-form function
+// at run time, and most constants) takes a mask or a shift, which also hold for negative dividends in two's
+// complement; anything else the integer division.
+__host__ __device__ inline int fa_py_mod(int a, int b) {
+  if (b > 0 && (b & (b - 1)) == 0) return a & (b - 1);
+  const int r = a % b;
+  return (r != 0 && ((r < 0) != (b < 0))) ? r + b : r;
+}
+__host__ __device__ inline int fa_py_floordiv(int a, int b) {
+  if (b > 0 && (b & (b - 1)) == 0) return a >> __builtin_ctz((unsigned)b);
+  const int q = a / b;
+  return ((a % b != 0) && ((a < 0) != (b < 0))) ? q - 1 : q;
+}
 __host__ __device__ inline float fa_py_fmod(float a, float b) { const float r = fmodf(a, b); return (r != 0.f && ((r < 0.f) != (b < 0.f))) ? r + b : r; }
-__host__ __device__ inline float fa_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+// Elementary functions: on the device the hardware's exp2 / log2 / rcp / sqrt (the arithmetic the kernels' own
+// softmax and soft-cap use; tanh as 1 - 2 / (e^2x + 1) saturates correctly and is good to a few 1e-7 absolute),
+// a handful of instructions per score where the library routines take several dozen; on the host, where the tests
+// evaluate the generated code, libm.
+__host__ __device__ inline float fa_exp(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_exp2f(x * 1.4426950408889634f);
+#else
+  return expf(x);
+#endif
+}
+__host__ __device__ inline float fa_log(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_logf(x) * 0.6931471805599453f;
+#else
+  return logf(x);
+#endif
+}
+__host__ __device__ inline float fa_sqrt(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_sqrtf(x);
+#else
+  return sqrtf(x);
+#endif
+}
+__host__ __device__ inline float fa_tanh(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x * 2.8853900817779268f) + 1.0f);
+#else
+  return tanhf(x);
+#endif
+}
+__host__ __device__ inline float fa_sigmoid(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+#else
+  return 1.0f / (1.0f + expf(-x));
+#endif
+}
 """
 
 
