@@ -230,12 +230,17 @@ def score_spec_c(score_fn: Optional[Callable], Hq: int, device, mod_q: int, mod_
             "compiler.compile_score_mod / compile_score_fn (which compile a Python function into the kernels)")
     slopes_ptr = None
     if spec.kind == _lib.SCORE_ALIBI:
-        if len(spec.slopes) != Hq:
-            raise ValueError(f"ALiBi has {len(spec.slopes)} slopes for {Hq} heads")
-        key = (spec.slopes, str(device))
+        slopes = spec.slopes
+        if slopes is None and spec.slopes_open is not None:
+            if Hq > len(spec.slopes_open):
+                raise NotImplementedError(f"the compiled ALiBi closure was checked for {len(spec.slopes_open)} heads, the call has {Hq}")
+            slopes = spec.slopes_open[:Hq]
+        if slopes is None or len(slopes) != Hq:
+            raise ValueError(f"ALiBi has {0 if slopes is None else len(slopes)} slopes for {Hq} heads")
+        key = (slopes, str(device))
         t = _slopes_cache.get(key)
         if t is None:
-            t = torch.tensor(spec.slopes, dtype=torch.float32, device=device)
+            t = torch.tensor(slopes, dtype=torch.float32, device=device)
             _slopes_cache.put(key, t)
         slopes_ptr = t.data_ptr()
     return _lib.ScoreSpecC(spec.kind, spec.cap, spec.slope, int(mod_q), int(mod_k), 0, slopes_ptr)

@@ -43,7 +43,7 @@ import torch
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 JIT_DIR = os.path.join(PKG_DIR, "_jit")
-CODEGEN_VERSION = 2
+CODEGEN_VERSION = 3
 
 
 # ------------------------------------------------------------------------------------------------
@@ -381,6 +381,27 @@ class Pow(Node):
         return self.a.uses_s()
 
 
+class PowF(Node):
+    """a ** b with a float result for a positive base (``2 ** (-8 * (h + 1) / 16)``, ``s ** 1.5``)."""
+    def __init__(self, a: Node, b: Node):
+        self.a, self.b, self.kind = a, b, "f"
+
+    def c(self):
+        return f"fa_pow({_as_float_c(self.a)}, {_as_float_c(self.b)})"
+
+    def ev(self, env):
+        return torch.pow(torch.as_tensor(self.a.ev(env), dtype=torch.float64), torch.as_tensor(self.b.ev(env), dtype=torch.float64))
+
+    def d(self):
+        if not self.uses_s():
+            return Const(0.0)
+        # d(a^b) = a^b (b' ln a + b a' / a)
+        return mul(self, add(mul(self.b.d(), Call("log", self.a)), div(mul(self.b, self.a.d()), self.a)))
+
+    def uses_s(self):
+        return self.a.uses_s() or self.b.uses_s()
+
+
 def walk(n: Node):
     yield n
     for attr in ("a", "b", "cond", "index"):
@@ -566,7 +587,13 @@ class Rewriter:
         if isinstance(e.op, ast.Pow):
             if isinstance(b, Const) and b.kind == "i" and 0 <= b.value <= 8:
                 return Pow(a, b.value)
-            self.fail(e, "only small non-negative integer powers are supported")
+            if a.kind == "b" or b.kind == "b":
+                self.fail(e, "'**' needs numbers")
+            if isinstance(a, Const) and isinstance(b, Const):
+                return Const(float(a.value) ** float(b.value))
+            if isinstance(a, Const) and a.value <= 0:
+                self.fail(e, "a power with a variable exponent needs a positive base")
+            return PowF(a, b)   # (the base must be positive where it is evaluated: exp2(b log2 a) on the device)
         if isinstance(e.op, (ast.BitAnd, ast.BitOr)):
             if a.kind != "b" or b.kind != "b":
                 self.fail(e, "'&' / '|' need boolean operands")
@@ -749,6 +776,13 @@ __host__ __device__ inline float fa_log(float x) {
   return logf(x);
 #endif
 }
+__host__ __device__ inline float fa_pow(float a, float b) {   // (a > 0)
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_exp2f(b * __builtin_amdgcn_logf(a));
+#else
+  return powf(a, b);
+#endif
+}
 __host__ __device__ inline float fa_sqrt(float x) {
 #if defined(__HIP_DEVICE_COMPILE__)
   return __builtin_amdgcn_sqrtf(x);
@@ -877,15 +911,96 @@ def _check_against_python(expr: Node, fn: Callable, form: str):
         raise NotImplementedError(f"the function could not be evaluated on torch probes: {e}") from e
     got = got.expand_as(want) if got.ndim <= want.ndim else got
     ok = torch.equal(got.to(torch.bool), want.to(torch.bool)) if form == "mask" else \
-        torch.allclose(got.to(torch.float64), want.to(torch.float64), rtol=1e-9, atol=1e-9)
+        torch.allclose(got.to(torch.float64), want.to(torch.float64), rtol=2e-6, atol=2e-6)
+    # (the tolerance of float32: torch evaluates a Python float times an integer index tensor in float32, the tree
+    # in float64; a misread construct differs by far more)
     if not ok:
         raise NotImplementedError("the compiled expression does not reproduce the Python function on random probes "
                                   "(a construct was misread): " + (inspect.getsource(fn).strip()[:200]))
 
 
-def compile_score_mod(fn: Callable) -> Callable:
+MAX_OPEN_HEADS = 256   # heads for which a slope computed from the head's index is checked ahead of the call
+
+
+def _recognised_score_spec(expr: Node):
+    """The ScoreSpec of a functor the kernels carry themselves (plain scores, tanh soft-cap, ALiBi with global
+    indices and a slope per head) if the expression equals one, else None.  Numeric, on the expression tree in
+    float64: soft-cap logits far into saturation give the cap, one (i, j) pair gives a head's slope, and the closed
+    form must then reproduce the expression on every probe (random and extreme logits, indices up to 70000,
+    several batch entries, every head).  A slope per head needs the number of heads: only functions that take it
+    from a table indexed by ``h`` qualify, and the table's length is the number of heads of the specification."""
+    from . import _lib
+    from .scores import ScoreSpec
+    nodes = list(walk(expr))
+    names = {n.name for n in nodes if isinstance(n, Var)}
+    if names & {"mq", "mk"}:
+        return None
+    head_tables = [n for n in nodes if isinstance(n, Table) and isinstance(n.index, Var) and n.index.name == "h"]
+    other_h = any(isinstance(n, Var) and n.name == "h" for n in nodes) and \
+        sum(1 for n in nodes if isinstance(n, Var) and n.name == "h") != len(head_tables)
+    H = min((len(t.values) for t in head_tables), default=None)
+    g = torch.Generator().manual_seed(5)
+    s = torch.cat([torch.randn(61, generator=g, dtype=torch.float64) * 4.0,
+                   torch.tensor([0.0, 1e5, -1e5], dtype=torch.float64)])[:, None, None]
+    i = torch.tensor([0, 1, 5, 130, 4095, 70000])[None, :, None]
+    j = torch.tensor([0, 2, 5, 131, 4000, 65536])[None, None, :]
+    shape = (s.shape[0], i.shape[1], j.shape[2])
+
+    def ev(b, h):
+        out = torch.as_tensor(expr.ev({"s": s, "b": b, "h": h, "i": i, "j": j}), dtype=torch.float64)
+        return out.expand(shape) if out.ndim else out.reshape(1, 1, 1).expand(shape)
+    try:
+        heads = list(range(H)) if H is not None else [0, 1, 5]
+        outs = {(b, h): ev(b, h) for b in (0, 3) for h in heads}
+    except Exception:  # noqa: BLE001  (a probe outside the function's domain: no closed form claimed)
+        return None
+    if not all(bool(torch.isfinite(o).all()) for o in outs.values()):
+        return None
+    se = s.expand(shape)
+    if all(bool(((o - se).abs() <= 1e-12 * (1.0 + se.abs())).all()) for o in outs.values()):
+        return ScoreSpec(kind=_lib.SCORE_NONE)
+    first = outs[(0, heads[0])]
+    same_everywhere = all(torch.equal(o, first) for o in outs.values()) and \
+        bool((first == first[:, :1, :1]).all())
+    if same_everywhere:
+        cap = float(first[-2, 0, 0])   # the logit 1e5
+        if cap > 0.0 and bool(((first - cap * torch.tanh(se / cap)).abs() <= 1e-9 * (1.0 + cap)).all()):
+            return ScoreSpec(kind=_lib.SCORE_SOFTCAP, cap=cap)
+        return None
+    dist = (j - i).to(torch.float64).expand(shape)
+
+    def slope_of(h):
+        """The head's slope if the expression is s + slope (j - i) for it, on every probe and batch entry."""
+        o0 = outs[(0, h)] if (0, h) in outs else ev(0, h)
+        a = float((o0 - se)[0, 0, 1] / dist[0, 0, 1])
+        for b in (0, 3):
+            o = outs[(b, h)] if (b, h) in outs else ev(b, h)
+            if not bool(torch.isfinite(o).all()) or \
+                    not bool(((o - se - a * dist).abs() <= 1e-9 * (1.0 + abs(a) * dist.abs())).all()):
+                return None
+        return a
+    if H is not None and not other_h:   # slopes from a table: as many heads as the table has entries
+        slopes = [slope_of(h) for h in heads]
+        return ScoreSpec(kind=_lib.SCORE_ALIBI, slopes=tuple(slopes)) if None not in slopes else None
+    # slopes computed from h (2 ** (-8 (h + 1) / H) and the like): checked for the first MAX_OPEN_HEADS heads, of
+    # which a call takes as many as it has
+    slopes = []
+    try:
+        for h in range(MAX_OPEN_HEADS):
+            slopes.append(slope_of(h))
+    except Exception:  # noqa: BLE001  (a table that ends, a domain error: the heads so far)
+        pass
+    if None in slopes or len(slopes) < 1 or (H is not None and len(slopes) < H):
+        return None
+    return ScoreSpec(kind=_lib.SCORE_ALIBI, slopes=None, slopes_open=tuple(slopes))
+
+
+def compile_score_mod(fn: Callable, recognise: bool = True) -> Callable:
     """``fn(s, b, h, q_idx, kv_idx) -> s'`` (element-wise; s = sm_scale <q, k>, global indices) compiled into
-    the kernels.  Returns a closure with the same call signature carrying ``.spec``."""
+    the kernels.  Returns a closure with the same call signature carrying ``.spec``.  A function that equals one
+    of the kernels' own functors (the identity, ``cap * tanh(s / cap)``, ``s + SLOPES[h] * (kv_idx - q_idx)``) gets
+    that functor's specification, and with it the generated-stream kernels, instead of a compiled functor
+    (``recognise=False`` compiles it regardless)."""
     from . import _lib
     from .scores import ScoreSpec
     rw = Rewriter(fn, "score_mod")
@@ -898,7 +1013,8 @@ def compile_score_mod(fn: Callable) -> Callable:
 
     def score_mod(s, b, h, q_idx, kv_idx):
         return fn(s, b, h, q_idx, kv_idx)
-    score_mod.spec = ScoreSpec(kind=_lib.SCORE_CUSTOM, custom=code)
+    builtin = _recognised_score_spec(expr) if recognise else None
+    score_mod.spec = builtin if builtin is not None else ScoreSpec(kind=_lib.SCORE_CUSTOM, custom=code)
     score_mod.expr = expr
     score_mod.__wrapped__ = fn
     return score_mod
@@ -939,11 +1055,58 @@ def compile_score_fn(fn: Callable) -> Callable:
     return score_fn
 
 
-def compile_mask_fn(fn: Callable, block_q: int, block_k: int) -> Tuple[Callable, Callable]:
+def _recognised_mask_fns(expr: Node, block_q: int, block_k: int):
+    """The (mask_fn, block_mask_fn) pair of this package's own factories (causal, sliding window, both) if the
+    predicate equals one of them, else None: those masks have closed-form block maps and run the generated-stream
+    kernels.  Numeric, on the expression tree: the keys kept by one query far out (position 2^22) give the
+    candidate's window, and the factory's own ``mask_fn`` must then agree with the predicate on index grids around
+    the origin, around that query and around both ends of its window."""
+    from . import masks
+    i0 = 1 << 22
+
+    def ev(qi, kj):
+        out = torch.as_tensor(expr.ev({"i": qi[:, None], "j": kj[None, :]}))
+        return out.to(torch.bool).expand(qi.numel(), kj.numel())
+    try:
+        row = ev(torch.tensor([i0]), torch.arange(0, i0 + 64))[0]
+    except Exception:  # noqa: BLE001
+        return None
+    kept = torch.nonzero(row).flatten()
+    if kept.numel() == 0:
+        return None
+    causal = int(kept[-1]) == i0
+    if not causal and int(kept[-1]) != i0 + 63:
+        return None
+    window = i0 - int(kept[0]) + 1 if int(kept[0]) > 0 else None
+    if not causal and window is None:
+        return None      # (keeps everything: no mask is the caller's way to say so)
+    if causal and window is None:
+        cand = masks.make_causal_mask_fns(block_q, block_k)
+    elif causal:
+        cand = masks.make_causal_sliding_window_mask_fns(block_q, block_k, window)
+    else:
+        cand = masks.make_sliding_window_mask_fns(block_q, block_k, window)
+    w = window or 0
+    grids = [(torch.arange(0, 320), torch.arange(0, 320)),
+             (torch.arange(i0 - 96, i0 + 96), torch.arange(i0 - 96, i0 + 96)),
+             (torch.arange(i0 - 96, i0 + 96), torch.arange(max(0, i0 - w - 96), i0 - w + 96)),
+             (torch.arange(max(0, w - 96), w + 96), torch.arange(0, 192))]
+    try:
+        for qi, kj in grids:
+            if not torch.equal(ev(qi, kj), torch.as_tensor(cand[0](qi, kj)).to(torch.bool)):
+                return None
+    except Exception:  # noqa: BLE001
+        return None
+    return cand
+
+
+def compile_mask_fn(fn: Callable, block_q: int, block_k: int, recognise: bool = True) -> Tuple[Callable, Callable]:
     """``fn(q_idx, k_idx) -> bool[Bq, Bk]`` on 1-D global index arrays (the reference's ``mask_fn``,
     masks.py:15-16) compiled into the kernels.  Returns ``(mask_fn, block_mask_fn)``: the block closure is
     ``any(mask_fn over the tile)``, which the GPU builder reproduces bit for bit by evaluating the compiled
-    predicate on every element of every tile."""
+    predicate on every element of every tile.  A predicate that equals one of this package's own masks (causal,
+    sliding window, both) returns that factory's pair instead: a closed-form block map and the generated-stream
+    kernels (``recognise=False`` compiles it regardless)."""
     from . import _lib
     from .masks import MaskSpec
     rw = Rewriter(fn, "mask")
@@ -953,6 +1116,10 @@ def compile_mask_fn(fn: Callable, block_q: int, block_k: int) -> Tuple[Callable,
     if any(isinstance(n, Var) and n.name not in ("i", "j") for n in walk(expr)):
         raise NotImplementedError("a mask function may depend on q_idx and k_idx only")
     _check_against_python(expr, fn, "mask")
+    if recognise:
+        builtin = _recognised_mask_fns(expr, block_q, block_k)
+        if builtin is not None:
+            return builtin
     code = CustomCode("mask", _function_text(rw.tables, expr, "b"), "", inspect.getsource(fn).strip())
     spec = MaskSpec(flags=_lib.MASK_CUSTOM, custom=code)
 

@@ -22,6 +22,9 @@ class ScoreSpec:
     cap: float = 0.0
     slope: float = 0.0
     slopes: Optional[Tuple[float, ...]] = None  # per-head slopes (global ALiBi)
+    # (global ALiBi of a compiled closure whose slope is a function of the head's index: the slopes of heads 0, 1, ...
+    # as far as they were checked; a call takes the first Hq of them)
+    slopes_open: Optional[Tuple[float, ...]] = None
     custom: Optional[object] = None             # compiler.CustomCode of a compiled closure (kind SCORE_CUSTOM)
 
 

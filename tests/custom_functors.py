@@ -23,6 +23,26 @@ def mixed_mod(s, b, h, q_idx, kv_idx):
     return torch.minimum(t, 3.0 + 0.1 * s) + 0.01 * SLOPES[h] * (q_idx % 7) + 0.2 * torch.tanh(0.5 * s) * (b + 1)
 
 
+def alibi_symmetric_mod(s, b, h, q_idx, kv_idx):
+    """a distance penalty on both sides with the usual slopes computed from the head's index (a power with a
+    variable exponent): none of the kernels' own functors"""
+    return s - 2.0 ** (-8.0 * (h + 1) / 4) * torch.abs(q_idx - kv_idx)
+
+
+def alibi_formula_mod(s, b, h, q_idx, kv_idx):
+    """global ALiBi with the slopes computed from the head's index: recognised as the kernels' own functor"""
+    return s + 2.0 ** (-8.0 * (h + 1) / 4) * (kv_idx - q_idx)
+
+
+def softcap30_mod(s, b, h, q_idx, kv_idx):
+    return 30.0 * torch.tanh(s / 30.0)
+
+
+def causal_window_mask(q_idx, k_idx):
+    d = q_idx[:, None] - k_idx[None, :]
+    return (d >= 0) & (d < 200)
+
+
 def prefix_lm_mask(q_idx, k_idx):
     """causal, plus a bidirectional prefix"""
     return (q_idx[:, None] >= k_idx[None, :]) | (k_idx[None, :] < PREFIX)
@@ -51,9 +71,11 @@ def compiled():
     """name -> (score closure or None, (mask_fn, block_mask_fn) or None), compiled at 128 x 128 granularity."""
     from flex_attention_tpu_amd import compiler, util
     return {
-        "alibi_mod": (compiler.compile_score_mod(alibi_mod), None),
-        "softcap_mod": (compiler.compile_score_mod(softcap_mod), None),
+        # (written to equal the kernels' own functors: compiled regardless, to compare the two)
+        "alibi_mod": (compiler.compile_score_mod(alibi_mod, recognise=False), None),
+        "softcap_mod": (compiler.compile_score_mod(softcap_mod, recognise=False), None),
         "mixed_mod": (compiler.compile_score_mod(mixed_mod), None),
+        "alibi_symmetric_mod": (compiler.compile_score_mod(alibi_symmetric_mod), None),
         "prefix_lm": (None, compiler.compile_mask_fn(prefix_lm_mask, 128, 128)),
         "checker": (None, compiler.compile_mask_fn(checker_mask, 128, 128)),
         "mixed_mod+prefix_lm": (compiler.compile_score_mod(mixed_mod), compiler.compile_mask_fn(prefix_lm_mask, 128, 128)),

@@ -28,7 +28,7 @@ def _grid(n=40, seed=3, tile=None):
 
 @pytest.mark.parametrize("fn", [cf.alibi_mod, cf.softcap_mod, cf.mixed_mod], ids=lambda f: f.__name__)
 def test_score_mod_tree_and_derivative(fn):
-    c = compiler.compile_score_mod(fn)
+    c = compiler.compile_score_mod(fn, recognise=False)
     assert c.spec.kind == _lib.SCORE_CUSTOM
     s, i, j = _grid()
     for b, h in ((0, 0), (1, 3)):
@@ -109,6 +109,82 @@ def test_recognised_closed_forms_keep_the_stream_kernels():
     assert util.make_jax_score_fn(clipped_alibi).spec.kind == _lib.SCORE_CUSTOM
 
 
+def _causal(q_idx, k_idx):
+    return q_idx[:, None] >= k_idx[None, :]
+
+
+def _window(q_idx, k_idx):
+    return q_idx[:, None] - k_idx[None, :] < 1000
+
+
+def _causal_window(q_idx, k_idx):
+    d = q_idx[:, None] - k_idx[None, :]
+    return (d >= 0) & (d <= 1024)
+
+
+def _causal_window_and_a_sink(q_idx, k_idx):
+    d = q_idx[:, None] - k_idx[None, :]
+    return ((d >= 0) & (d <= 1024)) | (k_idx[None, :] == 7)
+
+
+def _identity(s, b, h, q_idx, kv_idx):
+    return s
+
+
+def _softcap(s, b, h, q_idx, kv_idx):
+    return 50.0 * torch.tanh(s / 50.0)
+
+
+def _nearly_softcap(s, b, h, q_idx, kv_idx):
+    return 50.0 * torch.tanh(s / 50.0) + 1e-6 * s
+
+
+def _alibi_by_formula(s, b, h, q_idx, kv_idx):
+    return s + 2.0 ** (-8.0 * (h + 1) / 16) * (kv_idx - q_idx)
+
+
+def _alibi_symmetric(s, b, h, q_idx, kv_idx):
+    return s - 0.5 ** (h + 1) * torch.abs(q_idx - kv_idx)
+
+
+def test_closures_that_equal_a_builtin_functor_get_it():
+    """compile_score_mod / compile_mask_fn recognise the functors the kernels carry themselves (numerically, on
+    the expression tree) and hand out their specifications: those calls run the generated-stream kernels on
+    closed-form block maps.  Anything that differs anywhere on the probes stays a compiled functor."""
+    from flex_attention_tpu_amd import masks, scores
+    for fn, flags, window in ((_causal, _lib.MASK_CAUSAL, 0), (_window, _lib.MASK_WINDOW, 1000),
+                              (_causal_window, _lib.MASK_CAUSAL | _lib.MASK_WINDOW, 1025)):
+        mf, bf = compiler.compile_mask_fn(fn, 128, 64)
+        assert mf.spec.flags == flags and mf.spec.window == window and mf.spec.custom is None and bf.spec == mf.spec
+        qi, kj = torch.arange(900, 1300), torch.arange(0, 1400)
+        assert torch.equal(torch.as_tensor(mf(qi, kj)), torch.as_tensor(fn(qi, kj)))
+        assert compiler.compile_mask_fn(fn, 128, 64, recognise=False)[0].spec.flags == _lib.MASK_CUSTOM
+    assert compiler.compile_mask_fn(_causal_window_and_a_sink, 128, 64)[0].spec.flags == _lib.MASK_CUSTOM
+    assert compiler.compile_score_mod(_identity).spec == scores.ScoreSpec(kind=_lib.SCORE_NONE)
+    assert compiler.compile_score_mod(_softcap).spec == scores.ScoreSpec(kind=_lib.SCORE_SOFTCAP, cap=50.0)
+    assert compiler.compile_score_mod(_softcap, recognise=False).spec.kind == _lib.SCORE_CUSTOM
+    assert compiler.compile_score_mod(_nearly_softcap).spec.kind == _lib.SCORE_CUSTOM
+    assert compiler.compile_score_mod(_alibi_symmetric).spec.kind == _lib.SCORE_CUSTOM
+    assert compiler.compile_score_mod(cf.alibi_mod).spec == scores.ScoreSpec(kind=_lib.SCORE_ALIBI, slopes=cf.SLOPES)
+    spec = compiler.compile_score_mod(_alibi_by_formula).spec     # (slopes from the head's index: as many as a call has heads)
+    assert spec.kind == _lib.SCORE_ALIBI and spec.slopes is None and len(spec.slopes_open) == compiler.MAX_OPEN_HEADS
+    assert all(abs(a - b) <= 1e-12 for a, b in zip(spec.slopes_open[:16], scores.alibi_slopes(16)))
+    assert compiler.compile_score_mod(cf.mixed_mod).spec.kind == _lib.SCORE_CUSTOM
+
+
+def test_powers_with_variable_exponents():
+    def f(s, b, h, q_idx, kv_idx):
+        return s * 0.5 ** (h + 1) + (torch.abs(s) + 1.0) ** 1.5
+    g = compiler.compile_score_mod(f)
+    assert g.spec.kind == _lib.SCORE_CUSTOM and "fa_pow" in g.spec.custom.body and "fa_pow" in g.spec.custom.dbody
+    env = {"s": torch.linspace(-3, 3, 12, dtype=torch.float64), "b": 0, "h": 2, "i": 0, "j": 0}   # (not 0: |s| has no derivative there)
+    s = env["s"].clone().requires_grad_(True)
+    want = torch.autograd.grad(f(s, 0, 2, 0, 0).sum(), s)[0]
+    assert torch.allclose(torch.as_tensor(g.expr.d().ev(env), dtype=torch.float64), want, rtol=1e-12, atol=1e-12)
+    with pytest.raises(NotImplementedError, match="positive base"):
+        compiler.compile_score_mod(lambda s, b, h, q_idx, kv_idx: (-2.0) ** h + s)
+
+
 def test_unsupported_constructs_are_refused():
     def uses_softmax(s, b, h, q_idx, kv_idx):
         return torch.softmax(s, -1)
@@ -137,8 +213,8 @@ def test_unsupported_constructs_are_refused():
 
 
 def test_functor_keys_and_header_are_deterministic():
-    a = compiler.compile_score_mod(cf.softcap_mod).spec.custom
-    b = compiler.compile_score_mod(cf.softcap_mod).spec.custom
+    a = compiler.compile_score_mod(cf.softcap_mod, recognise=False).spec.custom
+    b = compiler.compile_score_mod(cf.softcap_mod, recognise=False).spec.custom
     m = compiler.compile_mask_fn(cf.prefix_lm_mask, 128, 128)[0].spec.custom
     assert a == b and compiler.functor_key(a, None) == compiler.functor_key(b, None)
     assert len({compiler.functor_key(a, None), compiler.functor_key(a, m), compiler.functor_key(None, m)}) == 3

@@ -33,7 +33,8 @@ def _oracle_kwargs(name, Sq, Sk):
     """Oracle keywords: the Python functions themselves (score_mod on tensors, dense mask from mask_fn)."""
     kw = {}
     parts = name.split("+")
-    mods = {"alibi_mod": cf.alibi_mod, "softcap_mod": cf.softcap_mod, "mixed_mod": cf.mixed_mod}
+    mods = {"alibi_mod": cf.alibi_mod, "softcap_mod": cf.softcap_mod, "mixed_mod": cf.mixed_mod,
+            "alibi_symmetric_mod": cf.alibi_symmetric_mod}
     masks = {"prefix_lm": cf.prefix_lm_mask, "checker": cf.checker_mask}
     for p in parts:
         if p in mods:
@@ -44,7 +45,8 @@ def _oracle_kwargs(name, Sq, Sk):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
-@pytest.mark.parametrize("name", ["alibi_mod", "softcap_mod", "mixed_mod", "prefix_lm", "checker", "mixed_mod+prefix_lm"])
+@pytest.mark.parametrize("name", ["alibi_mod", "softcap_mod", "mixed_mod", "alibi_symmetric_mod", "prefix_lm", "checker",
+                                  "mixed_mod+prefix_lm"])
 def test_compiled_closures_all_passes(F, compiled, name, dtype):
     _closures_all_passes(F, compiled, name, dtype, 128)
 
@@ -53,6 +55,34 @@ def test_compiled_closures_all_passes(F, compiled, name, dtype):
 def test_compiled_closures_head_dimension_256(F, compiled, name):
     """The functor libraries hold the bf16 kernels of head dimension 256 as well."""
     _closures_all_passes(F, compiled, name, torch.bfloat16, 256)
+
+
+def test_closures_that_equal_a_builtin_functor_run_its_kernels(F):
+    """Closures the compiler recognises (a soft-cap, global ALiBi with slopes computed from the head's index, a
+    causal window) carry the specifications of this package's own factories: the calls give the bits of the
+    factories' closures (the generated-stream kernels on a closed-form block map) and need no functor library."""
+    from flex_attention_tpu_amd import compiler, masks, scores
+    B, Hq, Hkv, S = 2, 4, 4, 1024
+    sc = 1 / math.sqrt(128)
+    q, k, v, do = [x.to(DEV) for x in O.make_inputs(B, Hq, Hkv, S, S, 128, dtype=torch.bfloat16, seed=73)]
+    mask_c = compiler.compile_mask_fn(cf.causal_window_mask, 128, 128)
+    mask_b = masks.make_causal_sliding_window_mask_fns(128, 128, 200)
+    assert mask_c[0].spec == mask_b[0].spec
+    for closure, factory in ((cf.softcap30_mod, scores.make_softcap_score_fn(30.0)),
+                             (cf.alibi_formula_mod, scores.make_alibi_global_score_fn(Hq))):
+        sfn = compiler.compile_score_mod(closure)
+        assert sfn.spec.custom is None and sfn.spec.kind == factory.spec.kind
+        results = []
+        for score_fn, (mf, bf) in ((sfn, mask_c), (factory, mask_b)):
+            o, l, m = F._flex_attention_impl(q, k, v, None, None, True, False, sc, 1, 128, 128, 128, False, bf, mf, score_fn)
+            grads = F.flex_attention_bwd(q, k, v, None, None, l, m, o, do, block_q=128, block_k=128, sm_scale=sc,
+                                         score_fn=score_fn, mask_fn=mf, block_mask_fn=bf)
+            results.append((o, l, m, *grads))
+        for name, a, b in zip(("o", "l", "m", "dq", "dk", "dv"), *results):
+            assert torch.equal(a, b), f"{closure.__name__}: {name} differs from the factory's"
+        ro = O.mha_reference(q.cpu(), k.cpu(), v.cpu(), sm_scale=sc, causal=True, window_size=200,
+                             score_mod=lambda s, b, h, i, j, f=closure: f(s, b, h, i, j))
+        assert_close(closure.__name__ + " o", results[0][0], ro, torch.bfloat16)
 
 
 def _closures_all_passes(F, compiled, name, dtype, D):
