@@ -187,6 +187,9 @@ __global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void fwd_bf16_kernel(FwdArgs 
     constexpr int kPanel = kTileElems * 2;   // bytes
     bf16x8 kf[NG][4];
     s16x4 vlo[4][4 * NP], vhi[4][4 * NP];  // [tt][db]
+    // Plain scores fetch the first half of V^T ahead of the softmax, which hides the latency; a score function's
+    // own arithmetic, or the wider rows, need those registers in the softmax (the compiler spilled otherwise)
+    constexpr bool kEarlyV = NP == 1 && (SCORE == FLEXATTN_SCORE_NONE || SCORE == kScoreBiasOnly);
     auto read_k = [&](int g) {
       const int c = g / (2 * NP), pn = (g % (2 * NP)) >> 1;
 #pragma unroll
@@ -210,7 +213,7 @@ __global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void fwd_bf16_kernel(FwdArgs 
     for (int g = 0; g < NG; ++g) {
       if (g < NG - 1) {
         read_k(g + 1);
-      } else {
+      } else if (kEarlyV) {
         read_v(0);
       }
       const int c = g / (2 * NP), pn = (g % (2 * NP)) >> 1;
@@ -227,7 +230,7 @@ __global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void fwd_bf16_kernel(FwdArgs 
         loader.load_block(v_next + 128 * (g >> 2), sV + ((buf ^ 1) * NP + (g >> 2)) * kTileElems, g & 3);
       }
     }
-    read_v(1);
+    if (kEarlyV) read_v(1);
 
     // ---- score mod, mask, online softmax ----
     // For the plain score the running maximum is kept on the raw dot products and the scale is
@@ -310,6 +313,10 @@ __global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void fwd_bf16_kernel(FwdArgs 
 
     // ---- O^T += V^T P^T ----
     __builtin_amdgcn_sched_barrier(0);
+    if (!kEarlyV) {
+      read_v(0);
+      read_v(1);
+    }
 #pragma unroll
     for (int tt = 0; tt < 4; ++tt) {
       if (tt < 2) read_v(tt + 2);
