@@ -175,24 +175,31 @@ static MapArgs col_view(const flexattn_block_map& m) {
   return r;
 }
 
+// Whether the dk/dv pass of this request runs the generated stream (else the kernel with a compiled main loop).
+static bool dkv_on_stream(const flexattn_bwd_params* p) {
+  return bwd_dkv_bf16_d128_on_stream(p->score.kind, p->flags, p->map.nq, p->ab.ptr != nullptr, p->Hq, p->Hkv);
+}
+
 // Whether the bf16 dk/dv and dq kernels of this request can hand dS over through a buffer: the generated-stream
 // dk/dv kernels for plain and softcap scores write it (the position-bias streams keep the key's share of the
-// bias out of their dS, compiled-loop kernels have no export).  Looks at shapes, score and flags only.
+// bias out of their dS), and so does the dk/dv kernel with a compiled main loop, for every score (compiled score
+// functions among them: the dq pass from dS then evaluates none).  Looks at shapes, score, flags and the map's size.
 static bool ds_exchange_ok(const flexattn_bwd_params* p) {
-#ifdef FLEXATTN_CUSTOM_ONLY
-  (void)p;
-  return false;
-#else
   if (p == nullptr || p->dtype != FLEXATTN_BF16 || p->D != 128) return false;
-  if ((p->flags & FLEXATTN_FLAG_COMPILED_LOOP) || p->ab.ptr != nullptr) return false;
-  if (p->score.kind != FLEXATTN_SCORE_NONE && p->score.kind != FLEXATTN_SCORE_SOFTCAP) return false;
-  if (p->B <= 0 || p->Hq <= 0 || p->Sq <= 0 || p->Sk <= 0) return false;
+  if (p->B <= 0 || p->Hq <= 0 || p->Hkv <= 0 || p->Sq <= 0 || p->Sk <= 0) return false;
+  if (dkv_on_stream(p) && p->score.kind != FLEXATTN_SCORE_NONE && p->score.kind != FLEXATTN_SCORE_SOFTCAP) return false;
   int bq = 0, bk = 0;
   bwd_dkv_bf16_d128_tile(&bq, &bk);
   if (p->Sq % bq != 0 || p->Sk % bk != 0) return false;
   if (p->ds_index.pairs <= 0 || p->ds_index.pairs > (int64_t)(p->Sq / bq) * (p->Sk / bk)) return false;
-  return p->Sq / bq <= 1024 && p->Sk / bk <= 1024;  // (both kernels cache a tile list in LDS)
-#endif
+  return p->Sq / bq <= 1024 && p->Sk / bk <= 1024;  // (the dq pass from dS caches a tile list in LDS)
+}
+
+// What the dq pass multiplies K by: the streams export dS without sm_scale (softcap: without its factor 4 either),
+// the kernel with a compiled main loop exports it complete.
+static float ds_out_scale(const flexattn_bwd_params* p) {
+  if (!dkv_on_stream(p)) return 1.0f;
+  return (p->score.kind == FLEXATTN_SCORE_SOFTCAP ? 4.f : 1.f) * p->sm_scale;
 }
 
 // one block of block_q x block_k bf16 values per (query head, kept tile pair)
@@ -427,7 +434,7 @@ int flexattn_bwd_delta(const void* o, const void* dout, float* delta, int64_t ro
 }
 
 static int launch_dq(const flexattn_bwd_params* p, BwdArgs a, hipStream_t s) {
-  if (p->ds != nullptr) return bwd_dq_from_ds(a, (p->score.kind == FLEXATTN_SCORE_SOFTCAP ? 4.f : 1.f) * p->sm_scale, s);
+  if (p->ds != nullptr) return bwd_dq_from_ds(a, ds_out_scale(p), s);
   if (p->dtype == FLEXATTN_BF16) {
     if (a.dab != nullptr) a.flags |= FLEXATTN_FLAG_COMPILED_LOOP;  // (the generated streams store no bias gradient)
     return p->D == 256 ? bwd_dq_bf16_d256(a, s) : bwd_dq_bf16_d128(a, s);

@@ -72,7 +72,10 @@ struct PinnedState {
       "+{a[176:179]}"(st.v[4]), "+{a[180:183]}"(st.v[5]), "+{a[184:187]}"(st.v[6]), "+{a[188:191]}"(st.v[7])
 
 // Score modifications: compiled C++ path, one 128 x 128 tile per loop iteration.
-template <int SCORE>
+// EXPORT: the kernel also writes the tile's bf16 dS (the B operands of the dk product: here with the score function's
+// derivative and sm_scale in them) to a.ds, in the block layout of the generated streams' export (see there), for
+// the dq pass from dS: a score function is then evaluated in one backward pass instead of two.
+template <int SCORE, bool EXPORT = false>
 __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
   using namespace dkv_cfg;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
@@ -273,6 +276,15 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_kernel(BwdArgs a) {
         elementwise(std::true_type{});
       } else {
         elementwise(std::false_type{});
+      }
+      if constexpr (EXPORT) {
+        // block of (query head, kept tile pair): head a.ds_pairs + a.ds_col[kv tile] + place of the q tile in the kv
+        // tile's list; inside it wave w writes 1 KB per (32-row q block cc, 16-row half u), lane L its 8 values
+        char* blk = static_cast<char*>(a.ds) +
+                    ((size_t)(b * a.Hq + hk * group + it / n_tiles) * (size_t)a.ds_pairs + (size_t)a.ds_col[kb] +
+                     (size_t)(it % n_tiles)) * kDsBlockBytes + 8192 * w + 16 * (2 * l32 + hh);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) *reinterpret_cast<bf16x8*>(blk + 1024 * (2 * cc + u)) = dsb[u];
       }
 
 #pragma unroll
@@ -1075,16 +1087,20 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_bf16_d128_plain_kernel(BwdArgs
 
 #endif  // FLEXATTN_CUSTOM_ONLY
 
-template <int SCORE>
-static int launch_dkv(const BwdArgs& a, hipStream_t stream) {
+template <int SCORE, bool EXPORT>
+static int launch_dkv_on(const BwdArgs& a, hipStream_t stream) {
   using namespace dkv_cfg;
-  auto kern = bwd_dkv_bf16_d128_kernel<SCORE>;
+  auto kern = bwd_dkv_bf16_d128_kernel<SCORE, EXPORT>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(dkv): %s", hipGetErrorString(attr));
   const int n_wg = a.B * a.Hkv * (a.Sk / BNK);
   hipLaunchKernelGGL(kern, dim3(n_wg), dim3(256), LDS_BYTES, stream, a);
   return check_launch("flexattn_bwd_dkv bf16");
+}
+template <int SCORE>
+static int launch_dkv(const BwdArgs& a, hipStream_t stream) {
+  return a.ds != nullptr ? launch_dkv_on<SCORE, true>(a, stream) : launch_dkv_on<SCORE, false>(a, stream);
 }
 
 #ifndef FLEXATTN_CUSTOM_ONLY
@@ -1117,6 +1133,24 @@ static int launch_dkv_plain(const BwdArgs& a, hipStream_t stream) {
 
 #endif  // FLEXATTN_CUSTOM_ONLY
 
+// Whether a request runs the generated-stream dk/dv kernel (else the one with a compiled main loop): the stream
+// caches the q tile list in LDS, has no additive bias, serves the global position bias for one query head per kv
+// head only, and a functor library of a compiled score function has no streams at all.
+bool bwd_dkv_bf16_d128_on_stream(int kind, int flags, int nq, bool has_ab, int Hq, int Hkv) {
+#ifdef FLEXATTN_CUSTOM_ONLY
+  (void)kind; (void)flags; (void)nq; (void)has_ab; (void)Hq; (void)Hkv;
+  return false;
+#else
+  const bool stream_ok = !(flags & FLEXATTN_FLAG_COMPILED_LOOP) && nq <= dkv_cfg::MAX_LIST && !has_ab;
+  switch (kind) {
+    case FLEXATTN_SCORE_NONE:
+    case FLEXATTN_SCORE_SOFTCAP: return stream_ok;
+    case FLEXATTN_SCORE_ALIBI: return stream_ok && Hq == Hkv;
+  }
+  return false;
+#endif
+}
+
 int bwd_dkv_bf16_d128(const BwdArgs& a, hipStream_t stream) {
 #ifdef FLEXATTN_CUSTOM_ONLY
   switch (a.score.kind) {
@@ -1125,17 +1159,14 @@ int bwd_dkv_bf16_d128(const BwdArgs& a, hipStream_t stream) {
   }
   return set_error(FLEXATTN_ENOTSUP, "this functor library holds the plain and the compiled score function only (kind %d asked)", a.score.kind);
 #else
-  // (the generated-stream kernel caches the q tile list in LDS)
-  // (and has no additive bias)
-  const bool stream_ok = !(a.flags & FLEXATTN_FLAG_COMPILED_LOOP) && a.map.nq <= dkv_cfg::MAX_LIST && a.score.ab == nullptr;
+  const bool on_stream = bwd_dkv_bf16_d128_on_stream(a.score.kind, a.flags, a.map.nq, a.score.ab != nullptr, a.Hq, a.Hkv);
   switch (a.score.kind) {
     case FLEXATTN_SCORE_NONE:
-      return stream_ok ? launch_dkv_plain<FLEXATTN_SCORE_NONE>(a, stream) : launch_dkv<FLEXATTN_SCORE_NONE>(a, stream);
+      return on_stream ? launch_dkv_plain<FLEXATTN_SCORE_NONE>(a, stream) : launch_dkv<FLEXATTN_SCORE_NONE>(a, stream);
     case FLEXATTN_SCORE_ALIBI:
-      return (stream_ok && a.Hq == a.Hkv) ? launch_dkv_plain<FLEXATTN_SCORE_ALIBI>(a, stream)
-                                          : launch_dkv<FLEXATTN_SCORE_ALIBI>(a, stream);
+      return on_stream ? launch_dkv_plain<FLEXATTN_SCORE_ALIBI>(a, stream) : launch_dkv<FLEXATTN_SCORE_ALIBI>(a, stream);
     case FLEXATTN_SCORE_SOFTCAP:
-      return stream_ok ? launch_dkv_plain<FLEXATTN_SCORE_SOFTCAP>(a, stream) : launch_dkv<FLEXATTN_SCORE_SOFTCAP>(a, stream);
+      return on_stream ? launch_dkv_plain<FLEXATTN_SCORE_SOFTCAP>(a, stream) : launch_dkv<FLEXATTN_SCORE_SOFTCAP>(a, stream);
     case FLEXATTN_SCORE_ALIBI_TILE: return launch_dkv<FLEXATTN_SCORE_ALIBI_TILE>(a, stream);
   }
   return set_error(FLEXATTN_EINVAL, "unknown score kind %d", a.score.kind);

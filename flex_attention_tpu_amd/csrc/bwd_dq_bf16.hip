@@ -179,7 +179,7 @@ __global__ __launch_bounds__(256, NP == 1 ? 2 : 1) void bwd_dq_bf16_kernel(BwdAr
     const char* kt = reinterpret_cast<const char*>(sK + buf * NP * kTileElems);
     const char* vt = reinterpret_cast<const char*>(sV + buf * NP * kTileElems);
 
-#pragma unroll(NP == 1 ? 2 : 1)   // (wider rows: rolled, which keeps the second block's operand loads out of the first block's registers: 1.37 -> 1.25 ms on B=4, H=16, S=4096, D=256)
+#pragma clang loop unroll_count(NP == 1 ? 2 : 1)   // (wider rows: rolled, which keeps the second block's operand loads out of the first block's registers: 1.37 -> 1.25 ms on B=4, H=16, S=4096, D=256)
     for (int c = 0; c < 2; ++c) {
       // ---- S^T and dP^T for kv rows [32c, 32c+32) ----
       f32x16 s_acc, dp_acc;

@@ -50,8 +50,6 @@ static_assert(NDS * DS_STAGE_BYTES >= 4 * 8192, "the epilogue stages 8 KB per wa
 static_assert(MAX_LIST == 1024, "a list entry packs the kv tile into 10 bits");
 }  // namespace dqds_cfg
 
-#ifndef FLEXATTN_CUSTOM_ONLY
-
 // s_waitcnt vmcnt(N) (vector-memory operations complete in issue order)
 template <int N>
 __device__ __forceinline__ void wait_vmem_but() {
@@ -246,14 +244,8 @@ __global__ __launch_bounds__(256, dqds_cfg::OCC) void bwd_dq_from_ds_kernel(BwdA
   }
 }
 
-#endif  // FLEXATTN_CUSTOM_ONLY
-
 // `a.map`: row lists of the block map at the dk/dv kernel's 128 x 128 tiles; `a.ds`: the buffer that kernel filled.
 int bwd_dq_from_ds(const BwdArgs& a, float out_scale, hipStream_t stream) {
-#ifdef FLEXATTN_CUSTOM_ONLY
-  (void)a; (void)out_scale; (void)stream;
-  return set_error(FLEXATTN_ENOTSUP, "this functor library has no dS exchange");
-#else
   using namespace dqds_cfg;
   if (a.map.nk > MAX_LIST) return set_error(FLEXATTN_ENOTSUP, "dq from dS: %d kv tiles, at most %d", a.map.nk, MAX_LIST);
   if (a.ds_rank == nullptr || a.ds_pairs <= 0 || a.ds_pairs > (1ll << 20))
@@ -265,7 +257,6 @@ int bwd_dq_from_ds(const BwdArgs& a, float out_scale, hipStream_t stream) {
   const int n_wg = a.B * a.Hq * (a.Sq / BQ);
   hipLaunchKernelGGL(kern, dim3(n_wg), dim3(256), LDS_BYTES, stream, a, out_scale);
   return check_launch("flexattn_bwd_dq (from dS) bf16");
-#endif
 }
 
 }  // namespace fa

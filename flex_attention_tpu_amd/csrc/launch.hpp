@@ -21,6 +21,9 @@ int bwd_dq_bf16_d256(const BwdArgs& a, hipStream_t stream);
 void bwd_dq_bf16_d128_tile(int* bq, int* bk);
 int bwd_dkv_bf16_d128(const BwdArgs& a, hipStream_t stream);
 int bwd_dkv_bf16_d256(const BwdArgs& a, hipStream_t stream);
+// (the dk/dv pass of such a request runs the generated stream: its exported dS then lacks sm_scale and the soft-cap's
+// factor 4; the kernel with a compiled main loop exports dS complete)
+bool bwd_dkv_bf16_d128_on_stream(int kind, int flags, int nq, bool has_ab, int Hq, int Hkv);
 void bwd_dkv_bf16_d128_tile(int* bq, int* bk);
 // dq = out_scale dS K from the dS blocks that the dk/dv stream kernels wrote to a.ds (a.map: row lists at the
 // dk/dv tiles)

@@ -57,7 +57,7 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
                 need = lib.flexattn_bwd_ds_bytes(C.byref(p))
                 buf = alloc_ds(need, q.device)
                 if buf is not None:
-                    ds = DsBlocks(buf, (B, Hq, Sq_p, Sk_p), index=bm.ds_index())
+                    ds = DsBlocks(buf, (B, Hq, Sq_p, Sk_p), index=bm.ds_index(), compiled_loop=bool(compiled_loop))
                     p.ds, p.ds_bytes = buf.data_ptr(), need
             if ds is None:
                 p.ds_index = _lib.DsIndexC()

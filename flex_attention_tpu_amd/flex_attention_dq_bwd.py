@@ -36,8 +36,10 @@ class DsBlocks:
     The reference's two backward kernels each recompute S, dP and dS (flex_attention_dq_bwd.py:340-378,
     flash_attention_dkv_bwd.py:232-302); handing dS over leaves the dq pass one contraction instead of three."""
 
-    def __init__(self, buf=None, shape=None, index=None):
-        self.buf, self.shape, self.index = buf, shape, index
+    def __init__(self, buf=None, shape=None, index=None, compiled_loop=False):
+        # (compiled_loop: the flag of the dk/dv call; the dq call must carry the same one, the kernel family decides
+        # whether the exported values already hold sm_scale)
+        self.buf, self.shape, self.index, self.compiled_loop = buf, shape, index, compiled_loop
 
 
 # The dS buffer is never allowed to take more than this share of the device's memory, and an out-of-memory error of
@@ -73,8 +75,13 @@ def ds_exchange_pays(score_fn, mask_fn=None, segment_ids=None) -> bool:
     0.56 -> 0.49; softcap, causal, B=4, H=32, S=4096: 2.08 -> 1.86; plain causal, same shape: 1.67 -> 1.68; plain
     causal GQA 4:1, B=2, Hq=32, S=8192: 3.09 -> 3.17."""
     kind = getattr(getattr(score_fn, "spec", None), "kind", _lib.SCORE_NONE if score_fn is None else None)
+    if kind in (_lib.SCORE_CUSTOM, _lib.SCORE_ALIBI_TILE):
+        # kernels with a compiled main loop in both passes: the dq pass from dS is half the recomputing one's time
+        # and evaluates no score function (a compiled closure then costs one backward pass its arithmetic, not two:
+        # B=4, H=32, S=4096, dq + dk/dv in ms, a soft-cap closure 3.12 -> 2.62, the test suite's mixed_mod 5.05 -> 3.50)
+        return True
     if kind not in (_lib.SCORE_NONE, _lib.SCORE_SOFTCAP):
-        return False   # (position biases and compiled score functions: their kernels exchange nothing)
+        return False   # (the global position bias: its dk/dv stream exports nothing, its dq stream is fast)
     if kind == _lib.SCORE_SOFTCAP:
         return True
     if segment_ids is not None:
@@ -133,7 +140,8 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     D_user, D = D, kernel_head_dim(D, q.dtype)   # smaller head dimensions: zero-padded columns
     q, do, k, v = pad_seq(q, D, 3), pad_seq(do, D, 3), pad_seq(k, D, 3), pad_seq(v, D, 3)
     o_p = pad_seq(pad_seq(o, Sq_p), D, 3) if fuse_delta else None
-    if ds is not None and (ds.buf is None or ds.index is None or ds.shape != (B, Hq, Sq_p, Sk_p) or ds.buf.device != q.device):
+    if ds is not None and (ds.buf is None or ds.index is None or ds.shape != (B, Hq, Sq_p, Sk_p) or ds.buf.device != q.device
+                           or ds.compiled_loop != bool(compiled_loop)):
         raise ValueError("ds does not come from a dk/dv pass of these arguments")
     # (the dS blocks lie at the dk/dv kernel's tiles: the dq pass walks that map's row lists)
     bm = kernel_block_map(_lib.PASS_DKV if ds is not None else _lib.PASS_DQ, spec, q, Sq_p, Sk_p, D, score_fn)

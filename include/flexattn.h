@@ -240,14 +240,16 @@ int flexattn_build_ds_index(const flexattn_block_map* map, int32_t* col, int32_t
 /* dS exchange between the two backward passes.  The reference's dq and dk/dv kernels each recompute S, dP and dS
  * (flex_attention_dq_bwd.py:340-378, flash_attention_dkv_bwd.py:232-302).  Here the dk/dv pass can leave its
  * bf16 dS in a caller-allocated device buffer `ds`, and a dq pass that is given the same buffer computes
- * dq = sm_scale dS K from it, one contraction instead of three.  Returns the bytes `ds` must hold for the request
+ * dq = dS K from it, one contraction instead of three (and a compiled score function is evaluated in one pass
+ * instead of two).  Returns the bytes `ds` must hold for the request
  * described by p (B Hq ds_index.pairs 32 KB: one block per query head and kept tile pair; only shapes, dtype, D,
- * flags, score, ab and ds_index.pairs are looked at), or 0 when the kernels of the request exchange nothing
- * (fp32, position biases, an additive bias, compiled score functions, FLEXATTN_FLAG_COMPILED_LOOP, more than
+ * flags, score, ab, the map's nq and ds_index.pairs are looked at), or 0 when the kernels of the request exchange
+ * nothing (fp32, head dimension 256, the global position bias with one query head per kv head, more than
  * 1024 tiles along a sequence, ds_index.pairs <= 0): then ds must stay NULL.
  * Order: flexattn_bwd_dkv with p->ds set, then flexattn_bwd_dq with the same p->ds on the same stream (or
- * ordered behind it); for that dq call p->map is the map at the granularity of FLEXATTN_PASS_DKV with its
- * kv_cnt / kv_idx lists.  With ds == NULL both passes work on their own as before. */
+ * ordered behind it) and the same score, ab and flags (they decide which dk/dv kernel wrote the buffer, and with
+ * it whether the values already carry sm_scale); for that dq call p->map is the map at the granularity of
+ * FLEXATTN_PASS_DKV with its kv_cnt / kv_idx lists.  With ds == NULL both passes work on their own as before. */
 int64_t flexattn_bwd_ds_bytes(const flexattn_bwd_params* p);
 
 /* dq backward.  Replaces the pallas_call in flex_attention_bwd_dq (flex_attention_dq_bwd.py:251-265). */

@@ -111,13 +111,19 @@ def test_ds_exchange_sizes_and_argument_checks(lib):
     assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 2 * 4 * 256 * 384 * 2   # every pair kept: the dense size
     p.score.kind = _lib.SCORE_SOFTCAP
     assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 2 * 4 * 256 * 384 * 2
+    # the dk/dv kernel with a compiled main loop exports too: the tile-local position bias, the global one where kv
+    # heads are grouped, any score on request; the global bias's dk/dv stream (one q head per kv head) does not
     for kind in (_lib.SCORE_ALIBI, _lib.SCORE_ALIBI_TILE):
         p.score.kind = kind
-        assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 0
-    p.score.kind = _lib.SCORE_NONE
-    p.flags = _lib.FLAG_COMPILED_LOOP
+        assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 2 * 4 * 256 * 384 * 2
+    p.score.kind, p.Hkv = _lib.SCORE_ALIBI, 4
     assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 0
-    p.flags, p.dtype = 0, _lib.F32
+    p.score.kind, p.Hkv = _lib.SCORE_NONE, 2
+    p.flags = _lib.FLAG_COMPILED_LOOP
+    assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 2 * 4 * 256 * 384 * 2
+    p.flags, p.D = 0, 256
+    assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 0          # (head dimension 256: no exchange)
+    p.D, p.dtype = 128, _lib.F32
     assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 0
     p.dtype, p.Sq = _lib.BF16, 200          # not a multiple of the dk/dv tile
     assert lib.flexattn_bwd_ds_bytes(C.byref(p)) == 0

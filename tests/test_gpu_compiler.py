@@ -85,6 +85,27 @@ def test_closures_that_equal_a_builtin_functor_run_its_kernels(F):
         assert_close(closure.__name__ + " o", results[0][0], ro, torch.bfloat16)
 
 
+def test_autograd_through_a_compiled_closure(F, compiled):
+    """torch.autograd.grad through flex_attention with a compiled score function and a compiled mask: the backward
+    hands dS from the dk/dv pass to the dq pass by itself (the score function is evaluated in one backward pass)."""
+    name = "mixed_mod+prefix_lm"
+    score_fn, mask_pair = compiled[name]
+    B, Hq, Hkv, S = 2, 4, 2, 512
+    sc = 1 / math.sqrt(128)
+    q, k, v, do = O.make_inputs(B, Hq, Hkv, S, S, 128, dtype=torch.bfloat16, seed=67)
+    okw = dict(sm_scale=sc, **_oracle_kwargs(name, S, S))
+    ro, rl, rm = O.mha_reference(q, k, v, save_residuals=True, **okw)
+    rdq, rdk, rdv = O.mha_bwd_reference(q, k, v, ro, do, rl, rm, **okw)
+    qg, kg, vg = [x.to(DEV).requires_grad_(True) for x in (q, k, v)]
+    o = F.flex_attention(qg, kg, vg, score_fn, mask_pair, sm_scale=sc)
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), do.to(DEV))
+    assert_close("o", o, ro, torch.bfloat16)
+    for nm, t, c in zip(("dq", "dk", "dv"), (dq, dk, dv), (rdq, rdk, rdv)):
+        assert_close(nm + " chain", t, c, torch.bfloat16, chain=True)
+    from flex_attention_tpu_amd.flex_attention_dq_bwd import ds_exchange_pays
+    assert ds_exchange_pays(score_fn, mask_pair[0])
+
+
 def _closures_all_passes(F, compiled, name, dtype, D):
     score_fn, mask_pair = compiled[name]
     B, Hq, Hkv, S = 2, 4, 2, 512
@@ -111,6 +132,18 @@ def _closures_all_passes(F, compiled, name, dtype, D):
     for nm, t, r, c in zip(("dq", "dk", "dv"), (dq, dk, dv), same, (rdq, rdk, rdv)):
         assert_close(nm, t, r, dtype)
         assert_close(nm + " chain", t, c, dtype, chain=True)
+    # the backward that hands dS from the dk/dv pass to the dq pass (bf16 at head dimension 128): the same dk, dv,
+    # and a dq for which no score function is evaluated a second time; a compiled mask alone runs the streams
+    kw = dict(block_b=1, block_q=128, block_k_major=128, block_k=128, sm_scale=sc, debug=False, score_fn=score_fn,
+              mask_fn=mf, block_mask_fn=bf)
+    dk2, dv2, ds = F.flash_attention_bwd_dkv(kg, vg, qg, None, None, l, m, d, dog, block_q_major=128, causal=False,
+                                             return_ds=True, **kw)
+    assert torch.equal(dk2, dk) and torch.equal(dv2, dv), "dk, dv change when dS is exported"
+    assert (ds is not None) == (dtype == torch.bfloat16 and D == 128)
+    if ds is not None:
+        dqx = F.flex_attention_bwd_dq(qg, kg, vg, None, None, l, m, o, dog, d, ds=ds, **kw)
+        assert_close("dq from dS", dqx, same[0], dtype)
+        assert_close("dq from dS chain", dqx, rdq, dtype, chain=True)
 
 
 def test_compiled_alibi_equals_the_builtin_functor(F, compiled):

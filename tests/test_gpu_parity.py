@@ -230,9 +230,10 @@ def test_small_shapes_all_passes(F, case, dtype):
                                         block_k=128, sm_scale=sc, debug=False, score_fn=score_fn, mask_fn=mf,
                                         block_mask_fn=bf, return_delta=True)
     assert torch.equal(d_f, d) and torch.equal(dq_f, dq), "delta taken by the dq pass differs from the delta kernel's"
-    # dS exchange: the bf16 stream kernels of plain and softcap scores offer it
+    # dS exchange: the bf16 stream kernels of plain and softcap scores offer it, and the dk/dv kernel with a compiled
+    # main loop (the tile-local position bias); the global position bias's dk/dv stream does not
     dqx = _exchanged_dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, score_fn, dk, dv,
-                        expect=dtype == torch.bfloat16 and not name.startswith("alibi"))
+                        expect=dtype == torch.bfloat16 and name != "alibi_global")
     if dqx is not None:
         _check_grads((dqx, dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, dtype, dict(sm_scale=sc, **okw), tag="exchange ")
 
