@@ -21,8 +21,8 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     of all query heads of a group are summed inside the kernel.  ``causal`` is honoured
     (the reference's north-star file ignores it; its mask-aware twin gets the same effect from
     ``mask_fn``).  ``return_ds=True`` returns (dk, dv, ds): ds is the pass's dS as a DsBlocks for
-    ``flex_attention_bwd_dq(..., ds=ds)``, or None when the kernels of the call exchange nothing (fp32, position
-    biases, ``ab``, compiled score functions) or the device has too little free memory for the buffer (one 32 KB
+    ``flex_attention_bwd_dq(..., ds=ds)``, or None when the kernels of the call exchange nothing (fp32, head
+    dimension 256, the global position bias with one query head per kv head) or the device has too little free memory for the buffer (one 32 KB
     block per query head and kept pair of 128 x 128 tiles): the dq pass then recomputes as usual."""
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v, do)
     for name, t in (("l", l), ("m", m), ("di", di)):
