@@ -74,6 +74,7 @@ class BlockMap:
         self.built_on = None   # stream the builder kernel was launched on
         self.ready = None      # event recorded behind it
         self._ds_index = None  # (col, rank, pairs) of the dS exchange buffer, built at first use
+        self._partial_share = None
 
     def _tensors(self):
         t = [self.state, self.kv_cnt, self.kv_idx, self.q_cnt, self.q_idx]
@@ -110,6 +111,14 @@ class BlockMap:
                 pairs = int(col[-1].item())
             self._ds_index = (col, rank, pairs)
         return self._ds_index
+
+    def partial_share(self) -> float:
+        """Share of the tiles that run which are partly masked (read back from the device once per map)."""
+        if self._partial_share is None:
+            self.wait_ready(self.state.device)
+            run = int((self.state != 0).sum().item())
+            self._partial_share = (int((self.state == 1).sum().item()) / run) if run else 0.0
+        return self._partial_share
 
     def ds_index_c(self) -> _lib.DsIndexC:
         col, rank, pairs = self.ds_index()

@@ -8,7 +8,7 @@ import torch
 
 from . import _lib
 from ._common import (on_device, bias_c, check_blocks, check_doc_batches, check_qkv, check_rows, dtype_code, kernel_block_map, kernel_head_dim, library_for,
-                      pad_seq, padded_len, resolve_mask, score_spec_c, stream_of)
+                      pad_seq, padded_len, mostly_partial_custom_mask, resolve_mask, score_spec_c, stream_of)
 from .block_mask import mask_spec_c
 
 
@@ -145,6 +145,8 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
         raise ValueError("ds does not come from a dk/dv pass of these arguments")
     # (the dS blocks lie at the dk/dv kernel's tiles: the dq pass walks that map's row lists)
     bm = kernel_block_map(_lib.PASS_DKV if ds is not None else _lib.PASS_DQ, spec, q, Sq_p, Sk_p, D, score_fn)
+    if ds is None and mostly_partial_custom_mask(spec, bm):
+        compiled_loop = True
     dq = torch.empty_like(q)
     ab_c, ab_keep = bias_c(ab, B, Hq, Sq, Sk, Sq_p, Sk_p, q.device)
     p = bwd_params(q, k, v, l, m, do, d_p, sm_scale, score_fn, spec, bm, block_q or 1, block_k or 1, dq=dq,

@@ -13,7 +13,7 @@ import torch
 
 from . import _lib
 from ._common import (on_device, bias_c, check_blocks, check_doc_batches, check_qkv, dtype_code, kernel_block_map, kernel_head_dim, library_for, pad_seq,
-                      padded_len, resolve_mask, score_spec_c, stream_of)
+                      padded_len, mostly_partial_custom_mask, resolve_mask, score_spec_c, stream_of)
 from .block_mask import mask_spec_c
 
 
@@ -39,6 +39,7 @@ def _flex_attention_impl(q, k, v, ab, segment_ids, save_residuals, causal, sm_sc
     D_user, D = D, kernel_head_dim(D, q.dtype)   # smaller head dimensions: zero-padded columns
     q, k, v = pad_seq(q, D, 3), pad_seq(k, D, 3), pad_seq(v, D, 3)
     bm = kernel_block_map(_lib.PASS_FWD, spec, q, Sq_p, Sk_p, D, score_fn)
+    compiled_loop = compiled_loop or mostly_partial_custom_mask(spec, bm)
     ab_c, ab_keep = bias_c(ab, B, Hq, Sq, Sk, Sq_p, Sk_p, q.device)
     o = torch.empty_like(q)
     l = m = None
