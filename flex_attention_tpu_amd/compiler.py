@@ -1056,8 +1056,8 @@ def compile_score_fn(fn: Callable) -> Callable:
 
 
 def _recognised_mask_fns(expr: Node, block_q: int, block_k: int):
-    """The (mask_fn, block_mask_fn) pair of this package's own factories (causal, sliding window, both) if the
-    predicate equals one of them, else None: those masks have closed-form block maps and run the generated-stream
+    """The (mask_fn, block_mask_fn) pair of this package's own factories (causal, sliding window, both, the S2 local
+    + strided mask) if the predicate equals one of them, else None: those masks have closed-form block maps and run the generated-stream
     kernels.  Numeric, on the expression tree: the keys kept by one query far out (position 2^22) give the
     candidate's window, and the factory's own ``mask_fn`` must then agree with the predicate on index grids around
     the origin, around that query and around both ends of its window."""
@@ -1077,27 +1077,41 @@ def _recognised_mask_fns(expr: Node, block_q: int, block_k: int):
     causal = int(kept[-1]) == i0
     if not causal and int(kept[-1]) != i0 + 63:
         return None
-    window = i0 - int(kept[0]) + 1 if int(kept[0]) > 0 else None
+    # the run of kept keys that ends at the query is the window; kept keys in front of it at equal distances from
+    # key 0 on are the strided part of the reference's S2 mask (masks.py:143-179)
+    gaps = torch.nonzero(kept[1:] - kept[:-1] != 1).flatten()
+    run_start = int(kept[int(gaps[-1]) + 1]) if gaps.numel() else int(kept[0])
+    stride = None
+    if causal and gaps.numel() and int(kept[0]) == 0 and kept.numel() > 1:
+        stride = int(kept[1])
+    window = i0 - run_start + 1 if run_start > 0 else None
     if not causal and window is None:
         return None      # (keeps everything: no mask is the caller's way to say so)
-    if causal and window is None:
-        cand = masks.make_causal_mask_fns(block_q, block_k)
+    if stride is not None and window is not None and stride > 1:
+        # (a strided key right in front of the window joins its run: the window one shorter is tried as well)
+        cands = [masks.make_s2_mask_fns(block_q, block_k, w_, stride) for w_ in (window, window - 1) if w_ > 0]
+    elif gaps.numel():
+        return None      # (kept keys in pieces that are no S2 pattern)
+    elif causal and window is None:
+        cands = [masks.make_causal_mask_fns(block_q, block_k)]
     elif causal:
-        cand = masks.make_causal_sliding_window_mask_fns(block_q, block_k, window)
+        cands = [masks.make_causal_sliding_window_mask_fns(block_q, block_k, window)]
     else:
-        cand = masks.make_sliding_window_mask_fns(block_q, block_k, window)
+        cands = [masks.make_sliding_window_mask_fns(block_q, block_k, window)]
     w = window or 0
     grids = [(torch.arange(0, 320), torch.arange(0, 320)),
              (torch.arange(i0 - 96, i0 + 96), torch.arange(i0 - 96, i0 + 96)),
              (torch.arange(i0 - 96, i0 + 96), torch.arange(max(0, i0 - w - 96), i0 - w + 96)),
-             (torch.arange(max(0, w - 96), w + 96), torch.arange(0, 192))]
+             (torch.arange(max(0, w - 96), w + 96), torch.arange(0, 192)),
+             (torch.arange(1000, 1192), torch.arange(0, 1200))]
     try:
-        for qi, kj in grids:
-            if not torch.equal(ev(qi, kj), torch.as_tensor(cand[0](qi, kj)).to(torch.bool)):
-                return None
+        want = [ev(qi, kj) for qi, kj in grids]
+        for cand in cands:
+            if all(torch.equal(x, torch.as_tensor(cand[0](qi, kj)).to(torch.bool)) for x, (qi, kj) in zip(want, grids)):
+                return cand
     except Exception:  # noqa: BLE001
         return None
-    return cand
+    return None
 
 
 def compile_mask_fn(fn: Callable, block_q: int, block_k: int, recognise: bool = True) -> Tuple[Callable, Callable]:

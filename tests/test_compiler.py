@@ -127,6 +127,16 @@ def _causal_window_and_a_sink(q_idx, k_idx):
     return ((d >= 0) & (d <= 1024)) | (k_idx[None, :] == 7)
 
 
+def _s2(q_idx, k_idx):
+    d = q_idx[:, None] - k_idx[None, :]
+    return ((d >= 0) & (d < 128)) | ((k_idx[None, :] % 64 == 0) & (d >= 0))
+
+
+def _s2_shifted(q_idx, k_idx):
+    d = q_idx[:, None] - k_idx[None, :]
+    return ((d >= 0) & (d < 128)) | ((k_idx[None, :] % 64 == 3) & (d >= 0))
+
+
 def _identity(s, b, h, q_idx, kv_idx):
     return s
 
@@ -160,6 +170,9 @@ def test_closures_that_equal_a_builtin_functor_get_it():
         assert torch.equal(torch.as_tensor(mf(qi, kj)), torch.as_tensor(fn(qi, kj)))
         assert compiler.compile_mask_fn(fn, 128, 64, recognise=False)[0].spec.flags == _lib.MASK_CUSTOM
     assert compiler.compile_mask_fn(_causal_window_and_a_sink, 128, 64)[0].spec.flags == _lib.MASK_CUSTOM
+    s2 = compiler.compile_mask_fn(_s2, 128, 64)[0].spec      # the reference's local + strided mask (masks.py:143-179)
+    assert (s2.flags, s2.window, s2.stride, s2.custom) == (_lib.MASK_S2, 128, 64, None)
+    assert compiler.compile_mask_fn(_s2_shifted, 128, 64)[0].spec.flags == _lib.MASK_CUSTOM
     assert compiler.compile_score_mod(_identity).spec == scores.ScoreSpec(kind=_lib.SCORE_NONE)
     assert compiler.compile_score_mod(_softcap).spec == scores.ScoreSpec(kind=_lib.SCORE_SOFTCAP, cap=50.0)
     assert compiler.compile_score_mod(_softcap, recognise=False).spec.kind == _lib.SCORE_CUSTOM
