@@ -115,6 +115,68 @@ def segment_doc_ids(segment_ids):
     return _doc_ids_of(segment_ids), None
 
 
+_tagged_closures = weakref.WeakKeyDictionary()   # plain Python closure -> its compiled (tagged) form
+
+
+def _remembered(fn):
+    try:
+        return _tagged_closures.get(fn)
+    except TypeError:   # (a callable that cannot be weakly referenced or hashed: compiled again at every call;
+        return None     #  the functor libraries themselves are cached by their source)
+
+
+def _remember(fn, compiled) -> None:
+    try:
+        _tagged_closures[fn] = compiled
+    except TypeError:
+        pass
+
+
+def tagged_closures(score_fn, mask_fn, block_mask_fn, block_q, block_k):
+    """(score_fn, mask_fn, block_mask_fn) with plain Python closures replaced by their compiled forms, so that a
+    caller may hand the entry points the functions themselves, as the reference's callers hand theirs to its
+    kernels (flex_attention_kernel.py:248-255, 278-288): a score function of two arguments is the reference's tile
+    form (util.make_jax_score_fn), one of five the element-wise ``score_mod(s, b, h, q_idx, kv_idx)``
+    (compiler.compile_score_mod); a ``mask_fn(q_idx, k_idx)`` goes to compiler.compile_mask_fn at the call's block
+    sizes, which also derives the block closure (a block closure without a mask function cannot be compiled: it
+    says which tiles run, not which elements).  Closures that carry a ``.spec`` pass through; the compiled form of
+    a function object is kept while the function lives."""
+    import inspect
+
+    def arity(fn):
+        try:
+            ps = inspect.signature(fn).parameters.values()
+        except (TypeError, ValueError):
+            return -1
+        return sum(1 for p in ps if p.kind in (p.POSITIONAL_ONLY, p.POSITIONAL_OR_KEYWORD) and p.default is p.empty)
+    if score_fn is not None and not isinstance(getattr(score_fn, "spec", None), ScoreSpec):
+        hit = _remembered(score_fn)
+        if hit is None:
+            n = arity(score_fn)
+            if n == 2:
+                from . import util
+                hit = util.make_jax_score_fn(score_fn)
+            elif n == 5:
+                from . import compiler
+                hit = compiler.compile_score_mod(score_fn)
+            else:
+                raise NotImplementedError("score_fn must take (q_tile, k_tile) or (s, b, h, q_idx, kv_idx), or come from "
+                                          "flex_attention_tpu_amd.scores / util.make_jax_score_fn / compiler.compile_score_mod")
+            _remember(score_fn, hit)
+        score_fn = hit
+    if mask_fn is not None and getattr(mask_fn, "spec", None) is None:
+        key = (int(block_q or SEQ_ALIGN), int(block_k or SEQ_ALIGN))
+        per_fn = _remembered(mask_fn)
+        if per_fn is None:
+            per_fn = {}
+            _remember(mask_fn, per_fn)
+        if key not in per_fn:
+            from . import compiler
+            per_fn[key] = compiler.compile_mask_fn(mask_fn, *key)
+        mask_fn, block_mask_fn = per_fn[key]
+    return score_fn, mask_fn, block_mask_fn
+
+
 def check_doc_batches(spec: MaskSpec, B: int) -> None:
     """Document ids with a row per batch entry must have one for every entry of the call."""
     for d in (spec.doc_ids, spec.doc_ids_k):

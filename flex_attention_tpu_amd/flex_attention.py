@@ -125,8 +125,11 @@ def flex_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, score_fn: 
                    ab: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Differentiable flex attention on ``[B, H, S, D]`` GPU tensors (k, v may have fewer heads: GQA).
 
-    ``score_fn``   closure from ``scores`` (or ``util.make_jax_score_fn``), or None
-    ``mask_fns``   ``(mask_fn, block_mask_fn)`` pair from ``masks``, or None
+    ``score_fn``   closure from ``scores`` (or ``util.make_jax_score_fn`` / ``compiler.compile_score_mod``), a plain
+                   Python function ``f(q_tile, k_tile)`` or ``f(s, b, h, q_idx, kv_idx)`` (compiled at first use), or None
+    ``mask_fns``   ``(mask_fn, block_mask_fn)`` pair from ``masks`` (or ``compiler.compile_mask_fn``), a pair whose
+                   ``mask_fn(q_idx, k_idx)`` is a plain Python function (compiled at first use, the block closure
+                   derived from it), such a function alone, or None
     ``segment_ids`` / ``causal``   as in the three entry points (ANDed with ``mask_fns``)
     ``sm_scale``   default 1 / sqrt(D)
     ``ab``         additive bias on the logits, [B or 1, H or 1, Sq, Sk]; a bias that requires grad receives
@@ -137,6 +140,11 @@ def flex_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, score_fn: 
     """
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(q.shape[-1])
-    mask_fn, block_mask_fn = mask_fns if mask_fns is not None else (None, None)
+    if callable(mask_fns):   # (a bare mask function instead of a pair)
+        mask_fn, block_mask_fn = mask_fns, None
+    else:
+        mask_fn, block_mask_fn = mask_fns if mask_fns is not None else (None, None)
+    from ._common import tagged_closures
+    score_fn, mask_fn, block_mask_fn = tagged_closures(score_fn, mask_fn, block_mask_fn, block_q, block_k)
     opts = (score_fn, mask_fn, block_mask_fn, segment_ids, bool(causal), float(sm_scale), int(block_q), int(block_k))
     return _FlexAttention.apply(q, k, v, ab, opts)

@@ -9,7 +9,7 @@ import torch
 
 from . import _lib
 from ._common import (on_device, bias_c, check_blocks, check_doc_batches, check_qkv, check_rows, kernel_block_map, kernel_head_dim, library_for, pad_seq,
-                      padded_len, resolve_mask, stream_of)
+                      padded_len, resolve_mask, stream_of, tagged_closures)
 from .flex_attention_dq_bwd import DsBlocks, alloc_ds, bwd_params
 
 
@@ -25,6 +25,7 @@ def flash_attention_bwd_dkv(k, v, q, ab, segment_ids, l, m, di, do, *, block_b=N
     dimension 256, the global position bias with one query head per kv head) or the device has too little free memory for the buffer (one 32 KB
     block per query head and kept pair of 128 x 128 tiles): the dq pass then recomputes as usual."""
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v, do)
+    score_fn, mask_fn, block_mask_fn = tagged_closures(score_fn, mask_fn, block_mask_fn, block_q, block_k_major)
     for name, t in (("l", l), ("m", m), ("di", di)):
         check_rows(name, t, B, Hq, Sq, q.device)
     check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k,

@@ -8,7 +8,7 @@ import torch
 
 from . import _lib
 from ._common import (on_device, bias_c, check_blocks, check_doc_batches, check_qkv, check_rows, dtype_code, kernel_block_map, kernel_head_dim, library_for,
-                      pad_seq, padded_len, mostly_partial_custom_mask, resolve_mask, score_spec_c, stream_of)
+                      pad_seq, padded_len, mostly_partial_custom_mask, resolve_mask, score_spec_c, stream_of, tagged_closures)
 from .block_mask import mask_spec_c
 
 
@@ -119,6 +119,7 @@ def flex_attention_bwd_dq(q, k, v, ab, segment_ids, l, m, o, do, d, *, block_b, 
     reference declares next to dk, dv (flash_attention_dkv_bwd.py:103-107,130-138) and its upstream dq kernel
     writes (jax_exp.py:1252-1255; there multiplied by sm_scale)."""
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v, do)
+    score_fn, mask_fn, block_mask_fn = tagged_closures(score_fn, mask_fn, block_mask_fn, block_q, block_k_major)
     if o is not None and tuple(o.shape) != tuple(q.shape):
         raise ValueError(f"o has shape {tuple(o.shape)}, expected {tuple(q.shape)}")
     fuse_delta = d is None

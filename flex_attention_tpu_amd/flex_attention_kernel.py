@@ -13,7 +13,7 @@ import torch
 
 from . import _lib
 from ._common import (on_device, bias_c, check_blocks, check_doc_batches, check_qkv, dtype_code, kernel_block_map, kernel_head_dim, library_for, pad_seq,
-                      padded_len, mostly_partial_custom_mask, resolve_mask, score_spec_c, stream_of)
+                      padded_len, mostly_partial_custom_mask, resolve_mask, score_spec_c, stream_of, tagged_closures)
 from .block_mask import mask_spec_c
 
 
@@ -30,6 +30,7 @@ def _flex_attention_impl(q, k, v, ab, segment_ids, save_residuals, causal, sm_sc
     """
     B, Hq, Hkv, Sq, Sk, D = check_qkv(q, k, v)
     check_blocks(Sq, Sk, block_q=block_q, block_k_major=block_k_major, block_k=block_k)
+    score_fn, mask_fn, block_mask_fn = tagged_closures(score_fn, mask_fn, block_mask_fn, block_q, block_k_major)
     # ragged lengths: the tensors are zero-padded to the kernels' tiles, a key bound drops the padded keys
     # and the padded query rows are cut off again
     Sq_p, Sk_p = padded_len(Sq), padded_len(Sk)

@@ -198,6 +198,30 @@ def test_powers_with_variable_exponents():
         compiler.compile_score_mod(lambda s, b, h, q_idx, kv_idx: (-2.0) ** h + s)
 
 
+def test_plain_closures_are_compiled_at_the_entry_points():
+    """tagged_closures, which every entry point calls first: a function object without a specification is compiled
+    by its form (two arguments: the reference's tile form; five: score_mod; a mask function at the call's block
+    sizes, with its block closure), once per function object; what carries a specification passes through."""
+    from flex_attention_tpu_amd import masks, scores
+    from flex_attention_tpu_amd._common import tagged_closures
+
+    def tile_softcap(q_tile, k_tile):
+        return 30.0 * torch.tanh(torch.matmul(q_tile, k_tile.T) / 30.0)
+    s1, m1, b1 = tagged_closures(tile_softcap, _causal_window, None, 128, 128)
+    assert s1.spec == scores.ScoreSpec(kind=_lib.SCORE_SOFTCAP, cap=30.0)
+    assert m1.spec.flags == _lib.MASK_CAUSAL | _lib.MASK_WINDOW and m1.spec.window == 1025 and b1.spec == m1.spec
+    s2, m2, b2 = tagged_closures(tile_softcap, _causal_window, None, 128, 128)
+    assert s2 is s1 and m2 is m1 and b2 is b1                       # (compiled once)
+    assert tagged_closures(_softcap, None, None, 128, 128)[0].spec.kind == _lib.SCORE_SOFTCAP
+    assert tagged_closures(cf.mixed_mod, cf.checker_mask, None, 128, 64)[0].spec.kind == _lib.SCORE_CUSTOM
+    assert tagged_closures(None, cf.checker_mask, None, 128, 64)[1].spec.flags == _lib.MASK_CUSTOM
+    fac_s, fac_m = scores.make_softcap_score_fn(5.0), masks.make_causal_mask_fns(128, 128)
+    assert tagged_closures(fac_s, fac_m[0], fac_m[1], 128, 128) == (fac_s, fac_m[0], fac_m[1])
+    assert tagged_closures(None, None, None, 128, 128) == (None, None, None)
+    with pytest.raises(NotImplementedError, match="score_fn must take"):
+        tagged_closures(lambda a, b, c: a, None, None, 128, 128)
+
+
 def test_unsupported_constructs_are_refused():
     def uses_softmax(s, b, h, q_idx, kv_idx):
         return torch.softmax(s, -1)

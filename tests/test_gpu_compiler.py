@@ -106,6 +106,38 @@ def test_autograd_through_a_compiled_closure(F, compiled):
     assert ds_exchange_pays(score_fn, mask_pair[0])
 
 
+def test_plain_python_closures_through_the_entry_points(F):
+    """Plain Python functions handed to the entry points and to flex_attention themselves (no factory, no explicit
+    compile step), as the reference's callers hand theirs to its kernels: these two are recognised, so the calls
+    give the bits of the factories' closures."""
+    from flex_attention_tpu_amd import masks, scores
+    B, Hq, Hkv, S = 1, 4, 2, 768
+    sc = 1 / math.sqrt(128)
+    q, k, v, do = [x.to(DEV) for x in O.make_inputs(B, Hq, Hkv, S, S, 128, dtype=torch.bfloat16, seed=79)]
+    fm, fs = masks.make_causal_sliding_window_mask_fns(128, 128, 200), scores.make_softcap_score_fn(30.0)
+    want = F._flex_attention_impl(q, k, v, None, None, True, False, sc, 1, 128, 128, 128, False, fm[1], fm[0], fs)
+    got = F._flex_attention_impl(q, k, v, None, None, True, False, sc, 1, 128, 128, 128, False, None, cf.causal_window_mask,
+                                 cf.softcap30_mod)
+    for name, a, b in zip(("o", "l", "m"), got, want):
+        assert torch.equal(a, b), name
+    o, l, m = want
+    d = F.compute_delta(o, do)
+    kw = dict(block_b=1, block_q=128, block_k_major=128, block_k=128, sm_scale=sc, debug=False)
+    dq = F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, score_fn=cf.softcap30_mod, mask_fn=cf.causal_window_mask, **kw)
+    dk, dv = F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_q_major=128, causal=False,
+                                       score_fn=cf.softcap30_mod, mask_fn=cf.causal_window_mask, **kw)
+    assert torch.equal(dq, F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, score_fn=fs, mask_fn=fm[0],
+                                                   block_mask_fn=fm[1], **kw))
+    wk, wv = F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_q_major=128, causal=False, score_fn=fs,
+                                       mask_fn=fm[0], block_mask_fn=fm[1], **kw)
+    assert torch.equal(dk, wk) and torch.equal(dv, wv)
+    qa = q.clone().requires_grad_(True)
+    oa = F.flex_attention(qa, k, v, cf.softcap30_mod, cf.causal_window_mask, sm_scale=sc)
+    assert torch.equal(oa.detach(), o)
+    (ga,) = torch.autograd.grad(oa, (qa,), do)
+    assert torch.equal(ga, dq)
+
+
 def _closures_all_passes(F, compiled, name, dtype, D):
     score_fn, mask_pair = compiled[name]
     B, Hq, Hkv, S = 2, 4, 2, 512
