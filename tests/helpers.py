@@ -30,7 +30,9 @@ def assert_close(name, test, ref, dtype, chain=False, tensor_scale=False):
     of the dS and k terms it sums (dS is rounded to bf16 for the product, in the reference's kernels as here), whose
     size is the row's, not the element's.  For tensors up to 2.56 in magnitude that is the literal 2e-2.
 
-    float32: max-abs <= 1e-5 and rel-L2 <= 1e-5, as written.
+    float32: max-abs <= 1e-5 and rel-L2 <= 1e-5, as written; with `tensor_scale=True` the absolute bound is
+    1e-5 max(1, max|ref|) (a float32 sum of a thousand terms that reaches 7 is spaced 5e-7 apart: 1e-5 is twenty
+    of its steps).
     bfloat16: rel-L2 <= 1e-2 and, element by element, |test - ref| <= max(2e-2, 2^-7 |ref|).  The
     second term only matters where |ref| > 2.56: a bf16 result is spaced 2^-7 |ref| apart there
     (two neighbours at |ref| = 4 are 0.031 apart), so the literal 2e-2 is finer than the output
@@ -59,7 +61,7 @@ def assert_close(name, test, ref, dtype, chain=False, tensor_scale=False):
         ratio = float(((test - ref).abs() / bound).max())
         rel_tol = BF16_REL
     else:
-        ratio = ma / F32_ABS
+        ratio = ma / (F32_ABS * (max(1.0, ref_max) if tensor_scale else 1.0))
         rel_tol = F32_REL
     REPORT.append((CURRENT, name, ref_max, ma, rl, ratio))
     assert rl <= rel_tol, f"{name}: rel-L2 {rl:.3e} > {rel_tol:.1e} (max-abs {ma:.3e})"
