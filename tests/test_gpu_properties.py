@@ -333,3 +333,37 @@ def test_segment_ids_per_batch_entry_properties(F):
         part = passes(*[x[b:b + 1].contiguous() for x in (q, k, v, do)], sid[b])
         for n, a, b_ in zip(names, part, full):
             _same(f"{n} of entry {b} alone", a, b_[b:b + 1])
+
+
+def test_tensors_beyond_2_31_elements(F):
+    """q, o, dO, dq of 2.3 * 2^30 elements each (B=16, Hq=136, S=8192, D=128; 36 GiB on the device for the eight
+    tensors): element offsets do not fit 32 bits from the thirteenth batch entry on.  The last entry of the launch
+    must equal that entry launched alone, bit for bit, in every pass; under a causal mask and under a causal window
+    with a softcap (stream kernels of two kinds, grouped kv heads, the persistent schedules)."""
+    import math
+    import warnings
+    from flex_attention_tpu_amd import masks, scores
+    warnings.filterwarnings("ignore", message="score_fn with sm_scale")
+    B, Hq, Hkv, S, D = 16, 136, 34, 8192, 128
+    assert B * Hq * S * D > 2 ** 31
+    free, _ = torch.cuda.mem_get_info()
+    if free < 60 * 2 ** 30:
+        pytest.skip("needs 60 GiB of free device memory")
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    q, k, v, do = [torch.randn(B, h, S, D, device=DEV, dtype=torch.bfloat16, generator=gen) for h in (Hq, Hkv, Hkv, Hq)]
+    sc = 1 / math.sqrt(D)
+    for (mf, bf), sfn in ((masks.make_causal_mask_fns(128, 128), None),
+                          (masks.make_causal_sliding_window_mask_fns(128, 128, 1000), scores.make_softcap_score_fn(30.0))):
+        def passes(q, k, v, do):
+            o, l, m = F._flex_attention_impl(q, k, v, None, None, True, False, sc, 1, 128, 128, 128, False, bf, mf, sfn)
+            d = F.compute_delta(o, do)
+            kw = dict(block_b=1, block_q=128, block_k_major=128, block_k=128, sm_scale=sc, debug=False, score_fn=sfn,
+                      mask_fn=mf, block_mask_fn=bf)
+            dq = F.flex_attention_bwd_dq(q, k, v, None, None, l, m, o, do, d, **kw)
+            dk, dv = F.flash_attention_bwd_dkv(k, v, q, None, None, l, m, d, do, block_q_major=128, causal=False, **kw)
+            return o, l, m, d, dq, dk, dv
+        full = [x[-1:].clone() for x in passes(q, k, v, do)]
+        alone = passes(*[x[-1:].contiguous() for x in (q, k, v, do)])
+        for n, a, b_ in zip(("o", "l", "m", "delta", "dq", "dk", "dv"), alone, full):
+            _same(f"{n} of the last entry alone", a, b_)
+        del full, alone
