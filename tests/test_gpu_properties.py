@@ -367,3 +367,54 @@ def test_tensors_beyond_2_31_elements(F):
         for n, a, b_ in zip(("o", "l", "m", "delta", "dq", "dk", "dv"), alone, full):
             _same(f"{n} of the last entry alone", a, b_)
         del full, alone
+
+
+@pytest.mark.parametrize("case", ["causal", "softcap_documents"])
+def test_entry_points_replayed_from_a_captured_graph(F, case):
+    """The three entry points recorded into a HIP graph (torch.cuda.graph, after two warm-up steps on a side stream:
+    the block map of a mask is built once and kept) and replayed on new inputs: every replay gives the bits of the
+    same calls made eagerly, the dS hand-over included.  Eager work and synchronisations lie between the replays."""
+    import math
+    import warnings
+    from flex_attention_tpu_amd import masks, scores
+    warnings.filterwarnings("ignore", message="score_fn with sm_scale")
+    B, Hq, Hkv, S, D = 2, 8, 2, 2048, 128
+    sc = 1 / math.sqrt(D)
+    gen = torch.Generator(device=DEV).manual_seed(3)
+    q, k, v, do = [torch.randn(B, h, S, D, device=DEV, dtype=torch.bfloat16, generator=gen) for h in (Hq, Hkv, Hkv, Hq)]
+    mf, bf, sfn, sid = *masks.make_causal_mask_fns(128, 128), None, None
+    if case == "softcap_documents":
+        mf = bf = None
+        sfn = scores.make_softcap_score_fn(30.0)
+        sid = torch.repeat_interleave(torch.arange(4), torch.tensor([300, 700, 48, 1000])).to(torch.int32)
+
+    def step(q, k, v, do):
+        o, l, m = F._flex_attention_impl(q, k, v, None, sid, True, sid is not None, sc, 1, 128, 128, 128, False, bf, mf, sfn)
+        d = F.compute_delta(o, do)
+        kw = dict(block_b=1, block_q=128, block_k_major=128, block_k=128, sm_scale=sc, debug=False, score_fn=sfn,
+                  mask_fn=mf, block_mask_fn=bf, causal=sid is not None)
+        dq = F.flex_attention_bwd_dq(q, k, v, None, sid, l, m, o, do, d, **kw)
+        dk, dv, ds = F.flash_attention_bwd_dkv(k, v, q, None, sid, l, m, d, do, block_q_major=128, return_ds=True, **kw)
+        dqx = F.flex_attention_bwd_dq(q, k, v, None, sid, l, m, o, do, d, ds=ds, **kw)
+        return o, l, m, dq, dk, dv, dqx
+    static = [x.clone() for x in (q, k, v, do)]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step(*static)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = step(*static)
+    for rep in range(3):
+        fresh = [x * (1 + 0.25 * rep) for x in (q, k, v, do)]
+        for s_, f_ in zip(static, fresh):
+            s_.copy_(f_)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = step(*fresh)
+        torch.cuda.synchronize()
+        for n, a, b_ in zip(("o", "l", "m", "dq", "dk", "dv", "dq from dS"), out, eager):
+            _same(f"{n} of replay {rep}", a, b_)
