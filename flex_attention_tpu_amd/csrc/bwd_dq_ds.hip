@@ -9,10 +9,12 @@
 // operands with transposing LDS reads: computed transposed, dq^T[d, i] += sum_j K^T[d, j] dS^T[j, i], the lane
 // that owned kv column j in the dk/dv kernel wrote 8 q rows of it contiguously, which is what
 // ds_read_b64_tr_b16 turns into "lane owns q row i, 4 consecutive j".  The kernel moves 32 KB of dS and 32 KB of K
-// per 32 MFMAs and wave; the matrix pipe is busy a quarter of the time.  Measured with cycle stamps per 32-column
-// stage and wave: waiting for the copies 180-255, barrier 100-140, issuing the wave's four copies 700 (an
-// LDS-direct copy of 1 KB holds the issuing wave about 175 cycles when all eight waves of the CU copy at once),
-// LDS reads and MFMAs 410.
+// per 32 MFMAs and computing wave; the matrix pipe is busy a quarter of the time and the copies bound the launch.
+// On B=4, H=32, S=4096 causal (2.2 GB of dS, as many bytes of K from the L2): 0.51 ms; the same launch without the
+// LDS reads and MFMAs 0.50 ms; the dS copies alone 0.41 ms (5.4 TB/s, what 80 KB in flight per CU draw from HBM:
+// the rings are the buffer of the bytes in flight and the LDS holds no deeper ones next to the K ring), the K copies
+// alone 0.18 ms.  Ring depths of 4-6 (dS) and 3-5 (K) stages time alike; two K stages, or one work-group per CU
+// with deeper rings, are 15-20 % slower.
 //
 // Layout of a dS block (written by the dk/dv kernel): kv columns 32 w' + jj (w' = 0..3), q rows 32 c + 16 u + ii:
 // byte 8192 w' + 1024 (2 c + u) + 16 (2 jj + hi) + 8 g + 2 e holds row ii = 8 g + 4 hi + e.
@@ -34,12 +36,20 @@ constexpr int K_STAGE_BYTES = STAGE_KV * D * 2;    // 8 KB: 32 rows of a K tile 
 #define DQDS_NK 3
 #define DQDS_OCC 2
 #endif
+#ifndef DQDS_PRODUCERS
+#define DQDS_PRODUCERS 1
+#endif
 // Two rings of stages in LDS.  dS comes from HBM and is read once: the rate depends on the bytes in flight per CU
 // (a plain streaming read on this GPU: 32 KB in flight per CU 2.9 TB/s, 64 KB 4.8 TB/s, 128 KB and more 6.4 TB/s),
 // so its ring is deep; a head's K tiles are shared by the head's q tiles and come from the XCD's L2.
 constexpr int NDS = DQDS_NDS;
 constexpr int NK = DQDS_NK;
 constexpr int OCC = DQDS_OCC;                      // work-groups per CU
+// Waves 4-7 of a work-group only copy (4, 5: dS; 6, 7: K) and waves 0-3 only compute: an LDS-direct copy holds the
+// wave that issues it until the texture path takes it (about 175 cycles per 1 KB copy when every work-group of the
+// CU copies), which the computing waves would otherwise sit out between their MFMAs (2 % of the launch).
+constexpr bool PRODUCERS = DQDS_PRODUCERS != 0;
+constexpr int THREADS = PRODUCERS ? 512 : 256;
 constexpr int MAX_LIST = 1024;
 constexpr int K_RING = NDS * DS_STAGE_BYTES;       // LDS offset of the K ring
 constexpr int LDS_BYTES = NDS * DS_STAGE_BYTES + NK * K_STAGE_BYTES + MAX_LIST * 4;
@@ -56,7 +66,7 @@ __device__ __forceinline__ void wait_vmem_but() {
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
-__global__ __launch_bounds__(256, dqds_cfg::OCC) void bwd_dq_from_ds_kernel(BwdArgs a, float out_scale) {
+__global__ __launch_bounds__(dqds_cfg::THREADS, dqds_cfg::OCC) void bwd_dq_from_ds_kernel(BwdArgs a, float out_scale) {
   using namespace dqds_cfg;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   int* sIdx = reinterpret_cast<int*>(smem_raw + NDS * DS_STAGE_BYTES + NK * K_STAGE_BYTES);
@@ -64,7 +74,10 @@ __global__ __launch_bounds__(256, dqds_cfg::OCC) void bwd_dq_from_ds_kernel(BwdA
   const int nQ = a.map.nq, nK = a.map.nk;
   const int n_wg = a.B * a.Hq * nQ;
   const int tid = threadIdx.x;
-  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool copies = !PRODUCERS || wave >= 4;    // the wave issues copies
+  const bool computes = !PRODUCERS || wave < 4;   // the wave runs the MFMAs and stores dq
+  const int w = wave & 3;                         // its number among the waves of its kind
   const int lane = tid & 63;
   const int hh = lane >> 5;
   const int l16 = lane & 15;
@@ -80,7 +93,7 @@ __global__ __launch_bounds__(256, dqds_cfg::OCC) void bwd_dq_from_ds_kernel(BwdA
   const int n_list = a.map.cnt[qb];
   const int* list = a.map.idx + (size_t)qb * nK;
   const int* rank = a.ds_rank + (size_t)qb * nK;
-  for (int t = tid; t < n_list; t += 256) {
+  for (int t = tid; t < n_list; t += THREADS) {
     const int kb = list[t];
     sIdx[t] = kb | (rank[kb] << 10);
   }
@@ -107,8 +120,8 @@ __global__ __launch_bounds__(256, dqds_cfg::OCC) void bwd_dq_from_ds_kernel(BwdA
 
   // stage s = part s % PARTS of the list's kv tile s / PARTS: that part's dS as it lies in the block and its 32 K
   // rows.  A wave's copies complete in issue order, so a copy from the L2 issued behind copies from HBM would
-  // wait for those: waves 0, 1 copy only dS (four pieces each), waves 2, 3 only K, and each kind runs as far ahead
-  // as its ring allows.
+  // wait for those: copying waves 0, 1 copy only dS (four pieces each), 2, 3 only K, and each kind runs as far
+  // ahead as its ring allows.
   auto tile_of = [&](int s) { return __builtin_amdgcn_readfirstlane(sIdx[s / PARTS] & 1023); };
   auto block_of = [&](int s) { return __builtin_amdgcn_readfirstlane((int)((unsigned)sIdx[s / PARTS] >> 10)); };
   const bool ds_wave = w < 2;
@@ -162,12 +175,13 @@ __global__ __launch_bounds__(256, dqds_cfg::OCC) void bwd_dq_from_ds_kernel(BwdA
     for (int i = 0; i < 16; ++i) acc[t >> 1][t & 1][i] = 0.f;
 
   const int n_stages = PARTS * n_list;
-  for (int s = 0; s < ring - 1 && s < n_stages; ++s) issue(s);
+  if (copies)
+    for (int s = 0; s < ring - 1 && s < n_stages; ++s) issue(s);
   for (int s = 0; s < n_stages; ++s) {
     // the wave's copy of stage s has landed once only its copies of the stages behind it are open
     int behind = n_stages - 1 - s;
     if (behind > ring - 2) behind = ring - 2;
-    switch (behind) {
+    if (copies) switch (behind) {
       case 0: wait_vmem_but<0>(); break;
       case 1: wait_vmem_but<4>(); break;
       case 2: wait_vmem_but<8>(); break;
@@ -186,7 +200,8 @@ __global__ __launch_bounds__(256, dqds_cfg::OCC) void bwd_dq_from_ds_kernel(BwdA
       default: wait_vmem_but<60>(); break;
     }
     __syncthreads();  // (also: every wave is done with the slots the next copies go to)
-    if (s + ring - 1 < n_stages) issue(s + ring - 1);
+    if (copies && s + ring - 1 < n_stages) issue(s + ring - 1);
+    if (!computes) continue;
     const char* st = smem_raw + (s % NDS) * DS_STAGE_BYTES;
     const bf16_t* sK = reinterpret_cast<const bf16_t*>(smem_raw + K_RING + (s % NK) * K_STAGE_BYTES);
 #pragma unroll
@@ -219,20 +234,23 @@ __global__ __launch_bounds__(256, dqds_cfg::OCC) void bwd_dq_from_ds_kernel(BwdA
   // four complete 256-byte rows; lane: q row lane & 31 of block 2 wq + qi, head columns 32 (2 wd + di) + 8 g + 4 hh + 0..3
   const int row_here = lane & 31;
   const unsigned wr = (unsigned)row_here * 256u + 8u * (unsigned)hh;
+  if (computes) {
 #pragma unroll
-  for (int qi = 0; qi < 2; ++qi)
+    for (int qi = 0; qi < 2; ++qi)
 #pragma unroll
-    for (int di = 0; di < 2; ++di)
+      for (int di = 0; di < 2; ++di)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const f32x16& x = acc[qi][di];
-        const bf16x2 lo = pack_bf16(x[4 * g] * out_scale, x[4 * g + 1] * out_scale);
-        const bf16x2 hi = pack_bf16(x[4 * g + 2] * out_scale, x[4 * g + 3] * out_scale);
-        const bf16x4 out = {lo[0], lo[1], hi[0], hi[1]};
-        *reinterpret_cast<bf16x4*>(smem_raw + (2 * wq + qi) * 8192 + wr
-                                   + (unsigned)(((4 * (2 * wd + di) + g) ^ (row_here & 15)) << 4)) = out;
-      }
+        for (int g = 0; g < 4; ++g) {
+          const f32x16& x = acc[qi][di];
+          const bf16x2 lo = pack_bf16(x[4 * g] * out_scale, x[4 * g + 1] * out_scale);
+          const bf16x2 hi = pack_bf16(x[4 * g + 2] * out_scale, x[4 * g + 3] * out_scale);
+          const bf16x4 out = {lo[0], lo[1], hi[0], hi[1]};
+          *reinterpret_cast<bf16x4*>(smem_raw + (2 * wq + qi) * 8192 + wr
+                                     + (unsigned)(((4 * (2 * wd + di) + g) ^ (row_here & 15)) << 4)) = out;
+        }
+  }
   __syncthreads();
+  if (!computes) return;
   const char* stage = smem_raw + w * 8192;  // wave w stores q block w
   bf16_t* dQg = static_cast<bf16_t*>(a.dq) + ((size_t)bh * a.Sq + (size_t)qb * BQ + (size_t)w * 32) * D;
   const int chunk = lane & 15;
@@ -255,7 +273,7 @@ int bwd_dq_from_ds(const BwdArgs& a, float out_scale, hipStream_t stream) {
                                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
   if (attr != hipSuccess) return set_error(FLEXATTN_ELAUNCH, "hipFuncSetAttribute(dq from dS): %s", hipGetErrorString(attr));
   const int n_wg = a.B * a.Hq * (a.Sq / BQ);
-  hipLaunchKernelGGL(kern, dim3(n_wg), dim3(256), LDS_BYTES, stream, a, out_scale);
+  hipLaunchKernelGGL(kern, dim3(n_wg), dim3(THREADS), LDS_BYTES, stream, a, out_scale);
   return check_launch("flexattn_bwd_dq (from dS) bf16");
 }
 
