@@ -898,6 +898,11 @@ def test_rows_that_keep_no_key(F, dtype):
         assert bool(torch.isfinite(t.float()).all())
     assert float(dq[:, :, first_empty:].float().abs().max()) == 0.0
     _check_grads((dq[:, :, :first_empty], dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, dtype, okw)
+    # dq from the dk/dv pass's dS: the last q tile's list of kv tiles is empty (its rows are written as zeros)
+    dqx = _exchanged_dq(F, q, k, v, l, m, o, do, d, sc, mf, bf, None, dk, dv, expect=dtype == torch.bfloat16)
+    if dqx is not None:
+        assert float(dqx[:, :, first_empty:].float().abs().max()) == 0.0
+        _check_grads((dqx[:, :, :first_empty], dk, dv), (rdq, rdk, rdv), qc, kc, vc, doc, o, l, m, dtype, okw, tag="exchange ")
 
 
 @pytest.mark.parametrize("case", ["causal", "gqa_softcap_docs", "alibi_window", "fp32_plain"])
