@@ -34,6 +34,13 @@ def alibi_formula_mod(s, b, h, q_idx, kv_idx):
     return s + 2.0 ** (-8.0 * (h + 1) / 4) * (kv_idx - q_idx)
 
 
+def elementary_mod(s, b, h, q_idx, kv_idx):
+    """every elementary function the compiler knows once (sigmoid, exp, sqrt, log, abs), clamp, maximum, //"""
+    gate = torch.sigmoid(0.5 * s) * torch.exp(-0.1 * torch.abs(s))
+    r = torch.sqrt(1.0 + 0.01 * torch.abs(q_idx - kv_idx)) - torch.log(1.0 + s * s)
+    return torch.clamp(s * gate + 0.2 * r, min=-4.0, max=6.0) + 0.05 * torch.maximum(s, 0.1 * (kv_idx // 64 - q_idx // 64))
+
+
 def softcap30_mod(s, b, h, q_idx, kv_idx):
     return 30.0 * torch.tanh(s / 30.0)
 
@@ -76,6 +83,7 @@ def compiled():
         "softcap_mod": (compiler.compile_score_mod(softcap_mod, recognise=False), None),
         "mixed_mod": (compiler.compile_score_mod(mixed_mod), None),
         "alibi_symmetric_mod": (compiler.compile_score_mod(alibi_symmetric_mod), None),
+        "elementary_mod": (compiler.compile_score_mod(elementary_mod), None),
         "prefix_lm": (None, compiler.compile_mask_fn(prefix_lm_mask, 128, 128)),
         "checker": (None, compiler.compile_mask_fn(checker_mask, 128, 128)),
         "mixed_mod+prefix_lm": (compiler.compile_score_mod(mixed_mod), compiler.compile_mask_fn(prefix_lm_mask, 128, 128)),

@@ -34,7 +34,7 @@ def _oracle_kwargs(name, Sq, Sk):
     kw = {}
     parts = name.split("+")
     mods = {"alibi_mod": cf.alibi_mod, "softcap_mod": cf.softcap_mod, "mixed_mod": cf.mixed_mod,
-            "alibi_symmetric_mod": cf.alibi_symmetric_mod}
+            "alibi_symmetric_mod": cf.alibi_symmetric_mod, "elementary_mod": cf.elementary_mod}
     masks = {"prefix_lm": cf.prefix_lm_mask, "checker": cf.checker_mask}
     for p in parts:
         if p in mods:
@@ -45,8 +45,8 @@ def _oracle_kwargs(name, Sq, Sk):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
-@pytest.mark.parametrize("name", ["alibi_mod", "softcap_mod", "mixed_mod", "alibi_symmetric_mod", "prefix_lm", "checker",
-                                  "mixed_mod+prefix_lm"])
+@pytest.mark.parametrize("name", ["alibi_mod", "softcap_mod", "mixed_mod", "alibi_symmetric_mod", "elementary_mod", "prefix_lm",
+                                  "checker", "mixed_mod+prefix_lm"])
 def test_compiled_closures_all_passes(F, compiled, name, dtype):
     _closures_all_passes(F, compiled, name, dtype, 128)
 

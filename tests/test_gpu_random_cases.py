@@ -26,7 +26,8 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 N_CASES, N_LONG = 192, 32   # (the last N_LONG with 1400 to 2600 queries)
 _CLOSURES = {"alibi_mod": cf.alibi_mod, "softcap_mod": cf.softcap_mod, "mixed_mod": cf.mixed_mod,
-             "alibi_symmetric_mod": cf.alibi_symmetric_mod, "mixed_mod+prefix_lm": cf.mixed_mod}
+             "alibi_symmetric_mod": cf.alibi_symmetric_mod, "elementary_mod": cf.elementary_mod,
+             "mixed_mod+prefix_lm": cf.mixed_mod}
 _CLOSURE_MASKS = {"prefix_lm": cf.prefix_lm_mask, "checker": cf.checker_mask, "mixed_mod+prefix_lm": cf.prefix_lm_mask}
 _TILE_FORMS = ("squared_tile", "tile_local_distance")
 
