@@ -418,3 +418,65 @@ def test_entry_points_replayed_from_a_captured_graph(F, case):
         torch.cuda.synchronize()
         for n, a, b_ in zip(("o", "l", "m", "dq", "dk", "dv", "dq from dS"), out, eager):
             _same(f"{n} of replay {rep}", a, b_)
+
+
+def test_host_threads_on_streams_of_their_own(F):
+    """Four host threads, each on a stream of its own, run different workloads (masks, scores, dtypes, the dS
+    hand-over) at the same time, eight steps each: every step gives the bits of the same calls made alone (the C
+    entry points keep no state between calls, the error text is per thread, the Python caches are only read and
+    extended)."""
+    import math
+    import threading
+    import warnings
+    from flex_attention_tpu_amd import masks, scores
+    warnings.filterwarnings("ignore", message="score_fn with sm_scale")
+    S, D = 1024, 128
+    docs = torch.repeat_interleave(torch.arange(3), torch.tensor([300, 600, 124])).to(torch.int32)
+    work = [
+        ("causal bf16", torch.bfloat16, 2, 8, 8, masks.make_causal_mask_fns(128, 128), None, None, False),
+        ("softcap documents bf16, dS hand-over", torch.bfloat16, 1, 8, 2, (None, None), scores.make_softcap_score_fn(30.0), docs, True),
+        ("position bias, window bf16", torch.bfloat16, 2, 4, 4, masks.make_causal_sliding_window_mask_fns(128, 128, 300),
+         scores.make_alibi_global_score_fn(4), None, False),
+        ("plain fp32", torch.float32, 1, 4, 4, (None, None), None, None, False),
+    ]
+
+    def step(item, q, k, v, do):
+        _, dtype, B, Hq, Hkv, (mf, bf), sfn, sid, exchange = item
+        sc = 1 / math.sqrt(D)
+        o, l, m = F._flex_attention_impl(q, k, v, None, sid, True, sid is not None, sc, 1, 128, 128, 128, False, bf, mf, sfn)
+        d = F.compute_delta(o, do)
+        kw = dict(block_b=1, block_q=128, block_k_major=128, block_k=128, sm_scale=sc, debug=False, score_fn=sfn,
+                  mask_fn=mf, block_mask_fn=bf, causal=sid is not None)
+        dk, dv, ds = F.flash_attention_bwd_dkv(k, v, q, None, sid, l, m, d, do, block_q_major=128, return_ds=exchange, **kw) \
+            if exchange else (*F.flash_attention_bwd_dkv(k, v, q, None, sid, l, m, d, do, block_q_major=128, **kw), None)
+        dq = F.flex_attention_bwd_dq(q, k, v, None, sid, l, m, o, do, d, ds=ds, **kw)
+        return o, l, m, dq, dk, dv
+    inputs, alone = [], []
+    for n, item in enumerate(work):
+        _, dtype, B, Hq, Hkv = item[:5]
+        gen = torch.Generator(device=DEV).manual_seed(40 + n)
+        t = [torch.randn(B, h, S, D, device=DEV, dtype=dtype, generator=gen) for h in (Hq, Hkv, Hkv, Hq)]
+        inputs.append(t)
+        alone.append(step(item, *t))
+    torch.cuda.synchronize()
+    failures = []
+
+    def run(n):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for rep in range(8):
+                    got = step(work[n], *inputs[n])
+                    stream.synchronize()
+                    for name, a, b_ in zip(("o", "l", "m", "dq", "dk", "dv"), got, alone[n]):
+                        if not torch.equal(a, b_):
+                            failures.append(f"{work[n][0]}: {name} of step {rep} differs")
+        except Exception as e:   # noqa: BLE001  (reported by the main thread)
+            failures.append(f"{work[n][0]}: {e!r}")
+    threads = [threading.Thread(target=run, args=(n,)) for n in range(len(work))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not failures, failures[:4]
