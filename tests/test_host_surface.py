@@ -274,3 +274,20 @@ def test_ds_exchange_policy():
     assert ds_exchange_pays(None, masks.make_jagged_mask_fns(128, 128, [100, 156])[0])
     assert ds_exchange_pays(None, None, segment_ids=[0] * 128 + [1] * 128)
 
+
+
+def test_no_compute_path_without_the_library(monkeypatch, tmp_path):
+    """Without libflexattn.so the loader raises, naming the build step: nothing falls back to the CPU, and the
+    package never imports the oracle (checked in a fresh interpreter, where no test has imported it)."""
+    import subprocess
+    import sys
+    from flex_attention_tpu_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libflexattn.so"))
+    with pytest.raises(ImportError, match="no other compute path"):
+        _lib.load()
+    code = ("import sys, flex_attention_tpu_amd as F; from flex_attention_tpu_amd import flex_attention, compiler, util, roofline; "
+            "bad = [m for m in sys.modules if m == 'oracle' or m.startswith('oracle.')]; print(bad); sys.exit(1 if bad else 0)")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
